@@ -1,0 +1,70 @@
+"""One registry from an architecture's name (config.json `architectures[0]`) to its model.
+
+picolm has no such table: it sniffs the architecture from substrings of GGUF metadata
+(picolm/model_gguf.c:729-751) and from which tensors exist.  Here an architecture is an
+entry with two callables: one that types the config.json, one that builds the model's
+parts from the typed configuration.
+"""
+from __future__ import annotations
+
+import json
+import os
+from dataclasses import dataclass
+from typing import Callable
+
+from .llama import ConfigError
+
+
+@dataclass(frozen=True)
+class Architecture:
+    name: str
+    parse_config: Callable[[dict], object]      # dict of config.json -> typed configuration
+    build: Callable[..., object]                # (config, runtime) -> DecoderModel
+
+
+_REGISTRY: dict[str, Architecture] = {}
+
+
+def register_architecture(name: str, parse_config, build, *, replace: bool = False) -> Architecture:
+    if name in _REGISTRY and not replace:
+        raise ConfigError(f"architecture '{name}' is already registered")
+    arch = Architecture(name, parse_config, build)
+    _REGISTRY[name] = arch
+    return arch
+
+
+def unregister_architecture(name: str) -> None:
+    _REGISTRY.pop(name, None)
+
+
+def known_architectures() -> list[str]:
+    return sorted(_REGISTRY)
+
+
+def architecture_name(config_dict: dict) -> str:
+    archs = config_dict.get("architectures")
+    if isinstance(archs, (list, tuple)) and archs:
+        return str(archs[0])
+    if isinstance(archs, str):
+        return archs
+    raise ConfigError("architectures: missing; config.json must name its architecture "
+                      f"(known: {', '.join(known_architectures())})")
+
+
+def resolve(config_dict: dict) -> Architecture:
+    name = architecture_name(config_dict)
+    if name not in _REGISTRY:
+        raise ConfigError(f"architectures: '{name}' is not registered "
+                          f"(known: {', '.join(known_architectures())})")
+    return _REGISTRY[name]
+
+
+def read_config_json(model_dir: str) -> dict:
+    path = os.path.join(model_dir, "config.json") if os.path.isdir(model_dir) else model_dir
+    try:
+        with open(path, "r", encoding="utf-8") as f:
+            return json.load(f)
+    except FileNotFoundError:
+        raise ConfigError(f"{path}: no config.json") from None
+    except json.JSONDecodeError as e:
+        raise ConfigError(f"{path}: not JSON ({e})") from None

@@ -1,0 +1,52 @@
+// C entry points of libpicolm_hip.so.  Pointers are device pointers unless said otherwise;
+// every function returns 0 on success and a negative code with a message in
+// picolm_last_error() otherwise.  Nothing here synchronises: work is queued on `stream`.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+const char* picolm_last_error(void);
+int picolm_abi_version(void);
+int picolm_device_check(void);     // 0 if the current device is a gfx950
+
+int picolm_embed(const void* table, int table_dt, const int32_t* tokens, float* x, int T, int D,
+                 int V, hipStream_t stream);
+int picolm_rmsnorm(const float* x, const float* w, void* out, int out_dt, const int32_t* rows,
+                   int n_rows, int D, float eps, hipStream_t stream);
+int picolm_rope_kv_store(const float* qkv, void* q_out, void* k_pages, void* v_pages, int dt,
+                         const float* cos_t, const float* sin_t, int style, const int32_t* tok_pos,
+                         const int32_t* tok_seq, const int32_t* seq_slot, const int32_t* page_table,
+                         int max_pages, int ring_pages, int T, int H, int G, int d,
+                         hipStream_t stream);
+int picolm_silu_mul(const void* gu, int in_dt, void* out, int out_dt, int64_t n_pairs,
+                    hipStream_t stream);
+int picolm_add_into(float* y, const void* x, int x_dt, int64_t n, hipStream_t stream);
+
+int picolm_gemm_generic(const void* A, int a_dt, const void* W, int w_dt, void* C, int c_dt, int M,
+                        int N, int K, int64_t lda, int64_t ldw, int64_t ldc, int epilogue,
+                        hipStream_t stream);
+
+int picolm_attn_prefill_tile_rows(void);
+int picolm_attn_prefill_generic(const void* q, const void* k_pages, const void* v_pages, void* out,
+                                int dt, const int32_t* tile_seq, const int32_t* tile_q0, int n_tiles,
+                                const int32_t* seq_slot, const int32_t* seq_pos0,
+                                const int32_t* seq_nnew, const int32_t* cu_seqlens,
+                                const int32_t* page_table, int max_pages, int ring_pages, int H,
+                                int G, int d, int window, float scale, hipStream_t stream);
+int picolm_attn_decode_generic(const void* q, const void* k_pages, const void* v_pages, void* out,
+                               float* partial, int dt, int n_seq, int n_splits,
+                               const int32_t* seq_slot, const int32_t* seq_pos0,
+                               const int32_t* cu_seqlens, const int32_t* page_table, int max_pages,
+                               int ring_pages, int H, int G, int d, int window, float scale,
+                               hipStream_t stream);
+
+int picolm_argmax(const float* logits, int32_t* out, int n_rows, int V, int64_t ld,
+                  hipStream_t stream);
+
+#ifdef __cplusplus
+}
+#endif

@@ -1,0 +1,309 @@
+// Attention over the paged cache on the vector ALU, for any head size that is a multiple of
+// 16 (up to 256), any number of heads and groups, float or bf16 storage.  One kernel serves
+// both kinds of step: a tile is up to 16 "rows" that share one KV head.
+//   prefill: rows = consecutive new tokens of one sequence, for one query head;
+//   decode : rows = the query heads of one KV group, for a sequence's single new token,
+//            optionally over a slice of the pages (split-K) whose partial results a second
+//            kernel merges.
+// The recurrence is picolm's online softmax (picolm/model_attention.c:43-140): running
+// maximum m, running sum l, accumulator rescaled by exp(m_old - m_new); key t is visible to
+// a query at position p iff t <= p (and p - t < window when a window is set).
+// picolm's split kernels keep (max, sum, acc) per split and merge with exp(m_i - M)
+// (picolm/backend_gpu_kernels.cu:802-963); the same shape is used here.
+#include "common.h"
+#include "api.h"
+
+#define AT_ROWS 16
+#define AT_THREADS 256
+#define AT_MAX_D 256
+#define NEG_BIG (-1e30f)
+
+struct AttnArgs {
+    const void* q;            // [T][H*d]
+    const void* k_pages;      // [n_pages][G][PAGE][d]
+    const void* v_pages;
+    void* out;                // [T][H*d]
+    float* partial;           // decode split-K: [n_seq][H][n_splits][d+2], or null
+    const int32_t* tile_seq;  // prefill: sequence of each tile
+    const int32_t* tile_q0;   // prefill: first new-token index of each tile
+    const int32_t* seq_slot;
+    const int32_t* seq_pos0;  // tokens the sequence held before this step
+    const int32_t* seq_nnew;
+    const int32_t* cu_seqlens;  // first token row of each sequence in this step
+    const int32_t* page_table;
+    int max_pages, ring_pages;
+    int H, G, d, window;
+    float scale;
+    int decode;     // 0 prefill tiles, 1 decode groups
+    int n_splits;   // decode only
+};
+
+template <typename T>
+__global__ __launch_bounds__(AT_THREADS) void attn_tile_kernel(AttnArgs a) {
+    extern __shared__ float lds[];
+    const int d = a.d, dp = d + 1;
+    float* Qs = lds;                            // [AT_ROWS][d]
+    float* KVs = Qs + AT_ROWS * d;              // [PAGE][d+1]
+    float* Ps = KVs + PAGE_TOKENS * dp;         // [AT_ROWS][PAGE]
+    float* alpha_s = Ps + AT_ROWS * PAGE_TOKENS;  // [AT_ROWS]
+    float* l_s = alpha_s + AT_ROWS;             // [AT_ROWS]
+    float* m_s = l_s + AT_ROWS;                 // [AT_ROWS]
+    __shared__ int row_tok[AT_ROWS], row_head[AT_ROWS], row_qpos[AT_ROWS];
+
+    const int tid = threadIdx.x, wave = tid / WAVE, lane = tid % WAVE;
+    const int R = a.H / a.G;
+    int seq, g, split = 0, n_rows;
+    if (a.decode) {
+        seq = blockIdx.x;
+        const int chunks = (R + AT_ROWS - 1) / AT_ROWS;
+        g = blockIdx.y / chunks;
+        const int chunk = blockIdx.y % chunks;
+        split = blockIdx.z;
+        n_rows = min(AT_ROWS, R - chunk * AT_ROWS);
+        if (tid < AT_ROWS) {
+            row_tok[tid] = a.cu_seqlens[seq];
+            row_head[tid] = g * R + chunk * AT_ROWS + tid;
+            row_qpos[tid] = a.seq_pos0[seq];
+        }
+    } else {
+        seq = a.tile_seq[blockIdx.x];
+        const int q0 = a.tile_q0[blockIdx.x];
+        const int h = blockIdx.y;
+        g = h / R;
+        n_rows = min(AT_ROWS, a.seq_nnew[seq] - q0);
+        if (tid < AT_ROWS) {
+            row_tok[tid] = a.cu_seqlens[seq] + q0 + tid;
+            row_head[tid] = h;
+            row_qpos[tid] = a.seq_pos0[seq] + q0 + tid;
+        }
+    }
+    __syncthreads();
+    // visible key range of the tile: [lo, hi]
+    const int qpos_first = row_qpos[0], qpos_last = row_qpos[n_rows - 1];
+    const int hi = qpos_last;
+    const int lo = a.window > 0 ? max(0, qpos_first - a.window + 1) : 0;
+    int page_lo = lo / PAGE_TOKENS, page_hi = hi / PAGE_TOKENS + 1;   // [page_lo, page_hi)
+    if (a.decode && a.n_splits > 1) {
+        const int np = page_hi - page_lo;
+        const int per = (np + a.n_splits - 1) / a.n_splits;
+        const int b = page_lo + split * per;
+        page_hi = min(page_hi, b + per);
+        page_lo = b;
+    }
+
+    const T* q = (const T*)a.q;
+    for (int idx = tid; idx < AT_ROWS * d; idx += AT_THREADS) {
+        const int r = idx / d, c = idx % d;
+        Qs[idx] = r < n_rows ? to_f32<T>(q[(size_t)row_tok[r] * a.H * d + (size_t)row_head[r] * d + c]) : 0.f;
+    }
+    // per-wave running statistics of its 4 rows (uniform across the wave)
+    float m_run[4], l_run[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        m_run[i] = NEG_BIG;
+        l_run[i] = 0.f;
+    }
+    // PV ownership: thread -> (row pr, column group pc), columns pc + 16*j
+    const int pr = tid / 16, pc = tid % 16;
+    const int n_cg = d / 16;
+    float acc[AT_MAX_D / 16];
+#pragma unroll
+    for (int j = 0; j < AT_MAX_D / 16; ++j) acc[j] = 0.f;
+
+    const int slot = a.seq_slot[seq];
+    const int32_t* pt = a.page_table + (size_t)slot * a.max_pages;
+    const size_t page_elems = (size_t)a.G * PAGE_TOKENS * d;
+
+    for (int page = page_lo; page < page_hi; ++page) {
+        const int phys = pt[page % a.ring_pages];
+        const size_t base = (size_t)phys * page_elems + (size_t)g * PAGE_TOKENS * d;
+        const int key0 = page * PAGE_TOKENS;
+        const int n_keys = min(PAGE_TOKENS, hi - key0 + 1);   // rows beyond are not this sequence's
+        __syncthreads();                                       // previous PV done with KVs / Ps
+        {
+            const T* kp = (const T*)a.k_pages + base;
+            for (int idx = tid; idx < PAGE_TOKENS * d; idx += AT_THREADS) {
+                const int r = idx / d, c = idx % d;
+                KVs[r * dp + c] = r < n_keys ? to_f32<T>(kp[idx]) : 0.f;
+            }
+        }
+        __syncthreads();
+        // scores: wave handles rows 4*wave .. +3, lane = key
+        {
+            float s[4] = {0.f, 0.f, 0.f, 0.f};
+            const float* kr = KVs + lane * dp;
+            const float* q0p = Qs + (4 * wave) * d;
+            for (int c = 0; c < d; ++c) {
+                const float kv = kr[c];
+#pragma unroll
+                for (int i = 0; i < 4; ++i) s[i] = fmaf(q0p[i * d + c], kv, s[i]);
+            }
+            const int kpos = key0 + lane;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int r = 4 * wave + i;
+                const int qp = row_qpos[r];
+                const bool vis = r < n_rows && kpos <= qp && (a.window <= 0 || qp - kpos < a.window);
+                const float sc = vis ? s[i] * a.scale : NEG_BIG;
+                const float m_new = fmaxf(m_run[i], wave_max(sc));
+                const float p = vis ? expf(sc - m_new) : 0.f;
+                const float al = expf(m_run[i] - m_new);
+                l_run[i] = l_run[i] * al + wave_sum(p);
+                m_run[i] = m_new;
+                Ps[r * PAGE_TOKENS + lane] = p;
+                if (lane == 0) alpha_s[r] = al;
+            }
+        }
+        __syncthreads();
+        {
+            const T* vp = (const T*)a.v_pages + base;
+            for (int idx = tid; idx < PAGE_TOKENS * d; idx += AT_THREADS) {
+                const int r = idx / d, c = idx % d;
+                KVs[r * dp + c] = r < n_keys ? to_f32<T>(vp[idx]) : 0.f;
+            }
+        }
+        __syncthreads();
+        {
+            const float al = alpha_s[pr];
+            const float* p = Ps + pr * PAGE_TOKENS;
+#pragma unroll
+            for (int j = 0; j < AT_MAX_D / 16; ++j) acc[j] *= al;
+            for (int key = 0; key < n_keys; ++key) {
+                const float pk = p[key];
+                const float* vr = KVs + key * dp + pc;
+#pragma unroll
+                for (int j = 0; j < AT_MAX_D / 16; ++j)
+                    if (j < n_cg) acc[j] = fmaf(pk, vr[16 * j], acc[j]);
+            }
+        }
+    }
+    if (lane == 0) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            l_s[4 * wave + i] = l_run[i];
+            m_s[4 * wave + i] = m_run[i];
+        }
+    }
+    __syncthreads();
+    if (pr >= n_rows) return;
+    const int tok = row_tok[pr], head = row_head[pr];
+    if (a.decode && a.partial) {
+        float* po = a.partial + (((size_t)seq * a.H + head) * a.n_splits + split) * (d + 2);
+        if (pc == 0) {
+            po[0] = m_s[pr];
+            po[1] = l_s[pr];
+        }
+#pragma unroll
+        for (int j = 0; j < AT_MAX_D / 16; ++j)
+            if (j < n_cg) po[2 + pc + 16 * j] = acc[j];
+    } else {
+        const float l = l_s[pr];
+        const float inv = l > 0.f ? 1.0f / l : 0.f;
+        T* o = (T*)a.out + (size_t)tok * a.H * d + (size_t)head * d;
+#pragma unroll
+        for (int j = 0; j < AT_MAX_D / 16; ++j)
+            if (j < n_cg) o[pc + 16 * j] = from_f32<T>(acc[j] * inv);
+    }
+}
+
+// out = sum_i exp(m_i - M) acc_i / sum_i exp(m_i - M) l_i over the splits of one (seq, head).
+template <typename T>
+__global__ void attn_merge_kernel(const float* __restrict__ partial, T* __restrict__ out,
+                                  const int32_t* __restrict__ cu_seqlens, int H, int d, int n_splits) {
+    const int seq = blockIdx.x / H, head = blockIdx.x % H;
+    const float* p = partial + ((size_t)seq * H + head) * n_splits * (d + 2);
+    float M = NEG_BIG;
+    for (int i = 0; i < n_splits; ++i) M = fmaxf(M, p[(size_t)i * (d + 2)]);
+    float L = 0.f;
+    for (int i = 0; i < n_splits; ++i) L += expf(p[(size_t)i * (d + 2)] - M) * p[(size_t)i * (d + 2) + 1];
+    const float inv = L > 0.f ? 1.0f / L : 0.f;
+    T* o = out + (size_t)cu_seqlens[seq] * H * d + (size_t)head * d;
+    for (int c = threadIdx.x; c < d; c += blockDim.x) {
+        float acc = 0.f;
+        for (int i = 0; i < n_splits; ++i)
+            acc += expf(p[(size_t)i * (d + 2)] - M) * p[(size_t)i * (d + 2) + 2 + c];
+        o[c] = from_f32<T>(acc * inv);
+    }
+}
+
+static size_t attn_lds_bytes(int d) {
+    return sizeof(float) * ((size_t)AT_ROWS * d + (size_t)PAGE_TOKENS * (d + 1) + AT_ROWS * PAGE_TOKENS + 3 * AT_ROWS);
+}
+
+template <typename T>
+static int launch_attn(const AttnArgs& a, dim3 grid, hipStream_t stream) {
+    const size_t lds = attn_lds_bytes(a.d);
+    static size_t raised = 48 * 1024;      // what a kernel may use without asking
+    if (lds > raised) {
+        hipError_t e = hipFuncSetAttribute((const void*)attn_tile_kernel<T>,
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        PICOLM_REQUIRE(e == hipSuccess, "attention: cannot raise the LDS limit to %zu: %s", lds,
+                       hipGetErrorString(e));
+        raised = lds;
+    }
+    attn_tile_kernel<T><<<grid, dim3(AT_THREADS), lds, stream>>>(a);
+    PICOLM_LAUNCH_CHECK("attention");
+    return 0;
+}
+
+static int check_attn_sizes(const char* who, int H, int G, int d, int max_pages, int ring_pages) {
+    PICOLM_REQUIRE(H > 0 && G > 0 && H % G == 0, "%s: %d heads do not split over %d groups", who, H, G);
+    PICOLM_REQUIRE(d >= 16 && d % 16 == 0 && d <= AT_MAX_D,
+                   "%s: head size %d is not a multiple of 16 in [16, %d]", who, d, AT_MAX_D);
+    PICOLM_REQUIRE(max_pages > 0 && ring_pages > 0 && ring_pages <= max_pages,
+                   "%s: bad page table geometry max_pages=%d ring_pages=%d", who, max_pages, ring_pages);
+    return 0;
+}
+
+extern "C" int picolm_attn_prefill_generic(const void* q, const void* k_pages, const void* v_pages,
+                                           void* out, int dt, const int32_t* tile_seq,
+                                           const int32_t* tile_q0, int n_tiles,
+                                           const int32_t* seq_slot, const int32_t* seq_pos0,
+                                           const int32_t* seq_nnew, const int32_t* cu_seqlens,
+                                           const int32_t* page_table, int max_pages, int ring_pages,
+                                           int H, int G, int d, int window, float scale,
+                                           hipStream_t stream) {
+    if (check_attn_sizes("attn_prefill", H, G, d, max_pages, ring_pages)) return -1;
+    PICOLM_REQUIRE(H <= 65535, "attn_prefill: %d heads exceed the grid", H);
+    if (n_tiles <= 0) return 0;
+    AttnArgs a = {q, k_pages, v_pages, out, nullptr, tile_seq, tile_q0, seq_slot, seq_pos0, seq_nnew,
+                  cu_seqlens, page_table, max_pages, ring_pages, H, G, d, window, scale, 0, 1};
+    dim3 grid(n_tiles, H);
+    if (dt == PICOLM_F32) return launch_attn<float>(a, grid, stream);
+    if (dt == PICOLM_BF16) return launch_attn<bf16_t>(a, grid, stream);
+    PICOLM_REQUIRE(false, "attn_prefill: unknown dtype %d", dt);
+}
+
+extern "C" int picolm_attn_prefill_tile_rows(void) { return AT_ROWS; }
+
+extern "C" int picolm_attn_decode_generic(const void* q, const void* k_pages, const void* v_pages,
+                                          void* out, float* partial, int dt, int n_seq, int n_splits,
+                                          const int32_t* seq_slot, const int32_t* seq_pos0,
+                                          const int32_t* cu_seqlens, const int32_t* page_table,
+                                          int max_pages, int ring_pages, int H, int G, int d,
+                                          int window, float scale, hipStream_t stream) {
+    if (check_attn_sizes("attn_decode", H, G, d, max_pages, ring_pages)) return -1;
+    PICOLM_REQUIRE(n_splits >= 1 && n_splits <= 65535, "attn_decode: bad split count %d", n_splits);
+    PICOLM_REQUIRE(n_splits == 1 || partial != nullptr, "attn_decode: splits need a partial buffer");
+    if (n_seq <= 0) return 0;
+    const int chunks = ceil_div(H / G, AT_ROWS);
+    PICOLM_REQUIRE(G * chunks <= 65535, "attn_decode: %d groups exceed the grid", G * chunks);
+    AttnArgs a = {q, k_pages, v_pages, out, n_splits > 1 ? partial : nullptr, nullptr, nullptr, seq_slot,
+                  seq_pos0, nullptr, cu_seqlens, page_table, max_pages, ring_pages, H, G, d, window,
+                  scale, 1, n_splits};
+    dim3 grid(n_seq, G * chunks, n_splits);
+    int rc;
+    if (dt == PICOLM_F32) rc = launch_attn<float>(a, grid, stream);
+    else if (dt == PICOLM_BF16) rc = launch_attn<bf16_t>(a, grid, stream);
+    else PICOLM_REQUIRE(false, "attn_decode: unknown dtype %d", dt);
+    if (rc) return rc;
+    if (n_splits > 1) {
+        dim3 mgrid(n_seq * H), mblock(d <= 64 ? 64 : (d <= 128 ? 128 : 256));
+        if (dt == PICOLM_F32)
+            attn_merge_kernel<float><<<mgrid, mblock, 0, stream>>>(partial, (float*)out, cu_seqlens, H, d, n_splits);
+        else
+            attn_merge_kernel<bf16_t><<<mgrid, mblock, 0, stream>>>(partial, (bf16_t*)out, cu_seqlens, H, d, n_splits);
+        PICOLM_LAUNCH_CHECK("attn_merge");
+    }
+    return 0;
+}

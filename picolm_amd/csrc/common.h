@@ -1,0 +1,82 @@
+// Shared device helpers for the gfx950 kernels: storage types, conversions, reductions,
+// and the error channel of the C entry points.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stdio.h>
+
+// ---- element types ------------------------------------------------------------------
+// Tensors are float (32-bit) or bf16 stored as uint16_t.  All arithmetic is float.
+enum { PICOLM_F32 = 0, PICOLM_BF16 = 1 };
+typedef uint16_t bf16_t;
+
+#define PAGE_TOKENS 64       // tokens of one cache page; also the key tile of attention
+#define WAVE 64
+
+__device__ __forceinline__ float bf16_bits_to_f32(bf16_t v) {
+    return __uint_as_float(((uint32_t)v) << 16);
+}
+// Round to nearest, ties to even; NaN stays NaN.
+__device__ __forceinline__ bf16_t f32_to_bf16_bits(float f) {
+    uint32_t u = __float_as_uint(f);
+    if ((u & 0x7fffffffu) > 0x7f800000u) return (bf16_t)((u >> 16) | 0x40u);
+    u += 0x7fffu + ((u >> 16) & 1u);
+    return (bf16_t)(u >> 16);
+}
+
+template <typename T> __device__ __forceinline__ float to_f32(T v);
+template <> __device__ __forceinline__ float to_f32<float>(float v) { return v; }
+template <> __device__ __forceinline__ float to_f32<bf16_t>(bf16_t v) { return bf16_bits_to_f32(v); }
+
+template <typename T> __device__ __forceinline__ T from_f32(float v);
+template <> __device__ __forceinline__ float from_f32<float>(float v) { return v; }
+template <> __device__ __forceinline__ bf16_t from_f32<bf16_t>(float v) { return f32_to_bf16_bits(v); }
+
+// ---- reductions ---------------------------------------------------------------------
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+    for (int o = WAVE / 2; o > 0; o >>= 1) v += __shfl_xor(v, o, WAVE);
+    return v;
+}
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+    for (int o = WAVE / 2; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, WAVE));
+    return v;
+}
+// Sum over a block of up to 1024 threads; `scratch` holds >= 16 floats of LDS.
+__device__ __forceinline__ float block_sum(float v, float* scratch) {
+    v = wave_sum(v);
+    const int wave = threadIdx.x / WAVE, lane = threadIdx.x % WAVE;
+    const int n_waves = (blockDim.x + WAVE - 1) / WAVE;
+    __syncthreads();
+    if (lane == 0) scratch[wave] = v;
+    __syncthreads();
+    float t = 0.f;
+    for (int i = 0; i < n_waves; ++i) t += scratch[i];
+    return t;
+}
+
+// ---- host side ------------------------------------------------------------------------
+// Every entry point returns 0 or a negative code and leaves a message for
+// picolm_last_error().
+void picolm_set_error(const char* fmt, ...);
+
+#define PICOLM_REQUIRE(cond, ...)                         \
+    do {                                                  \
+        if (!(cond)) {                                    \
+            picolm_set_error(__VA_ARGS__);                \
+            return -1;                                    \
+        }                                                 \
+    } while (0)
+
+#define PICOLM_LAUNCH_CHECK(name)                                                     \
+    do {                                                                              \
+        hipError_t e__ = hipGetLastError();                                           \
+        if (e__ != hipSuccess) {                                                      \
+            picolm_set_error("%s: launch failed: %s", name, hipGetErrorString(e__));  \
+            return -2;                                                                \
+        }                                                                             \
+    } while (0)
+
+static inline int ceil_div(int a, int b) { return (a + b - 1) / b; }
+static inline int64_t ceil_div64(int64_t a, int64_t b) { return (a + b - 1) / b; }

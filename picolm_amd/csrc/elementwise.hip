@@ -1,0 +1,205 @@
+// Row-wise kernels: embedding gather, RMSNorm, rotation + cache write, and the small
+// element-wise helpers.  One workgroup handles one row (token); all arithmetic is float.
+#include "common.h"
+#include "api.h"
+
+// ---- embedding: x[t][:] = table[tokens[t]][:] ------------------------------------------
+// picolm/model_core.c:1785-1786, :2758-2762: the row is converted to float, no scaling.
+template <typename TW>
+__global__ void embed_kernel(const TW* __restrict__ table, const int32_t* __restrict__ tokens,
+                             float* __restrict__ x, int D, int V) {
+    const int t = blockIdx.x;
+    int tok = tokens[t];
+    tok = tok < 0 ? 0 : (tok >= V ? V - 1 : tok);      // ids are checked on the host; stay in bounds anyway
+    const TW* row = table + (size_t)tok * D;
+    float* out = x + (size_t)t * D;
+    for (int i = threadIdx.x; i < D; i += blockDim.x) out[i] = to_f32<TW>(row[i]);
+}
+
+extern "C" int picolm_embed(const void* table, int table_dt, const int32_t* tokens, float* x,
+                            int T, int D, int V, hipStream_t stream) {
+    PICOLM_REQUIRE(T >= 0 && D > 0 && V > 0, "embed: bad sizes T=%d D=%d V=%d", T, D, V);
+    if (T == 0) return 0;
+    dim3 grid(T), block(256);
+    if (table_dt == PICOLM_F32)
+        embed_kernel<float><<<grid, block, 0, stream>>>((const float*)table, tokens, x, D, V);
+    else if (table_dt == PICOLM_BF16)
+        embed_kernel<bf16_t><<<grid, block, 0, stream>>>((const bf16_t*)table, tokens, x, D, V);
+    else
+        PICOLM_REQUIRE(false, "embed: unknown table dtype %d", table_dt);
+    PICOLM_LAUNCH_CHECK("embed");
+    return 0;
+}
+
+// ---- RMSNorm ---------------------------------------------------------------------------
+// picolm/tensor.c:2942-3064: ss = sum x^2; r = 1/sqrtf(ss/size + eps); out = (x*r)*w.
+// `rows` (optional) selects which rows of x are normed; output row i is dense.
+template <typename TO>
+__global__ void rmsnorm_kernel(const float* __restrict__ x, const float* __restrict__ w,
+                               TO* __restrict__ out, const int32_t* __restrict__ rows, int D,
+                               float eps) {
+    __shared__ float scratch[16];
+    const int i = blockIdx.x;
+    const int r = rows ? rows[i] : i;
+    const float* xr = x + (size_t)r * D;
+    TO* o = out + (size_t)i * D;
+    float ss = 0.f;
+    for (int j = threadIdx.x; j < D; j += blockDim.x) {
+        float v = xr[j];
+        ss += v * v;
+    }
+    ss = block_sum(ss, scratch);
+    const float scale = 1.0f / sqrtf(ss / (float)D + eps);
+    for (int j = threadIdx.x; j < D; j += blockDim.x) o[j] = from_f32<TO>((xr[j] * scale) * w[j]);
+}
+
+extern "C" int picolm_rmsnorm(const float* x, const float* w, void* out, int out_dt,
+                              const int32_t* rows, int n_rows, int D, float eps,
+                              hipStream_t stream) {
+    PICOLM_REQUIRE(n_rows >= 0 && D > 0, "rmsnorm: bad sizes rows=%d D=%d", n_rows, D);
+    if (n_rows == 0) return 0;
+    dim3 grid(n_rows), block(D >= 2048 ? 512 : 256);
+    if (out_dt == PICOLM_F32)
+        rmsnorm_kernel<float><<<grid, block, 0, stream>>>(x, w, (float*)out, rows, D, eps);
+    else if (out_dt == PICOLM_BF16)
+        rmsnorm_kernel<bf16_t><<<grid, block, 0, stream>>>(x, w, (bf16_t*)out, rows, D, eps);
+    else
+        PICOLM_REQUIRE(false, "rmsnorm: unknown output dtype %d", out_dt);
+    PICOLM_LAUNCH_CHECK("rmsnorm");
+    return 0;
+}
+
+// ---- rotation of q and k, and the cache write of k and v ------------------------------------
+// picolm rotates every q and k head of a token by its position's table row before k is
+// cached and leaves v alone (picolm/model_core.c:1908, :2915; picolm/tensor.c:3216-3304).
+// style 0: pairs (2i, 2i+1); style 1: pairs (i, i + d/2).  cos/sin == null: no rotation.
+// A token's cache row is page_table[slot][(pos / PAGE) % ring_pages], offset pos % PAGE.
+template <typename TC>
+__global__ void rope_kv_store_kernel(const float* __restrict__ qkv, TC* __restrict__ q_out,
+                                     TC* __restrict__ k_pages, TC* __restrict__ v_pages,
+                                     const float* __restrict__ cos_t, const float* __restrict__ sin_t,
+                                     int style, const int32_t* __restrict__ tok_pos,
+                                     const int32_t* __restrict__ tok_seq,
+                                     const int32_t* __restrict__ seq_slot,
+                                     const int32_t* __restrict__ page_table, int max_pages,
+                                     int ring_pages, int H, int G, int d) {
+    const int t = blockIdx.x;
+    const int pos = tok_pos[t];
+    const int half = d / 2;
+    const float* row = qkv + (size_t)t * (H + 2 * G) * d;
+    const float* c = cos_t ? cos_t + (size_t)pos * half : nullptr;
+    const float* s = sin_t ? sin_t + (size_t)pos * half : nullptr;
+
+    size_t cache_row = 0;
+    if (k_pages) {
+        const int slot = seq_slot[tok_seq[t]];
+        const int page = page_table[(size_t)slot * max_pages + (pos / PAGE_TOKENS) % ring_pages];
+        cache_row = ((size_t)page * G) * PAGE_TOKENS * d + (size_t)(pos % PAGE_TOKENS) * d;
+    }
+    // rotations: heads 0..H-1 are q, H..H+G-1 are k
+    const int n_rot = (H + G) * half;
+    for (int idx = threadIdx.x; idx < n_rot; idx += blockDim.x) {
+        const int head = idx / half, i = idx % half;
+        const int i0 = style == 0 ? 2 * i : i;
+        const int i1 = style == 0 ? 2 * i + 1 : i + half;
+        const float x0 = row[head * d + i0], x1 = row[head * d + i1];
+        float y0 = x0, y1 = x1;
+        if (c) {
+            const float cc = c[i], ss = s[i];
+            y0 = x0 * cc - x1 * ss;
+            y1 = x0 * ss + x1 * cc;
+        }
+        if (head < H) {
+            TC* q = q_out + (size_t)t * H * d + head * d;
+            q[i0] = from_f32<TC>(y0);
+            q[i1] = from_f32<TC>(y1);
+        } else if (k_pages) {
+            TC* k = k_pages + cache_row + (size_t)(head - H) * PAGE_TOKENS * d;
+            k[i0] = from_f32<TC>(y0);
+            k[i1] = from_f32<TC>(y1);
+        }
+    }
+    if (v_pages) {
+        const float* vrow = row + (H + G) * d;
+        for (int idx = threadIdx.x; idx < G * d; idx += blockDim.x) {
+            const int g = idx / d, i = idx % d;
+            v_pages[cache_row + (size_t)g * PAGE_TOKENS * d + i] = from_f32<TC>(vrow[idx]);
+        }
+    }
+}
+
+extern "C" int picolm_rope_kv_store(const float* qkv, void* q_out, void* k_pages, void* v_pages,
+                                    int dt, const float* cos_t, const float* sin_t, int style,
+                                    const int32_t* tok_pos, const int32_t* tok_seq,
+                                    const int32_t* seq_slot, const int32_t* page_table,
+                                    int max_pages, int ring_pages, int T, int H, int G, int d,
+                                    hipStream_t stream) {
+    PICOLM_REQUIRE(T >= 0 && H > 0 && G > 0 && d > 0 && d % 2 == 0,
+                   "rope_kv_store: bad sizes T=%d H=%d G=%d d=%d", T, H, G, d);
+    PICOLM_REQUIRE((cos_t == nullptr) == (sin_t == nullptr), "rope_kv_store: need both tables or none");
+    PICOLM_REQUIRE((k_pages == nullptr) == (v_pages == nullptr), "rope_kv_store: need both caches or none");
+    PICOLM_REQUIRE(!k_pages || (max_pages > 0 && ring_pages > 0 && ring_pages <= max_pages),
+                   "rope_kv_store: bad page table geometry max_pages=%d ring_pages=%d", max_pages, ring_pages);
+    PICOLM_REQUIRE(style == 0 || style == 1, "rope_kv_store: unknown pairing %d", style);
+    if (T == 0) return 0;
+    dim3 grid(T), block(256);
+    if (dt == PICOLM_F32)
+        rope_kv_store_kernel<float><<<grid, block, 0, stream>>>(
+            qkv, (float*)q_out, (float*)k_pages, (float*)v_pages, cos_t, sin_t, style, tok_pos, tok_seq,
+            seq_slot, page_table, max_pages, ring_pages, H, G, d);
+    else if (dt == PICOLM_BF16)
+        rope_kv_store_kernel<bf16_t><<<grid, block, 0, stream>>>(
+            qkv, (bf16_t*)q_out, (bf16_t*)k_pages, (bf16_t*)v_pages, cos_t, sin_t, style, tok_pos, tok_seq,
+            seq_slot, page_table, max_pages, ring_pages, H, G, d);
+    else
+        PICOLM_REQUIRE(false, "rope_kv_store: unknown dtype %d", dt);
+    PICOLM_LAUNCH_CHECK("rope_kv_store");
+    return 0;
+}
+
+// ---- silu(gate) * up on separate or interleaved inputs ------------------------------------
+// picolm/tensor.c:3306-3315 and :3325: g/(1+expf(-g)) * u.  `gu` holds rows of 2F values with
+// gate j at 2j and up j at 2j+1.
+template <typename TI, typename TO>
+__global__ void silu_mul_kernel(const TI* __restrict__ gu, TO* __restrict__ out, int64_t n_pairs) {
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n_pairs) return;
+    const float g = to_f32<TI>(gu[2 * i]), u = to_f32<TI>(gu[2 * i + 1]);
+    out[i] = from_f32<TO>(g / (1.0f + expf(-g)) * u);
+}
+
+extern "C" int picolm_silu_mul(const void* gu, int in_dt, void* out, int out_dt, int64_t n_pairs,
+                               hipStream_t stream) {
+    if (n_pairs <= 0) return 0;
+    dim3 block(256), grid((unsigned)ceil_div64(n_pairs, 256));
+    if (in_dt == PICOLM_F32 && out_dt == PICOLM_F32)
+        silu_mul_kernel<float, float><<<grid, block, 0, stream>>>((const float*)gu, (float*)out, n_pairs);
+    else if (in_dt == PICOLM_F32 && out_dt == PICOLM_BF16)
+        silu_mul_kernel<float, bf16_t><<<grid, block, 0, stream>>>((const float*)gu, (bf16_t*)out, n_pairs);
+    else if (in_dt == PICOLM_BF16 && out_dt == PICOLM_BF16)
+        silu_mul_kernel<bf16_t, bf16_t><<<grid, block, 0, stream>>>((const bf16_t*)gu, (bf16_t*)out, n_pairs);
+    else
+        PICOLM_REQUIRE(false, "silu_mul: unsupported dtypes %d -> %d", in_dt, out_dt);
+    PICOLM_LAUNCH_CHECK("silu_mul");
+    return 0;
+}
+
+// ---- y += x (float residual) ---------------------------------------------------------------
+template <typename TI>
+__global__ void add_into_kernel(float* __restrict__ y, const TI* __restrict__ x, int64_t n) {
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) y[i] += to_f32<TI>(x[i]);
+}
+
+extern "C" int picolm_add_into(float* y, const void* x, int x_dt, int64_t n, hipStream_t stream) {
+    if (n <= 0) return 0;
+    dim3 block(256), grid((unsigned)ceil_div64(n, 256));
+    if (x_dt == PICOLM_F32)
+        add_into_kernel<float><<<grid, block, 0, stream>>>(y, (const float*)x, n);
+    else if (x_dt == PICOLM_BF16)
+        add_into_kernel<bf16_t><<<grid, block, 0, stream>>>(y, (const bf16_t*)x, n);
+    else
+        PICOLM_REQUIRE(false, "add_into: unknown dtype %d", x_dt);
+    PICOLM_LAUNCH_CHECK("add_into");
+    return 0;
+}

@@ -1,0 +1,241 @@
+"""Python face of libpicolm_hip.so: each function checks its operands on the host (device,
+dtype, shape, contiguity) and queues one hand-written gfx950 kernel on torch's current
+stream.  There is no fallback: a missing library or a CPU tensor is an error.
+"""
+from __future__ import annotations
+
+import ctypes
+from ctypes import c_float, c_int, c_int64, c_void_p
+
+import torch
+
+from .csrc import build as _build
+
+F32, BF16 = 0, 1
+PAGE_TOKENS = 64
+_DT = {torch.float32: F32, torch.bfloat16: BF16}
+
+EPI_STORE, EPI_ACCUMULATE, EPI_SWIGLU = 0, 1, 2
+
+
+class KernelError(RuntimeError):
+    pass
+
+
+_lib = None
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        l = _build.load()
+        l.picolm_last_error.restype = ctypes.c_char_p
+        for name in dir_entry_points():
+            getattr(l, name).restype = c_int
+        if l.picolm_abi_version() != 1:
+            raise KernelError("libpicolm_hip.so has another ABI version; rebuild it")
+        _lib = l
+    return _lib
+
+
+def dir_entry_points():
+    return ["picolm_abi_version", "picolm_device_check", "picolm_embed", "picolm_rmsnorm",
+            "picolm_rope_kv_store", "picolm_silu_mul", "picolm_add_into", "picolm_gemm_generic",
+            "picolm_attn_prefill_tile_rows", "picolm_attn_prefill_generic",
+            "picolm_attn_decode_generic", "picolm_argmax"]
+
+
+def _check(rc: int) -> None:
+    if rc != 0:
+        raise KernelError(lib().picolm_last_error().decode("utf-8", "replace"))
+
+
+def require_device() -> None:
+    """Fail loudly unless a gfx950 GPU and the kernel library are there."""
+    if not torch.cuda.is_available():
+        raise KernelError("no GPU: picolm_amd runs on an MI355X (gfx950) only and has no CPU path")
+    _check(lib().picolm_device_check())
+
+
+def _stream() -> c_void_p:
+    return c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _ptr(t: torch.Tensor | None) -> c_void_p:
+    return c_void_p(0) if t is None else c_void_p(t.data_ptr())
+
+
+def _dev(name: str, t: torch.Tensor, dtype=None, dim=None):
+    if not isinstance(t, torch.Tensor) or not t.is_cuda:
+        raise KernelError(f"{name}: expected a GPU tensor")
+    if not t.is_contiguous():
+        raise KernelError(f"{name}: expected a contiguous tensor")
+    if dtype is not None:
+        ok = t.dtype in dtype if isinstance(dtype, (tuple, list)) else t.dtype == dtype
+        if not ok:
+            raise KernelError(f"{name}: dtype {t.dtype} is not {dtype}")
+    if dim is not None and t.dim() != dim:
+        raise KernelError(f"{name}: expected {dim} dimensions, got {tuple(t.shape)}")
+    return t
+
+
+def _i32(name, t, n=None):
+    _dev(name, t, torch.int32)
+    if n is not None and t.numel() < n:
+        raise KernelError(f"{name}: holds {t.numel()} entries, {n} are needed")
+    return t
+
+
+def dt_of(t: torch.Tensor) -> int:
+    try:
+        return _DT[t.dtype]
+    except KeyError:
+        raise KernelError(f"dtype {t.dtype} is neither float32 nor bfloat16") from None
+
+
+# --------------------------------------------------------------------------------------------
+def embed(table: torch.Tensor, tokens: torch.Tensor, out: torch.Tensor) -> None:
+    _dev("embed.table", table, (torch.float32, torch.bfloat16), 2)
+    _i32("embed.tokens", tokens)
+    _dev("embed.out", out, torch.float32, 2)
+    T, D = out.shape
+    if table.shape[1] != D or tokens.numel() < T:
+        raise KernelError(f"embed: table {tuple(table.shape)}, tokens {tokens.numel()}, out {tuple(out.shape)} do not fit")
+    _check(lib().picolm_embed(_ptr(table), dt_of(table), _ptr(tokens), _ptr(out), T, D, table.shape[0], _stream()))
+
+
+def rmsnorm(x: torch.Tensor, weight: torch.Tensor, eps: float, out: torch.Tensor,
+            rows: torch.Tensor | None = None) -> None:
+    _dev("rmsnorm.x", x, torch.float32, 2)
+    _dev("rmsnorm.weight", weight, torch.float32, 1)
+    _dev("rmsnorm.out", out, (torch.float32, torch.bfloat16), 2)
+    D = x.shape[1]
+    n = out.shape[0]
+    if weight.numel() != D or out.shape[1] != D:
+        raise KernelError(f"rmsnorm: x {tuple(x.shape)}, weight {tuple(weight.shape)}, out {tuple(out.shape)} do not fit")
+    if rows is None:
+        if n > x.shape[0]:
+            raise KernelError("rmsnorm: more output rows than input rows")
+    else:
+        _i32("rmsnorm.rows", rows, n)
+    _check(lib().picolm_rmsnorm(_ptr(x), _ptr(weight), _ptr(out), dt_of(out), _ptr(rows), n, D,
+                                c_float(eps), _stream()))
+
+
+def rope_kv_store(qkv, q_out, k_pages, v_pages, cos, sin, style: int, tok_pos, tok_seq, seq_slot,
+                  page_table, ring_pages: int, H: int, G: int, d: int) -> None:
+    _dev("rope.qkv", qkv, torch.float32, 2)
+    T = qkv.shape[0]
+    if qkv.shape[1] != (H + 2 * G) * d:
+        raise KernelError(f"rope: qkv has {qkv.shape[1]} columns, (H+2G)d = {(H + 2 * G) * d}")
+    _dev("rope.q_out", q_out, (torch.float32, torch.bfloat16), 2)
+    if tuple(q_out.shape) != (T, H * d):
+        raise KernelError(f"rope: q_out {tuple(q_out.shape)} is not {(T, H * d)}")
+    max_pages = 1
+    if k_pages is not None:
+        for nm, p in (("k_pages", k_pages), ("v_pages", v_pages)):
+            _dev("rope." + nm, p, q_out.dtype, 4)
+            if tuple(p.shape[1:]) != (G, PAGE_TOKENS, d):
+                raise KernelError(f"rope: {nm} {tuple(p.shape)} is not [pages, {G}, {PAGE_TOKENS}, {d}]")
+        _dev("rope.page_table", page_table, torch.int32, 2)
+        max_pages = page_table.shape[1]
+        _i32("rope.seq_slot", seq_slot)
+    if cos is not None:
+        _dev("rope.cos", cos, torch.float32, 2)
+        _dev("rope.sin", sin, torch.float32, 2)
+        if cos.shape[1] != d // 2 or sin.shape != cos.shape:
+            raise KernelError(f"rope: tables {tuple(cos.shape)} do not have d/2 = {d // 2} columns")
+    _i32("rope.tok_pos", tok_pos, T)
+    _i32("rope.tok_seq", tok_seq, T)
+    _check(lib().picolm_rope_kv_store(
+        _ptr(qkv), _ptr(q_out), _ptr(k_pages), _ptr(v_pages), dt_of(q_out), _ptr(cos), _ptr(sin), style,
+        _ptr(tok_pos), _ptr(tok_seq), _ptr(seq_slot), _ptr(page_table), max_pages, ring_pages, T, H, G, d,
+        _stream()))
+
+
+def silu_mul(gu: torch.Tensor, out: torch.Tensor) -> None:
+    _dev("silu_mul.gu", gu, (torch.float32, torch.bfloat16))
+    _dev("silu_mul.out", out, (torch.float32, torch.bfloat16))
+    if gu.numel() != 2 * out.numel():
+        raise KernelError("silu_mul: input must hold two values per output")
+    _check(lib().picolm_silu_mul(_ptr(gu), dt_of(gu), _ptr(out), dt_of(out), c_int64(out.numel()), _stream()))
+
+
+def add_into(y: torch.Tensor, x: torch.Tensor) -> None:
+    _dev("add_into.y", y, torch.float32)
+    _dev("add_into.x", x, (torch.float32, torch.bfloat16))
+    if x.numel() != y.numel():
+        raise KernelError("add_into: sizes differ")
+    _check(lib().picolm_add_into(_ptr(y), _ptr(x), dt_of(x), c_int64(y.numel()), _stream()))
+
+
+def gemm_generic(a: torch.Tensor, w: torch.Tensor, c: torch.Tensor, epilogue: int = EPI_STORE) -> None:
+    """c = a @ w.T (store), c += a @ w.T (accumulate) or the gated form over interleaved rows of w."""
+    M, N, K = _gemm_shapes(a, w, c, epilogue)
+    _check(lib().picolm_gemm_generic(_ptr(a), dt_of(a), _ptr(w), dt_of(w), _ptr(c), dt_of(c), M, N, K,
+                                     c_int64(K), c_int64(K), c_int64(c.shape[1]), epilogue, _stream()))
+
+
+def _gemm_shapes(a, w, c, epilogue):
+    _dev("gemm.a", a, (torch.float32, torch.bfloat16), 2)
+    _dev("gemm.w", w, (torch.float32, torch.bfloat16), 2)
+    _dev("gemm.c", c, (torch.float32, torch.bfloat16), 2)
+    M, K = a.shape
+    N = w.shape[0]
+    n_out = N // 2 if epilogue == EPI_SWIGLU else N
+    if w.shape[1] != K or tuple(c.shape) != (M, n_out):
+        raise KernelError(f"gemm: a {tuple(a.shape)}, w {tuple(w.shape)}, c {tuple(c.shape)} do not fit (epilogue {epilogue})")
+    return M, N, K
+
+
+def attn_prefill_tile_rows() -> int:
+    return lib().picolm_attn_prefill_tile_rows()
+
+
+def attn_prefill_generic(q, k_pages, v_pages, out, tile_seq, tile_q0, n_tiles, seq_slot, seq_pos0,
+                         seq_nnew, cu_seqlens, page_table, ring_pages, H, G, d, window, scale) -> None:
+    _attn_check(q, k_pages, v_pages, out, page_table, H, G, d)
+    _i32("attn.tile_seq", tile_seq, n_tiles)
+    _i32("attn.tile_q0", tile_q0, n_tiles)
+    for nm, t in (("seq_slot", seq_slot), ("seq_pos0", seq_pos0), ("seq_nnew", seq_nnew), ("cu_seqlens", cu_seqlens)):
+        _i32("attn." + nm, t)
+    _check(lib().picolm_attn_prefill_generic(
+        _ptr(q), _ptr(k_pages), _ptr(v_pages), _ptr(out), dt_of(q), _ptr(tile_seq), _ptr(tile_q0), n_tiles,
+        _ptr(seq_slot), _ptr(seq_pos0), _ptr(seq_nnew), _ptr(cu_seqlens), _ptr(page_table),
+        page_table.shape[1], ring_pages, H, G, d, window, c_float(scale), _stream()))
+
+
+def attn_decode_generic(q, k_pages, v_pages, out, partial, n_seq, n_splits, seq_slot, seq_pos0,
+                        cu_seqlens, page_table, ring_pages, H, G, d, window, scale) -> None:
+    _attn_check(q, k_pages, v_pages, out, page_table, H, G, d)
+    if n_splits > 1:
+        _dev("attn.partial", partial, torch.float32)
+        if partial.numel() < n_seq * H * n_splits * (d + 2):
+            raise KernelError("attn_decode: the partial buffer is too small")
+    if q.shape[0] < n_seq:
+        raise KernelError("attn_decode: fewer query rows than sequences")
+    for nm, t in (("seq_slot", seq_slot), ("seq_pos0", seq_pos0), ("cu_seqlens", cu_seqlens)):
+        _i32("attn." + nm, t, n_seq)
+    _check(lib().picolm_attn_decode_generic(
+        _ptr(q), _ptr(k_pages), _ptr(v_pages), _ptr(out), _ptr(partial if n_splits > 1 else None), dt_of(q),
+        n_seq, n_splits, _ptr(seq_slot), _ptr(seq_pos0), _ptr(cu_seqlens), _ptr(page_table),
+        page_table.shape[1], ring_pages, H, G, d, window, c_float(scale), _stream()))
+
+
+def _attn_check(q, k_pages, v_pages, out, page_table, H, G, d):
+    _dev("attn.q", q, (torch.float32, torch.bfloat16), 2)
+    _dev("attn.out", out, q.dtype, 2)
+    if q.shape[1] != H * d or out.shape != q.shape:
+        raise KernelError(f"attn: q {tuple(q.shape)} / out {tuple(out.shape)} are not [T, {H * d}]")
+    for nm, p in (("k_pages", k_pages), ("v_pages", v_pages)):
+        _dev("attn." + nm, p, q.dtype, 4)
+        if tuple(p.shape[1:]) != (G, PAGE_TOKENS, d):
+            raise KernelError(f"attn: {nm} {tuple(p.shape)} is not [pages, {G}, {PAGE_TOKENS}, {d}]")
+    _dev("attn.page_table", page_table, torch.int32, 2)
+
+
+def argmax(logits: torch.Tensor, out: torch.Tensor) -> None:
+    _dev("argmax.logits", logits, torch.float32, 2)
+    _i32("argmax.out", out, logits.shape[0])
+    _check(lib().picolm_argmax(_ptr(logits), _ptr(out), logits.shape[0], logits.shape[1],
+                               c_int64(logits.shape[1]), _stream()))
