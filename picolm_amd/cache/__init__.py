@@ -1,0 +1,6 @@
+from .slots import PAGE_TOKENS, CacheError, CacheFull, PagedGroupBook, PagePool, SlotTable, pages_for
+from .kv import Cache, CacheSpec, KVGroup, KVGroupSpec, StateGroupSpec, window_ring_pages
+
+__all__ = ["PAGE_TOKENS", "CacheError", "CacheFull", "PagedGroupBook", "PagePool", "SlotTable",
+           "pages_for", "Cache", "CacheSpec", "KVGroup", "KVGroupSpec", "StateGroupSpec",
+           "window_ring_pages"]

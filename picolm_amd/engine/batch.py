@@ -1,0 +1,108 @@
+"""One step's description: which sequences run, where each stands, which tokens it brings
+and which rows' logits are wanted.  Built and checked on the host, sent to the GPU as one
+int32 block.
+
+The sequences of a step either all bring their first tokens (a prefill step; lengths may
+differ) or each bring one more token (a decode step).  picolm has the two as separate
+single-sequence functions (`model_forward_prefill`, `model_forward`, picolm/model.h:538-539);
+here they are one step over a batch, and tokens are packed without padding.
+"""
+from __future__ import annotations
+
+import numpy as np
+import torch
+
+from ..cache.slots import PAGE_TOKENS, pages_for
+
+
+class StepError(ValueError):
+    """A step that cannot run: a dead slot, a token outside the vocabulary, no room."""
+
+
+class StepBatch:
+    def __init__(self, slots, pos0, new_tokens, want, vocab_size: int, device, target_blocks: int = 1024):
+        """slots[i]: cache slot of sequence i; pos0[i]: tokens it holds; new_tokens[i]: its
+        next tokens; want[i]: indices into new_tokens[i] whose logits are asked for."""
+        self.n_seq = len(slots)
+        if self.n_seq == 0:
+            raise StepError("a step needs at least one sequence")
+        if not (len(pos0) == len(new_tokens) == len(want) == self.n_seq):
+            raise StepError("slots, positions, tokens and wanted rows differ in length")
+        if len(set(slots)) != self.n_seq:
+            raise StepError("a slot appears twice in one step")
+        n_new = [len(t) for t in new_tokens]
+        if min(n_new) < 1:
+            raise StepError("every sequence of a step brings at least one token")
+        self.slots = list(slots)
+        self.pos0 = [int(p) for p in pos0]
+        self.n_new = n_new
+        self.max_new = max(n_new)
+        self.T = sum(n_new)
+        self.is_decode = self.max_new == 1
+        self.max_len = max(p + n for p, n in zip(self.pos0, n_new))
+        self._target_blocks = target_blocks
+
+        cu = np.zeros(self.n_seq + 1, dtype=np.int32)
+        cu[1:] = np.cumsum(n_new)
+        tokens = np.concatenate([np.asarray(t, dtype=np.int64) for t in new_tokens])
+        if tokens.min() < 0 or tokens.max() >= vocab_size:
+            bad = int(tokens[(tokens < 0) | (tokens >= vocab_size)][0])
+            raise StepError(f"token id {bad} is outside the vocabulary of {vocab_size}")
+        tok_pos = np.concatenate([np.arange(p, p + n, dtype=np.int32) for p, n in zip(self.pos0, n_new)])
+        tok_seq = np.repeat(np.arange(self.n_seq, dtype=np.int32), n_new)
+        rows = []
+        for i, w in enumerate(want):
+            for j in w:
+                if not 0 <= j < n_new[i]:
+                    raise StepError(f"wanted row {j} of a sequence that brings {n_new[i]} tokens")
+                rows.append(int(cu[i]) + int(j))
+        self.n_want = len(rows)
+        self.want_counts = [len(w) for w in want]
+
+        parts = {
+            "seq_slot": np.asarray(self.slots, dtype=np.int32),
+            "seq_pos0": np.asarray(self.pos0, dtype=np.int32),
+            "seq_nnew": np.asarray(n_new, dtype=np.int32),
+            "cu_seqlens": cu,
+            "tok_pos": tok_pos,
+            "tok_seq": tok_seq,
+            "tokens": tokens.astype(np.int32),
+            "want_rows": np.asarray(rows, dtype=np.int32),
+        }
+        self._host = parts
+        self._device = torch.device(device)
+        self._upload(parts)
+        self._tiles = {}
+
+    def _upload(self, parts) -> None:
+        sizes = [max(len(v), 1) for v in parts.values()]
+        flat = np.zeros(sum(sizes), dtype=np.int32)
+        off = 0
+        spans = {}
+        for (k, v), n in zip(parts.items(), sizes):
+            flat[off:off + len(v)] = v
+            spans[k] = (off, n)
+            off += n
+        dev = torch.from_numpy(flat).to(self._device)
+        for k, (o, n) in spans.items():
+            setattr(self, k, dev[o:o + n])
+
+    # -- derived launch geometry ----------------------------------------------------------
+    def prefill_tiles(self, rows_per_tile: int):
+        """(tile_seq, tile_q0, n_tiles) on the device: tiles of `rows_per_tile` new tokens."""
+        if rows_per_tile not in self._tiles:
+            seqs, q0s = [], []
+            for i, n in enumerate(self.n_new):
+                for q0 in range(0, n, rows_per_tile):
+                    seqs.append(i)
+                    q0s.append(q0)
+            flat = torch.tensor(seqs + q0s, dtype=torch.int32).to(self._device)
+            self._tiles[rows_per_tile] = (flat[:len(seqs)], flat[len(seqs):], len(seqs))
+        return self._tiles[rows_per_tile]
+
+    def decode_splits(self, blocks_per_seq: int) -> int:
+        """How many slices of pages each sequence's decode attention is cut into, so that the
+        launch has about `target_blocks` workgroups."""
+        pages = pages_for(self.max_len)
+        want = max(1, self._target_blocks // max(1, self.n_seq * blocks_per_seq))
+        return max(1, min(want, pages))

@@ -1,0 +1,124 @@
+"""A decoder put together from parts, and its one step function.
+
+embedding -> the layer calls of `order` -> final norm on the wanted rows -> head
+(picolm/model_core.c:1785, :1799-2210, :2213, :2220).  `order` is data: a list of layer
+calls, each naming a block (a block may be named twice) and either owning a cache entry or
+reading the entry of an earlier call.  Cache groups are derived from what the mixers ask
+for: calls whose mixers need the same kind of keys and values (heads, head size, window)
+share a group and its storage, as picolm's kv_layer_map does for its one kind
+(picolm/model_core.c:668-681).
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass
+
+import torch
+
+from .. import kernels
+from ..cache import Cache, CacheSpec, KVGroupSpec, StateGroupSpec
+from ..parts.base import CacheBinding, Runtime, StepContext, Workspace
+from ..weights import WeightFetcher, check_specs
+from .batch import StepBatch, StepError
+
+
+@dataclass(frozen=True)
+class LayerCall:
+    block: int                          # index into the model's blocks
+    reads_cache_of: int | None = None   # index of an earlier call whose cache entry this one reads
+
+
+class DecoderModel:
+    def __init__(self, config, embedding, blocks, final_norm, head, order=None):
+        self.config = config
+        self.embedding = embedding
+        self.blocks = list(blocks)
+        self.final_norm = final_norm
+        self.head = head
+        order = list(range(len(self.blocks))) if order is None else list(order)
+        self.order = [c if isinstance(c, LayerCall) else LayerCall(int(c)) for c in order]
+        for i, c in enumerate(self.order):
+            if not 0 <= c.block < len(self.blocks):
+                raise ValueError(f"layer call {i} names block {c.block}, there are {len(self.blocks)}")
+            if c.reads_cache_of is not None and not 0 <= c.reads_cache_of < i:
+                raise ValueError(f"layer call {i} can only read the cache of an earlier call")
+        self.runtime: Runtime | None = None
+        self._plan_cache()
+
+    # -- structure --------------------------------------------------------------------------
+    def parts(self):
+        return [self.embedding, *self.blocks, self.final_norm, self.head]
+
+    def tensor_specs(self):
+        out, seen = [], set()
+        for p in self.parts():
+            for s in p.all_specs():
+                if s.name not in seen:
+                    seen.add(s.name)
+                    out.append(s)
+        return out
+
+    def _plan_cache(self) -> None:
+        kv_keys, state_keys = [], []
+        kv_counts, state_counts = [], []
+        self.bindings: list[CacheBinding] = []
+        for i, call in enumerate(self.order):
+            kv_req, st_req = self.blocks[call.block].mixer.cache_requests()
+            if call.reads_cache_of is not None:
+                src = self.bindings[call.reads_cache_of]
+                src_call = self.order[call.reads_cache_of]
+                if self.blocks[src_call.block].mixer.cache_requests() != (kv_req, st_req):
+                    raise ValueError(f"layer call {i} reads a cache of another shape than it needs")
+                self.bindings.append(CacheBinding(src.kv, src.state, writes=False))
+                continue
+            kv = st = None
+            if kv_req is not None:
+                if kv_req not in kv_keys:
+                    kv_keys.append(kv_req)
+                    kv_counts.append(0)
+                g = kv_keys.index(kv_req)
+                kv = (g, kv_counts[g])
+                kv_counts[g] += 1
+            if st_req is not None:
+                if st_req not in state_keys:
+                    state_keys.append(st_req)
+                    state_counts.append(0)
+                g = state_keys.index(st_req)
+                st = (g, state_counts[g])
+                state_counts[g] += 1
+            self.bindings.append(CacheBinding(kv, st, writes=True))
+        self.cache_spec = CacheSpec(
+            [KVGroupSpec(n, k.n_kv_heads, k.head_dim, k.window) for k, n in zip(kv_keys, kv_counts)],
+            [StateGroupSpec(n, tuple(k.shape), k.dtype) for k, n in zip(state_keys, state_counts)])
+
+    # -- weights ----------------------------------------------------------------------------
+    def load(self, source, runtime: Runtime) -> "DecoderModel":
+        """Check `source` against every declared tensor, then bind."""
+        kernels.require_device()
+        check_specs(source, self.tensor_specs())
+        self.runtime = runtime
+        fetch = WeightFetcher(source, runtime.device)
+        for p in self.parts():
+            p.load_all(fetch, runtime)
+        return self
+
+    def new_cache(self, max_tokens: int, max_seq_len: int | None = None, n_slots: int | None = None) -> Cache:
+        limit = getattr(self.config, "max_position_embeddings", None) or max_tokens
+        max_seq_len = min(max_seq_len or limit, limit)
+        cache = Cache(self.cache_spec, max_tokens, max_seq_len, self.runtime.dtype, self.runtime.device, n_slots)
+        for b in self.blocks:
+            b.mixer.prepare(self.runtime, cache.max_seq_len)
+        return cache
+
+    # -- the step ---------------------------------------------------------------------------
+    def step(self, cache: Cache, batch: StepBatch, workspace: Workspace) -> torch.Tensor:
+        """Run the batch's new tokens from the cache; logits [n_want, vocab] float32, a view
+        of workspace memory valid until the next step."""
+        ctx = StepContext(self.runtime, batch, cache, workspace)
+        x = self.embedding.forward(ctx, batch.tokens, batch.T)
+        for call, binding in zip(self.order, self.bindings):
+            ctx.binding = binding
+            self.blocks[call.block].forward(ctx, x)
+        if batch.n_want == 0:
+            return workspace.get("logits", (0, self.head.V), torch.float32)
+        h = self.final_norm.forward(ctx, x, rows=batch.want_rows, n_rows=batch.n_want, out_name="norm.final")
+        return self.head.forward(ctx, h)

@@ -239,3 +239,22 @@ def argmax(logits: torch.Tensor, out: torch.Tensor) -> None:
     _i32("argmax.out", out, logits.shape[0])
     _check(lib().picolm_argmax(_ptr(logits), _ptr(out), logits.shape[0], logits.shape[1],
                                c_int64(logits.shape[1]), _stream()))
+
+
+def gemm(a: torch.Tensor, w: torch.Tensor, c: torch.Tensor, epilogue: int = EPI_STORE) -> None:
+    """The product the engine calls: picks the kernel for the operands' types and sizes."""
+    gemm_generic(a, w, c, epilogue)
+
+
+def attn_prefill(q, k_pages, v_pages, out, batch, page_table, ring_pages, H, G, d, window, scale) -> None:
+    """Attention of a step's new tokens over their sequences' cache pages."""
+    tile_seq, tile_q0, n_tiles = batch.prefill_tiles(attn_prefill_tile_rows())
+    attn_prefill_generic(q, k_pages, v_pages, out, tile_seq, tile_q0, n_tiles, batch.seq_slot, batch.seq_pos0,
+                         batch.seq_nnew, batch.cu_seqlens, page_table, ring_pages, H, G, d, window, scale)
+
+
+def attn_decode(q, k_pages, v_pages, out, partial, n_seq, n_splits, seq_slot, seq_pos0, cu_seqlens,
+                page_table, ring_pages, H, G, d, window, scale) -> None:
+    """Attention of one new token per sequence over its cache pages."""
+    attn_decode_generic(q, k_pages, v_pages, out, partial, n_seq, n_splits, seq_slot, seq_pos0, cu_seqlens,
+                        page_table, ring_pages, H, G, d, window, scale)

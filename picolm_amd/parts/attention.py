@@ -1,0 +1,77 @@
+"""Causal attention over the cache with grouped KV heads, an optional window, and any
+position encoding.
+
+picolm's order (picolm/model_core.c:1849-2151): q, k, v = W x (no bias); rotate q and k;
+write k, v to the cache; per query head h, KV head h // (H/G), online softmax of
+(q.k)/sqrt(d) over keys t <= pos (picolm/model_attention.c:43-140); output projection; add
+into the residual.  q, k and v come from one product over the stacked weights; the
+projection back adds into the residual inside the product's epilogue.
+"""
+from __future__ import annotations
+
+import math
+
+from .. import kernels
+from ..cache.slots import PAGE_TOKENS
+from .base import KVRequest, Mixer, Runtime, StepContext
+from .linear import Linear
+from .position import NoPosition, PositionEncoding
+import torch
+
+
+class Attention(Mixer):
+    def __init__(self, prefix: str, hidden_size: int, n_heads: int, n_kv_heads: int, head_dim: int,
+                 position: PositionEncoding | None = None, window: int = 0, scale: float | None = None,
+                 names=("q_proj.weight", "k_proj.weight", "v_proj.weight", "o_proj.weight")):
+        if n_heads % n_kv_heads:
+            raise ValueError(f"{n_heads} heads do not split over {n_kv_heads} KV heads")
+        if head_dim % 16 or not 16 <= head_dim <= 256:
+            raise ValueError(f"head size {head_dim}: the attention kernels take multiples of 16 up to 256")
+        self.H, self.G, self.d = n_heads, n_kv_heads, head_dim
+        self.window = int(window)
+        self.scale = float(scale) if scale is not None else 1.0 / math.sqrt(head_dim)   # model_core.c:2077
+        self.position = position or NoPosition()
+        self.qkv = Linear([prefix + n for n in names[:3]],
+                          [n_heads * head_dim, n_kv_heads * head_dim, n_kv_heads * head_dim], hidden_size)
+        self.o = Linear([prefix + names[3]], [hidden_size], n_heads * head_dim)
+
+    def children(self):
+        return [self.qkv, self.o, self.position]
+
+    def cache_requests(self):
+        return KVRequest(self.G, self.d, self.window), None
+
+    def prepare(self, runtime: Runtime, max_positions: int) -> None:
+        self.position.prepare(runtime, max_positions)
+
+    def forward(self, ctx: StepContext, h, residual) -> None:
+        b = ctx.batch
+        H, G, d = self.H, self.G, self.d
+        T = h.shape[0]
+        qkv = ctx.ws.get("attn.qkv", (T, (H + 2 * G) * d), torch.float32)
+        self.qkv.forward(h, qkv)
+        k_pages, v_pages, table, ring = ctx.kv()
+        tables = self.position.rotary_tables()
+        if tables is None:
+            self.position.apply(ctx, qkv, H, G, d)
+            cos = sin = None
+            style = 0
+        else:
+            cos, sin, style = tables
+        q = ctx.ws.get("attn.q", (T, H * d), ctx.dtype)
+        writes = ctx.binding.writes
+        kernels.rope_kv_store(qkv, q, k_pages if writes else None, v_pages if writes else None, cos, sin,
+                              style, b.tok_pos, b.tok_seq, b.seq_slot, table, ring, H, G, d)
+        out = ctx.ws.get("attn.out", (T, H * d), ctx.dtype)
+        if b.is_decode:
+            n_splits = b.decode_splits(G * ((H // G + 15) // 16))
+            partial = ctx.ws.get("attn.partial", (b.n_seq * H * n_splits * (d + 2),), torch.float32) \
+                if n_splits > 1 else None
+            kernels.attn_decode(q, k_pages, v_pages, out, partial, b.n_seq, n_splits, b.seq_slot, b.seq_pos0,
+                                b.cu_seqlens, table, ring, H, G, d, self.window, self.scale)
+        else:
+            if self.window > 0 and b.max_new > (ring - 1) * PAGE_TOKENS - self.window + 1 and ring < table.shape[1]:
+                raise kernels.KernelError(
+                    f"a step of {b.max_new} tokens overruns the ring of a window of {self.window} keys")
+            kernels.attn_prefill(q, k_pages, v_pages, out, b, table, ring, H, G, d, self.window, self.scale)
+        self.o.forward(out, residual, kernels.EPI_ACCUMULATE)

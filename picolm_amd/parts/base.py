@@ -1,0 +1,167 @@
+"""What every part of a layer is: something that declares its tensors and its cache needs,
+loads them, and acts on rows of a step.  No part knows which model it is in; its sizes and
+constants are constructor parameters (picolm passes them as arguments too:
+`rmsnorm(..., eps)` picolm/tensor.h:92, `rope(..., rope_type, half)` :102).
+
+Interfaces
+  Norm.forward(ctx, x[T,D] float32, rows=None)   -> h[n,D] in the compute dtype
+  PositionEncoding.rotary_tables(ctx)            -> (cos, sin, style) or None, and
+  PositionEncoding.apply(ctx, qkv, H, G, d)      in place, when it is not a rotation
+  Mixer.forward(ctx, h[T,D], residual[T,D] f32)  adds its output into `residual`
+  FeedForward.forward(ctx, h, residual)          adds its output into `residual`
+  Block.forward(ctx, x[T,D] f32)                 the arrangement of the four above
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass
+
+import torch
+
+from ..weights import TensorSpec
+
+
+@dataclass
+class Runtime:
+    """Where and in which precision a model runs."""
+    device: torch.device
+    dtype: torch.dtype              # torch.bfloat16: serving precision; torch.float32: true 32-bit
+
+    @property
+    def is_f32(self) -> bool:
+        return self.dtype == torch.float32
+
+
+class Workspace:
+    """Named scratch buffers that grow to the largest request and are reused by every
+    layer; nothing is allocated in a step whose sizes were seen before."""
+
+    def __init__(self, device):
+        self.device = device
+        self._bufs: dict[str, torch.Tensor] = {}
+
+    def get(self, name: str, shape, dtype: torch.dtype) -> torch.Tensor:
+        n = 1
+        for s in shape:
+            n *= int(s)
+        nbytes = n * torch.empty((), dtype=dtype).element_size()
+        buf = self._bufs.get(name)
+        if buf is None or buf.numel() < nbytes:
+            buf = torch.empty(max(nbytes, 256), dtype=torch.uint8, device=self.device)
+            self._bufs[name] = buf
+        return buf[:nbytes].view(dtype).view(*shape)
+
+    def bytes(self) -> int:
+        return sum(b.numel() for b in self._bufs.values())
+
+
+@dataclass(frozen=True)
+class KVRequest:
+    """A mixer's need for keys and values of each token."""
+    n_kv_heads: int
+    head_dim: int
+    window: int = 0
+
+
+@dataclass(frozen=True)
+class StateRequest:
+    """A mixer's need for a fixed-size tensor per sequence."""
+    shape: tuple
+    dtype: torch.dtype = torch.float32
+
+
+@dataclass
+class CacheBinding:
+    """Where one layer call finds its cache: (group, entry) for each of its requests, and
+    whether this call writes the entries or reads another call's."""
+    kv: tuple | None = None          # (group index, entry index)
+    state: tuple | None = None
+    writes: bool = True
+
+
+class StepContext:
+    """What a part sees of the step it runs in."""
+
+    def __init__(self, runtime: Runtime, batch, cache, workspace: Workspace):
+        self.runtime = runtime
+        self.batch = batch
+        self.cache = cache
+        self.ws = workspace
+        self.binding: CacheBinding | None = None
+
+    @property
+    def dtype(self) -> torch.dtype:
+        return self.runtime.dtype
+
+    def kv(self):
+        """(k_pages, v_pages, page_table, ring_pages) of the running layer call."""
+        gi, e = self.binding.kv
+        g = self.cache.kv[gi]
+        return g.k[e], g.v[e], g.table, g.ring_pages
+
+    def state(self) -> torch.Tensor:
+        """[n_slots, ...] state of the running layer call; index it with batch.seq_slot."""
+        gi, e = self.binding.state
+        return self.cache.state[gi][e]
+
+
+class Part:
+    def tensor_specs(self) -> list[TensorSpec]:
+        return []
+
+    def load(self, fetch, runtime: Runtime) -> None:
+        pass
+
+    def children(self) -> list["Part"]:
+        return []
+
+    def all_specs(self) -> list[TensorSpec]:
+        out = list(self.tensor_specs())
+        for c in self.children():
+            out.extend(c.all_specs())
+        return out
+
+    def load_all(self, fetch, runtime: Runtime) -> None:
+        self.load(fetch, runtime)
+        for c in self.children():
+            c.load_all(fetch, runtime)
+
+
+class Norm(Part):
+    def forward(self, ctx: StepContext, x: torch.Tensor, rows: torch.Tensor | None = None,
+                n_rows: int | None = None) -> torch.Tensor:
+        raise NotImplementedError
+
+
+class PositionEncoding(Part):
+    def prepare(self, runtime: Runtime, max_positions: int) -> None:
+        pass
+
+    def rotary_tables(self):
+        return None
+
+    def apply(self, ctx: StepContext, qkv: torch.Tensor, n_heads: int, n_kv_heads: int, head_dim: int) -> None:
+        pass
+
+
+class Mixer(Part):
+    def cache_requests(self) -> tuple:
+        """(KVRequest | None, StateRequest | None)"""
+        return (None, None)
+
+    def prepare(self, runtime: Runtime, max_positions: int) -> None:
+        pass
+
+    def forward(self, ctx: StepContext, h: torch.Tensor, residual: torch.Tensor) -> None:
+        raise NotImplementedError
+
+
+class FeedForward(Part):
+    def forward(self, ctx: StepContext, h: torch.Tensor, residual: torch.Tensor) -> None:
+        raise NotImplementedError
+
+
+class Block(Part):
+    mixer: Mixer
+
+    def forward(self, ctx: StepContext, x: torch.Tensor) -> None:
+        raise NotImplementedError

@@ -1,0 +1,52 @@
+"""Token embedding and the output head.  x = table[token] widened to float, no scaling
+(picolm/model_core.c:1785-1786); logits = W_out h, where W_out is the embedding table when
+the checkpoint has no `lm_head.weight` (picolm/safetensors.c:248-251) or the configuration
+ties them."""
+from __future__ import annotations
+
+import torch
+
+from .. import kernels
+from ..weights import TensorSpec
+from .base import Part, Runtime, StepContext
+
+
+class TokenEmbedding(Part):
+    def __init__(self, name: str, vocab_size: int, hidden_size: int):
+        self.name, self.V, self.D = name, vocab_size, hidden_size
+        self.table = None
+
+    def tensor_specs(self):
+        return [TensorSpec(self.name, (self.V, self.D))]
+
+    def load(self, fetch, runtime: Runtime) -> None:
+        t = fetch.get(self.name)
+        self.table = (t.to(torch.float32) if runtime.is_f32 else t).contiguous()
+
+    def forward(self, ctx: StepContext, tokens: torch.Tensor, n_tokens: int) -> torch.Tensor:
+        x = ctx.ws.get("residual", (n_tokens, self.D), torch.float32)
+        kernels.embed(self.table, tokens, x)
+        return x
+
+
+class LMHead(Part):
+    def __init__(self, name: str, vocab_size: int, hidden_size: int, embedding: TokenEmbedding, tied: bool):
+        self.name, self.V, self.D, self.embedding, self.tied = name, vocab_size, hidden_size, embedding, tied
+        self.weight = None
+
+    def tensor_specs(self):
+        # optional either way: absent -> the embedding table serves; a tied model's stray
+        # copy is ignored
+        return [TensorSpec(self.name, (self.V, self.D), optional=True, init=None if self.tied else "normal")]
+
+    def load(self, fetch, runtime: Runtime) -> None:
+        if self.tied or not fetch.has(self.name):
+            self.weight = self.embedding.table
+        else:
+            t = fetch.get(self.name)
+            self.weight = (t.to(torch.float32) if runtime.is_f32 else t).contiguous()
+
+    def forward(self, ctx: StepContext, h: torch.Tensor) -> torch.Tensor:
+        logits = ctx.ws.get("logits", (h.shape[0], self.V), torch.float32)
+        kernels.gemm(h, self.weight, logits, kernels.EPI_STORE)
+        return logits

@@ -1,0 +1,25 @@
+"""Gated feed-forward: down(silu(gate x) * (up x)), no bias (picolm/model_core.c:2182-2204,
+silu picolm/tensor.c:3306-3315).  gate and up are one product over row-interleaved weights
+whose epilogue applies silu(g) * u; the down product adds into the residual."""
+from __future__ import annotations
+
+from .. import kernels
+from .base import FeedForward, StepContext
+from .linear import Linear
+
+
+class SwiGLU(FeedForward):
+    def __init__(self, prefix: str, hidden_size: int, intermediate_size: int,
+                 names=("gate_proj.weight", "up_proj.weight", "down_proj.weight")):
+        self.D, self.F = hidden_size, intermediate_size
+        self.gate_up = Linear([prefix + names[0], prefix + names[1]], [intermediate_size] * 2, hidden_size,
+                              interleave=True)
+        self.down = Linear([prefix + names[2]], [hidden_size], intermediate_size)
+
+    def children(self):
+        return [self.gate_up, self.down]
+
+    def forward(self, ctx: StepContext, h, residual) -> None:
+        act = ctx.ws.get("ffn.act", (h.shape[0], self.F), ctx.dtype)
+        self.gate_up.forward(h, act, kernels.EPI_SWIGLU)
+        self.down.forward(act, residual, kernels.EPI_ACCUMULATE)
