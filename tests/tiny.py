@@ -1,0 +1,73 @@
+"""The tiny configurations the tests use, their random model folders, and helpers that run
+the plain implementation on them.  The two configurations differ in every size and option:
+head counts and grouping, widths that are no power of two, layers, vocabulary, eps, rope
+base and scaling, pairing style, tied or separate head, weight spread."""
+from __future__ import annotations
+
+import json
+import os
+
+import numpy as np
+
+TINY_A = dict(
+    architectures=["LlamaForCausalLM"], hidden_size=64, intermediate_size=176, num_attention_heads=4,
+    num_key_value_heads=2, num_hidden_layers=2, vocab_size=256, head_dim=16, rms_norm_eps=1e-5,
+    rope_theta=10000.0, rope_scaling=None, tie_word_embeddings=True, max_position_embeddings=128,
+    eos_token_id=2, rope_style="pairwise")
+TINY_A_WEIGHTS = dict(seed=0, std=0.02, norm_sigma=0.0)
+
+TINY_B = dict(
+    architectures=["LlamaForCausalLM"], hidden_size=96, intermediate_size=256, num_attention_heads=6,
+    num_key_value_heads=6, num_hidden_layers=3, vocab_size=384, head_dim=16, rms_norm_eps=1e-6,
+    rope_theta=500000.0,
+    rope_scaling=dict(rope_type="llama3", factor=8.0, low_freq_factor=1.0, high_freq_factor=4.0,
+                      original_max_position_embeddings=64),
+    tie_word_embeddings=False, max_position_embeddings=256, eos_token_id=[3, 7], rope_style="half")
+TINY_B_WEIGHTS = dict(seed=1, std=0.05, norm_sigma=0.1)
+
+# a third one for the sizes the other two share: head size 32 (48 heads*dim != hidden), GQA 3:1,
+# odd layer count, a vocabulary that is no multiple of anything
+TINY_C = dict(
+    architectures=["LlamaForCausalLM"], hidden_size=80, intermediate_size=112, num_attention_heads=3,
+    num_key_value_heads=1, num_hidden_layers=1, vocab_size=131, head_dim=32, rms_norm_eps=1e-4,
+    rope_theta=1000.0, rope_scaling=None, tie_word_embeddings=False, max_position_embeddings=512,
+    eos_token_id=5, rope_style="pairwise")
+TINY_C_WEIGHTS = dict(seed=2, std=0.08, norm_sigma=0.2)
+
+CONFIGS = {"A": (TINY_A, TINY_A_WEIGHTS), "B": (TINY_B, TINY_B_WEIGHTS), "C": (TINY_C, TINY_C_WEIGHTS)}
+
+
+def make_model_dir(tmp_path, which: str, dtype: str = "bfloat16") -> str:
+    from picolm_amd import LlamaConfig, write_random_model
+    cfg_dict, w = CONFIGS[which]
+    cfg = LlamaConfig.from_dict(cfg_dict)
+    out = os.path.join(str(tmp_path), f"tiny_{which}_{dtype}")
+    if not os.path.exists(os.path.join(out, "model.safetensors")):
+        write_random_model(cfg, out, dtype=dtype, **w)
+    return out
+
+
+def read_weights_f64(model_dir: str) -> dict:
+    """The folder's tensors as float64 arrays, read with the safetensors package (not with
+    the engine's own reader)."""
+    import torch
+    from safetensors import safe_open
+    out = {}
+    with safe_open(os.path.join(model_dir, "model.safetensors"), framework="pt") as f:
+        for k in f.keys():
+            out[k] = f.get_tensor(k).to(torch.float64).numpy()
+    return out
+
+
+def read_config(model_dir: str) -> dict:
+    with open(os.path.join(model_dir, "config.json")) as f:
+        return json.load(f)
+
+
+def plain_logits(model_dir: str, tokens) -> np.ndarray:
+    from plain import llama_plain as P
+    return P.forward(read_weights_f64(model_dir), read_config(model_dir), tokens)
+
+
+def random_tokens(rng: np.random.Generator, n: int, vocab: int) -> list[int]:
+    return [int(t) for t in rng.integers(0, vocab, size=n)]
