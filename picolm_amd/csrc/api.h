@@ -46,6 +46,11 @@ int picolm_attn_decode_generic(const void* q, const void* k_pages, const void* v
 
 int picolm_argmax(const float* logits, int32_t* out, int n_rows, int V, int64_t ld,
                   hipStream_t stream);
+// rng_states[state_index ? state_index[row] : row] is one xorshift64 state per sequence,
+// advanced by one draw when temperature > 0.
+int picolm_sample(const float* logits, int64_t ld, int n_rows, int V, float temperature, int top_k,
+                  float top_p, float min_p, uint64_t* rng_states, const int32_t* state_index,
+                  int32_t* out, hipStream_t stream);
 
 #ifdef __cplusplus
 }

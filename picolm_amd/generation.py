@@ -1,0 +1,189 @@
+"""The generation loop: prompts in one step, then sample / record / stop? / one more token
+(picolm/picolm.c:1502-1610), over batches of unequal prompts.
+
+Differences from picolm's loop, all deliberate: exactly `max_new_tokens` tokens are produced
+(picolm's bound runs one over, picolm/picolm.c:1496-1500, :1539); a stop token is recorded
+and ends its sequence (picolm/picolm.c:1574); a sequence also ends at the cache's capacity;
+sequences that end leave the batch and the others go on unchanged; when all of a batch have
+ended its slots are released and the next batch starts in them.
+
+The loop only decides; it never looks inside logits.  `stepper` needs begin(n) -> slots,
+step(slots, tokens) -> logits rows, release(slots), `capacity` (longest sequence) and
+fits(lengths) -> bool; `make_sampler(n)` returns an object with sample(logits, indices).
+"""
+from __future__ import annotations
+
+import time
+from dataclasses import dataclass, field
+
+from .sampling.params import SamplingParams
+
+
+@dataclass
+class Generated:
+    tokens: list = field(default_factory=list)
+    finish: str = ""          # "stop", "length" or "capacity"
+
+
+@dataclass
+class GenerationStats:
+    prompt_tokens: int = 0
+    prefill_seconds: float = 0.0
+    generated_tokens: int = 0
+    decode_seconds: float = 0.0
+    batches: int = 0
+    steps: int = 0
+
+
+class GenerationLoop:
+    def __init__(self, stepper, make_sampler, stop_ids=(), batch_size: int = 64, clock=time.perf_counter,
+                 sync=None):
+        self.stepper = stepper
+        self.make_sampler = make_sampler
+        self.stop_ids = frozenset(int(s) for s in stop_ids)
+        self.batch_size = max(1, int(batch_size))
+        self.clock = clock
+        self.sync = sync or (lambda: None)
+        self.stats = GenerationStats()
+
+    def _admit(self, prompts, first: int, max_new_tokens: int) -> int:
+        """How many requests from `first` on form the next batch."""
+        n = 0
+        lengths = []
+        while first + n < len(prompts) and n < self.batch_size:
+            need = min(len(prompts[first + n]) + max_new_tokens, self.stepper.capacity)
+            if not self.stepper.fits(lengths + [need]):
+                break
+            lengths.append(need)
+            n += 1
+        if n == 0:
+            raise ValueError(f"request {first} ({len(prompts[first])} prompt tokens, {max_new_tokens} new) "
+                             "does not fit the cache even alone")
+        return n
+
+    def run(self, prompts, max_new_tokens: int, on_token=None) -> list[Generated]:
+        for i, p in enumerate(prompts):
+            if len(p) == 0:
+                raise ValueError(f"request {i} has an empty prompt; give at least a start token")
+            if len(p) > self.stepper.capacity:
+                raise ValueError(f"request {i} has {len(p)} prompt tokens, the cache takes {self.stepper.capacity}")
+        results = [Generated() for _ in prompts]
+        sampler = self.make_sampler(len(prompts))
+        first = 0
+        while first < len(prompts):
+            n = self._admit(prompts, first, max_new_tokens)
+            self._run_batch(prompts, list(range(first, first + n)), results, sampler, max_new_tokens, on_token)
+            first += n
+            self.stats.batches += 1
+        return results
+
+    def _run_batch(self, prompts, ids, results, sampler, max_new_tokens, on_token) -> None:
+        st = self.stepper
+        slots = st.begin(len(ids))
+        slot_of = dict(zip(ids, slots))
+        length = {i: len(prompts[i]) for i in ids}
+        try:
+            if max_new_tokens <= 0:
+                for i in ids:
+                    results[i].finish = "length"
+                return
+            t0 = self.clock()
+            logits = st.step(slots, [list(prompts[i]) for i in ids])
+            self.sync()
+            self.stats.prefill_seconds += self.clock() - t0
+            self.stats.prompt_tokens += sum(length.values())
+            self.stats.steps += 1
+            live = list(ids)
+            t0 = self.clock()
+            while live:
+                tokens = sampler.sample(logits, live)
+                nxt = []
+                for i, tok in zip(live, tokens):
+                    tok = int(tok)
+                    results[i].tokens.append(tok)
+                    self.stats.generated_tokens += 1
+                    if on_token:
+                        on_token(i, tok)
+                    if tok in self.stop_ids:
+                        results[i].finish = "stop"
+                    elif len(results[i].tokens) >= max_new_tokens:
+                        results[i].finish = "length"
+                    elif length[i] + 1 > st.capacity:
+                        results[i].finish = "capacity"
+                    else:
+                        nxt.append(i)
+                # sequences that ended give their slots back at once; the rest go on
+                ended = [i for i in live if i not in set(nxt)]
+                if ended:
+                    st.release([slot_of.pop(i) for i in ended])
+                live = nxt
+                if not live:
+                    break
+                logits = st.step([slot_of[i] for i in live], [[results[i].tokens[-1]] for i in live])
+                self.stats.steps += 1
+                for i in live:
+                    length[i] += 1
+            self.sync()
+            self.stats.decode_seconds += self.clock() - t0
+        finally:
+            if slot_of:
+                st.release(list(slot_of.values()))
+
+
+# ---------------------------------------------------------------------------------------------
+def generate(model_or_session, prompts, max_new_tokens: int = 256, params: SamplingParams | None = None,
+             stop_ids=None, batch_size: int = 64, max_tokens: int | None = None, on_token=None,
+             return_stats: bool = False):
+    """The Python entry point: token ids in, generated token ids out.
+
+    `model_or_session`: a loaded model (a session sized for the work is made) or a Session.
+    `prompts`: a list of token-id lists.  `stop_ids`: default, the configuration's
+    eos_token_id.  Returns one `Generated` per prompt (and the timing record on request).
+    """
+    import torch
+
+    from .cache.slots import PAGE_TOKENS, pages_for
+    from .engine.session import Session
+    from .sampling.sampler import Sampler
+    params = params or SamplingParams()
+    prompts = [list(p) for p in prompts]
+    if isinstance(model_or_session, Session):
+        session = model_or_session
+    else:
+        if max_tokens is None:
+            per = sorted((pages_for(len(p) + max_new_tokens) for p in prompts), reverse=True)
+            max_tokens = max(1, sum(per[:batch_size])) * PAGE_TOKENS
+        session = Session(model_or_session, max_tokens=max_tokens)
+    if stop_ids is None:
+        stop_ids = getattr(session.model.config, "eos_token_ids", ())
+    device = session.model.runtime.device
+    loop = GenerationLoop(SessionStepper(session), lambda n: Sampler(params, n, device), stop_ids, batch_size,
+                          sync=lambda: torch.cuda.synchronize(device))
+    out = loop.run(prompts, max_new_tokens, on_token)
+    return (out, loop.stats) if return_stats else out
+
+
+class SessionStepper:
+    """The face of a Session that the loop needs."""
+
+    def __init__(self, session):
+        self.session = session
+        self.capacity = session.cache.max_seq_len
+
+    def begin(self, n):
+        return self.session.begin(n)
+
+    def step(self, slots, tokens):
+        return self.session.step(slots, tokens)
+
+    def release(self, slots):
+        self.session.release(slots)
+
+    def fits(self, lengths) -> bool:
+        from .cache.slots import PAGE_TOKENS
+        from .cache.slots import pages_for
+        c = self.session.cache
+        if len(lengths) > c.slots.n_free:
+            return False
+        need = sum(pages_for(n) for n in lengths)
+        return need * PAGE_TOKENS <= c.free_tokens()

@@ -42,7 +42,7 @@ def dir_entry_points():
     return ["picolm_abi_version", "picolm_device_check", "picolm_embed", "picolm_rmsnorm",
             "picolm_rope_kv_store", "picolm_silu_mul", "picolm_add_into", "picolm_gemm_generic",
             "picolm_attn_prefill_tile_rows", "picolm_attn_prefill_generic",
-            "picolm_attn_decode_generic", "picolm_argmax"]
+            "picolm_attn_decode_generic", "picolm_argmax", "picolm_sample"]
 
 
 def _check(rc: int) -> None:
@@ -258,3 +258,19 @@ def attn_decode(q, k_pages, v_pages, out, partial, n_seq, n_splits, seq_slot, se
     """Attention of one new token per sequence over its cache pages."""
     attn_decode_generic(q, k_pages, v_pages, out, partial, n_seq, n_splits, seq_slot, seq_pos0, cu_seqlens,
                         page_table, ring_pages, H, G, d, window, scale)
+
+
+def sample(logits: torch.Tensor, out: torch.Tensor, temperature: float, top_k: int, top_p: float,
+           min_p: float, rng_states: torch.Tensor | None, state_index: torch.Tensor | None) -> None:
+    """One token per row of `logits`; `rng_states` (int64 bits of xorshift64 states) advance."""
+    _dev("sample.logits", logits, torch.float32, 2)
+    n, V = logits.shape
+    _i32("sample.out", out, n)
+    if temperature > 0:
+        _dev("sample.rng_states", rng_states, torch.int64, 1)
+        if state_index is not None:
+            _i32("sample.state_index", state_index, n)
+        elif rng_states.numel() < n:
+            raise KernelError("sample: fewer generator states than rows")
+    _check(lib().picolm_sample(_ptr(logits), c_int64(V), n, V, c_float(temperature), int(top_k), c_float(top_p),
+                               c_float(min_p), _ptr(rng_states), _ptr(state_index), _ptr(out), _stream()))

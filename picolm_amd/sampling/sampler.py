@@ -1,0 +1,36 @@
+"""The sampler the engine uses: one GPU kernel call per step over the rows of logits."""
+from __future__ import annotations
+
+import torch
+
+from .. import kernels
+from .params import SamplingParams, stream_state
+
+
+def _as_i64(u: int) -> int:
+    return u - (1 << 64) if u >= (1 << 63) else u
+
+
+class Sampler:
+    """Holds one generator state per sequence on the device."""
+
+    def __init__(self, params: SamplingParams, n_sequences: int, device):
+        params.validate()
+        self.params = params
+        self.device = torch.device(device)
+        self.n = n_sequences
+        states = [_as_i64(stream_state(params.seed, i)) for i in range(n_sequences)]
+        self.states = torch.tensor(states, dtype=torch.int64).to(self.device)
+        self._out = torch.zeros(max(n_sequences, 1), dtype=torch.int32, device=self.device)
+
+    def sample(self, logits: torch.Tensor, sequence_indices) -> list[int]:
+        """`logits[i]` belongs to sequence `sequence_indices[i]`; returns one token each."""
+        n = logits.shape[0]
+        out = self._out[:n]
+        p = self.params
+        if p.greedy:
+            kernels.argmax(logits, out)
+        else:
+            idx = torch.tensor(list(sequence_indices), dtype=torch.int32).to(self.device)
+            kernels.sample(logits, out, p.temperature, p.top_k, p.top_p, p.min_p, self.states, idx)
+        return out.tolist()

@@ -46,6 +46,10 @@ def sample(logits, temperature: float, top_k: int, top_p: float, min_p: float,
     """One draw; returns (token, new rng state).  sampler.c:48-125."""
     logits = np.asarray(logits, dtype=np.float64)
     V = len(logits)
+    # the options are floats in picolm (sampler.h:6-12): round them as it does
+    temperature = float(np.float32(temperature))
+    top_p = float(np.float32(top_p))
+    min_p = float(np.float32(min_p))
     if temperature <= 0.0:
         return argmax_first(logits), state
     # 1. softmax of the raw logits (:59)
