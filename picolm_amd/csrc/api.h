@@ -30,6 +30,12 @@ int picolm_gemm_generic(const void* A, int a_dt, const void* W, int w_dt, void* 
                         int N, int K, int64_t lda, int64_t ldw, int64_t ldc, int epilogue,
                         hipStream_t stream);
 
+// bf16 operands on the matrix cores; K and the row strides must be multiples of 8.
+int picolm_gemm_skinny(const void* A, const void* W, void* C, int c_dt, int M, int N, int K, int64_t lda,
+                       int64_t ldw, int64_t ldc, int epilogue, int variant, hipStream_t stream);
+int picolm_gemm_tiled(const void* A, const void* W, void* C, int c_dt, int M, int N, int K, int64_t lda,
+                      int64_t ldw, int64_t ldc, int epilogue, hipStream_t stream);
+
 int picolm_attn_prefill_tile_rows(void);
 int picolm_attn_prefill_generic(const void* q, const void* k_pages, const void* v_pages, void* out,
                                 int dt, const int32_t* tile_seq, const int32_t* tile_q0, int n_tiles,

@@ -1,0 +1,331 @@
+// bf16 x bf16 -> float products on the matrix cores of gfx950: C[M,N] = A[M,K] * W[N,K]^T.
+//
+// Both kernels feed the weight tile as the MFMA's first operand and the activation tile as
+// its second, so an accumulator lane holds four consecutive output columns n of one row m:
+// gate/up pairs of the row-interleaved gated layout meet in one lane, and stores along n
+// are vectors.
+//
+//   skinny (M <= 64, the decode step): HBM-bound.  A wave streams 16*NT weight rows straight
+//     from global memory into MFMA operand registers, 16 bytes a lane; the waves of a block
+//     split K between them and reduce through LDS.  Every weight byte is read once.
+//   tiled (M > 64, the prefill step): 128x128x64 block tiles staged through LDS with an XOR
+//     swizzle of 16-byte chunks, register prefetch of the next tile, 32x32x16 MFMAs.
+//
+// The order of the K summation inside an MFMA does not matter, so a lane's 8-element chunk
+// may come from any K offset as long as both operands use the same offset.
+#include "common.h"
+#include "api.h"
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(4))) float f32x4;
+typedef __attribute__((ext_vector_type(16))) float f32x16;
+
+__device__ __forceinline__ bf16x8 load_chunk(const bf16_t* p) { return *(const bf16x8*)p; }
+__device__ __forceinline__ bf16x8 zero_chunk() {
+    bf16x8 z;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) z[i] = (__bf16)0.0f;
+    return z;
+}
+__device__ __forceinline__ float silu_mul(float g, float u) { return g / (1.0f + expf(-g)) * u; }
+
+// =============================================================================================
+// skinny
+// =============================================================================================
+#define SK_KSTEP 128      // K elements one wave consumes per step: 4 quarters x 32
+
+template <int MT, int NT, int WAVES, int EPI, typename TC>
+__global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const bf16_t* __restrict__ A,
+                                                                 const bf16_t* __restrict__ W,
+                                                                 TC* __restrict__ C, int M, int N, int K,
+                                                                 int64_t lda, int64_t ldw, int64_t ldc) {
+    extern __shared__ float red[];      // [WAVES][NT][MT][4][64]
+    const int wave = threadIdx.x / 64, lane = threadIdx.x % 64;
+    const int r16 = lane % 16, q = lane / 16;
+    const int n_base = blockIdx.x * (16 * NT);
+
+    const bf16_t* wrow[NT];
+#pragma unroll
+    for (int t = 0; t < NT; ++t) wrow[t] = W + (int64_t)min(n_base + t * 16 + r16, N - 1) * ldw;
+    const bf16_t* arow[MT];
+    bool mvalid[MT];
+#pragma unroll
+    for (int u = 0; u < MT; ++u) {
+        const int m = u * 16 + r16;
+        mvalid[u] = m < M;
+        arow[u] = A + (int64_t)(mvalid[u] ? m : 0) * lda;
+    }
+    f32x4 acc[NT][MT];
+#pragma unroll
+    for (int t = 0; t < NT; ++t)
+#pragma unroll
+        for (int u = 0; u < MT; ++u) acc[t][u] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+    const int n_steps = (K + SK_KSTEP - 1) / SK_KSTEP;
+#pragma unroll 2
+    for (int s = wave; s < n_steps; s += WAVES) {
+        const int k0 = s * SK_KSTEP + q * 32;
+        bf16x8 wv[NT][4], av[MT][4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int k = k0 + 8 * j;
+            const bool kvalid = k < K;
+#pragma unroll
+            for (int t = 0; t < NT; ++t) wv[t][j] = kvalid ? load_chunk(wrow[t] + k) : zero_chunk();
+#pragma unroll
+            for (int u = 0; u < MT; ++u) av[u][j] = (kvalid && mvalid[u]) ? load_chunk(arow[u] + k) : zero_chunk();
+        }
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+#pragma unroll
+            for (int t = 0; t < NT; ++t)
+#pragma unroll
+                for (int u = 0; u < MT; ++u)
+                    acc[t][u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wv[t][j], av[u][j], acc[t][u], 0, 0, 0);
+    }
+    // reduce over the waves
+#pragma unroll
+    for (int t = 0; t < NT; ++t)
+#pragma unroll
+        for (int u = 0; u < MT; ++u)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) red[(((wave * NT + t) * MT + u) * 4 + r) * 64 + lane] = acc[t][u][r];
+    __syncthreads();
+    constexpr int PER_WAVE = NT * MT * 4 * 64;
+    constexpr int STEP = (EPI == 2) ? 2 : 1;
+    // value v = ((t*MT + u)*4 + r)*64 + l ; the gated epilogue takes r and r+1 together
+    for (int v = threadIdx.x; v < PER_WAVE / STEP; v += WAVES * 64) {
+        int l, r, tu;
+        if (EPI == 2) {
+            l = v % 64;
+            r = 2 * ((v / 64) % 2);
+            tu = v / 128;
+        } else {
+            l = v % 64;
+            r = (v / 64) % 4;
+            tu = v / 256;
+        }
+        const int u = tu % MT, t = tu / MT;
+        const int idx = ((t * MT + u) * 4 + r) * 64 + l;
+        float s0 = 0.f, s1 = 0.f;
+#pragma unroll
+        for (int w = 0; w < WAVES; ++w) {
+            s0 += red[w * PER_WAVE + idx];
+            if (EPI == 2) s1 += red[w * PER_WAVE + idx + 64];
+        }
+        const int n = n_base + t * 16 + 4 * (l / 16) + r;
+        const int m = u * 16 + l % 16;
+        if (m >= M || n >= N) continue;
+        if (EPI == 2) {
+            C[(int64_t)m * ldc + n / 2] = from_f32<TC>(silu_mul(s0, s1));
+        } else if (EPI == 1) {
+            TC* p = C + (int64_t)m * ldc + n;
+            *p = from_f32<TC>(to_f32<TC>(*p) + s0);
+        } else {
+            C[(int64_t)m * ldc + n] = from_f32<TC>(s0);
+        }
+    }
+}
+
+template <int MT, int NT, int WAVES>
+static int launch_skinny(const void* A, const void* W, void* C, int c_dt, int M, int N, int K, int64_t lda,
+                         int64_t ldw, int64_t ldc, int epi, hipStream_t stream) {
+    dim3 grid(ceil_div(N, 16 * NT)), block(WAVES * 64);
+    const size_t lds = sizeof(float) * WAVES * NT * MT * 4 * 64;
+    const bf16_t* a = (const bf16_t*)A;
+    const bf16_t* w = (const bf16_t*)W;
+#define SK_LAUNCH(EPI, TC)                                                                              \
+    {                                                                                                   \
+        static size_t raised = 48 * 1024;                                                               \
+        if (lds > raised) {                                                                             \
+            hipError_t e = hipFuncSetAttribute((const void*)gemm_skinny_kernel<MT, NT, WAVES, EPI, TC>, \
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);   \
+            PICOLM_REQUIRE(e == hipSuccess, "gemm_skinny: cannot raise the LDS limit: %s",              \
+                           hipGetErrorString(e));                                                       \
+            raised = lds;                                                                               \
+        }                                                                                               \
+        gemm_skinny_kernel<MT, NT, WAVES, EPI, TC><<<grid, block, lds, stream>>>(a, w, (TC*)C, M, N, K, lda, ldw, ldc); \
+    }
+    if (epi == 0 && c_dt == PICOLM_F32) SK_LAUNCH(0, float)
+    else if (epi == 0 && c_dt == PICOLM_BF16) SK_LAUNCH(0, bf16_t)
+    else if (epi == 1 && c_dt == PICOLM_F32) SK_LAUNCH(1, float)
+    else if (epi == 2 && c_dt == PICOLM_BF16) SK_LAUNCH(2, bf16_t)
+    else if (epi == 2 && c_dt == PICOLM_F32) SK_LAUNCH(2, float)
+    else PICOLM_REQUIRE(false, "gemm_skinny: unsupported epilogue %d with output dtype %d", epi, c_dt);
+#undef SK_LAUNCH
+    PICOLM_LAUNCH_CHECK("gemm_skinny");
+    return 0;
+}
+
+static int check_mfma_operands(const char* who, const void* A, const void* W, int M, int N, int K, int64_t lda,
+                               int64_t ldw, int64_t ldc, int epi, int c_dt) {
+    PICOLM_REQUIRE(M >= 0 && N > 0 && K > 0, "%s: bad sizes M=%d N=%d K=%d", who, M, N, K);
+    PICOLM_REQUIRE(K % 8 == 0 && lda % 8 == 0 && ldw % 8 == 0,
+                   "%s: K=%d and the row strides (%lld, %lld) must be multiples of 8", who, K, (long long)lda,
+                   (long long)ldw);
+    PICOLM_REQUIRE(((uintptr_t)A % 16 == 0) && ((uintptr_t)W % 16 == 0), "%s: operands must be 16-byte aligned", who);
+    PICOLM_REQUIRE(epi >= 0 && epi <= 2, "%s: unknown epilogue %d", who, epi);
+    PICOLM_REQUIRE(epi != 1 || c_dt == PICOLM_F32, "%s: accumulation needs a float output", who);
+    PICOLM_REQUIRE(epi != 2 || N % 2 == 0, "%s: the gated epilogue needs an even N, got %d", who, N);
+    PICOLM_REQUIRE(lda >= K && ldw >= K && ldc >= (epi == 2 ? N / 2 : N), "%s: leading dimensions too small", who);
+    return 0;
+}
+
+// variant: 0 picks by M; otherwise 1..6 name (MT,NT,WAVES) combinations for tuning and tests
+extern "C" int picolm_gemm_skinny(const void* A, const void* W, void* C, int c_dt, int M, int N, int K,
+                                  int64_t lda, int64_t ldw, int64_t ldc, int epilogue, int variant,
+                                  hipStream_t stream) {
+    if (check_mfma_operands("gemm_skinny", A, W, M, N, K, lda, ldw, ldc, epilogue, c_dt)) return -1;
+    PICOLM_REQUIRE(M <= 64, "gemm_skinny: M=%d exceeds 64", M);
+    if (M == 0) return 0;
+    if (variant == 0) variant = M <= 16 ? 1 : (M <= 32 ? 3 : 5);
+    switch (variant) {
+        case 1: return launch_skinny<1, 1, 8>(A, W, C, c_dt, M, N, K, lda, ldw, ldc, epilogue, stream);
+        case 2: return launch_skinny<1, 2, 8>(A, W, C, c_dt, M, N, K, lda, ldw, ldc, epilogue, stream);
+        case 3: return launch_skinny<2, 1, 8>(A, W, C, c_dt, M, N, K, lda, ldw, ldc, epilogue, stream);
+        case 4: return launch_skinny<2, 2, 8>(A, W, C, c_dt, M, N, K, lda, ldw, ldc, epilogue, stream);
+        case 5: return launch_skinny<4, 1, 8>(A, W, C, c_dt, M, N, K, lda, ldw, ldc, epilogue, stream);
+        case 6: return launch_skinny<4, 2, 4>(A, W, C, c_dt, M, N, K, lda, ldw, ldc, epilogue, stream);
+    }
+    PICOLM_REQUIRE(false, "gemm_skinny: unknown variant %d", variant);
+}
+
+// =============================================================================================
+// tiled
+// =============================================================================================
+#define TG_BN 128
+#define TG_BM 128
+#define TG_BK 64
+#define TG_THREADS 256
+#define TG_CHUNKS (TG_BK / 8)        // 16-byte chunks per tile row
+
+// LDS tile: [rows][TG_BK] bf16, chunk c of row r stored at chunk slot c ^ (r % 8)
+__device__ __forceinline__ int tile_off(int row, int chunk) { return row * TG_BK + ((chunk ^ (row & 7)) << 3); }
+
+template <int EPI, typename TC>
+__global__ __launch_bounds__(TG_THREADS) void gemm_tiled_kernel(const bf16_t* __restrict__ A,
+                                                               const bf16_t* __restrict__ W,
+                                                               TC* __restrict__ C, int M, int N, int K,
+                                                               int64_t lda, int64_t ldw, int64_t ldc,
+                                                               int tiles_m, int tiles_n) {
+    __shared__ __attribute__((aligned(16))) bf16_t Ws[TG_BN * TG_BK];
+    __shared__ __attribute__((aligned(16))) bf16_t As[TG_BM * TG_BK];
+    // tile order: consecutive blocks walk down M inside a column band of N so that the
+    // weight band stays in cache while activations stream
+    const int tile = blockIdx.x;
+    const int band = 8;                                   // tiles of N per band
+    const int per_band = band * tiles_m;
+    const int b = tile / per_band, in_b = tile % per_band;
+    const int band_w = min(band, tiles_n - b * band);
+    const int tn = b * band + in_b % band_w, tm = in_b / band_w;
+    const int n0 = tn * TG_BN, m0 = tm * TG_BM;
+
+    const int tid = threadIdx.x, wave = tid / 64, lane = tid % 64;
+    const int wn = (wave % 2) * 64, wm = (wave / 2) * 64;     // the wave's 64x64 corner of the block tile
+    const int l32 = lane % 32, kq = lane / 32;
+
+    // global -> register staging: 4 chunks per operand per thread
+    const int ld_chunk = tid % TG_CHUNKS, ld_row = tid / TG_CHUNKS;      // rows ld_row + 32*i
+    const bf16_t* wsrc[4];
+    const bf16_t* asrc[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        wsrc[i] = W + (int64_t)min(n0 + ld_row + 32 * i, N - 1) * ldw + ld_chunk * 8;
+        asrc[i] = A + (int64_t)min(m0 + ld_row + 32 * i, M - 1) * lda + ld_chunk * 8;
+    }
+    bf16x8 wreg[4], areg[4];
+    auto fetch = [&](int k0) {
+        const bool kvalid = k0 + ld_chunk * 8 < K;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            wreg[i] = kvalid ? load_chunk(wsrc[i] + k0) : zero_chunk();
+            areg[i] = kvalid ? load_chunk(asrc[i] + k0) : zero_chunk();
+        }
+    };
+    auto stash = [&]() {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            *(bf16x8*)(Ws + tile_off(ld_row + 32 * i, ld_chunk)) = wreg[i];
+            *(bf16x8*)(As + tile_off(ld_row + 32 * i, ld_chunk)) = areg[i];
+        }
+    };
+
+    f32x16 acc[2][2];
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
+
+    fetch(0);
+    for (int k0 = 0; k0 < K; k0 += TG_BK) {
+        __syncthreads();            // everyone is done reading the previous tile
+        stash();
+        __syncthreads();
+        if (k0 + TG_BK < K) fetch(k0 + TG_BK);
+#pragma unroll
+        for (int ks = 0; ks < TG_BK / 16; ++ks) {
+            const int chunk = ks * 2 + kq;
+            bf16x8 wf[2], af[2];
+#pragma unroll
+            for (int i = 0; i < 2; ++i) {
+                wf[i] = *(const bf16x8*)(Ws + tile_off(wn + 32 * i + l32, chunk));
+                af[i] = *(const bf16x8*)(As + tile_off(wm + 32 * i + l32, chunk));
+            }
+#pragma unroll
+            for (int i = 0; i < 2; ++i)
+#pragma unroll
+                for (int j = 0; j < 2; ++j)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wf[i], af[j], acc[i][j], 0, 0, 0);
+        }
+    }
+    // accumulator element e of tile (i, j): n = wn + 32i + 8*(e/4) + 4*kq + e%4, m = wm + 32j + l32
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+        const int m = m0 + wm + 32 * j + l32;
+        if (m >= M) continue;
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                const int n = n0 + wn + 32 * i + 8 * g + 4 * kq;
+                if (EPI == 2) {
+                    TC* p = C + (int64_t)m * ldc + n / 2;
+                    if (n + 1 < N) p[0] = from_f32<TC>(silu_mul(acc[i][j][4 * g], acc[i][j][4 * g + 1]));
+                    if (n + 3 < N) p[1] = from_f32<TC>(silu_mul(acc[i][j][4 * g + 2], acc[i][j][4 * g + 3]));
+                } else {
+                    TC* p = C + (int64_t)m * ldc + n;
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        if (n + e >= N) continue;
+                        const float v = acc[i][j][4 * g + e];
+                        p[e] = from_f32<TC>(EPI == 1 ? to_f32<TC>(p[e]) + v : v);
+                    }
+                }
+            }
+        }
+    }
+}
+
+extern "C" int picolm_gemm_tiled(const void* A, const void* W, void* C, int c_dt, int M, int N, int K,
+                                 int64_t lda, int64_t ldw, int64_t ldc, int epilogue, hipStream_t stream) {
+    if (check_mfma_operands("gemm_tiled", A, W, M, N, K, lda, ldw, ldc, epilogue, c_dt)) return -1;
+    if (M == 0) return 0;
+    const int tiles_m = ceil_div(M, TG_BM), tiles_n = ceil_div(N, TG_BN);
+    PICOLM_REQUIRE((int64_t)tiles_m * tiles_n < (1ll << 31), "gemm_tiled: too many tiles");
+    dim3 grid(tiles_m * tiles_n), block(TG_THREADS);
+    const bf16_t* a = (const bf16_t*)A;
+    const bf16_t* w = (const bf16_t*)W;
+#define TG_LAUNCH(EPI, TC) \
+    gemm_tiled_kernel<EPI, TC><<<grid, block, 0, stream>>>(a, w, (TC*)C, M, N, K, lda, ldw, ldc, tiles_m, tiles_n)
+    if (epilogue == 0 && c_dt == PICOLM_F32) TG_LAUNCH(0, float);
+    else if (epilogue == 0 && c_dt == PICOLM_BF16) TG_LAUNCH(0, bf16_t);
+    else if (epilogue == 1 && c_dt == PICOLM_F32) TG_LAUNCH(1, float);
+    else if (epilogue == 2 && c_dt == PICOLM_BF16) TG_LAUNCH(2, bf16_t);
+    else if (epilogue == 2 && c_dt == PICOLM_F32) TG_LAUNCH(2, float);
+    else PICOLM_REQUIRE(false, "gemm_tiled: unsupported epilogue %d with output dtype %d", epilogue, c_dt);
+#undef TG_LAUNCH
+    PICOLM_LAUNCH_CHECK("gemm_tiled");
+    return 0;
+}

@@ -42,7 +42,7 @@ def dir_entry_points():
     return ["picolm_abi_version", "picolm_device_check", "picolm_embed", "picolm_rmsnorm",
             "picolm_rope_kv_store", "picolm_silu_mul", "picolm_add_into", "picolm_gemm_generic",
             "picolm_attn_prefill_tile_rows", "picolm_attn_prefill_generic",
-            "picolm_attn_decode_generic", "picolm_argmax", "picolm_sample"]
+            "picolm_attn_decode_generic", "picolm_argmax", "picolm_sample", "picolm_gemm_skinny", "picolm_gemm_tiled"]
 
 
 def _check(rc: int) -> None:
@@ -241,9 +241,45 @@ def argmax(logits: torch.Tensor, out: torch.Tensor) -> None:
                                c_int64(logits.shape[1]), _stream()))
 
 
+SKINNY_MAX_M = 64
+
+
+def gemm_skinny(a, w, c, epilogue: int = EPI_STORE, variant: int = 0) -> None:
+    """bf16 x bf16 on the matrix cores for M <= 64 rows: weights streamed once from HBM."""
+    M, N, K = _gemm_shapes(a, w, c, epilogue)
+    _check(lib().picolm_gemm_skinny(_ptr(a), _ptr(w), _ptr(c), dt_of(c), M, N, K, c_int64(K), c_int64(K),
+                                    c_int64(c.shape[1]), epilogue, variant, _stream()))
+
+
+def gemm_tiled(a, w, c, epilogue: int = EPI_STORE) -> None:
+    """bf16 x bf16 on the matrix cores, LDS-tiled, for many rows."""
+    M, N, K = _gemm_shapes(a, w, c, epilogue)
+    _check(lib().picolm_gemm_tiled(_ptr(a), _ptr(w), _ptr(c), dt_of(c), M, N, K, c_int64(K), c_int64(K),
+                                   c_int64(c.shape[1]), epilogue, _stream()))
+
+
+def mfma_gemm_takes(a, w, c, epilogue: int) -> bool:
+    """Whether the matrix-core kernels accept these operands; otherwise the float kernel runs."""
+    if a.dtype != torch.bfloat16 or w.dtype != torch.bfloat16:
+        return False
+    if a.shape[1] % 8 != 0 or a.data_ptr() % 16 or w.data_ptr() % 16:
+        return False
+    if epilogue == EPI_STORE:
+        return True
+    if epilogue == EPI_ACCUMULATE:
+        return c.dtype == torch.float32
+    return True
+
+
 def gemm(a: torch.Tensor, w: torch.Tensor, c: torch.Tensor, epilogue: int = EPI_STORE) -> None:
     """The product the engine calls: picks the kernel for the operands' types and sizes."""
-    gemm_generic(a, w, c, epilogue)
+    if mfma_gemm_takes(a, w, c, epilogue):
+        if a.shape[0] <= SKINNY_MAX_M:
+            gemm_skinny(a, w, c, epilogue)
+        else:
+            gemm_tiled(a, w, c, epilogue)
+    else:
+        gemm_generic(a, w, c, epilogue)
 
 
 def attn_prefill(q, k_pages, v_pages, out, batch, page_table, ring_pages, H, G, d, window, scale) -> None:
