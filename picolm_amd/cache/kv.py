@@ -1,8 +1,8 @@
 """The cache on the GPU: paged keys and values for each group of layers, a slot for each
 live sequence, and fixed-size per-sequence state beside them.
 
-Layout of one KV group: K and V are [entry][page][kv_head][PAGE_TOKENS][head_dim]; an
-entry is one layer call's cache.  A slot's row of the group's page table maps logical page
+Layout of one KV group: K is [entry][page][kv_head][PAGE_TOKENS][head_dim] and V is kept
+transposed, [entry][page][kv_head][head_dim][PAGE_TOKENS]; an entry is one layer call's cache.  A slot's row of the group's page table maps logical page
 j (tokens 64j .. 64j+63) to a page; a group that keeps a window of keys maps j modulo its
 ring.  picolm's cache is [kv_layer][pos][G*d] for its one sequence, indexed through
 kv_layer_ordinal (picolm/model_core.c:734-739, :668-681, :1880-1883); the per-layer-call
@@ -52,9 +52,9 @@ class KVGroup:
         per_slot = self.ring_pages if spec.window > 0 else max_pages
         n_pages = min(n_pages, n_slots * per_slot)
         self.book = PagedGroupBook(n_pages, n_slots, self.ring_pages if spec.window > 0 else 0)
-        shape = (spec.n_entries, max(n_pages, 1), spec.n_kv_heads, PAGE_TOKENS, spec.head_dim)
-        self.k = torch.zeros(shape, dtype=dtype, device=device)
-        self.v = torch.zeros(shape, dtype=dtype, device=device)
+        n = max(n_pages, 1)
+        self.k = torch.zeros((spec.n_entries, n, spec.n_kv_heads, PAGE_TOKENS, spec.head_dim), dtype=dtype, device=device)
+        self.v = torch.zeros((spec.n_entries, n, spec.n_kv_heads, spec.head_dim, PAGE_TOKENS), dtype=dtype, device=device)
         self.table_host = torch.zeros((n_slots, max_pages), dtype=torch.int32)
         self.table = torch.zeros((n_slots, max_pages), dtype=torch.int32, device=device)
         self.dirty: set[int] = set()

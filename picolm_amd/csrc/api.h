@@ -50,6 +50,22 @@ int picolm_attn_decode_generic(const void* q, const void* k_pages, const void* v
                                int ring_pages, int H, int G, int d, int window, float scale,
                                hipStream_t stream);
 
+int picolm_attn_merge(const float* partial, void* out, int dt, int n_seq, const int32_t* cu_seqlens, int H,
+                      int d, int n_splits, hipStream_t stream);
+// bf16 attention on the matrix cores, head sizes 32, 64, 128
+int picolm_attn_mfma_takes(int d);
+int picolm_attn_prefill_mfma_heads(int H, int G);
+int picolm_attn_prefill_mfma_tile_tokens(int H, int G);
+int picolm_attn_prefill_mfma(const void* q, const void* k_pages, const void* v_pages, void* out,
+                             const int32_t* tile_seq, const int32_t* tile_q0, int n_tiles,
+                             const int32_t* seq_slot, const int32_t* seq_pos0, const int32_t* seq_nnew,
+                             const int32_t* cu_seqlens, const int32_t* page_table, int max_pages,
+                             int ring_pages, int H, int G, int d, int window, float scale, hipStream_t stream);
+int picolm_attn_decode_mfma(const void* q, const void* k_pages, const void* v_pages, void* out, float* partial,
+                            int n_seq, int n_splits, const int32_t* seq_slot, const int32_t* seq_pos0,
+                            const int32_t* cu_seqlens, const int32_t* page_table, int max_pages, int ring_pages,
+                            int H, int G, int d, int window, float scale, hipStream_t stream);
+
 int picolm_argmax(const float* logits, int32_t* out, int n_rows, int V, int64_t ld,
                   hipStream_t stream);
 // rng_states[state_index ? state_index[row] : row] is one xorshift64 state per sequence,

@@ -12,31 +12,12 @@
 // (picolm/backend_gpu_kernels.cu:802-963); the same shape is used here.
 #include "common.h"
 #include "api.h"
+#include "attention.h"
 
 #define AT_ROWS 16
 #define AT_THREADS 256
 #define AT_MAX_D 256
-#define NEG_BIG (-1e30f)
 
-struct AttnArgs {
-    const void* q;            // [T][H*d]
-    const void* k_pages;      // [n_pages][G][PAGE][d]
-    const void* v_pages;
-    void* out;                // [T][H*d]
-    float* partial;           // decode split-K: [n_seq][H][n_splits][d+2], or null
-    const int32_t* tile_seq;  // prefill: sequence of each tile
-    const int32_t* tile_q0;   // prefill: first new-token index of each tile
-    const int32_t* seq_slot;
-    const int32_t* seq_pos0;  // tokens the sequence held before this step
-    const int32_t* seq_nnew;
-    const int32_t* cu_seqlens;  // first token row of each sequence in this step
-    const int32_t* page_table;
-    int max_pages, ring_pages;
-    int H, G, d, window;
-    float scale;
-    int decode;     // 0 prefill tiles, 1 decode groups
-    int n_splits;   // decode only
-};
 
 template <typename T>
 __global__ __launch_bounds__(AT_THREADS) void attn_tile_kernel(AttnArgs a) {
@@ -156,9 +137,9 @@ __global__ __launch_bounds__(AT_THREADS) void attn_tile_kernel(AttnArgs a) {
         }
         __syncthreads();
         {
-            const T* vp = (const T*)a.v_pages + base;
+            const T* vp = (const T*)a.v_pages + base;       // transposed: [d][PAGE]
             for (int idx = tid; idx < PAGE_TOKENS * d; idx += AT_THREADS) {
-                const int r = idx / d, c = idx % d;
+                const int c = idx / PAGE_TOKENS, r = idx % PAGE_TOKENS;
                 KVs[r * dp + c] = r < n_keys ? to_f32<T>(vp[idx]) : 0.f;
             }
         }
@@ -255,6 +236,21 @@ static int check_attn_sizes(const char* who, int H, int G, int d, int max_pages,
     return 0;
 }
 
+extern "C" int picolm_attn_merge(const float* partial, void* out, int dt, int n_seq, const int32_t* cu_seqlens,
+                                 int H, int d, int n_splits, hipStream_t stream) {
+    PICOLM_REQUIRE(n_seq >= 0 && H > 0 && d > 0 && n_splits >= 1, "attn_merge: bad sizes");
+    if (n_seq == 0) return 0;
+    dim3 mgrid(n_seq * H), mblock(d <= 64 ? 64 : (d <= 128 ? 128 : 256));
+    if (dt == PICOLM_F32)
+        attn_merge_kernel<float><<<mgrid, mblock, 0, stream>>>(partial, (float*)out, cu_seqlens, H, d, n_splits);
+    else if (dt == PICOLM_BF16)
+        attn_merge_kernel<bf16_t><<<mgrid, mblock, 0, stream>>>(partial, (bf16_t*)out, cu_seqlens, H, d, n_splits);
+    else
+        PICOLM_REQUIRE(false, "attn_merge: unknown dtype %d", dt);
+    PICOLM_LAUNCH_CHECK("attn_merge");
+    return 0;
+}
+
 extern "C" int picolm_attn_prefill_generic(const void* q, const void* k_pages, const void* v_pages,
                                            void* out, int dt, const int32_t* tile_seq,
                                            const int32_t* tile_q0, int n_tiles,
@@ -297,13 +293,6 @@ extern "C" int picolm_attn_decode_generic(const void* q, const void* k_pages, co
     else if (dt == PICOLM_BF16) rc = launch_attn<bf16_t>(a, grid, stream);
     else PICOLM_REQUIRE(false, "attn_decode: unknown dtype %d", dt);
     if (rc) return rc;
-    if (n_splits > 1) {
-        dim3 mgrid(n_seq * H), mblock(d <= 64 ? 64 : (d <= 128 ? 128 : 256));
-        if (dt == PICOLM_F32)
-            attn_merge_kernel<float><<<mgrid, mblock, 0, stream>>>(partial, (float*)out, cu_seqlens, H, d, n_splits);
-        else
-            attn_merge_kernel<bf16_t><<<mgrid, mblock, 0, stream>>>(partial, (bf16_t*)out, cu_seqlens, H, d, n_splits);
-        PICOLM_LAUNCH_CHECK("attn_merge");
-    }
+    if (n_splits > 1) return picolm_attn_merge(partial, out, dt, n_seq, cu_seqlens, H, d, n_splits, stream);
     return 0;
 }

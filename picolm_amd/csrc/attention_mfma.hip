@@ -1,0 +1,369 @@
+// bf16 attention over the paged cache on the matrix cores of gfx950, head sizes 32, 64, 128.
+//
+// Both kernels compute S^T = K Q^T with 32x32x16 MFMAs, so that an accumulator lane holds one
+// query (column) and 16 keys (rows): a query's maximum and sum are an in-lane reduction plus
+// one exchange with lane^32, and the rescaling of the output accumulator O^T = V^T P^T is a
+// per-lane scalar.  The rows of an S^T tile are a permutation of its 32 keys, chosen so that a
+// lane's 16 accumulator values are 16 consecutive keys; P^T then feeds the second MFMA
+// straight from registers, and V^T (values are cached transposed) is read 16 bytes at a time.
+// Softmax statistics are float, in the base-2 domain: p = exp2(s*scale*log2e - m).
+//
+//   prefill: a workgroup of 4 waves shares K and V^T tiles of one page through LDS; a wave
+//            owns 32 new tokens of one query head; with grouped heads the waves of a
+//            workgroup take different heads of the group, so a page is loaded once per group.
+//   decode : a wave streams its own pages straight from global memory into MFMA operands
+//            (columns = the query heads of one KV group); the 4 waves of a workgroup take
+//            pages in turn and merge through LDS; split-K partials go to a buffer that the
+//            merge kernel of the generic path combines.
+#include "common.h"
+#include "api.h"
+#include "attention.h"
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4;
+typedef __attribute__((ext_vector_type(16))) float f32x16;
+
+#define LOG2E 1.4426950408889634f
+#define LN2 0.6931471805599453f
+
+__device__ __forceinline__ bf16x8 ldg8(const bf16_t* p) { return *(const bf16x8*)p; }
+__device__ __forceinline__ bf16x8 zero8() {
+    bf16x8 z;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) z[i] = (__bf16)0.0f;
+    return z;
+}
+// row i of an S^T tile holds key 16*((i>>2)&1) + 4*(i>>3) + (i&3) of the tile's 32 keys
+__device__ __forceinline__ int key_of_row(int i) { return 16 * ((i >> 2) & 1) + 4 * (i >> 3) + (i & 3); }
+
+__device__ __forceinline__ __bf16 to_bf16(float f) {
+    bf16_t b = f32_to_bf16_bits(f);
+    return *reinterpret_cast<__bf16*>(&b);
+}
+
+// One page of one wave: scores, online softmax, and the update of O^T.  KOP(t, s) returns the
+// K operand of tile t, k-step s; VOP(dt, t, ks) the V^T operand of column block dt.
+template <int D, typename KOP, typename VOP>
+__device__ __forceinline__ void attend_page(const bf16x8 (&Qf)[D / 16], f32x16 (&O)[D / 32], float& m_run,
+                                            float& l_run, int key0, int qpos, bool q_ok, int window,
+                                            float scale2, int h, KOP kop, VOP vop) {
+    f32x16 S[2];
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+#pragma unroll
+        for (int e = 0; e < 16; ++e) S[t][e] = 0.f;
+#pragma unroll
+        for (int s = 0; s < D / 16; ++s) S[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kop(t, s), Qf[s], S[t], 0, 0, 0);
+    }
+    float mx = NEG_BIG;
+#pragma unroll
+    for (int t = 0; t < 2; ++t)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+            const int key = key0 + 32 * t + 16 * h + e;
+            const bool vis = q_ok && key <= qpos && (window <= 0 || qpos - key < window);
+            S[t][e] = vis ? S[t][e] * scale2 : NEG_BIG;
+            mx = fmaxf(mx, S[t][e]);
+        }
+    mx = fmaxf(mx, __shfl_xor(mx, 32, WAVE));
+    const float m_new = fmaxf(m_run, mx);
+    const float alpha = exp2f(m_run - m_new);
+    float sum = 0.f;
+    bf16x8 Pf[2][2];
+#pragma unroll
+    for (int t = 0; t < 2; ++t)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+            const float p = S[t][e] > 0.5f * NEG_BIG ? exp2f(S[t][e] - m_new) : 0.f;
+            sum += p;
+            Pf[t][e / 8][e % 8] = to_bf16(p);
+        }
+    sum += __shfl_xor(sum, 32, WAVE);
+    l_run = l_run * alpha + sum;
+    m_run = m_new;
+#pragma unroll
+    for (int dt = 0; dt < D / 32; ++dt) {
+#pragma unroll
+        for (int e = 0; e < 16; ++e) O[dt][e] *= alpha;
+#pragma unroll
+        for (int t = 0; t < 2; ++t)
+#pragma unroll
+            for (int ks = 0; ks < 2; ++ks)
+                O[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vop(dt, t, ks), Pf[t][ks], O[dt], 0, 0, 0);
+    }
+}
+
+// =============================================================================================
+template <int D>
+__global__ __launch_bounds__(256) void attn_prefill_mfma_kernel(AttnArgs a, int HB, int tile_tokens) {
+    constexpr int KCH = D / 8;                   // 16-byte chunks of a K row
+    constexpr int KSWZ = KCH < 8 ? KCH : 8;
+    __shared__ __attribute__((aligned(16))) bf16_t Ks[PAGE_TOKENS * D];    // [key][d], chunk c at c ^ (key % KSWZ)
+    __shared__ __attribute__((aligned(16))) bf16_t Vs[D * PAGE_TOKENS];    // [dcol][key], chunk c at c ^ (dcol % 8)
+    const int tid = threadIdx.x, wave = tid / WAVE, lane = tid % WAVE;
+    const int l32 = lane % 32, h = lane / 32;
+    const int R = a.H / a.G;
+    const int head_chunks = (R + HB - 1) / HB;
+    const int seq = a.tile_seq[blockIdx.x], q0 = a.tile_q0[blockIdx.x];
+    const int g = blockIdx.y / head_chunks, chunk = blockIdx.y % head_chunks;
+    const int head_local = chunk * HB + wave % HB;
+    const int tb = wave / HB;
+    const int nnew = a.seq_nnew[seq], pos0 = a.seq_pos0[seq];
+    const int w_first = q0 + 32 * tb;
+    const bool w_active = head_local < R && w_first < nnew;
+    const int head = g * R + (head_local < R ? head_local : 0);
+    const int qi = w_first + l32;
+    const bool q_ok = w_active && qi < nnew;
+    const int qpos = pos0 + qi;
+    const size_t tok = (size_t)a.cu_seqlens[seq] + (q_ok ? qi : 0);
+
+    const int b_qfirst = pos0 + q0, b_qlast = pos0 + min(q0 + tile_tokens, nnew) - 1;
+    const int page_lo = (a.window > 0 ? max(0, b_qfirst - a.window + 1) : 0) / PAGE_TOKENS;
+    const int page_hi = b_qlast / PAGE_TOKENS + 1;
+    const int w_qfirst = pos0 + w_first, w_qlast = pos0 + min(w_first + 32, nnew) - 1;
+    const int w_page_lo = (a.window > 0 ? max(0, w_qfirst - a.window + 1) : 0) / PAGE_TOKENS;
+    const int w_page_hi = w_active ? w_qlast / PAGE_TOKENS + 1 : 0;
+
+    bf16x8 Qf[D / 16];
+    {
+        const bf16_t* qp = (const bf16_t*)a.q + tok * a.H * D + (size_t)head * D + 8 * h;
+#pragma unroll
+        for (int s = 0; s < D / 16; ++s) Qf[s] = q_ok ? ldg8(qp + 16 * s) : zero8();
+    }
+    f32x16 O[D / 32];
+#pragma unroll
+    for (int dt = 0; dt < D / 32; ++dt)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) O[dt][e] = 0.f;
+    float m_run = NEG_BIG, l_run = 0.f;
+    const float scale2 = a.scale * LOG2E;
+    const int32_t* pt = a.page_table + (size_t)a.seq_slot[seq] * a.max_pages;
+    const size_t page_elems = (size_t)a.G * PAGE_TOKENS * D;
+
+    for (int page = page_lo; page < page_hi; ++page) {
+        const size_t base = (size_t)pt[page % a.ring_pages] * page_elems + (size_t)g * PAGE_TOKENS * D;
+        const bf16_t* kp = (const bf16_t*)a.k_pages + base;
+        const bf16_t* vp = (const bf16_t*)a.v_pages + base;
+        const int n_keys = min(PAGE_TOKENS, b_qlast - page * PAGE_TOKENS + 1);
+        __syncthreads();
+#pragma unroll
+        for (int idx = tid; idx < PAGE_TOKENS * KCH; idx += 256) {
+            const int row = idx / KCH, c = idx % KCH;
+            *(bf16x8*)(Ks + (row * KCH + (c ^ (row % KSWZ))) * 8) = ldg8(kp + (size_t)idx * 8);
+        }
+#pragma unroll
+        for (int idx = tid; idx < D * 8; idx += 256) {
+            const int row = idx / 8, c = idx % 8;
+            bf16x8 v = ldg8(vp + (size_t)idx * 8);
+            if (n_keys < PAGE_TOKENS) {          // keys past the sequence's end may hold anything
+#pragma unroll
+                for (int e = 0; e < 8; ++e)
+                    if (8 * c + e >= n_keys) v[e] = (__bf16)0.0f;
+            }
+            *(bf16x8*)(Vs + (row * 8 + (c ^ (row % 8))) * 8) = v;
+        }
+        __syncthreads();
+        if (page >= w_page_lo && page < w_page_hi) {
+            attend_page<D>(
+                Qf, O, m_run, l_run, page * PAGE_TOKENS, qpos, q_ok, a.window, scale2, h,
+                [&](int t, int s) {
+                    const int row = 32 * t + key_of_row(l32);
+                    return *(const bf16x8*)(Ks + (row * KCH + ((2 * s + h) ^ (row % KSWZ))) * 8);
+                },
+                [&](int dt, int t, int ks) {
+                    const int row = 32 * dt + l32;
+                    return *(const bf16x8*)(Vs + (row * 8 + ((4 * t + 2 * h + ks) ^ (row % 8))) * 8);
+                });
+        }
+    }
+    if (!q_ok) return;
+    const float inv = l_run > 0.f ? 1.0f / l_run : 0.f;
+    bf16_t* o = (bf16_t*)a.out + tok * a.H * D + (size_t)head * D;
+#pragma unroll
+    for (int dt = 0; dt < D / 32; ++dt)
+#pragma unroll
+        for (int q4 = 0; q4 < 4; ++q4) {
+            bf16x4 v;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) v[e] = to_bf16(O[dt][4 * q4 + e] * inv);
+            *(bf16x4*)(o + 32 * dt + 8 * q4 + 4 * h) = v;
+        }
+}
+
+// =============================================================================================
+template <int D>
+__global__ __launch_bounds__(256) void attn_decode_mfma_kernel(AttnArgs a) {
+    extern __shared__ float mrg[];       // [4 waves][Rc][D + 2]
+    const int tid = threadIdx.x, wave = tid / WAVE, lane = tid % WAVE;
+    const int l32 = lane % 32, h = lane / 32;
+    const int R = a.H / a.G;
+    const int chunks = (R + 31) / 32;
+    const int seq = blockIdx.x;
+    const int g = blockIdx.y / chunks, chunk = blockIdx.y % chunks;
+    const int split = blockIdx.z;
+    const int Rc = min(32, R - chunk * 32);
+    const bool q_ok = l32 < Rc;
+    const int head = g * R + chunk * 32 + (q_ok ? l32 : 0);
+    const size_t tok = (size_t)a.cu_seqlens[seq];
+    const int qpos = a.seq_pos0[seq];
+
+    int page_lo = (a.window > 0 ? max(0, qpos - a.window + 1) : 0) / PAGE_TOKENS;
+    int page_hi = qpos / PAGE_TOKENS + 1;
+    if (a.n_splits > 1) {
+        const int np = page_hi - page_lo;
+        const int per = (np + a.n_splits - 1) / a.n_splits;
+        const int b = page_lo + split * per;
+        page_hi = min(page_hi, b + per);
+        page_lo = b;
+    }
+    // k-step s of a lane covers d = (D/2)*h + 8s .. +8: a lane's K reads are one contiguous run
+    bf16x8 Qf[D / 16];
+    {
+        const bf16_t* qp = (const bf16_t*)a.q + tok * a.H * D + (size_t)head * D + (D / 2) * h;
+#pragma unroll
+        for (int s = 0; s < D / 16; ++s) Qf[s] = q_ok ? ldg8(qp + 8 * s) : zero8();
+    }
+    f32x16 O[D / 32];
+#pragma unroll
+    for (int dt = 0; dt < D / 32; ++dt)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) O[dt][e] = 0.f;
+    float m_run = NEG_BIG, l_run = 0.f;
+    const float scale2 = a.scale * LOG2E;
+    const int32_t* pt = a.page_table + (size_t)a.seq_slot[seq] * a.max_pages;
+    const size_t page_elems = (size_t)a.G * PAGE_TOKENS * D;
+
+    for (int page = page_lo + wave; page < page_hi; page += 4) {
+        const size_t base = (size_t)pt[page % a.ring_pages] * page_elems + (size_t)g * PAGE_TOKENS * D;
+        const bf16_t* kp = (const bf16_t*)a.k_pages + base + (D / 2) * h;
+        const bf16_t* vp = (const bf16_t*)a.v_pages + base + (size_t)l32 * PAGE_TOKENS + 16 * h;
+        const int key0 = page * PAGE_TOKENS;
+        const int n_keys = qpos - key0 + 1;          // >= 1; keys past it are not this sequence's
+        attend_page<D>(
+            Qf, O, m_run, l_run, key0, qpos, q_ok, a.window, scale2, h,
+            [&](int t, int s) { return ldg8(kp + (size_t)(32 * t + key_of_row(l32)) * D + 8 * s); },
+            [&](int dt, int t, int ks) {
+                bf16x8 v = ldg8(vp + (size_t)(32 * dt) * PAGE_TOKENS + 32 * t + 8 * ks);
+                if (n_keys < PAGE_TOKENS) {
+                    const int k = 32 * t + 16 * h + 8 * ks;
+#pragma unroll
+                    for (int e = 0; e < 8; ++e)
+                        if (k + e >= n_keys) v[e] = (__bf16)0.0f;
+                }
+                return v;
+            });
+    }
+    // merge the 4 waves
+    float* mine = mrg + (size_t)wave * Rc * (D + 2);
+    if (q_ok) {
+        float* row = mine + (size_t)l32 * (D + 2);
+        if (h == 0) {
+            row[0] = m_run;
+            row[1] = l_run;
+        }
+#pragma unroll
+        for (int dt = 0; dt < D / 32; ++dt)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) row[2 + 32 * dt + 8 * (e / 4) + 4 * h + e % 4] = O[dt][e];
+    }
+    __syncthreads();
+    for (int idx = tid; idx < Rc * D; idx += 256) {
+        const int q = idx / D, dcol = idx % D;
+        float M = NEG_BIG;
+#pragma unroll
+        for (int w = 0; w < 4; ++w) M = fmaxf(M, mrg[((size_t)w * Rc + q) * (D + 2)]);
+        float L = 0.f, acc = 0.f;
+#pragma unroll
+        for (int w = 0; w < 4; ++w) {
+            const float* row = mrg + ((size_t)w * Rc + q) * (D + 2);
+            const float f = exp2f(row[0] - M);
+            L += f * row[1];
+            acc += f * row[2 + dcol];
+        }
+        const int hq = g * R + chunk * 32 + q;
+        if (a.partial) {
+            float* po = a.partial + (((size_t)seq * a.H + hq) * a.n_splits + split) * (D + 2);
+            if (dcol == 0) {
+                po[0] = M * LN2;        // the merge kernel works with natural exponents
+                po[1] = L;
+            }
+            po[2 + dcol] = acc;
+        } else {
+            ((bf16_t*)a.out)[tok * a.H * D + (size_t)hq * D + dcol] = f32_to_bf16_bits(L > 0.f ? acc / L : 0.f);
+        }
+    }
+}
+
+// =============================================================================================
+static int check_sizes(const char* who, int H, int G, int d, int max_pages, int ring_pages) {
+    PICOLM_REQUIRE(H > 0 && G > 0 && H % G == 0, "%s: %d heads do not split over %d groups", who, H, G);
+    PICOLM_REQUIRE(d == 32 || d == 64 || d == 128, "%s: head size %d is not 32, 64 or 128", who, d);
+    PICOLM_REQUIRE(max_pages > 0 && ring_pages > 0 && ring_pages <= max_pages,
+                   "%s: bad page table geometry max_pages=%d ring_pages=%d", who, max_pages, ring_pages);
+    return 0;
+}
+
+extern "C" int picolm_attn_mfma_takes(int d) { return d == 32 || d == 64 || d == 128; }
+
+// heads of a group that share a workgroup, and the new tokens one workgroup covers
+extern "C" int picolm_attn_prefill_mfma_heads(int H, int G) {
+    const int R = H / G;
+    return R >= 3 ? 4 : (R == 2 ? 2 : 1);
+}
+extern "C" int picolm_attn_prefill_mfma_tile_tokens(int H, int G) {
+    return 32 * (4 / picolm_attn_prefill_mfma_heads(H, G));
+}
+
+extern "C" int picolm_attn_prefill_mfma(const void* q, const void* k_pages, const void* v_pages, void* out,
+                                        const int32_t* tile_seq, const int32_t* tile_q0, int n_tiles,
+                                        const int32_t* seq_slot, const int32_t* seq_pos0,
+                                        const int32_t* seq_nnew, const int32_t* cu_seqlens,
+                                        const int32_t* page_table, int max_pages, int ring_pages, int H, int G,
+                                        int d, int window, float scale, hipStream_t stream) {
+    if (check_sizes("attn_prefill_mfma", H, G, d, max_pages, ring_pages)) return -1;
+    if (n_tiles <= 0) return 0;
+    const int HB = picolm_attn_prefill_mfma_heads(H, G);
+    const int tile_tokens = 32 * (4 / HB);
+    const int head_chunks = ceil_div(H / G, HB);
+    PICOLM_REQUIRE(G * head_chunks <= 65535, "attn_prefill_mfma: %d head groups exceed the grid", G * head_chunks);
+    AttnArgs a = {q, k_pages, v_pages, out, nullptr, tile_seq, tile_q0, seq_slot, seq_pos0, seq_nnew,
+                  cu_seqlens, page_table, max_pages, ring_pages, H, G, d, window, scale, 0, 1};
+    dim3 grid(n_tiles, G * head_chunks), block(256);
+    if (d == 32) attn_prefill_mfma_kernel<32><<<grid, block, 0, stream>>>(a, HB, tile_tokens);
+    else if (d == 64) attn_prefill_mfma_kernel<64><<<grid, block, 0, stream>>>(a, HB, tile_tokens);
+    else attn_prefill_mfma_kernel<128><<<grid, block, 0, stream>>>(a, HB, tile_tokens);
+    PICOLM_LAUNCH_CHECK("attn_prefill_mfma");
+    return 0;
+}
+
+extern "C" int picolm_attn_decode_mfma(const void* q, const void* k_pages, const void* v_pages, void* out,
+                                       float* partial, int n_seq, int n_splits, const int32_t* seq_slot,
+                                       const int32_t* seq_pos0, const int32_t* cu_seqlens,
+                                       const int32_t* page_table, int max_pages, int ring_pages, int H, int G,
+                                       int d, int window, float scale, hipStream_t stream) {
+    if (check_sizes("attn_decode_mfma", H, G, d, max_pages, ring_pages)) return -1;
+    PICOLM_REQUIRE(n_splits >= 1 && n_splits <= 65535, "attn_decode_mfma: bad split count %d", n_splits);
+    PICOLM_REQUIRE(n_splits == 1 || partial != nullptr, "attn_decode_mfma: splits need a partial buffer");
+    if (n_seq <= 0) return 0;
+    const int R = H / G, chunks = ceil_div(R, 32);
+    PICOLM_REQUIRE(G * chunks <= 65535, "attn_decode_mfma: %d groups exceed the grid", G * chunks);
+    AttnArgs a = {q, k_pages, v_pages, out, n_splits > 1 ? partial : nullptr, nullptr, nullptr, seq_slot, seq_pos0,
+                  nullptr, cu_seqlens, page_table, max_pages, ring_pages, H, G, d, window, scale, 1, n_splits};
+    dim3 grid(n_seq, G * chunks, n_splits), block(256);
+    const size_t lds = sizeof(float) * 4 * (size_t)min(R, 32) * (d + 2);
+    if (d == 32) attn_decode_mfma_kernel<32><<<grid, block, lds, stream>>>(a);
+    else if (d == 64) attn_decode_mfma_kernel<64><<<grid, block, lds, stream>>>(a);
+    else {
+        static size_t raised = 48 * 1024;
+        if (lds > raised) {
+            hipError_t e = hipFuncSetAttribute((const void*)attn_decode_mfma_kernel<128>,
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+            PICOLM_REQUIRE(e == hipSuccess, "attn_decode_mfma: cannot raise the LDS limit: %s", hipGetErrorString(e));
+            raised = lds;
+        }
+        attn_decode_mfma_kernel<128><<<grid, block, lds, stream>>>(a);
+    }
+    PICOLM_LAUNCH_CHECK("attn_decode_mfma");
+    if (n_splits > 1) return picolm_attn_merge(partial, out, PICOLM_BF16, n_seq, cu_seqlens, H, d, n_splits, stream);
+    return 0;
+}

@@ -90,11 +90,15 @@ __global__ void rope_kv_store_kernel(const float* __restrict__ qkv, TC* __restri
     const float* c = cos_t ? cos_t + (size_t)pos * half : nullptr;
     const float* s = sin_t ? sin_t + (size_t)pos * half : nullptr;
 
-    size_t cache_row = 0;
+    // keys are [page][G][PAGE][d]; values are kept transposed, [page][G][d][PAGE], so that the
+    // attention kernels read eight consecutive keys of one column as one 16-byte chunk
+    size_t cache_row = 0, page_base = 0;
+    const int in_page = pos % PAGE_TOKENS;
     if (k_pages) {
         const int slot = seq_slot[tok_seq[t]];
         const int page = page_table[(size_t)slot * max_pages + (pos / PAGE_TOKENS) % ring_pages];
-        cache_row = ((size_t)page * G) * PAGE_TOKENS * d + (size_t)(pos % PAGE_TOKENS) * d;
+        page_base = ((size_t)page * G) * PAGE_TOKENS * d;
+        cache_row = page_base + (size_t)in_page * d;
     }
     // rotations: heads 0..H-1 are q, H..H+G-1 are k
     const int n_rot = (H + G) * half;
@@ -123,7 +127,7 @@ __global__ void rope_kv_store_kernel(const float* __restrict__ qkv, TC* __restri
         const float* vrow = row + (H + G) * d;
         for (int idx = threadIdx.x; idx < G * d; idx += blockDim.x) {
             const int g = idx / d, i = idx % d;
-            v_pages[cache_row + (size_t)g * PAGE_TOKENS * d + i] = from_f32<TC>(vrow[idx]);
+            v_pages[page_base + ((size_t)g * d + i) * PAGE_TOKENS + in_page] = from_f32<TC>(vrow[idx]);
         }
     }
 }

@@ -42,7 +42,9 @@ def dir_entry_points():
     return ["picolm_abi_version", "picolm_device_check", "picolm_embed", "picolm_rmsnorm",
             "picolm_rope_kv_store", "picolm_silu_mul", "picolm_add_into", "picolm_gemm_generic",
             "picolm_attn_prefill_tile_rows", "picolm_attn_prefill_generic",
-            "picolm_attn_decode_generic", "picolm_argmax", "picolm_sample", "picolm_gemm_skinny", "picolm_gemm_tiled"]
+            "picolm_attn_decode_generic", "picolm_argmax", "picolm_sample", "picolm_gemm_skinny", "picolm_gemm_tiled",
+            "picolm_attn_mfma_takes", "picolm_attn_prefill_mfma_heads", "picolm_attn_prefill_mfma_tile_tokens",
+            "picolm_attn_prefill_mfma", "picolm_attn_decode_mfma", "picolm_attn_merge"]
 
 
 def _check(rc: int) -> None:
@@ -133,10 +135,7 @@ def rope_kv_store(qkv, q_out, k_pages, v_pages, cos, sin, style: int, tok_pos, t
         raise KernelError(f"rope: q_out {tuple(q_out.shape)} is not {(T, H * d)}")
     max_pages = 1
     if k_pages is not None:
-        for nm, p in (("k_pages", k_pages), ("v_pages", v_pages)):
-            _dev("rope." + nm, p, q_out.dtype, 4)
-            if tuple(p.shape[1:]) != (G, PAGE_TOKENS, d):
-                raise KernelError(f"rope: {nm} {tuple(p.shape)} is not [pages, {G}, {PAGE_TOKENS}, {d}]")
+        _check_pages("rope", k_pages, v_pages, q_out.dtype, G, d)
         _dev("rope.page_table", page_table, torch.int32, 2)
         max_pages = page_table.shape[1]
         _i32("rope.seq_slot", seq_slot)
@@ -151,6 +150,16 @@ def rope_kv_store(qkv, q_out, k_pages, v_pages, cos, sin, style: int, tok_pos, t
         _ptr(qkv), _ptr(q_out), _ptr(k_pages), _ptr(v_pages), dt_of(q_out), _ptr(cos), _ptr(sin), style,
         _ptr(tok_pos), _ptr(tok_seq), _ptr(seq_slot), _ptr(page_table), max_pages, ring_pages, T, H, G, d,
         _stream()))
+
+
+def _check_pages(who, k_pages, v_pages, dtype, G, d):
+    """keys [pages, G, PAGE, d]; values transposed [pages, G, d, PAGE]"""
+    _dev(who + ".k_pages", k_pages, dtype, 4)
+    _dev(who + ".v_pages", v_pages, dtype, 4)
+    if tuple(k_pages.shape[1:]) != (G, PAGE_TOKENS, d):
+        raise KernelError(f"{who}: k_pages {tuple(k_pages.shape)} is not [pages, {G}, {PAGE_TOKENS}, {d}]")
+    if tuple(v_pages.shape[1:]) != (G, d, PAGE_TOKENS) or v_pages.shape[0] != k_pages.shape[0]:
+        raise KernelError(f"{who}: v_pages {tuple(v_pages.shape)} is not [{k_pages.shape[0]}, {G}, {d}, {PAGE_TOKENS}]")
 
 
 def silu_mul(gu: torch.Tensor, out: torch.Tensor) -> None:
@@ -227,10 +236,7 @@ def _attn_check(q, k_pages, v_pages, out, page_table, H, G, d):
     _dev("attn.out", out, q.dtype, 2)
     if q.shape[1] != H * d or out.shape != q.shape:
         raise KernelError(f"attn: q {tuple(q.shape)} / out {tuple(out.shape)} are not [T, {H * d}]")
-    for nm, p in (("k_pages", k_pages), ("v_pages", v_pages)):
-        _dev("attn." + nm, p, q.dtype, 4)
-        if tuple(p.shape[1:]) != (G, PAGE_TOKENS, d):
-            raise KernelError(f"attn: {nm} {tuple(p.shape)} is not [pages, {G}, {PAGE_TOKENS}, {d}]")
+    _check_pages("attn", k_pages, v_pages, q.dtype, G, d)
     _dev("attn.page_table", page_table, torch.int32, 2)
 
 
@@ -282,8 +288,41 @@ def gemm(a: torch.Tensor, w: torch.Tensor, c: torch.Tensor, epilogue: int = EPI_
         gemm_generic(a, w, c, epilogue)
 
 
+def attn_mfma_takes(q: torch.Tensor, d: int) -> bool:
+    return q.dtype == torch.bfloat16 and bool(lib().picolm_attn_mfma_takes(d))
+
+
+def attn_prefill_mfma(q, k_pages, v_pages, out, batch, page_table, ring_pages, H, G, d, window, scale) -> None:
+    _attn_check(q, k_pages, v_pages, out, page_table, H, G, d)
+    tile_seq, tile_q0, n_tiles = batch.prefill_tiles(lib().picolm_attn_prefill_mfma_tile_tokens(H, G))
+    _check(lib().picolm_attn_prefill_mfma(
+        _ptr(q), _ptr(k_pages), _ptr(v_pages), _ptr(out), _ptr(tile_seq), _ptr(tile_q0), n_tiles,
+        _ptr(batch.seq_slot), _ptr(batch.seq_pos0), _ptr(batch.seq_nnew), _ptr(batch.cu_seqlens), _ptr(page_table),
+        page_table.shape[1], ring_pages, H, G, d, window, c_float(scale), _stream()))
+
+
+def attn_decode_mfma(q, k_pages, v_pages, out, partial, n_seq, n_splits, seq_slot, seq_pos0, cu_seqlens,
+                     page_table, ring_pages, H, G, d, window, scale) -> None:
+    _attn_check(q, k_pages, v_pages, out, page_table, H, G, d)
+    if n_splits > 1:
+        _dev("attn.partial", partial, torch.float32)
+        if partial.numel() < n_seq * H * n_splits * (d + 2):
+            raise KernelError("attn_decode: the partial buffer is too small")
+    if q.shape[0] < n_seq:
+        raise KernelError("attn_decode: fewer query rows than sequences")
+    for nm, t in (("seq_slot", seq_slot), ("seq_pos0", seq_pos0), ("cu_seqlens", cu_seqlens)):
+        _i32("attn." + nm, t, n_seq)
+    _check(lib().picolm_attn_decode_mfma(
+        _ptr(q), _ptr(k_pages), _ptr(v_pages), _ptr(out), _ptr(partial if n_splits > 1 else None), n_seq, n_splits,
+        _ptr(seq_slot), _ptr(seq_pos0), _ptr(cu_seqlens), _ptr(page_table), page_table.shape[1], ring_pages,
+        H, G, d, window, c_float(scale), _stream()))
+
+
 def attn_prefill(q, k_pages, v_pages, out, batch, page_table, ring_pages, H, G, d, window, scale) -> None:
     """Attention of a step's new tokens over their sequences' cache pages."""
+    if attn_mfma_takes(q, d):
+        attn_prefill_mfma(q, k_pages, v_pages, out, batch, page_table, ring_pages, H, G, d, window, scale)
+        return
     tile_seq, tile_q0, n_tiles = batch.prefill_tiles(attn_prefill_tile_rows())
     attn_prefill_generic(q, k_pages, v_pages, out, tile_seq, tile_q0, n_tiles, batch.seq_slot, batch.seq_pos0,
                          batch.seq_nnew, batch.cu_seqlens, page_table, ring_pages, H, G, d, window, scale)
@@ -292,8 +331,9 @@ def attn_prefill(q, k_pages, v_pages, out, batch, page_table, ring_pages, H, G, 
 def attn_decode(q, k_pages, v_pages, out, partial, n_seq, n_splits, seq_slot, seq_pos0, cu_seqlens,
                 page_table, ring_pages, H, G, d, window, scale) -> None:
     """Attention of one new token per sequence over its cache pages."""
-    attn_decode_generic(q, k_pages, v_pages, out, partial, n_seq, n_splits, seq_slot, seq_pos0, cu_seqlens,
-                        page_table, ring_pages, H, G, d, window, scale)
+    fn = attn_decode_mfma if attn_mfma_takes(q, d) else attn_decode_generic
+    fn(q, k_pages, v_pages, out, partial, n_seq, n_splits, seq_slot, seq_pos0, cu_seqlens,
+       page_table, ring_pages, H, G, d, window, scale)
 
 
 def sample(logits: torch.Tensor, out: torch.Tensor, temperature: float, top_k: int, top_p: float,

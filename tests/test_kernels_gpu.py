@@ -1,0 +1,333 @@
+"""Each hand-written kernel alone against a plain float64 reference, at sizes other than the
+tiny models': head sizes 16..256, odd head counts and groups, widths and vocabularies that are
+no power of two, ragged row counts."""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+from plain import llama_plain as P
+from plain import sampler_plain as SP
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+PAGE = 64
+
+
+def K():
+    from picolm_amd import kernels
+    return kernels
+
+
+def tol(dtype, scale):
+    return (2e-2 if dtype == torch.bfloat16 else 2e-5) * scale + (1e-3 if dtype == torch.bfloat16 else 1e-6)
+
+
+# ------------------------------------------------------------------------------------------ rows
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("T,D,V", [(1, 80, 131), (37, 4096, 500)])
+def test_embed(dtype, T, D, V):
+    g = torch.Generator().manual_seed(0)
+    table = torch.randn(V, D, generator=g).to(dtype).to(DEV)
+    tokens = torch.randint(0, V, (T,), generator=g, dtype=torch.int32).to(DEV)
+    out = torch.empty(T, D, device=DEV)
+    K().embed(table, tokens, out)
+    assert torch.equal(out, table.float()[tokens.long()])
+
+
+@pytest.mark.parametrize("out_dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("T,D,eps", [(1, 80, 1e-5), (19, 4096, 1e-6), (5, 1000, 1e-2)])
+def test_rmsnorm(out_dtype, T, D, eps):
+    g = torch.Generator().manual_seed(1)
+    x = (torch.randn(T, D, generator=g) * 3).to(DEV)
+    w = (1 + 0.3 * torch.randn(D, generator=g)).to(DEV)
+    out = torch.empty(T, D, dtype=out_dtype, device=DEV)
+    K().rmsnorm(x, w, eps, out)
+    ref = P.rmsnorm(x.cpu().numpy(), w.cpu().numpy(), eps)
+    err = np.abs(out.double().cpu().numpy() - ref).max()
+    assert err <= tol(out_dtype, np.abs(ref).max())
+    # selected rows
+    rows = torch.tensor([T - 1, 0], dtype=torch.int32, device=DEV)
+    out2 = torch.empty(2, D, dtype=out_dtype, device=DEV)
+    K().rmsnorm(x, w, eps, out2, rows)
+    assert torch.equal(out2[0], out[T - 1]) and torch.equal(out2[1], out[0])
+
+
+def test_silu_mul_and_add():
+    g = torch.Generator().manual_seed(2)
+    gu = torch.randn(7, 2 * 33, generator=g).to(DEV)
+    out = torch.empty(7, 33, device=DEV)
+    K().silu_mul(gu, out)
+    ref = P.silu(gu[:, 0::2].double().cpu().numpy()) * gu[:, 1::2].double().cpu().numpy()
+    assert np.abs(out.double().cpu().numpy() - ref).max() < 1e-6
+    y = torch.randn(5, 9, generator=g).to(DEV)
+    x = torch.randn(5, 9, generator=g).to(torch.bfloat16).to(DEV)
+    want = y + x.float()
+    K().add_into(y, x)
+    assert torch.equal(y, want)
+
+
+# ------------------------------------------------------------------------------------------ gemm
+def gemm_ref(a, w, epi, c0):
+    y = a.double().cpu() @ w.double().cpu().T
+    if epi == 1:
+        return c0.double().cpu() + y
+    if epi == 2:
+        g_, u = y[:, 0::2], y[:, 1::2]
+        return g_ / (1 + torch.exp(-g_)) * u
+    return y
+
+
+def run_gemm(fn, M, N, Kd, epi, adt, wdt, cdt, **kw):
+    g = torch.Generator().manual_seed(M * 7 + N)
+    a = torch.randn(M, Kd, generator=g).to(adt).to(DEV)
+    w = (torch.randn(N, Kd, generator=g) * 0.1).to(wdt).to(DEV)
+    c = torch.randn(M, N // 2 if epi == 2 else N, generator=g).to(cdt).to(DEV)
+    c0 = c.clone()
+    fn(a, w, c, epi, **kw)
+    ref = gemm_ref(a, w, epi, c0)
+    err = (c.double().cpu() - ref).abs().max().item()
+    assert err <= tol(cdt, ref.abs().max().item()), (M, N, Kd, epi, err)
+
+
+@pytest.mark.parametrize("M", [1, 3, 17, 64, 65, 200])
+@pytest.mark.parametrize("N,Kd", [(6, 5), (130, 77), (352, 176)])
+def test_gemm_generic_f32(M, N, Kd):
+    for epi in (0, 1, 2):
+        run_gemm(K().gemm_generic, M, N, Kd, epi, torch.float32, torch.float32, torch.float32)
+
+
+def test_gemm_generic_mixed_types():
+    for adt, wdt, cdt in [(torch.bfloat16, torch.float32, torch.float32), (torch.float32, torch.bfloat16, torch.bfloat16),
+                          (torch.bfloat16, torch.bfloat16, torch.bfloat16)]:
+        for epi in (0, 2):
+            run_gemm(K().gemm_generic, 9, 70, 45, epi, adt, wdt, cdt)
+    run_gemm(K().gemm_generic, 9, 70, 45, 1, torch.bfloat16, torch.float32, torch.float32)
+
+
+@pytest.mark.parametrize("M", [1, 2, 15, 16, 17, 33, 64])
+@pytest.mark.parametrize("N,Kd", [(96, 64), (130, 264), (1000, 1000), (4096, 1024)])
+def test_gemm_skinny(M, N, Kd):
+    for epi, cdt in ((0, torch.float32), (0, torch.bfloat16), (1, torch.float32), (2, torch.bfloat16)):
+        run_gemm(K().gemm_skinny, M, N, Kd, epi, torch.bfloat16, torch.bfloat16, cdt)
+
+
+@pytest.mark.parametrize("variant", [1, 2, 3, 4, 5, 6])
+def test_gemm_skinny_variants(variant):
+    M = {1: 16, 2: 13, 3: 32, 4: 21, 5: 64, 6: 50}[variant]
+    for epi, cdt in ((0, torch.float32), (2, torch.bfloat16), (1, torch.float32)):
+        run_gemm(K().gemm_skinny, M, 530, 1032, epi, torch.bfloat16, torch.bfloat16, cdt, variant=variant)
+
+
+@pytest.mark.parametrize("M", [65, 128, 300, 1111])
+@pytest.mark.parametrize("N,Kd", [(96, 64), (130, 264), (1000, 1000), (512, 2048)])
+def test_gemm_tiled(M, N, Kd):
+    for epi, cdt in ((0, torch.float32), (0, torch.bfloat16), (1, torch.float32), (2, torch.bfloat16)):
+        run_gemm(K().gemm_tiled, M, N, Kd, epi, torch.bfloat16, torch.bfloat16, cdt)
+
+
+def test_gemm_refuses_what_it_cannot_do():
+    k = K()
+    a = torch.zeros(4, 12, dtype=torch.bfloat16, device=DEV)
+    w = torch.zeros(8, 12, dtype=torch.bfloat16, device=DEV)
+    c = torch.zeros(4, 8, device=DEV)
+    with pytest.raises(k.KernelError):
+        k.gemm_skinny(a, w, c)                       # K = 12 is no multiple of 8
+    k.gemm(a, w, c)                                  # the dispatcher falls back to the float kernel
+    with pytest.raises(k.KernelError):
+        k.gemm_generic(a.cpu(), w, c)
+    with pytest.raises(k.KernelError):
+        k.gemm_generic(a, w, torch.zeros(4, 9, device=DEV))
+
+
+# ------------------------------------------------------------------------------------------ attention
+class PagedCase:
+    """Sequences with dense float64 q/k/v, and the same k/v scattered over shuffled cache pages."""
+
+    def __init__(self, H, G, d, lens_old, lens_new, dtype, seed=0, poison=True, scale_q=None):
+        rng = np.random.default_rng(seed)
+        self.H, self.G, self.d, self.dtype = H, G, d, dtype
+        n = len(lens_old)
+        self.totals = [a + b for a, b in zip(lens_old, lens_new)]
+        self.lens_old, self.lens_new = lens_old, lens_new
+        self.q = [rng.standard_normal((t, H, d)) for t in self.totals]
+        self.k = [rng.standard_normal((t, G, d)) for t in self.totals]
+        self.v = [rng.standard_normal((t, G, d)) for t in self.totals]
+        if scale_q is not None:
+            scale_q(self)
+        max_pages = max((t + PAGE - 1) // PAGE for t in self.totals)
+        n_pages = sum((t + PAGE - 1) // PAGE for t in self.totals) + 3
+        perm = rng.permutation(n_pages)
+        fill = float("nan") if poison else 0.0
+        kp = torch.full((n_pages, G, PAGE, d), fill, dtype=torch.float32)
+        vp = torch.full((n_pages, G, d, PAGE), fill, dtype=torch.float32)
+        table = torch.zeros((n + 2, max_pages), dtype=torch.int32)
+        self.slots = list(rng.permutation(n + 2)[:n])
+        nxt = 0
+        for i, t in enumerate(self.totals):
+            for j in range((t + PAGE - 1) // PAGE):
+                pg = int(perm[nxt]); nxt += 1
+                table[self.slots[i], j] = pg
+                m = min(PAGE, t - j * PAGE)
+                kp[pg, :, :m, :] = torch.from_numpy(self.k[i][j * PAGE:j * PAGE + m]).permute(1, 0, 2).float()
+                vp[pg, :, :, :m] = torch.from_numpy(self.v[i][j * PAGE:j * PAGE + m]).permute(1, 2, 0).float()
+        self.k_pages = kp.to(dtype).to(DEV)
+        self.v_pages = vp.to(dtype).to(DEV)
+        self.table = table.to(DEV)
+        # what the kernel sees after rounding to its storage type
+        rd = lambda x: torch.from_numpy(x).to(dtype).double().numpy()
+        self.q = [rd(x) for x in self.q]
+        self.k = [rd(x) for x in self.k]
+        self.v = [rd(x) for x in self.v]
+        qnew = np.concatenate([q[o:] for q, o in zip(self.q, lens_old)])
+        self.q_dev = torch.from_numpy(qnew).reshape(-1, H * d).to(dtype).to(DEV)
+
+    def batch(self):
+        from picolm_amd.engine.batch import StepBatch
+        toks = [[0] * n for n in self.lens_new]
+        return StepBatch([int(s) for s in self.slots], self.lens_old, toks, [[] for _ in toks], 10, DEV)
+
+    def reference(self, window=0):
+        outs = []
+        for q, k, v, o in zip(self.q, self.k, self.v, self.lens_old):
+            outs.append(P.causal_attention(q, k, v, window)[o:])
+        return np.concatenate(outs).reshape(-1, self.H * self.d)
+
+
+ATTN_SHAPES = [(4, 2, 16), (6, 6, 32), (3, 1, 32), (8, 2, 64), (32, 8, 128), (5, 5, 128), (2, 1, 256), (40, 1, 64)]
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("H,G,d", ATTN_SHAPES)
+@pytest.mark.parametrize("window", [0, 70])
+def test_attention_prefill(dtype, H, G, d, window):
+    case = PagedCase(H, G, d, [0, 0, 5, 130], [1, 200, 67, 33], dtype, seed=H + d)
+    b = case.batch()
+    out = torch.zeros_like(case.q_dev)
+    K().attn_prefill(case.q_dev, case.k_pages, case.v_pages, out, b, case.table, case.table.shape[1], H, G, d,
+                     window, 1.0 / math.sqrt(d))
+    ref = case.reference(window)
+    err = np.abs(out.double().cpu().numpy() - ref).max()
+    assert err <= tol(dtype, np.abs(ref).max()), err
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("H,G,d", ATTN_SHAPES)
+@pytest.mark.parametrize("n_splits,window", [(1, 0), (3, 0), (16, 0), (2, 100)])
+def test_attention_decode(dtype, H, G, d, n_splits, window):
+    case = PagedCase(H, G, d, [0, 63, 64, 700, 129], [1, 1, 1, 1, 1], dtype, seed=H * d + n_splits)
+    b = case.batch()
+    out = torch.zeros_like(case.q_dev)
+    partial = torch.full((b.n_seq * H * n_splits * (d + 2),), float("nan"), device=DEV)
+    K().attn_decode(case.q_dev, case.k_pages, case.v_pages, out, partial, b.n_seq, n_splits, b.seq_slot, b.seq_pos0,
+                    b.cu_seqlens, case.table, case.table.shape[1], H, G, d, window, 1.0 / math.sqrt(d))
+    ref = case.reference(window)
+    err = np.abs(out.double().cpu().numpy() - ref).max()
+    assert err <= tol(dtype, np.abs(ref).max()), err
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_attention_finds_a_far_key(dtype):
+    """One key among hundreds is made to dominate: the output must be its value row.  A kernel
+    that drops a page, a split or the window's edge returns something else."""
+    H, G, d = 4, 2, 64
+    target = 130
+
+    def boost(c):
+        for i in range(len(c.totals)):
+            if c.totals[i] > target:
+                c.k[i][target] = 0.0
+                c.k[i][target, :, 0] = 30.0
+                c.q[i][-1] = 0.0
+                c.q[i][-1, :, 0] = 30.0
+    case = PagedCase(H, G, d, [699], [1], dtype, seed=3, scale_q=boost)
+    b = case.batch()
+    for n_splits in (1, 4):
+        out = torch.zeros_like(case.q_dev)
+        partial = torch.zeros(b.n_seq * H * n_splits * (d + 2), device=DEV)
+        K().attn_decode(case.q_dev, case.k_pages, case.v_pages, out, partial, 1, n_splits, b.seq_slot, b.seq_pos0,
+                        b.cu_seqlens, case.table, case.table.shape[1], H, G, d, 0, 1.0 / math.sqrt(d))
+        got = out.double().cpu().numpy().reshape(H, d)
+        for h in range(H):
+            assert np.abs(got[h] - case.v[0][target, h // 2]).max() < 2e-2
+
+
+# ------------------------------------------------------------------------------------------ rope
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("style", ["pairwise", "half"])
+def test_rope_kv_store(dtype, style):
+    from picolm_amd.engine.batch import StepBatch
+    H, G, d = 3, 1, 32
+    rng = np.random.default_rng(0)
+    slots, pos0, n_new = [2, 0], [61, 0], [5, 70]
+    T = sum(n_new)
+    qkv = rng.standard_normal((T, (H + 2 * G) * d)).astype(np.float32)
+    inv = P.rope_inv_freq(d, 1000.0)
+    b = StepBatch(slots, pos0, [[0] * n for n in n_new], [[], []], 10, DEV)
+    positions = np.concatenate([np.arange(p, p + n) for p, n in zip(pos0, n_new)])
+    cos, sin = P.rope_tables(np.arange(200), inv)
+    table = torch.tensor([[4, 1], [0, 0], [3, 5]], dtype=torch.int32, device=DEV)
+    kp = torch.zeros(6, G, PAGE, d, dtype=dtype, device=DEV)
+    vp = torch.zeros(6, G, d, PAGE, dtype=dtype, device=DEV)
+    q_out = torch.zeros(T, H * d, dtype=dtype, device=DEV)
+    K().rope_kv_store(torch.from_numpy(qkv).to(DEV), q_out, kp, vp, torch.from_numpy(cos).float().to(DEV),
+                      torch.from_numpy(sin).float().to(DEV), 0 if style == "pairwise" else 1, b.tok_pos, b.tok_seq,
+                      b.seq_slot, table, 2, H, G, d)
+    x = qkv.astype(np.float64).reshape(T, H + 2 * G, d)
+    c, s = P.rope_tables(positions, inv)
+    q_ref = P.apply_rope(x[:, :H], c, s, style).reshape(T, H * d)
+    k_ref = P.apply_rope(x[:, H:H + G], c, s, style)
+    v_ref = x[:, H + G:]
+    t_ = tol(dtype, 4.0)
+    assert np.abs(q_out.double().cpu().numpy() - q_ref).max() <= t_
+    kp, vp, tab = kp.double().cpu().numpy(), vp.double().cpu().numpy(), table.cpu().numpy()
+    seq_of = np.repeat(np.arange(2), n_new)
+    for t in range(T):
+        pg = tab[slots[seq_of[t]], positions[t] // PAGE]
+        assert np.abs(kp[pg, :, positions[t] % PAGE, :] - k_ref[t]).max() <= t_
+        assert np.abs(vp[pg, :, :, positions[t] % PAGE] - v_ref[t]).max() <= t_
+
+
+# ------------------------------------------------------------------------------------------ sampling
+def test_argmax_first_maximum():
+    lg = torch.zeros(3, 1001)
+    lg[0, 17] = lg[0, 900] = 2.0
+    lg[1, :] = -1.0
+    lg[2, 1000] = 5.0
+    out = torch.zeros(3, dtype=torch.int32, device=DEV)
+    K().argmax(lg.to(DEV), out)
+    assert out.tolist() == [17, 0, 1000]
+
+
+@pytest.mark.parametrize("V,scale", [(131, 1.0), (5000, 0.5), (128256, 1.0)])
+@pytest.mark.parametrize("opts", [(0.8, 0, 1.0, 0.0), (0.8, 40, 0.9, 0.05), (1.3, 0, 0.7, 0.0), (0.5, 7, 1.0, 0.2),
+                                  (1.0, 0, 1.0, 0.3), (0.0, 0, 1.0, 0.0)])
+def test_sampler_equals_plain(V, scale, opts):
+    from picolm_amd.sampling import Sampler, SamplingParams, stream_state
+    T, k, p, mp = opts
+    rng = np.random.default_rng(V)
+    n = 5 if V > 10000 else 16
+    logits = (rng.standard_normal((n, V)) * scale).astype(np.float32)
+    logits[0, :] = 0.25                 # all equal
+    logits[1, ::2] = logits[1, 1]       # many equal
+    logits[2, 5] = 40.0                 # one dominates
+    smp = Sampler(SamplingParams(T, k, p, mp, seed=7), n, DEV)
+    lg = torch.from_numpy(logits).to(DEV)
+    states = [stream_state(7, i) for i in range(n)]
+    for _ in range(3):
+        got = smp.sample(lg, list(range(n)))
+        for i in range(n):
+            want, states[i] = SP.sample(logits[i], T, k, p, mp, states[i])
+            assert got[i] == want, (i, got[i], want)
+
+
+def test_sampler_streams_do_not_depend_on_the_batch():
+    from picolm_amd.sampling import Sampler, SamplingParams
+    rng = np.random.default_rng(0)
+    logits = torch.from_numpy(rng.standard_normal((4, 300)).astype(np.float32)).to(DEV)
+    a = Sampler(SamplingParams(1.0, seed=3), 4, DEV)
+    b = Sampler(SamplingParams(1.0, seed=3), 4, DEV)
+    full = [a.sample(logits, [0, 1, 2, 3]) for _ in range(4)]
+    part = [b.sample(logits[[1, 3]], [1, 3]) for _ in range(4)]
+    assert [[f[1], f[3]] for f in full] == part
