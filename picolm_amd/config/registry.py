@@ -26,6 +26,7 @@ _REGISTRY: dict[str, Architecture] = {}
 
 
 def register_architecture(name: str, parse_config, build, *, replace: bool = False) -> Architecture:
+    _load_builtin()
     if name in _REGISTRY and not replace:
         raise ConfigError(f"architecture '{name}' is already registered")
     arch = Architecture(name, parse_config, build)
@@ -37,7 +38,19 @@ def unregister_architecture(name: str) -> None:
     _REGISTRY.pop(name, None)
 
 
+_BUILTIN_LOADED = False
+
+
+def _load_builtin() -> None:
+    """The architectures that ship with the library register themselves when imported."""
+    global _BUILTIN_LOADED
+    if not _BUILTIN_LOADED:
+        _BUILTIN_LOADED = True
+        from ..engine import llama  # noqa: F401
+
+
 def known_architectures() -> list[str]:
+    _load_builtin()
     return sorted(_REGISTRY)
 
 
@@ -52,6 +65,7 @@ def architecture_name(config_dict: dict) -> str:
 
 
 def resolve(config_dict: dict) -> Architecture:
+    _load_builtin()
     name = architecture_name(config_dict)
     if name not in _REGISTRY:
         raise ConfigError(f"architectures: '{name}' is not registered "

@@ -1,0 +1,290 @@
+"""The engine against the plain implementation on the GPU, in 32-bit and in bfloat16, under
+every way of cutting the work: each request whole; its last 32 tokens one by one; batches of
+unequal lengths whose shorter requests end earlier, one batch after another in a cache that
+only holds one batch, so that slots and pages are used again.  The first three go through
+bin/trace_run as a subprocess, the rest through the library in this process."""
+import json
+import os
+import subprocess
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+import tiny
+from plain import llama_plain as P
+from plain import sampler_plain as SP
+from replay_util import ROOT, TraceRun
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+LENGTHS = {"A": [33, 47, 64, 65, 100, 128], "B": [33, 40, 64, 129, 200, 256], "C": [34, 63, 65, 128, 190, 300]}
+
+
+def tolerance(dtype, ref):
+    scale = max(1.0, float(np.abs(ref).max()))
+    return (2e-5 if dtype == "float32" else 2e-2) * scale
+
+
+@pytest.fixture(scope="module")
+def folders(tmp_path_factory):
+    tmp = tmp_path_factory.mktemp("models")
+    return {w: tiny.make_model_dir(tmp, w) for w in "ABC"}
+
+
+@pytest.fixture(scope="module")
+def requests_and_truth(folders):
+    out = {}
+    for w, d in folders.items():
+        V = tiny.read_config(d)["vocab_size"]
+        rng = np.random.default_rng(ord(w))
+        reqs = [tiny.random_tokens(rng, n, V) for n in LENGTHS[w]]
+        out[w] = (reqs, [tiny.plain_logits(d, r) for r in reqs])
+    return out
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("which", ["A", "B", "C"])
+def test_replay_whole_tail_and_batches(which, dtype, folders, requests_and_truth, tmp_path):
+    reqs, truth = requests_and_truth[which]
+    one_batch = sum((len(r) + 63) // 64 for r in reqs[3:]) * 64          # room for the larger batch only
+    tr = TraceRun(folders[which], dtype, str(tmp_path / "out"), one_batch)
+    worst = 0.0
+
+    def check(got, ref, what):
+        nonlocal worst
+        err = float(np.abs(got.astype(np.float64) - ref).max())
+        worst = max(worst, err)
+        assert err <= tolerance(dtype, ref), f"{which} {dtype} {what}: {err}"
+    # 1. each request alone and whole, every position wanted
+    for i, r in enumerate(reqs):
+        got = tr.step([(f"w{i}", r, range(len(r)))], end=[f"w{i}"])
+        check(got, truth[i], f"whole request {i}")
+    # 2. each request alone, the last 32 tokens one by one
+    for i, r in enumerate(reqs):
+        n0 = len(r) - 32
+        got = tr.step([(f"t{i}", r[:n0], [n0 - 1])])
+        check(got, truth[i][n0 - 1:n0], f"tail request {i} prompt")
+        for j in range(n0, len(r)):
+            got = tr.step([(f"t{i}", [r[j]], [0])], end=[f"t{i}"] if j == len(r) - 1 else [])
+            check(got, truth[i][j:j + 1], f"tail request {i} position {j}")
+    # 3. two batches of unequal lengths, one after the other; requests decode 3, 9, 20 tokens
+    for ids in ([0, 1, 2], [3, 4, 5]):
+        n_dec = dict(zip(ids, (3, 9, 20)))
+        pos = {i: len(reqs[i]) - n_dec[i] for i in ids}
+        got = tr.step([(f"b{i}", reqs[i][:pos[i]], [0, pos[i] - 1]) for i in ids])
+        for k, i in enumerate(ids):
+            check(got[2 * k:2 * k + 2], truth[i][[0, pos[i] - 1]], f"batch prompt of request {i}")
+        live = list(ids)
+        while live:
+            ending = [i for i in live if pos[i] == len(reqs[i]) - 1]
+            got = tr.step([(f"b{i}", [reqs[i][pos[i]]], [0]) for i in live], end=[f"b{i}" for i in ending])
+            for k, i in enumerate(live):
+                check(got[k:k + 1], truth[i][pos[i]:pos[i] + 1], f"batch decode of request {i} at {pos[i]}")
+                pos[i] += 1
+            live = [i for i in live if i not in ending]
+    # a step that wants nothing writes nothing
+    assert tr.step([("z", reqs[0][:5], [])], end=["z"]) is None
+    tr.close()
+    print(f"{which} {dtype}: worst error {worst:.3e}")
+
+
+def test_replay_reports_a_full_cache(folders, tmp_path):
+    tr = TraceRun(folders["A"], "float32", str(tmp_path / "o"), 64)
+    assert tr.step([("a", [1] * 60, [59])]).shape == (1, 256)
+    with pytest.raises(RuntimeError):
+        tr.step([("b", [1] * 10, [0])])          # no page left: the program stops with an error
+    assert tr.proc.wait(timeout=60) != 0
+
+
+# -------------------------------------------------------------------------------------------
+def session(folder, dtype, max_tokens=2048, **kw):
+    from picolm_amd.engine import Session, load_model
+    return Session(load_model(folder, dtype=dtype), max_tokens=max_tokens, **kw)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_long_decoding_and_first_tokens(dtype, folders):
+    d = folders["C"]
+    rng = np.random.default_rng(11)
+    toks = tiny.random_tokens(rng, 400, tiny.TINY_C["vocab_size"])
+    ref = tiny.plain_logits(d, toks)
+    s = session(d, dtype)
+    [a] = s.begin(1)
+    for j, t in enumerate(toks):                 # a prompt of one token, then 399 single steps
+        got = s.step([a], [[t]]).double().cpu().numpy()
+        err = np.abs(got[0] - ref[j]).max()
+        assert err <= tolerance(dtype, ref), (j, err)
+    assert s.length(a) == 400
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_stale_cache_contents_change_nothing(dtype, folders):
+    d = folders["B"]
+    rng = np.random.default_rng(12)
+    V = tiny.TINY_B["vocab_size"]
+    s = session(d, dtype, max_tokens=256)
+    for g in s.cache.kv:                         # whatever a freed slot leaves behind must not matter
+        g.k.fill_(float("nan"))
+        g.v.fill_(float("nan"))
+    for n in (70, 3, 129):
+        toks = tiny.random_tokens(rng, n, V)
+        ref = tiny.plain_logits(d, toks)
+        [a] = s.begin(1)
+        got = s.step([a], [toks[:-1]], [list(range(n - 1))]).double().cpu().numpy() if n > 1 else None
+        last = s.step([a], [[toks[-1]]]).double().cpu().numpy()
+        s.release([a])
+        assert np.abs(got - ref[:-1]).max() <= tolerance(dtype, ref)
+        assert np.abs(last[0] - ref[-1]).max() <= tolerance(dtype, ref)
+
+
+def test_padding_free_batch_equals_each_alone_bitwise_in_f32(folders):
+    """What else is in the batch may change a result by rounding only; with the float kernels,
+    whose summation order per row does not depend on the batch, not at all."""
+    d = folders["A"]
+    rng = np.random.default_rng(13)
+    prompts = [tiny.random_tokens(rng, n, 256) for n in (5, 11, 17)]
+    s = session(d, "float32")
+    alone = []
+    for p in prompts:
+        [a] = s.begin(1)
+        alone.append(s.step([a], [p]).clone())
+        s.release([a])
+    slots = s.begin(3)
+    together = s.step(slots, prompts)
+    for i in range(3):
+        assert torch.equal(together[i], alone[i][0])
+
+
+def test_step_errors(folders):
+    from picolm_amd.cache import CacheFull
+    from picolm_amd.engine import StepError
+    s = session(folders["A"], "float32", max_tokens=128)
+    [a] = s.begin(1)
+    with pytest.raises(StepError, match="vocabulary"):
+        s.step([a], [[1, 256]])
+    with pytest.raises(StepError, match="not live"):
+        s.step([5], [[1]])
+    with pytest.raises(StepError, match="twice"):
+        s.step([a, a], [[1], [2]])
+    with pytest.raises(CacheFull):
+        s.step([a], [[1] * 129])                 # longer than max_position_embeddings / the cache
+    assert s.length(a) == 0                      # a refused step leaves the sequence where it was
+    s.step([a], [[1] * 128])
+    with pytest.raises(CacheFull):
+        s.step([a], [[1]])
+
+
+# ------------------------------------------------------------------------------------------- generation
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_greedy_generation_through_the_entry_point(dtype, folders):
+    from picolm_amd.engine import load_model
+    from picolm_amd.generation import generate
+    d = folders["A"]
+    rng = np.random.default_rng(0)
+    prompts = [tiny.random_tokens(rng, n, 256) for n in (5, 11, 17)]       # BASELINE's tiny workload: 8 greedy steps
+    model = load_model(d, dtype=dtype)
+    got = generate(model, prompts, max_new_tokens=8, stop_ids=())
+    for p, r in zip(prompts, got):
+        seq = list(p)
+        for k in range(8):
+            lg = tiny.plain_logits(d, seq)[-1]
+            top2 = np.sort(lg)[-2:]
+            if top2[1] - top2[0] < 2 * tolerance(dtype, lg):
+                break                              # a near tie: either choice is right
+            assert r.tokens[k] == int(np.argmax(lg)), (k, r.tokens)
+            seq.append(r.tokens[k])
+        assert len(r.tokens) == 8 and r.finish == "length"
+
+
+def test_temperature_generation_follows_the_plain_sampler(folders):
+    """Tiny B's workload: prompts of 1/9/30/64 tokens, 12 steps at temperature 0.8, fixed seed.
+    Each sampled token must be what the plain sampler draws from the plain logits of the
+    engine's own sequence so far, with that request's generator stream."""
+    from picolm_amd.engine import load_model
+    from picolm_amd.generation import generate
+    from picolm_amd.sampling import SamplingParams, stream_state
+    d = folders["B"]
+    rng = np.random.default_rng(1)
+    prompts = [tiny.random_tokens(rng, n, 384) for n in (1, 9, 30, 64)]
+    model = load_model(d, dtype="float32")
+    for batch_size in (4, 3):                     # the streams do not depend on the batching
+        got = generate(model, prompts, max_new_tokens=12, params=SamplingParams(temperature=0.8, seed=5), stop_ids=(),
+                       batch_size=batch_size)
+        for i, (p, r) in enumerate(zip(prompts, got)):
+            state = stream_state(5, i)
+            seq = list(p)
+            for k in range(12):
+                lg = tiny.plain_logits(d, seq)[-1]
+                want, state = SP.sample(lg, 0.8, 0, 1.0, 0.0, state)
+                assert want == r.tokens[k], f"request {i} token {k}: engine {r.tokens[k]} plain {want}"
+                seq.append(want)
+
+
+def test_stop_tokens_end_sequences_early(folders):
+    from picolm_amd.engine import load_model
+    from picolm_amd.generation import generate
+    d = folders["A"]
+    model = load_model(d, dtype="float32")
+    rng = np.random.default_rng(2)
+    prompts = [tiny.random_tokens(rng, n, 256) for n in (4, 9, 15, 6)]
+    free = generate(model, prompts, max_new_tokens=10, stop_ids=())
+    stop = free[1].tokens[3]                      # make request 1 stop at its fourth token
+    got = generate(model, prompts, max_new_tokens=10, stop_ids=[stop], batch_size=2)
+    for f, g in zip(free, got):
+        if stop in f.tokens:
+            cut = f.tokens.index(stop) + 1
+            assert g.tokens == f.tokens[:cut] and g.finish == "stop"
+        else:
+            assert g.tokens == f.tokens and g.finish == "length"
+    assert got[1].finish == "stop" and len(got[1].tokens) <= 4
+
+
+def test_command_line(folders, tmp_path):
+    d = folders["A"]
+    env = dict(os.environ, PYTHONPATH=ROOT)
+    r = subprocess.run([sys.executable, os.path.join(ROOT, "bin", "picolm"), d, "-p", "5 17, 3", "-n", "6", "-t", "0",
+                        "--dtype", "float32"], capture_output=True, text=True, env=env, timeout=300)
+    assert r.returncode == 0, r.stderr
+    toks = [int(t) for t in r.stdout.split()]
+    seq = [5, 17, 3]
+    for t in toks:
+        if t == 2:                                 # the configuration's stop token
+            break
+        assert t == int(np.argmax(tiny.plain_logits(d, seq)[-1]))
+        seq.append(t)
+    assert len(toks) <= 6 and "Prefill: 3 tokens" in r.stderr and "Generation:" in r.stderr
+    # several prompts from standard input make a batch; a seed makes sampling repeatable
+    cmd = [sys.executable, "-m", "picolm_amd", d, "-n", "5", "-s", "7", "--dtype", "float32", "--json"]
+    a = subprocess.run(cmd, input="1 2 3\n9 8\n", capture_output=True, text=True, env=env, timeout=300, cwd=ROOT)
+    b = subprocess.run(cmd, input="1 2 3\n9 8\n", capture_output=True, text=True, env=env, timeout=300, cwd=ROOT)
+    assert a.returncode == 0 and a.stdout == b.stdout or json.loads(a.stdout)["tokens"] == json.loads(b.stdout)["tokens"]
+    assert len(json.loads(a.stdout)["tokens"]) == 2
+    # the random-weights mode writes a folder that loads
+    cfg = tmp_path / "c.json"
+    cfg.write_text(json.dumps(tiny.TINY_C))
+    w = subprocess.run([sys.executable, "-m", "picolm_amd", "--random-model", str(tmp_path / "m"), "--config", str(cfg),
+                        "-s", "3"], capture_output=True, text=True, env=env, timeout=300, cwd=ROOT)
+    assert w.returncode == 0, w.stderr
+    ls = subprocess.run([sys.executable, "-m", "picolm_amd", str(tmp_path / "m"), "--list-tensors"], capture_output=True,
+                        text=True, env=env, timeout=300, cwd=ROOT)
+    assert "model.layers.0.self_attn.q_proj.weight\t[96, 80]\tbfloat16" in ls.stdout
+
+
+def test_missing_tensor_is_reported_when_loading(folders, tmp_path):
+    from safetensors.torch import load_file, save_file
+    from picolm_amd import WeightsError
+    from picolm_amd.engine import load_model
+    d = str(tmp_path / "broken")
+    os.makedirs(d)
+    w = load_file(os.path.join(folders["A"], "model.safetensors"))
+    del w["model.layers.1.mlp.gate_proj.weight"]
+    w["model.layers.0.self_attn.v_proj.weight"] = w["model.layers.0.self_attn.v_proj.weight"][:16].contiguous()
+    save_file(w, os.path.join(d, "model.safetensors"))
+    open(os.path.join(d, "config.json"), "w").write(open(os.path.join(folders["A"], "config.json")).read())
+    with pytest.raises(WeightsError) as e:
+        load_model(d)
+    assert e.value.missing == ["model.layers.1.mlp.gate_proj.weight"]
+    assert e.value.wrong_shape == [("model.layers.0.self_attn.v_proj.weight", (32, 64), (16, 64))]

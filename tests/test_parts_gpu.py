@@ -1,0 +1,268 @@
+"""Each part of a layer alone against its plain function, and a toy architecture whose mixer
+keeps state of its own: defined, registered, built, loaded from a random model folder and
+stepped here, without a change to the library's files."""
+import json
+import math
+import os
+
+import numpy as np
+import pytest
+import torch
+
+import tiny
+from plain import llama_plain as P
+
+pytestmark = pytest.mark.gpu
+DEV = torch.device("cuda:0")
+
+
+def harness(dtype, requests, slots, pos0, new_lens, n_slots=4, max_tokens=1024):
+    """A step context over a fresh cache that holds what `requests` ask for."""
+    from picolm_amd.cache import Cache, CacheSpec, KVGroupSpec, StateGroupSpec
+    from picolm_amd.engine.batch import StepBatch
+    from picolm_amd.parts import CacheBinding, Runtime, StepContext, Workspace
+    kv_req, st_req = requests
+    spec = CacheSpec([KVGroupSpec(1, kv_req.n_kv_heads, kv_req.head_dim, kv_req.window)] if kv_req else [],
+                     [StateGroupSpec(1, tuple(st_req.shape), st_req.dtype)] if st_req else [])
+    rt = Runtime(DEV, dtype)
+    cache = Cache(spec, max_tokens, 512, dtype, DEV, n_slots)
+    for _ in range(n_slots):
+        cache.alloc_slot()
+    cache.reserve_many(slots, [p + n for p, n in zip(pos0, new_lens)])
+    cache.flush()
+    batch = StepBatch(slots, pos0, [[0] * n for n in new_lens], [[] for _ in slots], 10, DEV)
+    ctx = StepContext(rt, batch, cache, Workspace(DEV))
+    ctx.binding = CacheBinding((0, 0) if kv_req else None, (0, 0) if st_req else None, True)
+    return rt, ctx
+
+
+def tol(dtype, ref):
+    return (3e-5 if dtype == torch.float32 else 3e-2) * max(1.0, float(np.abs(ref).max()))
+
+
+def rounded(x, dtype):
+    return torch.from_numpy(x).to(dtype).double().numpy()
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_rmsnorm_part(dtype):
+    from picolm_amd.parts import RMSNorm
+    from picolm_amd.weights import TensorDict, WeightFetcher
+    rng = np.random.default_rng(0)
+    w = rng.standard_normal(96)
+    x = rng.standard_normal((7, 96)) * 4
+    rt, ctx = harness(dtype, (None, None), [0], [0], [7])
+    part = RMSNorm("n.weight", 96, 1e-3)
+    assert [(s.name, s.shape, s.init) for s in part.tensor_specs()] == [("n.weight", (96,), "ones")]
+    part.load_all(WeightFetcher(TensorDict({"n.weight": torch.from_numpy(w).to(torch.bfloat16)}), DEV), rt)
+    out = part.forward(ctx, torch.from_numpy(x).float().to(DEV))
+    ref = P.rmsnorm(x.astype(np.float32), rounded(w, torch.bfloat16), 1e-3)
+    assert out.dtype == dtype and np.abs(out.double().cpu().numpy() - ref).max() <= tol(dtype, ref)
+    shifted = RMSNorm("n.weight", 96, 1e-3, weight_offset=1.0)            # the convention of other architectures
+    shifted.load_all(WeightFetcher(TensorDict({"n.weight": torch.from_numpy(w).float()}), DEV), rt)
+    out = shifted.forward(ctx, torch.from_numpy(x).float().to(DEV))
+    ref = P.rmsnorm(x.astype(np.float32), w.astype(np.float32).astype(np.float64) + 1.0, 1e-3)
+    assert np.abs(out.double().cpu().numpy() - ref).max() <= tol(dtype, ref)
+
+
+def test_rotary_tables():
+    from picolm_amd.config import RopeScaling
+    from picolm_amd.parts import RotaryEmbedding, Runtime
+    sc = dict(rope_type="llama3", factor=8.0, low_freq_factor=1.0, high_freq_factor=4.0, original_max_position_embeddings=64)
+    for d, theta, scaling in ((16, 10000.0, None), (32, 500000.0, sc), (128, 500000.0, dict(sc, original_max_position_embeddings=8192))):
+        rot = RotaryEmbedding(d, theta, RopeScaling.from_dict(scaling), "half")
+        rot.prepare(Runtime(DEV, torch.float32), 300)
+        cos, sin, style = rot.rotary_tables()
+        assert style == 1 and tuple(cos.shape) == (300, d // 2)
+        rc, rs = P.rope_tables(np.arange(300), P.rope_inv_freq(d, theta, scaling))
+        # the engine's angle is a 32-bit product: half an ulp of the largest angle
+        assert np.abs(cos.double().cpu().numpy() - rc).max() < 300 * 2.0 ** -24 + 1e-7
+        assert np.abs(sin.double().cpu().numpy() - rs).max() < 300 * 2.0 ** -24 + 1e-7
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("H,G,d,style,window", [(4, 2, 16, "pairwise", 0), (6, 6, 32, "half", 0), (8, 2, 64, "pairwise", 0),
+                                                (3, 1, 32, "half", 40)])
+def test_attention_part(dtype, H, G, d, style, window):
+    from picolm_amd.parts import Attention, RotaryEmbedding
+    from picolm_amd.weights import TensorDict, WeightFetcher
+    rng = np.random.default_rng(H * d)
+    D = 80
+    names = ["a.q_proj.weight", "a.k_proj.weight", "a.v_proj.weight", "a.o_proj.weight"]
+    shapes = [(H * d, D), (G * d, D), (G * d, D), (D, H * d)]
+    w = {n: rounded(rng.standard_normal(s) * 0.2, torch.bfloat16) for n, s in zip(names, shapes)}
+    part = Attention("a.", D, H, G, d, position=RotaryEmbedding(d, 1000.0, None, style), window=window)
+    assert sorted(s.name for s in part.all_specs()) == sorted(names)
+    lens = [70, 9] if window == 0 else [40, 9]          # a windowed step must fit its ring
+    rt, ctx = harness(dtype, part.cache_requests(), [2, 0], [0, 0], lens)
+    part.load_all(WeightFetcher(TensorDict({k: torch.from_numpy(v).to(torch.bfloat16) for k, v in w.items()}), DEV), rt)
+    part.prepare(rt, 512)
+    hs = [rounded(rng.standard_normal((n, D)), dtype) for n in lens]
+    h = torch.from_numpy(np.concatenate(hs)).to(dtype).to(DEV)
+    res = torch.zeros(sum(lens), D, device=DEV)
+    part.forward(ctx, h, res)
+    cfg = dict(num_attention_heads=H, num_key_value_heads=G, head_dim=d, rope_theta=1000.0, rope_style=style, window=window)
+    pw = {"self_attn." + k[2:]: v for k, v in w.items()}
+    ref = np.concatenate([P.attention_block(x, pw, "self_attn.", cfg, np.arange(len(x))) for x in hs])
+    assert np.abs(res.double().cpu().numpy() - ref).max() <= tol(dtype, ref)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_swiglu_and_block_parts(dtype):
+    from picolm_amd.parts import Attention, NoPosition, PreNormBlock, RMSNorm, SwiGLU
+    from picolm_amd.weights import TensorDict, WeightFetcher
+    rng = np.random.default_rng(5)
+    D, F, H, G, d = 48, 104, 3, 3, 16
+    shapes = {"f.gate_proj.weight": (F, D), "f.up_proj.weight": (F, D), "f.down_proj.weight": (D, F),
+              "a.q_proj.weight": (H * d, D), "a.k_proj.weight": (G * d, D), "a.v_proj.weight": (G * d, D),
+              "a.o_proj.weight": (D, H * d), "n1": (D,), "n2": (D,)}
+    w = {n: rounded(rng.standard_normal(s) * 0.3, torch.bfloat16) for n, s in shapes.items()}
+    ffn = SwiGLU("f.", D, F)
+    block = PreNormBlock(RMSNorm("n1", D, 1e-5), Attention("a.", D, H, G, d, position=NoPosition()), RMSNorm("n2", D, 1e-5), ffn)
+    rt, ctx = harness(dtype, block.mixer.cache_requests(), [1], [0], [21])
+    block.load_all(WeightFetcher(TensorDict({k: torch.from_numpy(v).to(torch.bfloat16) for k, v in w.items()}), DEV), rt)
+    block.mixer.prepare(rt, 512)
+    x = rng.standard_normal((21, D))
+    # the feed-forward alone
+    hin = rounded(x, dtype)
+    res = torch.zeros(21, D, device=DEV)
+    ffn.forward(ctx, torch.from_numpy(hin).to(dtype).to(DEV), res)
+    ref = P.swiglu(hin, w["f.gate_proj.weight"], w["f.up_proj.weight"], w["f.down_proj.weight"])
+    assert np.abs(res.double().cpu().numpy() - ref).max() <= tol(dtype, ref)
+    # the block: x += attn(norm(x)); x += ffn(norm(x)), here without any rotation
+    xf = x.astype(np.float32).astype(np.float64)
+    xt = torch.from_numpy(xf).float().to(DEV)
+    block.forward(ctx, xt)
+    hh = P.rmsnorm(xf, w["n1"], 1e-5)
+    T = len(xf)
+    q = (hh @ w["a.q_proj.weight"].T).reshape(T, H, d)
+    k = (hh @ w["a.k_proj.weight"].T).reshape(T, G, d)
+    v = (hh @ w["a.v_proj.weight"].T).reshape(T, G, d)
+    y = xf + P.causal_attention(q, k, v).reshape(T, H * d) @ w["a.o_proj.weight"].T
+    y = y + P.swiglu(P.rmsnorm(y, w["n2"], 1e-5), w["f.gate_proj.weight"], w["f.up_proj.weight"], w["f.down_proj.weight"])
+    assert np.abs(xt.double().cpu().numpy() - y).max() <= tol(dtype, y)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_embedding_and_head_parts(dtype):
+    from picolm_amd.parts import LMHead, TokenEmbedding
+    from picolm_amd.weights import TensorDict, WeightFetcher
+    rng = np.random.default_rng(6)
+    V, D = 131, 40
+    e, hd = rounded(rng.standard_normal((V, D)), torch.bfloat16), rounded(rng.standard_normal((V, D)), torch.bfloat16)
+    rt, ctx = harness(dtype, (None, None), [0], [0], [5])
+    for tied, have_head in ((True, False), (False, True), (False, False), (True, True)):
+        emb = TokenEmbedding("e", V, D)
+        head = LMHead("h", V, D, emb, tied)
+        t = {"e": torch.from_numpy(e).to(torch.bfloat16)}
+        if have_head:
+            t["h"] = torch.from_numpy(hd).to(torch.bfloat16)
+        f = WeightFetcher(TensorDict(t), DEV)
+        emb.load_all(f, rt)
+        head.load_all(f, rt)
+        toks = torch.tensor([3, 130, 0, 7, 7], dtype=torch.int32, device=DEV)
+        x = emb.forward(ctx, toks, 5)
+        assert x.dtype == torch.float32 and np.array_equal(x.double().cpu().numpy(), e[[3, 130, 0, 7, 7]])
+        hrows = rounded(rng.standard_normal((5, D)), dtype)
+        lg = head.forward(ctx, torch.from_numpy(hrows).to(dtype).to(DEV))
+        table = hd if (have_head and not tied) else e
+        ref = hrows @ table.T
+        assert np.abs(lg.double().cpu().numpy() - ref).max() <= tol(dtype, ref)
+
+
+# ------------------------------------------------------------------------------------------- a toy architecture
+def test_toy_architecture_with_a_stateful_mixer(tmp_path):
+    """A mixer that keeps, per sequence, the running sum of its inputs and their count: its
+    output at a position is W times the mean of all inputs so far.  It needs no keys or
+    values, only a state row per slot.  The layer order names its block twice and the second
+    call has a state entry of its own."""
+    from picolm_amd.config import register_architecture, unregister_architecture
+    from picolm_amd.engine import DecoderModel, Session, load_model
+    from picolm_amd.parts import LMHead, Mixer, PreNormBlock, RMSNorm, StateRequest, SwiGLU, TokenEmbedding
+    from picolm_amd.weights import TensorSpec, write_random_model
+
+    class ToyConfig:
+        def __init__(self, d):
+            self.d = dict(d)
+            self.hidden_size, self.vocab_size, self.intermediate_size = d["hidden_size"], d["vocab_size"], d["intermediate_size"]
+            self.max_position_embeddings = d["max_position_embeddings"]
+            self.torch_dtype = "bfloat16"
+            self.eos_token_ids = ()
+
+        def to_dict(self):
+            return dict(self.d)
+
+    class RunningMean(Mixer):
+        def __init__(self, name, D):
+            self.name, self.D, self.w = name, D, None
+
+        def tensor_specs(self):
+            return [TensorSpec(self.name, (self.D, self.D))]
+
+        def load(self, fetch, runtime):
+            self.w = fetch.get(self.name).float()
+
+        def cache_requests(self):
+            return None, StateRequest((self.D + 1,), torch.float32)
+
+        def forward(self, ctx, h, residual):
+            state = ctx.state()                                   # [n_slots, D + 1]
+            b = ctx.batch
+            row = 0
+            for slot, n in zip(b.slots, b.n_new):                  # each sequence's rows in order
+                x = h[row:row + n].float()
+                sums = state[slot, :self.D] + torch.cumsum(x, dim=0)
+                counts = state[slot, self.D] + torch.arange(1, n + 1, device=x.device, dtype=torch.float32)
+                residual[row:row + n] += (sums / counts[:, None]) @ self.w.T
+                state[slot, :self.D] = sums[-1]
+                state[slot, self.D] = counts[-1]
+                row += n
+
+    def build(cfg):
+        D = cfg.hidden_size
+        emb = TokenEmbedding("emb.weight", cfg.vocab_size, D)
+        block = PreNormBlock(RMSNorm("norm1.weight", D, 1e-5), RunningMean("mean.weight", D),
+                             RMSNorm("norm2.weight", D, 1e-5), SwiGLU("ffn.", D, cfg.intermediate_size))
+        return DecoderModel(cfg, emb, [block], RMSNorm("final.weight", D, 1e-5),
+                            LMHead("head.weight", cfg.vocab_size, D, emb, tied=True), order=[0, 0])
+
+    register_architecture("ToyRunningMeanLM", ToyConfig, build)
+    try:
+        cfg = ToyConfig(dict(architectures=["ToyRunningMeanLM"], hidden_size=40, vocab_size=77, intermediate_size=56,
+                             max_position_embeddings=256))
+        d = write_random_model(cfg, str(tmp_path / "toy"), seed=4, std=0.3)
+        model = load_model(d, dtype="float32")
+        assert model.cache_spec.kv_groups == [] and model.cache_spec.state_groups[0].n_entries == 2
+        # the plain form of the same model
+        w = tiny.read_weights_f64(d)
+
+        def plain(tokens):
+            x = w["emb.weight"][tokens]
+            for _ in range(2):
+                hh = P.rmsnorm(x, w["norm1.weight"], 1e-5)
+                mean = np.cumsum(hh, axis=0) / np.arange(1, len(tokens) + 1)[:, None]
+                x = x + mean @ w["mean.weight"].T
+                x = x + P.swiglu(P.rmsnorm(x, w["norm2.weight"], 1e-5), w["ffn.gate_proj.weight"],
+                                 w["ffn.up_proj.weight"], w["ffn.down_proj.weight"])
+            return P.rmsnorm(x, w["final.weight"], 1e-5) @ w["emb.weight"].T
+        rng = np.random.default_rng(7)
+        reqs = [tiny.random_tokens(rng, n, 77) for n in (19, 3, 40)]
+        truth = [plain(r) for r in reqs]
+        s = Session(model, max_tokens=512, n_slots=3)
+        slots = s.begin(3)                                        # whole, as one unequal batch
+        got = s.step(slots, reqs, [list(range(len(r))) for r in reqs]).double().cpu().numpy()
+        assert np.abs(got - np.concatenate(truth)).max() < 5e-5
+        s.release(slots)
+        slots = s.begin(3)                                        # reused slots: state starts from zero again
+        cut = [7, 1, 33]
+        s.step(slots, [r[:c] for r, c in zip(reqs, cut)])
+        pos = dict(zip(range(3), cut))
+        live = [0, 1, 2]
+        while live:
+            out = s.step([slots[i] for i in live], [[reqs[i][pos[i]]] for i in live]).double().cpu().numpy()
+            for k, i in enumerate(live):
+                assert np.abs(out[k] - truth[i][pos[i]]).max() < 5e-5
+                pos[i] += 1
+            live = [i for i in live if pos[i] < len(reqs[i])]
+    finally:
+        unregister_architecture("ToyRunningMeanLM")
