@@ -40,9 +40,14 @@ class CacheSpec:
     state_groups: list = field(default_factory=list)
 
 
-def window_ring_pages(window: int) -> int:
-    """Pages that hold any `window` consecutive positions."""
-    return pages_for(window - 1) + 1 if window > 1 else 1
+WINDOW_STEP_TOKENS = 256     # new tokens of one sequence that a windowed group takes in at once
+
+
+def window_ring_pages(window: int, step_tokens: int = WINDOW_STEP_TOKENS) -> int:
+    """Pages of a slot's ring in a group that keeps `window` keys: enough for the window of the
+    first query of a chunk of `step_tokens` new tokens together with the whole chunk, which is
+    written before its queries are answered."""
+    return pages_for(window - 1 + step_tokens) + 1
 
 
 class KVGroup:

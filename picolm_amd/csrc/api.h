@@ -21,7 +21,7 @@ int picolm_rope_kv_store(const float* qkv, void* q_out, void* k_pages, void* v_p
                          const float* cos_t, const float* sin_t, int style, const int32_t* tok_pos,
                          const int32_t* tok_seq, const int32_t* seq_slot, const int32_t* page_table,
                          int max_pages, int ring_pages, int T, int H, int G, int d,
-                         hipStream_t stream);
+                         const int32_t* rows /* null: rows 0..T-1 */, hipStream_t stream);
 int picolm_silu_mul(const void* gu, int in_dt, void* out, int out_dt, int64_t n_pairs,
                     hipStream_t stream);
 int picolm_add_into(float* y, const void* x, int x_dt, int64_t n, hipStream_t stream);

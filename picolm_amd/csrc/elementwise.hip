@@ -82,8 +82,9 @@ __global__ void rope_kv_store_kernel(const float* __restrict__ qkv, TC* __restri
                                      const int32_t* __restrict__ tok_seq,
                                      const int32_t* __restrict__ seq_slot,
                                      const int32_t* __restrict__ page_table, int max_pages,
-                                     int ring_pages, int H, int G, int d) {
-    const int t = blockIdx.x;
+                                     int ring_pages, int H, int G, int d,
+                                     const int32_t* __restrict__ rows) {
+    const int t = rows ? rows[blockIdx.x] : blockIdx.x;      // `rows`: the token rows this launch handles
     const int pos = tok_pos[t];
     const int half = d / 2;
     const float* row = qkv + (size_t)t * (H + 2 * G) * d;
@@ -137,7 +138,7 @@ extern "C" int picolm_rope_kv_store(const float* qkv, void* q_out, void* k_pages
                                     const int32_t* tok_pos, const int32_t* tok_seq,
                                     const int32_t* seq_slot, const int32_t* page_table,
                                     int max_pages, int ring_pages, int T, int H, int G, int d,
-                                    hipStream_t stream) {
+                                    const int32_t* rows, hipStream_t stream) {
     PICOLM_REQUIRE(T >= 0 && H > 0 && G > 0 && d > 0 && d % 2 == 0,
                    "rope_kv_store: bad sizes T=%d H=%d G=%d d=%d", T, H, G, d);
     PICOLM_REQUIRE((cos_t == nullptr) == (sin_t == nullptr), "rope_kv_store: need both tables or none");
@@ -150,11 +151,11 @@ extern "C" int picolm_rope_kv_store(const float* qkv, void* q_out, void* k_pages
     if (dt == PICOLM_F32)
         rope_kv_store_kernel<float><<<grid, block, 0, stream>>>(
             qkv, (float*)q_out, (float*)k_pages, (float*)v_pages, cos_t, sin_t, style, tok_pos, tok_seq,
-            seq_slot, page_table, max_pages, ring_pages, H, G, d);
+            seq_slot, page_table, max_pages, ring_pages, H, G, d, rows);
     else if (dt == PICOLM_BF16)
         rope_kv_store_kernel<bf16_t><<<grid, block, 0, stream>>>(
             qkv, (bf16_t*)q_out, (bf16_t*)k_pages, (bf16_t*)v_pages, cos_t, sin_t, style, tok_pos, tok_seq,
-            seq_slot, page_table, max_pages, ring_pages, H, G, d);
+            seq_slot, page_table, max_pages, ring_pages, H, G, d, rows);
     else
         PICOLM_REQUIRE(false, "rope_kv_store: unknown dtype %d", dt);
     PICOLM_LAUNCH_CHECK("rope_kv_store");

@@ -100,9 +100,44 @@ class StepBatch:
             self._tiles[rows_per_tile] = (flat[:len(seqs)], flat[len(seqs):], len(seqs))
         return self._tiles[rows_per_tile]
 
+    def chunks(self, chunk_tokens: int):
+        """The step cut along positions: chunk c holds, of every sequence, its new tokens
+        c*chunk_tokens .. (c+1)*chunk_tokens - 1.  Each chunk looks like a step of its own to
+        the attention kernels (`rows` lists its token rows)."""
+        n_chunks = (self.max_new + chunk_tokens - 1) // chunk_tokens
+        cu = self._host["cu_seqlens"]
+        for c in range(n_chunks):
+            lo = c * chunk_tokens
+            seqs = [i for i, n in enumerate(self.n_new) if n > lo]
+            yield _Chunk(self, seqs, lo, [min(chunk_tokens, self.n_new[i] - lo) for i in seqs],
+                         [int(cu[i]) + lo for i in seqs])
+
     def decode_splits(self, blocks_per_seq: int) -> int:
         """How many slices of pages each sequence's decode attention is cut into, so that the
         launch has about `target_blocks` workgroups."""
         pages = pages_for(self.max_len)
         want = max(1, self._target_blocks // max(1, self.n_seq * blocks_per_seq))
         return max(1, min(want, pages))
+
+
+class _Chunk:
+    """A slice of a step along positions, with the fields the attention kernels read."""
+
+    def __init__(self, parent: StepBatch, seqs, lo, n_new, first_rows):
+        self.n_seq = len(seqs)
+        self.n_new = n_new
+        self.max_new = max(n_new)
+        self.is_decode = False
+        rows = np.concatenate([np.arange(r, r + n, dtype=np.int32) for r, n in zip(first_rows, n_new)])
+        self.n_rows = len(rows)
+        self._device = parent._device
+        self._tiles = {}
+        StepBatch._upload(self, {
+            "seq_slot": np.asarray([parent.slots[i] for i in seqs], dtype=np.int32),
+            "seq_pos0": np.asarray([parent.pos0[i] + lo for i in seqs], dtype=np.int32),
+            "seq_nnew": np.asarray(n_new, dtype=np.int32),
+            "cu_seqlens": np.asarray(first_rows, dtype=np.int32),
+            "rows": rows,
+        })
+
+    prefill_tiles = StepBatch.prefill_tiles

@@ -125,7 +125,8 @@ def rmsnorm(x: torch.Tensor, weight: torch.Tensor, eps: float, out: torch.Tensor
 
 
 def rope_kv_store(qkv, q_out, k_pages, v_pages, cos, sin, style: int, tok_pos, tok_seq, seq_slot,
-                  page_table, ring_pages: int, H: int, G: int, d: int) -> None:
+                  page_table, ring_pages: int, H: int, G: int, d: int, rows=None, n_rows: int | None = None) -> None:
+    """Rotate q and k of every token row (or of `rows` only) and write k, v to the cache."""
     _dev("rope.qkv", qkv, torch.float32, 2)
     T = qkv.shape[0]
     if qkv.shape[1] != (H + 2 * G) * d:
@@ -146,10 +147,16 @@ def rope_kv_store(qkv, q_out, k_pages, v_pages, cos, sin, style: int, tok_pos, t
             raise KernelError(f"rope: tables {tuple(cos.shape)} do not have d/2 = {d // 2} columns")
     _i32("rope.tok_pos", tok_pos, T)
     _i32("rope.tok_seq", tok_seq, T)
+    n_launch = T
+    if rows is not None:
+        n_launch = rows.numel() if n_rows is None else n_rows
+        _i32("rope.rows", rows, n_launch)
+        if n_launch > T:
+            raise KernelError("rope: more rows listed than there are")
     _check(lib().picolm_rope_kv_store(
         _ptr(qkv), _ptr(q_out), _ptr(k_pages), _ptr(v_pages), dt_of(q_out), _ptr(cos), _ptr(sin), style,
-        _ptr(tok_pos), _ptr(tok_seq), _ptr(seq_slot), _ptr(page_table), max_pages, ring_pages, T, H, G, d,
-        _stream()))
+        _ptr(tok_pos), _ptr(tok_seq), _ptr(seq_slot), _ptr(page_table), max_pages, ring_pages, n_launch, H, G, d,
+        _ptr(rows), _stream()))
 
 
 def _check_pages(who, k_pages, v_pages, dtype, G, d):

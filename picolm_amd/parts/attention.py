@@ -12,7 +12,7 @@ from __future__ import annotations
 import math
 
 from .. import kernels
-from ..cache.slots import PAGE_TOKENS
+from ..cache.kv import WINDOW_STEP_TOKENS
 from .base import KVRequest, Mixer, Runtime, StepContext
 from .linear import Linear
 from .position import NoPosition, PositionEncoding
@@ -59,19 +59,25 @@ class Attention(Mixer):
         else:
             cos, sin, style = tables
         q = ctx.ws.get("attn.q", (T, H * d), ctx.dtype)
-        writes = ctx.binding.writes
-        kernels.rope_kv_store(qkv, q, k_pages if writes else None, v_pages if writes else None, cos, sin,
-                              style, b.tok_pos, b.tok_seq, b.seq_slot, table, ring, H, G, d)
         out = ctx.ws.get("attn.out", (T, H * d), ctx.dtype)
+        writes = ctx.binding.writes
+        kp, vp = (k_pages, v_pages) if writes else (None, None)
         if b.is_decode:
+            kernels.rope_kv_store(qkv, q, kp, vp, cos, sin, style, b.tok_pos, b.tok_seq, b.seq_slot, table, ring,
+                                  H, G, d)
             n_splits = b.decode_splits(G * ((H // G + 15) // 16))
             partial = ctx.ws.get("attn.partial", (b.n_seq * H * n_splits * (d + 2),), torch.float32) \
                 if n_splits > 1 else None
             kernels.attn_decode(q, k_pages, v_pages, out, partial, b.n_seq, n_splits, b.seq_slot, b.seq_pos0,
                                 b.cu_seqlens, table, ring, H, G, d, self.window, self.scale)
+        elif self.window > 0 and ring < table.shape[1] and b.max_new > WINDOW_STEP_TOKENS:
+            # a ring holds a window and one chunk: write and answer the step chunk by chunk
+            for c in b.chunks(WINDOW_STEP_TOKENS):
+                kernels.rope_kv_store(qkv, q, kp, vp, cos, sin, style, b.tok_pos, b.tok_seq, b.seq_slot, table, ring,
+                                      H, G, d, rows=c.rows, n_rows=c.n_rows)
+                kernels.attn_prefill(q, k_pages, v_pages, out, c, table, ring, H, G, d, self.window, self.scale)
         else:
-            if self.window > 0 and b.max_new > (ring - 1) * PAGE_TOKENS - self.window + 1 and ring < table.shape[1]:
-                raise kernels.KernelError(
-                    f"a step of {b.max_new} tokens overruns the ring of a window of {self.window} keys")
+            kernels.rope_kv_store(qkv, q, kp, vp, cos, sin, style, b.tok_pos, b.tok_seq, b.seq_slot, table, ring,
+                                  H, G, d)
             kernels.attn_prefill(q, k_pages, v_pages, out, b, table, ring, H, G, d, self.window, self.scale)
         self.o.forward(out, residual, kernels.EPI_ACCUMULATE)

@@ -40,8 +40,9 @@ def test_slot_table():
 
 
 def test_window_ring():
-    assert window_ring_pages(1) == 1 and window_ring_pages(64) == 2 and window_ring_pages(65) == 2
-    assert window_ring_pages(66) == 3
+    # a ring holds a window and one chunk of new tokens, wherever they start in a page
+    assert window_ring_pages(1, 64) == 2 and window_ring_pages(65, 64) == 3 and window_ring_pages(66, 64) == 4
+    assert window_ring_pages(100) == pages_for(99 + 256) + 1 == 7
     book = PagedGroupBook(10, 2, ring_pages=3)
     assert [j for j, _ in book.grow(0, 1000)] == [0, 1, 2]     # never more than the ring
     assert book.grow(0, 5000) == []
@@ -59,7 +60,7 @@ def test_cache_shapes_and_groups():
     c = make_cache()
     full, win = c.kv
     assert tuple(full.k.shape) == (2, 8, 2, 64, 16) and tuple(full.v.shape) == (2, 8, 2, 16, 64)
-    assert win.ring_pages == 3 and tuple(win.k.shape) == (1, 8, 1, 64, 32)     # min(8, 4 slots * 3)
+    assert win.ring_pages == 5 and tuple(win.k.shape) == (1, 8, 1, 64, 32)     # capped by a sequence's 5 pages
     assert full.k.data_ptr() != win.k.data_ptr()
     assert tuple(c.state[0].shape) == (3, 4, 4, 2)
     assert c.max_seq_len == 320 and c.max_pages == 5

@@ -93,7 +93,7 @@ def test_attention_part(dtype, H, G, d, style, window):
     w = {n: rounded(rng.standard_normal(s) * 0.2, torch.bfloat16) for n, s in zip(names, shapes)}
     part = Attention("a.", D, H, G, d, position=RotaryEmbedding(d, 1000.0, None, style), window=window)
     assert sorted(s.name for s in part.all_specs()) == sorted(names)
-    lens = [70, 9] if window == 0 else [40, 9]          # a windowed step must fit its ring
+    lens = [70, 9] if window == 0 else [300, 9]         # longer than one chunk of a windowed group's ring
     rt, ctx = harness(dtype, part.cache_requests(), [2, 0], [0, 0], lens)
     part.load_all(WeightFetcher(TensorDict({k: torch.from_numpy(v).to(torch.bfloat16) for k, v in w.items()}), DEV), rt)
     part.prepare(rt, 512)
