@@ -113,11 +113,16 @@ class StepBatch:
                          [int(cu[i]) + lo for i in seqs])
 
     def decode_splits(self, blocks_per_seq: int) -> int:
-        """How many slices of pages each sequence's decode attention is cut into, so that the
-        launch has about `target_blocks` workgroups."""
-        pages = pages_for(self.max_len)
-        want = max(1, self._target_blocks // max(1, self.n_seq * blocks_per_seq))
-        return max(1, min(want, pages))
+        """How many slices of pages each sequence's decode attention is cut into."""
+        return decode_splits(self.n_seq, self.max_len, blocks_per_seq, self._target_blocks)
+
+
+def decode_splits(n_seq: int, max_len: int, blocks_per_seq: int, target_blocks: int = 1024) -> int:
+    """A power of two, so that a launch has about `target_blocks` workgroups and no more
+    slices than the longest sequence has pages."""
+    want = max(1, target_blocks // max(1, n_seq * blocks_per_seq))
+    want = min(want, pages_for(max_len))
+    return 1 << (want.bit_length() - 1)
 
 
 class _Chunk:
@@ -141,3 +146,49 @@ class _Chunk:
         })
 
     prefill_tiles = StepBatch.prefill_tiles
+
+
+class DecodeBatch:
+    """A decode step (one new token per sequence) over buffers that stay in place, so that the
+    step's kernel launches can be recorded once as a HIP graph and replayed: only the contents
+    of the int32 block change from step to step."""
+
+    is_decode = True
+    max_new = 1
+
+    def __init__(self, n_seq: int, n_splits: int, device):
+        self.n_seq = self.T = self.n_want = n_seq
+        self.n_splits = n_splits
+        self.n_new = [1] * n_seq
+        self.want_counts = [1] * n_seq
+        n = n_seq
+        self._spans = {}
+        off = 0
+        for name, size in (("seq_slot", n), ("seq_pos0", n), ("seq_nnew", n), ("cu_seqlens", n + 1), ("tok_pos", n),
+                           ("tok_seq", n), ("tokens", n), ("want_rows", n)):
+            self._spans[name] = (off, size)
+            off += size
+        self._host = torch.zeros(off, dtype=torch.int32).pin_memory() if torch.cuda.is_available() \
+            else torch.zeros(off, dtype=torch.int32)
+        self._dev = torch.zeros(off, dtype=torch.int32, device=device)
+        h = self._host.numpy()
+        ar = np.arange(n + 1, dtype=np.int32)
+        self._np = {k: h[o:o + s] for k, (o, s) in self._spans.items()}
+        self._np["seq_nnew"][:] = 1
+        self._np["cu_seqlens"][:] = ar
+        self._np["tok_seq"][:] = ar[:n]
+        self._np["want_rows"][:] = ar[:n]
+        for k, (o, s) in self._spans.items():
+            setattr(self, k, self._dev[o:o + s])
+        self.slots, self.pos0 = [], []
+
+    def fill(self, slots, pos0, tokens) -> None:
+        self.slots, self.pos0 = list(slots), list(pos0)
+        self._np["seq_slot"][:] = slots
+        self._np["seq_pos0"][:] = pos0
+        self._np["tok_pos"][:] = pos0
+        self._np["tokens"][:] = tokens
+        self._dev.copy_(self._host, non_blocking=False)
+
+    def decode_splits(self, blocks_per_seq: int) -> int:
+        return self.n_splits

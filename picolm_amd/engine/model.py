@@ -90,6 +90,22 @@ class DecoderModel:
             [KVGroupSpec(n, k.n_kv_heads, k.head_dim, k.window) for k, n in zip(kv_keys, kv_counts)],
             [StateGroupSpec(n, tuple(k.shape), k.dtype) for k, n in zip(state_keys, state_counts)])
 
+    def graph_safe(self) -> bool:
+        """Whether a decode step's launches depend on device memory only, so that they can be
+        recorded once and replayed."""
+        def safe(p):
+            return getattr(p, "graph_safe", False) and all(safe(c) for c in p.children())
+        return all(safe(p) for p in self.parts())
+
+    def decode_blocks_per_seq(self) -> int:
+        """Workgroups per sequence of the widest decode attention launch (for split sizing)."""
+        out = 1
+        for b in self.blocks:
+            m = b.mixer
+            if hasattr(m, "G") and hasattr(m, "H"):
+                out = max(out, m.G * ((m.H // m.G + 15) // 16))
+        return out
+
     # -- weights ----------------------------------------------------------------------------
     def load(self, source, runtime: Runtime) -> "DecoderModel":
         """Check `source` against every declared tensor, then bind."""

@@ -10,19 +10,53 @@ import torch
 
 from ..cache import Cache, CacheFull
 from ..parts.base import Workspace
-from .batch import StepBatch, StepError
+from .batch import DecodeBatch, StepBatch, StepError, decode_splits
 from .model import DecoderModel
+
+
+class _DecodeGraph:
+    """The kernel launches of one decode step of `n_seq` sequences, recorded as a HIP graph."""
+
+    def __init__(self, session: "Session", n_seq: int, n_splits: int):
+        self.session = session
+        self.batch = DecodeBatch(n_seq, n_splits, session.model.runtime.device)
+        self.workspace = Workspace(session.model.runtime.device)      # its own: recorded addresses must stay
+        self.graph = None
+        self.logits = None
+        self.uses = 0
+
+    def run(self, slots, pos0, tokens) -> torch.Tensor:
+        s = self.session
+        self.batch.fill(slots, pos0, tokens)
+        self.uses += 1
+        if self.graph is not None:
+            self.graph.replay()
+            return self.logits
+        logits = s.model.step(s.cache, self.batch, self.workspace)
+        if self.uses >= 2:
+            # the sizes have been seen, so the workspace is allocated: record the same launches
+            # (recording runs nothing; this step's result came from the eager run above)
+            g = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(g):
+                self.logits = s.model.step(s.cache, self.batch, self.workspace)
+            self.graph = g
+        return logits
 
 
 class Session:
     def __init__(self, model: DecoderModel, max_tokens: int, max_seq_len: int | None = None,
-                 n_slots: int | None = None):
+                 n_slots: int | None = None, graphs: bool = True):
         if model.runtime is None:
             raise StepError("the model has no weights loaded")
         self.model = model
         self.cache: Cache = model.new_cache(max_tokens, max_seq_len, n_slots)
         self.workspace = Workspace(model.runtime.device)
         self.vocab_size = model.head.V
+        # decode steps replay recorded HIP graphs when every part's launches depend on device
+        # memory only (a part says so with `graph_safe`)
+        self.graphs = graphs and model.graph_safe()
+        self._decode_graphs: dict[tuple, _DecodeGraph] = {}
+        self._blocks_per_seq = model.decode_blocks_per_seq()
 
     # -- slots -------------------------------------------------------------------------------
     def begin(self, n: int = 1) -> list[int]:
@@ -59,10 +93,30 @@ class Session:
             want = [[len(t) - 1] for t in new_tokens]
         pos0 = [self.cache.length(s) for s in slots]
         n_new = [len(t) for t in new_tokens]
+        if self.graphs and slots and max(n_new) == 1 and min(n_new) == 1 and all(list(w) == [0] for w in want):
+            return self._decode_step(slots, pos0, [int(t[0]) for t in new_tokens])
         batch = StepBatch(slots, pos0, new_tokens, want, self.vocab_size, self.model.runtime.device)
         self.cache.reserve_many(slots, [p + n for p, n in zip(pos0, n_new)])
         self.cache.flush()
         logits = self.model.step(self.cache, batch, self.workspace)
         for s, p, n in zip(slots, pos0, n_new):
             self.cache.set_length(s, p + n)
+        return logits
+
+    def _decode_step(self, slots, pos0, tokens) -> torch.Tensor:
+        if len(set(slots)) != len(slots):
+            raise StepError("a slot appears twice in one step")
+        for t in tokens:
+            if not 0 <= t < self.vocab_size:
+                raise StepError(f"token id {t} is outside the vocabulary of {self.vocab_size}")
+        self.cache.reserve_many(slots, [p + 1 for p in pos0])
+        self.cache.flush()
+        n_splits = decode_splits(len(slots), max(pos0) + 1, self._blocks_per_seq)
+        key = (len(slots), n_splits)
+        g = self._decode_graphs.get(key)
+        if g is None:
+            g = self._decode_graphs[key] = _DecodeGraph(self, len(slots), n_splits)
+        logits = g.run(slots, pos0, tokens)
+        for s, p in zip(slots, pos0):
+            self.cache.set_length(s, p + 1)
         return logits

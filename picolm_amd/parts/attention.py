@@ -20,6 +20,8 @@ import torch
 
 
 class Attention(Mixer):
+    graph_safe = True      # launches depend on device memory only
+
     def __init__(self, prefix: str, hidden_size: int, n_heads: int, n_kv_heads: int, head_dim: int,
                  position: PositionEncoding | None = None, window: int = 0, scale: float | None = None,
                  names=("q_proj.weight", "k_proj.weight", "v_proj.weight", "o_proj.weight")):

@@ -8,6 +8,8 @@ from .base import Block, FeedForward, Mixer, Norm, StepContext
 
 
 class PreNormBlock(Block):
+    graph_safe = True      # launches depend on device memory only
+
     def __init__(self, mixer_norm: Norm, mixer: Mixer, ffn_norm: Norm | None, ffn: FeedForward | None):
         self.mixer_norm, self.mixer, self.ffn_norm, self.ffn = mixer_norm, mixer, ffn_norm, ffn
 

@@ -12,6 +12,8 @@ from .base import Part, Runtime, StepContext
 
 
 class TokenEmbedding(Part):
+    graph_safe = True      # launches depend on device memory only
+
     def __init__(self, name: str, vocab_size: int, hidden_size: int):
         self.name, self.V, self.D = name, vocab_size, hidden_size
         self.table = None
@@ -30,6 +32,8 @@ class TokenEmbedding(Part):
 
 
 class LMHead(Part):
+    graph_safe = True      # launches depend on device memory only
+
     def __init__(self, name: str, vocab_size: int, hidden_size: int, embedding: TokenEmbedding, tied: bool):
         self.name, self.V, self.D, self.embedding, self.tied = name, vocab_size, hidden_size, embedding, tied
         self.weight = None

@@ -9,6 +9,8 @@ from .linear import Linear
 
 
 class SwiGLU(FeedForward):
+    graph_safe = True      # launches depend on device memory only
+
     def __init__(self, prefix: str, hidden_size: int, intermediate_size: int,
                  names=("gate_proj.weight", "up_proj.weight", "down_proj.weight")):
         self.D, self.F = hidden_size, intermediate_size

@@ -20,6 +20,8 @@ class Linear(Part):
     `interleave=True` stacks exactly two matrices row by row (row 2j of the first, row
     2j+1 of the second): the layout the gated epilogue reads.
     """
+    graph_safe = True      # launches depend on device memory only
+
 
     def __init__(self, names, out_sizes, in_size: int, interleave: bool = False):
         self.names = list(names)

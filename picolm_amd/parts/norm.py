@@ -9,6 +9,8 @@ from .base import Norm, Runtime, StepContext
 
 
 class RMSNorm(Norm):
+    graph_safe = True      # launches depend on device memory only
+
     def __init__(self, name: str, size: int, eps: float, weight_offset: float = 0.0):
         self.name = name
         self.size = size

@@ -29,6 +29,8 @@ def rotary_inv_freq(head_dim: int, theta: float, scaling=None) -> torch.Tensor:
 
 
 class RotaryEmbedding(PositionEncoding):
+    graph_safe = True      # launches depend on device memory only
+
     def __init__(self, head_dim: int, theta: float, scaling=None, style: str = "pairwise"):
         if head_dim % 2:
             raise ValueError(f"rotary head size {head_dim} is odd")
@@ -56,3 +58,5 @@ class RotaryEmbedding(PositionEncoding):
 
 class NoPosition(PositionEncoding):
     """Keys and queries are used as projected."""
+    graph_safe = True      # launches depend on device memory only
+

@@ -288,3 +288,34 @@ def test_missing_tensor_is_reported_when_loading(folders, tmp_path):
         load_model(d)
     assert e.value.missing == ["model.layers.1.mlp.gate_proj.weight"]
     assert e.value.wrong_shape == [("model.layers.0.self_attn.v_proj.weight", (32, 64), (16, 64))]
+
+
+def test_recorded_decode_steps_equal_eager_ones(folders):
+    """Decode steps replay a recorded HIP graph from their third use on; every replay must give
+    what the same step gives when its kernels are launched one by one, with the program's own
+    other work (prefills of other requests, releases) between the replays."""
+    from picolm_amd.engine import Session, load_model
+    d = folders["C"]
+    model = load_model(d, dtype="bfloat16")
+    rng = np.random.default_rng(21)
+    V = tiny.TINY_C["vocab_size"]
+    prompts = [tiny.random_tokens(rng, n, V) for n in (70, 5, 33)]
+    cont = [tiny.random_tokens(rng, 40, V) for _ in prompts]
+    outs = {}
+    for graphs in (True, False):
+        s = Session(model, max_tokens=1024, graphs=graphs)
+        slots = s.begin(3)
+        s.step(slots, prompts)
+        rows = []
+        for j in range(40):
+            rows.append(s.step(slots, [[c[j]] for c in cont]).clone())
+            if j % 7 == 3:                        # unrelated work between replays
+                [x] = s.begin(1)
+                s.step([x], [tiny.random_tokens(rng, 90, V)])
+                s.release([x])
+        outs[graphs] = torch.stack(rows)
+        if graphs:
+            assert any(g.graph is not None for g in s._decode_graphs.values())
+        else:
+            assert not s._decode_graphs
+    assert torch.equal(outs[True], outs[False])
