@@ -6,6 +6,8 @@ runs tokens it was not given: the prompt once, then one token each.
 """
 from __future__ import annotations
 
+import gc
+
 import torch
 
 from ..cache import Cache, CacheFull
@@ -18,15 +20,13 @@ class _DecodeGraph:
     """The kernel launches of one decode step of `n_seq` sequences, recorded as a HIP graph."""
 
     def __init__(self, session: "Session", n_seq: int, n_splits: int):
-        self.session = session
         self.batch = DecodeBatch(n_seq, n_splits, session.model.runtime.device)
         self.workspace = Workspace(session.model.runtime.device)      # its own: recorded addresses must stay
         self.graph = None
         self.logits = None
         self.uses = 0
 
-    def run(self, slots, pos0, tokens) -> torch.Tensor:
-        s = self.session
+    def run(self, s: "Session", slots, pos0, tokens) -> torch.Tensor:
         self.batch.fill(slots, pos0, tokens)
         self.uses += 1
         if self.graph is not None:
@@ -36,9 +36,17 @@ class _DecodeGraph:
         if self.uses >= 2:
             # the sizes have been seen, so the workspace is allocated: record the same launches
             # (recording runs nothing; this step's result came from the eager run above)
+            # Python's collector must not run while the stream records: freeing a GPU object
+            # in the middle of a recording aborts the process
             g = torch.cuda.CUDAGraph()
-            with torch.cuda.graph(g):
-                self.logits = s.model.step(s.cache, self.batch, self.workspace)
+            was_enabled = gc.isenabled()
+            gc.disable()
+            try:
+                with torch.cuda.graph(g):
+                    self.logits = s.model.step(s.cache, self.batch, self.workspace)
+            finally:
+                if was_enabled:
+                    gc.enable()
             self.graph = g
         return logits
 
@@ -116,7 +124,7 @@ class Session:
         g = self._decode_graphs.get(key)
         if g is None:
             g = self._decode_graphs[key] = _DecodeGraph(self, len(slots), n_splits)
-        logits = g.run(slots, pos0, tokens)
+        logits = g.run(self, slots, pos0, tokens)
         for s, p in zip(slots, pos0):
             self.cache.set_length(s, p + 1)
         return logits
