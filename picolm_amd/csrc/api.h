@@ -13,6 +13,9 @@ const char* picolm_last_error(void);
 int picolm_abi_version(void);
 int picolm_device_check(void);     // 0 if the current device is a gfx950
 
+// reads `bytes` from `src` once; for bandwidth measurements
+int picolm_read_probe(const void* src, size_t bytes, void* sink, int blocks, int unroll4, hipStream_t stream);
+
 int picolm_embed(const void* table, int table_dt, const int32_t* tokens, float* x, int T, int D,
                  int V, hipStream_t stream);
 int picolm_rmsnorm(const float* x, const float* w, void* out, int out_dt, const int32_t* rows,

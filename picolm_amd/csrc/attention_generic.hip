@@ -188,21 +188,47 @@ __global__ __launch_bounds__(AT_THREADS) void attn_tile_kernel(AttnArgs a) {
 }
 
 // out = sum_i exp(m_i - M) acc_i / sum_i exp(m_i - M) l_i over the splits of one (seq, head).
+// One wave per (seq, head): lanes take splits for the statistics, then columns for the sum.
+#define MERGE_WAVES 4
 template <typename T>
-__global__ void attn_merge_kernel(const float* __restrict__ partial, T* __restrict__ out,
-                                  const int32_t* __restrict__ cu_seqlens, int H, int d, int n_splits) {
-    const int seq = blockIdx.x / H, head = blockIdx.x % H;
-    const float* p = partial + ((size_t)seq * H + head) * n_splits * (d + 2);
-    float M = NEG_BIG;
-    for (int i = 0; i < n_splits; ++i) M = fmaxf(M, p[(size_t)i * (d + 2)]);
-    float L = 0.f;
-    for (int i = 0; i < n_splits; ++i) L += expf(p[(size_t)i * (d + 2)] - M) * p[(size_t)i * (d + 2) + 1];
+__global__ __launch_bounds__(MERGE_WAVES * WAVE) void attn_merge_kernel(const float* __restrict__ partial,
+                                                                        T* __restrict__ out,
+                                                                        const int32_t* __restrict__ cu_seqlens,
+                                                                        int n_units, int H, int d, int n_splits) {
+    const int unit = blockIdx.x * MERGE_WAVES + threadIdx.x / WAVE;
+    const int lane = threadIdx.x % WAVE;
+    if (unit >= n_units) return;
+    const int seq = unit / H, head = unit % H;
+    const int stride = d + 2;
+    const float* p = partial + (size_t)unit * n_splits * stride;
+    // the first splits' columns are asked for together with the statistics, so that the sum
+    // does not wait for a second trip to memory
+    constexpr int EARLY = 8;
+    float early[EARLY][4];
+#pragma unroll
+    for (int i = 0; i < EARLY; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int c = lane + j * WAVE;
+            early[i][j] = (i < n_splits && c < d) ? p[(size_t)i * stride + 2 + c] : 0.f;
+        }
+    float m = NEG_BIG;
+    for (int i = lane; i < n_splits; i += WAVE) m = fmaxf(m, p[(size_t)i * stride]);
+    const float M = wave_max(m);
+    float l = 0.f;
+    for (int i = lane; i < n_splits; i += WAVE) l += expf(p[(size_t)i * stride] - M) * p[(size_t)i * stride + 1];
+    const float L = wave_sum(l);
     const float inv = L > 0.f ? 1.0f / L : 0.f;
     T* o = out + (size_t)cu_seqlens[seq] * H * d + (size_t)head * d;
-    for (int c = threadIdx.x; c < d; c += blockDim.x) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const int c = lane + j * WAVE;
+        if (c >= d) break;
         float acc = 0.f;
-        for (int i = 0; i < n_splits; ++i)
-            acc += expf(p[(size_t)i * (d + 2)] - M) * p[(size_t)i * (d + 2) + 2 + c];
+#pragma unroll
+        for (int i = 0; i < EARLY; ++i)
+            if (i < n_splits) acc += expf(p[(size_t)i * stride] - M) * early[i][j];
+        for (int i = EARLY; i < n_splits; ++i) acc += expf(p[(size_t)i * stride] - M) * p[(size_t)i * stride + 2 + c];
         o[c] = from_f32<T>(acc * inv);
     }
 }
@@ -240,11 +266,12 @@ extern "C" int picolm_attn_merge(const float* partial, void* out, int dt, int n_
                                  int H, int d, int n_splits, hipStream_t stream) {
     PICOLM_REQUIRE(n_seq >= 0 && H > 0 && d > 0 && n_splits >= 1, "attn_merge: bad sizes");
     if (n_seq == 0) return 0;
-    dim3 mgrid(n_seq * H), mblock(d <= 64 ? 64 : (d <= 128 ? 128 : 256));
+    const int n_units = n_seq * H;
+    dim3 mgrid(ceil_div(n_units, MERGE_WAVES)), mblock(MERGE_WAVES * WAVE);
     if (dt == PICOLM_F32)
-        attn_merge_kernel<float><<<mgrid, mblock, 0, stream>>>(partial, (float*)out, cu_seqlens, H, d, n_splits);
+        attn_merge_kernel<float><<<mgrid, mblock, 0, stream>>>(partial, (float*)out, cu_seqlens, n_units, H, d, n_splits);
     else if (dt == PICOLM_BF16)
-        attn_merge_kernel<bf16_t><<<mgrid, mblock, 0, stream>>>(partial, (bf16_t*)out, cu_seqlens, H, d, n_splits);
+        attn_merge_kernel<bf16_t><<<mgrid, mblock, 0, stream>>>(partial, (bf16_t*)out, cu_seqlens, n_units, H, d, n_splits);
     else
         PICOLM_REQUIRE(false, "attn_merge: unknown dtype %d", dt);
     PICOLM_LAUNCH_CHECK("attn_merge");

@@ -93,6 +93,49 @@ __device__ __forceinline__ void attend_page(const bf16x8 (&Qf)[D / 16], f32x16 (
     }
 }
 
+// The same for one tile of 32 keys whose operands are already in registers (decode).
+template <int D>
+__device__ __forceinline__ void attend_tile(const bf16x8 (&Qf)[D / 16], const bf16x8 (&Kf)[D / 16],
+                                            const bf16x8 (&Vf)[D / 32][2], f32x16 (&O)[D / 32], float& m_run,
+                                            float& l_run, int key0, int qpos, bool q_ok, int window, float scale2,
+                                            int h) {
+    f32x16 S;
+#pragma unroll
+    for (int e = 0; e < 16; ++e) S[e] = 0.f;
+#pragma unroll
+    for (int s = 0; s < D / 16; ++s) S = __builtin_amdgcn_mfma_f32_32x32x16_bf16(Kf[s], Qf[s], S, 0, 0, 0);
+    float mx = NEG_BIG;
+#pragma unroll
+    for (int e = 0; e < 16; ++e) {
+        const int key = key0 + 16 * h + e;
+        const bool vis = q_ok && key <= qpos && (window <= 0 || qpos - key < window);
+        S[e] = vis ? S[e] * scale2 : NEG_BIG;
+        mx = fmaxf(mx, S[e]);
+    }
+    mx = fmaxf(mx, __shfl_xor(mx, 32, WAVE));
+    const float m_new = fmaxf(m_run, mx);
+    const float alpha = exp2f(m_run - m_new);
+    float sum = 0.f;
+    bf16x8 Pf[2];
+#pragma unroll
+    for (int e = 0; e < 16; ++e) {
+        const float p = S[e] > 0.5f * NEG_BIG ? exp2f(S[e] - m_new) : 0.f;
+        sum += p;
+        Pf[e / 8][e % 8] = to_bf16(p);
+    }
+    sum += __shfl_xor(sum, 32, WAVE);
+    l_run = l_run * alpha + sum;
+    m_run = m_new;
+#pragma unroll
+    for (int dt = 0; dt < D / 32; ++dt) {
+#pragma unroll
+        for (int e = 0; e < 16; ++e) O[dt][e] *= alpha;
+#pragma unroll
+        for (int ks = 0; ks < 2; ++ks)
+            O[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(Vf[dt][ks], Pf[ks], O[dt], 0, 0, 0);
+    }
+}
+
 // =============================================================================================
 template <int D>
 __global__ __launch_bounds__(256) void attn_prefill_mfma_kernel(AttnArgs a, int HB, int tile_tokens) {
@@ -192,7 +235,7 @@ __global__ __launch_bounds__(256) void attn_prefill_mfma_kernel(AttnArgs a, int 
 
 // =============================================================================================
 template <int D>
-__global__ __launch_bounds__(256) void attn_decode_mfma_kernel(AttnArgs a) {
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void attn_decode_mfma_kernel(AttnArgs a) {
     extern __shared__ float mrg[];       // [4 waves][Rc][D + 2]
     const int tid = threadIdx.x, wave = tid / WAVE, lane = tid % WAVE;
     const int l32 = lane % 32, h = lane / 32;
@@ -239,19 +282,31 @@ __global__ __launch_bounds__(256) void attn_decode_mfma_kernel(AttnArgs a) {
         const bf16_t* vp = (const bf16_t*)a.v_pages + base + (size_t)l32 * PAGE_TOKENS + 16 * h;
         const int key0 = page * PAGE_TOKENS;
         const int n_keys = qpos - key0 + 1;          // >= 1; keys past it are not this sequence's
-        attend_page<D>(
-            Qf, O, m_run, l_run, key0, qpos, q_ok, a.window, scale2, h,
-            [&](int t, int s) { return ldg8(kp + (size_t)(32 * t + key_of_row(l32)) * D + 8 * s); },
-            [&](int dt, int t, int ks) {
-                bf16x8 v = ldg8(vp + (size_t)(32 * dt) * PAGE_TOKENS + 32 * t + 8 * ks);
-                if (n_keys < PAGE_TOKENS) {
-                    const int k = 32 * t + 16 * h + 8 * ks;
+        // a page is two tiles of 32 keys; all operands of a tile are requested before the first
+        // MFMA waits for one
 #pragma unroll
-                    for (int e = 0; e < 8; ++e)
-                        if (k + e >= n_keys) v[e] = (__bf16)0.0f;
-                }
-                return v;
-            });
+        for (int t = 0; t < 2; ++t) {
+            if (key0 + 32 * t > qpos) break;                 // nothing of this tile is visible
+            bf16x8 Kf[D / 16], Vf[D / 32][2];
+#pragma unroll
+            for (int s = 0; s < D / 16; ++s) Kf[s] = ldg8(kp + (size_t)(32 * t + key_of_row(l32)) * D + 8 * s);
+#pragma unroll
+            for (int dt = 0; dt < D / 32; ++dt)
+#pragma unroll
+                for (int ks = 0; ks < 2; ++ks) Vf[dt][ks] = ldg8(vp + (size_t)(32 * dt) * PAGE_TOKENS + 32 * t + 8 * ks);
+            if (n_keys < 32 * (t + 1)) {                     // keys past the end may hold anything
+#pragma unroll
+                for (int dt = 0; dt < D / 32; ++dt)
+#pragma unroll
+                    for (int ks = 0; ks < 2; ++ks) {
+                        const int k = 32 * t + 16 * h + 8 * ks;
+#pragma unroll
+                        for (int e = 0; e < 8; ++e)
+                            if (k + e >= n_keys) Vf[dt][ks][e] = (__bf16)0.0f;
+                    }
+            }
+            attend_tile<D>(Qf, Kf, Vf, O, m_run, l_run, key0 + 32 * t, qpos, q_ok, a.window, scale2, h);
+        }
     }
     // merge the 4 waves
     float* mine = mrg + (size_t)wave * Rc * (D + 2);

@@ -34,16 +34,51 @@ extern "C" int picolm_embed(const void* table, int table_dt, const int32_t* toke
 // ---- RMSNorm ---------------------------------------------------------------------------
 // picolm/tensor.c:2942-3064: ss = sum x^2; r = 1/sqrtf(ss/size + eps); out = (x*r)*w.
 // `rows` (optional) selects which rows of x are normed; output row i is dense.
+#define NORM_THREADS 256
+#define NORM_REGS 16        // a row of up to NORM_THREADS * 4 * NORM_REGS values stays in registers
 template <typename TO>
-__global__ void rmsnorm_kernel(const float* __restrict__ x, const float* __restrict__ w,
-                               TO* __restrict__ out, const int32_t* __restrict__ rows, int D,
-                               float eps) {
+__global__ __launch_bounds__(NORM_THREADS) void rmsnorm_kernel(const float* __restrict__ x,
+                                                               const float* __restrict__ w,
+                                                               TO* __restrict__ out,
+                                                               const int32_t* __restrict__ rows, int D,
+                                                               float eps) {
     __shared__ float scratch[16];
     const int i = blockIdx.x;
     const int r = rows ? rows[i] : i;
     const float* xr = x + (size_t)r * D;
     TO* o = out + (size_t)i * D;
     float ss = 0.f;
+    if (D % 4 == 0 && D <= NORM_THREADS * 4 * NORM_REGS) {
+        // the row is read once, as float4, and kept
+        float4 v[NORM_REGS], ww[NORM_REGS];
+        const int nv = D / 4;
+#pragma unroll
+        for (int j = 0; j < NORM_REGS; ++j) {
+            const int idx = threadIdx.x + j * NORM_THREADS;
+            if (idx < nv) {
+                v[j] = ((const float4*)xr)[idx];
+                ww[j] = ((const float4*)w)[idx];         // asked for now: one trip to memory, not two
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < NORM_REGS; ++j) {
+            const int idx = threadIdx.x + j * NORM_THREADS;
+            if (idx < nv) ss += v[j].x * v[j].x + v[j].y * v[j].y + v[j].z * v[j].z + v[j].w * v[j].w;
+        }
+        ss = block_sum(ss, scratch);
+        const float scale = 1.0f / sqrtf(ss / (float)D + eps);
+#pragma unroll
+        for (int j = 0; j < NORM_REGS; ++j) {
+            const int idx = threadIdx.x + j * NORM_THREADS;
+            if (idx < nv) {
+                o[4 * idx + 0] = from_f32<TO>((v[j].x * scale) * ww[j].x);
+                o[4 * idx + 1] = from_f32<TO>((v[j].y * scale) * ww[j].y);
+                o[4 * idx + 2] = from_f32<TO>((v[j].z * scale) * ww[j].z);
+                o[4 * idx + 3] = from_f32<TO>((v[j].w * scale) * ww[j].w);
+            }
+        }
+        return;
+    }
     for (int j = threadIdx.x; j < D; j += blockDim.x) {
         float v = xr[j];
         ss += v * v;
@@ -58,7 +93,7 @@ extern "C" int picolm_rmsnorm(const float* x, const float* w, void* out, int out
                               hipStream_t stream) {
     PICOLM_REQUIRE(n_rows >= 0 && D > 0, "rmsnorm: bad sizes rows=%d D=%d", n_rows, D);
     if (n_rows == 0) return 0;
-    dim3 grid(n_rows), block(D >= 2048 ? 512 : 256);
+    dim3 grid(n_rows), block(NORM_THREADS);
     if (out_dt == PICOLM_F32)
         rmsnorm_kernel<float><<<grid, block, 0, stream>>>(x, w, (float*)out, rows, D, eps);
     else if (out_dt == PICOLM_BF16)
@@ -74,6 +109,7 @@ extern "C" int picolm_rmsnorm(const float* x, const float* w, void* out, int out
 // cached and leaves v alone (picolm/model_core.c:1908, :2915; picolm/tensor.c:3216-3304).
 // style 0: pairs (2i, 2i+1); style 1: pairs (i, i + d/2).  cos/sin == null: no rotation.
 // A token's cache row is page_table[slot][(pos / PAGE) % ring_pages], offset pos % PAGE.
+#define ROPE_HEADS 4
 template <typename TC>
 __global__ void rope_kv_store_kernel(const float* __restrict__ qkv, TC* __restrict__ q_out,
                                      TC* __restrict__ k_pages, TC* __restrict__ v_pages,
@@ -101,34 +137,35 @@ __global__ void rope_kv_store_kernel(const float* __restrict__ qkv, TC* __restri
         page_base = ((size_t)page * G) * PAGE_TOKENS * d;
         cache_row = page_base + (size_t)in_page * d;
     }
-    // rotations: heads 0..H-1 are q, H..H+G-1 are k
-    const int n_rot = (H + G) * half;
-    for (int idx = threadIdx.x; idx < n_rot; idx += blockDim.x) {
-        const int head = idx / half, i = idx % half;
-        const int i0 = style == 0 ? 2 * i : i;
-        const int i1 = style == 0 ? 2 * i + 1 : i + half;
-        const float x0 = row[head * d + i0], x1 = row[head * d + i1];
-        float y0 = x0, y1 = x1;
-        if (c) {
-            const float cc = c[i], ss = s[i];
-            y0 = x0 * cc - x1 * ss;
-            y1 = x0 * ss + x1 * cc;
-        }
-        if (head < H) {
-            TC* q = q_out + (size_t)t * H * d + head * d;
-            q[i0] = from_f32<TC>(y0);
-            q[i1] = from_f32<TC>(y1);
-        } else if (k_pages) {
-            TC* k = k_pages + cache_row + (size_t)(head - H) * PAGE_TOKENS * d;
-            k[i0] = from_f32<TC>(y0);
-            k[i1] = from_f32<TC>(y1);
-        }
-    }
-    if (v_pages) {
-        const float* vrow = row + (H + G) * d;
-        for (int idx = threadIdx.x; idx < G * d; idx += blockDim.x) {
-            const int g = idx / d, i = idx % d;
-            v_pages[page_base + ((size_t)g * d + i) * PAGE_TOKENS + in_page] = from_f32<TC>(vrow[idx]);
+    // blockIdx.y takes ROPE_HEADS heads of the row: heads 0..H-1 are q, H..H+G-1 are k, then v
+    const int head_lo = blockIdx.y * ROPE_HEADS, head_hi = min(head_lo + ROPE_HEADS, H + 2 * G);
+    for (int head = head_lo; head < head_hi; ++head) {
+        if (head < H + G) {
+            for (int i = threadIdx.x; i < half; i += blockDim.x) {
+                const int i0 = style == 0 ? 2 * i : i;
+                const int i1 = style == 0 ? 2 * i + 1 : i + half;
+                const float x0 = row[head * d + i0], x1 = row[head * d + i1];
+                float y0 = x0, y1 = x1;
+                if (c) {
+                    const float cc = c[i], ss = s[i];
+                    y0 = x0 * cc - x1 * ss;
+                    y1 = x0 * ss + x1 * cc;
+                }
+                if (head < H) {
+                    TC* q = q_out + (size_t)t * H * d + head * d;
+                    q[i0] = from_f32<TC>(y0);
+                    q[i1] = from_f32<TC>(y1);
+                } else if (k_pages) {
+                    TC* k = k_pages + cache_row + (size_t)(head - H) * PAGE_TOKENS * d;
+                    k[i0] = from_f32<TC>(y0);
+                    k[i1] = from_f32<TC>(y1);
+                }
+            }
+        } else if (v_pages) {
+            const int g = head - H - G;
+            const float* vrow = row + (size_t)head * d;
+            for (int i = threadIdx.x; i < d; i += blockDim.x)
+                v_pages[page_base + ((size_t)g * d + i) * PAGE_TOKENS + in_page] = from_f32<TC>(vrow[i]);
         }
     }
 }
@@ -147,7 +184,7 @@ extern "C" int picolm_rope_kv_store(const float* qkv, void* q_out, void* k_pages
                    "rope_kv_store: bad page table geometry max_pages=%d ring_pages=%d", max_pages, ring_pages);
     PICOLM_REQUIRE(style == 0 || style == 1, "rope_kv_store: unknown pairing %d", style);
     if (T == 0) return 0;
-    dim3 grid(T), block(256);
+    dim3 grid(T, ceil_div(H + 2 * G, ROPE_HEADS)), block(d / 2 >= 64 ? 64 : 32);
     if (dt == PICOLM_F32)
         rope_kv_store_kernel<float><<<grid, block, 0, stream>>>(
             qkv, (float*)q_out, (float*)k_pages, (float*)v_pages, cos_t, sin_t, style, tok_pos, tok_seq,

@@ -32,9 +32,9 @@ __device__ __forceinline__ float silu_mul(float g, float u) { return g / (1.0f +
 // =============================================================================================
 // skinny
 // =============================================================================================
-#define SK_KSTEP 128      // K elements one wave consumes per step: 4 quarters x 32
+#define SK_KSTEP 128      // K elements one wave consumes per step: 4 MFMAs of 32
 
-template <int MT, int NT, int WAVES, int EPI, typename TC>
+template <int MT, int NT, int WAVES, int EPI, typename TC, bool NOA = false>
 __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const bf16_t* __restrict__ A,
                                                                  const bf16_t* __restrict__ W,
                                                                  TC* __restrict__ C, int M, int N, int K,
@@ -61,27 +61,65 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const bf16_t* _
 #pragma unroll
         for (int u = 0; u < MT; ++u) acc[t][u] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-    const int n_steps = (K + SK_KSTEP - 1) / SK_KSTEP;
-#pragma unroll 2
-    for (int s = wave; s < n_steps; s += WAVES) {
-        const int k0 = s * SK_KSTEP + q * 32;
-        bf16x8 wv[NT][4], av[MT][4];
+    // Two register buffers: the loads of a wave's next step are in flight while the MFMAs of
+    // the current one run.  Loads in the main loop carry no predicate (a predicate makes the
+    // compiler fence every load): rows m >= M read row 0 and their results are never stored;
+    // the K tail, if any, is a separate last step.
+    const int n_full = K / SK_KSTEP;
+    bf16x8 wv[2][NT][4], av[2][MT][4];
+    auto fetch = [&](int buf, int s) {
+        // load j of a step reads, of every row, the 64 contiguous bytes at 64*j: the four quarter
+        // lanes of a row take 16 bytes each
+        const int k0 = s * SK_KSTEP + q * 8;
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
-            const int k = k0 + 8 * j;
-            const bool kvalid = k < K;
 #pragma unroll
-            for (int t = 0; t < NT; ++t) wv[t][j] = kvalid ? load_chunk(wrow[t] + k) : zero_chunk();
+            for (int t = 0; t < NT; ++t) wv[buf][t][j] = load_chunk(wrow[t] + k0 + 32 * j);
 #pragma unroll
-            for (int u = 0; u < MT; ++u) av[u][j] = (kvalid && mvalid[u]) ? load_chunk(arow[u] + k) : zero_chunk();
+            for (int u = 0; u < MT; ++u)
+                if (!NOA) av[buf][u][j] = load_chunk(arow[u] + k0 + 32 * j);
         }
+    };
+    auto multiply = [&](int buf) {
 #pragma unroll
         for (int j = 0; j < 4; ++j)
 #pragma unroll
             for (int t = 0; t < NT; ++t)
 #pragma unroll
                 for (int u = 0; u < MT; ++u)
-                    acc[t][u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wv[t][j], av[u][j], acc[t][u], 0, 0, 0);
+                    acc[t][u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wv[buf][t][j], av[buf][u][j], acc[t][u], 0, 0, 0);
+    };
+    if (NOA) {
+#pragma unroll
+        for (int b = 0; b < 2; ++b)
+#pragma unroll
+            for (int u = 0; u < MT; ++u)
+#pragma unroll
+                for (int j = 0; j < 4; ++j) av[b][u][j] = zero_chunk();
+    }
+    int s = wave;
+    if (s < n_full) fetch(0, s);
+    while (s < n_full) {
+        if (s + WAVES < n_full) fetch(1, s + WAVES);
+        multiply(0);
+        s += WAVES;
+        if (s >= n_full) break;
+        if (s + WAVES < n_full) fetch(0, s + WAVES);
+        multiply(1);
+        s += WAVES;
+    }
+    if (K % SK_KSTEP != 0 && wave == n_full % WAVES) {
+        const int k0 = n_full * SK_KSTEP + q * 8;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int k = k0 + 32 * j;
+            const bool kvalid = k < K;
+#pragma unroll
+            for (int t = 0; t < NT; ++t) wv[0][t][j] = kvalid ? load_chunk(wrow[t] + k) : zero_chunk();
+#pragma unroll
+            for (int u = 0; u < MT; ++u) av[0][u][j] = kvalid ? load_chunk(arow[u] + k) : zero_chunk();
+        }
+        multiply(0);
     }
     // reduce over the waves
 #pragma unroll
@@ -178,7 +216,7 @@ extern "C" int picolm_gemm_skinny(const void* A, const void* W, void* C, int c_d
     if (check_mfma_operands("gemm_skinny", A, W, M, N, K, lda, ldw, ldc, epilogue, c_dt)) return -1;
     PICOLM_REQUIRE(M <= 64, "gemm_skinny: M=%d exceeds 64", M);
     if (M == 0) return 0;
-    if (variant == 0) variant = M <= 16 ? 1 : (M <= 32 ? 3 : 5);
+    if (variant == 0) variant = M <= 16 ? 1 : (M <= 32 ? 3 : (N >= 8192 ? 6 : 5));
     switch (variant) {
         case 1: return launch_skinny<1, 1, 8>(A, W, C, c_dt, M, N, K, lda, ldw, ldc, epilogue, stream);
         case 2: return launch_skinny<1, 2, 8>(A, W, C, c_dt, M, N, K, lda, ldw, ldc, epilogue, stream);
@@ -186,6 +224,16 @@ extern "C" int picolm_gemm_skinny(const void* A, const void* W, void* C, int c_d
         case 4: return launch_skinny<2, 2, 8>(A, W, C, c_dt, M, N, K, lda, ldw, ldc, epilogue, stream);
         case 5: return launch_skinny<4, 1, 8>(A, W, C, c_dt, M, N, K, lda, ldw, ldc, epilogue, stream);
         case 6: return launch_skinny<4, 2, 4>(A, W, C, c_dt, M, N, K, lda, ldw, ldc, epilogue, stream);
+        case 11: {
+            dim3 grid(ceil_div(N, 16)), block(512);
+            gemm_skinny_kernel<1, 1, 8, 0, float, true><<<grid, block, sizeof(float) * 8 * 4 * 64, stream>>>(
+                (const bf16_t*)A, (const bf16_t*)W, (float*)C, M, N, K, lda, ldw, ldc);
+            return 0;
+        }
+        case 7: return launch_skinny<1, 1, 4>(A, W, C, c_dt, M, N, K, lda, ldw, ldc, epilogue, stream);
+        case 8: return launch_skinny<1, 1, 16>(A, W, C, c_dt, M, N, K, lda, ldw, ldc, epilogue, stream);
+        case 9: return launch_skinny<1, 2, 4>(A, W, C, c_dt, M, N, K, lda, ldw, ldc, epilogue, stream);
+        case 10: return launch_skinny<1, 4, 4>(A, W, C, c_dt, M, N, K, lda, ldw, ldc, epilogue, stream);
     }
     PICOLM_REQUIRE(false, "gemm_skinny: unknown variant %d", variant);
 }

@@ -20,7 +20,7 @@ class StepError(ValueError):
 
 
 class StepBatch:
-    def __init__(self, slots, pos0, new_tokens, want, vocab_size: int, device, target_blocks: int = 1024):
+    def __init__(self, slots, pos0, new_tokens, want, vocab_size: int, device, target_blocks: int = 512):
         """slots[i]: cache slot of sequence i; pos0[i]: tokens it holds; new_tokens[i]: its
         next tokens; want[i]: indices into new_tokens[i] whose logits are asked for."""
         self.n_seq = len(slots)
@@ -117,12 +117,12 @@ class StepBatch:
         return decode_splits(self.n_seq, self.max_len, blocks_per_seq, self._target_blocks)
 
 
-def decode_splits(n_seq: int, max_len: int, blocks_per_seq: int, target_blocks: int = 1024) -> int:
-    """A power of two, so that a launch has about `target_blocks` workgroups and no more
-    slices than the longest sequence has pages."""
+def decode_splits(n_seq: int, max_len: int, blocks_per_seq: int, target_blocks: int = 512) -> int:
+    """A power of two: as many slices as give every wave of a 4-wave workgroup a page of its
+    own, within about `target_blocks` workgroups for the whole launch (two per CU)."""
     want = max(1, target_blocks // max(1, n_seq * blocks_per_seq))
-    want = min(want, pages_for(max_len))
-    return 1 << (want.bit_length() - 1)
+    want = min(want, (pages_for(max_len) + 3) // 4)
+    return 1 << (max(want, 1).bit_length() - 1)
 
 
 class _Chunk:

@@ -44,7 +44,7 @@ def dir_entry_points():
             "picolm_attn_prefill_tile_rows", "picolm_attn_prefill_generic",
             "picolm_attn_decode_generic", "picolm_argmax", "picolm_sample", "picolm_gemm_skinny", "picolm_gemm_tiled",
             "picolm_attn_mfma_takes", "picolm_attn_prefill_mfma_heads", "picolm_attn_prefill_mfma_tile_tokens",
-            "picolm_attn_prefill_mfma", "picolm_attn_decode_mfma", "picolm_attn_merge"]
+            "picolm_attn_prefill_mfma", "picolm_attn_decode_mfma", "picolm_attn_merge", "picolm_read_probe"]
 
 
 def _check(rc: int) -> None:
@@ -357,3 +357,11 @@ def sample(logits: torch.Tensor, out: torch.Tensor, temperature: float, top_k: i
             raise KernelError("sample: fewer generator states than rows")
     _check(lib().picolm_sample(_ptr(logits), c_int64(V), n, V, c_float(temperature), int(top_k), c_float(top_p),
                                c_float(min_p), _ptr(rng_states), _ptr(state_index), _ptr(out), _stream()))
+
+
+def read_probe(src: torch.Tensor, sink: torch.Tensor, blocks: int = 4096, unroll4: bool = True) -> None:
+    """Sweep `src` once with a plain read kernel (for bandwidth measurements)."""
+    _dev("read_probe.src", src)
+    _dev("read_probe.sink", sink, torch.int32)
+    nbytes = src.numel() * src.element_size()
+    _check(lib().picolm_read_probe(_ptr(src), ctypes.c_size_t(nbytes - nbytes % 16), _ptr(sink), blocks, int(unroll4), _stream()))
