@@ -16,6 +16,9 @@ int picolm_device_check(void);     // 0 if the current device is a gfx950
 // reads `bytes` from `src` once; for bandwidth measurements
 int picolm_read_probe(const void* src, size_t bytes, void* sink, int blocks, int unroll4, hipStream_t stream);
 
+// runs blocks*4 waves of `iters` x 8 MFMAs (32x32x16 bf16) on registers; for MFMA-rate measurements
+int picolm_mfma_probe(void* sink, int blocks, int iters, hipStream_t stream);
+
 int picolm_embed(const void* table, int table_dt, const int32_t* tokens, float* x, int T, int D,
                  int V, hipStream_t stream);
 int picolm_rmsnorm(const float* x, const float* w, void* out, int out_dt, const int32_t* rows,
@@ -37,7 +40,7 @@ int picolm_gemm_generic(const void* A, int a_dt, const void* W, int w_dt, void* 
 int picolm_gemm_skinny(const void* A, const void* W, void* C, int c_dt, int M, int N, int K, int64_t lda,
                        int64_t ldw, int64_t ldc, int epilogue, int variant, hipStream_t stream);
 int picolm_gemm_tiled(const void* A, const void* W, void* C, int c_dt, int M, int N, int K, int64_t lda,
-                      int64_t ldw, int64_t ldc, int epilogue, hipStream_t stream);
+                      int64_t ldw, int64_t ldc, int epilogue, int variant, hipStream_t stream);
 
 int picolm_attn_prefill_tile_rows(void);
 int picolm_attn_prefill_generic(const void* q, const void* k_pages, const void* v_pages, void* out,

@@ -1,15 +1,15 @@
 // bf16 x bf16 -> float products on the matrix cores of gfx950: C[M,N] = A[M,K] * W[N,K]^T.
 //
-// Both kernels feed the weight tile as the MFMA's first operand and the activation tile as
-// its second, so an accumulator lane holds four consecutive output columns n of one row m:
-// gate/up pairs of the row-interleaved gated layout meet in one lane, and stores along n
-// are vectors.
+// The skinny kernel feeds the weight tile as the MFMA's first operand and the activation tile
+// as its second, so an accumulator lane holds four consecutive output columns n of one row m
+// and gate/up pairs of the row-interleaved gated layout meet in one lane.
 //
 //   skinny (M <= 64, the decode step): HBM-bound.  A wave streams 16*NT weight rows straight
 //     from global memory into MFMA operand registers, 16 bytes a lane; the waves of a block
 //     split K between them and reduce through LDS.  Every weight byte is read once.
-//   tiled (M > 64, the prefill step): 128x128x64 block tiles staged through LDS with an XOR
-//     swizzle of 16-byte chunks, register prefetch of the next tile, 32x32x16 MFMAs.
+//   tiled (M > 64, the prefill step): block tiles of 128x128 to 256x256 staged through two LDS
+//     stages with an XOR swizzle of 16-byte chunks, loads two steps ahead, 32x32x16 MFMAs; here
+//     the activation tile is the first operand, so that stores are whole 128-byte runs.
 //
 // The order of the K summation inside an MFMA does not matter, so a lane's 8-element chunk
 // may come from any K offset as long as both operands use the same offset.
@@ -241,139 +241,248 @@ extern "C" int picolm_gemm_skinny(const void* A, const void* W, void* C, int c_d
 // =============================================================================================
 // tiled
 // =============================================================================================
-#define TG_BN 128
-#define TG_BM 128
+// A block of WN x WM waves computes a (32*TN*WN) x (32*TM*WM) tile of C; a wave owns TN x TM MFMA
+// tiles of 32 x 32.  Here the activation tile is the MFMA's first operand and the weight tile its
+// second, so that an accumulator lane holds one column n and the 32 lanes of a half wave write
+// 32 consecutive n of one row: stores are whole 128-byte runs.  K advances in steps of 64 through
+// two LDS stages and two sets of staging registers: the loads of step it+2 are in flight while
+// step it is multiplied and step it+1 is written to LDS; one barrier a step.  LDS rows are 64
+// bf16 (128 bytes, half of the 64 banks); 16-byte chunk c of row r sits at c ^ ((r / 2) % 8), so
+// that 16 consecutive rows of one chunk column touch every bank once.
 #define TG_BK 64
-#define TG_THREADS 256
-#define TG_CHUNKS (TG_BK / 8)        // 16-byte chunks per tile row
+#define TG_CHUNKS (TG_BK / 8)
 
-// LDS tile: [rows][TG_BK] bf16, chunk c of row r stored at chunk slot c ^ (r % 8)
-__device__ __forceinline__ int tile_off(int row, int chunk) { return row * TG_BK + ((chunk ^ (row & 7)) << 3); }
+__device__ __forceinline__ int tile_off(int row, int chunk) { return row * TG_BK + ((chunk ^ ((row >> 1) & 7)) << 3); }
 
-template <int EPI, typename TC>
-__global__ __launch_bounds__(TG_THREADS) void gemm_tiled_kernel(const bf16_t* __restrict__ A,
-                                                               const bf16_t* __restrict__ W,
-                                                               TC* __restrict__ C, int M, int N, int K,
-                                                               int64_t lda, int64_t ldw, int64_t ldc,
-                                                               int tiles_m, int tiles_n) {
-    __shared__ __attribute__((aligned(16))) bf16_t Ws[TG_BN * TG_BK];
-    __shared__ __attribute__((aligned(16))) bf16_t As[TG_BM * TG_BK];
-    // tile order: consecutive blocks walk down M inside a column band of N so that the
-    // weight band stays in cache while activations stream
-    const int tile = blockIdx.x;
-    const int band = 8;                                   // tiles of N per band
+template <int TN, int TM, int WN, int WM, int DEPTH, int EPI, typename TC>
+__global__ __launch_bounds__(64 * WN * WM) void gemm_tiled_kernel(const bf16_t* __restrict__ A,
+                                                                  const bf16_t* __restrict__ W,
+                                                                  TC* __restrict__ C, int M, int N, int K,
+                                                                  int64_t lda, int64_t ldw, int64_t ldc,
+                                                                  int tiles_m, int tiles_n) {
+    constexpr int THREADS = 64 * WN * WM;
+    constexpr int BN = 32 * TN * WN, BM = 32 * TM * WM;
+    constexpr int STAGE = (BN + BM) * TG_BK;
+    constexpr int ROWS_PER_PASS = THREADS / TG_CHUNKS;
+    constexpr int WP = BN / ROWS_PER_PASS, AP = BM / ROWS_PER_PASS;       // staging passes
+    static_assert(BN % ROWS_PER_PASS == 0 && BM % ROWS_PER_PASS == 0, "tile does not split over the threads");
+    extern __shared__ __attribute__((aligned(16))) bf16_t lds[];
+    // Workgroups are dealt to the 8 XCDs in turn and each XCD has an L2 of its own: workgroup b
+    // takes the (b / 8)-th tile of XCD (b % 8)'s contiguous share, so that neighbours in tile
+    // order meet in one L2.  Tile order walks down M inside a band of 8 tiles of N, so that a
+    // band of weights stays in cache while activations stream.
+    int tile;
+    {
+        const int nb = gridDim.x, per = nb / 8, rem = nb % 8;
+        const int xcd = blockIdx.x % 8, idx = blockIdx.x / 8;
+        tile = (xcd < rem ? xcd * (per + 1) : rem * (per + 1) + (xcd - rem) * per) + idx;
+    }
+    const int band = 8;
     const int per_band = band * tiles_m;
     const int b = tile / per_band, in_b = tile % per_band;
     const int band_w = min(band, tiles_n - b * band);
     const int tn = b * band + in_b % band_w, tm = in_b / band_w;
-    const int n0 = tn * TG_BN, m0 = tm * TG_BM;
+    const int n0 = tn * BN, m0 = tm * BM;
 
     const int tid = threadIdx.x, wave = tid / 64, lane = tid % 64;
-    const int wn = (wave % 2) * 64, wm = (wave / 2) * 64;     // the wave's 64x64 corner of the block tile
+    const int wn = (wave % WN) * (32 * TN), wm = (wave / WN) * (32 * TM);
     const int l32 = lane % 32, kq = lane / 32;
 
-    // global -> register staging: 4 chunks per operand per thread
-    const int ld_chunk = tid % TG_CHUNKS, ld_row = tid / TG_CHUNKS;      // rows ld_row + 32*i
-    const bf16_t* wsrc[4];
-    const bf16_t* asrc[4];
+    // global -> register staging: a thread carries chunk `ld_chunk` of rows ld_row + ROWS_PER_PASS*i
+    const int ld_chunk = tid % TG_CHUNKS, ld_row = tid / TG_CHUNKS;
+    const bf16_t* wsrc[WP];
+    const bf16_t* asrc[AP];
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        wsrc[i] = W + (int64_t)min(n0 + ld_row + 32 * i, N - 1) * ldw + ld_chunk * 8;
-        asrc[i] = A + (int64_t)min(m0 + ld_row + 32 * i, M - 1) * lda + ld_chunk * 8;
-    }
-    bf16x8 wreg[4], areg[4];
-    auto fetch = [&](int k0) {
+    for (int i = 0; i < WP; ++i) wsrc[i] = W + (int64_t)min(n0 + ld_row + ROWS_PER_PASS * i, N - 1) * ldw + ld_chunk * 8;
+#pragma unroll
+    for (int i = 0; i < AP; ++i) asrc[i] = A + (int64_t)min(m0 + ld_row + ROWS_PER_PASS * i, M - 1) * lda + ld_chunk * 8;
+    bf16x8 wreg[DEPTH][WP], areg[DEPTH][AP];
+    auto fetch = [&](bf16x8 (&wr)[WP], bf16x8 (&ar)[AP], int k0) {      // a whole step inside K
+#pragma unroll
+        for (int i = 0; i < WP; ++i) wr[i] = load_chunk(wsrc[i] + k0);
+#pragma unroll
+        for (int i = 0; i < AP; ++i) ar[i] = load_chunk(asrc[i] + k0);
+    };
+    auto fetch_any = [&](bf16x8 (&wr)[WP], bf16x8 (&ar)[AP], int k0) {  // chunks past K are zero
         const bool kvalid = k0 + ld_chunk * 8 < K;
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            wreg[i] = kvalid ? load_chunk(wsrc[i] + k0) : zero_chunk();
-            areg[i] = kvalid ? load_chunk(asrc[i] + k0) : zero_chunk();
-        }
-    };
-    auto stash = [&]() {
+        for (int i = 0; i < WP; ++i) wr[i] = kvalid ? load_chunk(wsrc[i] + k0) : zero_chunk();
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            *(bf16x8*)(Ws + tile_off(ld_row + 32 * i, ld_chunk)) = wreg[i];
-            *(bf16x8*)(As + tile_off(ld_row + 32 * i, ld_chunk)) = areg[i];
-        }
+        for (int i = 0; i < AP; ++i) ar[i] = kvalid ? load_chunk(asrc[i] + k0) : zero_chunk();
+    };
+    auto stash = [&](const bf16x8 (&wr)[WP], const bf16x8 (&ar)[AP], int stage) {
+        bf16_t* Ws = lds + stage * STAGE;
+        bf16_t* As = Ws + BN * TG_BK;
+#pragma unroll
+        for (int i = 0; i < WP; ++i) *(bf16x8*)(Ws + tile_off(ld_row + ROWS_PER_PASS * i, ld_chunk)) = wr[i];
+#pragma unroll
+        for (int i = 0; i < AP; ++i) *(bf16x8*)(As + tile_off(ld_row + ROWS_PER_PASS * i, ld_chunk)) = ar[i];
     };
 
-    f32x16 acc[2][2];
+    f32x16 acc[TN][TM];
 #pragma unroll
-    for (int i = 0; i < 2; ++i)
+    for (int i = 0; i < TN; ++i)
 #pragma unroll
-        for (int j = 0; j < 2; ++j)
+        for (int j = 0; j < TM; ++j)
 #pragma unroll
             for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
 
-    fetch(0);
-    for (int k0 = 0; k0 < K; k0 += TG_BK) {
-        __syncthreads();            // everyone is done reading the previous tile
-        stash();
-        __syncthreads();
-        if (k0 + TG_BK < K) fetch(k0 + TG_BK);
+    auto compute = [&](int stage) {
+        const bf16_t* Ws = lds + stage * STAGE;
+        const bf16_t* As = Ws + BN * TG_BK;
 #pragma unroll
         for (int ks = 0; ks < TG_BK / 16; ++ks) {
             const int chunk = ks * 2 + kq;
-            bf16x8 wf[2], af[2];
+            bf16x8 wf[TN], af[TM];
 #pragma unroll
-            for (int i = 0; i < 2; ++i) {
-                wf[i] = *(const bf16x8*)(Ws + tile_off(wn + 32 * i + l32, chunk));
-                af[i] = *(const bf16x8*)(As + tile_off(wm + 32 * i + l32, chunk));
+            for (int i = 0; i < TN; ++i) wf[i] = *(const bf16x8*)(Ws + tile_off(wn + 32 * i + l32, chunk));
+#pragma unroll
+            for (int j = 0; j < TM; ++j) af[j] = *(const bf16x8*)(As + tile_off(wm + 32 * j + l32, chunk));
+#pragma unroll
+            for (int i = 0; i < TN; ++i)
+#pragma unroll
+                for (int j = 0; j < TM; ++j)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[j], wf[i], acc[i][j], 0, 0, 0);
+        }
+    };
+    // Steps are numbered 0 .. n_iter-1; the last one may be partial.  The steady-state loop has
+    // no branch between a load and its use (a branch there makes the compiler wait for the loads
+    // at once) and scheduling barriers keep the loads where they are written.
+    const int n_iter = (K + TG_BK - 1) / TG_BK;
+    const int n_full = K / TG_BK;
+    fetch_any(wreg[0], areg[0], 0);
+    stash(wreg[0], areg[0], 0);
+    int cur = 0, it = 0;
+    if (DEPTH == 2) {
+        if (n_iter > 1) fetch_any(wreg[0], areg[0], TG_BK);       // step 1, in flight
+        __syncthreads();
+        int held = 0;                                              // the register set with step it+1
+        while (it + 3 < n_full) {                                   // steps it+2 and it+3 are whole
+            fetch(wreg[DEPTH - 1], areg[DEPTH - 1], (it + 2) * TG_BK);
+            __builtin_amdgcn_sched_barrier(0);
+            compute(cur);
+            __builtin_amdgcn_sched_barrier(0);
+            stash(wreg[0], areg[0], cur ^ 1);
+            __syncthreads();
+            fetch(wreg[0], areg[0], (it + 3) * TG_BK);
+            __builtin_amdgcn_sched_barrier(0);
+            compute(cur ^ 1);
+            __builtin_amdgcn_sched_barrier(0);
+            stash(wreg[DEPTH - 1], areg[DEPTH - 1], cur);
+            __syncthreads();
+            it += 2;
+        }
+        while (it < n_iter) {                                       // the last steps, one at a time
+            if (it + 2 < n_iter) {
+                if (held == 0) fetch_any(wreg[DEPTH - 1], areg[DEPTH - 1], (it + 2) * TG_BK);
+                else fetch_any(wreg[0], areg[0], (it + 2) * TG_BK);
             }
-#pragma unroll
-            for (int i = 0; i < 2; ++i)
-#pragma unroll
-                for (int j = 0; j < 2; ++j)
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wf[i], af[j], acc[i][j], 0, 0, 0);
+            compute(cur);
+            if (it + 1 < n_iter) {
+                if (held == 0) stash(wreg[0], areg[0], cur ^ 1);
+                else stash(wreg[DEPTH - 1], areg[DEPTH - 1], cur ^ 1);
+                __syncthreads();
+                cur ^= 1;
+                held ^= 1;
+            }
+            ++it;
+        }
+    } else {
+        __syncthreads();
+        while (it + 1 < n_full) {                                   // step it+1 is whole
+            fetch(wreg[0], areg[0], (it + 1) * TG_BK);
+            __builtin_amdgcn_sched_barrier(0);
+            compute(cur);
+            __builtin_amdgcn_sched_barrier(0);
+            stash(wreg[0], areg[0], cur ^ 1);
+            __syncthreads();
+            cur ^= 1;
+            ++it;
+        }
+        while (it < n_iter) {
+            if (it + 1 < n_iter) fetch_any(wreg[0], areg[0], (it + 1) * TG_BK);
+            compute(cur);
+            if (it + 1 < n_iter) {
+                stash(wreg[0], areg[0], cur ^ 1);
+                __syncthreads();
+                cur ^= 1;
+            }
+            ++it;
         }
     }
-    // accumulator element e of tile (i, j): n = wn + 32i + 8*(e/4) + 4*kq + e%4, m = wm + 32j + l32
+    // accumulator element e of tile (i, j): m = wm + 32j + 8*(e/4) + 4*kq + e%4, n = wn + 32i + l32
 #pragma unroll
-    for (int j = 0; j < 2; ++j) {
-        const int m = m0 + wm + 32 * j + l32;
-        if (m >= M) continue;
+    for (int i = 0; i < TN; ++i) {
+        const int n = n0 + wn + 32 * i + l32;
 #pragma unroll
-        for (int i = 0; i < 2; ++i) {
+        for (int j = 0; j < TM; ++j) {
 #pragma unroll
-            for (int g = 0; g < 4; ++g) {
-                const int n = n0 + wn + 32 * i + 8 * g + 4 * kq;
+            for (int e = 0; e < 16; ++e) {
+                const int m = m0 + wm + 32 * j + 8 * (e / 4) + 4 * kq + e % 4;
+                const float v = acc[i][j][e];
                 if (EPI == 2) {
-                    TC* p = C + (int64_t)m * ldc + n / 2;
-                    if (n + 1 < N) p[0] = from_f32<TC>(silu_mul(acc[i][j][4 * g], acc[i][j][4 * g + 1]));
-                    if (n + 3 < N) p[1] = from_f32<TC>(silu_mul(acc[i][j][4 * g + 2], acc[i][j][4 * g + 3]));
-                } else {
+                    // gate at even n, up at odd n: the odd lane hands its value to the even one
+                    const float up = __shfl_xor(v, 1, WAVE);
+                    if (m < M && (l32 & 1) == 0 && n + 1 < N) C[(int64_t)m * ldc + n / 2] = from_f32<TC>(silu_mul(v, up));
+                } else if (m < M && n < N) {
                     TC* p = C + (int64_t)m * ldc + n;
-#pragma unroll
-                    for (int e = 0; e < 4; ++e) {
-                        if (n + e >= N) continue;
-                        const float v = acc[i][j][4 * g + e];
-                        p[e] = from_f32<TC>(EPI == 1 ? to_f32<TC>(p[e]) + v : v);
-                    }
+                    *p = from_f32<TC>(EPI == 1 ? to_f32<TC>(*p) + v : v);
                 }
             }
         }
     }
 }
 
-extern "C" int picolm_gemm_tiled(const void* A, const void* W, void* C, int c_dt, int M, int N, int K,
-                                 int64_t lda, int64_t ldw, int64_t ldc, int epilogue, hipStream_t stream) {
-    if (check_mfma_operands("gemm_tiled", A, W, M, N, K, lda, ldw, ldc, epilogue, c_dt)) return -1;
-    if (M == 0) return 0;
-    const int tiles_m = ceil_div(M, TG_BM), tiles_n = ceil_div(N, TG_BN);
+template <int TN, int TM, int WN, int WM, int DEPTH>
+static int launch_tiled(const void* A, const void* W, void* C, int c_dt, int M, int N, int K, int64_t lda,
+                        int64_t ldw, int64_t ldc, int epilogue, hipStream_t stream) {
+    constexpr int BN = 32 * TN * WN, BM = 32 * TM * WM;
+    const int tiles_m = ceil_div(M, BM), tiles_n = ceil_div(N, BN);
     PICOLM_REQUIRE((int64_t)tiles_m * tiles_n < (1ll << 31), "gemm_tiled: too many tiles");
-    dim3 grid(tiles_m * tiles_n), block(TG_THREADS);
+    dim3 grid(tiles_m * tiles_n), block(64 * WN * WM);
+    const size_t lds = 2 * (size_t)(BN + BM) * TG_BK * sizeof(bf16_t);
     const bf16_t* a = (const bf16_t*)A;
     const bf16_t* w = (const bf16_t*)W;
-#define TG_LAUNCH(EPI, TC) \
-    gemm_tiled_kernel<EPI, TC><<<grid, block, 0, stream>>>(a, w, (TC*)C, M, N, K, lda, ldw, ldc, tiles_m, tiles_n)
-    if (epilogue == 0 && c_dt == PICOLM_F32) TG_LAUNCH(0, float);
-    else if (epilogue == 0 && c_dt == PICOLM_BF16) TG_LAUNCH(0, bf16_t);
-    else if (epilogue == 1 && c_dt == PICOLM_F32) TG_LAUNCH(1, float);
-    else if (epilogue == 2 && c_dt == PICOLM_BF16) TG_LAUNCH(2, bf16_t);
-    else if (epilogue == 2 && c_dt == PICOLM_F32) TG_LAUNCH(2, float);
+#define TG_LAUNCH(EPI, TC)                                                                                 \
+    {                                                                                                      \
+        static size_t raised = 48 * 1024;                                                                  \
+        if (lds > raised) {                                                                                \
+            hipError_t e = hipFuncSetAttribute((const void*)gemm_tiled_kernel<TN, TM, WN, WM, DEPTH, EPI, TC>,    \
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);      \
+            PICOLM_REQUIRE(e == hipSuccess, "gemm_tiled: cannot raise the LDS limit: %s",                  \
+                           hipGetErrorString(e));                                                          \
+            raised = lds;                                                                                  \
+        }                                                                                                  \
+        gemm_tiled_kernel<TN, TM, WN, WM, DEPTH, EPI, TC><<<grid, block, lds, stream>>>(a, w, (TC*)C, M, N, K, lda, \
+                                                                                ldw, ldc, tiles_m, tiles_n); \
+    }
+    if (epilogue == 0 && c_dt == PICOLM_F32) TG_LAUNCH(0, float)
+    else if (epilogue == 0 && c_dt == PICOLM_BF16) TG_LAUNCH(0, bf16_t)
+    else if (epilogue == 1 && c_dt == PICOLM_F32) TG_LAUNCH(1, float)
+    else if (epilogue == 2 && c_dt == PICOLM_BF16) TG_LAUNCH(2, bf16_t)
+    else if (epilogue == 2 && c_dt == PICOLM_F32) TG_LAUNCH(2, float)
     else PICOLM_REQUIRE(false, "gemm_tiled: unsupported epilogue %d with output dtype %d", epilogue, c_dt);
 #undef TG_LAUNCH
     PICOLM_LAUNCH_CHECK("gemm_tiled");
     return 0;
+}
+
+// variant: 0 picks the block tile by the number of tiles;
+// 1: 128x128 (4 waves), 2: 256(n)x128(m) (4 waves), 3: 256x256 (4 waves), 4: 256x256 (8 waves)
+extern "C" int picolm_gemm_tiled(const void* A, const void* W, void* C, int c_dt, int M, int N, int K,
+                                 int64_t lda, int64_t ldw, int64_t ldc, int epilogue, int variant,
+                                 hipStream_t stream) {
+    if (check_mfma_operands("gemm_tiled", A, W, M, N, K, lda, ldw, ldc, epilogue, c_dt)) return -1;
+    if (M == 0) return 0;
+    if (variant == 0) {
+        const int64_t t256 = (int64_t)ceil_div(M, 256) * ceil_div(N, 256);
+        variant = t256 >= 512 ? 4 : 1;      // the 256x256 tile pays once there are two rounds of it
+    }
+    switch (variant) {
+        case 1: return launch_tiled<2, 2, 2, 2, 2>(A, W, C, c_dt, M, N, K, lda, ldw, ldc, epilogue, stream);
+        case 2: return launch_tiled<4, 2, 2, 2, 2>(A, W, C, c_dt, M, N, K, lda, ldw, ldc, epilogue, stream);
+        case 3: return launch_tiled<4, 4, 2, 2, 1>(A, W, C, c_dt, M, N, K, lda, ldw, ldc, epilogue, stream);
+        case 4: return launch_tiled<2, 4, 4, 2, 1>(A, W, C, c_dt, M, N, K, lda, ldw, ldc, epilogue, stream);
+    }
+    PICOLM_REQUIRE(false, "gemm_tiled: unknown variant %d", variant);
 }

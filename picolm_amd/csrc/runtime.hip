@@ -56,3 +56,37 @@ extern "C" int picolm_read_probe(const void* src, size_t bytes, void* sink, int 
     PICOLM_LAUNCH_CHECK("read_probe");
     return 0;
 }
+
+// A compute-only kernel: what the matrix cores sustain on this machine with operands in
+// registers (no memory traffic), for the measurement harness's "achievable" MFMA rate.
+typedef __attribute__((ext_vector_type(8))) __bf16 probe_bf16x8;
+typedef __attribute__((ext_vector_type(16))) float probe_f32x16;
+__global__ __launch_bounds__(256) void mfma_probe_kernel(float* __restrict__ sink, int iters) {
+    probe_bf16x8 a, b;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        a[i] = (__bf16)(float)(threadIdx.x % 7);
+        b[i] = (__bf16)(float)(threadIdx.x % 5);
+    }
+    probe_f32x16 acc[8];
+#pragma unroll
+    for (int t = 0; t < 8; ++t)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) acc[t][e] = 0.f;
+    for (int it = 0; it < iters; ++it) {
+#pragma unroll
+        for (int t = 0; t < 8; ++t) acc[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, acc[t], 0, 0, 0);
+    }
+    float s = 0.f;
+#pragma unroll
+    for (int t = 0; t < 8; ++t) s += acc[t][0];
+    if (s == 12345.678f) sink[0] = s;
+}
+
+// flops done: blocks * 4 waves * iters * 8 * 32768
+extern "C" int picolm_mfma_probe(void* sink, int blocks, int iters, hipStream_t stream) {
+    PICOLM_REQUIRE(blocks > 0 && iters > 0, "mfma_probe: bad sizes");
+    mfma_probe_kernel<<<dim3(blocks), dim3(256), 0, stream>>>((float*)sink, iters);
+    PICOLM_LAUNCH_CHECK("mfma_probe");
+    return 0;
+}

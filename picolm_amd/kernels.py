@@ -44,7 +44,7 @@ def dir_entry_points():
             "picolm_attn_prefill_tile_rows", "picolm_attn_prefill_generic",
             "picolm_attn_decode_generic", "picolm_argmax", "picolm_sample", "picolm_gemm_skinny", "picolm_gemm_tiled",
             "picolm_attn_mfma_takes", "picolm_attn_prefill_mfma_heads", "picolm_attn_prefill_mfma_tile_tokens",
-            "picolm_attn_prefill_mfma", "picolm_attn_decode_mfma", "picolm_attn_merge", "picolm_read_probe"]
+            "picolm_attn_prefill_mfma", "picolm_attn_decode_mfma", "picolm_attn_merge", "picolm_read_probe", "picolm_mfma_probe"]
 
 
 def _check(rc: int) -> None:
@@ -264,11 +264,11 @@ def gemm_skinny(a, w, c, epilogue: int = EPI_STORE, variant: int = 0) -> None:
                                     c_int64(c.shape[1]), epilogue, variant, _stream()))
 
 
-def gemm_tiled(a, w, c, epilogue: int = EPI_STORE) -> None:
+def gemm_tiled(a, w, c, epilogue: int = EPI_STORE, variant: int = 0) -> None:
     """bf16 x bf16 on the matrix cores, LDS-tiled, for many rows."""
     M, N, K = _gemm_shapes(a, w, c, epilogue)
     _check(lib().picolm_gemm_tiled(_ptr(a), _ptr(w), _ptr(c), dt_of(c), M, N, K, c_int64(K), c_int64(K),
-                                   c_int64(c.shape[1]), epilogue, _stream()))
+                                   c_int64(c.shape[1]), epilogue, variant, _stream()))
 
 
 def mfma_gemm_takes(a, w, c, epilogue: int) -> bool:
@@ -365,3 +365,10 @@ def read_probe(src: torch.Tensor, sink: torch.Tensor, blocks: int = 4096, unroll
     _dev("read_probe.sink", sink, torch.int32)
     nbytes = src.numel() * src.element_size()
     _check(lib().picolm_read_probe(_ptr(src), ctypes.c_size_t(nbytes - nbytes % 16), _ptr(sink), blocks, int(unroll4), _stream()))
+
+
+def mfma_probe(sink: torch.Tensor, blocks: int, iters: int) -> float:
+    """Queue a compute-only MFMA kernel; returns the flops it performs."""
+    _dev("mfma_probe.sink", sink, torch.float32)
+    _check(lib().picolm_mfma_probe(_ptr(sink), blocks, iters, _stream()))
+    return blocks * 4 * iters * 8 * 32768.0

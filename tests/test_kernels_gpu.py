@@ -127,6 +127,13 @@ def test_gemm_tiled(M, N, Kd):
         run_gemm(K().gemm_tiled, M, N, Kd, epi, torch.bfloat16, torch.bfloat16, cdt)
 
 
+@pytest.mark.parametrize("variant", [1, 2, 3, 4])
+def test_gemm_tiled_block_tiles(variant):
+    for M, N, Kd in ((300, 530, 1032), (70, 260, 72), (513, 100, 200)):
+        for epi, cdt in ((0, torch.float32), (2, torch.bfloat16), (1, torch.float32)):
+            run_gemm(K().gemm_tiled, M, N, Kd, epi, torch.bfloat16, torch.bfloat16, cdt, variant=variant)
+
+
 def test_gemm_refuses_what_it_cannot_do():
     k = K()
     a = torch.zeros(4, 12, dtype=torch.bfloat16, device=DEV)
