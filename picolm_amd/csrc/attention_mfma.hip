@@ -36,14 +36,11 @@ __device__ __forceinline__ bf16x8 zero8() {
 // row i of an S^T tile holds key 16*((i>>2)&1) + 4*(i>>3) + (i&3) of the tile's 32 keys
 __device__ __forceinline__ int key_of_row(int i) { return 16 * ((i >> 2) & 1) + 4 * (i >> 3) + (i & 3); }
 
-__device__ __forceinline__ __bf16 to_bf16(float f) {
-    bf16_t b = f32_to_bf16_bits(f);
-    return *reinterpret_cast<__bf16*>(&b);
-}
+__device__ __forceinline__ __bf16 to_bf16(float f) { return (__bf16)f; }      // the hardware's round-to-nearest-even
 
 // One page of one wave: scores, online softmax, and the update of O^T.  KOP(t, s) returns the
 // K operand of tile t, k-step s; VOP(dt, t, ks) the V^T operand of column block dt.
-template <int D, typename KOP, typename VOP>
+template <int D, bool MASKED, typename KOP, typename VOP>
 __device__ __forceinline__ void attend_page(const bf16x8 (&Qf)[D / 16], f32x16 (&O)[D / 32], float& m_run,
                                             float& l_run, int key0, int qpos, bool q_ok, int window,
                                             float scale2, int h, KOP kop, VOP vop) {
@@ -60,9 +57,13 @@ __device__ __forceinline__ void attend_page(const bf16x8 (&Qf)[D / 16], f32x16 (
     for (int t = 0; t < 2; ++t)
 #pragma unroll
         for (int e = 0; e < 16; ++e) {
-            const int key = key0 + 32 * t + 16 * h + e;
-            const bool vis = q_ok && key <= qpos && (window <= 0 || qpos - key < window);
-            S[t][e] = vis ? S[t][e] * scale2 : NEG_BIG;
+            if (MASKED) {
+                const int key = key0 + 32 * t + 16 * h + e;
+                const bool vis = q_ok && key <= qpos && (window <= 0 || qpos - key < window);
+                S[t][e] = vis ? S[t][e] * scale2 : NEG_BIG;
+            } else {
+                S[t][e] *= scale2;          // every key of the page is visible to every query of the wave
+            }
             mx = fmaxf(mx, S[t][e]);
         }
     mx = fmaxf(mx, __shfl_xor(mx, 32, WAVE));
@@ -74,7 +75,7 @@ __device__ __forceinline__ void attend_page(const bf16x8 (&Qf)[D / 16], f32x16 (
     for (int t = 0; t < 2; ++t)
 #pragma unroll
         for (int e = 0; e < 16; ++e) {
-            const float p = S[t][e] > 0.5f * NEG_BIG ? exp2f(S[t][e] - m_new) : 0.f;
+            const float p = (!MASKED || S[t][e] > 0.5f * NEG_BIG) ? exp2f(S[t][e] - m_new) : 0.f;
             sum += p;
             Pf[t][e / 8][e % 8] = to_bf16(p);
         }
@@ -137,17 +138,31 @@ __device__ __forceinline__ void attend_tile(const bf16x8 (&Qf)[D / 16], const bf
 }
 
 // =============================================================================================
+// LDS tiles of the prefill kernel.  K rows are D bf16 (for D = 128 a row spans all 64 banks), V^T
+// rows are 64 bf16 (half of the banks); the 16-byte chunks of a row are XOR-permuted so that the
+// 16 lanes served in one LDS cycle touch every bank once.
 template <int D>
-__global__ __launch_bounds__(256) void attn_prefill_mfma_kernel(AttnArgs a, int HB, int tile_tokens) {
-    constexpr int KCH = D / 8;                   // 16-byte chunks of a K row
-    constexpr int KSWZ = KCH < 8 ? KCH : 8;
-    __shared__ __attribute__((aligned(16))) bf16_t Ks[PAGE_TOKENS * D];    // [key][d], chunk c at c ^ (key % KSWZ)
-    __shared__ __attribute__((aligned(16))) bf16_t Vs[D * PAGE_TOKENS];    // [dcol][key], chunk c at c ^ (dcol % 8)
+__device__ __forceinline__ int k_off(int row, int chunk) {
+    constexpr int KCH = D / 8;
+    constexpr int ROWS_PER_SPAN = KCH >= 16 ? 1 : 16 / KCH;      // rows that share a 256-byte bank span
+    return (row * KCH + (chunk ^ ((row / ROWS_PER_SPAN) % KCH))) * 8;
+}
+__device__ __forceinline__ int v_off(int row, int chunk) { return (row * 8 + (chunk ^ ((row >> 1) & 7))) * 8; }
+
+template <int D>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void attn_prefill_mfma_kernel(AttnArgs a, int HB, int tile_tokens) {
+    constexpr int KCH = D / 8;                        // 16-byte chunks of a K row
+    constexpr int KP = PAGE_TOKENS * KCH / 256;       // K chunks a thread stages per page
+    constexpr int VP = D * 8 / 256;                   // V^T chunks a thread stages per page
+    constexpr int STAGE = 2 * PAGE_TOKENS * D;        // K tile + V^T tile, in bf16
+    extern __shared__ __attribute__((aligned(16))) bf16_t lds[];      // two stages
     const int tid = threadIdx.x, wave = tid / WAVE, lane = tid % WAVE;
     const int l32 = lane % 32, h = lane / 32;
     const int R = a.H / a.G;
     const int head_chunks = (R + HB - 1) / HB;
-    const int seq = a.tile_seq[blockIdx.x], q0 = a.tile_q0[blockIdx.x];
+    // long tiles first: the last tiles of a sequence see the most keys
+    const int tile_id = gridDim.x - 1 - blockIdx.x;
+    const int seq = a.tile_seq[tile_id], q0 = a.tile_q0[tile_id];
     const int g = blockIdx.y / head_chunks, chunk = blockIdx.y % head_chunks;
     const int head_local = chunk * HB + wave % HB;
     const int tb = wave / HB;
@@ -183,42 +198,65 @@ __global__ __launch_bounds__(256) void attn_prefill_mfma_kernel(AttnArgs a, int 
     const int32_t* pt = a.page_table + (size_t)a.seq_slot[seq] * a.max_pages;
     const size_t page_elems = (size_t)a.G * PAGE_TOKENS * D;
 
-    for (int page = page_lo; page < page_hi; ++page) {
+    bf16x8 kreg[KP], vreg[VP];
+    auto fetch = [&](int page) {
         const size_t base = (size_t)pt[page % a.ring_pages] * page_elems + (size_t)g * PAGE_TOKENS * D;
         const bf16_t* kp = (const bf16_t*)a.k_pages + base;
         const bf16_t* vp = (const bf16_t*)a.v_pages + base;
-        const int n_keys = min(PAGE_TOKENS, b_qlast - page * PAGE_TOKENS + 1);
+#pragma unroll
+        for (int i = 0; i < KP; ++i) kreg[i] = ldg8(kp + (size_t)(tid + 256 * i) * 8);
+#pragma unroll
+        for (int i = 0; i < VP; ++i) vreg[i] = ldg8(vp + (size_t)(tid + 256 * i) * 8);
+    };
+    auto stash = [&](int stage, int page) {
+        bf16_t* Ks = lds + stage * STAGE;
+        bf16_t* Vs = Ks + PAGE_TOKENS * D;
+        // keys past the sequence's end may hold anything: their values are zeroed, without a branch
+        const int n_keys = b_qlast - page * PAGE_TOKENS + 1;
+#pragma unroll
+        for (int i = 0; i < KP; ++i) {
+            const int idx = tid + 256 * i;
+            *(bf16x8*)(Ks + k_off<D>(idx / KCH, idx % KCH)) = kreg[i];
+        }
+#pragma unroll
+        for (int i = 0; i < VP; ++i) {
+            const int idx = tid + 256 * i;
+            const int c = idx % 8;
+            bf16x8 v = vreg[i];
+#pragma unroll
+            for (int e = 0; e < 8; ++e) v[e] = (8 * c + e < n_keys) ? v[e] : (__bf16)0.0f;
+            *(bf16x8*)(Vs + v_off(idx / 8, c)) = v;
+        }
+    };
+    auto compute = [&](int stage, int page) {
+        if (page < w_page_lo || page >= w_page_hi) return;
+        const bf16_t* Ks = lds + stage * STAGE;
+        const bf16_t* Vs = Ks + PAGE_TOKENS * D;
+        auto kop = [&](int t, int s) { return *(const bf16x8*)(Ks + k_off<D>(32 * t + key_of_row(l32), 2 * s + h)); };
+        auto vop = [&](int dt, int t, int ks) { return *(const bf16x8*)(Vs + v_off(32 * dt + l32, 4 * t + 2 * h + ks)); };
+        // a page wholly before the wave's first query needs no mask (rows without a query are
+        // never stored, whatever they hold)
+        if (a.window <= 0 && page * PAGE_TOKENS + PAGE_TOKENS - 1 <= w_qfirst)
+            attend_page<D, false>(Qf, O, m_run, l_run, page * PAGE_TOKENS, qpos, q_ok, a.window, scale2, h, kop, vop);
+        else
+            attend_page<D, true>(Qf, O, m_run, l_run, page * PAGE_TOKENS, qpos, q_ok, a.window, scale2, h, kop, vop);
+    };
+
+    fetch(page_lo);
+    stash(0, page_lo);
+    __syncthreads();
+    int cur = 0;
+    for (int page = page_lo; page + 1 < page_hi; ++page) {
+        fetch(page + 1);                          // in flight while this page is attended to
+        __builtin_amdgcn_sched_barrier(0);
+        compute(cur, page);
+        __builtin_amdgcn_sched_barrier(0);
+        stash(cur ^ 1, page + 1);
         __syncthreads();
-#pragma unroll
-        for (int idx = tid; idx < PAGE_TOKENS * KCH; idx += 256) {
-            const int row = idx / KCH, c = idx % KCH;
-            *(bf16x8*)(Ks + (row * KCH + (c ^ (row % KSWZ))) * 8) = ldg8(kp + (size_t)idx * 8);
-        }
-#pragma unroll
-        for (int idx = tid; idx < D * 8; idx += 256) {
-            const int row = idx / 8, c = idx % 8;
-            bf16x8 v = ldg8(vp + (size_t)idx * 8);
-            if (n_keys < PAGE_TOKENS) {          // keys past the sequence's end may hold anything
-#pragma unroll
-                for (int e = 0; e < 8; ++e)
-                    if (8 * c + e >= n_keys) v[e] = (__bf16)0.0f;
-            }
-            *(bf16x8*)(Vs + (row * 8 + (c ^ (row % 8))) * 8) = v;
-        }
-        __syncthreads();
-        if (page >= w_page_lo && page < w_page_hi) {
-            attend_page<D>(
-                Qf, O, m_run, l_run, page * PAGE_TOKENS, qpos, q_ok, a.window, scale2, h,
-                [&](int t, int s) {
-                    const int row = 32 * t + key_of_row(l32);
-                    return *(const bf16x8*)(Ks + (row * KCH + ((2 * s + h) ^ (row % KSWZ))) * 8);
-                },
-                [&](int dt, int t, int ks) {
-                    const int row = 32 * dt + l32;
-                    return *(const bf16x8*)(Vs + (row * 8 + ((4 * t + 2 * h + ks) ^ (row % 8))) * 8);
-                });
-        }
+        cur ^= 1;
     }
+    compute(cur, page_hi - 1);
+
     if (!q_ok) return;
     const float inv = l_run > 0.f ? 1.0f / l_run : 0.f;
     bf16_t* o = (bf16_t*)a.out + tok * a.H * D + (size_t)head * D;
@@ -384,9 +422,19 @@ extern "C" int picolm_attn_prefill_mfma(const void* q, const void* k_pages, cons
     AttnArgs a = {q, k_pages, v_pages, out, nullptr, tile_seq, tile_q0, seq_slot, seq_pos0, seq_nnew,
                   cu_seqlens, page_table, max_pages, ring_pages, H, G, d, window, scale, 0, 1};
     dim3 grid(n_tiles, G * head_chunks), block(256);
-    if (d == 32) attn_prefill_mfma_kernel<32><<<grid, block, 0, stream>>>(a, HB, tile_tokens);
-    else if (d == 64) attn_prefill_mfma_kernel<64><<<grid, block, 0, stream>>>(a, HB, tile_tokens);
-    else attn_prefill_mfma_kernel<128><<<grid, block, 0, stream>>>(a, HB, tile_tokens);
+    const size_t lds = 2 * 2 * (size_t)PAGE_TOKENS * d * sizeof(bf16_t);       // two stages of K and V^T
+    if (d == 32) attn_prefill_mfma_kernel<32><<<grid, block, lds, stream>>>(a, HB, tile_tokens);
+    else if (d == 64) attn_prefill_mfma_kernel<64><<<grid, block, lds, stream>>>(a, HB, tile_tokens);
+    else {
+        static bool raised = false;
+        if (!raised) {
+            hipError_t e = hipFuncSetAttribute((const void*)attn_prefill_mfma_kernel<128>,
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+            PICOLM_REQUIRE(e == hipSuccess, "attn_prefill_mfma: cannot raise the LDS limit: %s", hipGetErrorString(e));
+            raised = true;
+        }
+        attn_prefill_mfma_kernel<128><<<grid, block, lds, stream>>>(a, HB, tile_tokens);
+    }
     PICOLM_LAUNCH_CHECK("attn_prefill_mfma");
     return 0;
 }
