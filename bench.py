@@ -59,6 +59,7 @@ def main() -> int:
     ap.add_argument("--batch", type=int, default=8)
     ap.add_argument("--layers", type=int, default=0, help="fewer layers than the 32 of the shape (0: all)")
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 / 64 points and the prefill")
+    ap.add_argument("--prefill-only", action="store_true", help="run only the 2,048-token prefill (for profiling)")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py measures one GPU; --gpus {args.gpus} is not supported by this single-GPU library")
@@ -130,6 +131,10 @@ def main() -> int:
         torch.cuda.empty_cache()
         return float(np.median(times[1:]))
 
+    if args.prefill_only:
+        sec = prefill_run(PREFILL_TOKENS)
+        print(json.dumps({"prefill_ms": round(sec * 1e3, 3), "tokens": PREFILL_TOKENS, "layers": cfg.num_hidden_layers}))
+        return 0
     tok_s, s_per_step, ctx_tokens = decode_run(args.batch, args.steps, args.warmup)
     step_bytes = weight_bytes(cfg) + ctx_tokens * kv_bytes_per_token(cfg)
     achieved = step_bytes / s_per_step / 1e9
