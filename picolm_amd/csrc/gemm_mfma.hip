@@ -468,7 +468,8 @@ static int launch_tiled(const void* A, const void* W, void* C, int c_dt, int M, 
 }
 
 // variant: 0 picks the block tile by the number of tiles;
-// 1: 128x128 (4 waves), 2: 256(n)x128(m) (4 waves), 3: 256x256 (4 waves), 4: 256x256 (8 waves)
+// 1: 128x128 (4 waves), 2: 256(n)x128(m) (4 waves), 3: 256x256 (4 waves), 4: 256x256 (8 waves);
+// 5-8: 64 rows of activations against 128 or 64 weight rows, for decode batches too wide for the skinny kernel
 extern "C" int picolm_gemm_tiled(const void* A, const void* W, void* C, int c_dt, int M, int N, int K,
                                  int64_t lda, int64_t ldw, int64_t ldc, int epilogue, int variant,
                                  hipStream_t stream) {
@@ -483,6 +484,10 @@ extern "C" int picolm_gemm_tiled(const void* A, const void* W, void* C, int c_dt
         case 2: return launch_tiled<4, 2, 2, 2, 2>(A, W, C, c_dt, M, N, K, lda, ldw, ldc, epilogue, stream);
         case 3: return launch_tiled<4, 4, 2, 2, 1>(A, W, C, c_dt, M, N, K, lda, ldw, ldc, epilogue, stream);
         case 4: return launch_tiled<2, 4, 4, 2, 1>(A, W, C, c_dt, M, N, K, lda, ldw, ldc, epilogue, stream);
+        case 5: return launch_tiled<2, 2, 2, 1, 2>(A, W, C, c_dt, M, N, K, lda, ldw, ldc, epilogue, stream);
+        case 6: return launch_tiled<2, 1, 2, 2, 2>(A, W, C, c_dt, M, N, K, lda, ldw, ldc, epilogue, stream);
+        case 7: return launch_tiled<1, 2, 4, 1, 2>(A, W, C, c_dt, M, N, K, lda, ldw, ldc, epilogue, stream);
+        case 8: return launch_tiled<1, 2, 2, 1, 2>(A, W, C, c_dt, M, N, K, lda, ldw, ldc, epilogue, stream);
     }
     PICOLM_REQUIRE(false, "gemm_tiled: unknown variant %d", variant);
 }

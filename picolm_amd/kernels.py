@@ -287,10 +287,16 @@ def mfma_gemm_takes(a, w, c, epilogue: int) -> bool:
 def gemm(a: torch.Tensor, w: torch.Tensor, c: torch.Tensor, epilogue: int = EPI_STORE) -> None:
     """The product the engine calls: picks the kernel for the operands' types and sizes."""
     if mfma_gemm_takes(a, w, c, epilogue):
-        if a.shape[0] <= SKINNY_MAX_M:
-            gemm_skinny(a, w, c, epilogue)
-        else:
+        M, N = a.shape[0], w.shape[0]
+        if M > SKINNY_MAX_M:
             gemm_tiled(a, w, c, epilogue)
+        elif M > 8 and N >= 16384:
+            # many output columns: weights through LDS in 128-row tiles, all rows in one 64-row tile
+            gemm_tiled(a, w, c, epilogue, variant=7)
+        elif M > 32 and N >= 6144:
+            gemm_tiled(a, w, c, epilogue, variant=8)
+        else:
+            gemm_skinny(a, w, c, epilogue)
     else:
         gemm_generic(a, w, c, epilogue)
 

@@ -127,9 +127,9 @@ def test_gemm_tiled(M, N, Kd):
         run_gemm(K().gemm_tiled, M, N, Kd, epi, torch.bfloat16, torch.bfloat16, cdt)
 
 
-@pytest.mark.parametrize("variant", [1, 2, 3, 4])
+@pytest.mark.parametrize("variant", [1, 2, 3, 4, 5, 6, 7, 8])
 def test_gemm_tiled_block_tiles(variant):
-    for M, N, Kd in ((300, 530, 1032), (70, 260, 72), (513, 100, 200)):
+    for M, N, Kd in ((300, 530, 1032), (70, 260, 72), (513, 100, 200), (9, 700, 136), (64, 130, 64)):
         for epi, cdt in ((0, torch.float32), (2, torch.bfloat16), (1, torch.float32)):
             run_gemm(K().gemm_tiled, M, N, Kd, epi, torch.bfloat16, torch.bfloat16, cdt, variant=variant)
 
