@@ -60,6 +60,7 @@ def main() -> int:
     ap.add_argument("--layers", type=int, default=0, help="fewer layers than the 32 of the shape (0: all)")
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 / 64 points and the prefill")
     ap.add_argument("--prefill-only", action="store_true", help="run only the 2,048-token prefill (for profiling)")
+    ap.add_argument("--batch-only", action="store_true", help="run only the decode at --batch (for profiling)")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py measures one GPU; --gpus {args.gpus} is not supported by this single-GPU library")
@@ -156,7 +157,7 @@ def main() -> int:
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBS, 4)},
     }
-    if not args.no_points:
+    if not (args.no_points or args.batch_only):
         sec = prefill_run(PREFILL_TOKENS)
         fl = prefill_flops(cfg, PREFILL_TOKENS)
         record["prefill"] = {"value": round(PREFILL_TOKENS / sec, 1), "tokens": PREFILL_TOKENS, "ms": round(sec * 1e3, 3),

@@ -34,12 +34,14 @@ __global__ __launch_bounds__(AT_THREADS) void attn_tile_kernel(AttnArgs a) {
     const int tid = threadIdx.x, wave = tid / WAVE, lane = tid % WAVE;
     const int R = a.H / a.G;
     int seq, g, split = 0, n_rows;
+    DecodeWork work = {0, 0, 0, 0, 1};
     if (a.decode) {
-        seq = blockIdx.x;
+        if (!decode_work(a, work)) return;
+        seq = work.seq;
+        split = work.split;
         const int chunks = (R + AT_ROWS - 1) / AT_ROWS;
         g = blockIdx.y / chunks;
         const int chunk = blockIdx.y % chunks;
-        split = blockIdx.z;
         n_rows = min(AT_ROWS, R - chunk * AT_ROWS);
         if (tid < AT_ROWS) {
             row_tok[tid] = a.cu_seqlens[seq];
@@ -64,12 +66,9 @@ __global__ __launch_bounds__(AT_THREADS) void attn_tile_kernel(AttnArgs a) {
     const int hi = qpos_last;
     const int lo = a.window > 0 ? max(0, qpos_first - a.window + 1) : 0;
     int page_lo = lo / PAGE_TOKENS, page_hi = hi / PAGE_TOKENS + 1;   // [page_lo, page_hi)
-    if (a.decode && a.n_splits > 1) {
-        const int np = page_hi - page_lo;
-        const int per = (np + a.n_splits - 1) / a.n_splits;
-        const int b = page_lo + split * per;
-        page_hi = min(page_hi, b + per);
-        page_lo = b;
+    if (a.decode) {
+        page_lo = work.page_lo;
+        page_hi = work.page_hi;
     }
 
     const T* q = (const T*)a.q;
@@ -168,8 +167,8 @@ __global__ __launch_bounds__(AT_THREADS) void attn_tile_kernel(AttnArgs a) {
     __syncthreads();
     if (pr >= n_rows) return;
     const int tok = row_tok[pr], head = row_head[pr];
-    if (a.decode && a.partial) {
-        float* po = a.partial + (((size_t)seq * a.H + head) * a.n_splits + split) * (d + 2);
+    if (a.decode && work.n_chunks > 1) {
+        float* po = a.partial + (((size_t)seq * a.H + head) * a.max_splits + split) * (d + 2);
         if (pc == 0) {
             po[0] = m_s[pr];
             po[1] = l_s[pr];
@@ -191,16 +190,17 @@ __global__ __launch_bounds__(AT_THREADS) void attn_tile_kernel(AttnArgs a) {
 // One wave per (seq, head): lanes take splits for the statistics, then columns for the sum.
 #define MERGE_WAVES 4
 template <typename T>
-__global__ __launch_bounds__(MERGE_WAVES * WAVE) void attn_merge_kernel(const float* __restrict__ partial,
-                                                                        T* __restrict__ out,
-                                                                        const int32_t* __restrict__ cu_seqlens,
-                                                                        int n_units, int H, int d, int n_splits) {
+__global__ __launch_bounds__(MERGE_WAVES * WAVE) void attn_merge_kernel(AttnArgs a, int n_units) {
     const int unit = blockIdx.x * MERGE_WAVES + threadIdx.x / WAVE;
     const int lane = threadIdx.x % WAVE;
     if (unit >= n_units) return;
+    const int H = a.H, d = a.d;
     const int seq = unit / H, head = unit % H;
+    const int qpos = a.seq_pos0[seq];
+    const int n_splits = (qpos / 64 + 1 - decode_first_page(a, qpos) + a.pages_per_chunk - 1) / a.pages_per_chunk;
+    if (n_splits <= 1) return;                         // its one workgroup wrote the result itself
     const int stride = d + 2;
-    const float* p = partial + (size_t)unit * n_splits * stride;
+    const float* p = a.partial + (size_t)unit * a.max_splits * stride;
     // the first splits' columns are asked for together with the statistics, so that the sum
     // does not wait for a second trip to memory
     constexpr int EARLY = 8;
@@ -219,7 +219,7 @@ __global__ __launch_bounds__(MERGE_WAVES * WAVE) void attn_merge_kernel(const fl
     for (int i = lane; i < n_splits; i += WAVE) l += expf(p[(size_t)i * stride] - M) * p[(size_t)i * stride + 1];
     const float L = wave_sum(l);
     const float inv = L > 0.f ? 1.0f / L : 0.f;
-    T* o = out + (size_t)cu_seqlens[seq] * H * d + (size_t)head * d;
+    T* o = (T*)a.out + (size_t)a.cu_seqlens[seq] * H * d + (size_t)head * d;
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
         const int c = lane + j * WAVE;
@@ -253,6 +253,15 @@ static int launch_attn(const AttnArgs& a, dim3 grid, hipStream_t stream) {
     return 0;
 }
 
+int check_decode_chunks(const char* who, const float* partial, const int32_t* chunk_seq, const int32_t* chunk_idx,
+                        int n_chunks, int pages_per_chunk, int max_splits) {
+    PICOLM_REQUIRE(chunk_seq && chunk_idx && n_chunks >= 0, "%s: needs the step's work list", who);
+    PICOLM_REQUIRE(pages_per_chunk >= 1 && max_splits >= 1, "%s: bad chunking (%d pages a chunk, %d chunks a sequence)", who,
+                   pages_per_chunk, max_splits);
+    PICOLM_REQUIRE(max_splits == 1 || partial != nullptr, "%s: several chunks a sequence need a partial buffer", who);
+    return 0;
+}
+
 static int check_attn_sizes(const char* who, int H, int G, int d, int max_pages, int ring_pages) {
     PICOLM_REQUIRE(H > 0 && G > 0 && H % G == 0, "%s: %d heads do not split over %d groups", who, H, G);
     PICOLM_REQUIRE(d >= 16 && d % 16 == 0 && d <= AT_MAX_D,
@@ -262,18 +271,11 @@ static int check_attn_sizes(const char* who, int H, int G, int d, int max_pages,
     return 0;
 }
 
-extern "C" int picolm_attn_merge(const float* partial, void* out, int dt, int n_seq, const int32_t* cu_seqlens,
-                                 int H, int d, int n_splits, hipStream_t stream) {
-    PICOLM_REQUIRE(n_seq >= 0 && H > 0 && d > 0 && n_splits >= 1, "attn_merge: bad sizes");
-    if (n_seq == 0) return 0;
-    const int n_units = n_seq * H;
+int picolm_attn_merge_launch(const AttnArgs& a, int dt, int n_seq, hipStream_t stream) {
+    const int n_units = n_seq * a.H;
     dim3 mgrid(ceil_div(n_units, MERGE_WAVES)), mblock(MERGE_WAVES * WAVE);
-    if (dt == PICOLM_F32)
-        attn_merge_kernel<float><<<mgrid, mblock, 0, stream>>>(partial, (float*)out, cu_seqlens, n_units, H, d, n_splits);
-    else if (dt == PICOLM_BF16)
-        attn_merge_kernel<bf16_t><<<mgrid, mblock, 0, stream>>>(partial, (bf16_t*)out, cu_seqlens, n_units, H, d, n_splits);
-    else
-        PICOLM_REQUIRE(false, "attn_merge: unknown dtype %d", dt);
+    if (dt == PICOLM_F32) attn_merge_kernel<float><<<mgrid, mblock, 0, stream>>>(a, n_units);
+    else attn_merge_kernel<bf16_t><<<mgrid, mblock, 0, stream>>>(a, n_units);
     PICOLM_LAUNCH_CHECK("attn_merge");
     return 0;
 }
@@ -290,7 +292,7 @@ extern "C" int picolm_attn_prefill_generic(const void* q, const void* k_pages, c
     PICOLM_REQUIRE(H <= 65535, "attn_prefill: %d heads exceed the grid", H);
     if (n_tiles <= 0) return 0;
     AttnArgs a = {q, k_pages, v_pages, out, nullptr, tile_seq, tile_q0, seq_slot, seq_pos0, seq_nnew,
-                  cu_seqlens, page_table, max_pages, ring_pages, H, G, d, window, scale, 0, 1};
+                  cu_seqlens, page_table, max_pages, ring_pages, H, G, d, window, scale, 0, nullptr, nullptr, 0, 1};
     dim3 grid(n_tiles, H);
     if (dt == PICOLM_F32) return launch_attn<float>(a, grid, stream);
     if (dt == PICOLM_BF16) return launch_attn<bf16_t>(a, grid, stream);
@@ -300,26 +302,23 @@ extern "C" int picolm_attn_prefill_generic(const void* q, const void* k_pages, c
 extern "C" int picolm_attn_prefill_tile_rows(void) { return AT_ROWS; }
 
 extern "C" int picolm_attn_decode_generic(const void* q, const void* k_pages, const void* v_pages,
-                                          void* out, float* partial, int dt, int n_seq, int n_splits,
-                                          const int32_t* seq_slot, const int32_t* seq_pos0,
-                                          const int32_t* cu_seqlens, const int32_t* page_table,
-                                          int max_pages, int ring_pages, int H, int G, int d,
-                                          int window, float scale, hipStream_t stream) {
+                                          void* out, float* partial, int dt, int n_seq,
+                                          const int32_t* chunk_seq, const int32_t* chunk_idx, int n_chunks,
+                                          int pages_per_chunk, int max_splits, const int32_t* seq_slot,
+                                          const int32_t* seq_pos0, const int32_t* cu_seqlens,
+                                          const int32_t* page_table, int max_pages, int ring_pages, int H,
+                                          int G, int d, int window, float scale, hipStream_t stream) {
     if (check_attn_sizes("attn_decode", H, G, d, max_pages, ring_pages)) return -1;
-    PICOLM_REQUIRE(n_splits >= 1 && n_splits <= 65535, "attn_decode: bad split count %d", n_splits);
-    PICOLM_REQUIRE(n_splits == 1 || partial != nullptr, "attn_decode: splits need a partial buffer");
-    if (n_seq <= 0) return 0;
+    if (check_decode_chunks("attn_decode", partial, chunk_seq, chunk_idx, n_chunks, pages_per_chunk, max_splits)) return -1;
+    PICOLM_REQUIRE(dt == PICOLM_F32 || dt == PICOLM_BF16, "attn_decode: unknown dtype %d", dt);
+    if (n_seq <= 0 || n_chunks <= 0) return 0;
     const int chunks = ceil_div(H / G, AT_ROWS);
     PICOLM_REQUIRE(G * chunks <= 65535, "attn_decode: %d groups exceed the grid", G * chunks);
-    AttnArgs a = {q, k_pages, v_pages, out, n_splits > 1 ? partial : nullptr, nullptr, nullptr, seq_slot,
-                  seq_pos0, nullptr, cu_seqlens, page_table, max_pages, ring_pages, H, G, d, window,
-                  scale, 1, n_splits};
-    dim3 grid(n_seq, G * chunks, n_splits);
-    int rc;
-    if (dt == PICOLM_F32) rc = launch_attn<float>(a, grid, stream);
-    else if (dt == PICOLM_BF16) rc = launch_attn<bf16_t>(a, grid, stream);
-    else PICOLM_REQUIRE(false, "attn_decode: unknown dtype %d", dt);
+    AttnArgs a = {q, k_pages, v_pages, out, partial, nullptr, nullptr, seq_slot, seq_pos0, nullptr, cu_seqlens,
+                  page_table, max_pages, ring_pages, H, G, d, window, scale, 1, chunk_seq, chunk_idx,
+                  pages_per_chunk, max_splits};
+    dim3 grid(n_chunks, G * chunks);
+    const int rc = dt == PICOLM_F32 ? launch_attn<float>(a, grid, stream) : launch_attn<bf16_t>(a, grid, stream);
     if (rc) return rc;
-    if (n_splits > 1) return picolm_attn_merge(partial, out, dt, n_seq, cu_seqlens, H, d, n_splits, stream);
-    return 0;
+    return max_splits > 1 ? picolm_attn_merge_launch(a, dt, n_seq, stream) : 0;
 }

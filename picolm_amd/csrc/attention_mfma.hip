@@ -33,8 +33,17 @@ __device__ __forceinline__ bf16x8 zero8() {
     for (int i = 0; i < 8; ++i) z[i] = (__bf16)0.0f;
     return z;
 }
-// row i of an S^T tile holds key 16*((i>>2)&1) + 4*(i>>3) + (i&3) of the tile's 32 keys
-__device__ __forceinline__ int key_of_row(int i) { return 16 * ((i >> 2) & 1) + 4 * (i >> 3) + (i & 3); }
+// Row i of an S^T tile holds key_of_row(i) of the tile's 32 keys.  The accumulator of a lane in
+// wave half h holds rows 8a + 4h + b (a = 0..3, b = 0..3) as element 4a + b; with this map they
+// are the keys 8h .. 8h+7 (elements 0..7) and 16+8h .. 16+8h+7 (elements 8..15): P^T for step ks
+// of the second MFMA is elements 8ks .. 8ks+7 as they are, and the two halves of a wave read
+// adjacent 16-byte chunks of a V^T row.
+__device__ __forceinline__ int key_of_row(int i) {
+    const int hh = (i >> 2) & 1, aa = i >> 3, bb = i & 3;
+    return 16 * (aa >> 1) + 8 * hh + 4 * (aa & 1) + bb;
+}
+// key (within the tile) of accumulator element e of a lane in half h
+__device__ __forceinline__ int key_of_elem(int e, int h) { return 16 * (e >> 3) + 8 * h + (e & 7); }
 
 __device__ __forceinline__ __bf16 to_bf16(float f) { return (__bf16)f; }      // the hardware's round-to-nearest-even
 
@@ -58,7 +67,7 @@ __device__ __forceinline__ void attend_page(const bf16x8 (&Qf)[D / 16], f32x16 (
 #pragma unroll
         for (int e = 0; e < 16; ++e) {
             if (MASKED) {
-                const int key = key0 + 32 * t + 16 * h + e;
+                const int key = key0 + 32 * t + key_of_elem(e, h);
                 const bool vis = q_ok && key <= qpos && (window <= 0 || qpos - key < window);
                 S[t][e] = vis ? S[t][e] * scale2 : NEG_BIG;
             } else {
@@ -108,7 +117,7 @@ __device__ __forceinline__ void attend_tile(const bf16x8 (&Qf)[D / 16], const bf
     float mx = NEG_BIG;
 #pragma unroll
     for (int e = 0; e < 16; ++e) {
-        const int key = key0 + 16 * h + e;
+        const int key = key0 + key_of_elem(e, h);
         const bool vis = q_ok && key <= qpos && (window <= 0 || qpos - key < window);
         S[e] = vis ? S[e] * scale2 : NEG_BIG;
         mx = fmaxf(mx, S[e]);
@@ -233,7 +242,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void a
         const bf16_t* Ks = lds + stage * STAGE;
         const bf16_t* Vs = Ks + PAGE_TOKENS * D;
         auto kop = [&](int t, int s) { return *(const bf16x8*)(Ks + k_off<D>(32 * t + key_of_row(l32), 2 * s + h)); };
-        auto vop = [&](int dt, int t, int ks) { return *(const bf16x8*)(Vs + v_off(32 * dt + l32, 4 * t + 2 * h + ks)); };
+        auto vop = [&](int dt, int t, int ks) { return *(const bf16x8*)(Vs + v_off(32 * dt + l32, 4 * t + 2 * ks + h)); };
         // a page wholly before the wave's first query needs no mask (rows without a query are
         // never stored, whatever they hold)
         if (a.window <= 0 && page * PAGE_TOKENS + PAGE_TOKENS - 1 <= w_qfirst)
@@ -279,30 +288,23 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void a
     const int l32 = lane % 32, h = lane / 32;
     const int R = a.H / a.G;
     const int chunks = (R + 31) / 32;
-    const int seq = blockIdx.x;
+    DecodeWork work;
+    if (!decode_work(a, work)) return;
+    const int seq = work.seq, split = work.split;
     const int g = blockIdx.y / chunks, chunk = blockIdx.y % chunks;
-    const int split = blockIdx.z;
     const int Rc = min(32, R - chunk * 32);
     const bool q_ok = l32 < Rc;
     const int head = g * R + chunk * 32 + (q_ok ? l32 : 0);
     const size_t tok = (size_t)a.cu_seqlens[seq];
     const int qpos = a.seq_pos0[seq];
 
-    int page_lo = (a.window > 0 ? max(0, qpos - a.window + 1) : 0) / PAGE_TOKENS;
-    int page_hi = qpos / PAGE_TOKENS + 1;
-    if (a.n_splits > 1) {
-        const int np = page_hi - page_lo;
-        const int per = (np + a.n_splits - 1) / a.n_splits;
-        const int b = page_lo + split * per;
-        page_hi = min(page_hi, b + per);
-        page_lo = b;
-    }
-    // k-step s of a lane covers d = (D/2)*h + 8s .. +8: a lane's K reads are one contiguous run
+    const int page_lo = work.page_lo, page_hi = work.page_hi;
+    // k-step s of a lane covers d = 16s + 8h .. +8: the two halves of a wave read 32 adjacent bytes of a key
     bf16x8 Qf[D / 16];
     {
-        const bf16_t* qp = (const bf16_t*)a.q + tok * a.H * D + (size_t)head * D + (D / 2) * h;
+        const bf16_t* qp = (const bf16_t*)a.q + tok * a.H * D + (size_t)head * D + 8 * h;
 #pragma unroll
-        for (int s = 0; s < D / 16; ++s) Qf[s] = q_ok ? ldg8(qp + 8 * s) : zero8();
+        for (int s = 0; s < D / 16; ++s) Qf[s] = q_ok ? ldg8(qp + 16 * s) : zero8();
     }
     f32x16 O[D / 32];
 #pragma unroll
@@ -316,8 +318,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void a
 
     for (int page = page_lo + wave; page < page_hi; page += 4) {
         const size_t base = (size_t)pt[page % a.ring_pages] * page_elems + (size_t)g * PAGE_TOKENS * D;
-        const bf16_t* kp = (const bf16_t*)a.k_pages + base + (D / 2) * h;
-        const bf16_t* vp = (const bf16_t*)a.v_pages + base + (size_t)l32 * PAGE_TOKENS + 16 * h;
+        const bf16_t* kp = (const bf16_t*)a.k_pages + base + 8 * h;
+        const bf16_t* vp = (const bf16_t*)a.v_pages + base + (size_t)l32 * PAGE_TOKENS + 8 * h;
         const int key0 = page * PAGE_TOKENS;
         const int n_keys = qpos - key0 + 1;          // >= 1; keys past it are not this sequence's
         // a page is two tiles of 32 keys; all operands of a tile are requested before the first
@@ -327,17 +329,17 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void a
             if (key0 + 32 * t > qpos) break;                 // nothing of this tile is visible
             bf16x8 Kf[D / 16], Vf[D / 32][2];
 #pragma unroll
-            for (int s = 0; s < D / 16; ++s) Kf[s] = ldg8(kp + (size_t)(32 * t + key_of_row(l32)) * D + 8 * s);
+            for (int s = 0; s < D / 16; ++s) Kf[s] = ldg8(kp + (size_t)(32 * t + key_of_row(l32)) * D + 16 * s);
 #pragma unroll
             for (int dt = 0; dt < D / 32; ++dt)
 #pragma unroll
-                for (int ks = 0; ks < 2; ++ks) Vf[dt][ks] = ldg8(vp + (size_t)(32 * dt) * PAGE_TOKENS + 32 * t + 8 * ks);
+                for (int ks = 0; ks < 2; ++ks) Vf[dt][ks] = ldg8(vp + (size_t)(32 * dt) * PAGE_TOKENS + 32 * t + 16 * ks);
             if (n_keys < 32 * (t + 1)) {                     // keys past the end may hold anything
 #pragma unroll
                 for (int dt = 0; dt < D / 32; ++dt)
 #pragma unroll
                     for (int ks = 0; ks < 2; ++ks) {
-                        const int k = 32 * t + 16 * h + 8 * ks;
+                        const int k = 32 * t + 16 * ks + 8 * h;
 #pragma unroll
                         for (int e = 0; e < 8; ++e)
                             if (k + e >= n_keys) Vf[dt][ks][e] = (__bf16)0.0f;
@@ -374,8 +376,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void a
             acc += f * row[2 + dcol];
         }
         const int hq = g * R + chunk * 32 + q;
-        if (a.partial) {
-            float* po = a.partial + (((size_t)seq * a.H + hq) * a.n_splits + split) * (D + 2);
+        if (work.n_chunks > 1) {
+            float* po = a.partial + (((size_t)seq * a.H + hq) * a.max_splits + split) * (D + 2);
             if (dcol == 0) {
                 po[0] = M * LN2;        // the merge kernel works with natural exponents
                 po[1] = L;
@@ -420,7 +422,7 @@ extern "C" int picolm_attn_prefill_mfma(const void* q, const void* k_pages, cons
     const int head_chunks = ceil_div(H / G, HB);
     PICOLM_REQUIRE(G * head_chunks <= 65535, "attn_prefill_mfma: %d head groups exceed the grid", G * head_chunks);
     AttnArgs a = {q, k_pages, v_pages, out, nullptr, tile_seq, tile_q0, seq_slot, seq_pos0, seq_nnew,
-                  cu_seqlens, page_table, max_pages, ring_pages, H, G, d, window, scale, 0, 1};
+                  cu_seqlens, page_table, max_pages, ring_pages, H, G, d, window, scale, 0, nullptr, nullptr, 0, 1};
     dim3 grid(n_tiles, G * head_chunks), block(256);
     const size_t lds = 2 * 2 * (size_t)PAGE_TOKENS * d * sizeof(bf16_t);       // two stages of K and V^T
     if (d == 32) attn_prefill_mfma_kernel<32><<<grid, block, lds, stream>>>(a, HB, tile_tokens);
@@ -439,20 +441,26 @@ extern "C" int picolm_attn_prefill_mfma(const void* q, const void* k_pages, cons
     return 0;
 }
 
+int check_decode_chunks(const char* who, const float* partial, const int32_t* chunk_seq, const int32_t* chunk_idx,
+                        int n_chunks, int pages_per_chunk, int max_splits);
+int picolm_attn_merge_launch(const AttnArgs& a, int dt, int n_seq, hipStream_t stream);
+
 extern "C" int picolm_attn_decode_mfma(const void* q, const void* k_pages, const void* v_pages, void* out,
-                                       float* partial, int n_seq, int n_splits, const int32_t* seq_slot,
-                                       const int32_t* seq_pos0, const int32_t* cu_seqlens,
-                                       const int32_t* page_table, int max_pages, int ring_pages, int H, int G,
-                                       int d, int window, float scale, hipStream_t stream) {
+                                       float* partial, int n_seq, const int32_t* chunk_seq,
+                                       const int32_t* chunk_idx, int n_chunks, int pages_per_chunk,
+                                       int max_splits, const int32_t* seq_slot, const int32_t* seq_pos0,
+                                       const int32_t* cu_seqlens, const int32_t* page_table, int max_pages,
+                                       int ring_pages, int H, int G, int d, int window, float scale,
+                                       hipStream_t stream) {
     if (check_sizes("attn_decode_mfma", H, G, d, max_pages, ring_pages)) return -1;
-    PICOLM_REQUIRE(n_splits >= 1 && n_splits <= 65535, "attn_decode_mfma: bad split count %d", n_splits);
-    PICOLM_REQUIRE(n_splits == 1 || partial != nullptr, "attn_decode_mfma: splits need a partial buffer");
-    if (n_seq <= 0) return 0;
+    if (check_decode_chunks("attn_decode_mfma", partial, chunk_seq, chunk_idx, n_chunks, pages_per_chunk, max_splits)) return -1;
+    if (n_seq <= 0 || n_chunks <= 0) return 0;
     const int R = H / G, chunks = ceil_div(R, 32);
     PICOLM_REQUIRE(G * chunks <= 65535, "attn_decode_mfma: %d groups exceed the grid", G * chunks);
-    AttnArgs a = {q, k_pages, v_pages, out, n_splits > 1 ? partial : nullptr, nullptr, nullptr, seq_slot, seq_pos0,
-                  nullptr, cu_seqlens, page_table, max_pages, ring_pages, H, G, d, window, scale, 1, n_splits};
-    dim3 grid(n_seq, G * chunks, n_splits), block(256);
+    AttnArgs a = {q, k_pages, v_pages, out, partial, nullptr, nullptr, seq_slot, seq_pos0, nullptr, cu_seqlens,
+                  page_table, max_pages, ring_pages, H, G, d, window, scale, 1, chunk_seq, chunk_idx,
+                  pages_per_chunk, max_splits};
+    dim3 grid(n_chunks, G * chunks), block(256);
     const size_t lds = sizeof(float) * 4 * (size_t)min(R, 32) * (d + 2);
     if (d == 32) attn_decode_mfma_kernel<32><<<grid, block, lds, stream>>>(a);
     else if (d == 64) attn_decode_mfma_kernel<64><<<grid, block, lds, stream>>>(a);
@@ -467,6 +475,5 @@ extern "C" int picolm_attn_decode_mfma(const void* q, const void* k_pages, const
         attn_decode_mfma_kernel<128><<<grid, block, lds, stream>>>(a);
     }
     PICOLM_LAUNCH_CHECK("attn_decode_mfma");
-    if (n_splits > 1) return picolm_attn_merge(partial, out, PICOLM_BF16, n_seq, cu_seqlens, H, d, n_splits, stream);
-    return 0;
+    return max_splits > 1 ? picolm_attn_merge_launch(a, PICOLM_BF16, n_seq, stream) : 0;
 }

@@ -20,28 +20,25 @@
 #define SM_LIST 1024
 #define SM_WAVES (SM_THREADS / WAVE)
 
-__global__ __launch_bounds__(1024) void argmax_kernel(const float* __restrict__ logits,
-                                                      int32_t* __restrict__ out, int V, int64_t ld) {
-    __shared__ float sv[16];
-    __shared__ int si[16];
-    const float* row = logits + (int64_t)blockIdx.x * ld;
-    float best = -INFINITY;
-    int best_i = 0x7fffffff;
-    for (int i = threadIdx.x; i < V; i += blockDim.x) {
-        const float v = row[i];
-        if (v > best || best_i == 0x7fffffff) {   // first element seen, or strictly greater
-            best = v;
-            best_i = i;
-        }
+// Stage 1: a row is cut into slices of ARGMAX_SLICE values, one workgroup each, which leave their
+// (maximum, lowest index of it) in `part`; stage 2 picks among a row's slices.  A row of 128k
+// logits is 32 workgroups instead of one.
+#define ARGMAX_SLICE 4096
+#define ARGMAX_THREADS 256
+
+__device__ __forceinline__ void argmax_merge(float& best, int& best_i, float ov, int oi) {
+    if (oi != 0x7fffffff && (best_i == 0x7fffffff || ov > best || (ov == best && oi < best_i))) {
+        best = ov;
+        best_i = oi;
     }
+}
+
+__device__ __forceinline__ void argmax_block(float& best, int& best_i, float* sv, int* si) {
 #pragma unroll
     for (int o = WAVE / 2; o > 0; o >>= 1) {
         const float ov = __shfl_xor(best, o, WAVE);
         const int oi = __shfl_xor(best_i, o, WAVE);
-        if (oi != 0x7fffffff && (best_i == 0x7fffffff || ov > best || (ov == best && oi < best_i))) {
-            best = ov;
-            best_i = oi;
-        }
+        argmax_merge(best, best_i, ov, oi);
     }
     const int wave = threadIdx.x / WAVE, lane = threadIdx.x % WAVE;
     if (lane == 0) {
@@ -49,24 +46,63 @@ __global__ __launch_bounds__(1024) void argmax_kernel(const float* __restrict__ 
         si[wave] = best_i;
     }
     __syncthreads();
-    if (threadIdx.x == 0) {
-        const int n_waves = blockDim.x / WAVE;
-        for (int w = 1; w < n_waves; ++w) {
-            if (si[w] != 0x7fffffff && (best_i == 0x7fffffff || sv[w] > best || (sv[w] == best && si[w] < best_i))) {
-                best = sv[w];
-                best_i = si[w];
-            }
+    if (threadIdx.x == 0)
+        for (int w = 1; w < (int)blockDim.x / WAVE; ++w) argmax_merge(best, best_i, sv[w], si[w]);
+}
+
+__global__ __launch_bounds__(ARGMAX_THREADS) void argmax_slice_kernel(const float* __restrict__ logits,
+                                                                      float* __restrict__ part_v,
+                                                                      int32_t* __restrict__ part_i, int V,
+                                                                      int64_t ld, int n_slices) {
+    __shared__ float sv[16];
+    __shared__ int si[16];
+    const float* row = logits + (int64_t)blockIdx.y * ld;
+    const int lo = blockIdx.x * ARGMAX_SLICE, hi = min(V, lo + ARGMAX_SLICE);
+    float best = -INFINITY;
+    int best_i = 0x7fffffff;
+    for (int i = lo + threadIdx.x; i < hi; i += ARGMAX_THREADS) {
+        const float v = row[i];
+        if (v > best || best_i == 0x7fffffff) {      // the first element seen, or strictly greater
+            best = v;
+            best_i = i;
         }
-        out[blockIdx.x] = best_i == 0x7fffffff ? 0 : best_i;
+    }
+    argmax_block(best, best_i, sv, si);
+    if (threadIdx.x == 0) {
+        part_v[(size_t)blockIdx.y * n_slices + blockIdx.x] = best;
+        part_i[(size_t)blockIdx.y * n_slices + blockIdx.x] = best_i;
     }
 }
 
-extern "C" int picolm_argmax(const float* logits, int32_t* out, int n_rows, int V, int64_t ld,
+__global__ __launch_bounds__(ARGMAX_THREADS) void argmax_pick_kernel(const float* __restrict__ part_v,
+                                                                     const int32_t* __restrict__ part_i,
+                                                                     int32_t* __restrict__ out, int n_slices) {
+    __shared__ float sv[16];
+    __shared__ int si[16];
+    float best = -INFINITY;
+    int best_i = 0x7fffffff;
+    for (int s = threadIdx.x; s < n_slices; s += ARGMAX_THREADS)
+        argmax_merge(best, best_i, part_v[(size_t)blockIdx.x * n_slices + s], part_i[(size_t)blockIdx.x * n_slices + s]);
+    argmax_block(best, best_i, sv, si);
+    if (threadIdx.x == 0) out[blockIdx.x] = best_i == 0x7fffffff ? 0 : best_i;
+}
+
+extern "C" int picolm_argmax_scratch_floats(int n_rows, int V) { return 2 * n_rows * ceil_div(V, ARGMAX_SLICE); }
+
+// `scratch`: picolm_argmax_scratch_floats(n_rows, V) floats of device memory
+extern "C" int picolm_argmax(const float* logits, int32_t* out, int n_rows, int V, int64_t ld, float* scratch,
                              hipStream_t stream) {
     PICOLM_REQUIRE(n_rows >= 0 && V > 0 && ld >= V, "argmax: bad sizes rows=%d V=%d ld=%lld", n_rows, V,
                    (long long)ld);
+    PICOLM_REQUIRE(scratch != nullptr, "argmax: needs its scratch buffer");
+    PICOLM_REQUIRE(n_rows <= 65535, "argmax: %d rows exceed the grid", n_rows);
     if (n_rows == 0) return 0;
-    argmax_kernel<<<dim3(n_rows), dim3(1024), 0, stream>>>(logits, out, V, ld);
+    const int n_slices = ceil_div(V, ARGMAX_SLICE);
+    float* part_v = scratch;
+    int32_t* part_i = (int32_t*)(scratch + (size_t)n_rows * n_slices);
+    argmax_slice_kernel<<<dim3(n_slices, n_rows), dim3(ARGMAX_THREADS), 0, stream>>>(logits, part_v, part_i, V, ld, n_slices);
+    PICOLM_LAUNCH_CHECK("argmax");
+    argmax_pick_kernel<<<dim3(n_rows), dim3(ARGMAX_THREADS), 0, stream>>>(part_v, part_i, out, n_slices);
     PICOLM_LAUNCH_CHECK("argmax");
     return 0;
 }

@@ -20,7 +20,7 @@ class StepError(ValueError):
 
 
 class StepBatch:
-    def __init__(self, slots, pos0, new_tokens, want, vocab_size: int, device, target_blocks: int = 512):
+    def __init__(self, slots, pos0, new_tokens, want, vocab_size: int, device, target_blocks: int = 1024):
         """slots[i]: cache slot of sequence i; pos0[i]: tokens it holds; new_tokens[i]: its
         next tokens; want[i]: indices into new_tokens[i] whose logits are asked for."""
         self.n_seq = len(slots)
@@ -73,6 +73,7 @@ class StepBatch:
         self._device = torch.device(device)
         self._upload(parts)
         self._tiles = {}
+        self._chunks = {}
 
     def _upload(self, parts) -> None:
         sizes = [max(len(v), 1) for v in parts.values()]
@@ -112,17 +113,37 @@ class StepBatch:
             yield _Chunk(self, seqs, lo, [min(chunk_tokens, self.n_new[i] - lo) for i in seqs],
                          [int(cu[i]) + lo for i in seqs])
 
-    def decode_splits(self, blocks_per_seq: int) -> int:
-        """How many slices of pages each sequence's decode attention is cut into."""
-        return decode_splits(self.n_seq, self.max_len, blocks_per_seq, self._target_blocks)
+    def decode_chunks(self, blocks_per_chunk: int, window: int, max_pages: int):
+        """The decode attention's work list for this step: (chunk_seq, chunk_idx, n_chunks,
+        pages_per_chunk, max_splits), the first two on the device."""
+        key = (blocks_per_chunk, window)
+        if key not in self._chunks:
+            ppc = decode_pages_per_chunk(self.pos0, blocks_per_chunk, self._target_blocks)
+            seq, idx, most = decode_chunk_list(self.pos0, window, ppc)
+            flat = torch.from_numpy(np.concatenate([seq, idx])).to(self._device)
+            self._chunks[key] = (flat[:len(seq)], flat[len(seq):], len(seq), ppc, most)
+        return self._chunks[key]
 
 
-def decode_splits(n_seq: int, max_len: int, blocks_per_seq: int, target_blocks: int = 512) -> int:
-    """A power of two: as many slices as give every wave of a 4-wave workgroup a page of its
-    own, within about `target_blocks` workgroups for the whole launch (two per CU)."""
-    want = max(1, target_blocks // max(1, n_seq * blocks_per_seq))
-    want = min(want, (pages_for(max_len) + 3) // 4)
-    return 1 << (max(want, 1).bit_length() - 1)
+def decode_pages_per_chunk(pos0, blocks_per_chunk: int, target_blocks: int = 1024) -> int:
+    """Pages that one workgroup of the decode attention takes: a power of two, at least one
+    page for each of its four waves, and more when the step would otherwise have far more
+    than `target_blocks` workgroups (a few for every CU)."""
+    total_pages = sum(int(p) // PAGE_TOKENS + 1 for p in pos0)
+    want = total_pages * max(1, blocks_per_chunk) // max(1, target_blocks)
+    return max(4, 1 << (max(want, 1).bit_length() - 1))
+
+
+def decode_chunk_list(pos0, window: int, pages_per_chunk: int):
+    """(chunk_seq, chunk_idx, most chunks of one sequence): every sequence's visible pages
+    (those of its last `window` keys, or all) cut into runs of `pages_per_chunk`.  The
+    kernels derive each chunk's pages from the same arithmetic."""
+    pos = np.asarray(pos0, dtype=np.int64)
+    first = (np.maximum(0, pos - window + 1) if window > 0 else np.zeros_like(pos)) // PAGE_TOKENS
+    n = (pos // PAGE_TOKENS + 1 - first + pages_per_chunk - 1) // pages_per_chunk
+    seq = np.repeat(np.arange(len(pos), dtype=np.int32), n)
+    idx = (np.arange(int(n.sum())) - np.repeat(np.cumsum(n) - n, n)).astype(np.int32)
+    return seq, idx, int(n.max())
 
 
 class _Chunk:
@@ -156,9 +177,9 @@ class DecodeBatch:
     is_decode = True
     max_new = 1
 
-    def __init__(self, n_seq: int, n_splits: int, device):
+    def __init__(self, n_seq: int, pages_per_chunk: int, device):
         self.n_seq = self.T = self.n_want = n_seq
-        self.n_splits = n_splits
+        self.pages_per_chunk = pages_per_chunk
         self.n_new = [1] * n_seq
         self.want_counts = [1] * n_seq
         n = n_seq
@@ -168,8 +189,8 @@ class DecodeBatch:
                            ("tok_seq", n), ("tokens", n), ("want_rows", n)):
             self._spans[name] = (off, size)
             off += size
-        self._host = torch.zeros(off, dtype=torch.int32).pin_memory() if torch.cuda.is_available() \
-            else torch.zeros(off, dtype=torch.int32)
+        self._device = torch.device(device)
+        self._host = self._host_block(off)
         self._dev = torch.zeros(off, dtype=torch.int32, device=device)
         h = self._host.numpy()
         ar = np.arange(n + 1, dtype=np.int32)
@@ -181,6 +202,13 @@ class DecodeBatch:
         for k, (o, s) in self._spans.items():
             setattr(self, k, self._dev[o:o + s])
         self.slots, self.pos0 = [], []
+        self._lists = {}        # window -> (host block, device block, max_splits)
+        self.frozen = False     # set once the launches are recorded: no further work list can join
+
+    @staticmethod
+    def _host_block(n: int):
+        t = torch.zeros(n, dtype=torch.int32)
+        return t.pin_memory() if torch.cuda.is_available() else t
 
     def fill(self, slots, pos0, tokens) -> None:
         self.slots, self.pos0 = list(slots), list(pos0)
@@ -189,6 +217,31 @@ class DecodeBatch:
         self._np["tok_pos"][:] = pos0
         self._np["tokens"][:] = tokens
         self._dev.copy_(self._host, non_blocking=False)
+        for window in self._lists:
+            self._fill_list(window)
 
-    def decode_splits(self, blocks_per_seq: int) -> int:
-        return self.n_splits
+    def _fill_list(self, window: int) -> None:
+        host, dev, most = self._lists[window]
+        seq, idx, n_most = decode_chunk_list(self.pos0, window, self.pages_per_chunk)
+        if n_most > most:
+            raise StepError(f"a sequence of {max(self.pos0) + 1} tokens has more pages than the cache was sized for")
+        cap = len(host) // 2
+        h = host.numpy()
+        h[:len(seq)] = seq
+        h[len(seq):cap] = -1            # workgroups of unused entries leave at once
+        h[cap:cap + len(idx)] = idx
+        dev.copy_(host, non_blocking=False)
+
+    def decode_chunks(self, blocks_per_chunk: int, window: int, max_pages: int):
+        """As StepBatch.decode_chunks, over a list of fixed capacity (every sequence at the
+        cache's full length) that `fill` rewrites in place."""
+        if window not in self._lists:
+            if self.frozen:
+                raise StepError("a recorded decode step cannot take another work list")
+            most = (max_pages + self.pages_per_chunk - 1) // self.pages_per_chunk
+            cap = self.n_seq * most
+            self._lists[window] = (self._host_block(2 * cap), torch.zeros(2 * cap, dtype=torch.int32, device=self._device), most)
+            self._fill_list(window)
+        host, dev, most = self._lists[window]
+        cap = len(host) // 2
+        return dev[:cap], dev[cap:], cap, self.pages_per_chunk, most

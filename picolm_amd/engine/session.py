@@ -12,15 +12,15 @@ import torch
 
 from ..cache import Cache, CacheFull
 from ..parts.base import Workspace
-from .batch import DecodeBatch, StepBatch, StepError, decode_splits
+from .batch import DecodeBatch, StepBatch, StepError, decode_pages_per_chunk
 from .model import DecoderModel
 
 
 class _DecodeGraph:
     """The kernel launches of one decode step of `n_seq` sequences, recorded as a HIP graph."""
 
-    def __init__(self, session: "Session", n_seq: int, n_splits: int):
-        self.batch = DecodeBatch(n_seq, n_splits, session.model.runtime.device)
+    def __init__(self, session: "Session", n_seq: int, pages_per_chunk: int):
+        self.batch = DecodeBatch(n_seq, pages_per_chunk, session.model.runtime.device)
         self.workspace = Workspace(session.model.runtime.device)      # its own: recorded addresses must stay
         self.graph = None
         self.logits = None
@@ -48,6 +48,7 @@ class _DecodeGraph:
                 if was_enabled:
                     gc.enable()
             self.graph = g
+            self.batch.frozen = True
         return logits
 
 
@@ -119,11 +120,11 @@ class Session:
                 raise StepError(f"token id {t} is outside the vocabulary of {self.vocab_size}")
         self.cache.reserve_many(slots, [p + 1 for p in pos0])
         self.cache.flush()
-        n_splits = decode_splits(len(slots), max(pos0) + 1, self._blocks_per_seq)
-        key = (len(slots), n_splits)
+        ppc = decode_pages_per_chunk(pos0, self._blocks_per_seq)
+        key = (len(slots), ppc)
         g = self._decode_graphs.get(key)
         if g is None:
-            g = self._decode_graphs[key] = _DecodeGraph(self, len(slots), n_splits)
+            g = self._decode_graphs[key] = _DecodeGraph(self, len(slots), ppc)
         logits = g.run(self, slots, pos0, tokens)
         for s, p in zip(slots, pos0):
             self.cache.set_length(s, p + 1)

@@ -42,9 +42,9 @@ def dir_entry_points():
     return ["picolm_abi_version", "picolm_device_check", "picolm_embed", "picolm_rmsnorm",
             "picolm_rope_kv_store", "picolm_silu_mul", "picolm_add_into", "picolm_gemm_generic",
             "picolm_attn_prefill_tile_rows", "picolm_attn_prefill_generic",
-            "picolm_attn_decode_generic", "picolm_argmax", "picolm_sample", "picolm_gemm_skinny", "picolm_gemm_tiled",
+            "picolm_attn_decode_generic", "picolm_argmax", "picolm_argmax_scratch_floats", "picolm_sample", "picolm_gemm_skinny", "picolm_gemm_tiled",
             "picolm_attn_mfma_takes", "picolm_attn_prefill_mfma_heads", "picolm_attn_prefill_mfma_tile_tokens",
-            "picolm_attn_prefill_mfma", "picolm_attn_decode_mfma", "picolm_attn_merge", "picolm_read_probe", "picolm_mfma_probe"]
+            "picolm_attn_prefill_mfma", "picolm_attn_decode_mfma", "picolm_read_probe", "picolm_mfma_probe"]
 
 
 def _check(rc: int) -> None:
@@ -221,21 +221,33 @@ def attn_prefill_generic(q, k_pages, v_pages, out, tile_seq, tile_q0, n_tiles, s
         page_table.shape[1], ring_pages, H, G, d, window, c_float(scale), _stream()))
 
 
-def attn_decode_generic(q, k_pages, v_pages, out, partial, n_seq, n_splits, seq_slot, seq_pos0,
-                        cu_seqlens, page_table, ring_pages, H, G, d, window, scale) -> None:
-    _attn_check(q, k_pages, v_pages, out, page_table, H, G, d)
-    if n_splits > 1:
+def _decode_check(q, partial, n_seq, chunk_seq, chunk_idx, n_chunks, pages_per_chunk, max_splits, seq_slot,
+                  seq_pos0, cu_seqlens, H, d) -> None:
+    if max_splits > 1:
         _dev("attn.partial", partial, torch.float32)
-        if partial.numel() < n_seq * H * n_splits * (d + 2):
+        if partial.numel() < n_seq * H * max_splits * (d + 2):
             raise KernelError("attn_decode: the partial buffer is too small")
     if q.shape[0] < n_seq:
         raise KernelError("attn_decode: fewer query rows than sequences")
+    if pages_per_chunk < 1 or max_splits < 1:
+        raise KernelError(f"attn_decode: {pages_per_chunk} pages a chunk, {max_splits} chunks a sequence")
+    _i32("attn.chunk_seq", chunk_seq, n_chunks)
+    _i32("attn.chunk_idx", chunk_idx, n_chunks)
     for nm, t in (("seq_slot", seq_slot), ("seq_pos0", seq_pos0), ("cu_seqlens", cu_seqlens)):
         _i32("attn." + nm, t, n_seq)
+
+
+def attn_decode_generic(q, k_pages, v_pages, out, partial, n_seq, chunk_seq, chunk_idx, n_chunks, pages_per_chunk,
+                        max_splits, seq_slot, seq_pos0, cu_seqlens, page_table, ring_pages, H, G, d, window,
+                        scale) -> None:
+    _attn_check(q, k_pages, v_pages, out, page_table, H, G, d)
+    _decode_check(q, partial, n_seq, chunk_seq, chunk_idx, n_chunks, pages_per_chunk, max_splits, seq_slot, seq_pos0,
+                  cu_seqlens, H, d)
     _check(lib().picolm_attn_decode_generic(
-        _ptr(q), _ptr(k_pages), _ptr(v_pages), _ptr(out), _ptr(partial if n_splits > 1 else None), dt_of(q),
-        n_seq, n_splits, _ptr(seq_slot), _ptr(seq_pos0), _ptr(cu_seqlens), _ptr(page_table),
-        page_table.shape[1], ring_pages, H, G, d, window, c_float(scale), _stream()))
+        _ptr(q), _ptr(k_pages), _ptr(v_pages), _ptr(out), _ptr(partial if max_splits > 1 else None), dt_of(q),
+        n_seq, _ptr(chunk_seq), _ptr(chunk_idx), n_chunks, pages_per_chunk, max_splits, _ptr(seq_slot),
+        _ptr(seq_pos0), _ptr(cu_seqlens), _ptr(page_table), page_table.shape[1], ring_pages, H, G, d, window,
+        c_float(scale), _stream()))
 
 
 def _attn_check(q, k_pages, v_pages, out, page_table, H, G, d):
@@ -247,11 +259,22 @@ def _attn_check(q, k_pages, v_pages, out, page_table, H, G, d):
     _dev("attn.page_table", page_table, torch.int32, 2)
 
 
-def argmax(logits: torch.Tensor, out: torch.Tensor) -> None:
+def argmax_scratch_floats(n_rows: int, V: int) -> int:
+    return lib().picolm_argmax_scratch_floats(n_rows, V)
+
+
+def argmax(logits: torch.Tensor, out: torch.Tensor, scratch: torch.Tensor | None = None) -> None:
+    """The first maximum of every row; `scratch` (float32, argmax_scratch_floats) is made if not given."""
     _dev("argmax.logits", logits, torch.float32, 2)
-    _i32("argmax.out", out, logits.shape[0])
-    _check(lib().picolm_argmax(_ptr(logits), _ptr(out), logits.shape[0], logits.shape[1],
-                               c_int64(logits.shape[1]), _stream()))
+    n, V = logits.shape
+    _i32("argmax.out", out, n)
+    need = argmax_scratch_floats(n, V)
+    if scratch is None:
+        scratch = torch.empty(max(need, 1), dtype=torch.float32, device=logits.device)
+    _dev("argmax.scratch", scratch, torch.float32)
+    if scratch.numel() < need:
+        raise KernelError(f"argmax: scratch holds {scratch.numel()} floats, {need} are needed")
+    _check(lib().picolm_argmax(_ptr(logits), _ptr(out), n, V, c_int64(V), _ptr(scratch), _stream()))
 
 
 SKINNY_MAX_M = 64
@@ -314,21 +337,17 @@ def attn_prefill_mfma(q, k_pages, v_pages, out, batch, page_table, ring_pages, H
         page_table.shape[1], ring_pages, H, G, d, window, c_float(scale), _stream()))
 
 
-def attn_decode_mfma(q, k_pages, v_pages, out, partial, n_seq, n_splits, seq_slot, seq_pos0, cu_seqlens,
-                     page_table, ring_pages, H, G, d, window, scale) -> None:
+def attn_decode_mfma(q, k_pages, v_pages, out, partial, n_seq, chunk_seq, chunk_idx, n_chunks, pages_per_chunk,
+                     max_splits, seq_slot, seq_pos0, cu_seqlens, page_table, ring_pages, H, G, d, window,
+                     scale) -> None:
     _attn_check(q, k_pages, v_pages, out, page_table, H, G, d)
-    if n_splits > 1:
-        _dev("attn.partial", partial, torch.float32)
-        if partial.numel() < n_seq * H * n_splits * (d + 2):
-            raise KernelError("attn_decode: the partial buffer is too small")
-    if q.shape[0] < n_seq:
-        raise KernelError("attn_decode: fewer query rows than sequences")
-    for nm, t in (("seq_slot", seq_slot), ("seq_pos0", seq_pos0), ("cu_seqlens", cu_seqlens)):
-        _i32("attn." + nm, t, n_seq)
+    _decode_check(q, partial, n_seq, chunk_seq, chunk_idx, n_chunks, pages_per_chunk, max_splits, seq_slot, seq_pos0,
+                  cu_seqlens, H, d)
     _check(lib().picolm_attn_decode_mfma(
-        _ptr(q), _ptr(k_pages), _ptr(v_pages), _ptr(out), _ptr(partial if n_splits > 1 else None), n_seq, n_splits,
-        _ptr(seq_slot), _ptr(seq_pos0), _ptr(cu_seqlens), _ptr(page_table), page_table.shape[1], ring_pages,
-        H, G, d, window, c_float(scale), _stream()))
+        _ptr(q), _ptr(k_pages), _ptr(v_pages), _ptr(out), _ptr(partial if max_splits > 1 else None), n_seq,
+        _ptr(chunk_seq), _ptr(chunk_idx), n_chunks, pages_per_chunk, max_splits, _ptr(seq_slot), _ptr(seq_pos0),
+        _ptr(cu_seqlens), _ptr(page_table), page_table.shape[1], ring_pages, H, G, d, window, c_float(scale),
+        _stream()))
 
 
 def attn_prefill(q, k_pages, v_pages, out, batch, page_table, ring_pages, H, G, d, window, scale) -> None:
@@ -341,12 +360,13 @@ def attn_prefill(q, k_pages, v_pages, out, batch, page_table, ring_pages, H, G, 
                          batch.seq_nnew, batch.cu_seqlens, page_table, ring_pages, H, G, d, window, scale)
 
 
-def attn_decode(q, k_pages, v_pages, out, partial, n_seq, n_splits, seq_slot, seq_pos0, cu_seqlens,
-                page_table, ring_pages, H, G, d, window, scale) -> None:
-    """Attention of one new token per sequence over its cache pages."""
+def attn_decode(q, k_pages, v_pages, out, partial, n_seq, chunk_seq, chunk_idx, n_chunks, pages_per_chunk,
+                max_splits, seq_slot, seq_pos0, cu_seqlens, page_table, ring_pages, H, G, d, window, scale) -> None:
+    """Attention of one new token per sequence over its cache pages.  (chunk_seq, chunk_idx) is
+    the step's work list: entry x gives workgroup x `pages_per_chunk` pages of one sequence."""
     fn = attn_decode_mfma if attn_mfma_takes(q, d) else attn_decode_generic
-    fn(q, k_pages, v_pages, out, partial, n_seq, n_splits, seq_slot, seq_pos0, cu_seqlens,
-       page_table, ring_pages, H, G, d, window, scale)
+    fn(q, k_pages, v_pages, out, partial, n_seq, chunk_seq, chunk_idx, n_chunks, pages_per_chunk, max_splits,
+       seq_slot, seq_pos0, cu_seqlens, page_table, ring_pages, H, G, d, window, scale)
 
 
 def sample(logits: torch.Tensor, out: torch.Tensor, temperature: float, top_k: int, top_p: float,

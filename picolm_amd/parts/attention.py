@@ -67,11 +67,11 @@ class Attention(Mixer):
         if b.is_decode:
             kernels.rope_kv_store(qkv, q, kp, vp, cos, sin, style, b.tok_pos, b.tok_seq, b.seq_slot, table, ring,
                                   H, G, d)
-            n_splits = b.decode_splits(G * ((H // G + 15) // 16))
-            partial = ctx.ws.get("attn.partial", (b.n_seq * H * n_splits * (d + 2),), torch.float32) \
-                if n_splits > 1 else None
-            kernels.attn_decode(q, k_pages, v_pages, out, partial, b.n_seq, n_splits, b.seq_slot, b.seq_pos0,
-                                b.cu_seqlens, table, ring, H, G, d, self.window, self.scale)
+            chunk_seq, chunk_idx, n_chunks, ppc, most = b.decode_chunks(G * ((H // G + 15) // 16), self.window,
+                                                                         table.shape[1])
+            partial = ctx.ws.get("attn.partial", (b.n_seq * H * most * (d + 2),), torch.float32) if most > 1 else None
+            kernels.attn_decode(q, k_pages, v_pages, out, partial, b.n_seq, chunk_seq, chunk_idx, n_chunks, ppc, most,
+                                b.seq_slot, b.seq_pos0, b.cu_seqlens, table, ring, H, G, d, self.window, self.scale)
         elif self.window > 0 and ring < table.shape[1] and b.max_new > WINDOW_STEP_TOKENS:
             # a ring holds a window and one chunk: write and answer the step chunk by chunk
             for c in b.chunks(WINDOW_STEP_TOKENS):

@@ -22,6 +22,7 @@ class Sampler:
         states = [_as_i64(stream_state(params.seed, i)) for i in range(n_sequences)]
         self.states = torch.tensor(states, dtype=torch.int64).to(self.device)
         self._out = torch.zeros(max(n_sequences, 1), dtype=torch.int32, device=self.device)
+        self._scratch = None
 
     def sample(self, logits: torch.Tensor, sequence_indices) -> list[int]:
         """`logits[i]` belongs to sequence `sequence_indices[i]`; returns one token each."""
@@ -29,7 +30,10 @@ class Sampler:
         out = self._out[:n]
         p = self.params
         if p.greedy:
-            kernels.argmax(logits, out)
+            need = kernels.argmax_scratch_floats(n, logits.shape[1])
+            if self._scratch is None or self._scratch.numel() < need:
+                self._scratch = torch.empty(need, dtype=torch.float32, device=self.device)
+            kernels.argmax(logits, out, self._scratch)
         else:
             idx = torch.tensor(list(sequence_indices), dtype=torch.int32).to(self.device)
             kernels.sample(logits, out, p.temperature, p.top_k, p.top_p, p.min_p, self.states, idx)

@@ -219,16 +219,29 @@ def test_attention_prefill(dtype, H, G, d, window):
     assert err <= tol(dtype, np.abs(ref).max()), err
 
 
+def decode_work_list(pos0, window, pages_per_chunk, spare=0):
+    """The work list the engine would build, with `spare` unused entries mixed in."""
+    from picolm_amd.engine.batch import decode_chunk_list
+    seq, idx, most = decode_chunk_list(pos0, window, pages_per_chunk)
+    if spare:
+        seq = np.concatenate([seq[:1], np.full(spare, -1, np.int32), seq[1:], np.full(spare, -1, np.int32)])
+        idx = np.concatenate([idx[:1], np.full(spare, 7, np.int32), idx[1:], np.full(spare, 0, np.int32)])
+    return torch.from_numpy(seq).to(DEV), torch.from_numpy(idx).to(DEV), len(seq), most
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("H,G,d", ATTN_SHAPES)
-@pytest.mark.parametrize("n_splits,window", [(1, 0), (3, 0), (16, 0), (2, 100)])
-def test_attention_decode(dtype, H, G, d, n_splits, window):
-    case = PagedCase(H, G, d, [0, 63, 64, 700, 129], [1, 1, 1, 1, 1], dtype, seed=H * d + n_splits)
+@pytest.mark.parametrize("pages_per_chunk,window,spare", [(64, 0, 0), (4, 0, 3), (1, 0, 0), (2, 100, 1), (3, 200, 0)])
+def test_attention_decode(dtype, H, G, d, pages_per_chunk, window, spare):
+    pos0 = [0, 63, 64, 700, 129]
+    case = PagedCase(H, G, d, pos0, [1, 1, 1, 1, 1], dtype, seed=H * d + pages_per_chunk)
     b = case.batch()
     out = torch.zeros_like(case.q_dev)
-    partial = torch.full((b.n_seq * H * n_splits * (d + 2),), float("nan"), device=DEV)
-    K().attn_decode(case.q_dev, case.k_pages, case.v_pages, out, partial, b.n_seq, n_splits, b.seq_slot, b.seq_pos0,
-                    b.cu_seqlens, case.table, case.table.shape[1], H, G, d, window, 1.0 / math.sqrt(d))
+    chunk_seq, chunk_idx, n_chunks, most = decode_work_list(pos0, window, pages_per_chunk, spare)
+    partial = torch.full((b.n_seq * H * most * (d + 2),), float("nan"), device=DEV)
+    K().attn_decode(case.q_dev, case.k_pages, case.v_pages, out, partial, b.n_seq, chunk_seq, chunk_idx, n_chunks,
+                    pages_per_chunk, most, b.seq_slot, b.seq_pos0, b.cu_seqlens, case.table, case.table.shape[1],
+                    H, G, d, window, 1.0 / math.sqrt(d))
     ref = case.reference(window)
     err = np.abs(out.double().cpu().numpy() - ref).max()
     assert err <= tol(dtype, np.abs(ref).max()), err
@@ -250,11 +263,13 @@ def test_attention_finds_a_far_key(dtype):
                 c.q[i][-1, :, 0] = 30.0
     case = PagedCase(H, G, d, [699], [1], dtype, seed=3, scale_q=boost)
     b = case.batch()
-    for n_splits in (1, 4):
+    for pages_per_chunk in (16, 4, 1):
         out = torch.zeros_like(case.q_dev)
-        partial = torch.zeros(b.n_seq * H * n_splits * (d + 2), device=DEV)
-        K().attn_decode(case.q_dev, case.k_pages, case.v_pages, out, partial, 1, n_splits, b.seq_slot, b.seq_pos0,
-                        b.cu_seqlens, case.table, case.table.shape[1], H, G, d, 0, 1.0 / math.sqrt(d))
+        chunk_seq, chunk_idx, n_chunks, most = decode_work_list([699], 0, pages_per_chunk)
+        partial = torch.zeros(b.n_seq * H * most * (d + 2), device=DEV)
+        K().attn_decode(case.q_dev, case.k_pages, case.v_pages, out, partial, 1, chunk_seq, chunk_idx, n_chunks,
+                        pages_per_chunk, most, b.seq_slot, b.seq_pos0, b.cu_seqlens, case.table, case.table.shape[1],
+                        H, G, d, 0, 1.0 / math.sqrt(d))
         got = out.double().cpu().numpy().reshape(H, d)
         for h in range(H):
             assert np.abs(got[h] - case.v[0][target, h // 2]).max() < 2e-2
