@@ -7,9 +7,11 @@
 //   skinny (M <= 64, the decode step): HBM-bound.  A wave streams 16*NT weight rows straight
 //     from global memory into MFMA operand registers, 16 bytes a lane; the waves of a block
 //     split K between them and reduce through LDS.  Every weight byte is read once.
-//   tiled (M > 64, the prefill step): block tiles of 128x128 to 256x256 staged through two LDS
-//     stages with an XOR swizzle of 16-byte chunks, loads two steps ahead, 32x32x16 MFMAs; here
-//     the activation tile is the first operand, so that stores are whole 128-byte runs.
+//   tiled (M > 64, the prefill step): block tiles of 128x128 to 256x256 in LDS with an XOR swizzle
+//     of 16-byte chunks, 32x32x16 MFMAs; here the activation tile is the first operand, so that
+//     stores are whole 128-byte runs.  Tiles reach LDS straight from global memory
+//     (global_load_lds) when K is a multiple of 64, else through staging registers.  These
+//     kernels are bound by what L2 delivers to the CUs, not by the matrix cores.
 //
 // The order of the K summation inside an MFMA does not matter, so a lane's 8-element chunk
 // may come from any K offset as long as both operands use the same offset.
@@ -34,7 +36,7 @@ __device__ __forceinline__ float silu_mul(float g, float u) { return g / (1.0f +
 // =============================================================================================
 #define SK_KSTEP 128      // K elements one wave consumes per step: 4 MFMAs of 32
 
-template <int MT, int NT, int WAVES, int EPI, typename TC, bool NOA = false>
+template <int MT, int NT, int WAVES, int EPI, typename TC>
 __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const bf16_t* __restrict__ A,
                                                                  const bf16_t* __restrict__ W,
                                                                  TC* __restrict__ C, int M, int N, int K,
@@ -77,7 +79,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const bf16_t* _
             for (int t = 0; t < NT; ++t) wv[buf][t][j] = load_chunk(wrow[t] + k0 + 32 * j);
 #pragma unroll
             for (int u = 0; u < MT; ++u)
-                if (!NOA) av[buf][u][j] = load_chunk(arow[u] + k0 + 32 * j);
+                av[buf][u][j] = load_chunk(arow[u] + k0 + 32 * j);
         }
     };
     auto multiply = [&](int buf) {
@@ -89,14 +91,6 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const bf16_t* _
                 for (int u = 0; u < MT; ++u)
                     acc[t][u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wv[buf][t][j], av[buf][u][j], acc[t][u], 0, 0, 0);
     };
-    if (NOA) {
-#pragma unroll
-        for (int b = 0; b < 2; ++b)
-#pragma unroll
-            for (int u = 0; u < MT; ++u)
-#pragma unroll
-                for (int j = 0; j < 4; ++j) av[b][u][j] = zero_chunk();
-    }
     int s = wave;
     if (s < n_full) fetch(0, s);
     while (s < n_full) {
@@ -224,16 +218,6 @@ extern "C" int picolm_gemm_skinny(const void* A, const void* W, void* C, int c_d
         case 4: return launch_skinny<2, 2, 8>(A, W, C, c_dt, M, N, K, lda, ldw, ldc, epilogue, stream);
         case 5: return launch_skinny<4, 1, 8>(A, W, C, c_dt, M, N, K, lda, ldw, ldc, epilogue, stream);
         case 6: return launch_skinny<4, 2, 4>(A, W, C, c_dt, M, N, K, lda, ldw, ldc, epilogue, stream);
-        case 11: {
-            dim3 grid(ceil_div(N, 16)), block(512);
-            gemm_skinny_kernel<1, 1, 8, 0, float, true><<<grid, block, sizeof(float) * 8 * 4 * 64, stream>>>(
-                (const bf16_t*)A, (const bf16_t*)W, (float*)C, M, N, K, lda, ldw, ldc);
-            return 0;
-        }
-        case 7: return launch_skinny<1, 1, 4>(A, W, C, c_dt, M, N, K, lda, ldw, ldc, epilogue, stream);
-        case 8: return launch_skinny<1, 1, 16>(A, W, C, c_dt, M, N, K, lda, ldw, ldc, epilogue, stream);
-        case 9: return launch_skinny<1, 2, 4>(A, W, C, c_dt, M, N, K, lda, ldw, ldc, epilogue, stream);
-        case 10: return launch_skinny<1, 4, 4>(A, W, C, c_dt, M, N, K, lda, ldw, ldc, epilogue, stream);
     }
     PICOLM_REQUIRE(false, "gemm_skinny: unknown variant %d", variant);
 }
@@ -467,27 +451,263 @@ static int launch_tiled(const void* A, const void* W, void* C, int c_dt, int M, 
     return 0;
 }
 
-// variant: 0 picks the block tile by the number of tiles;
-// 1: 128x128 (4 waves), 2: 256(n)x128(m) (4 waves), 3: 256x256 (4 waves), 4: 256x256 (8 waves);
-// 5-8: 64 rows of activations against 128 or 64 weight rows, for decode batches too wide for the skinny kernel
+// =============================================================================================
+// tiled, with tiles loaded straight into LDS
+// =============================================================================================
+// The same block tiles and MFMA layout as above, but global memory is read by
+// global_load_lds_dwordx4: a wave's 64 lanes bring 16 bytes each to 1 KB of consecutive LDS, with
+// no staging registers and no LDS store instructions.  That leaves room for NS stages of BK
+// columns, NS-1 of them in flight while one is multiplied, so that memory latency of several
+// steps is covered by a single wave per SIMD.  The XOR swizzle is applied on the global side:
+// the lane that fills LDS position p of a row fetches the chunk that belongs there.
+//
+// The loads are inline assembly so that the wait for "all but the newest steps" (s_waitcnt
+// vmcnt(n)) stays as written: the compiler, when it knows of such loads, waits for all of them
+// before any LDS read.  M0 carries the LDS address of a wave's 1 KB; nothing else here uses M0.
+template <int BK>
+__device__ __forceinline__ int swizzled_chunk(int row, int chunk) {
+    return BK == 32 ? chunk ^ ((row >> 2) & 3) : chunk ^ ((row >> 1) & 7);
+}
+__device__ __forceinline__ void load_16_bytes_to_lds(unsigned byte_offset, const void* base, unsigned lds_address) {
+    asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dwordx4 %0, %1"
+                 :
+                 : "v"(byte_offset), "s"(base), "s"(lds_address)
+                 : "memory");
+}
+template <int N_OUTSTANDING>
+__device__ __forceinline__ void wait_for_loads() {      // vmcnt(N), other counters untouched
+    static_assert(N_OUTSTANDING < 64, "vmcnt has six bits");
+    __builtin_amdgcn_s_waitcnt((N_OUTSTANDING & 15) | (7 << 4) | (15 << 8) | ((N_OUTSTANDING >> 4) << 14));
+}
+
+template <int TN, int TM, int WN, int WM, int BK, int NS, int EPI, typename TC>
+__global__ __launch_bounds__(64 * WN * WM) void gemm_direct_kernel(const bf16_t* __restrict__ A,
+                                                                   const bf16_t* __restrict__ W,
+                                                                   TC* __restrict__ C, int M, int N, int K,
+                                                                   int64_t lda, int64_t ldw, int64_t ldc,
+                                                                   int tiles_m, int tiles_n) {
+    constexpr int NW = WN * WM;
+    constexpr int BN = 32 * TN * WN, BM = 32 * TM * WM;
+    constexpr int CH = BK / 8;                 // 16-byte chunks in a row of a stage
+    constexpr int RG = 64 / CH;                // rows that one wave-wide load fills
+    constexpr int STAGE = (BN + BM) * BK;      // bf16 elements
+    constexpr int W_LOADS = BN / RG / NW, A_LOADS = BM / RG / NW;     // per wave and step
+    static_assert((BN / RG) % NW == 0 && (BM / RG) % NW == 0, "tile does not split over the waves");
+    extern __shared__ __attribute__((aligned(1024))) bf16_t lds[];
+    int tile;
+    {
+        const int nb = gridDim.x, per = nb / 8, rem = nb % 8;
+        const int xcd = blockIdx.x % 8, idx = blockIdx.x / 8;
+        tile = (xcd < rem ? xcd * (per + 1) : rem * (per + 1) + (xcd - rem) * per) + idx;
+    }
+    const int band = 8;
+    const int per_band = band * tiles_m;
+    const int b = tile / per_band, in_b = tile % per_band;
+    const int band_w = min(band, tiles_n - b * band);
+    const int tn = b * band + in_b % band_w, tm = in_b / band_w;
+    const int n0 = tn * BN, m0 = tm * BM;
+
+    const int tid = threadIdx.x, wave = tid / 64, lane = tid % 64;
+    const int wn = (wave % WN) * (32 * TN), wm = (wave / WN) * (32 * TM);
+    const int l32 = lane % 32, kq = lane / 32;
+
+    // load j of a wave fills rows (j * NW + wave) * RG .. + RG - 1 of the W (then the A) tile
+    const int lrow = lane / CH, lpos = lane % CH;
+    unsigned w_off[W_LOADS], a_off[A_LOADS];
+#pragma unroll
+    for (int j = 0; j < W_LOADS; ++j) {
+        const int row = (j * NW + wave) * RG + lrow;
+        const int r = min(n0 + row, N - 1) - n0;
+        w_off[j] = (unsigned)((r * ldw + swizzled_chunk<BK>(row, lpos) * 8) * 2);
+    }
+#pragma unroll
+    for (int j = 0; j < A_LOADS; ++j) {
+        const int row = (j * NW + wave) * RG + lrow;
+        const int r = min(m0 + row, M - 1) - m0;
+        a_off[j] = (unsigned)((r * lda + swizzled_chunk<BK>(row, lpos) * 8) * 2);
+    }
+    const bf16_t* w_tile = W + (int64_t)n0 * ldw;
+    const bf16_t* a_tile = A + (int64_t)m0 * lda;
+    const unsigned lds_wave = __builtin_amdgcn_readfirstlane(
+        (unsigned)(size_t)(__attribute__((address_space(3))) bf16_t*)lds + wave * (RG * BK * 2));
+    auto issue = [&](int stage, int step) {
+        const unsigned to = lds_wave + stage * (STAGE * 2);
+        const bf16_t* wsrc = w_tile + step * BK;
+        const bf16_t* asrc = a_tile + step * BK;
+#pragma unroll
+        for (int j = 0; j < W_LOADS; ++j) load_16_bytes_to_lds(w_off[j], wsrc, to + j * (NW * RG * BK * 2));
+#pragma unroll
+        for (int j = 0; j < A_LOADS; ++j) load_16_bytes_to_lds(a_off[j], asrc, to + (BN * BK * 2) + j * (NW * RG * BK * 2));
+    };
+
+    f32x16 acc[TN][TM];
+#pragma unroll
+    for (int i = 0; i < TN; ++i)
+#pragma unroll
+        for (int j = 0; j < TM; ++j)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
+
+    // Fragments of k-slice g+1 are read from LDS while the MFMAs of slice g run; the wait, the
+    // barrier and the next loads of a step sit in the middle of the last slice of the step before.
+    constexpr int KS = BK / 16;
+    static_assert(KS % 2 == 0, "fragment sets alternate by slice");
+    bf16x8 wf[2][TN], af[2][TM];
+    auto read_frags = [&](int stage, int ks, bf16x8 (&w)[TN], bf16x8 (&a)[TM]) {
+        const bf16_t* Ws = lds + stage * STAGE;
+        const bf16_t* As = Ws + BN * BK;
+        const int chunk = ks * 2 + kq;
+#pragma unroll
+        for (int i = 0; i < TN; ++i) {
+            const int row = wn + 32 * i + l32;
+            w[i] = *(const bf16x8*)(Ws + row * BK + swizzled_chunk<BK>(row, chunk) * 8);
+        }
+#pragma unroll
+        for (int j = 0; j < TM; ++j) {
+            const int row = wm + 32 * j + l32;
+            a[j] = *(const bf16x8*)(As + row * BK + swizzled_chunk<BK>(row, chunk) * 8);
+        }
+    };
+    auto multiply = [&](const bf16x8 (&w)[TN], const bf16x8 (&a)[TM], int i_lo, int i_hi) {
+#pragma unroll
+        for (int i = i_lo; i < i_hi; ++i)
+#pragma unroll
+            for (int j = 0; j < TM; ++j)
+                acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[j], w[i], acc[i][j], 0, 0, 0);
+    };
+    // K is a whole number of steps (the host sees to that).  Steps past the end load the last
+    // step again into a stage nobody reads, so that the count of loads in flight stays the same.
+    const int n_steps = K / BK;
+#pragma unroll
+    for (int s = 0; s < NS - 1; ++s) issue(s, min(s, n_steps - 1));
+    // begin step j: its loads have landed for every wave, the stage of step j-1 is read out and
+    // takes the loads of step j+NS-1
+    wait_for_loads<(W_LOADS + A_LOADS) * (NS - 2)>();
+    __syncthreads();
+    __builtin_amdgcn_sched_barrier(0);
+    issue(NS - 1, min(NS - 1, n_steps - 1));
+    read_frags(0, 0, wf[0], af[0]);
+    int stage = 0;
+    for (int it = 0; it < n_steps; ++it) {
+        const int next_stage = stage + 1 == NS ? 0 : stage + 1;
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+            if (ks + 1 < KS) {
+                read_frags(stage, ks + 1, wf[(ks + 1) & 1], af[(ks + 1) & 1]);
+                multiply(wf[ks & 1], af[ks & 1], 0, TN);
+#pragma unroll
+                for (int r = 0; r < TN + TM; ++r) {      // the reads early, one after each MFMA
+                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                    __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+                }
+                __builtin_amdgcn_sched_barrier(0);
+            } else {
+                multiply(wf[ks & 1], af[ks & 1], 0, TN / 2);
+                __builtin_amdgcn_sched_barrier(0);
+                wait_for_loads<(W_LOADS + A_LOADS) * (NS - 2)>();
+                __syncthreads();
+                __builtin_amdgcn_sched_barrier(0);
+                issue(stage, min(it + NS, n_steps - 1));
+                read_frags(next_stage, 0, wf[0], af[0]);       // past the last step: a stage of repeats
+                multiply(wf[ks & 1], af[ks & 1], TN / 2, TN);
+#pragma unroll
+                for (int r = 0; r < TN + TM; ++r) {
+                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                    __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+                }
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        }
+        stage = next_stage;
+    }
+    wait_for_loads<0>();
+#pragma unroll
+    for (int i = 0; i < TN; ++i) {
+        const int n = n0 + wn + 32 * i + l32;
+#pragma unroll
+        for (int j = 0; j < TM; ++j) {
+#pragma unroll
+            for (int e = 0; e < 16; ++e) {
+                const int m = m0 + wm + 32 * j + 8 * (e / 4) + 4 * kq + e % 4;
+                const float v = acc[i][j][e];
+                if (EPI == 2) {
+                    const float up = __shfl_xor(v, 1, WAVE);
+                    if (m < M && (l32 & 1) == 0 && n + 1 < N) C[(int64_t)m * ldc + n / 2] = from_f32<TC>(silu_mul(v, up));
+                } else if (m < M && n < N) {
+                    TC* p = C + (int64_t)m * ldc + n;
+                    *p = from_f32<TC>(EPI == 1 ? to_f32<TC>(*p) + v : v);
+                }
+            }
+        }
+    }
+}
+
+template <int TN, int TM, int WN, int WM, int BK, int NS>
+static int launch_direct(const void* A, const void* W, void* C, int c_dt, int M, int N, int K, int64_t lda,
+                         int64_t ldw, int64_t ldc, int epilogue, hipStream_t stream) {
+    constexpr int BN = 32 * TN * WN, BM = 32 * TM * WM;
+    PICOLM_REQUIRE(K % BK == 0, "gemm_tiled: K = %d is no multiple of %d, which this variant needs", K, BK);
+    PICOLM_REQUIRE((int64_t)BN * ldw < (1ll << 30) && (int64_t)BM * lda < (1ll << 30),
+                   "gemm_tiled: row strides %lld / %lld overflow the tile's 32-bit offsets", (long long)lda, (long long)ldw);
+    const int tiles_m = ceil_div(M, BM), tiles_n = ceil_div(N, BN);
+    PICOLM_REQUIRE((int64_t)tiles_m * tiles_n < (1ll << 31), "gemm_tiled: too many tiles");
+    dim3 grid(tiles_m * tiles_n), block(64 * WN * WM);
+    const size_t lds = (size_t)NS * (BN + BM) * BK * sizeof(bf16_t);
+    static_assert((size_t)NS * (BN + BM) * BK * 2 <= 160 * 1024, "stages exceed the LDS");
+    const bf16_t* a = (const bf16_t*)A;
+    const bf16_t* w = (const bf16_t*)W;
+#define TD_LAUNCH(EPI, TC)                                                                                 \
+    {                                                                                                      \
+        static size_t raised = 48 * 1024;                                                                  \
+        if (lds > raised) {                                                                                \
+            hipError_t e = hipFuncSetAttribute((const void*)gemm_direct_kernel<TN, TM, WN, WM, BK, NS, EPI, TC>, \
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);      \
+            PICOLM_REQUIRE(e == hipSuccess, "gemm_tiled: cannot raise the LDS limit: %s",                  \
+                           hipGetErrorString(e));                                                          \
+            raised = lds;                                                                                  \
+        }                                                                                                  \
+        gemm_direct_kernel<TN, TM, WN, WM, BK, NS, EPI, TC><<<grid, block, lds, stream>>>(a, w, (TC*)C, M, N, K,  \
+                                                                                  lda, ldw, ldc, tiles_m, tiles_n); \
+    }
+    if (epilogue == 0 && c_dt == PICOLM_F32) TD_LAUNCH(0, float)
+    else if (epilogue == 0 && c_dt == PICOLM_BF16) TD_LAUNCH(0, bf16_t)
+    else if (epilogue == 1 && c_dt == PICOLM_F32) TD_LAUNCH(1, float)
+    else if (epilogue == 2 && c_dt == PICOLM_BF16) TD_LAUNCH(2, bf16_t)
+    else if (epilogue == 2 && c_dt == PICOLM_F32) TD_LAUNCH(2, float)
+    else PICOLM_REQUIRE(false, "gemm_tiled: unsupported epilogue %d with output dtype %d", epilogue, c_dt);
+#undef TD_LAUNCH
+    PICOLM_LAUNCH_CHECK("gemm_tiled");
+    return 0;
+}
+
+// variant 0 picks by shape.  Tiles loaded straight into LDS (K a multiple of 64):
+//   9: 256x256, 8 waves, two stages of 64 columns;  10: 256(n)x128(m), 8 waves, three stages;
+//   11: 128x128, 4 waves, four stages.
+// Tiles staged through registers (any K that is a multiple of 8):
+//   1: 128x128 (4 waves), 4: 256x256 (8 waves);
+//   7, 8: 64 rows of activations against 128 or 64 weight rows, for decode batches too wide for
+//   the skinny kernel.
 extern "C" int picolm_gemm_tiled(const void* A, const void* W, void* C, int c_dt, int M, int N, int K,
                                  int64_t lda, int64_t ldw, int64_t ldc, int epilogue, int variant,
                                  hipStream_t stream) {
     if (check_mfma_operands("gemm_tiled", A, W, M, N, K, lda, ldw, ldc, epilogue, c_dt)) return -1;
     if (M == 0) return 0;
     if (variant == 0) {
+        // Every variant moves about the same bytes a second from L2 into LDS, so the largest
+        // tile wins once its workgroups fill most of the 256 CUs.
         const int64_t t256 = (int64_t)ceil_div(M, 256) * ceil_div(N, 256);
-        variant = t256 >= 512 ? 4 : 1;      // the 256x256 tile pays once there are two rounds of it
+        const int64_t t128m = (int64_t)ceil_div(M, 128) * ceil_div(N, 256);
+        if (K % 64 == 0) variant = t256 >= 192 ? 9 : t128m >= 192 ? 10 : 11;
+        else variant = t256 >= 512 ? 4 : 1;
     }
     switch (variant) {
         case 1: return launch_tiled<2, 2, 2, 2, 2>(A, W, C, c_dt, M, N, K, lda, ldw, ldc, epilogue, stream);
-        case 2: return launch_tiled<4, 2, 2, 2, 2>(A, W, C, c_dt, M, N, K, lda, ldw, ldc, epilogue, stream);
-        case 3: return launch_tiled<4, 4, 2, 2, 1>(A, W, C, c_dt, M, N, K, lda, ldw, ldc, epilogue, stream);
         case 4: return launch_tiled<2, 4, 4, 2, 1>(A, W, C, c_dt, M, N, K, lda, ldw, ldc, epilogue, stream);
-        case 5: return launch_tiled<2, 2, 2, 1, 2>(A, W, C, c_dt, M, N, K, lda, ldw, ldc, epilogue, stream);
-        case 6: return launch_tiled<2, 1, 2, 2, 2>(A, W, C, c_dt, M, N, K, lda, ldw, ldc, epilogue, stream);
         case 7: return launch_tiled<1, 2, 4, 1, 2>(A, W, C, c_dt, M, N, K, lda, ldw, ldc, epilogue, stream);
         case 8: return launch_tiled<1, 2, 2, 1, 2>(A, W, C, c_dt, M, N, K, lda, ldw, ldc, epilogue, stream);
+        case 9: return launch_direct<2, 4, 4, 2, 64, 2>(A, W, C, c_dt, M, N, K, lda, ldw, ldc, epilogue, stream);
+        case 10: return launch_direct<2, 2, 4, 2, 64, 3>(A, W, C, c_dt, M, N, K, lda, ldw, ldc, epilogue, stream);
+        case 11: return launch_direct<2, 2, 2, 2, 64, 4>(A, W, C, c_dt, M, N, K, lda, ldw, ldc, epilogue, stream);
     }
     PICOLM_REQUIRE(false, "gemm_tiled: unknown variant %d", variant);
 }

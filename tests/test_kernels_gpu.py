@@ -127,11 +127,22 @@ def test_gemm_tiled(M, N, Kd):
         run_gemm(K().gemm_tiled, M, N, Kd, epi, torch.bfloat16, torch.bfloat16, cdt)
 
 
-@pytest.mark.parametrize("variant", [1, 2, 3, 4, 5, 6, 7, 8])
+@pytest.mark.parametrize("variant", [1, 4, 7, 8])
 def test_gemm_tiled_block_tiles(variant):
     for M, N, Kd in ((300, 530, 1032), (70, 260, 72), (513, 100, 200), (9, 700, 136), (64, 130, 64)):
         for epi, cdt in ((0, torch.float32), (2, torch.bfloat16), (1, torch.float32)):
             run_gemm(K().gemm_tiled, M, N, Kd, epi, torch.bfloat16, torch.bfloat16, cdt, variant=variant)
+
+
+@pytest.mark.parametrize("variant", [9, 10, 11])
+def test_gemm_tiled_direct_to_lds(variant):
+    """The variants whose tiles go from global memory straight into LDS: K in whole steps of 64,
+    fewer steps than stages, many steps (every stage is reused), ragged M and N."""
+    for M, N, Kd in ((300, 530, 1024), (70, 260, 64), (513, 100, 192), (9, 700, 128), (257, 258, 2048)):
+        for epi, cdt in ((0, torch.float32), (2, torch.bfloat16), (1, torch.float32), (0, torch.bfloat16)):
+            run_gemm(K().gemm_tiled, M, N, Kd, epi, torch.bfloat16, torch.bfloat16, cdt, variant=variant)
+    with pytest.raises(Exception, match="multiple"):
+        run_gemm(K().gemm_tiled, 70, 64, 72, 0, torch.bfloat16, torch.bfloat16, torch.float32, variant=variant)
 
 
 def test_gemm_refuses_what_it_cannot_do():
