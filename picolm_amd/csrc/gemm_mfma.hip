@@ -695,10 +695,28 @@ extern "C" int picolm_gemm_tiled(const void* A, const void* W, void* C, int c_dt
     if (variant == 0) {
         // Every variant moves about the same bytes a second from L2 into LDS, so the largest
         // tile wins once its workgroups fill most of the 256 CUs.
-        const int64_t t256 = (int64_t)ceil_div(M, 256) * ceil_div(N, 256);
-        const int64_t t128m = (int64_t)ceil_div(M, 128) * ceil_div(N, 256);
-        if (K % 64 == 0) variant = t256 >= 192 ? 9 : t128m >= 192 ? 10 : 11;
-        else variant = t256 >= 512 ? 4 : 1;
+        const int tiles_m = ceil_div(M, 256), tiles_n = ceil_div(N, 256);
+        const int64_t t256 = (int64_t)tiles_m * tiles_n;
+        const int64_t t128m = (int64_t)ceil_div(M, 128) * tiles_n;
+        if (K % 64 == 0) {
+            // A last round that fills half of the CUs or less costs nearly a whole round: those
+            // columns of tiles go to the 256x128 tile instead, which gives them twice the workgroups.
+            const int64_t whole = t256 / 256 * 256, left = t256 - whole;
+            const int n_first = (int)(whole / tiles_m);
+            const int64_t rest = (int64_t)(tiles_n - n_first) * ceil_div(M, 128);
+            if (whole > 0 && left > 0 && left <= 160 && n_first > 0 && rest <= 288) {
+                const int N1 = n_first * 256;
+                const size_t c_item = c_dt == PICOLM_F32 ? 4 : 2;
+                const int rc = picolm_gemm_tiled(A, W, C, c_dt, M, N1, K, lda, ldw, ldc, epilogue, 9, stream);
+                if (rc) return rc;
+                return picolm_gemm_tiled(A, (const bf16_t*)W + (int64_t)N1 * ldw,
+                                         (char*)C + c_item * (epilogue == 2 ? N1 / 2 : N1), c_dt, M, N - N1, K, lda,
+                                         ldw, ldc, epilogue, 10, stream);
+            }
+            variant = t256 >= 192 ? 9 : t128m >= 192 ? 10 : 11;
+        } else {
+            variant = t256 >= 512 ? 4 : 1;
+        }
     }
     switch (variant) {
         case 1: return launch_tiled<2, 2, 2, 2, 2>(A, W, C, c_dt, M, N, K, lda, ldw, ldc, epilogue, stream);

@@ -127,6 +127,14 @@ def test_gemm_tiled(M, N, Kd):
         run_gemm(K().gemm_tiled, M, N, Kd, epi, torch.bfloat16, torch.bfloat16, cdt)
 
 
+def test_gemm_tiled_splits_a_partial_last_round():
+    """300 tiles of 256x256 on 256 CUs: the columns past the first 256 tiles take the half-height
+    tile in a launch of their own; the seam must not show in any epilogue."""
+    for epi, cdt in ((0, torch.float32), (2, torch.bfloat16), (1, torch.float32)):
+        run_gemm(K().gemm_tiled, 512, 150 * 256 - 10, 64, epi, torch.bfloat16, torch.bfloat16, cdt)
+        run_gemm(K().gemm_tiled, 300, 150 * 256 - 10, 128, epi, torch.bfloat16, torch.bfloat16, cdt)
+
+
 @pytest.mark.parametrize("variant", [1, 4, 7, 8])
 def test_gemm_tiled_block_tiles(variant):
     for M, N, Kd in ((300, 530, 1032), (70, 260, 72), (513, 100, 200), (9, 700, 136), (64, 130, 64)):
