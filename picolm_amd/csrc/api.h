@@ -49,14 +49,15 @@ int picolm_attn_prefill_generic(const void* q, const void* k_pages, const void* 
                                 const int32_t* seq_nnew, const int32_t* cu_seqlens,
                                 const int32_t* page_table, int max_pages, int ring_pages, int H,
                                 int G, int d, int window, float scale, hipStream_t stream);
-// Decode: workgroup x of the launch is entry x of the step's work list (chunk_seq, chunk_idx):
-// pages_per_chunk pages of one sequence, or nothing where chunk_seq is -1.  A sequence has at
-// most max_splits chunks; where it has several, their partial results
-// (partial: [n_seq][H][max_splits][d+2] floats) are combined by a merge kernel that follows.
+// Decode (row i of q and out is sequence i): workgroup x of the launch takes entry x of the
+// step's work list, eight ints: {sequence or -1 for nothing, which chunk of the sequence, position
+// of the new token, cache slot, physical pages of the chunk's first four pages}.  A chunk is
+// pages_per_chunk pages; a sequence has at most max_splits chunks, and where it has several their
+// partial results (partial: [n_seq][H][max_splits][d+2] floats) are combined by a merge kernel
+// that follows.
 int picolm_attn_decode_generic(const void* q, const void* k_pages, const void* v_pages, void* out,
-                               float* partial, int dt, int n_seq, const int32_t* chunk_seq,
-                               const int32_t* chunk_idx, int n_chunks, int pages_per_chunk, int max_splits,
-                               const int32_t* seq_slot, const int32_t* seq_pos0, const int32_t* cu_seqlens,
+                               float* partial, int dt, int n_seq, const int32_t* chunk_list, int n_chunks,
+                               int pages_per_chunk, int max_splits, const int32_t* seq_pos0,
                                const int32_t* page_table, int max_pages, int ring_pages, int H, int G, int d,
                                int window, float scale, hipStream_t stream);
 
@@ -70,11 +71,9 @@ int picolm_attn_prefill_mfma(const void* q, const void* k_pages, const void* v_p
                              const int32_t* cu_seqlens, const int32_t* page_table, int max_pages,
                              int ring_pages, int H, int G, int d, int window, float scale, hipStream_t stream);
 int picolm_attn_decode_mfma(const void* q, const void* k_pages, const void* v_pages, void* out, float* partial,
-                            int n_seq, const int32_t* chunk_seq, const int32_t* chunk_idx, int n_chunks,
-                            int pages_per_chunk, int max_splits, const int32_t* seq_slot,
-                            const int32_t* seq_pos0, const int32_t* cu_seqlens, const int32_t* page_table,
-                            int max_pages, int ring_pages, int H, int G, int d, int window, float scale,
-                            hipStream_t stream);
+                            int n_seq, const int32_t* chunk_list, int n_chunks, int pages_per_chunk,
+                            int max_splits, const int32_t* seq_pos0, const int32_t* page_table, int max_pages,
+                            int ring_pages, int H, int G, int d, int window, float scale, hipStream_t stream);
 
 int picolm_argmax_scratch_floats(int n_rows, int V);
 int picolm_argmax(const float* logits, int32_t* out, int n_rows, int V, int64_t ld, float* scratch,

@@ -21,28 +21,38 @@ struct AttnArgs {
     int H, G, d, window;
     float scale;
     int decode;     // 0 prefill tiles, 1 decode groups
-    // decode: workgroup x is chunk x of the step's work list: pages_per_chunk pages of one sequence
-    const int32_t* chunk_seq;   // sequence of each chunk, or -1 for an unused entry
-    const int32_t* chunk_idx;   // which chunk of its sequence
+    // decode: workgroup x takes entry x of the step's work list, eight ints each:
+    // {sequence or -1, which chunk of the sequence, position of the new token, cache slot,
+    //  physical pages of the chunk's first four pages (-1 past its end)}
+    const int32_t* chunk_list;
     int pages_per_chunk;
     int max_splits;             // chunks a sequence can have: stride of `partial`
 };
 
 // What a decode workgroup has to do.  A sequence whose visible pages fit one chunk is finished by
 // its workgroup; otherwise every chunk leaves (max, sum, acc) in `partial` and the merge kernel
-// combines them.  The host's work list is built from the same arithmetic.
+// combines them.  The host's work list is built from the same arithmetic.  In a decode step row
+// i of q and of the output belongs to sequence i.
 struct DecodeWork {
-    int seq, split, page_lo, page_hi, n_chunks;
+    int seq, split, qpos, slot, page_lo, page_hi, n_chunks;
+    int phys[4];
 };
-__device__ __forceinline__ int decode_first_page(const AttnArgs& a, int qpos) {
-    return (a.window > 0 ? max(0, qpos - a.window + 1) : 0) / 64;
+__device__ __forceinline__ int decode_first_page(int window, int qpos) {
+    return (window > 0 ? max(0, qpos - window + 1) : 0) / 64;
 }
 __device__ __forceinline__ bool decode_work(const AttnArgs& a, DecodeWork& w) {
-    w.seq = a.chunk_seq[blockIdx.x];
+    const int4* e = (const int4*)a.chunk_list + 2 * (size_t)blockIdx.x;
+    const int4 e0 = e[0], e1 = e[1];
+    w.seq = e0.x;
     if (w.seq < 0) return false;
-    w.split = a.chunk_idx[blockIdx.x];
-    const int qpos = a.seq_pos0[w.seq];
-    const int first = decode_first_page(a, qpos), end = qpos / 64 + 1;
+    w.split = e0.y;
+    w.qpos = e0.z;
+    w.slot = e0.w;
+    w.phys[0] = e1.x;
+    w.phys[1] = e1.y;
+    w.phys[2] = e1.z;
+    w.phys[3] = e1.w;
+    const int first = decode_first_page(a.window, w.qpos), end = w.qpos / 64 + 1;
     w.n_chunks = (end - first + a.pages_per_chunk - 1) / a.pages_per_chunk;
     w.page_lo = first + w.split * a.pages_per_chunk;
     w.page_hi = min(end, w.page_lo + a.pages_per_chunk);

@@ -34,7 +34,7 @@ __global__ __launch_bounds__(AT_THREADS) void attn_tile_kernel(AttnArgs a) {
     const int tid = threadIdx.x, wave = tid / WAVE, lane = tid % WAVE;
     const int R = a.H / a.G;
     int seq, g, split = 0, n_rows;
-    DecodeWork work = {0, 0, 0, 0, 1};
+    DecodeWork work = {};
     if (a.decode) {
         if (!decode_work(a, work)) return;
         seq = work.seq;
@@ -44,9 +44,9 @@ __global__ __launch_bounds__(AT_THREADS) void attn_tile_kernel(AttnArgs a) {
         const int chunk = blockIdx.y % chunks;
         n_rows = min(AT_ROWS, R - chunk * AT_ROWS);
         if (tid < AT_ROWS) {
-            row_tok[tid] = a.cu_seqlens[seq];
+            row_tok[tid] = seq;
             row_head[tid] = g * R + chunk * AT_ROWS + tid;
-            row_qpos[tid] = a.seq_pos0[seq];
+            row_qpos[tid] = work.qpos;
         }
     } else {
         seq = a.tile_seq[blockIdx.x];
@@ -90,7 +90,7 @@ __global__ __launch_bounds__(AT_THREADS) void attn_tile_kernel(AttnArgs a) {
 #pragma unroll
     for (int j = 0; j < AT_MAX_D / 16; ++j) acc[j] = 0.f;
 
-    const int slot = a.seq_slot[seq];
+    const int slot = a.decode ? work.slot : a.seq_slot[seq];
     const int32_t* pt = a.page_table + (size_t)slot * a.max_pages;
     const size_t page_elems = (size_t)a.G * PAGE_TOKENS * d;
 
@@ -197,7 +197,7 @@ __global__ __launch_bounds__(MERGE_WAVES * WAVE) void attn_merge_kernel(AttnArgs
     const int H = a.H, d = a.d;
     const int seq = unit / H, head = unit % H;
     const int qpos = a.seq_pos0[seq];
-    const int n_splits = (qpos / 64 + 1 - decode_first_page(a, qpos) + a.pages_per_chunk - 1) / a.pages_per_chunk;
+    const int n_splits = (qpos / 64 + 1 - decode_first_page(a.window, qpos) + a.pages_per_chunk - 1) / a.pages_per_chunk;
     if (n_splits <= 1) return;                         // its one workgroup wrote the result itself
     const int stride = d + 2;
     const float* p = a.partial + (size_t)unit * a.max_splits * stride;
@@ -219,7 +219,7 @@ __global__ __launch_bounds__(MERGE_WAVES * WAVE) void attn_merge_kernel(AttnArgs
     for (int i = lane; i < n_splits; i += WAVE) l += expf(p[(size_t)i * stride] - M) * p[(size_t)i * stride + 1];
     const float L = wave_sum(l);
     const float inv = L > 0.f ? 1.0f / L : 0.f;
-    T* o = (T*)a.out + (size_t)a.cu_seqlens[seq] * H * d + (size_t)head * d;
+    T* o = (T*)a.out + (size_t)seq * H * d + (size_t)head * d;
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
         const int c = lane + j * WAVE;
@@ -253,9 +253,10 @@ static int launch_attn(const AttnArgs& a, dim3 grid, hipStream_t stream) {
     return 0;
 }
 
-int check_decode_chunks(const char* who, const float* partial, const int32_t* chunk_seq, const int32_t* chunk_idx,
-                        int n_chunks, int pages_per_chunk, int max_splits) {
-    PICOLM_REQUIRE(chunk_seq && chunk_idx && n_chunks >= 0, "%s: needs the step's work list", who);
+int check_decode_chunks(const char* who, const float* partial, const int32_t* chunk_list, int n_chunks,
+                        int pages_per_chunk, int max_splits) {
+    PICOLM_REQUIRE(chunk_list && n_chunks >= 0, "%s: needs the step's work list", who);
+    PICOLM_REQUIRE(((uintptr_t)chunk_list & 15) == 0, "%s: the work list must be 16-byte aligned", who);
     PICOLM_REQUIRE(pages_per_chunk >= 1 && max_splits >= 1, "%s: bad chunking (%d pages a chunk, %d chunks a sequence)", who,
                    pages_per_chunk, max_splits);
     PICOLM_REQUIRE(max_splits == 1 || partial != nullptr, "%s: several chunks a sequence need a partial buffer", who);
@@ -292,7 +293,7 @@ extern "C" int picolm_attn_prefill_generic(const void* q, const void* k_pages, c
     PICOLM_REQUIRE(H <= 65535, "attn_prefill: %d heads exceed the grid", H);
     if (n_tiles <= 0) return 0;
     AttnArgs a = {q, k_pages, v_pages, out, nullptr, tile_seq, tile_q0, seq_slot, seq_pos0, seq_nnew,
-                  cu_seqlens, page_table, max_pages, ring_pages, H, G, d, window, scale, 0, nullptr, nullptr, 0, 1};
+                  cu_seqlens, page_table, max_pages, ring_pages, H, G, d, window, scale, 0, nullptr, 0, 1};
     dim3 grid(n_tiles, H);
     if (dt == PICOLM_F32) return launch_attn<float>(a, grid, stream);
     if (dt == PICOLM_BF16) return launch_attn<bf16_t>(a, grid, stream);
@@ -303,20 +304,18 @@ extern "C" int picolm_attn_prefill_tile_rows(void) { return AT_ROWS; }
 
 extern "C" int picolm_attn_decode_generic(const void* q, const void* k_pages, const void* v_pages,
                                           void* out, float* partial, int dt, int n_seq,
-                                          const int32_t* chunk_seq, const int32_t* chunk_idx, int n_chunks,
-                                          int pages_per_chunk, int max_splits, const int32_t* seq_slot,
-                                          const int32_t* seq_pos0, const int32_t* cu_seqlens,
-                                          const int32_t* page_table, int max_pages, int ring_pages, int H,
-                                          int G, int d, int window, float scale, hipStream_t stream) {
+                                          const int32_t* chunk_list, int n_chunks, int pages_per_chunk,
+                                          int max_splits, const int32_t* seq_pos0, const int32_t* page_table,
+                                          int max_pages, int ring_pages, int H, int G, int d, int window,
+                                          float scale, hipStream_t stream) {
     if (check_attn_sizes("attn_decode", H, G, d, max_pages, ring_pages)) return -1;
-    if (check_decode_chunks("attn_decode", partial, chunk_seq, chunk_idx, n_chunks, pages_per_chunk, max_splits)) return -1;
+    if (check_decode_chunks("attn_decode", partial, chunk_list, n_chunks, pages_per_chunk, max_splits)) return -1;
     PICOLM_REQUIRE(dt == PICOLM_F32 || dt == PICOLM_BF16, "attn_decode: unknown dtype %d", dt);
     if (n_seq <= 0 || n_chunks <= 0) return 0;
     const int chunks = ceil_div(H / G, AT_ROWS);
     PICOLM_REQUIRE(G * chunks <= 65535, "attn_decode: %d groups exceed the grid", G * chunks);
-    AttnArgs a = {q, k_pages, v_pages, out, partial, nullptr, nullptr, seq_slot, seq_pos0, nullptr, cu_seqlens,
-                  page_table, max_pages, ring_pages, H, G, d, window, scale, 1, chunk_seq, chunk_idx,
-                  pages_per_chunk, max_splits};
+    AttnArgs a = {q, k_pages, v_pages, out, partial, nullptr, nullptr, nullptr, seq_pos0, nullptr, nullptr,
+                  page_table, max_pages, ring_pages, H, G, d, window, scale, 1, chunk_list, pages_per_chunk, max_splits};
     dim3 grid(n_chunks, G * chunks);
     const int rc = dt == PICOLM_F32 ? launch_attn<float>(a, grid, stream) : launch_attn<bf16_t>(a, grid, stream);
     if (rc) return rc;

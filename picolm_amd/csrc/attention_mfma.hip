@@ -281,9 +281,15 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void a
 }
 
 // =============================================================================================
-template <int D>
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void attn_decode_mfma_kernel(AttnArgs a) {
-    extern __shared__ float mrg[];       // [4 waves][Rc][D + 2]
+// One new token per sequence.  A workgroup takes a chunk of pages of one sequence and one KV
+// group; its waves take the chunk's tiles of 32 keys in turn, each asking for a whole tile (keys
+// and values) before it waits for any of it.  What a workgroup needs to find its pages comes in
+// one 32-byte entry of the work list, so that only two trips to memory lie between the launch
+// and the first MFMA.  Eight waves give a short step for a few sequences; with many sequences
+// four waves, two workgroups a CU, move more bytes.
+template <int D, int DEC_WAVES>
+__global__ __launch_bounds__(DEC_WAVES * 64) __attribute__((amdgpu_waves_per_eu(2))) void attn_decode_mfma_kernel(AttnArgs a) {
+    extern __shared__ float mrg[];       // [DEC_WAVES][Rc][D + 2]
     const int tid = threadIdx.x, wave = tid / WAVE, lane = tid % WAVE;
     const int l32 = lane % 32, h = lane / 32;
     const int R = a.H / a.G;
@@ -295,8 +301,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void a
     const int Rc = min(32, R - chunk * 32);
     const bool q_ok = l32 < Rc;
     const int head = g * R + chunk * 32 + (q_ok ? l32 : 0);
-    const size_t tok = (size_t)a.cu_seqlens[seq];
-    const int qpos = a.seq_pos0[seq];
+    const size_t tok = (size_t)seq;
+    const int qpos = work.qpos;
 
     const int page_lo = work.page_lo, page_hi = work.page_hi;
     // k-step s of a lane covers d = 16s + 8h .. +8: the two halves of a wave read 32 adjacent bytes of a key
@@ -313,42 +319,47 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void a
         for (int e = 0; e < 16; ++e) O[dt][e] = 0.f;
     float m_run = NEG_BIG, l_run = 0.f;
     const float scale2 = a.scale * LOG2E;
-    const int32_t* pt = a.page_table + (size_t)a.seq_slot[seq] * a.max_pages;
+    const int32_t* pt = a.page_table + (size_t)work.slot * a.max_pages;
     const size_t page_elems = (size_t)a.G * PAGE_TOKENS * D;
 
-    for (int page = page_lo + wave; page < page_hi; page += 4) {
-        const size_t base = (size_t)pt[page % a.ring_pages] * page_elems + (size_t)g * PAGE_TOKENS * D;
+    // tile tt of the chunk: keys 32*tt .. 32*tt+31 counted from the chunk's first page
+    const int n_tiles = 2 * (page_hi - page_lo);
+    auto page_of_tile = [&](int tt) {                       // the first eight tiles' pages came with the entry
+        if (tt >= 8) return pt[(page_lo + tt / 2) % a.ring_pages];
+        return tt < 2 ? work.phys[0] : tt < 4 ? work.phys[1] : tt < 6 ? work.phys[2] : work.phys[3];
+    };
+    int phys = page_of_tile(wave);
+    for (int tt = wave; tt < n_tiles; tt += DEC_WAVES) {
+        const int page = page_lo + tt / 2, t = tt & 1;
+        const int key0 = page * PAGE_TOKENS + 32 * t;
+        if (key0 > qpos) break;                              // nothing of this tile, or of a later one, is visible
+        const int next_phys = tt + DEC_WAVES < n_tiles ? page_of_tile(tt + DEC_WAVES) : 0;   // asked for before this tile's data
+        const size_t base = (size_t)phys * page_elems + (size_t)g * PAGE_TOKENS * D;
         const bf16_t* kp = (const bf16_t*)a.k_pages + base + 8 * h;
         const bf16_t* vp = (const bf16_t*)a.v_pages + base + (size_t)l32 * PAGE_TOKENS + 8 * h;
-        const int key0 = page * PAGE_TOKENS;
-        const int n_keys = qpos - key0 + 1;          // >= 1; keys past it are not this sequence's
-        // a page is two tiles of 32 keys; all operands of a tile are requested before the first
-        // MFMA waits for one
+        const int n_keys = qpos - key0 + 1;                  // >= 1; keys past it are not this sequence's
+        bf16x8 Kf[D / 16], Vf[D / 32][2];
 #pragma unroll
-        for (int t = 0; t < 2; ++t) {
-            if (key0 + 32 * t > qpos) break;                 // nothing of this tile is visible
-            bf16x8 Kf[D / 16], Vf[D / 32][2];
+        for (int s = 0; s < D / 16; ++s) Kf[s] = ldg8(kp + (size_t)(32 * t + key_of_row(l32)) * D + 16 * s);
 #pragma unroll
-            for (int s = 0; s < D / 16; ++s) Kf[s] = ldg8(kp + (size_t)(32 * t + key_of_row(l32)) * D + 16 * s);
+        for (int dt = 0; dt < D / 32; ++dt)
+#pragma unroll
+            for (int ks = 0; ks < 2; ++ks) Vf[dt][ks] = ldg8(vp + (size_t)(32 * dt) * PAGE_TOKENS + 32 * t + 16 * ks);
+        if (n_keys < 32) {                                   // keys past the end may hold anything
 #pragma unroll
             for (int dt = 0; dt < D / 32; ++dt)
 #pragma unroll
-                for (int ks = 0; ks < 2; ++ks) Vf[dt][ks] = ldg8(vp + (size_t)(32 * dt) * PAGE_TOKENS + 32 * t + 16 * ks);
-            if (n_keys < 32 * (t + 1)) {                     // keys past the end may hold anything
+                for (int ks = 0; ks < 2; ++ks) {
+                    const int k = 16 * ks + 8 * h;
 #pragma unroll
-                for (int dt = 0; dt < D / 32; ++dt)
-#pragma unroll
-                    for (int ks = 0; ks < 2; ++ks) {
-                        const int k = 32 * t + 16 * ks + 8 * h;
-#pragma unroll
-                        for (int e = 0; e < 8; ++e)
-                            if (k + e >= n_keys) Vf[dt][ks][e] = (__bf16)0.0f;
-                    }
-            }
-            attend_tile<D>(Qf, Kf, Vf, O, m_run, l_run, key0 + 32 * t, qpos, q_ok, a.window, scale2, h);
+                    for (int e = 0; e < 8; ++e)
+                        if (k + e >= n_keys) Vf[dt][ks][e] = (__bf16)0.0f;
+                }
         }
+        attend_tile<D>(Qf, Kf, Vf, O, m_run, l_run, key0, qpos, q_ok, a.window, scale2, h);
+        phys = next_phys;
     }
-    // merge the 4 waves
+    // merge the waves
     float* mine = mrg + (size_t)wave * Rc * (D + 2);
     if (q_ok) {
         float* row = mine + (size_t)l32 * (D + 2);
@@ -362,14 +373,14 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void a
             for (int e = 0; e < 16; ++e) row[2 + 32 * dt + 8 * (e / 4) + 4 * h + e % 4] = O[dt][e];
     }
     __syncthreads();
-    for (int idx = tid; idx < Rc * D; idx += 256) {
+    for (int idx = tid; idx < Rc * D; idx += DEC_WAVES * 64) {
         const int q = idx / D, dcol = idx % D;
         float M = NEG_BIG;
 #pragma unroll
-        for (int w = 0; w < 4; ++w) M = fmaxf(M, mrg[((size_t)w * Rc + q) * (D + 2)]);
+        for (int w = 0; w < DEC_WAVES; ++w) M = fmaxf(M, mrg[((size_t)w * Rc + q) * (D + 2)]);
         float L = 0.f, acc = 0.f;
 #pragma unroll
-        for (int w = 0; w < 4; ++w) {
+        for (int w = 0; w < DEC_WAVES; ++w) {
             const float* row = mrg + ((size_t)w * Rc + q) * (D + 2);
             const float f = exp2f(row[0] - M);
             L += f * row[1];
@@ -422,7 +433,7 @@ extern "C" int picolm_attn_prefill_mfma(const void* q, const void* k_pages, cons
     const int head_chunks = ceil_div(H / G, HB);
     PICOLM_REQUIRE(G * head_chunks <= 65535, "attn_prefill_mfma: %d head groups exceed the grid", G * head_chunks);
     AttnArgs a = {q, k_pages, v_pages, out, nullptr, tile_seq, tile_q0, seq_slot, seq_pos0, seq_nnew,
-                  cu_seqlens, page_table, max_pages, ring_pages, H, G, d, window, scale, 0, nullptr, nullptr, 0, 1};
+                  cu_seqlens, page_table, max_pages, ring_pages, H, G, d, window, scale, 0, nullptr, 0, 1};
     dim3 grid(n_tiles, G * head_chunks), block(256);
     const size_t lds = 2 * 2 * (size_t)PAGE_TOKENS * d * sizeof(bf16_t);       // two stages of K and V^T
     if (d == 32) attn_prefill_mfma_kernel<32><<<grid, block, lds, stream>>>(a, HB, tile_tokens);
@@ -441,39 +452,44 @@ extern "C" int picolm_attn_prefill_mfma(const void* q, const void* k_pages, cons
     return 0;
 }
 
-int check_decode_chunks(const char* who, const float* partial, const int32_t* chunk_seq, const int32_t* chunk_idx,
-                        int n_chunks, int pages_per_chunk, int max_splits);
+int check_decode_chunks(const char* who, const float* partial, const int32_t* chunk_list, int n_chunks,
+                        int pages_per_chunk, int max_splits);
 int picolm_attn_merge_launch(const AttnArgs& a, int dt, int n_seq, hipStream_t stream);
 
 extern "C" int picolm_attn_decode_mfma(const void* q, const void* k_pages, const void* v_pages, void* out,
-                                       float* partial, int n_seq, const int32_t* chunk_seq,
-                                       const int32_t* chunk_idx, int n_chunks, int pages_per_chunk,
-                                       int max_splits, const int32_t* seq_slot, const int32_t* seq_pos0,
-                                       const int32_t* cu_seqlens, const int32_t* page_table, int max_pages,
-                                       int ring_pages, int H, int G, int d, int window, float scale,
-                                       hipStream_t stream) {
+                                       float* partial, int n_seq, const int32_t* chunk_list, int n_chunks,
+                                       int pages_per_chunk, int max_splits, const int32_t* seq_pos0,
+                                       const int32_t* page_table, int max_pages, int ring_pages, int H, int G,
+                                       int d, int window, float scale, hipStream_t stream) {
     if (check_sizes("attn_decode_mfma", H, G, d, max_pages, ring_pages)) return -1;
-    if (check_decode_chunks("attn_decode_mfma", partial, chunk_seq, chunk_idx, n_chunks, pages_per_chunk, max_splits)) return -1;
+    if (check_decode_chunks("attn_decode_mfma", partial, chunk_list, n_chunks, pages_per_chunk, max_splits)) return -1;
     if (n_seq <= 0 || n_chunks <= 0) return 0;
     const int R = H / G, chunks = ceil_div(R, 32);
     PICOLM_REQUIRE(G * chunks <= 65535, "attn_decode_mfma: %d groups exceed the grid", G * chunks);
-    AttnArgs a = {q, k_pages, v_pages, out, partial, nullptr, nullptr, seq_slot, seq_pos0, nullptr, cu_seqlens,
-                  page_table, max_pages, ring_pages, H, G, d, window, scale, 1, chunk_seq, chunk_idx,
-                  pages_per_chunk, max_splits};
-    dim3 grid(n_chunks, G * chunks), block(256);
-    const size_t lds = sizeof(float) * 4 * (size_t)min(R, 32) * (d + 2);
-    if (d == 32) attn_decode_mfma_kernel<32><<<grid, block, lds, stream>>>(a);
-    else if (d == 64) attn_decode_mfma_kernel<64><<<grid, block, lds, stream>>>(a);
-    else {
-        static size_t raised = 48 * 1024;
-        if (lds > raised) {
-            hipError_t e = hipFuncSetAttribute((const void*)attn_decode_mfma_kernel<128>,
-                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-            PICOLM_REQUIRE(e == hipSuccess, "attn_decode_mfma: cannot raise the LDS limit: %s", hipGetErrorString(e));
-            raised = lds;
-        }
-        attn_decode_mfma_kernel<128><<<grid, block, lds, stream>>>(a);
+    AttnArgs a = {q, k_pages, v_pages, out, partial, nullptr, nullptr, nullptr, seq_pos0, nullptr, nullptr,
+                  page_table, max_pages, ring_pages, H, G, d, window, scale, 1, chunk_list, pages_per_chunk, max_splits};
+    const int waves = (int64_t)n_seq * G * chunks >= 256 ? 4 : 8;
+    dim3 grid(n_chunks, G * chunks), block(waves * 64);
+    const size_t lds = sizeof(float) * waves * (size_t)min(R, 32) * (d + 2);
+#define DEC_LAUNCH(D, W)                                                                                    \
+    {                                                                                                       \
+        static size_t raised = 48 * 1024;                                                                   \
+        if (lds > raised) {                                                                                 \
+            hipError_t e = hipFuncSetAttribute((const void*)attn_decode_mfma_kernel<D, W>,                  \
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);       \
+            PICOLM_REQUIRE(e == hipSuccess, "attn_decode_mfma: cannot raise the LDS limit: %s",             \
+                           hipGetErrorString(e));                                                           \
+            raised = lds;                                                                                   \
+        }                                                                                                   \
+        attn_decode_mfma_kernel<D, W><<<grid, block, lds, stream>>>(a);                                     \
     }
+    if (d == 32 && waves == 4) DEC_LAUNCH(32, 4)
+    else if (d == 32) DEC_LAUNCH(32, 8)
+    else if (d == 64 && waves == 4) DEC_LAUNCH(64, 4)
+    else if (d == 64) DEC_LAUNCH(64, 8)
+    else if (waves == 4) DEC_LAUNCH(128, 4)
+    else DEC_LAUNCH(128, 8)
+#undef DEC_LAUNCH
     PICOLM_LAUNCH_CHECK("attn_decode_mfma");
     return max_splits > 1 ? picolm_attn_merge_launch(a, PICOLM_BF16, n_seq, stream) : 0;
 }

@@ -20,7 +20,7 @@ class StepError(ValueError):
 
 
 class StepBatch:
-    def __init__(self, slots, pos0, new_tokens, want, vocab_size: int, device, target_blocks: int = 1024):
+    def __init__(self, slots, pos0, new_tokens, want, vocab_size: int, device, target_blocks: int = 512):
         """slots[i]: cache slot of sequence i; pos0[i]: tokens it holds; new_tokens[i]: its
         next tokens; want[i]: indices into new_tokens[i] whose logits are asked for."""
         self.n_seq = len(slots)
@@ -113,19 +113,18 @@ class StepBatch:
             yield _Chunk(self, seqs, lo, [min(chunk_tokens, self.n_new[i] - lo) for i in seqs],
                          [int(cu[i]) + lo for i in seqs])
 
-    def decode_chunks(self, blocks_per_chunk: int, window: int, max_pages: int):
-        """The decode attention's work list for this step: (chunk_seq, chunk_idx, n_chunks,
-        pages_per_chunk, max_splits), the first two on the device."""
-        key = (blocks_per_chunk, window)
+    def decode_chunks(self, blocks_per_chunk: int, window: int, group: int, table_host, ring_pages: int):
+        """The decode attention's work list for this step over one cache group's pages:
+        (entries on the device, number of entries, pages_per_chunk, most chunks of a sequence)."""
+        key = (blocks_per_chunk, window, group)
         if key not in self._chunks:
             ppc = decode_pages_per_chunk(self.pos0, blocks_per_chunk, self._target_blocks)
-            seq, idx, most = decode_chunk_list(self.pos0, window, ppc)
-            flat = torch.from_numpy(np.concatenate([seq, idx])).to(self._device)
-            self._chunks[key] = (flat[:len(seq)], flat[len(seq):], len(seq), ppc, most)
+            entries, most = decode_chunk_list(self.slots, self.pos0, window, ppc, table_host, ring_pages)
+            self._chunks[key] = (torch.from_numpy(entries).to(self._device), len(entries), ppc, most)
         return self._chunks[key]
 
 
-def decode_pages_per_chunk(pos0, blocks_per_chunk: int, target_blocks: int = 1024) -> int:
+def decode_pages_per_chunk(pos0, blocks_per_chunk: int, target_blocks: int = 512) -> int:
     """Pages that one workgroup of the decode attention takes: a power of two, at least one
     page for each of its four waves, and more when the step would otherwise have far more
     than `target_blocks` workgroups (a few for every CU)."""
@@ -134,16 +133,34 @@ def decode_pages_per_chunk(pos0, blocks_per_chunk: int, target_blocks: int = 102
     return max(4, 1 << (max(want, 1).bit_length() - 1))
 
 
-def decode_chunk_list(pos0, window: int, pages_per_chunk: int):
-    """(chunk_seq, chunk_idx, most chunks of one sequence): every sequence's visible pages
-    (those of its last `window` keys, or all) cut into runs of `pages_per_chunk`.  The
-    kernels derive each chunk's pages from the same arithmetic."""
+CHUNK_ENTRY_INTS = 8
+
+
+def decode_chunk_list(slots, pos0, window: int, pages_per_chunk: int, table_host, ring_pages: int):
+    """(entries [n][8] int32, most chunks of one sequence): every sequence's visible pages
+    (those of its last `window` keys, or all) cut into runs of `pages_per_chunk`.  An entry is
+    {sequence, which chunk, position of the new token, slot, physical pages of the chunk's first
+    four pages or -1}; the kernels derive each chunk's pages from the same arithmetic."""
     pos = np.asarray(pos0, dtype=np.int64)
+    slot = np.asarray(slots, dtype=np.int64)
     first = (np.maximum(0, pos - window + 1) if window > 0 else np.zeros_like(pos)) // PAGE_TOKENS
-    n = (pos // PAGE_TOKENS + 1 - first + pages_per_chunk - 1) // pages_per_chunk
-    seq = np.repeat(np.arange(len(pos), dtype=np.int32), n)
-    idx = (np.arange(int(n.sum())) - np.repeat(np.cumsum(n) - n, n)).astype(np.int32)
-    return seq, idx, int(n.max())
+    end = pos // PAGE_TOKENS + 1
+    n = (end - first + pages_per_chunk - 1) // pages_per_chunk
+    seq = np.repeat(np.arange(len(pos), dtype=np.int64), n)
+    idx = np.arange(int(n.sum())) - np.repeat(np.cumsum(n) - n, n)
+    entries = np.empty((len(seq), CHUNK_ENTRY_INTS), dtype=np.int32)
+    entries[:, 0] = seq
+    entries[:, 1] = idx
+    entries[:, 2] = pos[seq]
+    entries[:, 3] = slot[seq]
+    table = table_host.numpy() if hasattr(table_host, "numpy") else np.asarray(table_host)
+    page0 = first[seq] + idx * pages_per_chunk
+    for w in range(4):
+        page = page0 + w
+        inside = (page < end[seq]) & (w < pages_per_chunk)
+        phys = table[slot[seq], np.where(inside, page, 0) % ring_pages]
+        entries[:, 4 + w] = np.where(inside, phys, -1)
+    return entries, int(n.max())
 
 
 class _Chunk:
@@ -202,7 +219,7 @@ class DecodeBatch:
         for k, (o, s) in self._spans.items():
             setattr(self, k, self._dev[o:o + s])
         self.slots, self.pos0 = [], []
-        self._lists = {}        # window -> (host block, device block, max_splits)
+        self._lists = {}        # (window, group) -> (host block, device block, most chunks, page table, ring)
         self.frozen = False     # set once the launches are recorded: no further work list can join
 
     @staticmethod
@@ -217,31 +234,31 @@ class DecodeBatch:
         self._np["tok_pos"][:] = pos0
         self._np["tokens"][:] = tokens
         self._dev.copy_(self._host, non_blocking=False)
-        for window in self._lists:
-            self._fill_list(window)
+        for key in self._lists:
+            self._fill_list(key)
 
-    def _fill_list(self, window: int) -> None:
-        host, dev, most = self._lists[window]
-        seq, idx, n_most = decode_chunk_list(self.pos0, window, self.pages_per_chunk)
+    def _fill_list(self, key) -> None:
+        host, dev, most, table_host, ring_pages = self._lists[key]
+        entries, n_most = decode_chunk_list(self.slots, self.pos0, key[0], self.pages_per_chunk, table_host, ring_pages)
         if n_most > most:
             raise StepError(f"a sequence of {max(self.pos0) + 1} tokens has more pages than the cache was sized for")
-        cap = len(host) // 2
-        h = host.numpy()
-        h[:len(seq)] = seq
-        h[len(seq):cap] = -1            # workgroups of unused entries leave at once
-        h[cap:cap + len(idx)] = idx
+        h = host.numpy().reshape(-1, CHUNK_ENTRY_INTS)
+        h[:len(entries)] = entries
+        h[len(entries):, 0] = -1        # workgroups of unused entries leave at once
         dev.copy_(host, non_blocking=False)
 
-    def decode_chunks(self, blocks_per_chunk: int, window: int, max_pages: int):
+    def decode_chunks(self, blocks_per_chunk: int, window: int, group: int, table_host, ring_pages: int):
         """As StepBatch.decode_chunks, over a list of fixed capacity (every sequence at the
         cache's full length) that `fill` rewrites in place."""
-        if window not in self._lists:
+        key = (window, group)
+        if key not in self._lists:
             if self.frozen:
                 raise StepError("a recorded decode step cannot take another work list")
-            most = (max_pages + self.pages_per_chunk - 1) // self.pages_per_chunk
+            most = (table_host.shape[1] + self.pages_per_chunk - 1) // self.pages_per_chunk
             cap = self.n_seq * most
-            self._lists[window] = (self._host_block(2 * cap), torch.zeros(2 * cap, dtype=torch.int32, device=self._device), most)
-            self._fill_list(window)
-        host, dev, most = self._lists[window]
-        cap = len(host) // 2
-        return dev[:cap], dev[cap:], cap, self.pages_per_chunk, most
+            self._lists[key] = (self._host_block(cap * CHUNK_ENTRY_INTS),
+                                torch.zeros(cap * CHUNK_ENTRY_INTS, dtype=torch.int32, device=self._device), most,
+                                table_host, ring_pages)
+            self._fill_list(key)
+        host, dev, most, _, _ = self._lists[key]
+        return dev, len(host) // CHUNK_ENTRY_INTS, self.pages_per_chunk, most

@@ -221,8 +221,7 @@ def attn_prefill_generic(q, k_pages, v_pages, out, tile_seq, tile_q0, n_tiles, s
         page_table.shape[1], ring_pages, H, G, d, window, c_float(scale), _stream()))
 
 
-def _decode_check(q, partial, n_seq, chunk_seq, chunk_idx, n_chunks, pages_per_chunk, max_splits, seq_slot,
-                  seq_pos0, cu_seqlens, H, d) -> None:
+def _decode_check(q, partial, n_seq, chunk_list, n_chunks, pages_per_chunk, max_splits, seq_pos0, H, d) -> None:
     if max_splits > 1:
         _dev("attn.partial", partial, torch.float32)
         if partial.numel() < n_seq * H * max_splits * (d + 2):
@@ -231,23 +230,18 @@ def _decode_check(q, partial, n_seq, chunk_seq, chunk_idx, n_chunks, pages_per_c
         raise KernelError("attn_decode: fewer query rows than sequences")
     if pages_per_chunk < 1 or max_splits < 1:
         raise KernelError(f"attn_decode: {pages_per_chunk} pages a chunk, {max_splits} chunks a sequence")
-    _i32("attn.chunk_seq", chunk_seq, n_chunks)
-    _i32("attn.chunk_idx", chunk_idx, n_chunks)
-    for nm, t in (("seq_slot", seq_slot), ("seq_pos0", seq_pos0), ("cu_seqlens", cu_seqlens)):
-        _i32("attn." + nm, t, n_seq)
+    _i32("attn.chunk_list", chunk_list, 8 * n_chunks)
+    _i32("attn.seq_pos0", seq_pos0, n_seq)
 
 
-def attn_decode_generic(q, k_pages, v_pages, out, partial, n_seq, chunk_seq, chunk_idx, n_chunks, pages_per_chunk,
-                        max_splits, seq_slot, seq_pos0, cu_seqlens, page_table, ring_pages, H, G, d, window,
-                        scale) -> None:
+def attn_decode_generic(q, k_pages, v_pages, out, partial, n_seq, chunk_list, n_chunks, pages_per_chunk,
+                        max_splits, seq_pos0, page_table, ring_pages, H, G, d, window, scale) -> None:
     _attn_check(q, k_pages, v_pages, out, page_table, H, G, d)
-    _decode_check(q, partial, n_seq, chunk_seq, chunk_idx, n_chunks, pages_per_chunk, max_splits, seq_slot, seq_pos0,
-                  cu_seqlens, H, d)
+    _decode_check(q, partial, n_seq, chunk_list, n_chunks, pages_per_chunk, max_splits, seq_pos0, H, d)
     _check(lib().picolm_attn_decode_generic(
         _ptr(q), _ptr(k_pages), _ptr(v_pages), _ptr(out), _ptr(partial if max_splits > 1 else None), dt_of(q),
-        n_seq, _ptr(chunk_seq), _ptr(chunk_idx), n_chunks, pages_per_chunk, max_splits, _ptr(seq_slot),
-        _ptr(seq_pos0), _ptr(cu_seqlens), _ptr(page_table), page_table.shape[1], ring_pages, H, G, d, window,
-        c_float(scale), _stream()))
+        n_seq, _ptr(chunk_list), n_chunks, pages_per_chunk, max_splits, _ptr(seq_pos0), _ptr(page_table),
+        page_table.shape[1], ring_pages, H, G, d, window, c_float(scale), _stream()))
 
 
 def _attn_check(q, k_pages, v_pages, out, page_table, H, G, d):
@@ -337,17 +331,14 @@ def attn_prefill_mfma(q, k_pages, v_pages, out, batch, page_table, ring_pages, H
         page_table.shape[1], ring_pages, H, G, d, window, c_float(scale), _stream()))
 
 
-def attn_decode_mfma(q, k_pages, v_pages, out, partial, n_seq, chunk_seq, chunk_idx, n_chunks, pages_per_chunk,
-                     max_splits, seq_slot, seq_pos0, cu_seqlens, page_table, ring_pages, H, G, d, window,
-                     scale) -> None:
+def attn_decode_mfma(q, k_pages, v_pages, out, partial, n_seq, chunk_list, n_chunks, pages_per_chunk,
+                     max_splits, seq_pos0, page_table, ring_pages, H, G, d, window, scale) -> None:
     _attn_check(q, k_pages, v_pages, out, page_table, H, G, d)
-    _decode_check(q, partial, n_seq, chunk_seq, chunk_idx, n_chunks, pages_per_chunk, max_splits, seq_slot, seq_pos0,
-                  cu_seqlens, H, d)
+    _decode_check(q, partial, n_seq, chunk_list, n_chunks, pages_per_chunk, max_splits, seq_pos0, H, d)
     _check(lib().picolm_attn_decode_mfma(
         _ptr(q), _ptr(k_pages), _ptr(v_pages), _ptr(out), _ptr(partial if max_splits > 1 else None), n_seq,
-        _ptr(chunk_seq), _ptr(chunk_idx), n_chunks, pages_per_chunk, max_splits, _ptr(seq_slot), _ptr(seq_pos0),
-        _ptr(cu_seqlens), _ptr(page_table), page_table.shape[1], ring_pages, H, G, d, window, c_float(scale),
-        _stream()))
+        _ptr(chunk_list), n_chunks, pages_per_chunk, max_splits, _ptr(seq_pos0), _ptr(page_table),
+        page_table.shape[1], ring_pages, H, G, d, window, c_float(scale), _stream()))
 
 
 def attn_prefill(q, k_pages, v_pages, out, batch, page_table, ring_pages, H, G, d, window, scale) -> None:
@@ -360,13 +351,14 @@ def attn_prefill(q, k_pages, v_pages, out, batch, page_table, ring_pages, H, G, 
                          batch.seq_nnew, batch.cu_seqlens, page_table, ring_pages, H, G, d, window, scale)
 
 
-def attn_decode(q, k_pages, v_pages, out, partial, n_seq, chunk_seq, chunk_idx, n_chunks, pages_per_chunk,
-                max_splits, seq_slot, seq_pos0, cu_seqlens, page_table, ring_pages, H, G, d, window, scale) -> None:
-    """Attention of one new token per sequence over its cache pages.  (chunk_seq, chunk_idx) is
-    the step's work list: entry x gives workgroup x `pages_per_chunk` pages of one sequence."""
+def attn_decode(q, k_pages, v_pages, out, partial, n_seq, chunk_list, n_chunks, pages_per_chunk, max_splits,
+                seq_pos0, page_table, ring_pages, H, G, d, window, scale) -> None:
+    """Attention of one new token per sequence (row i of q is sequence i) over its cache pages.
+    `chunk_list` is the step's work list, eight ints an entry: entry x gives workgroup x
+    `pages_per_chunk` pages of one sequence."""
     fn = attn_decode_mfma if attn_mfma_takes(q, d) else attn_decode_generic
-    fn(q, k_pages, v_pages, out, partial, n_seq, chunk_seq, chunk_idx, n_chunks, pages_per_chunk, max_splits,
-       seq_slot, seq_pos0, cu_seqlens, page_table, ring_pages, H, G, d, window, scale)
+    fn(q, k_pages, v_pages, out, partial, n_seq, chunk_list, n_chunks, pages_per_chunk, max_splits, seq_pos0,
+       page_table, ring_pages, H, G, d, window, scale)
 
 
 def sample(logits: torch.Tensor, out: torch.Tensor, temperature: float, top_k: int, top_p: float,

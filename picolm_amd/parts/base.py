@@ -98,6 +98,11 @@ class StepContext:
         g = self.cache.kv[gi]
         return g.k[e], g.v[e], g.table, g.ring_pages
 
+    def kv_host(self):
+        """(cache group index, the group's page table on the host) of the running layer call."""
+        gi, _ = self.binding.kv
+        return gi, self.cache.kv[gi].table_host
+
     def state(self) -> torch.Tensor:
         """[n_slots, ...] state of the running layer call; index it with batch.seq_slot."""
         gi, e = self.binding.state

@@ -200,6 +200,7 @@ class PagedCase:
                 vp[pg, :, :, :m] = torch.from_numpy(self.v[i][j * PAGE:j * PAGE + m]).permute(1, 2, 0).float()
         self.k_pages = kp.to(dtype).to(DEV)
         self.v_pages = vp.to(dtype).to(DEV)
+        self.table_host = table
         self.table = table.to(DEV)
         # what the kernel sees after rounding to its storage type
         rd = lambda x: torch.from_numpy(x).to(dtype).double().numpy()
@@ -238,14 +239,17 @@ def test_attention_prefill(dtype, H, G, d, window):
     assert err <= tol(dtype, np.abs(ref).max()), err
 
 
-def decode_work_list(pos0, window, pages_per_chunk, spare=0):
+def decode_work_list(case, window, pages_per_chunk, spare=0):
     """The work list the engine would build, with `spare` unused entries mixed in."""
     from picolm_amd.engine.batch import decode_chunk_list
-    seq, idx, most = decode_chunk_list(pos0, window, pages_per_chunk)
+    b = case.batch()
+    entries, most = decode_chunk_list(b.slots, b.pos0, window, pages_per_chunk, case.table_host,
+                                      case.table_host.shape[1])
     if spare:
-        seq = np.concatenate([seq[:1], np.full(spare, -1, np.int32), seq[1:], np.full(spare, -1, np.int32)])
-        idx = np.concatenate([idx[:1], np.full(spare, 7, np.int32), idx[1:], np.full(spare, 0, np.int32)])
-    return torch.from_numpy(seq).to(DEV), torch.from_numpy(idx).to(DEV), len(seq), most
+        unused = np.full((spare, 8), 7, np.int32)
+        unused[:, 0] = -1
+        entries = np.concatenate([entries[:1], unused, entries[1:], unused])
+    return torch.from_numpy(entries).to(DEV), len(entries), most
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
@@ -256,14 +260,34 @@ def test_attention_decode(dtype, H, G, d, pages_per_chunk, window, spare):
     case = PagedCase(H, G, d, pos0, [1, 1, 1, 1, 1], dtype, seed=H * d + pages_per_chunk)
     b = case.batch()
     out = torch.zeros_like(case.q_dev)
-    chunk_seq, chunk_idx, n_chunks, most = decode_work_list(pos0, window, pages_per_chunk, spare)
+    chunk_list, n_chunks, most = decode_work_list(case, window, pages_per_chunk, spare)
     partial = torch.full((b.n_seq * H * most * (d + 2),), float("nan"), device=DEV)
-    K().attn_decode(case.q_dev, case.k_pages, case.v_pages, out, partial, b.n_seq, chunk_seq, chunk_idx, n_chunks,
-                    pages_per_chunk, most, b.seq_slot, b.seq_pos0, b.cu_seqlens, case.table, case.table.shape[1],
-                    H, G, d, window, 1.0 / math.sqrt(d))
+    K().attn_decode(case.q_dev, case.k_pages, case.v_pages, out, partial, b.n_seq, chunk_list, n_chunks,
+                    pages_per_chunk, most, b.seq_pos0, case.table, case.table.shape[1], H, G, d, window,
+                    1.0 / math.sqrt(d))
     ref = case.reference(window)
     err = np.abs(out.double().cpu().numpy() - ref).max()
     assert err <= tol(dtype, np.abs(ref).max()), err
+
+
+@pytest.mark.parametrize("d", [64, 128])
+@pytest.mark.parametrize("pages_per_chunk", [1, 4, 8])
+def test_attention_decode_many_sequences(d, pages_per_chunk):
+    """With many sequences the matrix-core kernel runs four waves a workgroup instead of eight."""
+    H, G = 16, 8
+    rng = np.random.default_rng(d + pages_per_chunk)
+    pos0 = [int(x) for x in rng.integers(0, 900, size=40)]
+    case = PagedCase(H, G, d, pos0, [1] * len(pos0), torch.bfloat16, seed=d)
+    b = case.batch()
+    out = torch.zeros_like(case.q_dev)
+    chunk_list, n_chunks, most = decode_work_list(case, 0, pages_per_chunk, spare=2)
+    partial = torch.full((b.n_seq * H * most * (d + 2),), float("nan"), device=DEV)
+    K().attn_decode(case.q_dev, case.k_pages, case.v_pages, out, partial, b.n_seq, chunk_list, n_chunks,
+                    pages_per_chunk, most, b.seq_pos0, case.table, case.table.shape[1], H, G, d, 0,
+                    1.0 / math.sqrt(d))
+    ref = case.reference(0)
+    err = np.abs(out.double().cpu().numpy() - ref).max()
+    assert err <= tol(torch.bfloat16, np.abs(ref).max()), err
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
@@ -284,11 +308,11 @@ def test_attention_finds_a_far_key(dtype):
     b = case.batch()
     for pages_per_chunk in (16, 4, 1):
         out = torch.zeros_like(case.q_dev)
-        chunk_seq, chunk_idx, n_chunks, most = decode_work_list([699], 0, pages_per_chunk)
+        chunk_list, n_chunks, most = decode_work_list(case, 0, pages_per_chunk)
         partial = torch.zeros(b.n_seq * H * most * (d + 2), device=DEV)
-        K().attn_decode(case.q_dev, case.k_pages, case.v_pages, out, partial, 1, chunk_seq, chunk_idx, n_chunks,
-                        pages_per_chunk, most, b.seq_slot, b.seq_pos0, b.cu_seqlens, case.table, case.table.shape[1],
-                        H, G, d, 0, 1.0 / math.sqrt(d))
+        K().attn_decode(case.q_dev, case.k_pages, case.v_pages, out, partial, 1, chunk_list, n_chunks,
+                        pages_per_chunk, most, b.seq_pos0, case.table, case.table.shape[1], H, G, d, 0,
+                        1.0 / math.sqrt(d))
         got = out.double().cpu().numpy().reshape(H, d)
         for h in range(H):
             assert np.abs(got[h] - case.v[0][target, h // 2]).max() < 2e-2

@@ -7,18 +7,30 @@ from picolm_amd.engine.batch import (DecodeBatch, StepBatch, StepError, decode_c
                                      decode_pages_per_chunk)
 
 
-def pages_of_list(pos0, window, ppc):
+def make_table(pos0, ring_pages, seed=0):
+    """A page table with distinct physical pages for every (slot, ring position)."""
+    rng = np.random.default_rng(seed)
+    slots = list(rng.permutation(len(pos0) + 3)[:len(pos0)])
+    table = rng.permutation((len(pos0) + 3) * ring_pages).astype(np.int32).reshape(len(pos0) + 3, ring_pages)
+    return slots, table
+
+
+def pages_of_list(pos0, window, ppc, ring_pages=64):
     """Every (sequence, page) the work list covers, by the arithmetic the kernels use."""
-    seq, idx, most = decode_chunk_list(pos0, window, ppc)
+    slots, table = make_table(pos0, ring_pages)
+    entries, most = decode_chunk_list(slots, pos0, window, ppc, table, ring_pages)
     covered = []
-    for s, i in zip(seq, idx):
-        p = pos0[s]
-        first = (max(0, p - window + 1) if window > 0 else 0) // 64
-        end = p // 64 + 1
+    for s, i, qpos, slot, *phys in entries:
+        assert qpos == pos0[s] and slot == slots[s]
+        first = (max(0, qpos - window + 1) if window > 0 else 0) // 64
+        end = qpos // 64 + 1
         lo = first + i * ppc
         hi = min(end, lo + ppc)
         assert lo < hi, "an empty chunk"
         assert i < most
+        for w in range(4):
+            want = table[slot, (lo + w) % ring_pages] if lo + w < hi else -1
+            assert phys[w] == want
         covered += [(int(s), page) for page in range(lo, hi)]
     return covered
 
@@ -34,6 +46,12 @@ def test_work_list_covers_every_visible_page_once(window, ppc):
         expect += [(s, page) for page in range(lo // 64, p // 64 + 1)]
     assert sorted(covered) == sorted(expect)
     assert len(set(covered)) == len(covered)
+
+
+def test_work_list_of_a_ring():
+    """A windowed group keeps a ring of pages: page p lives at ring position p % ring_pages."""
+    covered = pages_of_list([5000, 100], 200, 2, ring_pages=9)
+    assert sorted(covered) == [(0, p) for p in range(75, 79)] + [(1, 0), (1, 1)]
 
 
 def test_pages_per_chunk_grows_with_the_work():
@@ -60,23 +78,31 @@ def test_step_batch_packs_without_padding():
 
 
 def test_decode_batch_rewrites_its_lists_in_place():
+    import torch
+    table = torch.arange(4 * 16, dtype=torch.int32).reshape(4, 16)
     b = DecodeBatch(3, 4, "cpu")
     b.fill([2, 0, 1], [10, 300, 64], [1, 2, 3])
-    seq, idx, cap, ppc, most = b.decode_chunks(8, 0, max_pages=16)
+    dev, cap, ppc, most = b.decode_chunks(8, 0, 0, table, 16)
     assert cap == 3 * 4 and ppc == 4 and most == 4
-    assert seq.tolist() == [0, 1, 1, 2] + [-1] * 8
-    assert idx.tolist()[:4] == [0, 0, 1, 0]
-    addr = seq.data_ptr()
+    rows = dev.reshape(-1, 8)
+    assert rows[:, 0].tolist() == [0, 1, 1, 2] + [-1] * 8
+    assert rows[:4, 1].tolist() == [0, 0, 1, 0]
+    assert rows[:4, 2].tolist() == [10, 300, 300, 64]
+    assert rows[:4, 3].tolist() == [2, 0, 0, 1]
+    assert rows[1, 4:].tolist() == [0, 1, 2, 3] and rows[2, 4:].tolist() == [4, -1, -1, -1]
+    assert rows[0, 4:].tolist() == [32, -1, -1, -1]
+    addr = dev.data_ptr()
     b.fill([2, 0, 1], [1000, 301, 65], [1, 2, 3])
-    seq2, idx2, *_ = b.decode_chunks(8, 0, max_pages=16)
-    assert seq2.data_ptr() == addr
-    assert seq2.tolist() == [0, 0, 0, 0, 1, 1, 2] + [-1] * 5
-    assert idx2.tolist()[:7] == [0, 1, 2, 3, 0, 1, 0]
-    # a windowed layer has a list of its own
-    wseq, *_ = b.decode_chunks(8, 64, max_pages=16)
-    assert wseq.tolist()[:4] == [0, 1, 2, -1]
+    dev2, *_ = b.decode_chunks(8, 0, 0, table, 16)
+    assert dev2.data_ptr() == addr
+    rows = dev2.reshape(-1, 8)
+    assert rows[:, 0].tolist() == [0, 0, 0, 0, 1, 1, 2] + [-1] * 5
+    assert rows[:7, 1].tolist() == [0, 1, 2, 3, 0, 1, 0]
+    # a windowed layer, or another cache group, has a list of its own
+    wdev, *_ = b.decode_chunks(8, 64, 0, table, 16)
+    assert wdev.reshape(-1, 8)[:4, 0].tolist() == [0, 1, 2, -1]
     with pytest.raises(StepError):
         b.fill([2, 0, 1], [1024, 0, 0], [1, 2, 3])       # 17 pages in a cache of 16
     b.frozen = True
     with pytest.raises(StepError):
-        b.decode_chunks(8, 128, max_pages=16)
+        b.decode_chunks(8, 128, 0, table, 16)
