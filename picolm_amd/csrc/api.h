@@ -25,9 +25,8 @@ int picolm_rmsnorm(const float* x, const float* w, void* out, int out_dt, const 
                    int n_rows, int D, float eps, hipStream_t stream);
 int picolm_rope_kv_store(const float* qkv, void* q_out, void* k_pages, void* v_pages, int dt,
                          const float* cos_t, const float* sin_t, int style, const int32_t* tok_pos,
-                         const int32_t* tok_seq, const int32_t* seq_slot, const int32_t* page_table,
-                         int max_pages, int ring_pages, int T, int H, int G, int d,
-                         const int32_t* rows /* null: rows 0..T-1 */, hipStream_t stream);
+                         const int32_t* tok_page /* physical cache page of every token */, int T, int H, int G,
+                         int d, const int32_t* rows /* null: rows 0..T-1 */, hipStream_t stream);
 int picolm_silu_mul(const void* gu, int in_dt, void* out, int out_dt, int64_t n_pairs,
                     hipStream_t stream);
 int picolm_add_into(float* y, const void* x, int x_dt, int64_t n, hipStream_t stream);

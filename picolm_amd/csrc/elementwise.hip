@@ -108,17 +108,15 @@ extern "C" int picolm_rmsnorm(const float* x, const float* w, void* out, int out
 // picolm rotates every q and k head of a token by its position's table row before k is
 // cached and leaves v alone (picolm/model_core.c:1908, :2915; picolm/tensor.c:3216-3304).
 // style 0: pairs (2i, 2i+1); style 1: pairs (i, i + d/2).  cos/sin == null: no rotation.
-// A token's cache row is page_table[slot][(pos / PAGE) % ring_pages], offset pos % PAGE.
+// A token's cache row is row pos % PAGE of physical page tok_page[t], which the host looked up
+// in its copy of the page table: page_table[slot][(pos / PAGE) % ring_pages].
 #define ROPE_HEADS 4
 template <typename TC>
 __global__ void rope_kv_store_kernel(const float* __restrict__ qkv, TC* __restrict__ q_out,
                                      TC* __restrict__ k_pages, TC* __restrict__ v_pages,
                                      const float* __restrict__ cos_t, const float* __restrict__ sin_t,
                                      int style, const int32_t* __restrict__ tok_pos,
-                                     const int32_t* __restrict__ tok_seq,
-                                     const int32_t* __restrict__ seq_slot,
-                                     const int32_t* __restrict__ page_table, int max_pages,
-                                     int ring_pages, int H, int G, int d,
+                                     const int32_t* __restrict__ tok_page, int H, int G, int d,
                                      const int32_t* __restrict__ rows) {
     const int t = rows ? rows[blockIdx.x] : blockIdx.x;      // `rows`: the token rows this launch handles
     const int pos = tok_pos[t];
@@ -132,8 +130,7 @@ __global__ void rope_kv_store_kernel(const float* __restrict__ qkv, TC* __restri
     size_t cache_row = 0, page_base = 0;
     const int in_page = pos % PAGE_TOKENS;
     if (k_pages) {
-        const int slot = seq_slot[tok_seq[t]];
-        const int page = page_table[(size_t)slot * max_pages + (pos / PAGE_TOKENS) % ring_pages];
+        const int page = tok_page[t];
         page_base = ((size_t)page * G) * PAGE_TOKENS * d;
         cache_row = page_base + (size_t)in_page * d;
     }
@@ -172,27 +169,24 @@ __global__ void rope_kv_store_kernel(const float* __restrict__ qkv, TC* __restri
 
 extern "C" int picolm_rope_kv_store(const float* qkv, void* q_out, void* k_pages, void* v_pages,
                                     int dt, const float* cos_t, const float* sin_t, int style,
-                                    const int32_t* tok_pos, const int32_t* tok_seq,
-                                    const int32_t* seq_slot, const int32_t* page_table,
-                                    int max_pages, int ring_pages, int T, int H, int G, int d,
-                                    const int32_t* rows, hipStream_t stream) {
+                                    const int32_t* tok_pos, const int32_t* tok_page, int T, int H, int G,
+                                    int d, const int32_t* rows, hipStream_t stream) {
     PICOLM_REQUIRE(T >= 0 && H > 0 && G > 0 && d > 0 && d % 2 == 0,
                    "rope_kv_store: bad sizes T=%d H=%d G=%d d=%d", T, H, G, d);
     PICOLM_REQUIRE((cos_t == nullptr) == (sin_t == nullptr), "rope_kv_store: need both tables or none");
     PICOLM_REQUIRE((k_pages == nullptr) == (v_pages == nullptr), "rope_kv_store: need both caches or none");
-    PICOLM_REQUIRE(!k_pages || (max_pages > 0 && ring_pages > 0 && ring_pages <= max_pages),
-                   "rope_kv_store: bad page table geometry max_pages=%d ring_pages=%d", max_pages, ring_pages);
+    PICOLM_REQUIRE(!k_pages || tok_page, "rope_kv_store: writing the cache needs every token's page");
     PICOLM_REQUIRE(style == 0 || style == 1, "rope_kv_store: unknown pairing %d", style);
     if (T == 0) return 0;
     dim3 grid(T, ceil_div(H + 2 * G, ROPE_HEADS)), block(d / 2 >= 64 ? 64 : 32);
     if (dt == PICOLM_F32)
         rope_kv_store_kernel<float><<<grid, block, 0, stream>>>(
-            qkv, (float*)q_out, (float*)k_pages, (float*)v_pages, cos_t, sin_t, style, tok_pos, tok_seq,
-            seq_slot, page_table, max_pages, ring_pages, H, G, d, rows);
+            qkv, (float*)q_out, (float*)k_pages, (float*)v_pages, cos_t, sin_t, style, tok_pos, tok_page,
+            H, G, d, rows);
     else if (dt == PICOLM_BF16)
         rope_kv_store_kernel<bf16_t><<<grid, block, 0, stream>>>(
-            qkv, (bf16_t*)q_out, (bf16_t*)k_pages, (bf16_t*)v_pages, cos_t, sin_t, style, tok_pos, tok_seq,
-            seq_slot, page_table, max_pages, ring_pages, H, G, d, rows);
+            qkv, (bf16_t*)q_out, (bf16_t*)k_pages, (bf16_t*)v_pages, cos_t, sin_t, style, tok_pos, tok_page,
+            H, G, d, rows);
     else
         PICOLM_REQUIRE(false, "rope_kv_store: unknown dtype %d", dt);
     PICOLM_LAUNCH_CHECK("rope_kv_store");

@@ -74,6 +74,7 @@ class StepBatch:
         self._upload(parts)
         self._tiles = {}
         self._chunks = {}
+        self._write_pages = {}
 
     def _upload(self, parts) -> None:
         sizes = [max(len(v), 1) for v in parts.values()]
@@ -113,6 +114,14 @@ class StepBatch:
             yield _Chunk(self, seqs, lo, [min(chunk_tokens, self.n_new[i] - lo) for i in seqs],
                          [int(cu[i]) + lo for i in seqs])
 
+    def write_pages(self, group: int, table_host, ring_pages: int):
+        """For every token of the step the physical page of cache group `group` that takes its
+        key and value (device int32 [T])."""
+        if group not in self._write_pages:
+            pages = token_pages(self._host["tok_seq"], self._host["tok_pos"], self.slots, table_host, ring_pages)
+            self._write_pages[group] = torch.from_numpy(pages).to(self._device)
+        return self._write_pages[group]
+
     def decode_chunks(self, blocks_per_chunk: int, window: int, group: int, table_host, ring_pages: int):
         """The decode attention's work list for this step over one cache group's pages:
         (entries on the device, number of entries, pages_per_chunk, most chunks of a sequence)."""
@@ -122,6 +131,12 @@ class StepBatch:
             entries, most = decode_chunk_list(self.slots, self.pos0, window, ppc, table_host, ring_pages)
             self._chunks[key] = (torch.from_numpy(entries).to(self._device), len(entries), ppc, most)
         return self._chunks[key]
+
+
+def token_pages(tok_seq, tok_pos, slots, table_host, ring_pages: int):
+    table = table_host.numpy() if hasattr(table_host, "numpy") else np.asarray(table_host)
+    slot = np.asarray(slots, dtype=np.int64)[np.asarray(tok_seq, dtype=np.int64)]
+    return table[slot, (np.asarray(tok_pos, dtype=np.int64) // PAGE_TOKENS) % ring_pages].astype(np.int32)
 
 
 def decode_pages_per_chunk(pos0, blocks_per_chunk: int, target_blocks: int = 512) -> int:
@@ -220,6 +235,7 @@ class DecodeBatch:
             setattr(self, k, self._dev[o:o + s])
         self.slots, self.pos0 = [], []
         self._lists = {}        # (window, group) -> (host block, device block, most chunks, page table, ring)
+        self._pages = {}        # group -> (host block, device block, page table, ring)
         self.frozen = False     # set once the launches are recorded: no further work list can join
 
     @staticmethod
@@ -236,6 +252,22 @@ class DecodeBatch:
         self._dev.copy_(self._host, non_blocking=False)
         for key in self._lists:
             self._fill_list(key)
+        for group in self._pages:
+            self._fill_pages(group)
+
+    def _fill_pages(self, group: int) -> None:
+        host, dev, table_host, ring_pages = self._pages[group]
+        host.numpy()[:] = token_pages(np.arange(self.n_seq), self.pos0, self.slots, table_host, ring_pages)
+        dev.copy_(host, non_blocking=False)
+
+    def write_pages(self, group: int, table_host, ring_pages: int):
+        if group not in self._pages:
+            if self.frozen:
+                raise StepError("a recorded decode step cannot take another cache group")
+            self._pages[group] = (self._host_block(self.n_seq), torch.zeros(self.n_seq, dtype=torch.int32, device=self._device),
+                                  table_host, ring_pages)
+            self._fill_pages(group)
+        return self._pages[group][1]
 
     def _fill_list(self, key) -> None:
         host, dev, most, table_host, ring_pages = self._lists[key]

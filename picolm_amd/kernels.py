@@ -124,9 +124,10 @@ def rmsnorm(x: torch.Tensor, weight: torch.Tensor, eps: float, out: torch.Tensor
                                 c_float(eps), _stream()))
 
 
-def rope_kv_store(qkv, q_out, k_pages, v_pages, cos, sin, style: int, tok_pos, tok_seq, seq_slot,
-                  page_table, ring_pages: int, H: int, G: int, d: int, rows=None, n_rows: int | None = None) -> None:
-    """Rotate q and k of every token row (or of `rows` only) and write k, v to the cache."""
+def rope_kv_store(qkv, q_out, k_pages, v_pages, cos, sin, style: int, tok_pos, tok_page, H: int, G: int, d: int,
+                  rows=None, n_rows: int | None = None) -> None:
+    """Rotate q and k of every token row (or of `rows` only) and write k, v to the cache: token
+    t goes to row tok_pos[t] % 64 of physical page tok_page[t]."""
     _dev("rope.qkv", qkv, torch.float32, 2)
     T = qkv.shape[0]
     if qkv.shape[1] != (H + 2 * G) * d:
@@ -134,19 +135,15 @@ def rope_kv_store(qkv, q_out, k_pages, v_pages, cos, sin, style: int, tok_pos, t
     _dev("rope.q_out", q_out, (torch.float32, torch.bfloat16), 2)
     if tuple(q_out.shape) != (T, H * d):
         raise KernelError(f"rope: q_out {tuple(q_out.shape)} is not {(T, H * d)}")
-    max_pages = 1
     if k_pages is not None:
         _check_pages("rope", k_pages, v_pages, q_out.dtype, G, d)
-        _dev("rope.page_table", page_table, torch.int32, 2)
-        max_pages = page_table.shape[1]
-        _i32("rope.seq_slot", seq_slot)
+        _i32("rope.tok_page", tok_page, T)
     if cos is not None:
         _dev("rope.cos", cos, torch.float32, 2)
         _dev("rope.sin", sin, torch.float32, 2)
         if cos.shape[1] != d // 2 or sin.shape != cos.shape:
             raise KernelError(f"rope: tables {tuple(cos.shape)} do not have d/2 = {d // 2} columns")
     _i32("rope.tok_pos", tok_pos, T)
-    _i32("rope.tok_seq", tok_seq, T)
     n_launch = T
     if rows is not None:
         n_launch = rows.numel() if n_rows is None else n_rows
@@ -155,8 +152,7 @@ def rope_kv_store(qkv, q_out, k_pages, v_pages, cos, sin, style: int, tok_pos, t
             raise KernelError("rope: more rows listed than there are")
     _check(lib().picolm_rope_kv_store(
         _ptr(qkv), _ptr(q_out), _ptr(k_pages), _ptr(v_pages), dt_of(q_out), _ptr(cos), _ptr(sin), style,
-        _ptr(tok_pos), _ptr(tok_seq), _ptr(seq_slot), _ptr(page_table), max_pages, ring_pages, n_launch, H, G, d,
-        _ptr(rows), _stream()))
+        _ptr(tok_pos), _ptr(tok_page if k_pages is not None else None), n_launch, H, G, d, _ptr(rows), _stream()))
 
 
 def _check_pages(who, k_pages, v_pages, dtype, G, d):

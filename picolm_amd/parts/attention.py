@@ -64,10 +64,10 @@ class Attention(Mixer):
         out = ctx.ws.get("attn.out", (T, H * d), ctx.dtype)
         writes = ctx.binding.writes
         kp, vp = (k_pages, v_pages) if writes else (None, None)
+        group, table_host = ctx.kv_host()
+        tok_page = b.write_pages(group, table_host, ring) if writes else None
         if b.is_decode:
-            kernels.rope_kv_store(qkv, q, kp, vp, cos, sin, style, b.tok_pos, b.tok_seq, b.seq_slot, table, ring,
-                                  H, G, d)
-            group, table_host = ctx.kv_host()
+            kernels.rope_kv_store(qkv, q, kp, vp, cos, sin, style, b.tok_pos, tok_page, H, G, d)
             chunk_list, n_chunks, ppc, most = b.decode_chunks(G * ((H // G + 15) // 16), self.window, group,
                                                                table_host, ring)
             partial = ctx.ws.get("attn.partial", (b.n_seq * H * most * (d + 2),), torch.float32) if most > 1 else None
@@ -76,11 +76,10 @@ class Attention(Mixer):
         elif self.window > 0 and ring < table.shape[1] and b.max_new > WINDOW_STEP_TOKENS:
             # a ring holds a window and one chunk: write and answer the step chunk by chunk
             for c in b.chunks(WINDOW_STEP_TOKENS):
-                kernels.rope_kv_store(qkv, q, kp, vp, cos, sin, style, b.tok_pos, b.tok_seq, b.seq_slot, table, ring,
-                                      H, G, d, rows=c.rows, n_rows=c.n_rows)
+                kernels.rope_kv_store(qkv, q, kp, vp, cos, sin, style, b.tok_pos, tok_page, H, G, d,
+                                      rows=c.rows, n_rows=c.n_rows)
                 kernels.attn_prefill(q, k_pages, v_pages, out, c, table, ring, H, G, d, self.window, self.scale)
         else:
-            kernels.rope_kv_store(qkv, q, kp, vp, cos, sin, style, b.tok_pos, b.tok_seq, b.seq_slot, table, ring,
-                                  H, G, d)
+            kernels.rope_kv_store(qkv, q, kp, vp, cos, sin, style, b.tok_pos, tok_page, H, G, d)
             kernels.attn_prefill(q, k_pages, v_pages, out, b, table, ring, H, G, d, self.window, self.scale)
         self.o.forward(out, residual, kernels.EPI_ACCUMULATE)

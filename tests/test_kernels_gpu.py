@@ -332,13 +332,14 @@ def test_rope_kv_store(dtype, style):
     b = StepBatch(slots, pos0, [[0] * n for n in n_new], [[], []], 10, DEV)
     positions = np.concatenate([np.arange(p, p + n) for p, n in zip(pos0, n_new)])
     cos, sin = P.rope_tables(np.arange(200), inv)
-    table = torch.tensor([[4, 1], [0, 0], [3, 5]], dtype=torch.int32, device=DEV)
+    table_host = torch.tensor([[4, 1], [0, 0], [3, 5]], dtype=torch.int32)
+    table = table_host.to(DEV)
     kp = torch.zeros(6, G, PAGE, d, dtype=dtype, device=DEV)
     vp = torch.zeros(6, G, d, PAGE, dtype=dtype, device=DEV)
     q_out = torch.zeros(T, H * d, dtype=dtype, device=DEV)
     K().rope_kv_store(torch.from_numpy(qkv).to(DEV), q_out, kp, vp, torch.from_numpy(cos).float().to(DEV),
-                      torch.from_numpy(sin).float().to(DEV), 0 if style == "pairwise" else 1, b.tok_pos, b.tok_seq,
-                      b.seq_slot, table, 2, H, G, d)
+                      torch.from_numpy(sin).float().to(DEV), 0 if style == "pairwise" else 1, b.tok_pos,
+                      b.write_pages(0, table_host, 2), H, G, d)
     x = qkv.astype(np.float64).reshape(T, H + 2 * G, d)
     c, s = P.rope_tables(positions, inv)
     q_ref = P.apply_rope(x[:, :H], c, s, style).reshape(T, H * d)

@@ -56,7 +56,7 @@ def test_work_list_of_a_ring():
 
 def test_pages_per_chunk_grows_with_the_work():
     assert decode_pages_per_chunk([100], 8) == 4
-    assert decode_pages_per_chunk([4095] * 8, 8) == 4
+    assert decode_pages_per_chunk([1000] * 8, 8) == 4
     big = decode_pages_per_chunk([4095] * 64, 8)
     assert big > 4 and big & (big - 1) == 0
     assert decode_pages_per_chunk([4095] * 64, 8, target_blocks=10 ** 9) == 4
@@ -75,6 +75,16 @@ def test_step_batch_packs_without_padding():
         StepBatch([1], [0], [[10]], [[0]], 10, "cpu")
     with pytest.raises(StepError):
         StepBatch([1], [0], [[1]], [[1]], 10, "cpu")
+
+
+def test_write_pages_follow_the_page_table():
+    table = np.arange(3 * 5, dtype=np.int32).reshape(3, 5) + 100
+    b = StepBatch([2, 0], [61, 0], [[1] * 5, [2] * 70], [[], []], 10, "cpu")
+    pages = b.write_pages(0, table, 5).tolist()
+    assert pages[:5] == [110, 110, 110, 111, 111]            # slot 2: positions 61..65
+    assert pages[5:5 + 64] == [100] * 64 and pages[69:75] == [101] * 6
+    ring = b.write_pages(1, table, 1).tolist()                 # a ring of one page
+    assert ring[:5] == [110] * 5 and ring[5:] == [100] * 70
 
 
 def test_decode_batch_rewrites_its_lists_in_place():
@@ -101,6 +111,10 @@ def test_decode_batch_rewrites_its_lists_in_place():
     # a windowed layer, or another cache group, has a list of its own
     wdev, *_ = b.decode_chunks(8, 64, 0, table, 16)
     assert wdev.reshape(-1, 8)[:4, 0].tolist() == [0, 1, 2, -1]
+    pages = b.write_pages(0, table, 16)
+    assert pages.tolist() == [32 + 15, 4, 16 + 1]          # positions 1000, 301, 65 of slots 2, 0, 1
+    b.fill([2, 0, 1], [64, 0, 128], [1, 2, 3])
+    assert pages.tolist() == [33, 0, 18]
     with pytest.raises(StepError):
         b.fill([2, 0, 1], [1024, 0, 0], [1, 2, 3])       # 17 pages in a cache of 16
     b.frozen = True
