@@ -41,6 +41,11 @@ int picolm_gemm_skinny(const void* A, const void* W, void* C, int c_dt, int M, i
 int picolm_gemm_tiled(const void* A, const void* W, void* C, int c_dt, int M, int N, int K, int64_t lda,
                       int64_t ldw, int64_t ldc, int epilogue, int variant, hipStream_t stream);
 
+// ws: splits * M * N floats; variants 9 and up
+int picolm_gemm_tiled_splitk(const void* A, const void* W, void* C, int c_dt, int M, int N, int K, int64_t lda,
+                             int64_t ldw, int64_t ldc, int epilogue, int variant, int splits, float* ws,
+                             hipStream_t stream);
+
 int picolm_attn_prefill_tile_rows(void);
 int picolm_attn_prefill_generic(const void* q, const void* k_pages, const void* v_pages, void* out,
                                 int dt, const int32_t* tile_seq, const int32_t* tile_q0, int n_tiles,

@@ -189,6 +189,119 @@ static int launch_skinny(const void* A, const void* W, void* C, int c_dt, int M,
     return 0;
 }
 
+// ---- skinny, with the activations resident ---------------------------------------------------
+// For M <= 16 and K <= STEPS * 1024: a wave keeps the activation chunks of its K slices in
+// registers for the whole launch and a workgroup walks over many tiles of 16 weight rows, with
+// the next tile's weights in flight while the current one is multiplied and reduced.  The
+// activations are read once per workgroup instead of once per tile, and the gap between tiles
+// (the reduction through LDS, the epilogue) no longer leaves the memory pipe empty.
+template <int STEPS, int EPI, typename TC>
+__global__ __launch_bounds__(512) void gemm_skinny_resident_kernel(const bf16_t* __restrict__ A,
+                                                                   const bf16_t* __restrict__ W,
+                                                                   TC* __restrict__ C, int M, int N, int K,
+                                                                   int64_t lda, int64_t ldw, int64_t ldc) {
+    constexpr int WAVES = 8;
+    __shared__ float red[2][WAVES][4][64];
+    const int wave = threadIdx.x / 64, lane = threadIdx.x % 64;
+    const int r16 = lane % 16, q = lane / 16;
+    const int n_full = K / SK_KSTEP;            // K is a whole number of steps (the host sees to that)
+    const int n_tiles = (N + 15) / 16;
+
+    bf16x8 av[STEPS][4];
+    int koff[STEPS];                            // element offset of this lane's first chunk of step i
+#pragma unroll
+    for (int i = 0; i < STEPS; ++i) {
+        const int s = wave + i * WAVES;
+        const bool valid = s < n_full && r16 < M;
+        koff[i] = min(s, n_full - 1) * SK_KSTEP + q * 8;      // a step past the end reads the last one; its activations are zero
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+            av[i][j] = valid ? load_chunk(A + (int64_t)r16 * lda + koff[i] + 32 * j) : zero_chunk();
+    }
+    auto fetch = [&](bf16x8 (&wv)[STEPS][4], int tile) {
+        const bf16_t* wrow = W + (int64_t)min(tile * 16 + r16, N - 1) * ldw;
+#pragma unroll
+        for (int i = 0; i < STEPS; ++i)
+#pragma unroll
+            for (int j = 0; j < 4; ++j) wv[i][j] = load_chunk(wrow + koff[i] + 32 * j);
+    };
+    auto finish = [&](const bf16x8 (&wv)[STEPS][4], int tile, int buf) {
+        f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int i = 0; i < STEPS; ++i)
+#pragma unroll
+            for (int j = 0; j < 4; ++j) acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wv[i][j], av[i][j], acc, 0, 0, 0);
+#pragma unroll
+        for (int r = 0; r < 4; ++r) red[buf][wave][r][lane] = acc[r];
+        __syncthreads();
+        // value (r, l): n = 16*tile + 4*(l/16) + r, m = l%16; the gated epilogue takes r and r+1 together
+        constexpr int STEP = (EPI == 2) ? 2 : 1;
+        const int v = threadIdx.x;
+        if (v < 256 / STEP) {
+            const int l = v % 64, r = EPI == 2 ? 2 * (v / 64) : v / 64;
+            float s0 = 0.f, s1 = 0.f;
+#pragma unroll
+            for (int w = 0; w < WAVES; ++w) {
+                s0 += red[buf][w][r][l];
+                if (EPI == 2) s1 += red[buf][w][r + 1][l];
+            }
+            const int n = tile * 16 + 4 * (l / 16) + r, m = l % 16;
+            if (m < M && n < N) {
+                if (EPI == 2) {
+                    C[(int64_t)m * ldc + n / 2] = from_f32<TC>(silu_mul(s0, s1));
+                } else if (EPI == 1) {
+                    TC* p = C + (int64_t)m * ldc + n;
+                    *p = from_f32<TC>(to_f32<TC>(*p) + s0);
+                } else {
+                    C[(int64_t)m * ldc + n] = from_f32<TC>(s0);
+                }
+            }
+        }
+    };
+    // two register sets of weights and two LDS buffers alternate, so that one barrier a tile is
+    // enough; tiles past the end read the last tile again and are not finished
+    bf16x8 w0[STEPS][4], w1[STEPS][4];
+    const int stride = gridDim.x;
+    int tile = blockIdx.x;
+    fetch(w0, min(tile, n_tiles - 1));
+    while (tile < n_tiles) {
+        fetch(w1, min(tile + stride, n_tiles - 1));
+        __builtin_amdgcn_sched_barrier(0);      // the next tile is asked for before this one is waited for
+        finish(w0, tile, 0);
+        tile += stride;
+        if (tile >= n_tiles) break;
+        fetch(w0, min(tile + stride, n_tiles - 1));
+        __builtin_amdgcn_sched_barrier(0);
+        finish(w1, tile, 1);
+        tile += stride;
+    }
+}
+
+template <int STEPS>
+static int launch_skinny_resident(const void* A, const void* W, void* C, int c_dt, int M, int N, int K, int64_t lda,
+                                  int64_t ldw, int64_t ldc, int epi, hipStream_t stream) {
+    PICOLM_REQUIRE(M <= 16 && K % SK_KSTEP == 0 && K <= STEPS * 8 * SK_KSTEP,
+                   "gemm_skinny: the resident variant takes M <= 16 and K a multiple of %d up to %d, got M=%d K=%d",
+                   SK_KSTEP, STEPS * 8 * SK_KSTEP, M, K);
+    // one workgroup a CU; the same number of tiles for every workgroup where that is possible
+    const int n_tiles = ceil_div(N, 16);
+    const int rounds = ceil_div(n_tiles, 256);
+    dim3 grid(ceil_div(n_tiles, rounds)), block(512);
+    const bf16_t* a = (const bf16_t*)A;
+    const bf16_t* w = (const bf16_t*)W;
+#define SR_LAUNCH(EPI, TC) \
+    gemm_skinny_resident_kernel<STEPS, EPI, TC><<<grid, block, 0, stream>>>(a, w, (TC*)C, M, N, K, lda, ldw, ldc);
+    if (epi == 0 && c_dt == PICOLM_F32) SR_LAUNCH(0, float)
+    else if (epi == 0 && c_dt == PICOLM_BF16) SR_LAUNCH(0, bf16_t)
+    else if (epi == 1 && c_dt == PICOLM_F32) SR_LAUNCH(1, float)
+    else if (epi == 2 && c_dt == PICOLM_BF16) SR_LAUNCH(2, bf16_t)
+    else if (epi == 2 && c_dt == PICOLM_F32) SR_LAUNCH(2, float)
+    else PICOLM_REQUIRE(false, "gemm_skinny: unsupported epilogue %d with output dtype %d", epi, c_dt);
+#undef SR_LAUNCH
+    PICOLM_LAUNCH_CHECK("gemm_skinny");
+    return 0;
+}
+
 static int check_mfma_operands(const char* who, const void* A, const void* W, int M, int N, int K, int64_t lda,
                                int64_t ldw, int64_t ldc, int epi, int c_dt) {
     PICOLM_REQUIRE(M >= 0 && N > 0 && K > 0, "%s: bad sizes M=%d N=%d K=%d", who, M, N, K);
@@ -203,14 +316,21 @@ static int check_mfma_operands(const char* who, const void* A, const void* W, in
     return 0;
 }
 
-// variant: 0 picks by M; otherwise 1..6 name (MT,NT,WAVES) combinations for tuning and tests
+// variant: 0 picks by shape; 1..6 name (MT,NT,WAVES) combinations for tuning and tests, 7 is
+// the variant with resident activations
 extern "C" int picolm_gemm_skinny(const void* A, const void* W, void* C, int c_dt, int M, int N, int K,
                                   int64_t lda, int64_t ldw, int64_t ldc, int epilogue, int variant,
                                   hipStream_t stream) {
     if (check_mfma_operands("gemm_skinny", A, W, M, N, K, lda, ldw, ldc, epilogue, c_dt)) return -1;
     PICOLM_REQUIRE(M <= 64, "gemm_skinny: M=%d exceeds 64", M);
     if (M == 0) return 0;
-    if (variant == 0) variant = M <= 16 ? 1 : (M <= 32 ? 3 : (N >= 8192 ? 6 : 5));
+    if (variant == 0) {
+        // many tiles a CU and several rows: the resident variant reads the activations once and
+        // keeps the memory pipe full between tiles (a few rows cost little to re-read, and then
+        // several workgroups a CU hide more latency); few tiles: one workgroup a tile
+        if (M > 4 && M <= 16 && N >= 16384 && K % SK_KSTEP == 0 && K <= 4 * 8 * SK_KSTEP) variant = 7;
+        else variant = M <= 16 ? 1 : (M <= 32 ? 3 : (N >= 8192 ? 6 : 5));
+    }
     switch (variant) {
         case 1: return launch_skinny<1, 1, 8>(A, W, C, c_dt, M, N, K, lda, ldw, ldc, epilogue, stream);
         case 2: return launch_skinny<1, 2, 8>(A, W, C, c_dt, M, N, K, lda, ldw, ldc, epilogue, stream);
@@ -218,6 +338,7 @@ extern "C" int picolm_gemm_skinny(const void* A, const void* W, void* C, int c_d
         case 4: return launch_skinny<2, 2, 8>(A, W, C, c_dt, M, N, K, lda, ldw, ldc, epilogue, stream);
         case 5: return launch_skinny<4, 1, 8>(A, W, C, c_dt, M, N, K, lda, ldw, ldc, epilogue, stream);
         case 6: return launch_skinny<4, 2, 4>(A, W, C, c_dt, M, N, K, lda, ldw, ldc, epilogue, stream);
+        case 7: return launch_skinny_resident<4>(A, W, C, c_dt, M, N, K, lda, ldw, ldc, epilogue, stream);
     }
     PICOLM_REQUIRE(false, "gemm_skinny: unknown variant %d", variant);
 }
@@ -485,7 +606,12 @@ __global__ __launch_bounds__(64 * WN * WM) void gemm_direct_kernel(const bf16_t*
                                                                    const bf16_t* __restrict__ W,
                                                                    TC* __restrict__ C, int M, int N, int K,
                                                                    int64_t lda, int64_t ldw, int64_t ldc,
-                                                                   int tiles_m, int tiles_n) {
+                                                                   int tiles_m, int tiles_n, int64_t c_split_stride) {
+    // K here is the length of one split: workgroup row y of the grid takes columns y*K .. of A
+    // and W and writes its sums to C + y * c_split_stride
+    A += (int64_t)blockIdx.y * K;
+    W += (int64_t)blockIdx.y * K;
+    C += (int64_t)blockIdx.y * c_split_stride;
     constexpr int NW = WN * WM;
     constexpr int BN = 32 * TN * WN, BM = 32 * TM * WM;
     constexpr int CH = BK / 8;                 // 16-byte chunks in a row of a stage
@@ -530,8 +656,17 @@ __global__ __launch_bounds__(64 * WN * WM) void gemm_direct_kernel(const bf16_t*
     const bf16_t* a_tile = A + (int64_t)m0 * lda;
     const unsigned lds_wave = __builtin_amdgcn_readfirstlane(
         (unsigned)(size_t)(__attribute__((address_space(3))) bf16_t*)lds + wave * (RG * BK * 2));
+    // With one row of tiles every weight is read once, from memory: then workgroups start at
+    // different places of K and wrap around.  If all of them walked K in step, all rows would be
+    // read at the same column at the same time, and rows lie a power of two apart, so that few
+    // memory channels would take all the traffic.  With several rows of tiles the tiles that share
+    // a slice must stay in step, so that one of them finds it in L2.
+    const int n_steps = K / BK;
+    const int first_step = tiles_m == 1 ? (int)(((unsigned)tile * 5u + blockIdx.y * 3u) % (unsigned)n_steps) : 0;
     auto issue = [&](int stage, int step) {
         const unsigned to = lds_wave + stage * (STAGE * 2);
+        step += first_step;
+        if (step >= n_steps) step -= n_steps;
         const bf16_t* wsrc = w_tile + step * BK;
         const bf16_t* asrc = a_tile + step * BK;
 #pragma unroll
@@ -577,7 +712,6 @@ __global__ __launch_bounds__(64 * WN * WM) void gemm_direct_kernel(const bf16_t*
     };
     // K is a whole number of steps (the host sees to that).  Steps past the end load the last
     // step again into a stage nobody reads, so that the count of loads in flight stays the same.
-    const int n_steps = K / BK;
 #pragma unroll
     for (int s = 0; s < NS - 1; ++s) issue(s, min(s, n_steps - 1));
     // begin step j: its loads have landed for every wave, the stage of step j-1 is read out and
@@ -644,18 +778,21 @@ __global__ __launch_bounds__(64 * WN * WM) void gemm_direct_kernel(const bf16_t*
 
 template <int TN, int TM, int WN, int WM, int BK, int NS>
 static int launch_direct(const void* A, const void* W, void* C, int c_dt, int M, int N, int K, int64_t lda,
-                         int64_t ldw, int64_t ldc, int epilogue, hipStream_t stream) {
+                         int64_t ldw, int64_t ldc, int epilogue, hipStream_t stream, int splits = 1,
+                         int64_t c_split_stride = 0) {
     constexpr int BN = 32 * TN * WN, BM = 32 * TM * WM;
-    PICOLM_REQUIRE(K % BK == 0, "gemm_tiled: K = %d is no multiple of %d, which this variant needs", K, BK);
+    PICOLM_REQUIRE(splits >= 1 && K % (BK * splits) == 0,
+                   "gemm_tiled: K = %d is no multiple of %d times %d splits, which this variant needs", K, BK, splits);
     PICOLM_REQUIRE((int64_t)BN * ldw < (1ll << 30) && (int64_t)BM * lda < (1ll << 30),
                    "gemm_tiled: row strides %lld / %lld overflow the tile's 32-bit offsets", (long long)lda, (long long)ldw);
     const int tiles_m = ceil_div(M, BM), tiles_n = ceil_div(N, BN);
     PICOLM_REQUIRE((int64_t)tiles_m * tiles_n < (1ll << 31), "gemm_tiled: too many tiles");
-    dim3 grid(tiles_m * tiles_n), block(64 * WN * WM);
+    dim3 grid(tiles_m * tiles_n, splits), block(64 * WN * WM);
     const size_t lds = (size_t)NS * (BN + BM) * BK * sizeof(bf16_t);
     static_assert((size_t)NS * (BN + BM) * BK * 2 <= 160 * 1024, "stages exceed the LDS");
     const bf16_t* a = (const bf16_t*)A;
     const bf16_t* w = (const bf16_t*)W;
+    const int k_len = K / splits;
 #define TD_LAUNCH(EPI, TC)                                                                                 \
     {                                                                                                      \
         static size_t raised = 48 * 1024;                                                                  \
@@ -666,8 +803,8 @@ static int launch_direct(const void* A, const void* W, void* C, int c_dt, int M,
                            hipGetErrorString(e));                                                          \
             raised = lds;                                                                                  \
         }                                                                                                  \
-        gemm_direct_kernel<TN, TM, WN, WM, BK, NS, EPI, TC><<<grid, block, lds, stream>>>(a, w, (TC*)C, M, N, K,  \
-                                                                                  lda, ldw, ldc, tiles_m, tiles_n); \
+        gemm_direct_kernel<TN, TM, WN, WM, BK, NS, EPI, TC><<<grid, block, lds, stream>>>(                 \
+            a, w, (TC*)C, M, N, k_len, lda, ldw, ldc, tiles_m, tiles_n, c_split_stride);                   \
     }
     if (epilogue == 0 && c_dt == PICOLM_F32) TD_LAUNCH(0, float)
     else if (epilogue == 0 && c_dt == PICOLM_BF16) TD_LAUNCH(0, bf16_t)
@@ -680,13 +817,52 @@ static int launch_direct(const void* A, const void* W, void* C, int c_dt, int M,
     return 0;
 }
 
+// ---- split K ---------------------------------------------------------------------------------
+// A product with few output tiles is cut along K so that every CU has a workgroup: split z
+// writes its partial sums to ws[z][M][N]; the kernel below adds the splits in order (the same
+// order every time) and applies the epilogue.
+template <int EPI, typename TC>
+__global__ __launch_bounds__(256) void splitk_reduce_kernel(const float* __restrict__ ws, TC* __restrict__ C, int M, int N,
+                                                            int64_t ldc, int splits) {
+    constexpr int PER = EPI == 2 ? 2 : 1;
+    const int64_t i = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) * 4;      // four floats of a row
+    if (i >= (int64_t)M * N) return;
+    const int m = (int)(i / N), n = (int)(i % N);        // N is a multiple of 4 (the host sees to that)
+    f32x4 sum = {0.f, 0.f, 0.f, 0.f};
+    for (int z = 0; z < splits; ++z) sum += *(const f32x4*)(ws + (int64_t)z * M * N + i);
+    if (EPI == 2) {
+        TC* p = C + (int64_t)m * ldc + n / 2;
+        p[0] = from_f32<TC>(silu_mul(sum[0], sum[1]));
+        p[1] = from_f32<TC>(silu_mul(sum[2], sum[3]));
+    } else {
+        TC* p = C + (int64_t)m * ldc + n;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) p[e] = from_f32<TC>(EPI == 1 ? to_f32<TC>(p[e]) + sum[e] : sum[e]);
+    }
+    (void)PER;
+}
+
+static int launch_splitk_reduce(const float* ws, void* C, int c_dt, int M, int N, int64_t ldc, int splits, int epilogue,
+                                hipStream_t stream) {
+    const int64_t quads = (int64_t)M * N / 4;
+    dim3 grid((unsigned)ceil_div64(quads, 256)), block(256);
+    if (epilogue == 0 && c_dt == PICOLM_F32) splitk_reduce_kernel<0, float><<<grid, block, 0, stream>>>(ws, (float*)C, M, N, ldc, splits);
+    else if (epilogue == 0 && c_dt == PICOLM_BF16) splitk_reduce_kernel<0, bf16_t><<<grid, block, 0, stream>>>(ws, (bf16_t*)C, M, N, ldc, splits);
+    else if (epilogue == 1 && c_dt == PICOLM_F32) splitk_reduce_kernel<1, float><<<grid, block, 0, stream>>>(ws, (float*)C, M, N, ldc, splits);
+    else if (epilogue == 2 && c_dt == PICOLM_BF16) splitk_reduce_kernel<2, bf16_t><<<grid, block, 0, stream>>>(ws, (bf16_t*)C, M, N, ldc, splits);
+    else if (epilogue == 2 && c_dt == PICOLM_F32) splitk_reduce_kernel<2, float><<<grid, block, 0, stream>>>(ws, (float*)C, M, N, ldc, splits);
+    else PICOLM_REQUIRE(false, "gemm_splitk: unsupported epilogue %d with output dtype %d", epilogue, c_dt);
+    PICOLM_LAUNCH_CHECK("gemm_splitk_reduce");
+    return 0;
+}
+
 // variant 0 picks by shape.  Tiles loaded straight into LDS (K a multiple of 64):
 //   9: 256x256, 8 waves, two stages of 64 columns;  10: 256(n)x128(m), 8 waves, three stages;
-//   11: 128x128, 4 waves, four stages.
+//   11: 128x128, 4 waves, four stages;
+//   12: 128(n)x64(m), 4 waves, three stages: for decode batches of up to 64 rows, where the
+//   weights stream once and K may be split.
 // Tiles staged through registers (any K that is a multiple of 8):
-//   1: 128x128 (4 waves), 4: 256x256 (8 waves);
-//   7, 8: 64 rows of activations against 128 or 64 weight rows, for decode batches too wide for
-//   the skinny kernel.
+//   1: 128x128 (4 waves), 4: 256x256 (8 waves).
 extern "C" int picolm_gemm_tiled(const void* A, const void* W, void* C, int c_dt, int M, int N, int K,
                                  int64_t lda, int64_t ldw, int64_t ldc, int epilogue, int variant,
                                  hipStream_t stream) {
@@ -721,11 +897,34 @@ extern "C" int picolm_gemm_tiled(const void* A, const void* W, void* C, int c_dt
     switch (variant) {
         case 1: return launch_tiled<2, 2, 2, 2, 2>(A, W, C, c_dt, M, N, K, lda, ldw, ldc, epilogue, stream);
         case 4: return launch_tiled<2, 4, 4, 2, 1>(A, W, C, c_dt, M, N, K, lda, ldw, ldc, epilogue, stream);
-        case 7: return launch_tiled<1, 2, 4, 1, 2>(A, W, C, c_dt, M, N, K, lda, ldw, ldc, epilogue, stream);
-        case 8: return launch_tiled<1, 2, 2, 1, 2>(A, W, C, c_dt, M, N, K, lda, ldw, ldc, epilogue, stream);
         case 9: return launch_direct<2, 4, 4, 2, 64, 2>(A, W, C, c_dt, M, N, K, lda, ldw, ldc, epilogue, stream);
         case 10: return launch_direct<2, 2, 4, 2, 64, 3>(A, W, C, c_dt, M, N, K, lda, ldw, ldc, epilogue, stream);
         case 11: return launch_direct<2, 2, 2, 2, 64, 4>(A, W, C, c_dt, M, N, K, lda, ldw, ldc, epilogue, stream);
+        case 12: return launch_direct<1, 2, 4, 1, 64, 3>(A, W, C, c_dt, M, N, K, lda, ldw, ldc, epilogue, stream);
     }
     PICOLM_REQUIRE(false, "gemm_tiled: unknown variant %d", variant);
+}
+
+// The tiled product cut into `splits` along K (variants 9 and up only); ws holds
+// splits * M * N floats.  N must be a multiple of 4.
+extern "C" int picolm_gemm_tiled_splitk(const void* A, const void* W, void* C, int c_dt, int M, int N, int K,
+                                        int64_t lda, int64_t ldw, int64_t ldc, int epilogue, int variant,
+                                        int splits, float* ws, hipStream_t stream) {
+    if (check_mfma_operands("gemm_splitk", A, W, M, N, K, lda, ldw, ldc, epilogue, c_dt)) return -1;
+    PICOLM_REQUIRE(splits >= 1 && splits <= 64, "gemm_splitk: %d splits", splits);
+    if (splits == 1) return picolm_gemm_tiled(A, W, C, c_dt, M, N, K, lda, ldw, ldc, epilogue, variant, stream);
+    PICOLM_REQUIRE(ws != nullptr && ((uintptr_t)ws & 15) == 0, "gemm_splitk: needs a 16-byte aligned workspace");
+    PICOLM_REQUIRE(N % 4 == 0, "gemm_splitk: N = %d is no multiple of 4", N);
+    if (M == 0) return 0;
+    const int64_t stride = (int64_t)M * N;
+    int rc;
+    switch (variant) {
+        case 9: rc = launch_direct<2, 4, 4, 2, 64, 2>(A, W, ws, PICOLM_F32, M, N, K, lda, ldw, N, 0, stream, splits, stride); break;
+        case 10: rc = launch_direct<2, 2, 4, 2, 64, 3>(A, W, ws, PICOLM_F32, M, N, K, lda, ldw, N, 0, stream, splits, stride); break;
+        case 11: rc = launch_direct<2, 2, 2, 2, 64, 4>(A, W, ws, PICOLM_F32, M, N, K, lda, ldw, N, 0, stream, splits, stride); break;
+        case 12: rc = launch_direct<1, 2, 4, 1, 64, 3>(A, W, ws, PICOLM_F32, M, N, K, lda, ldw, N, 0, stream, splits, stride); break;
+        default: PICOLM_REQUIRE(false, "gemm_splitk: variant %d cannot split K", variant);
+    }
+    if (rc) return rc;
+    return launch_splitk_reduce(ws, C, c_dt, M, N, ldc, splits, epilogue, stream);
 }

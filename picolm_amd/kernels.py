@@ -42,7 +42,7 @@ def dir_entry_points():
     return ["picolm_abi_version", "picolm_device_check", "picolm_embed", "picolm_rmsnorm",
             "picolm_rope_kv_store", "picolm_silu_mul", "picolm_add_into", "picolm_gemm_generic",
             "picolm_attn_prefill_tile_rows", "picolm_attn_prefill_generic",
-            "picolm_attn_decode_generic", "picolm_argmax", "picolm_argmax_scratch_floats", "picolm_sample", "picolm_gemm_skinny", "picolm_gemm_tiled",
+            "picolm_attn_decode_generic", "picolm_argmax", "picolm_argmax_scratch_floats", "picolm_sample", "picolm_gemm_skinny", "picolm_gemm_tiled", "picolm_gemm_tiled_splitk",
             "picolm_attn_mfma_takes", "picolm_attn_prefill_mfma_heads", "picolm_attn_prefill_mfma_tile_tokens",
             "picolm_attn_prefill_mfma", "picolm_attn_decode_mfma", "picolm_read_probe", "picolm_mfma_probe"]
 
@@ -284,6 +284,28 @@ def gemm_tiled(a, w, c, epilogue: int = EPI_STORE, variant: int = 0) -> None:
                                    c_int64(c.shape[1]), epilogue, variant, _stream()))
 
 
+SPLITK_WS_FLOATS = 4 << 20        # 16 MB of partial sums: splits * M * N may not exceed it
+_splitk_ws: dict = {}
+
+
+def splitk_workspace(device) -> torch.Tensor:
+    """One buffer per GPU for the partial sums of products cut along K; kernels of one stream
+    run in order, so they can share it."""
+    key = torch.device(device).index or 0
+    if key not in _splitk_ws:
+        _splitk_ws[key] = torch.empty(SPLITK_WS_FLOATS, dtype=torch.float32, device=device)
+    return _splitk_ws[key]
+
+
+def gemm_tiled_splitk(a, w, c, epilogue: int, variant: int, splits: int) -> None:
+    M, N, K = _gemm_shapes(a, w, c, epilogue)
+    if splits > 1 and splits * M * N > SPLITK_WS_FLOATS:
+        raise KernelError(f"gemm: {splits} splits of {M}x{N} exceed the workspace")
+    ws = splitk_workspace(a.device) if splits > 1 else None
+    _check(lib().picolm_gemm_tiled_splitk(_ptr(a), _ptr(w), _ptr(c), dt_of(c), M, N, K, c_int64(K), c_int64(K),
+                                          c_int64(c.shape[1]), epilogue, variant, splits, _ptr(ws), _stream()))
+
+
 def mfma_gemm_takes(a, w, c, epilogue: int) -> bool:
     """Whether the matrix-core kernels accept these operands; otherwise the float kernel runs."""
     if a.dtype != torch.bfloat16 or w.dtype != torch.bfloat16:
@@ -297,17 +319,28 @@ def mfma_gemm_takes(a, w, c, epilogue: int) -> bool:
     return True
 
 
+def medium_gemm_splits(M: int, N: int, K: int) -> int:
+    """Into how many parts along K a product of 17..64 rows is cut: its tiles hold 128 weight
+    rows each, and every CU should have one."""
+    tiles = (N + 127) // 128
+    if tiles >= 200 or N % 4:
+        return 1
+    s = 8
+    while s > 1 and (tiles * s > 320 or K % (64 * s) or s * M * N > SPLITK_WS_FLOATS):
+        s //= 2
+    return s
+
+
 def gemm(a: torch.Tensor, w: torch.Tensor, c: torch.Tensor, epilogue: int = EPI_STORE) -> None:
     """The product the engine calls: picks the kernel for the operands' types and sizes."""
     if mfma_gemm_takes(a, w, c, epilogue):
-        M, N = a.shape[0], w.shape[0]
+        M, N, K = a.shape[0], w.shape[0], a.shape[1]
         if M > SKINNY_MAX_M:
             gemm_tiled(a, w, c, epilogue)
-        elif M > 8 and N >= 16384:
-            # many output columns: weights through LDS in 128-row tiles, all rows in one 64-row tile
-            gemm_tiled(a, w, c, epilogue, variant=7)
-        elif M > 32 and N >= 6144:
-            gemm_tiled(a, w, c, epilogue, variant=8)
+        elif M > 16 and K % 64 == 0:
+            # a decode batch too wide to re-read its activations for every 16 weight rows: tiles
+            # of 128 weight rows through LDS, cut along K where there are few of them
+            gemm_tiled_splitk(a, w, c, epilogue, 12, medium_gemm_splits(M, N, K))
         else:
             gemm_skinny(a, w, c, epilogue)
     else:
