@@ -20,7 +20,8 @@ from replay_util import ROOT, TraceRun
 pytestmark = pytest.mark.gpu
 DEV = "cuda:0"
 
-LENGTHS = {"A": [33, 47, 64, 65, 100, 128], "B": [33, 40, 64, 129, 200, 256], "C": [34, 63, 65, 128, 190, 300]}
+LENGTHS = {"A": [33, 47, 64, 65, 100, 128], "B": [33, 40, 64, 129, 200, 256], "C": [34, 63, 65, 128, 190, 300],
+           "D": [33, 50, 64, 127, 130, 260]}
 
 
 def tolerance(dtype, ref):
@@ -31,7 +32,7 @@ def tolerance(dtype, ref):
 @pytest.fixture(scope="module")
 def folders(tmp_path_factory):
     tmp = tmp_path_factory.mktemp("models")
-    return {w: tiny.make_model_dir(tmp, w) for w in "ABC"}
+    return {w: tiny.make_model_dir(tmp, w) for w in tiny.CONFIGS}
 
 
 @pytest.fixture(scope="module")
@@ -46,7 +47,7 @@ def requests_and_truth(folders):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("which", ["A", "B", "C"])
+@pytest.mark.parametrize("which", ["A", "B", "C", "D"])
 def test_replay_whole_tail_and_batches(which, dtype, folders, requests_and_truth, tmp_path):
     reqs, truth = requests_and_truth[which]
     one_batch = sum((len(r) + 63) // 64 for r in reqs[3:]) * 64          # room for the larger batch only

@@ -34,7 +34,18 @@ TINY_C = dict(
     eos_token_id=5, rope_style="pairwise")
 TINY_C_WEIGHTS = dict(seed=2, std=0.08, norm_sigma=0.2)
 
-CONFIGS = {"A": (TINY_A, TINY_A_WEIGHTS), "B": (TINY_B, TINY_B_WEIGHTS), "C": (TINY_C, TINY_C_WEIGHTS)}
+# a fourth whose widths are multiples of 128 and 64, as real checkpoints' are: the kernels that
+# want such widths (the product with the norm inside, tiles loaded straight into LDS, split K,
+# matrix-core attention at head size 64) run in the engine only with this one
+TINY_D = dict(
+    architectures=["LlamaForCausalLM"], hidden_size=256, intermediate_size=320, num_attention_heads=4,
+    num_key_value_heads=2, num_hidden_layers=2, vocab_size=515, head_dim=64, rms_norm_eps=1e-5,
+    rope_theta=10000.0, rope_scaling=None, tie_word_embeddings=False, max_position_embeddings=512,
+    eos_token_id=1, rope_style="half")
+TINY_D_WEIGHTS = dict(seed=3, std=0.04, norm_sigma=0.3)
+
+CONFIGS = {"A": (TINY_A, TINY_A_WEIGHTS), "B": (TINY_B, TINY_B_WEIGHTS), "C": (TINY_C, TINY_C_WEIGHTS),
+           "D": (TINY_D, TINY_D_WEIGHTS)}
 
 
 def make_model_dir(tmp_path, which: str, dtype: str = "bfloat16") -> str:
