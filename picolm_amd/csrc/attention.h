@@ -27,6 +27,15 @@ struct AttnArgs {
     const int32_t* chunk_list;
     int pages_per_chunk;
     int max_splits;             // chunks a sequence can have: stride of `partial`
+    // decode with the rotation inside (matrix-core kernel only): q, and the new token's k and v,
+    // are taken from the float rows qkv[n_seq][(H+2G)*d]; q and k are rotated by the tables
+    // (cos_t null: no rotation), the new key and value join the attention from registers and are
+    // written to row position % 64 of physical page tok_page[sequence]
+    const float* qkv;
+    const float* cos_t;
+    const float* sin_t;
+    const int32_t* tok_page;
+    int rope_style;             // 0 pairs (2i, 2i+1), 1 pairs (i, i + d/2)
 };
 
 // What a decode workgroup has to do.  A sequence whose visible pages fit one chunk is finished by

@@ -293,7 +293,8 @@ extern "C" int picolm_attn_prefill_generic(const void* q, const void* k_pages, c
     PICOLM_REQUIRE(H <= 65535, "attn_prefill: %d heads exceed the grid", H);
     if (n_tiles <= 0) return 0;
     AttnArgs a = {q, k_pages, v_pages, out, nullptr, tile_seq, tile_q0, seq_slot, seq_pos0, seq_nnew,
-                  cu_seqlens, page_table, max_pages, ring_pages, H, G, d, window, scale, 0, nullptr, 0, 1};
+                  cu_seqlens, page_table, max_pages, ring_pages, H, G, d, window, scale, 0, nullptr, 0, 1,
+                  nullptr, nullptr, nullptr, nullptr, 0};
     dim3 grid(n_tiles, H);
     if (dt == PICOLM_F32) return launch_attn<float>(a, grid, stream);
     if (dt == PICOLM_BF16) return launch_attn<bf16_t>(a, grid, stream);
@@ -315,7 +316,8 @@ extern "C" int picolm_attn_decode_generic(const void* q, const void* k_pages, co
     const int chunks = ceil_div(H / G, AT_ROWS);
     PICOLM_REQUIRE(G * chunks <= 65535, "attn_decode: %d groups exceed the grid", G * chunks);
     AttnArgs a = {q, k_pages, v_pages, out, partial, nullptr, nullptr, nullptr, seq_pos0, nullptr, nullptr,
-                  page_table, max_pages, ring_pages, H, G, d, window, scale, 1, chunk_list, pages_per_chunk, max_splits};
+                  page_table, max_pages, ring_pages, H, G, d, window, scale, 1, chunk_list, pages_per_chunk, max_splits,
+                  nullptr, nullptr, nullptr, nullptr, 0};
     dim3 grid(n_chunks, G * chunks);
     const int rc = dt == PICOLM_F32 ? launch_attn<float>(a, grid, stream) : launch_attn<bf16_t>(a, grid, stream);
     if (rc) return rc;

@@ -22,6 +22,7 @@
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4;
 typedef __attribute__((ext_vector_type(16))) float f32x16;
+typedef __attribute__((ext_vector_type(4))) float f32x4;
 
 #define LOG2E 1.4426950408889634f
 #define LN2 0.6931471805599453f
@@ -107,8 +108,8 @@ __device__ __forceinline__ void attend_page(const bf16x8 (&Qf)[D / 16], f32x16 (
 template <int D>
 __device__ __forceinline__ void attend_tile(const bf16x8 (&Qf)[D / 16], const bf16x8 (&Kf)[D / 16],
                                             const bf16x8 (&Vf)[D / 32][2], f32x16 (&O)[D / 32], float& m_run,
-                                            float& l_run, int key0, int qpos, bool q_ok, int window, float scale2,
-                                            int h) {
+                                            float& l_run, int key0, int key_max, int qpos, bool q_ok, int window,
+                                            float scale2, int h) {
     f32x16 S;
 #pragma unroll
     for (int e = 0; e < 16; ++e) S[e] = 0.f;
@@ -118,7 +119,7 @@ __device__ __forceinline__ void attend_tile(const bf16x8 (&Qf)[D / 16], const bf
 #pragma unroll
     for (int e = 0; e < 16; ++e) {
         const int key = key0 + key_of_elem(e, h);
-        const bool vis = q_ok && key <= qpos && (window <= 0 || qpos - key < window);
+        const bool vis = q_ok && key <= key_max && (window <= 0 || qpos - key < window);
         S[e] = vis ? S[e] * scale2 : NEG_BIG;
         mx = fmaxf(mx, S[e]);
     }
@@ -287,9 +288,64 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void a
 // one 32-byte entry of the work list, so that only two trips to memory lie between the launch
 // and the first MFMA.  Eight waves give a short step for a few sequences; with many sequences
 // four waves, two workgroups a CU, move more bytes.
+// With a.qkv set the rotation and the cache write of the new token happen here too: q is rotated
+// on its way into the MFMA operands; the workgroups of a sequence's last chunk rotate the new key,
+// round key and value to bfloat16 as the cache holds them, put them into the merge below as one
+// more partial result (score, weight 1, value), and one of them writes them to the cache for
+// later steps.  The cache row of the new token is not read in this step.
+template <int D>
+__device__ __forceinline__ void rotated_q(const AttnArgs& a, const float* row, int pos, int h, bool ok, bf16x8 (&Qf)[D / 16]) {
+    const float* c = a.cos_t ? a.cos_t + (size_t)pos * (D / 2) : nullptr;
+    const float* sn = a.sin_t ? a.sin_t + (size_t)pos * (D / 2) : nullptr;
+#pragma unroll
+    for (int s = 0; s < D / 16; ++s) Qf[s] = zero8();
+    if (!ok) return;
+    if (!c) {
+#pragma unroll
+        for (int s = 0; s < D / 16; ++s) {
+            const f32x4 x0 = *(const f32x4*)(row + 16 * s + 8 * h), x1 = *(const f32x4*)(row + 16 * s + 8 * h + 4);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                Qf[s][e] = to_bf16(x0[e]);
+                Qf[s][4 + e] = to_bf16(x1[e]);
+            }
+        }
+    } else if (a.rope_style == 0) {
+#pragma unroll
+        for (int s = 0; s < D / 16; ++s) {
+            const int d0 = 16 * s + 8 * h;
+            const f32x4 x0 = *(const f32x4*)(row + d0), x1 = *(const f32x4*)(row + d0 + 4);
+            const f32x4 cc = *(const f32x4*)(c + d0 / 2), ss = *(const f32x4*)(sn + d0 / 2);
+            Qf[s][0] = to_bf16(x0[0] * cc[0] - x0[1] * ss[0]);
+            Qf[s][1] = to_bf16(x0[0] * ss[0] + x0[1] * cc[0]);
+            Qf[s][2] = to_bf16(x0[2] * cc[1] - x0[3] * ss[1]);
+            Qf[s][3] = to_bf16(x0[2] * ss[1] + x0[3] * cc[1]);
+            Qf[s][4] = to_bf16(x1[0] * cc[2] - x1[1] * ss[2]);
+            Qf[s][5] = to_bf16(x1[0] * ss[2] + x1[1] * cc[2]);
+            Qf[s][6] = to_bf16(x1[2] * cc[3] - x1[3] * ss[3]);
+            Qf[s][7] = to_bf16(x1[2] * ss[3] + x1[3] * cc[3]);
+        }
+    } else {
+#pragma unroll
+        for (int s = 0; s < D / 32; ++s) {
+            const int d0 = 16 * s + 8 * h;          // below d/2; its partner is d0 + d/2, k-step s + D/32 of this lane
+#pragma unroll
+            for (int half4 = 0; half4 < 2; ++half4) {
+                const f32x4 lo = *(const f32x4*)(row + d0 + 4 * half4), hi = *(const f32x4*)(row + d0 + D / 2 + 4 * half4);
+                const f32x4 cc = *(const f32x4*)(c + d0 + 4 * half4), ss = *(const f32x4*)(sn + d0 + 4 * half4);
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    Qf[s][4 * half4 + e] = to_bf16(lo[e] * cc[e] - hi[e] * ss[e]);
+                    Qf[s + D / 32][4 * half4 + e] = to_bf16(lo[e] * ss[e] + hi[e] * cc[e]);
+                }
+            }
+        }
+    }
+}
+
 template <int D, int DEC_WAVES>
 __global__ __launch_bounds__(DEC_WAVES * 64) __attribute__((amdgpu_waves_per_eu(2))) void attn_decode_mfma_kernel(AttnArgs a) {
-    extern __shared__ float mrg[];       // [DEC_WAVES][Rc][D + 2]
+    extern __shared__ float mrg[];       // [DEC_WAVES + 1][Rc][D + 2], then the new key and value [2][D]
     const int tid = threadIdx.x, wave = tid / WAVE, lane = tid % WAVE;
     const int l32 = lane % 32, h = lane / 32;
     const int R = a.H / a.G;
@@ -303,11 +359,36 @@ __global__ __launch_bounds__(DEC_WAVES * 64) __attribute__((amdgpu_waves_per_eu(
     const int head = g * R + chunk * 32 + (q_ok ? l32 : 0);
     const size_t tok = (size_t)seq;
     const int qpos = work.qpos;
+    const bool fused = a.qkv != nullptr;
+    const bool takes_new = fused && split == work.n_chunks - 1;       // this chunk ends with the new token
+    const int key_max = fused ? qpos - 1 : qpos;                       // the last key read from the cache
+    float* knew = mrg + (size_t)(DEC_WAVES + 1) * Rc * (D + 2);
+    float* vnew = knew + D;
 
     const int page_lo = work.page_lo, page_hi = work.page_hi;
     // k-step s of a lane covers d = 16s + 8h .. +8: the two halves of a wave read 32 adjacent bytes of a key
     bf16x8 Qf[D / 16];
-    {
+    if (fused) {
+        const float* row = a.qkv + tok * (size_t)(a.H + 2 * a.G) * D;
+        rotated_q<D>(a, row + (size_t)head * D, qpos, h, q_ok, Qf);
+        if (takes_new) {
+            const float* krow = row + (size_t)(a.H + g) * D;
+            const float* vrow = row + (size_t)(a.H + a.G + g) * D;
+            if (tid < D / 2) {
+                const int i0 = a.rope_style == 0 ? 2 * tid : tid, i1 = a.rope_style == 0 ? 2 * tid + 1 : tid + D / 2;
+                const float x0 = krow[i0], x1 = krow[i1];
+                float y0 = x0, y1 = x1;
+                if (a.cos_t) {
+                    const float cc = a.cos_t[(size_t)qpos * (D / 2) + tid], ss = a.sin_t[(size_t)qpos * (D / 2) + tid];
+                    y0 = x0 * cc - x1 * ss;
+                    y1 = x0 * ss + x1 * cc;
+                }
+                knew[i0] = (float)to_bf16(y0);
+                knew[i1] = (float)to_bf16(y1);
+            }
+            if (tid >= 64 && tid < 64 + D) vnew[tid - 64] = (float)to_bf16(vrow[tid - 64]);
+        }
+    } else {
         const bf16_t* qp = (const bf16_t*)a.q + tok * a.H * D + (size_t)head * D + 8 * h;
 #pragma unroll
         for (int s = 0; s < D / 16; ++s) Qf[s] = q_ok ? ldg8(qp + 16 * s) : zero8();
@@ -332,12 +413,12 @@ __global__ __launch_bounds__(DEC_WAVES * 64) __attribute__((amdgpu_waves_per_eu(
     for (int tt = wave; tt < n_tiles; tt += DEC_WAVES) {
         const int page = page_lo + tt / 2, t = tt & 1;
         const int key0 = page * PAGE_TOKENS + 32 * t;
-        if (key0 > qpos) break;                              // nothing of this tile, or of a later one, is visible
+        if (key0 > key_max) break;                           // nothing of this tile, or of a later one, is visible
         const int next_phys = tt + DEC_WAVES < n_tiles ? page_of_tile(tt + DEC_WAVES) : 0;   // asked for before this tile's data
         const size_t base = (size_t)phys * page_elems + (size_t)g * PAGE_TOKENS * D;
         const bf16_t* kp = (const bf16_t*)a.k_pages + base + 8 * h;
         const bf16_t* vp = (const bf16_t*)a.v_pages + base + (size_t)l32 * PAGE_TOKENS + 8 * h;
-        const int n_keys = qpos - key0 + 1;                  // >= 1; keys past it are not this sequence's
+        const int n_keys = key_max - key0 + 1;               // >= 1; keys past it are not this sequence's, or not written yet
         bf16x8 Kf[D / 16], Vf[D / 32][2];
 #pragma unroll
         for (int s = 0; s < D / 16; ++s) Kf[s] = ldg8(kp + (size_t)(32 * t + key_of_row(l32)) * D + 16 * s);
@@ -356,7 +437,7 @@ __global__ __launch_bounds__(DEC_WAVES * 64) __attribute__((amdgpu_waves_per_eu(
                         if (k + e >= n_keys) Vf[dt][ks][e] = (__bf16)0.0f;
                 }
         }
-        attend_tile<D>(Qf, Kf, Vf, O, m_run, l_run, key0, qpos, q_ok, a.window, scale2, h);
+        attend_tile<D>(Qf, Kf, Vf, O, m_run, l_run, key0, key_max, qpos, q_ok, a.window, scale2, h);
         phys = next_phys;
     }
     // merge the waves
@@ -373,18 +454,41 @@ __global__ __launch_bounds__(DEC_WAVES * 64) __attribute__((amdgpu_waves_per_eu(
             for (int e = 0; e < 16; ++e) row[2 + 32 * dt + 8 * (e / 4) + 4 * h + e % 4] = O[dt][e];
     }
     __syncthreads();
+    if (takes_new) {
+        // the new token as the partial result of one more wave: its score with every head of this
+        // workgroup, weight 1, its value
+        if (wave == 0 && q_ok) {
+            float dot = 0.f;
+#pragma unroll
+            for (int s = 0; s < D / 16; ++s)
+#pragma unroll
+                for (int e = 0; e < 8; ++e) dot += (float)Qf[s][e] * knew[16 * s + 8 * h + e];
+            dot += __shfl_xor(dot, 32, WAVE);
+            if (h == 0) {
+                float* row = mrg + ((size_t)DEC_WAVES * Rc + l32) * (D + 2);
+                row[0] = dot * scale2;
+                row[1] = 1.0f;
+            }
+        }
+        if (chunk == 0 && tid < D) {                        // one workgroup of the group writes the cache
+            const size_t base = (size_t)a.tok_page[seq] * page_elems + (size_t)g * PAGE_TOKENS * D;
+            const int in_page = qpos % PAGE_TOKENS;
+            ((bf16_t*)a.k_pages)[base + (size_t)in_page * D + tid] = f32_to_bf16_bits(knew[tid]);
+            ((bf16_t*)a.v_pages)[base + (size_t)tid * PAGE_TOKENS + in_page] = f32_to_bf16_bits(vnew[tid]);
+        }
+        __syncthreads();
+    }
+    const int n_parts = takes_new ? DEC_WAVES + 1 : DEC_WAVES;
     for (int idx = tid; idx < Rc * D; idx += DEC_WAVES * 64) {
         const int q = idx / D, dcol = idx % D;
         float M = NEG_BIG;
-#pragma unroll
-        for (int w = 0; w < DEC_WAVES; ++w) M = fmaxf(M, mrg[((size_t)w * Rc + q) * (D + 2)]);
+        for (int w = 0; w < n_parts; ++w) M = fmaxf(M, mrg[((size_t)w * Rc + q) * (D + 2)]);
         float L = 0.f, acc = 0.f;
-#pragma unroll
-        for (int w = 0; w < DEC_WAVES; ++w) {
+        for (int w = 0; w < n_parts; ++w) {
             const float* row = mrg + ((size_t)w * Rc + q) * (D + 2);
             const float f = exp2f(row[0] - M);
             L += f * row[1];
-            acc += f * row[2 + dcol];
+            acc += f * (w < DEC_WAVES ? row[2 + dcol] : vnew[dcol]);
         }
         const int hq = g * R + chunk * 32 + q;
         if (work.n_chunks > 1) {
@@ -433,7 +537,8 @@ extern "C" int picolm_attn_prefill_mfma(const void* q, const void* k_pages, cons
     const int head_chunks = ceil_div(H / G, HB);
     PICOLM_REQUIRE(G * head_chunks <= 65535, "attn_prefill_mfma: %d head groups exceed the grid", G * head_chunks);
     AttnArgs a = {q, k_pages, v_pages, out, nullptr, tile_seq, tile_q0, seq_slot, seq_pos0, seq_nnew,
-                  cu_seqlens, page_table, max_pages, ring_pages, H, G, d, window, scale, 0, nullptr, 0, 1};
+                  cu_seqlens, page_table, max_pages, ring_pages, H, G, d, window, scale, 0, nullptr, 0, 1,
+                  nullptr, nullptr, nullptr, nullptr, 0};
     dim3 grid(n_tiles, G * head_chunks), block(256);
     const size_t lds = 2 * 2 * (size_t)PAGE_TOKENS * d * sizeof(bf16_t);       // two stages of K and V^T
     if (d == 32) attn_prefill_mfma_kernel<32><<<grid, block, lds, stream>>>(a, HB, tile_tokens);
@@ -456,21 +561,12 @@ int check_decode_chunks(const char* who, const float* partial, const int32_t* ch
                         int pages_per_chunk, int max_splits);
 int picolm_attn_merge_launch(const AttnArgs& a, int dt, int n_seq, hipStream_t stream);
 
-extern "C" int picolm_attn_decode_mfma(const void* q, const void* k_pages, const void* v_pages, void* out,
-                                       float* partial, int n_seq, const int32_t* chunk_list, int n_chunks,
-                                       int pages_per_chunk, int max_splits, const int32_t* seq_pos0,
-                                       const int32_t* page_table, int max_pages, int ring_pages, int H, int G,
-                                       int d, int window, float scale, hipStream_t stream) {
-    if (check_sizes("attn_decode_mfma", H, G, d, max_pages, ring_pages)) return -1;
-    if (check_decode_chunks("attn_decode_mfma", partial, chunk_list, n_chunks, pages_per_chunk, max_splits)) return -1;
-    if (n_seq <= 0 || n_chunks <= 0) return 0;
-    const int R = H / G, chunks = ceil_div(R, 32);
-    PICOLM_REQUIRE(G * chunks <= 65535, "attn_decode_mfma: %d groups exceed the grid", G * chunks);
-    AttnArgs a = {q, k_pages, v_pages, out, partial, nullptr, nullptr, nullptr, seq_pos0, nullptr, nullptr,
-                  page_table, max_pages, ring_pages, H, G, d, window, scale, 1, chunk_list, pages_per_chunk, max_splits};
-    const int waves = (int64_t)n_seq * G * chunks >= 256 ? 4 : 8;
-    dim3 grid(n_chunks, G * chunks), block(waves * 64);
-    const size_t lds = sizeof(float) * waves * (size_t)min(R, 32) * (d + 2);
+static int launch_decode_mfma(const AttnArgs& a, int n_seq, int n_chunks, hipStream_t stream) {
+    const int R = a.H / a.G, chunks = ceil_div(R, 32), d = a.d;
+    PICOLM_REQUIRE(a.G * chunks <= 65535, "attn_decode_mfma: %d groups exceed the grid", a.G * chunks);
+    const int waves = (int64_t)n_seq * a.G * chunks >= 256 ? 4 : 8;
+    dim3 grid(n_chunks, a.G * chunks), block(waves * 64);
+    const size_t lds = sizeof(float) * ((waves + 1) * (size_t)min(R, 32) * (d + 2) + 2 * d);
 #define DEC_LAUNCH(D, W)                                                                                    \
     {                                                                                                       \
         static size_t raised = 48 * 1024;                                                                   \
@@ -491,5 +587,43 @@ extern "C" int picolm_attn_decode_mfma(const void* q, const void* k_pages, const
     else DEC_LAUNCH(128, 8)
 #undef DEC_LAUNCH
     PICOLM_LAUNCH_CHECK("attn_decode_mfma");
-    return max_splits > 1 ? picolm_attn_merge_launch(a, PICOLM_BF16, n_seq, stream) : 0;
+    return a.max_splits > 1 ? picolm_attn_merge_launch(a, PICOLM_BF16, n_seq, stream) : 0;
+}
+
+extern "C" int picolm_attn_decode_mfma(const void* q, const void* k_pages, const void* v_pages, void* out,
+                                       float* partial, int n_seq, const int32_t* chunk_list, int n_chunks,
+                                       int pages_per_chunk, int max_splits, const int32_t* seq_pos0,
+                                       const int32_t* page_table, int max_pages, int ring_pages, int H, int G,
+                                       int d, int window, float scale, hipStream_t stream) {
+    if (check_sizes("attn_decode_mfma", H, G, d, max_pages, ring_pages)) return -1;
+    if (check_decode_chunks("attn_decode_mfma", partial, chunk_list, n_chunks, pages_per_chunk, max_splits)) return -1;
+    if (n_seq <= 0 || n_chunks <= 0) return 0;
+    AttnArgs a = {q, k_pages, v_pages, out, partial, nullptr, nullptr, nullptr, seq_pos0, nullptr, nullptr,
+                  page_table, max_pages, ring_pages, H, G, d, window, scale, 1, chunk_list, pages_per_chunk, max_splits,
+                  nullptr, nullptr, nullptr, nullptr, 0};
+    return launch_decode_mfma(a, n_seq, n_chunks, stream);
+}
+
+// The decode step's rotation, cache write and attention in one launch: q, k, v of the new tokens
+// come as the float rows qkv[n_seq][(H+2G)*d]; tok_page[i] is the physical page that takes
+// sequence i's new key and value.  cos_t, sin_t [positions][d/2] or both null for no rotation.
+extern "C" int picolm_attn_decode_rope_mfma(const float* qkv, void* k_pages, void* v_pages, void* out,
+                                            float* partial, int n_seq, const int32_t* chunk_list, int n_chunks,
+                                            int pages_per_chunk, int max_splits, const int32_t* seq_pos0,
+                                            const int32_t* page_table, int max_pages, int ring_pages, int H,
+                                            int G, int d, int window, float scale, const float* cos_t,
+                                            const float* sin_t, int style, const int32_t* tok_page,
+                                            hipStream_t stream) {
+    if (check_sizes("attn_decode_rope_mfma", H, G, d, max_pages, ring_pages)) return -1;
+    if (check_decode_chunks("attn_decode_rope_mfma", partial, chunk_list, n_chunks, pages_per_chunk, max_splits)) return -1;
+    PICOLM_REQUIRE(qkv && tok_page, "attn_decode_rope_mfma: needs the qkv rows and every token's page");
+    PICOLM_REQUIRE(((uintptr_t)qkv & 15) == 0 && ((uintptr_t)cos_t & 15) == 0 && ((uintptr_t)sin_t & 15) == 0,
+                   "attn_decode_rope_mfma: qkv and the tables must be 16-byte aligned");
+    PICOLM_REQUIRE((cos_t == nullptr) == (sin_t == nullptr), "attn_decode_rope_mfma: need both tables or none");
+    PICOLM_REQUIRE(style == 0 || style == 1, "attn_decode_rope_mfma: unknown pairing %d", style);
+    if (n_seq <= 0 || n_chunks <= 0) return 0;
+    AttnArgs a = {nullptr, k_pages, v_pages, out, partial, nullptr, nullptr, nullptr, seq_pos0, nullptr, nullptr,
+                  page_table, max_pages, ring_pages, H, G, d, window, scale, 1, chunk_list, pages_per_chunk, max_splits,
+                  qkv, cos_t, sin_t, tok_page, style};
+    return launch_decode_mfma(a, n_seq, n_chunks, stream);
 }

@@ -44,7 +44,7 @@ def dir_entry_points():
             "picolm_attn_prefill_tile_rows", "picolm_attn_prefill_generic",
             "picolm_attn_decode_generic", "picolm_argmax", "picolm_argmax_scratch_floats", "picolm_sample", "picolm_gemm_skinny", "picolm_gemm_tiled", "picolm_gemm_tiled_splitk",
             "picolm_attn_mfma_takes", "picolm_attn_prefill_mfma_heads", "picolm_attn_prefill_mfma_tile_tokens",
-            "picolm_attn_prefill_mfma", "picolm_attn_decode_mfma", "picolm_read_probe", "picolm_mfma_probe"]
+            "picolm_attn_prefill_mfma", "picolm_attn_decode_mfma", "picolm_attn_decode_rope_mfma", "picolm_read_probe", "picolm_mfma_probe"]
 
 
 def _check(rc: int) -> None:
@@ -368,6 +368,45 @@ def attn_decode_mfma(q, k_pages, v_pages, out, partial, n_seq, chunk_list, n_chu
         _ptr(q), _ptr(k_pages), _ptr(v_pages), _ptr(out), _ptr(partial if max_splits > 1 else None), n_seq,
         _ptr(chunk_list), n_chunks, pages_per_chunk, max_splits, _ptr(seq_pos0), _ptr(page_table),
         page_table.shape[1], ring_pages, H, G, d, window, c_float(scale), _stream()))
+
+
+def attn_decode_rope_takes(dtype: torch.dtype, d: int) -> bool:
+    """Whether the decode kernel that rotates and writes the cache itself takes this case."""
+    return dtype == torch.bfloat16 and bool(lib().picolm_attn_mfma_takes(d))
+
+
+def attn_decode_rope(qkv, k_pages, v_pages, out, partial, n_seq, chunk_list, n_chunks, pages_per_chunk, max_splits,
+                     seq_pos0, page_table, ring_pages, H, G, d, window, scale, cos, sin, style, tok_page) -> None:
+    """A decode step's rotation, cache write and attention in one launch (bfloat16 cache, head
+    sizes of the matrix-core kernels): `qkv` are the float rows [n_seq, (H+2G)d] of the new tokens,
+    `tok_page[i]` the physical page that takes sequence i's new key and value."""
+    _dev("attn.qkv", qkv, torch.float32, 2)
+    if qkv.shape[0] < n_seq or qkv.shape[1] != (H + 2 * G) * d:
+        raise KernelError(f"attn_decode_rope: qkv {tuple(qkv.shape)} is not [>= {n_seq}, {(H + 2 * G) * d}]")
+    _dev("attn.out", out, torch.bfloat16, 2)
+    if out.shape[0] < n_seq or out.shape[1] != H * d:
+        raise KernelError(f"attn_decode_rope: out {tuple(out.shape)} is not [>= {n_seq}, {H * d}]")
+    _check_pages("attn", k_pages, v_pages, torch.bfloat16, G, d)
+    _dev("attn.page_table", page_table, torch.int32, 2)
+    if max_splits > 1:
+        _dev("attn.partial", partial, torch.float32)
+        if partial.numel() < n_seq * H * max_splits * (d + 2):
+            raise KernelError("attn_decode_rope: the partial buffer is too small")
+    if pages_per_chunk < 1 or max_splits < 1:
+        raise KernelError(f"attn_decode_rope: {pages_per_chunk} pages a chunk, {max_splits} chunks a sequence")
+    _i32("attn.chunk_list", chunk_list, 8 * n_chunks)
+    _i32("attn.seq_pos0", seq_pos0, n_seq)
+    _i32("attn.tok_page", tok_page, n_seq)
+    if cos is not None:
+        _dev("rope.cos", cos, torch.float32, 2)
+        _dev("rope.sin", sin, torch.float32, 2)
+        if cos.shape[1] != d // 2 or sin.shape != cos.shape:
+            raise KernelError(f"rope: tables {tuple(cos.shape)} do not have d/2 = {d // 2} columns")
+    _check(lib().picolm_attn_decode_rope_mfma(
+        _ptr(qkv), _ptr(k_pages), _ptr(v_pages), _ptr(out), _ptr(partial if max_splits > 1 else None), n_seq,
+        _ptr(chunk_list), n_chunks, pages_per_chunk, max_splits, _ptr(seq_pos0), _ptr(page_table),
+        page_table.shape[1], ring_pages, H, G, d, window, c_float(scale), _ptr(cos), _ptr(sin), style, _ptr(tok_page),
+        _stream()))
 
 
 def attn_prefill(q, k_pages, v_pages, out, batch, page_table, ring_pages, H, G, d, window, scale) -> None:

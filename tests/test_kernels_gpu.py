@@ -337,6 +337,57 @@ def test_attention_decode_many_sequences(d, pages_per_chunk):
     assert err <= tol(torch.bfloat16, np.abs(ref).max()), err
 
 
+@pytest.mark.parametrize("H,G,d", [(6, 6, 32), (8, 2, 64), (32, 8, 128), (40, 1, 64)])
+@pytest.mark.parametrize("style", ["pairwise", "half", None])
+@pytest.mark.parametrize("pages_per_chunk,window", [(4, 0), (1, 0), (16, 0), (2, 100), (4, 1)])
+def test_attention_decode_with_rotation_and_cache_write_inside(H, G, d, style, pages_per_chunk, window):
+    """The one-launch decode step: q, k, v of the new tokens come unrotated in float; the kernel
+    must give what rotation + cache write + attention give, and leave the same rows in the cache.
+    The cache rows of the new tokens hold NaN beforehand: they must not be read.  Positions at the
+    start of a sequence, at a page's first and last row, and deep into a sequence."""
+    pos0 = [0, 63, 64, 700, 129, 31, 32]
+    n = len(pos0)
+    case = PagedCase(H, G, d, pos0, [1] * n, torch.bfloat16, seed=H + d + pages_per_chunk)
+    b = case.batch()
+    rng = np.random.default_rng(7)
+    qkv = rng.standard_normal((n, (H + 2 * G) * d)).astype(np.float32)
+    inv = P.rope_inv_freq(d, 10000.0)
+    cos, sin = P.rope_tables(np.arange(800), inv)
+    x = qkv.astype(np.float64).reshape(n, H + 2 * G, d)
+    if style is None:
+        q_ref, k_ref = x[:, :H], x[:, H:H + G]
+    else:
+        c, s = P.rope_tables(np.asarray(pos0), inv)
+        q_ref, k_ref = P.apply_rope(x[:, :H], c, s, style), P.apply_rope(x[:, H:H + G], c, s, style)
+    v_ref = x[:, H + G:]
+    bf = lambda t: torch.from_numpy(np.ascontiguousarray(t)).to(torch.bfloat16)
+    # the reference: the paged case with its last key and value replaced by the new token's
+    for i in range(n):
+        case.q[i][-1] = bf(q_ref[i]).double().numpy()
+        case.k[i][-1] = bf(k_ref[i]).double().numpy()
+        case.v[i][-1] = bf(v_ref[i]).double().numpy()
+    ref = case.reference(window)
+    # poison the new tokens' cache rows
+    tok_page = b.write_pages(0, case.table_host, case.table_host.shape[1])
+    for i in range(n):
+        pg, row = int(tok_page[i]), pos0[i] % PAGE
+        case.k_pages[pg, :, row, :] = float("nan")
+        case.v_pages[pg, :, :, row] = float("nan")
+    out = torch.zeros(n, H * d, dtype=torch.bfloat16, device=DEV)
+    chunk_list, n_chunks, most = decode_work_list(case, window, pages_per_chunk, spare=1)
+    partial = torch.full((n * H * most * (d + 2),), float("nan"), device=DEV)
+    dev = lambda t: None if style is None else torch.from_numpy(t).float().to(DEV)
+    K().attn_decode_rope(torch.from_numpy(qkv).to(DEV), case.k_pages, case.v_pages, out, partial, n, chunk_list, n_chunks,
+                         pages_per_chunk, most, b.seq_pos0, case.table, case.table.shape[1], H, G, d, window,
+                         1.0 / math.sqrt(d), dev(cos), dev(sin), 0 if style != "half" else 1, tok_page)
+    err = np.abs(out.double().cpu().numpy() - ref).max()
+    assert err <= tol(torch.bfloat16, np.abs(ref).max()), err
+    for i in range(n):
+        pg, row = int(tok_page[i]), pos0[i] % PAGE
+        assert torch.equal(case.k_pages[pg, :, row, :].cpu(), bf(k_ref[i]))
+        assert torch.equal(case.v_pages[pg, :, :, row].cpu(), bf(v_ref[i]))
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_attention_finds_a_far_key(dtype):
     """One key among hundreds is made to dominate: the output must be its value row.  A kernel
