@@ -53,9 +53,10 @@ int picolm_attn_prefill_generic(const void* q, const void* k_pages, const void* 
                                 const int32_t* seq_nnew, const int32_t* cu_seqlens,
                                 const int32_t* page_table, int max_pages, int ring_pages, int H,
                                 int G, int d, int window, float scale, hipStream_t stream);
-// Decode (row i of q and out is sequence i): workgroup x of the launch takes entry x of the
-// step's work list, eight ints: {sequence or -1 for nothing, which chunk of the sequence, position
-// of the new token, cache slot, physical pages of the chunk's first four pages}.  A chunk is
+// Decode (row i of q and out is sequence i).  chunk_list is the step's work list of 1 + n_chunks
+// entries of eight ints: a header whose first int says how many entries are in use, then
+// {sequence, which chunk of the sequence, position of the new token, cache slot, physical pages of
+// the chunk's first four pages}; workgroup x of the launch takes entry 1 + x.  A chunk is
 // pages_per_chunk pages; a sequence has at most max_splits chunks, and where it has several their
 // partial results (partial: [n_seq][H][max_splits][d+2] floats) are combined by a merge kernel
 // that follows.
@@ -74,6 +75,7 @@ int picolm_attn_prefill_mfma(const void* q, const void* k_pages, const void* v_p
                              const int32_t* seq_slot, const int32_t* seq_pos0, const int32_t* seq_nnew,
                              const int32_t* cu_seqlens, const int32_t* page_table, int max_pages,
                              int ring_pages, int H, int G, int d, int window, float scale, hipStream_t stream);
+int picolm_attn_decode_mfma_waves(int n_seq, int H, int G);      // waves a decode workgroup will have
 int picolm_attn_decode_mfma(const void* q, const void* k_pages, const void* v_pages, void* out, float* partial,
                             int n_seq, const int32_t* chunk_list, int n_chunks, int pages_per_chunk,
                             int max_splits, const int32_t* seq_pos0, const int32_t* page_table, int max_pages,

@@ -21,8 +21,9 @@ struct AttnArgs {
     int H, G, d, window;
     float scale;
     int decode;     // 0 prefill tiles, 1 decode groups
-    // decode: workgroup x takes entry x of the step's work list, eight ints each:
-    // {sequence or -1, which chunk of the sequence, position of the new token, cache slot,
+    // decode: the step's work list, eight ints an entry.  Entry 0 is a header whose first int is
+    // the number of entries in use; workgroup x takes entry 1 + x if x is below that number:
+    // {sequence, which chunk of the sequence, position of the new token, cache slot,
     //  physical pages of the chunk's first four pages (-1 past its end)}
     const int32_t* chunk_list;
     int pages_per_chunk;
@@ -49,11 +50,17 @@ struct DecodeWork {
 __device__ __forceinline__ int decode_first_page(int window, int qpos) {
     return (window > 0 ? max(0, qpos - window + 1) : 0) / 64;
 }
-__device__ __forceinline__ bool decode_work(const AttnArgs& a, DecodeWork& w) {
-    const int4* e = (const int4*)a.chunk_list + 2 * (size_t)blockIdx.x;
+// The decode grid is one-dimensional: workgroup b takes entry b / per_entry and is number
+// b % per_entry (KV group, chunk of heads) of that entry's workgroups, so that all workgroups of
+// entries in use are handed out before those that find nothing to do.
+__device__ __forceinline__ bool decode_work(const AttnArgs& a, int per_entry, DecodeWork& w, int& which) {
+    const int entry = blockIdx.x / per_entry;
+    which = blockIdx.x % per_entry;
+    // the count is one scalar load for the whole workgroup: those past it leave at once
+    if (entry >= a.chunk_list[0]) return false;
+    const int4* e = (const int4*)a.chunk_list + 2 * ((size_t)entry + 1);
     const int4 e0 = e[0], e1 = e[1];
     w.seq = e0.x;
-    if (w.seq < 0) return false;
     w.split = e0.y;
     w.qpos = e0.z;
     w.slot = e0.w;

@@ -36,12 +36,13 @@ __global__ __launch_bounds__(AT_THREADS) void attn_tile_kernel(AttnArgs a) {
     int seq, g, split = 0, n_rows;
     DecodeWork work = {};
     if (a.decode) {
-        if (!decode_work(a, work)) return;
+        const int chunks = (R + AT_ROWS - 1) / AT_ROWS;
+        int which;
+        if (!decode_work(a, a.G * chunks, work, which)) return;
         seq = work.seq;
         split = work.split;
-        const int chunks = (R + AT_ROWS - 1) / AT_ROWS;
-        g = blockIdx.y / chunks;
-        const int chunk = blockIdx.y % chunks;
+        g = which / chunks;
+        const int chunk = which % chunks;
         n_rows = min(AT_ROWS, R - chunk * AT_ROWS);
         if (tid < AT_ROWS) {
             row_tok[tid] = seq;
@@ -314,11 +315,11 @@ extern "C" int picolm_attn_decode_generic(const void* q, const void* k_pages, co
     PICOLM_REQUIRE(dt == PICOLM_F32 || dt == PICOLM_BF16, "attn_decode: unknown dtype %d", dt);
     if (n_seq <= 0 || n_chunks <= 0) return 0;
     const int chunks = ceil_div(H / G, AT_ROWS);
-    PICOLM_REQUIRE(G * chunks <= 65535, "attn_decode: %d groups exceed the grid", G * chunks);
+    PICOLM_REQUIRE((int64_t)n_chunks * G * chunks < (1ll << 31), "attn_decode: %d chunks of %d workgroups exceed the grid", n_chunks, G * chunks);
     AttnArgs a = {q, k_pages, v_pages, out, partial, nullptr, nullptr, nullptr, seq_pos0, nullptr, nullptr,
                   page_table, max_pages, ring_pages, H, G, d, window, scale, 1, chunk_list, pages_per_chunk, max_splits,
                   nullptr, nullptr, nullptr, nullptr, 0};
-    dim3 grid(n_chunks, G * chunks);
+    dim3 grid(n_chunks * G * chunks);
     const int rc = dt == PICOLM_F32 ? launch_attn<float>(a, grid, stream) : launch_attn<bf16_t>(a, grid, stream);
     if (rc) return rc;
     return max_splits > 1 ? picolm_attn_merge_launch(a, dt, n_seq, stream) : 0;

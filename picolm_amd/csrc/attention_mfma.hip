@@ -351,9 +351,10 @@ __global__ __launch_bounds__(DEC_WAVES * 64) __attribute__((amdgpu_waves_per_eu(
     const int R = a.H / a.G;
     const int chunks = (R + 31) / 32;
     DecodeWork work;
-    if (!decode_work(a, work)) return;
+    int which;
+    if (!decode_work(a, a.G * chunks, work, which)) return;
     const int seq = work.seq, split = work.split;
-    const int g = blockIdx.y / chunks, chunk = blockIdx.y % chunks;
+    const int g = which / chunks, chunk = which % chunks;
     const int Rc = min(32, R - chunk * 32);
     const bool q_ok = l32 < Rc;
     const int head = g * R + chunk * 32 + (q_ok ? l32 : 0);
@@ -561,11 +562,18 @@ int check_decode_chunks(const char* who, const float* partial, const int32_t* ch
                         int pages_per_chunk, int max_splits);
 int picolm_attn_merge_launch(const AttnArgs& a, int dt, int n_seq, hipStream_t stream);
 
+// waves of a decode workgroup: eight give a short step for a few sequences; with many sequences
+// four waves, two workgroups a CU, move more bytes
+extern "C" int picolm_attn_decode_mfma_waves(int n_seq, int H, int G) {
+    const int chunks = ceil_div(H / (G > 0 ? G : 1), 32);
+    return (int64_t)n_seq * G * chunks >= 256 ? 4 : 8;
+}
+
 static int launch_decode_mfma(const AttnArgs& a, int n_seq, int n_chunks, hipStream_t stream) {
     const int R = a.H / a.G, chunks = ceil_div(R, 32), d = a.d;
-    PICOLM_REQUIRE(a.G * chunks <= 65535, "attn_decode_mfma: %d groups exceed the grid", a.G * chunks);
-    const int waves = (int64_t)n_seq * a.G * chunks >= 256 ? 4 : 8;
-    dim3 grid(n_chunks, a.G * chunks), block(waves * 64);
+    PICOLM_REQUIRE((int64_t)n_chunks * a.G * chunks < (1ll << 31), "attn_decode_mfma: %d chunks of %d workgroups exceed the grid", n_chunks, a.G * chunks);
+    const int waves = picolm_attn_decode_mfma_waves(n_seq, a.H, a.G);
+    dim3 grid(n_chunks * a.G * chunks), block(waves * 64);
     const size_t lds = sizeof(float) * ((waves + 1) * (size_t)min(R, 32) * (d + 2) + 2 * d);
 #define DEC_LAUNCH(D, W)                                                                                    \
     {                                                                                                       \

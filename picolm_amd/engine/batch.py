@@ -20,7 +20,7 @@ class StepError(ValueError):
 
 
 class StepBatch:
-    def __init__(self, slots, pos0, new_tokens, want, vocab_size: int, device, target_blocks: int = 512):
+    def __init__(self, slots, pos0, new_tokens, want, vocab_size: int, device):
         """slots[i]: cache slot of sequence i; pos0[i]: tokens it holds; new_tokens[i]: its
         next tokens; want[i]: indices into new_tokens[i] whose logits are asked for."""
         self.n_seq = len(slots)
@@ -40,7 +40,6 @@ class StepBatch:
         self.T = sum(n_new)
         self.is_decode = self.max_new == 1
         self.max_len = max(p + n for p, n in zip(self.pos0, n_new))
-        self._target_blocks = target_blocks
 
         cu = np.zeros(self.n_seq + 1, dtype=np.int32)
         cu[1:] = np.cumsum(n_new)
@@ -122,14 +121,17 @@ class StepBatch:
             self._write_pages[group] = torch.from_numpy(pages).to(self._device)
         return self._write_pages[group]
 
-    def decode_chunks(self, blocks_per_chunk: int, window: int, group: int, table_host, ring_pages: int):
+    def decode_chunks(self, blocks_per_chunk: int, max_pages_per_chunk: int, window: int, group: int, table_host,
+                      ring_pages: int):
         """The decode attention's work list for this step over one cache group's pages:
-        (entries on the device, number of entries, pages_per_chunk, most chunks of a sequence)."""
-        key = (blocks_per_chunk, window, group)
+        (header and entries on the device, number of entries, pages_per_chunk, most chunks of a
+        sequence)."""
+        key = (blocks_per_chunk, max_pages_per_chunk, window, group)
         if key not in self._chunks:
-            ppc = decode_pages_per_chunk(self.pos0, blocks_per_chunk, self._target_blocks)
+            ppc = decode_pages_per_chunk(self.pos0, blocks_per_chunk, max_pages_per_chunk)
             entries, most = decode_chunk_list(self.slots, self.pos0, window, ppc, table_host, ring_pages)
-            self._chunks[key] = (torch.from_numpy(entries).to(self._device), len(entries), ppc, most)
+            self._chunks[key] = (torch.from_numpy(with_header(entries, len(entries))).to(self._device), len(entries),
+                                 ppc, most)
         return self._chunks[key]
 
 
@@ -139,13 +141,26 @@ def token_pages(tok_seq, tok_pos, slots, table_host, ring_pages: int):
     return table[slot, (np.asarray(tok_pos, dtype=np.int64) // PAGE_TOKENS) % ring_pages].astype(np.int32)
 
 
-def decode_pages_per_chunk(pos0, blocks_per_chunk: int, target_blocks: int = 512) -> int:
-    """Pages that one workgroup of the decode attention takes: a power of two, at least one
-    page for each of its four waves, and more when the step would otherwise have far more
-    than `target_blocks` workgroups (a few for every CU)."""
-    total_pages = sum(int(p) // PAGE_TOKENS + 1 for p in pos0)
-    want = total_pages * max(1, blocks_per_chunk) // max(1, target_blocks)
-    return max(4, 1 << (max(want, 1).bit_length() - 1))
+def decode_pages_per_chunk(pos0, blocks_per_chunk: int, max_pages_per_chunk: int = 16, min_blocks: int = 160) -> int:
+    """Pages that one workgroup of the decode attention takes: the largest of 4, 8, 16 within
+    `max_pages_per_chunk` (a wave should not walk over more than about four tiles one after the
+    other) that still leaves `min_blocks` workgroups for the launch, which is most of the CUs;
+    4 (a page for each of four waves) if none does.  Fewer, larger chunks mean fewer partial
+    results to merge."""
+    pages = [int(p) // PAGE_TOKENS + 1 for p in pos0]
+    for ppc in (16, 8):
+        if ppc <= max_pages_per_chunk and sum((n + ppc - 1) // ppc for n in pages) * max(1, blocks_per_chunk) >= min_blocks:
+            return ppc
+    return 4
+
+
+def with_header(entries, n_live: int):
+    """The work list as the kernels read it: a header entry whose first int is the number of
+    entries in use, then the entries."""
+    out = np.zeros((len(entries) + 1, CHUNK_ENTRY_INTS), dtype=np.int32)
+    out[0, 0] = n_live
+    out[1:] = entries
+    return out
 
 
 CHUNK_ENTRY_INTS = 8
@@ -275,22 +290,24 @@ class DecodeBatch:
         if n_most > most:
             raise StepError(f"a sequence of {max(self.pos0) + 1} tokens has more pages than the cache was sized for")
         h = host.numpy().reshape(-1, CHUNK_ENTRY_INTS)
-        h[:len(entries)] = entries
-        h[len(entries):, 0] = -1        # workgroups of unused entries leave at once
+        h[0, 0] = len(entries)          # workgroups past this count leave at once
+        h[1:1 + len(entries)] = entries
         dev.copy_(host, non_blocking=False)
 
-    def decode_chunks(self, blocks_per_chunk: int, window: int, group: int, table_host, ring_pages: int):
+    def decode_chunks(self, blocks_per_chunk: int, max_pages_per_chunk: int, window: int, group: int, table_host,
+                      ring_pages: int):
         """As StepBatch.decode_chunks, over a list of fixed capacity (every sequence at the
-        cache's full length) that `fill` rewrites in place."""
+        cache's full length) that `fill` rewrites in place; the chunk size was chosen when the
+        batch was made."""
         key = (window, group)
         if key not in self._lists:
             if self.frozen:
                 raise StepError("a recorded decode step cannot take another work list")
             most = (table_host.shape[1] + self.pages_per_chunk - 1) // self.pages_per_chunk
             cap = self.n_seq * most
-            self._lists[key] = (self._host_block(cap * CHUNK_ENTRY_INTS),
-                                torch.zeros(cap * CHUNK_ENTRY_INTS, dtype=torch.int32, device=self._device), most,
+            self._lists[key] = (self._host_block((cap + 1) * CHUNK_ENTRY_INTS),
+                                torch.zeros((cap + 1) * CHUNK_ENTRY_INTS, dtype=torch.int32, device=self._device), most,
                                 table_host, ring_pages)
             self._fill_list(key)
         host, dev, most, _, _ = self._lists[key]
-        return dev, len(host) // CHUNK_ENTRY_INTS, self.pages_per_chunk, most
+        return dev, len(host) // CHUNK_ENTRY_INTS - 1, self.pages_per_chunk, most

@@ -97,14 +97,16 @@ class DecoderModel:
             return getattr(p, "graph_safe", False) and all(safe(c) for c in p.children())
         return all(safe(p) for p in self.parts())
 
-    def decode_blocks_per_seq(self) -> int:
-        """Workgroups per sequence of the widest decode attention launch (for split sizing)."""
-        out = 1
+    def decode_geometry(self, n_seq: int) -> tuple[int, int]:
+        """(workgroups per chunk, most pages a chunk should have) over the mixers that run a
+        decode attention: the widest launch and the tightest limit size the step's work list."""
+        per_chunk, max_pages = 1, 16
         for b in self.blocks:
-            m = b.mixer
-            if hasattr(m, "G") and hasattr(m, "H"):
-                out = max(out, m.G * ((m.H // m.G + 15) // 16))
-        return out
+            f = getattr(b.mixer, "decode_geometry", None)
+            if f is not None:
+                p, m = f(self.runtime.dtype, n_seq)
+                per_chunk, max_pages = max(per_chunk, p), min(max_pages, m)
+        return per_chunk, max_pages
 
     # -- weights ----------------------------------------------------------------------------
     def load(self, source, runtime: Runtime) -> "DecoderModel":

@@ -65,7 +65,6 @@ class Session:
         # memory only (a part says so with `graph_safe`)
         self.graphs = graphs and model.graph_safe()
         self._decode_graphs: dict[tuple, _DecodeGraph] = {}
-        self._blocks_per_seq = model.decode_blocks_per_seq()
 
     # -- slots -------------------------------------------------------------------------------
     def begin(self, n: int = 1) -> list[int]:
@@ -120,7 +119,7 @@ class Session:
                 raise StepError(f"token id {t} is outside the vocabulary of {self.vocab_size}")
         self.cache.reserve_many(slots, [p + 1 for p in pos0])
         self.cache.flush()
-        ppc = decode_pages_per_chunk(pos0, self._blocks_per_seq)
+        ppc = decode_pages_per_chunk(pos0, *self.model.decode_geometry(len(slots)))
         key = (len(slots), ppc)
         g = self._decode_graphs.get(key)
         if g is None:

@@ -44,7 +44,7 @@ def dir_entry_points():
             "picolm_attn_prefill_tile_rows", "picolm_attn_prefill_generic",
             "picolm_attn_decode_generic", "picolm_argmax", "picolm_argmax_scratch_floats", "picolm_sample", "picolm_gemm_skinny", "picolm_gemm_tiled", "picolm_gemm_tiled_splitk",
             "picolm_attn_mfma_takes", "picolm_attn_prefill_mfma_heads", "picolm_attn_prefill_mfma_tile_tokens",
-            "picolm_attn_prefill_mfma", "picolm_attn_decode_mfma", "picolm_attn_decode_rope_mfma", "picolm_read_probe", "picolm_mfma_probe"]
+            "picolm_attn_prefill_mfma", "picolm_attn_decode_mfma", "picolm_attn_decode_rope_mfma", "picolm_attn_decode_mfma_waves", "picolm_read_probe", "picolm_mfma_probe"]
 
 
 def _check(rc: int) -> None:
@@ -226,8 +226,18 @@ def _decode_check(q, partial, n_seq, chunk_list, n_chunks, pages_per_chunk, max_
         raise KernelError("attn_decode: fewer query rows than sequences")
     if pages_per_chunk < 1 or max_splits < 1:
         raise KernelError(f"attn_decode: {pages_per_chunk} pages a chunk, {max_splits} chunks a sequence")
-    _i32("attn.chunk_list", chunk_list, 8 * n_chunks)
+    _i32("attn.chunk_list", chunk_list, 8 * (n_chunks + 1))
     _i32("attn.seq_pos0", seq_pos0, n_seq)
+
+
+def attn_decode_geometry(dtype: torch.dtype, n_seq: int, H: int, G: int, d: int) -> tuple[int, int]:
+    """(workgroups per chunk of the work list, the most pages a chunk should have) of the decode
+    attention kernel that will run for these sizes."""
+    R = H // G
+    if attn_decode_rope_takes(dtype, d):
+        waves = lib().picolm_attn_decode_mfma_waves(n_seq, H, G)
+        return G * ((R + 31) // 32), 2 * waves        # up to four tiles of 32 keys a wave
+    return G * ((R + 15) // 16), 16
 
 
 def attn_decode_generic(q, k_pages, v_pages, out, partial, n_seq, chunk_list, n_chunks, pages_per_chunk,
@@ -394,7 +404,7 @@ def attn_decode_rope(qkv, k_pages, v_pages, out, partial, n_seq, chunk_list, n_c
             raise KernelError("attn_decode_rope: the partial buffer is too small")
     if pages_per_chunk < 1 or max_splits < 1:
         raise KernelError(f"attn_decode_rope: {pages_per_chunk} pages a chunk, {max_splits} chunks a sequence")
-    _i32("attn.chunk_list", chunk_list, 8 * n_chunks)
+    _i32("attn.chunk_list", chunk_list, 8 * (n_chunks + 1))
     _i32("attn.seq_pos0", seq_pos0, n_seq)
     _i32("attn.tok_page", tok_page, n_seq)
     if cos is not None:
@@ -422,8 +432,8 @@ def attn_prefill(q, k_pages, v_pages, out, batch, page_table, ring_pages, H, G, 
 def attn_decode(q, k_pages, v_pages, out, partial, n_seq, chunk_list, n_chunks, pages_per_chunk, max_splits,
                 seq_pos0, page_table, ring_pages, H, G, d, window, scale) -> None:
     """Attention of one new token per sequence (row i of q is sequence i) over its cache pages.
-    `chunk_list` is the step's work list, eight ints an entry: entry x gives workgroup x
-    `pages_per_chunk` pages of one sequence."""
+    `chunk_list` is the step's work list, eight ints an entry behind a header entry: entry 1 + x
+    gives workgroup x `pages_per_chunk` pages of one sequence."""
     fn = attn_decode_mfma if attn_mfma_takes(q, d) else attn_decode_generic
     fn(q, k_pages, v_pages, out, partial, n_seq, chunk_list, n_chunks, pages_per_chunk, max_splits, seq_pos0,
        page_table, ring_pages, H, G, d, window, scale)

@@ -43,6 +43,11 @@ class Attention(Mixer):
     def cache_requests(self):
         return KVRequest(self.G, self.d, self.window), None
 
+    def decode_geometry(self, dtype, n_seq: int):
+        """(workgroups per chunk, most pages a chunk should have) of this layer's decode
+        attention: what sizes the step's work list."""
+        return kernels.attn_decode_geometry(dtype, n_seq, self.H, self.G, self.d)
+
     def prepare(self, runtime: Runtime, max_positions: int) -> None:
         self.position.prepare(runtime, max_positions)
 
@@ -67,8 +72,8 @@ class Attention(Mixer):
         group, table_host = ctx.kv_host()
         tok_page = b.write_pages(group, table_host, ring) if writes else None
         if b.is_decode:
-            chunk_list, n_chunks, ppc, most = b.decode_chunks(G * ((H // G + 15) // 16), self.window, group,
-                                                               table_host, ring)
+            chunk_list, n_chunks, ppc, most = b.decode_chunks(*self.decode_geometry(ctx.dtype, b.n_seq), self.window,
+                                                               group, table_host, ring)
             partial = ctx.ws.get("attn.partial", (b.n_seq * H * most * (d + 2),), torch.float32) if most > 1 else None
             if writes and kernels.attn_decode_rope_takes(ctx.dtype, d):
                 # rotation (if the position encoding is one), cache write and attention in one launch

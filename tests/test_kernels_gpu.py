@@ -287,16 +287,16 @@ def test_attention_prefill(dtype, H, G, d, window):
 
 
 def decode_work_list(case, window, pages_per_chunk, spare=0):
-    """The work list the engine would build, with `spare` unused entries mixed in."""
-    from picolm_amd.engine.batch import decode_chunk_list
+    """The work list the engine would build, with room for `spare` more entries behind it (a
+    recorded step's list has room for full-length sequences): those hold garbage."""
+    from picolm_amd.engine.batch import decode_chunk_list, with_header
     b = case.batch()
     entries, most = decode_chunk_list(b.slots, b.pos0, window, pages_per_chunk, case.table_host,
                                       case.table_host.shape[1])
+    n_live = len(entries)
     if spare:
-        unused = np.full((spare, 8), 7, np.int32)
-        unused[:, 0] = -1
-        entries = np.concatenate([entries[:1], unused, entries[1:], unused])
-    return torch.from_numpy(entries).to(DEV), len(entries), most
+        entries = np.concatenate([entries, np.full((spare, 8), 12345, np.int32)])
+    return torch.from_numpy(with_header(entries, n_live)).to(DEV), len(entries), most
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])

@@ -55,11 +55,12 @@ def test_work_list_of_a_ring():
 
 
 def test_pages_per_chunk_grows_with_the_work():
-    assert decode_pages_per_chunk([100], 8) == 4
-    assert decode_pages_per_chunk([1000] * 8, 8) == 4
-    big = decode_pages_per_chunk([4095] * 64, 8)
-    assert big > 4 and big & (big - 1) == 0
-    assert decode_pages_per_chunk([4095] * 64, 8, target_blocks=10 ** 9) == 4
+    assert decode_pages_per_chunk([100], 8) == 4                       # too little work for larger chunks
+    assert decode_pages_per_chunk([1100] * 8, 8) == 8                  # 18 pages each: 3 chunks of 8 x 8 x 8 = 192 workgroups
+    assert decode_pages_per_chunk([4095] * 8, 8) == 16
+    assert decode_pages_per_chunk([4095] * 8, 8, max_pages_per_chunk=8) == 8
+    assert decode_pages_per_chunk([1100] * 64, 8, max_pages_per_chunk=8) == 8
+    assert decode_pages_per_chunk([4095] * 64, 8, min_blocks=10 ** 9) == 4
 
 
 def test_step_batch_packs_without_padding():
@@ -92,10 +93,11 @@ def test_decode_batch_rewrites_its_lists_in_place():
     table = torch.arange(4 * 16, dtype=torch.int32).reshape(4, 16)
     b = DecodeBatch(3, 4, "cpu")
     b.fill([2, 0, 1], [10, 300, 64], [1, 2, 3])
-    dev, cap, ppc, most = b.decode_chunks(8, 0, 0, table, 16)
+    dev, cap, ppc, most = b.decode_chunks(8, 16, 0, 0, table, 16)
     assert cap == 3 * 4 and ppc == 4 and most == 4
-    rows = dev.reshape(-1, 8)
-    assert rows[:, 0].tolist() == [0, 1, 1, 2] + [-1] * 8
+    assert dev.reshape(-1, 8)[0, 0] == 4                    # the header: entries in use
+    rows = dev.reshape(-1, 8)[1:]
+    assert rows[:4, 0].tolist() == [0, 1, 1, 2]
     assert rows[:4, 1].tolist() == [0, 0, 1, 0]
     assert rows[:4, 2].tolist() == [10, 300, 300, 64]
     assert rows[:4, 3].tolist() == [2, 0, 0, 1]
@@ -103,14 +105,15 @@ def test_decode_batch_rewrites_its_lists_in_place():
     assert rows[0, 4:].tolist() == [32, -1, -1, -1]
     addr = dev.data_ptr()
     b.fill([2, 0, 1], [1000, 301, 65], [1, 2, 3])
-    dev2, *_ = b.decode_chunks(8, 0, 0, table, 16)
+    dev2, *_ = b.decode_chunks(8, 16, 0, 0, table, 16)
     assert dev2.data_ptr() == addr
-    rows = dev2.reshape(-1, 8)
-    assert rows[:, 0].tolist() == [0, 0, 0, 0, 1, 1, 2] + [-1] * 5
+    assert dev2.reshape(-1, 8)[0, 0] == 7
+    rows = dev2.reshape(-1, 8)[1:]
+    assert rows[:7, 0].tolist() == [0, 0, 0, 0, 1, 1, 2]
     assert rows[:7, 1].tolist() == [0, 1, 2, 3, 0, 1, 0]
     # a windowed layer, or another cache group, has a list of its own
-    wdev, *_ = b.decode_chunks(8, 64, 0, table, 16)
-    assert wdev.reshape(-1, 8)[:4, 0].tolist() == [0, 1, 2, -1]
+    wdev, *_ = b.decode_chunks(8, 16, 64, 0, table, 16)
+    assert wdev.reshape(-1, 8)[0, 0] == 3 and wdev.reshape(-1, 8)[1:4, 0].tolist() == [0, 1, 2]
     pages = b.write_pages(0, table, 16)
     assert pages.tolist() == [32 + 15, 4, 16 + 1]          # positions 1000, 301, 65 of slots 2, 0, 1
     b.fill([2, 0, 1], [64, 0, 128], [1, 2, 3])
@@ -119,4 +122,4 @@ def test_decode_batch_rewrites_its_lists_in_place():
         b.fill([2, 0, 1], [1024, 0, 0], [1, 2, 3])       # 17 pages in a cache of 16
     b.frozen = True
     with pytest.raises(StepError):
-        b.decode_chunks(8, 128, 0, table, 16)
+        b.decode_chunks(8, 16, 128, 0, table, 16)
