@@ -859,8 +859,8 @@ static int launch_splitk_reduce(const float* ws, void* C, int c_dt, int M, int N
 // variant 0 picks by shape.  Tiles loaded straight into LDS (K a multiple of 64):
 //   9: 256x256, 8 waves, two stages of 64 columns;  10: 256(n)x128(m), 8 waves, three stages;
 //   11: 128x128, 4 waves, four stages;
-//   12: 128(n)x64(m), 4 waves, three stages: for decode batches of up to 64 rows, where the
-//   weights stream once and K may be split.
+//   12: 128(n)x64(m), 4 waves, three stages;  13: 128(n)x32(m), 4 waves, four stages: for decode
+//   batches of up to 64 or 32 rows, where the weights stream once and K may be split.
 // Tiles staged through registers (any K that is a multiple of 8):
 //   1: 128x128 (4 waves), 4: 256x256 (8 waves).
 extern "C" int picolm_gemm_tiled(const void* A, const void* W, void* C, int c_dt, int M, int N, int K,
@@ -901,6 +901,7 @@ extern "C" int picolm_gemm_tiled(const void* A, const void* W, void* C, int c_dt
         case 10: return launch_direct<2, 2, 4, 2, 64, 3>(A, W, C, c_dt, M, N, K, lda, ldw, ldc, epilogue, stream);
         case 11: return launch_direct<2, 2, 2, 2, 64, 4>(A, W, C, c_dt, M, N, K, lda, ldw, ldc, epilogue, stream);
         case 12: return launch_direct<1, 2, 4, 1, 64, 3>(A, W, C, c_dt, M, N, K, lda, ldw, ldc, epilogue, stream);
+        case 13: return launch_direct<1, 1, 4, 1, 64, 4>(A, W, C, c_dt, M, N, K, lda, ldw, ldc, epilogue, stream);
     }
     PICOLM_REQUIRE(false, "gemm_tiled: unknown variant %d", variant);
 }
@@ -923,6 +924,7 @@ extern "C" int picolm_gemm_tiled_splitk(const void* A, const void* W, void* C, i
         case 10: rc = launch_direct<2, 2, 4, 2, 64, 3>(A, W, ws, PICOLM_F32, M, N, K, lda, ldw, N, 0, stream, splits, stride); break;
         case 11: rc = launch_direct<2, 2, 2, 2, 64, 4>(A, W, ws, PICOLM_F32, M, N, K, lda, ldw, N, 0, stream, splits, stride); break;
         case 12: rc = launch_direct<1, 2, 4, 1, 64, 3>(A, W, ws, PICOLM_F32, M, N, K, lda, ldw, N, 0, stream, splits, stride); break;
+        case 13: rc = launch_direct<1, 1, 4, 1, 64, 4>(A, W, ws, PICOLM_F32, M, N, K, lda, ldw, N, 0, stream, splits, stride); break;
         default: PICOLM_REQUIRE(false, "gemm_splitk: variant %d cannot split K", variant);
     }
     if (rc) return rc;

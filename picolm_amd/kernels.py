@@ -351,6 +351,10 @@ def gemm(a: torch.Tensor, w: torch.Tensor, c: torch.Tensor, epilogue: int = EPI_
             # a decode batch too wide to re-read its activations for every 16 weight rows: tiles
             # of 128 weight rows through LDS, cut along K where there are few of them
             gemm_tiled_splitk(a, w, c, epilogue, 12, medium_gemm_splits(M, N, K))
+        elif M > 4 and K % 64 == 0 and 16384 <= N <= 128 * 256:
+            # several rows and one round of 128-row tiles for the CUs: the tiles share the
+            # activations through LDS (more rounds suit the skinny kernel's resident variant better)
+            gemm_tiled_splitk(a, w, c, epilogue, 13, 1)
         else:
             gemm_skinny(a, w, c, epilogue)
     else:

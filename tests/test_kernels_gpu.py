@@ -141,7 +141,7 @@ def test_gemm_skinny_resident_activations(M):
         run_gemm(K().gemm_skinny, M, 64, 1032, 0, torch.bfloat16, torch.bfloat16, torch.float32, variant=7)
 
 
-@pytest.mark.parametrize("variant,splits", [(12, 2), (12, 8), (11, 4), (9, 3)])
+@pytest.mark.parametrize("variant,splits", [(12, 2), (12, 8), (13, 4), (11, 4), (9, 3)])
 def test_gemm_tiled_split_along_k(variant, splits):
     """K cut into parts whose partial sums a second kernel adds in order: every epilogue, ragged
     M and N, and the same bits on every run."""
@@ -169,7 +169,8 @@ def test_gemm_medium_batches_pick_their_splits():
     assert medium_gemm_splits(64, 4096, 14336) == 8
     assert medium_gemm_splits(64, 4096, 64 * 3) == 1         # K does not split evenly
     assert medium_gemm_splits(33, 130, 4096) == 1            # N no multiple of 4
-    for M, N, Kd in ((64, 4096, 4096), (40, 6144, 1024), (17, 260, 192), (64, 28672 // 4, 512)):
+    for M, N, Kd in ((64, 4096, 4096), (40, 6144, 1024), (17, 260, 192), (64, 28672 // 4, 512), (8, 16384 + 2, 128),
+                     (5, 128 * 256, 64)):
         for epi, cdt in ((0, torch.float32), (2, torch.bfloat16), (1, torch.float32)):
             run_gemm(K().gemm, M, N, Kd, epi, torch.bfloat16, torch.bfloat16, cdt)
 
@@ -189,7 +190,7 @@ def test_gemm_tiled_block_tiles(variant):
             run_gemm(K().gemm_tiled, M, N, Kd, epi, torch.bfloat16, torch.bfloat16, cdt, variant=variant)
 
 
-@pytest.mark.parametrize("variant", [9, 10, 11, 12])
+@pytest.mark.parametrize("variant", [9, 10, 11, 12, 13])
 def test_gemm_tiled_direct_to_lds(variant):
     """The variants whose tiles go from global memory straight into LDS: K in whole steps of 64,
     fewer steps than stages, many steps (every stage is reused), ragged M and N."""
