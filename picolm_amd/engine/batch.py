@@ -224,7 +224,10 @@ class DecodeBatch:
     is_decode = True
     max_new = 1
 
-    def __init__(self, n_seq: int, pages_per_chunk: int, device):
+    def __init__(self, n_seq: int, pages_per_chunk: int, device, reserve_ints: int = 0):
+        """`reserve_ints`: room behind the step's arrays for the work lists and page arrays that
+        parts ask for, so that everything goes to the device in one copy; what does not fit gets
+        a block and a copy of its own."""
         self.n_seq = self.T = self.n_want = n_seq
         self.pages_per_chunk = pages_per_chunk
         self.n_new = [1] * n_seq
@@ -236,9 +239,11 @@ class DecodeBatch:
                            ("tok_seq", n), ("tokens", n), ("want_rows", n)):
             self._spans[name] = (off, size)
             off += size
+        off = (off + 3) // 4 * 4                    # what follows is read 16 bytes at a time
+        self._used, self._size = off, off + (reserve_ints + 3) // 4 * 4
         self._device = torch.device(device)
-        self._host = self._host_block(off)
-        self._dev = torch.zeros(off, dtype=torch.int32, device=device)
+        self._host = self._host_block(self._size)
+        self._dev = torch.zeros(self._size, dtype=torch.int32, device=device)
         h = self._host.numpy()
         ar = np.arange(n + 1, dtype=np.int32)
         self._np = {k: h[o:o + s] for k, (o, s) in self._spans.items()}
@@ -249,8 +254,9 @@ class DecodeBatch:
         for k, (o, s) in self._spans.items():
             setattr(self, k, self._dev[o:o + s])
         self.slots, self.pos0 = [], []
-        self._lists = {}        # (window, group) -> (host block, device block, most chunks, page table, ring)
-        self._pages = {}        # group -> (host block, device block, page table, ring)
+        self._lists = {}        # (window, group) -> (host array, device array, most chunks, page table, ring, own block or None)
+        self._pages = {}        # group -> (host array, device array, page table, ring, own block or None)
+        self._live = {}         # (window, group) -> entries in use
         self.frozen = False     # set once the launches are recorded: no further work list can join
 
     @staticmethod
@@ -258,41 +264,61 @@ class DecodeBatch:
         t = torch.zeros(n, dtype=torch.int32)
         return t.pin_memory() if torch.cuda.is_available() else t
 
+    def _region(self, n_ints: int):
+        """(host numpy view, device view, own host block or None) of n_ints more ints."""
+        n4 = (n_ints + 3) // 4 * 4
+        if self._used + n4 <= self._size:
+            o = self._used
+            self._used += n4
+            return self._host.numpy()[o:o + n_ints], self._dev[o:o + n_ints], None
+        own = self._host_block(n_ints)
+        return own.numpy(), torch.zeros(n_ints, dtype=torch.int32, device=self._device), own
+
     def fill(self, slots, pos0, tokens) -> None:
+        # between page boundaries only the positions move: the lists and pages stay as they are
+        same_pages = (list(slots) == self.slots and len(pos0) == len(self.pos0)
+                      and all(p == q + 1 and p % PAGE_TOKENS for p, q in zip(pos0, self.pos0)))
         self.slots, self.pos0 = list(slots), list(pos0)
         self._np["seq_slot"][:] = slots
         self._np["seq_pos0"][:] = pos0
         self._np["tok_pos"][:] = pos0
         self._np["tokens"][:] = tokens
-        self._dev.copy_(self._host, non_blocking=False)
         for key in self._lists:
-            self._fill_list(key)
-        for group in self._pages:
-            self._fill_pages(group)
+            if same_pages and key[0] == 0:          # (a window's first page can move on any step)
+                self._lists[key][0].reshape(-1, CHUNK_ENTRY_INTS)[1:1 + self._live[key], 2] += 1
+            else:
+                self._fill_list(key)
+        if not same_pages:
+            for group in self._pages:
+                self._fill_pages(group)
+        self._dev.copy_(self._host, non_blocking=False)
+        for host, dev, *_, own in list(self._lists.values()) + list(self._pages.values()):
+            if own is not None:
+                dev.copy_(own, non_blocking=False)
 
     def _fill_pages(self, group: int) -> None:
-        host, dev, table_host, ring_pages = self._pages[group]
-        host.numpy()[:] = token_pages(np.arange(self.n_seq), self.pos0, self.slots, table_host, ring_pages)
-        dev.copy_(host, non_blocking=False)
+        host, dev, table_host, ring_pages, own = self._pages[group]
+        host[:] = token_pages(np.arange(self.n_seq), self.pos0, self.slots, table_host, ring_pages)
 
     def write_pages(self, group: int, table_host, ring_pages: int):
         if group not in self._pages:
             if self.frozen:
                 raise StepError("a recorded decode step cannot take another cache group")
-            self._pages[group] = (self._host_block(self.n_seq), torch.zeros(self.n_seq, dtype=torch.int32, device=self._device),
-                                  table_host, ring_pages)
+            host, dev, own = self._region(self.n_seq)
+            self._pages[group] = (host, dev, table_host, ring_pages, own)
             self._fill_pages(group)
+            dev.copy_(torch.from_numpy(host), non_blocking=False)
         return self._pages[group][1]
 
     def _fill_list(self, key) -> None:
-        host, dev, most, table_host, ring_pages = self._lists[key]
+        host, dev, most, table_host, ring_pages, own = self._lists[key]
         entries, n_most = decode_chunk_list(self.slots, self.pos0, key[0], self.pages_per_chunk, table_host, ring_pages)
         if n_most > most:
             raise StepError(f"a sequence of {max(self.pos0) + 1} tokens has more pages than the cache was sized for")
-        h = host.numpy().reshape(-1, CHUNK_ENTRY_INTS)
+        h = host.reshape(-1, CHUNK_ENTRY_INTS)
         h[0, 0] = len(entries)          # workgroups past this count leave at once
         h[1:1 + len(entries)] = entries
-        dev.copy_(host, non_blocking=False)
+        self._live[key] = len(entries)
 
     def decode_chunks(self, blocks_per_chunk: int, max_pages_per_chunk: int, window: int, group: int, table_host,
                       ring_pages: int):
@@ -305,9 +331,15 @@ class DecodeBatch:
                 raise StepError("a recorded decode step cannot take another work list")
             most = (table_host.shape[1] + self.pages_per_chunk - 1) // self.pages_per_chunk
             cap = self.n_seq * most
-            self._lists[key] = (self._host_block((cap + 1) * CHUNK_ENTRY_INTS),
-                                torch.zeros((cap + 1) * CHUNK_ENTRY_INTS, dtype=torch.int32, device=self._device), most,
-                                table_host, ring_pages)
+            host, dev, own = self._region((cap + 1) * CHUNK_ENTRY_INTS)
+            self._lists[key] = (host, dev, most, table_host, ring_pages, own)
             self._fill_list(key)
-        host, dev, most, _, _ = self._lists[key]
+            dev.copy_(torch.from_numpy(host), non_blocking=False)
+        host, dev, most, *_ = self._lists[key]
         return dev, len(host) // CHUNK_ENTRY_INTS - 1, self.pages_per_chunk, most
+
+    @staticmethod
+    def ints_for(n_seq: int, pages_per_chunk: int, max_pages: int) -> int:
+        """Room that one cache group's work list and page array take (see `reserve_ints`)."""
+        most = (max_pages + pages_per_chunk - 1) // pages_per_chunk
+        return (n_seq * most + 1) * CHUNK_ENTRY_INTS + n_seq + 8

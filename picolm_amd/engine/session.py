@@ -11,6 +11,7 @@ import gc
 import torch
 
 from ..cache import Cache, CacheFull
+from ..cache.slots import PAGE_TOKENS
 from ..parts.base import Workspace
 from .batch import DecodeBatch, StepBatch, StepError, decode_pages_per_chunk
 from .model import DecoderModel
@@ -20,7 +21,8 @@ class _DecodeGraph:
     """The kernel launches of one decode step of `n_seq` sequences, recorded as a HIP graph."""
 
     def __init__(self, session: "Session", n_seq: int, pages_per_chunk: int):
-        self.batch = DecodeBatch(n_seq, pages_per_chunk, session.model.runtime.device)
+        reserve = sum(DecodeBatch.ints_for(n_seq, pages_per_chunk, g.table_host.shape[1]) for g in session.cache.kv)
+        self.batch = DecodeBatch(n_seq, pages_per_chunk, session.model.runtime.device, reserve)
         self.workspace = Workspace(session.model.runtime.device)      # its own: recorded addresses must stay
         self.graph = None
         self.logits = None
@@ -65,6 +67,7 @@ class Session:
         # memory only (a part says so with `graph_safe`)
         self.graphs = graphs and model.graph_safe()
         self._decode_graphs: dict[tuple, _DecodeGraph] = {}
+        self._decode_geometry: dict[int, tuple] = {}
 
     # -- slots -------------------------------------------------------------------------------
     def begin(self, n: int = 1) -> list[int]:
@@ -117,9 +120,14 @@ class Session:
         for t in tokens:
             if not 0 <= t < self.vocab_size:
                 raise StepError(f"token id {t} is outside the vocabulary of {self.vocab_size}")
-        self.cache.reserve_many(slots, [p + 1 for p in pos0])
-        self.cache.flush()
-        ppc = decode_pages_per_chunk(pos0, *self.model.decode_geometry(len(slots)))
+        # unless a sequence starts a page (or runs out of room), every new token stays in its sequence's last page
+        if not all(p % PAGE_TOKENS for p in pos0) or max(pos0) >= self.cache.max_seq_len:
+            self.cache.reserve_many(slots, [p + 1 for p in pos0])
+            self.cache.flush()
+        geometry = self._decode_geometry.get(len(slots))
+        if geometry is None:
+            geometry = self._decode_geometry[len(slots)] = self.model.decode_geometry(len(slots))
+        ppc = decode_pages_per_chunk(pos0, *geometry)
         key = (len(slots), ppc)
         g = self._decode_graphs.get(key)
         if g is None:

@@ -22,6 +22,10 @@ class Sampler:
         states = [_as_i64(stream_state(params.seed, i)) for i in range(n_sequences)]
         self.states = torch.tensor(states, dtype=torch.int64).to(self.device)
         self._out = torch.zeros(max(n_sequences, 1), dtype=torch.int32, device=self.device)
+        # the tokens come back through pinned memory: one copy, no staging buffer
+        self._host_out = torch.zeros(max(n_sequences, 1), dtype=torch.int32)
+        if self.device.type == "cuda":
+            self._host_out = self._host_out.pin_memory()
         self._scratch = None
 
     def sample(self, logits: torch.Tensor, sequence_indices) -> list[int]:
@@ -37,4 +41,7 @@ class Sampler:
         else:
             idx = torch.tensor(list(sequence_indices), dtype=torch.int32).to(self.device)
             kernels.sample(logits, out, p.temperature, p.top_k, p.top_p, p.min_p, self.states, idx)
-        return out.tolist()
+        host = self._host_out[:n]
+        host.copy_(out, non_blocking=True)
+        torch.cuda.current_stream().synchronize()
+        return host.tolist()

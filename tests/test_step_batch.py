@@ -123,3 +123,27 @@ def test_decode_batch_rewrites_its_lists_in_place():
     b.frozen = True
     with pytest.raises(StepError):
         b.decode_chunks(8, 16, 128, 0, table, 16)
+
+
+def test_decode_batch_between_page_boundaries_only_moves_positions():
+    """Filling step by step (the short way when no sequence starts a page) gives the same blocks
+    as filling a fresh batch; a step that starts a page rebuilds the lists."""
+    import torch
+    table = torch.from_numpy(np.random.default_rng(0).permutation(4 * 16).astype(np.int32).reshape(4, 16))
+    slots = [2, 0, 1]
+    walked = DecodeBatch(3, 4, "cpu", reserve_ints=2 * DecodeBatch.ints_for(3, 4, 16))
+    pos = [60, 300, 125]
+    walked.fill(slots, pos, [1, 2, 3])
+    lists = [walked.decode_chunks(8, 16, w, 0, table, 16)[0] for w in (0, 100)]
+    pages = walked.write_pages(0, table, 16)
+    for step in range(1, 8):                     # positions 64 and 128 start pages on the way
+        pos = [p + 1 for p in pos]
+        walked.fill(slots, pos, [step] * 3)
+        fresh = DecodeBatch(3, 4, "cpu")
+        fresh.fill(slots, pos, [step] * 3)
+        for w, got in zip((0, 100), lists):
+            want = fresh.decode_chunks(8, 16, w, 0, table, 16)[0]
+            n = int(want.reshape(-1, 8)[0, 0])
+            assert got.reshape(-1, 8)[:n + 1].tolist() == want.reshape(-1, 8)[:n + 1].tolist(), (step, w)
+        assert pages.tolist() == fresh.write_pages(0, table, 16).tolist()
+        assert walked.seq_pos0.tolist() == pos and walked.tokens.tolist() == [step] * 3
