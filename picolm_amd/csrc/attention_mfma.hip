@@ -26,6 +26,7 @@ typedef __attribute__((ext_vector_type(4))) float f32x4;
 
 #define LOG2E 1.4426950408889634f
 #define LN2 0.6931471805599453f
+#define LAZY_MAX_STEP 8.0f
 
 __device__ __forceinline__ bf16x8 ldg8(const bf16_t* p) { return *(const bf16x8*)p; }
 __device__ __forceinline__ bf16x8 zero8() {
@@ -70,22 +71,28 @@ __device__ __forceinline__ void attend_page(const bf16x8 (&Qf)[D / 16], f32x16 (
             if (MASKED) {
                 const int key = key0 + 32 * t + key_of_elem(e, h);
                 const bool vis = q_ok && key <= qpos && (window <= 0 || qpos - key < window);
-                S[t][e] = vis ? S[t][e] * scale2 : NEG_BIG;
-            } else {
-                S[t][e] *= scale2;          // every key of the page is visible to every query of the wave
-            }
+                S[t][e] = vis ? S[t][e] : NEG_BIG;
+            }                               // else every key of the page is visible to every query of the wave
             mx = fmaxf(mx, S[t][e]);
         }
-    mx = fmaxf(mx, __shfl_xor(mx, 32, WAVE));
-    const float m_new = fmaxf(m_run, mx);
-    const float alpha = exp2f(m_run - m_new);
+    // the scores stay unscaled (the scale is positive, so their order is that of the scaled ones):
+    // the scale goes into the exponent's multiply-add below
+    mx = fmaxf(mx, __shfl_xor(mx, 32, WAVE)) * scale2;
+    // m_run is the reference point of the exponentials, not necessarily the maximum: it follows
+    // the maximum only when that has grown by more than LAZY_MAX_STEP (in powers of two), so that
+    // most pages leave it alone and O^T need not be rescaled.  The result is the same in exact
+    // arithmetic; probabilities may reach 2^LAZY_MAX_STEP instead of 1 meanwhile.
+    const bool grow = mx > m_run + LAZY_MAX_STEP;
+    const float m_new = grow ? mx : m_run;
+    const float alpha = grow ? exp2f(m_run - m_new) : 1.0f;
+    const bool rescale = __any(grow);
     float sum = 0.f;
     bf16x8 Pf[2][2];
 #pragma unroll
     for (int t = 0; t < 2; ++t)
 #pragma unroll
         for (int e = 0; e < 16; ++e) {
-            const float p = (!MASKED || S[t][e] > 0.5f * NEG_BIG) ? exp2f(S[t][e] - m_new) : 0.f;
+            const float p = (!MASKED || S[t][e] > 0.5f * NEG_BIG) ? exp2f(fmaf(S[t][e], scale2, -m_new)) : 0.f;
             sum += p;
             Pf[t][e / 8][e % 8] = to_bf16(p);
         }
@@ -94,8 +101,10 @@ __device__ __forceinline__ void attend_page(const bf16x8 (&Qf)[D / 16], f32x16 (
     m_run = m_new;
 #pragma unroll
     for (int dt = 0; dt < D / 32; ++dt) {
+        if (rescale) {
 #pragma unroll
-        for (int e = 0; e < 16; ++e) O[dt][e] *= alpha;
+            for (int e = 0; e < 16; ++e) O[dt][e] *= alpha;
+        }
 #pragma unroll
         for (int t = 0; t < 2; ++t)
 #pragma unroll
