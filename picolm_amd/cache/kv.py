@@ -84,6 +84,7 @@ class Cache:
         self.max_pages = pages_for(self.max_seq_len)
         self.n_slots = n_slots if n_slots is not None else n_pages
         self.slots = SlotTable(self.n_slots)
+        self.version = 0        # moves whenever a slot or a page changes hands: what was looked up before is stale
         self.kv = [KVGroup(g, n_pages, self.n_slots, self.max_pages, dtype, self.device)
                    for g in spec.kv_groups]
         self.state = [torch.zeros((g.n_entries, self.n_slots, *g.shape), dtype=g.dtype, device=self.device)
@@ -92,12 +93,14 @@ class Cache:
     # -- slots ---------------------------------------------------------------------------
     def alloc_slot(self) -> int:
         s = self.slots.alloc()
+        self.version += 1
         for st in self.state:
             st[:, s].zero_()
         return s
 
     def free_slot(self, slot: int) -> None:
         self.slots.free(slot)            # raises on a double free before any page moves
+        self.version += 1
         for g in self.kv:
             g.book.release(slot)
 
@@ -119,6 +122,7 @@ class Cache:
             for j, p in g.book.grow(slot, n_tokens):
                 g.table_host[slot, j] = p
                 g.dirty.add(slot)
+                self.version += 1
 
     def reserve_many(self, slots, lengths) -> None:
         """All or nothing for a whole batch."""

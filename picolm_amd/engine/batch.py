@@ -257,6 +257,7 @@ class DecodeBatch:
         self._lists = {}        # (window, group) -> (host array, device array, most chunks, page table, ring, own block or None)
         self._pages = {}        # group -> (host array, device array, page table, ring, own block or None)
         self._live = {}         # (window, group) -> entries in use
+        self._cache_version = None
         self.frozen = False     # set once the launches are recorded: no further work list can join
 
     @staticmethod
@@ -274,10 +275,14 @@ class DecodeBatch:
         own = self._host_block(n_ints)
         return own.numpy(), torch.zeros(n_ints, dtype=torch.int32, device=self._device), own
 
-    def fill(self, slots, pos0, tokens) -> None:
+    def fill(self, slots, pos0, tokens, cache_version=None) -> None:
+        """`cache_version`: the cache's counter of slot and page changes; while it stands still
+        (and is given), what the last fill looked up in the page tables still holds."""
         # between page boundaries only the positions move: the lists and pages stay as they are
-        same_pages = (list(slots) == self.slots and len(pos0) == len(self.pos0)
+        same_pages = (cache_version is not None and cache_version == self._cache_version
+                      and list(slots) == self.slots and len(pos0) == len(self.pos0)
                       and all(p == q + 1 and p % PAGE_TOKENS for p, q in zip(pos0, self.pos0)))
+        self._cache_version = cache_version
         self.slots, self.pos0 = list(slots), list(pos0)
         self._np["seq_slot"][:] = slots
         self._np["seq_pos0"][:] = pos0

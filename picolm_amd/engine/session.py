@@ -29,7 +29,7 @@ class _DecodeGraph:
         self.uses = 0
 
     def run(self, s: "Session", slots, pos0, tokens) -> torch.Tensor:
-        self.batch.fill(slots, pos0, tokens)
+        self.batch.fill(slots, pos0, tokens, s.cache.version)
         self.uses += 1
         if self.graph is not None:
             self.graph.replay()

@@ -320,3 +320,32 @@ def test_recorded_decode_steps_equal_eager_ones(folders):
         else:
             assert not s._decode_graphs
     assert torch.equal(outs[True], outs[False])
+
+
+@pytest.mark.parametrize("which", ["C", "D"])
+def test_a_batch_that_continues_where_another_stopped(which, folders):
+    """One batch ends and gives its slots back; the next gets the same slots (with other pages)
+    and its sequences happen to be exactly one token longer than the last ones were.  To the
+    recorded decode step that looks like the next step of the old batch; it must not keep what it
+    looked up in the page tables for the old one."""
+    d = folders[which]
+    V = tiny.CONFIGS[which][0]["vocab_size"]
+    rng = np.random.default_rng(5)
+    s = session(d, "bfloat16", max_tokens=1024)
+    hold = s.begin(1)                                   # keeps a page, so that the pages of the second batch differ
+    s.step(hold, [tiny.random_tokens(rng, 3, V)])
+    first = [tiny.random_tokens(rng, n, V) for n in (40, 70)]
+    slots = s.begin(2)
+    s.step(slots, [t[:-4] for t in first])
+    for j in range(4, 0, -1):                           # decode steps at positions 36..39 and 66..69
+        s.step(slots, [[t[-j]] for t in first])
+    s.release(slots)
+    s.step(hold, [tiny.random_tokens(rng, 130, V)])     # takes pages that the first batch gave back
+    second = [tiny.random_tokens(rng, n, V) for n in (41, 71)]
+    assert sorted(s.begin(2)) == sorted(slots)
+    again = slots                                       # the same slots in the same order as before
+    s.step(again, [t[:-1] for t in second])             # prompts of 40 and 70 tokens
+    got = s.step(again, [[t[-1]] for t in second]).cpu().numpy()      # decode at positions 40 and 70
+    for i, t in enumerate(second):
+        ref = tiny.plain_logits(d, t)[-1]
+        assert np.abs(got[i] - ref).max() <= tolerance("bfloat16", ref)

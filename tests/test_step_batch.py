@@ -133,12 +133,12 @@ def test_decode_batch_between_page_boundaries_only_moves_positions():
     slots = [2, 0, 1]
     walked = DecodeBatch(3, 4, "cpu", reserve_ints=2 * DecodeBatch.ints_for(3, 4, 16))
     pos = [60, 300, 125]
-    walked.fill(slots, pos, [1, 2, 3])
+    walked.fill(slots, pos, [1, 2, 3], cache_version=7)
     lists = [walked.decode_chunks(8, 16, w, 0, table, 16)[0] for w in (0, 100)]
     pages = walked.write_pages(0, table, 16)
     for step in range(1, 8):                     # positions 64 and 128 start pages on the way
         pos = [p + 1 for p in pos]
-        walked.fill(slots, pos, [step] * 3)
+        walked.fill(slots, pos, [step] * 3, cache_version=7)
         fresh = DecodeBatch(3, 4, "cpu")
         fresh.fill(slots, pos, [step] * 3)
         for w, got in zip((0, 100), lists):
@@ -147,3 +147,23 @@ def test_decode_batch_between_page_boundaries_only_moves_positions():
             assert got.reshape(-1, 8)[:n + 1].tolist() == want.reshape(-1, 8)[:n + 1].tolist(), (step, w)
         assert pages.tolist() == fresh.write_pages(0, table, 16).tolist()
         assert walked.seq_pos0.tolist() == pos and walked.tokens.tolist() == [step] * 3
+
+
+def test_decode_batch_looks_pages_up_again_when_the_cache_changed():
+    """The same slots one position further, but the slots changed hands in between (another batch
+    got them): the page ids of the last fill are stale and must not be kept."""
+    import torch
+    table = torch.arange(2 * 8, dtype=torch.int32).reshape(2, 8).clone()
+    b = DecodeBatch(2, 4, "cpu", reserve_ints=DecodeBatch.ints_for(2, 4, 8))
+    b.fill([0, 1], [10, 70], [1, 1], cache_version=3)
+    dev = b.decode_chunks(8, 16, 0, 0, table, 8)[0]
+    pages = b.write_pages(0, table, 8)
+    table += 100                                        # other pages now
+    b.fill([0, 1], [11, 71], [1, 1], cache_version=4)
+    assert pages.tolist() == [100, 109]
+    assert dev.reshape(-1, 8)[1, 4] == 100
+    b.fill([0, 1], [12, 72], [1, 1], cache_version=4)   # nothing changed: positions only
+    assert dev.reshape(-1, 8)[1:3, 2].tolist() == [12, 72] and pages.tolist() == [100, 109]
+    table += 100
+    b.fill([0, 1], [13, 73], [1, 1])                    # no version given: never the short way
+    assert pages.tolist() == [200, 209]
