@@ -266,3 +266,101 @@ def test_toy_architecture_with_a_stateful_mixer(tmp_path):
             live = [i for i in live if pos[i] < len(reqs[i])]
     finally:
         unregister_architecture("ToyRunningMeanLM")
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_toy_position_encoding_that_is_no_rotation(dtype):
+    """A position encoding defined here: it damps queries and keys with their position.  The
+    attention part takes it through `PositionEncoding.apply`, in a prefill step and in decode steps
+    (where the bfloat16 kernel that writes the cache itself gets rows that are already encoded)."""
+    from picolm_amd.cache.slots import PAGE_TOKENS
+    from picolm_amd.engine.batch import StepBatch
+    from picolm_amd.parts import Attention, PositionEncoding
+    from picolm_amd.weights import TensorDict, WeightFetcher
+
+    class Damping(PositionEncoding):
+        """q and k of the token at position p are multiplied by 1 / (1 + p / 32)."""
+
+        def apply(self, ctx, qkv, H, G, d):
+            f = 1.0 / (1.0 + ctx.batch.tok_pos[:qkv.shape[0]].float() / 32.0)
+            qkv[:, :(H + G) * d] *= f[:, None]
+
+    H, G, d, D = 4, 2, 32, 48
+    rng = np.random.default_rng(9)
+    names = ["a.q_proj.weight", "a.k_proj.weight", "a.v_proj.weight", "a.o_proj.weight"]
+    shapes = [(H * d, D), (G * d, D), (G * d, D), (D, H * d)]
+    w = {n: rounded(rng.standard_normal(s) * 0.2, torch.bfloat16) for n, s in zip(names, shapes)}
+    part = Attention("a.", D, H, G, d, position=Damping())
+    lens, tail = [70, 9], 3
+    rt, ctx = harness(dtype, part.cache_requests(), [2, 0], [0, 0], [n + tail for n in lens])
+    part.load_all(WeightFetcher(TensorDict({k: torch.from_numpy(v).to(torch.bfloat16) for k, v in w.items()}), DEV), rt)
+    part.prepare(rt, 512)
+    hs = [rounded(rng.standard_normal((n + tail, D)), dtype) for n in lens]
+
+    def plain(x):
+        T = len(x)
+        f = 1.0 / (1.0 + np.arange(T) / 32.0)
+        q = (x @ w["a.q_proj.weight"].T).reshape(T, H, d) * f[:, None, None]
+        k = (x @ w["a.k_proj.weight"].T).reshape(T, G, d) * f[:, None, None]
+        v = (x @ w["a.v_proj.weight"].T).reshape(T, G, d)
+        return P.causal_attention(q, k, v).reshape(T, H * d) @ w["a.o_proj.weight"].T
+    ref = [plain(x) for x in hs]
+    # the prompts in one step, then one token each
+    ctx.batch = StepBatch([2, 0], [0, 0], [[0] * n for n in lens], [[], []], 10, DEV)
+    res = torch.zeros(sum(lens), D, device=DEV)
+    part.forward(ctx, torch.from_numpy(np.concatenate([x[:n] for x, n in zip(hs, lens)])).to(dtype).to(DEV), res)
+    want = np.concatenate([r[:n] for r, n in zip(ref, lens)])
+    assert np.abs(res.double().cpu().numpy() - want).max() <= tol(dtype, want)
+    for j in range(tail):
+        ctx.batch = StepBatch([2, 0], [n + j for n in lens], [[0], [0]], [[], []], 10, DEV)
+        res = torch.zeros(2, D, device=DEV)
+        part.forward(ctx, torch.from_numpy(np.stack([x[n + j] for x, n in zip(hs, lens)])).to(dtype).to(DEV), res)
+        want = np.stack([r[n + j] for r, n in zip(ref, lens)])
+        assert np.abs(res.double().cpu().numpy() - want).max() <= tol(dtype, want)
+
+
+def test_toy_feed_forward_with_routing():
+    """A feed-forward defined here: two gated experts and a router that sends every row to the
+    expert with the larger logit (router logits in float).  It is built from the library's Linear
+    and SwiGLU parts and runs in a block next to attention, without a change to the library."""
+    from picolm_amd.parts import FeedForward, Linear, SwiGLU
+    from picolm_amd.weights import TensorDict, WeightFetcher
+
+    class TwoExperts(FeedForward):
+        def __init__(self, prefix, D, F):
+            self.router = Linear([prefix + "router.weight"], [2], D)
+            self.experts = [SwiGLU(prefix + f"experts.{i}.", D, F) for i in range(2)]
+
+        def children(self):
+            return [self.router] + self.experts
+
+        def forward(self, ctx, h, residual):
+            logits = torch.zeros(h.shape[0], 2, device=h.device)
+            self.router.forward(h, logits)
+            choice = logits.argmax(dim=1)
+            for i, expert in enumerate(self.experts):
+                rows = torch.nonzero(choice == i).flatten()
+                if rows.numel():
+                    out = torch.zeros(rows.numel(), residual.shape[1], device=h.device)
+                    expert.forward(ctx, h.index_select(0, rows).contiguous(), out)
+                    residual.index_add_(0, rows, out)
+
+    D, F, T = 64, 96, 37
+    rng = np.random.default_rng(3)
+    shapes = {"f.router.weight": (2, D)}
+    for i in range(2):
+        shapes.update({f"f.experts.{i}.gate_proj.weight": (F, D), f"f.experts.{i}.up_proj.weight": (F, D),
+                       f"f.experts.{i}.down_proj.weight": (D, F)})
+    w = {n: rounded(rng.standard_normal(s) * 0.3, torch.bfloat16) for n, s in shapes.items()}
+    ffn = TwoExperts("f.", D, F)
+    assert sorted(s.name for s in ffn.all_specs()) == sorted(shapes)
+    rt, ctx = harness(torch.bfloat16, (None, None), [0], [0], [T])
+    ffn.load_all(WeightFetcher(TensorDict({k: torch.from_numpy(v).to(torch.bfloat16) for k, v in w.items()}), DEV), rt)
+    x = rounded(rng.standard_normal((T, D)), torch.bfloat16)
+    res = torch.zeros(T, D, device=DEV)
+    ffn.forward(ctx, torch.from_numpy(x).to(torch.bfloat16).to(DEV), res)
+    choice = (x @ w["f.router.weight"].T).argmax(axis=1)
+    assert 0 < choice.sum() < T                          # both experts get rows
+    ref = np.stack([P.swiglu(x[t:t + 1], w[f"f.experts.{c}.gate_proj.weight"], w[f"f.experts.{c}.up_proj.weight"],
+                             w[f"f.experts.{c}.down_proj.weight"])[0] for t, c in enumerate(choice)])
+    assert np.abs(res.double().cpu().numpy() - ref).max() <= tol(torch.bfloat16, ref)
