@@ -46,6 +46,16 @@ int picolm_gemm_tiled_splitk(const void* A, const void* W, void* C, int c_dt, in
                              int64_t ldw, int64_t ldc, int epilogue, int variant, int splits, float* ws,
                              hipStream_t stream);
 
+// A decode step's products with an RMSNorm split between them, up to 16 rows.  A product with the
+// accumulating epilogue (skinny variant 0/1) can prepare the norm that follows: next_h[M][ldc] =
+// bf16(x * next_w) and next_ssq[16][next_parts] partial sums of x^2 (next_parts >= ceil(N / 16)).
+// A product whose input rows are such a next_h takes ssq[16][n_parts], the norm's row length and
+// eps and multiplies its sums by 1 / sqrt(sum / len + eps).  tiled != 0: tile variant 12 or 13.
+int picolm_gemm_linked(const void* A, const void* W, void* C, int c_dt, int M, int N, int K, int64_t lda,
+                       int64_t ldw, int64_t ldc, int epilogue, int tiled, int variant, const float* next_w,
+                       void* next_h, float* next_ssq, int next_parts, const float* ssq, int n_parts,
+                       int norm_len, float eps, hipStream_t stream);
+
 int picolm_attn_prefill_tile_rows(void);
 int picolm_attn_prefill_generic(const void* q, const void* k_pages, const void* v_pages, void* out,
                                 int dt, const int32_t* tile_seq, const int32_t* tile_q0, int n_tiles,

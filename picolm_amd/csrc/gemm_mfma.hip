@@ -32,6 +32,64 @@ __device__ __forceinline__ bf16x8 zero_chunk() {
 __device__ __forceinline__ float silu_mul(float g, float u) { return g / (1.0f + expf(-g)) * u; }
 
 // =============================================================================================
+// a norm split between two products
+// =============================================================================================
+// In a decode step an RMSNorm of a few rows is all launch latency.  It can ride on the products
+// around it instead: the product that finishes the rows of the residual stream (epilogue 1) also
+// leaves, for the norm that follows, next_h = bf16(x * w) and one partial sum of x^2 per row and
+// workgroup; the product that consumes the normed rows takes next_h as its input and multiplies its
+// sums by 1 / sqrt(sum(x^2) / len + eps) in float.  Both sides only for up to 16 rows.
+struct NormLink {
+    const float* next_w;    // producer: weights of the norm that follows [N], or null
+    bf16_t* next_h;         //   [M][ld of C] what the next product reads
+    float* next_ssq;        //   [16][next_parts] partial sums of x^2, one column per workgroup
+    int next_parts;
+    const float* ssq;       // consumer: the partial sums a producer left [16][n_parts], or null
+    int n_parts;
+    float inv_len, eps;     //   1 / row length of the norm, its eps
+};
+
+// Consumer side.  `begin` has every thread ask for its share of the partial sums (row tid % 16,
+// every (THREADS/16)-th part) before the main loop; `finish` adds them up in a fixed order and
+// leaves the 16 row factors in LDS.  Both are called by all THREADS threads of the workgroup.
+template <int THREADS>
+__device__ __forceinline__ float row_scale_begin(const NormLink& k, int M) {
+    float mine = 0.f;
+    if (k.ssq) {
+        const int m = threadIdx.x % 16;
+        if (m < M) {
+            // eight loads are asked for before the first is added: one trip to memory, not eight
+            constexpr int STRIDE = THREADS / 16;
+            const float* row = k.ssq + (size_t)m * k.n_parts;
+            for (int p0 = threadIdx.x / 16; p0 < k.n_parts; p0 += 8 * STRIDE) {
+                float v[8];
+#pragma unroll
+                for (int i = 0; i < 8; ++i) v[i] = row[min(p0 + i * STRIDE, k.n_parts - 1)];
+#pragma unroll
+                for (int i = 0; i < 8; ++i) mine += p0 + i * STRIDE < k.n_parts ? v[i] : 0.f;
+            }
+        }
+    }
+    return mine;
+}
+template <int THREADS>
+__device__ __forceinline__ void row_scale_finish(const NormLink& k, float mine, float (&scratch)[THREADS / 64][16],
+                                                 float (&scale)[16]) {
+    if (!k.ssq) return;          // uniform over the workgroup
+    mine += __shfl_xor(mine, 16, WAVE);
+    mine += __shfl_xor(mine, 32, WAVE);
+    if (threadIdx.x % 64 < 16) scratch[threadIdx.x / 64][threadIdx.x % 16] = mine;
+    __syncthreads();
+    if (threadIdx.x < 16) {
+        float total = 0.f;
+#pragma unroll
+        for (int w = 0; w < THREADS / 64; ++w) total += scratch[w][threadIdx.x];
+        scale[threadIdx.x] = 1.0f / sqrtf(total * k.inv_len + k.eps);
+    }
+    __syncthreads();
+}
+
+// =============================================================================================
 // skinny
 // =============================================================================================
 #define SK_KSTEP 128      // K elements one wave consumes per step: 4 MFMAs of 32
@@ -40,8 +98,10 @@ template <int MT, int NT, int WAVES, int EPI, typename TC>
 __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const bf16_t* __restrict__ A,
                                                                  const bf16_t* __restrict__ W,
                                                                  TC* __restrict__ C, int M, int N, int K,
-                                                                 int64_t lda, int64_t ldw, int64_t ldc) {
+                                                                 int64_t lda, int64_t ldw, int64_t ldc, NormLink link) {
     extern __shared__ float red[];      // [WAVES][NT][MT][4][64]
+    __shared__ float link_scratch[WAVES][16], link_scale[16];
+    const float link_mine = row_scale_begin<WAVES * 64>(link, M);
     const int wave = threadIdx.x / 64, lane = threadIdx.x % 64;
     const int r16 = lane % 16, q = lane / 16;
     const int n_base = blockIdx.x * (16 * NT);
@@ -123,8 +183,10 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const bf16_t* _
 #pragma unroll
             for (int r = 0; r < 4; ++r) red[(((wave * NT + t) * MT + u) * 4 + r) * 64 + lane] = acc[t][u][r];
     __syncthreads();
+    row_scale_finish<WAVES * 64>(link, link_mine, link_scratch, link_scale);
     constexpr int PER_WAVE = NT * MT * 4 * 64;
     constexpr int STEP = (EPI == 2) ? 2 : 1;
+    float next_sq = 0.f;                // producer side: x^2 of the value this thread finishes (MT = NT = 1 only)
     // value v = ((t*MT + u)*4 + r)*64 + l ; the gated epilogue takes r and r+1 together
     for (int v = threadIdx.x; v < PER_WAVE / STEP; v += WAVES * 64) {
         int l, r, tu;
@@ -148,20 +210,44 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const bf16_t* _
         const int n = n_base + t * 16 + 4 * (l / 16) + r;
         const int m = u * 16 + l % 16;
         if (m >= M || n >= N) continue;
+        if (link.ssq) {
+            s0 *= link_scale[m];
+            s1 *= link_scale[m];
+        }
         if (EPI == 2) {
             C[(int64_t)m * ldc + n / 2] = from_f32<TC>(silu_mul(s0, s1));
         } else if (EPI == 1) {
             TC* p = C + (int64_t)m * ldc + n;
-            *p = from_f32<TC>(to_f32<TC>(*p) + s0);
+            const float x = to_f32<TC>(*p) + s0;
+            *p = from_f32<TC>(x);
+            if (link.next_w) {
+                link.next_h[(int64_t)m * ldc + n] = f32_to_bf16_bits(x * link.next_w[n]);
+                next_sq = x * x;
+            }
         } else {
             C[(int64_t)m * ldc + n] = from_f32<TC>(s0);
         }
+    }
+    if (EPI == 1 && MT == 1 && NT == 1 && link.next_w) {
+        // this workgroup's 16 columns of every row: lanes l, l+16, l+32, l+48 of the first four
+        // waves hold them (r = wave); rows past M and columns past N added nothing
+        next_sq += __shfl_xor(next_sq, 16, WAVE);
+        next_sq += __shfl_xor(next_sq, 32, WAVE);
+        __syncthreads();                    // link_scratch may still be read as the consumer's
+        if (wave < 4 && lane < 16) link_scratch[wave][lane] = next_sq;
+        __syncthreads();
+        if (threadIdx.x < 16)
+            link.next_ssq[(size_t)threadIdx.x * link.next_parts + blockIdx.x] =
+                link_scratch[0][threadIdx.x] + link_scratch[1][threadIdx.x] + link_scratch[2][threadIdx.x] + link_scratch[3][threadIdx.x];
     }
 }
 
 template <int MT, int NT, int WAVES>
 static int launch_skinny(const void* A, const void* W, void* C, int c_dt, int M, int N, int K, int64_t lda,
-                         int64_t ldw, int64_t ldc, int epi, hipStream_t stream) {
+                         int64_t ldw, int64_t ldc, int epi, hipStream_t stream, NormLink link = NormLink{}) {
+    PICOLM_REQUIRE(!link.next_w || (MT == 1 && NT == 1 && WAVES == 8 && epi == 1 && link.next_parts >= ceil_div(N, 16)),
+                   "gemm_skinny: only the 16x16 tile with the accumulating epilogue prepares a norm");
+    PICOLM_REQUIRE(!link.ssq || M <= 16, "gemm_skinny: a norm's statistics are taken for up to 16 rows, got %d", M);
     dim3 grid(ceil_div(N, 16 * NT)), block(WAVES * 64);
     const size_t lds = sizeof(float) * WAVES * NT * MT * 4 * 64;
     const bf16_t* a = (const bf16_t*)A;
@@ -176,7 +262,7 @@ static int launch_skinny(const void* A, const void* W, void* C, int c_dt, int M,
                            hipGetErrorString(e));                                                       \
             raised = lds;                                                                               \
         }                                                                                               \
-        gemm_skinny_kernel<MT, NT, WAVES, EPI, TC><<<grid, block, lds, stream>>>(a, w, (TC*)C, M, N, K, lda, ldw, ldc); \
+        gemm_skinny_kernel<MT, NT, WAVES, EPI, TC><<<grid, block, lds, stream>>>(a, w, (TC*)C, M, N, K, lda, ldw, ldc, link); \
     }
     if (epi == 0 && c_dt == PICOLM_F32) SK_LAUNCH(0, float)
     else if (epi == 0 && c_dt == PICOLM_BF16) SK_LAUNCH(0, bf16_t)
@@ -199,9 +285,11 @@ template <int STEPS, int EPI, typename TC>
 __global__ __launch_bounds__(512) void gemm_skinny_resident_kernel(const bf16_t* __restrict__ A,
                                                                    const bf16_t* __restrict__ W,
                                                                    TC* __restrict__ C, int M, int N, int K,
-                                                                   int64_t lda, int64_t ldw, int64_t ldc) {
+                                                                   int64_t lda, int64_t ldw, int64_t ldc, NormLink link) {
     constexpr int WAVES = 8;
     __shared__ float red[2][WAVES][4][64];
+    __shared__ float link_scratch[WAVES][16], link_scale[16];
+    const float link_mine = row_scale_begin<WAVES * 64>(link, M);
     const int wave = threadIdx.x / 64, lane = threadIdx.x % 64;
     const int r16 = lane % 16, q = lane / 16;
     const int n_full = K / SK_KSTEP;            // K is a whole number of steps (the host sees to that)
@@ -247,6 +335,10 @@ __global__ __launch_bounds__(512) void gemm_skinny_resident_kernel(const bf16_t*
             }
             const int n = tile * 16 + 4 * (l / 16) + r, m = l % 16;
             if (m < M && n < N) {
+                if (link.ssq) {
+                    s0 *= link_scale[m];
+                    s1 *= link_scale[m];
+                }
                 if (EPI == 2) {
                     C[(int64_t)m * ldc + n / 2] = from_f32<TC>(silu_mul(s0, s1));
                 } else if (EPI == 1) {
@@ -264,6 +356,7 @@ __global__ __launch_bounds__(512) void gemm_skinny_resident_kernel(const bf16_t*
     const int stride = gridDim.x;
     int tile = blockIdx.x;
     fetch(w0, min(tile, n_tiles - 1));
+    row_scale_finish<WAVES * 64>(link, link_mine, link_scratch, link_scale);
     while (tile < n_tiles) {
         fetch(w1, min(tile + stride, n_tiles - 1));
         __builtin_amdgcn_sched_barrier(0);      // the next tile is asked for before this one is waited for
@@ -279,7 +372,8 @@ __global__ __launch_bounds__(512) void gemm_skinny_resident_kernel(const bf16_t*
 
 template <int STEPS>
 static int launch_skinny_resident(const void* A, const void* W, void* C, int c_dt, int M, int N, int K, int64_t lda,
-                                  int64_t ldw, int64_t ldc, int epi, hipStream_t stream) {
+                                  int64_t ldw, int64_t ldc, int epi, hipStream_t stream, NormLink link = NormLink{}) {
+    PICOLM_REQUIRE(!link.next_w, "gemm_skinny: the resident variant prepares no norm");
     PICOLM_REQUIRE(M <= 16 && K % SK_KSTEP == 0 && K <= STEPS * 8 * SK_KSTEP,
                    "gemm_skinny: the resident variant takes M <= 16 and K a multiple of %d up to %d, got M=%d K=%d",
                    SK_KSTEP, STEPS * 8 * SK_KSTEP, M, K);
@@ -290,7 +384,7 @@ static int launch_skinny_resident(const void* A, const void* W, void* C, int c_d
     const bf16_t* a = (const bf16_t*)A;
     const bf16_t* w = (const bf16_t*)W;
 #define SR_LAUNCH(EPI, TC) \
-    gemm_skinny_resident_kernel<STEPS, EPI, TC><<<grid, block, 0, stream>>>(a, w, (TC*)C, M, N, K, lda, ldw, ldc);
+    gemm_skinny_resident_kernel<STEPS, EPI, TC><<<grid, block, 0, stream>>>(a, w, (TC*)C, M, N, K, lda, ldw, ldc, link);
     if (epi == 0 && c_dt == PICOLM_F32) SR_LAUNCH(0, float)
     else if (epi == 0 && c_dt == PICOLM_BF16) SR_LAUNCH(0, bf16_t)
     else if (epi == 1 && c_dt == PICOLM_F32) SR_LAUNCH(1, float)
@@ -606,7 +700,10 @@ __global__ __launch_bounds__(64 * WN * WM) void gemm_direct_kernel(const bf16_t*
                                                                    const bf16_t* __restrict__ W,
                                                                    TC* __restrict__ C, int M, int N, int K,
                                                                    int64_t lda, int64_t ldw, int64_t ldc,
-                                                                   int tiles_m, int tiles_n, int64_t c_split_stride) {
+                                                                   int tiles_m, int tiles_n, int64_t c_split_stride,
+                                                                   NormLink link) {
+    __shared__ float link_scratch[WN * WM][16], link_scale[16];
+    const float link_mine = row_scale_begin<64 * WN * WM>(link, M);
     // K here is the length of one split: workgroup row y of the grid takes columns y*K .. of A
     // and W and writes its sums to C + y * c_split_stride
     A += (int64_t)blockIdx.y * K;
@@ -755,6 +852,7 @@ __global__ __launch_bounds__(64 * WN * WM) void gemm_direct_kernel(const bf16_t*
         stage = next_stage;
     }
     wait_for_loads<0>();
+    row_scale_finish<64 * WN * WM>(link, link_mine, link_scratch, link_scale);
 #pragma unroll
     for (int i = 0; i < TN; ++i) {
         const int n = n0 + wn + 32 * i + l32;
@@ -763,7 +861,8 @@ __global__ __launch_bounds__(64 * WN * WM) void gemm_direct_kernel(const bf16_t*
 #pragma unroll
             for (int e = 0; e < 16; ++e) {
                 const int m = m0 + wm + 32 * j + 8 * (e / 4) + 4 * kq + e % 4;
-                const float v = acc[i][j][e];
+                float v = acc[i][j][e];
+                if (link.ssq && m < 16) v *= link_scale[m];      // (the host admits this for M <= 16 only)
                 if (EPI == 2) {
                     const float up = __shfl_xor(v, 1, WAVE);
                     if (m < M && (l32 & 1) == 0 && n + 1 < N) C[(int64_t)m * ldc + n / 2] = from_f32<TC>(silu_mul(v, up));
@@ -779,7 +878,10 @@ __global__ __launch_bounds__(64 * WN * WM) void gemm_direct_kernel(const bf16_t*
 template <int TN, int TM, int WN, int WM, int BK, int NS>
 static int launch_direct(const void* A, const void* W, void* C, int c_dt, int M, int N, int K, int64_t lda,
                          int64_t ldw, int64_t ldc, int epilogue, hipStream_t stream, int splits = 1,
-                         int64_t c_split_stride = 0) {
+                         int64_t c_split_stride = 0, NormLink link = NormLink{}) {
+    PICOLM_REQUIRE(!link.next_w, "gemm_tiled: the tiled kernels prepare no norm");
+    PICOLM_REQUIRE(!link.ssq || (M <= 16 && splits == 1),
+                   "gemm_tiled: a norm's statistics are taken for up to 16 rows of an uncut product");
     constexpr int BN = 32 * TN * WN, BM = 32 * TM * WM;
     PICOLM_REQUIRE(splits >= 1 && K % (BK * splits) == 0,
                    "gemm_tiled: K = %d is no multiple of %d times %d splits, which this variant needs", K, BK, splits);
@@ -804,7 +906,7 @@ static int launch_direct(const void* A, const void* W, void* C, int c_dt, int M,
             raised = lds;                                                                                  \
         }                                                                                                  \
         gemm_direct_kernel<TN, TM, WN, WM, BK, NS, EPI, TC><<<grid, block, lds, stream>>>(                 \
-            a, w, (TC*)C, M, N, k_len, lda, ldw, ldc, tiles_m, tiles_n, c_split_stride);                   \
+            a, w, (TC*)C, M, N, k_len, lda, ldw, ldc, tiles_m, tiles_n, c_split_stride, link);             \
     }
     if (epilogue == 0 && c_dt == PICOLM_F32) TD_LAUNCH(0, float)
     else if (epilogue == 0 && c_dt == PICOLM_BF16) TD_LAUNCH(0, bf16_t)
@@ -929,4 +1031,34 @@ extern "C" int picolm_gemm_tiled_splitk(const void* A, const void* W, void* C, i
     }
     if (rc) return rc;
     return launch_splitk_reduce(ws, C, c_dt, M, N, ldc, splits, epilogue, stream);
+}
+
+// The products of a decode step with a norm split between them (see NormLink): `variant` as in
+// picolm_gemm_skinny (0, 1, 7) or, with tiled != 0, a tile variant of picolm_gemm_tiled that
+// loads straight into LDS (12, 13).  next_*: this product (epilogue 1, skinny variant 0 or 1)
+// prepares the norm that follows; ssq, n_parts, norm_len, eps: this product's input rows are
+// the next_h of a product that prepared their norm.  Up to 16 rows.
+extern "C" int picolm_gemm_linked(const void* A, const void* W, void* C, int c_dt, int M, int N, int K, int64_t lda,
+                                  int64_t ldw, int64_t ldc, int epilogue, int tiled, int variant,
+                                  const float* next_w, void* next_h, float* next_ssq, int next_parts,
+                                  const float* ssq, int n_parts, int norm_len, float eps, hipStream_t stream) {
+    if (check_mfma_operands("gemm_linked", A, W, M, N, K, lda, ldw, ldc, epilogue, c_dt)) return -1;
+    PICOLM_REQUIRE(M <= 16, "gemm_linked: up to 16 rows, got %d", M);
+    PICOLM_REQUIRE(!next_w || (next_h && next_ssq && next_parts > 0), "gemm_linked: an incomplete description of the next norm");
+    PICOLM_REQUIRE(!ssq || (n_parts > 0 && norm_len > 0), "gemm_linked: an incomplete description of the norm's statistics");
+    if (M == 0) return 0;
+    NormLink link = {next_w, (bf16_t*)next_h, next_ssq, next_parts, ssq, n_parts, norm_len > 0 ? 1.0f / (float)norm_len : 0.f, eps};
+    if (tiled) {
+        switch (variant) {
+            case 12: return launch_direct<1, 2, 4, 1, 64, 3>(A, W, C, c_dt, M, N, K, lda, ldw, ldc, epilogue, stream, 1, 0, link);
+            case 13: return launch_direct<1, 1, 4, 1, 64, 4>(A, W, C, c_dt, M, N, K, lda, ldw, ldc, epilogue, stream, 1, 0, link);
+        }
+        PICOLM_REQUIRE(false, "gemm_linked: tile variant %d cannot take a norm's statistics", variant);
+    }
+    if (variant == 0) variant = (M > 4 && N >= 16384 && K % SK_KSTEP == 0 && K <= 4 * 8 * SK_KSTEP && !next_w) ? 7 : 1;
+    switch (variant) {
+        case 1: return launch_skinny<1, 1, 8>(A, W, C, c_dt, M, N, K, lda, ldw, ldc, epilogue, stream, link);
+        case 7: return launch_skinny_resident<4>(A, W, C, c_dt, M, N, K, lda, ldw, ldc, epilogue, stream, link);
+    }
+    PICOLM_REQUIRE(false, "gemm_linked: skinny variant %d cannot take part in a split norm", variant);
 }

@@ -57,6 +57,7 @@ class StepBatch:
                 rows.append(int(cu[i]) + int(j))
         self.n_want = len(rows)
         self.want_counts = [len(w) for w in want]
+        self.wants_every_row = rows == list(range(self.T))
 
         parts = {
             "seq_slot": np.asarray(self.slots, dtype=np.int32),
@@ -223,6 +224,7 @@ class DecodeBatch:
 
     is_decode = True
     max_new = 1
+    wants_every_row = True
 
     def __init__(self, n_seq: int, pages_per_chunk: int, device, reserve_ints: int = 0):
         """`reserve_ints`: room behind the step's arrays for the work lists and page arrays that

@@ -133,10 +133,24 @@ class DecoderModel:
         of workspace memory valid until the next step."""
         ctx = StepContext(self.runtime, batch, cache, workspace)
         x = self.embedding.forward(ctx, batch.tokens, batch.T)
-        for call, binding in zip(self.order, self.bindings):
+        # a block is told which norm meets the residual stream after it (the next block's first one,
+        # or the final norm when every row's logits are wanted), so that its last product can
+        # prepare that norm (see NormedRows)
+        every_row = getattr(batch, "wants_every_row", False)
+        for i, (call, binding) in enumerate(zip(self.order, self.bindings)):
             ctx.binding = binding
-            self.blocks[call.block].forward(ctx, x)
+            block = self.blocks[call.block]
+            if i + 1 < len(self.order):
+                after = getattr(self.blocks[self.order[i + 1].block], "first_norm", lambda: None)()
+            else:
+                after = self.final_norm if every_row and batch.n_want else None
+            ctx.norm_after_block = after
+            block.forward(ctx, x)
         if batch.n_want == 0:
             return workspace.get("logits", (0, self.head.V), torch.float32)
-        h = self.final_norm.forward(ctx, x, rows=batch.want_rows, n_rows=batch.n_want, out_name="norm.final")
+        if every_row:
+            h = ctx.normed(self.final_norm, x, self.head)
+        else:
+            ctx.prepared_norm = None
+            h = self.final_norm.forward(ctx, x, rows=batch.want_rows, n_rows=batch.n_want, out_name="norm.final")
         return self.head.forward(ctx, h)

@@ -42,7 +42,7 @@ def dir_entry_points():
     return ["picolm_abi_version", "picolm_device_check", "picolm_embed", "picolm_rmsnorm",
             "picolm_rope_kv_store", "picolm_silu_mul", "picolm_add_into", "picolm_gemm_generic",
             "picolm_attn_prefill_tile_rows", "picolm_attn_prefill_generic",
-            "picolm_attn_decode_generic", "picolm_argmax", "picolm_argmax_scratch_floats", "picolm_sample", "picolm_gemm_skinny", "picolm_gemm_tiled", "picolm_gemm_tiled_splitk",
+            "picolm_attn_decode_generic", "picolm_argmax", "picolm_argmax_scratch_floats", "picolm_sample", "picolm_gemm_skinny", "picolm_gemm_tiled", "picolm_gemm_tiled_splitk", "picolm_gemm_linked",
             "picolm_attn_mfma_takes", "picolm_attn_prefill_mfma_heads", "picolm_attn_prefill_mfma_tile_tokens",
             "picolm_attn_prefill_mfma", "picolm_attn_decode_mfma", "picolm_attn_decode_rope_mfma", "picolm_attn_decode_mfma_waves", "picolm_read_probe", "picolm_mfma_probe"]
 
@@ -327,6 +327,58 @@ def mfma_gemm_takes(a, w, c, epilogue: int) -> bool:
     if epilogue == EPI_ACCUMULATE:
         return c.dtype == torch.float32
     return True
+
+
+LINKED_NORM_MAX_M = 16
+
+
+def linked_norm_parts(N: int) -> int:
+    """Partial sums per row that a product of N output columns leaves for the norm that follows."""
+    return (N + 15) // 16
+
+
+def gemm_links_norms(a, w, c, epilogue: int) -> bool:
+    """Whether the product for these operands can take part in a norm split between two products
+    (prepare the next one with the accumulating epilogue, or take a prepared one's statistics):
+    the matrix-core kernels for up to 16 rows."""
+    return a.shape[0] <= LINKED_NORM_MAX_M and a.dim() == 2 and mfma_gemm_takes(a, w, c, epilogue)
+
+
+def gemm_linked(a, w, c, epilogue: int, prepare=None, prepared=None) -> None:
+    """The product of a decode step next to an RMSNorm that is split between two products.
+
+    prepare = (norm weights f32 [N], h_out bf16 [M, N], ssq_out f32 [16, parts]): with the
+    accumulating epilogue, also leave h_out = bf16(c * weights) and the partial sums of c^2.
+    prepared = (ssq f32 [16, parts], row length of the norm, eps): `a` is such an h_out; the sums
+    are multiplied by 1 / sqrt(sum(x^2) / length + eps)."""
+    M, N, K = _gemm_shapes(a, w, c, epilogue)
+    if not gemm_links_norms(a, w, c, epilogue):
+        raise KernelError(f"gemm_linked: a {tuple(a.shape)} {a.dtype}, w {tuple(w.shape)} {w.dtype} are not taken")
+    nw = nh = nssq = ssq = None
+    next_parts = n_parts = norm_len = 0
+    eps = 0.0
+    if prepare is not None:
+        nw, nh, nssq = prepare
+        if epilogue != EPI_ACCUMULATE:
+            raise KernelError("gemm_linked: only the accumulating epilogue prepares a norm")
+        _dev("gemm_linked.norm_weight", nw, torch.float32, 1)
+        _dev("gemm_linked.h_out", nh, torch.bfloat16, 2)
+        _dev("gemm_linked.ssq_out", nssq, torch.float32, 2)
+        next_parts = nssq.shape[1]
+        if nw.numel() != N or tuple(nh.shape) != (M, N) or nssq.shape[0] != 16 or next_parts < linked_norm_parts(N):
+            raise KernelError("gemm_linked: the buffers for the next norm do not fit the product")
+    if prepared is not None:
+        ssq, norm_len, eps = prepared
+        _dev("gemm_linked.ssq", ssq, torch.float32, 2)
+        n_parts = ssq.shape[1]
+        if ssq.shape[0] != 16 or norm_len != K:
+            raise KernelError("gemm_linked: the statistics are not those of this product's input rows")
+    tiled, variant = 0, 0
+    if prepare is None and M > 4 and K % 64 == 0 and 16384 <= N <= 128 * 256:
+        tiled, variant = 1, 13          # as in gemm()
+    _check(lib().picolm_gemm_linked(_ptr(a), _ptr(w), _ptr(c), dt_of(c), M, N, K, c_int64(K), c_int64(K),
+                                    c_int64(c.shape[1]), epilogue, tiled, variant, _ptr(nw), _ptr(nh), _ptr(nssq), next_parts,
+                                    _ptr(ssq), n_parts, int(norm_len), c_float(eps), _stream()))
 
 
 def medium_gemm_splits(M: int, N: int, K: int) -> int:

@@ -21,6 +21,7 @@ import torch
 
 class Attention(Mixer):
     graph_safe = True      # launches depend on device memory only
+    takes_normed_rows = True   # the input goes to a Linear unchanged
 
     def __init__(self, prefix: str, hidden_size: int, n_heads: int, n_kv_heads: int, head_dim: int,
                  position: PositionEncoding | None = None, window: int = 0, scale: float | None = None,
@@ -93,4 +94,4 @@ class Attention(Mixer):
         else:
             kernels.rope_kv_store(qkv, q, kp, vp, cos, sin, style, b.tok_pos, tok_page, H, G, d)
             kernels.attn_prefill(q, k_pages, v_pages, out, b, table, ring, H, G, d, self.window, self.scale)
-        self.o.forward(out, residual, kernels.EPI_ACCUMULATE)
+        self.o.forward(out, residual, kernels.EPI_ACCUMULATE, ctx)

@@ -38,6 +38,7 @@ class Workspace:
     def __init__(self, device):
         self.device = device
         self._bufs: dict[str, torch.Tensor] = {}
+        self._flips: dict[str, int] = {}
 
     def get(self, name: str, shape, dtype: torch.dtype) -> torch.Tensor:
         n = 1
@@ -49,6 +50,11 @@ class Workspace:
             buf = torch.empty(max(nbytes, 256), dtype=torch.uint8, device=self.device)
             self._bufs[name] = buf
         return buf[:nbytes].view(dtype).view(*shape)
+
+    def flip(self, name: str) -> int:
+        """0, 1, 0, 1, ... per name: for a pair of buffers used in turn."""
+        self._flips[name] = 1 - self._flips.get(name, 1)
+        return self._flips[name]
 
     def bytes(self) -> int:
         return sum(b.numel() for b in self._bufs.values())
@@ -87,6 +93,12 @@ class StepContext:
         self.cache = cache
         self.ws = workspace
         self.binding: CacheBinding | None = None
+        # the norm that will be applied to the residual stream after the running part has added to
+        # it (set by the block; a Linear that adds into the stream may prepare it) and what such a
+        # Linear prepared (picked up by whoever applies that norm next)
+        self.norm_after: Norm | None = None
+        self.prepared_norm: NormedRows | None = None
+        self.norm_after_block: Norm | None = None      # set by the model for the block it calls
 
     @property
     def dtype(self) -> torch.dtype:
@@ -102,6 +114,14 @@ class StepContext:
         """(cache group index, the group's page table on the host) of the running layer call."""
         gi, _ = self.binding.kv
         return gi, self.cache.kv[gi].table_host
+
+    def normed(self, norm: "Norm", x: torch.Tensor, part=None):
+        """norm(x) for `part`: what a Linear prepared for this very norm and x if there is such a
+        thing and the part passes it on to a Linear, else the norm's own kernel."""
+        got, self.prepared_norm = self.prepared_norm, None
+        if got is not None and got.norm is norm and got.x is x:
+            return got if getattr(part, "takes_normed_rows", False) else got.tensor()
+        return norm.forward(self, x)
 
     def state(self) -> torch.Tensor:
         """[n_slots, ...] state of the running layer call; index it with batch.seq_slot."""
@@ -135,6 +155,36 @@ class Norm(Part):
     def forward(self, ctx: StepContext, x: torch.Tensor, rows: torch.Tensor | None = None,
                 n_rows: int | None = None) -> torch.Tensor:
         raise NotImplementedError
+
+    def rms_parameters(self):
+        """(float weights, eps) if this norm is y = x / sqrt(mean(x^2) + eps) * weights, which the
+        products around it can compute between them (see NormedRows); None otherwise."""
+        return None
+
+
+class NormedRows:
+    """norm(x) where the norm has not run as a kernel of its own.
+
+    In a decode step a norm over a few rows is all launch latency, so the products around it
+    share it: the Linear that finished x (adding into the residual stream) has left
+    bf16(x * weights) and partial sums of x^2 (`prepared`), and the Linear that takes this object
+    as its input multiplies its sums by 1 / sqrt(mean(x^2) + eps).  A part says with
+    `takes_normed_rows = True` that it hands its input to a Linear unchanged; any other part is
+    given `tensor()`, which runs the norm's own kernel on x."""
+
+    def __init__(self, ctx: StepContext, norm: Norm, x: torch.Tensor, prepared=None):
+        self.ctx, self.norm, self.x = ctx, norm, x
+        self.prepared = prepared            # (h bf16 [T, D], ssq f32 [16, parts]) or None
+        self._tensor = None
+
+    @property
+    def shape(self):
+        return self.x.shape
+
+    def tensor(self) -> torch.Tensor:
+        if self._tensor is None:
+            self._tensor = self.norm.forward(self.ctx, self.x)
+        return self._tensor
 
 
 class PositionEncoding(Part):

@@ -16,9 +16,19 @@ class PreNormBlock(Block):
     def children(self):
         return [p for p in (self.mixer_norm, self.mixer, self.ffn_norm, self.ffn) if p is not None]
 
+    def first_norm(self):
+        """The norm this block applies to the residual stream on entry: the block before may
+        have it prepared (see NormedRows)."""
+        return self.mixer_norm
+
     def forward(self, ctx: StepContext, x) -> None:
-        h = self.mixer_norm.forward(ctx, x)
+        """x += mixer(norm(x)); x += ffn(norm(x))."""
+        after = ctx.norm_after_block                # the norm that meets x after this block, if the caller knows it
+        h = ctx.normed(self.mixer_norm, x, self.mixer)
+        ctx.norm_after = self.ffn_norm if self.ffn is not None else after
         self.mixer.forward(ctx, h, x)
         if self.ffn is not None:
-            h = self.ffn_norm.forward(ctx, x)
+            h = ctx.normed(self.ffn_norm, x, self.ffn)
+            ctx.norm_after = after
             self.ffn.forward(ctx, h, x)
+        ctx.norm_after = None

@@ -8,7 +8,7 @@ import torch
 
 from .. import kernels
 from ..weights import TensorSpec
-from .base import Part, Runtime, StepContext
+from .base import NormedRows, Part, Runtime, StepContext
 
 
 class TokenEmbedding(Part):
@@ -50,7 +50,17 @@ class LMHead(Part):
             t = fetch.get(self.name)
             self.weight = (t.to(torch.float32) if runtime.is_f32 else t).contiguous()
 
-    def forward(self, ctx: StepContext, h: torch.Tensor) -> torch.Tensor:
+    takes_normed_rows = True   # the input goes to the product unchanged
+
+    def forward(self, ctx: StepContext, h) -> torch.Tensor:
+        """h: the final hidden rows, or NormedRows of them."""
         logits = ctx.ws.get("logits", (h.shape[0], self.V), torch.float32)
+        if isinstance(h, NormedRows):
+            rms = h.norm.rms_parameters()
+            hp = h.prepared[0] if h.prepared is not None else None
+            if hp is not None and rms is not None and kernels.gemm_links_norms(hp, self.weight, logits, kernels.EPI_STORE):
+                kernels.gemm_linked(hp, self.weight, logits, kernels.EPI_STORE, None, (h.prepared[1], h.x.shape[1], rms[1]))
+                return logits
+            h = h.tensor()
         kernels.gemm(h, self.weight, logits, kernels.EPI_STORE)
         return logits

@@ -10,6 +10,7 @@ from .linear import Linear
 
 class SwiGLU(FeedForward):
     graph_safe = True      # launches depend on device memory only
+    takes_normed_rows = True   # the input goes to a Linear unchanged
 
     def __init__(self, prefix: str, hidden_size: int, intermediate_size: int,
                  names=("gate_proj.weight", "up_proj.weight", "down_proj.weight")):
@@ -24,4 +25,4 @@ class SwiGLU(FeedForward):
     def forward(self, ctx: StepContext, h, residual) -> None:
         act = ctx.ws.get("ffn.act", (h.shape[0], self.F), ctx.dtype)
         self.gate_up.forward(h, act, kernels.EPI_SWIGLU)
-        self.down.forward(act, residual, kernels.EPI_ACCUMULATE)
+        self.down.forward(act, residual, kernels.EPI_ACCUMULATE, ctx)

@@ -11,7 +11,7 @@ import torch
 
 from .. import kernels
 from ..weights import TensorSpec
-from .base import Part, Runtime
+from .base import NormedRows, Part, Runtime
 
 
 class Linear(Part):
@@ -52,5 +52,30 @@ class Linear(Part):
             w = ws[0] if len(ws) == 1 else torch.cat(ws, dim=0)
         self.weight = w.contiguous()
 
-    def forward(self, a: torch.Tensor, out: torch.Tensor, epilogue: int = kernels.EPI_STORE) -> None:
-        kernels.gemm(a, self.weight, out, epilogue)
+    def forward(self, a, out: torch.Tensor, epilogue: int = kernels.EPI_STORE, ctx=None) -> None:
+        """out (=, +=, = silu-gated) a W^T.  `a` is a tensor, or NormedRows: rows whose norm the
+        products compute between them.  With `ctx` and the accumulating epilogue, the norm that
+        the context says comes after (`ctx.norm_after`) is prepared for the product that follows,
+        where the kernels can do that; the result is left in `ctx.prepared_norm`."""
+        prepared = None
+        if isinstance(a, NormedRows):
+            rms = a.norm.rms_parameters()
+            h = a.prepared[0] if a.prepared is not None else None
+            if h is not None and rms is not None and kernels.gemm_links_norms(h, self.weight, out, epilogue):
+                prepared = (a.prepared[1], a.x.shape[1], rms[1])
+                a = h
+            else:
+                a = a.tensor()
+        prepare = None
+        nxt = ctx.norm_after if ctx is not None and epilogue == kernels.EPI_ACCUMULATE else None
+        if nxt is not None and nxt.rms_parameters() is not None and kernels.gemm_links_norms(a, self.weight, out, epilogue):
+            T, N = out.shape
+            which = ctx.ws.flip("norm.prepared")
+            prepare = (nxt.rms_parameters()[0], ctx.ws.get(f"norm.prepared.h{which}", (T, N), torch.bfloat16),
+                       ctx.ws.get(f"norm.prepared.ssq{which}", (16, kernels.linked_norm_parts(N)), torch.float32))
+        if prepare is None and prepared is None:
+            kernels.gemm(a, self.weight, out, epilogue)
+            return
+        kernels.gemm_linked(a, self.weight, out, epilogue, prepare, prepared)
+        if prepare is not None:
+            ctx.prepared_norm = NormedRows(ctx, nxt, out, prepared=(prepare[1], prepare[2]))

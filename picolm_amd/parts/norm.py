@@ -30,6 +30,9 @@ class RMSNorm(Norm):
             w = w + self.weight_offset
         self.weight = w.contiguous()
 
+    def rms_parameters(self):
+        return self.weight, self.eps
+
     def forward(self, ctx: StepContext, x, rows=None, n_rows=None, out_name="norm.out"):
         n = x.shape[0] if rows is None else (n_rows if n_rows is not None else rows.numel())
         out = ctx.ws.get(out_name, (n, self.size), ctx.dtype)

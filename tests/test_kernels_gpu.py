@@ -175,6 +175,44 @@ def test_gemm_medium_batches_pick_their_splits():
             run_gemm(K().gemm, M, N, Kd, epi, torch.bfloat16, torch.bfloat16, cdt)
 
 
+@pytest.mark.parametrize("M", [1, 8, 16])
+@pytest.mark.parametrize("D", [48, 256, 4096])
+def test_gemm_with_a_norm_split_between_two_products(M, D):
+    """The product that finishes rows of the residual stream prepares the RMSNorm that follows
+    (bf16(x * w) and partial sums of x^2), the next product applies 1 / sqrt(mean(x^2) + eps) to
+    its sums: together they must give norm-then-product.  Rows of very different size, so that a
+    factor taken from the wrong row shows; every kernel that can be the consumer."""
+    g = torch.Generator().manual_seed(M * 31 + D)
+    eps, K1 = 1e-5, 192
+    x0 = torch.randn(M, D, generator=g) * (10.0 ** torch.arange(M).remainder(5).sub(2).float())[:, None]
+    a1 = torch.randn(M, K1, generator=g).to(torch.bfloat16)
+    w1 = (torch.randn(D, K1, generator=g) * 0.05).to(torch.bfloat16)
+    nw = 1.0 + 0.3 * torch.randn(D, generator=g)
+    x = x0.clone().to(DEV)
+    h = torch.full((M, D), float("nan"), dtype=torch.bfloat16, device=DEV)
+    ssq = torch.full((16, K().linked_norm_parts(D)), float("nan"), device=DEV)
+    K().gemm_linked(a1.to(DEV), w1.to(DEV), x, 1, prepare=(nw.to(DEV), h, ssq))
+    x_ref = x0.double() + a1.double() @ w1.double().T
+    assert (x.double().cpu() - x_ref).abs().max() <= tol(torch.float32, x_ref.abs().max().item()) + 1e-2 * 0
+    assert torch.equal(h.cpu(), (x.cpu() * nw).to(torch.bfloat16))          # from the very values it stored
+    total = ssq[:M].double().sum(dim=1).cpu()
+    want = (x.double().cpu() ** 2).sum(dim=1)
+    assert ((total - want).abs() <= 1e-5 * want + 1e-30).all()
+    normed = x.double().cpu() / torch.sqrt((x.double().cpu() ** 2).mean(dim=1, keepdim=True) + eps) * nw.double()
+    if D % 8:
+        return
+    for N2 in (48, 16 * 300 - 6, 16384 + 32, 40000):
+        if N2 > 20000 and D > 256:
+            continue                        # (a large reference product on the CPU for nothing new)
+        w2 = (torch.randn(N2, D, generator=g) * 0.1).to(torch.bfloat16)
+        for epi, cdt in ((0, torch.float32), (2, torch.bfloat16), (1, torch.float32)):
+            c = torch.randn(M, N2 // 2 if epi == 2 else N2, generator=g).to(cdt).to(DEV)
+            ref = gemm_ref(normed, w2, epi, c.clone())
+            K().gemm_linked(h, w2.to(DEV), c, epi, prepared=(ssq, D, eps))
+            err = (c.double().cpu() - ref).abs().max().item()
+            assert err <= tol(torch.bfloat16, ref.abs().max().item()), (M, D, N2, epi, err)
+
+
 def test_gemm_tiled_splits_a_partial_last_round():
     """300 tiles of 256x256 on 256 CUs: the columns past the first 256 tiles take the half-height
     tile in a launch of their own; the seam must not show in any epilogue."""
