@@ -48,8 +48,8 @@ int picolm_gemm_tiled_splitk(const void* A, const void* W, void* C, int c_dt, in
 
 // A decode step's products with an RMSNorm split between them, up to 16 rows.  A product with the
 // accumulating epilogue (skinny variant 0/1) can prepare the norm that follows: next_h[M][ldc] =
-// bf16(x * next_w) and next_ssq[16][next_parts] partial sums of x^2 (next_parts >= ceil(N / 16)).
-// A product whose input rows are such a next_h takes ssq[16][n_parts], the norm's row length and
+// bf16(x * next_w) and next_ssq[next_parts][16] partial sums of x^2 (next_parts >= ceil(N / 16)).
+// A product whose input rows are such a next_h takes ssq[n_parts][16], the norm's row length and
 // eps and multiplies its sums by 1 / sqrt(sum / len + eps).  tiled != 0: tile variant 12 or 13.
 int picolm_gemm_linked(const void* A, const void* W, void* C, int c_dt, int M, int N, int K, int64_t lda,
                        int64_t ldw, int64_t ldc, int epilogue, int tiled, int variant, const float* next_w,

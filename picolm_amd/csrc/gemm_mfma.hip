@@ -42,9 +42,9 @@ __device__ __forceinline__ float silu_mul(float g, float u) { return g / (1.0f +
 struct NormLink {
     const float* next_w;    // producer: weights of the norm that follows [N], or null
     bf16_t* next_h;         //   [M][ld of C] what the next product reads
-    float* next_ssq;        //   [16][next_parts] partial sums of x^2, one column per workgroup
+    float* next_ssq;        //   [next_parts][16] partial sums of x^2, one row of 16 per workgroup
     int next_parts;
-    const float* ssq;       // consumer: the partial sums a producer left [16][n_parts], or null
+    const float* ssq;       // consumer: the partial sums a producer left [n_parts][16], or null
     int n_parts;
     float inv_len, eps;     //   1 / row length of the norm, its eps
 };
@@ -60,11 +60,10 @@ __device__ __forceinline__ float row_scale_begin(const NormLink& k, int M) {
         if (m < M) {
             // eight loads are asked for before the first is added: one trip to memory, not eight
             constexpr int STRIDE = THREADS / 16;
-            const float* row = k.ssq + (size_t)m * k.n_parts;
             for (int p0 = threadIdx.x / 16; p0 < k.n_parts; p0 += 8 * STRIDE) {
                 float v[8];
 #pragma unroll
-                for (int i = 0; i < 8; ++i) v[i] = row[min(p0 + i * STRIDE, k.n_parts - 1)];
+                for (int i = 0; i < 8; ++i) v[i] = k.ssq[(size_t)min(p0 + i * STRIDE, k.n_parts - 1) * 16 + m];
 #pragma unroll
                 for (int i = 0; i < 8; ++i) mine += p0 + i * STRIDE < k.n_parts ? v[i] : 0.f;
             }
@@ -237,7 +236,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const bf16_t* _
         if (wave < 4 && lane < 16) link_scratch[wave][lane] = next_sq;
         __syncthreads();
         if (threadIdx.x < 16)
-            link.next_ssq[(size_t)threadIdx.x * link.next_parts + blockIdx.x] =
+            link.next_ssq[(size_t)blockIdx.x * 16 + threadIdx.x] =
                 link_scratch[0][threadIdx.x] + link_scratch[1][threadIdx.x] + link_scratch[2][threadIdx.x] + link_scratch[3][threadIdx.x];
     }
 }

@@ -347,9 +347,9 @@ def gemm_links_norms(a, w, c, epilogue: int) -> bool:
 def gemm_linked(a, w, c, epilogue: int, prepare=None, prepared=None) -> None:
     """The product of a decode step next to an RMSNorm that is split between two products.
 
-    prepare = (norm weights f32 [N], h_out bf16 [M, N], ssq_out f32 [16, parts]): with the
+    prepare = (norm weights f32 [N], h_out bf16 [M, N], ssq_out f32 [parts, 16]): with the
     accumulating epilogue, also leave h_out = bf16(c * weights) and the partial sums of c^2.
-    prepared = (ssq f32 [16, parts], row length of the norm, eps): `a` is such an h_out; the sums
+    prepared = (ssq f32 [parts, 16], row length of the norm, eps): `a` is such an h_out; the sums
     are multiplied by 1 / sqrt(sum(x^2) / length + eps)."""
     M, N, K = _gemm_shapes(a, w, c, epilogue)
     if not gemm_links_norms(a, w, c, epilogue):
@@ -364,14 +364,14 @@ def gemm_linked(a, w, c, epilogue: int, prepare=None, prepared=None) -> None:
         _dev("gemm_linked.norm_weight", nw, torch.float32, 1)
         _dev("gemm_linked.h_out", nh, torch.bfloat16, 2)
         _dev("gemm_linked.ssq_out", nssq, torch.float32, 2)
-        next_parts = nssq.shape[1]
-        if nw.numel() != N or tuple(nh.shape) != (M, N) or nssq.shape[0] != 16 or next_parts < linked_norm_parts(N):
+        next_parts = nssq.shape[0]
+        if nw.numel() != N or tuple(nh.shape) != (M, N) or nssq.shape[1] != 16 or next_parts < linked_norm_parts(N):
             raise KernelError("gemm_linked: the buffers for the next norm do not fit the product")
     if prepared is not None:
         ssq, norm_len, eps = prepared
         _dev("gemm_linked.ssq", ssq, torch.float32, 2)
-        n_parts = ssq.shape[1]
-        if ssq.shape[0] != 16 or norm_len != K:
+        n_parts = ssq.shape[0]
+        if ssq.shape[1] != 16 or norm_len != K:
             raise KernelError("gemm_linked: the statistics are not those of this product's input rows")
     tiled, variant = 0, 0
     if prepare is None and M > 4 and K % 64 == 0 and 16384 <= N <= 128 * 256:

@@ -174,7 +174,7 @@ class NormedRows:
 
     def __init__(self, ctx: StepContext, norm: Norm, x: torch.Tensor, prepared=None):
         self.ctx, self.norm, self.x = ctx, norm, x
-        self.prepared = prepared            # (h bf16 [T, D], ssq f32 [16, parts]) or None
+        self.prepared = prepared            # (h bf16 [T, D], ssq f32 [parts, 16]) or None
         self._tensor = None
 
     @property

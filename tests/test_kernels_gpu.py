@@ -190,12 +190,12 @@ def test_gemm_with_a_norm_split_between_two_products(M, D):
     nw = 1.0 + 0.3 * torch.randn(D, generator=g)
     x = x0.clone().to(DEV)
     h = torch.full((M, D), float("nan"), dtype=torch.bfloat16, device=DEV)
-    ssq = torch.full((16, K().linked_norm_parts(D)), float("nan"), device=DEV)
+    ssq = torch.full((K().linked_norm_parts(D), 16), float("nan"), device=DEV)
     K().gemm_linked(a1.to(DEV), w1.to(DEV), x, 1, prepare=(nw.to(DEV), h, ssq))
     x_ref = x0.double() + a1.double() @ w1.double().T
     assert (x.double().cpu() - x_ref).abs().max() <= tol(torch.float32, x_ref.abs().max().item()) + 1e-2 * 0
     assert torch.equal(h.cpu(), (x.cpu() * nw).to(torch.bfloat16))          # from the very values it stored
-    total = ssq[:M].double().sum(dim=1).cpu()
+    total = ssq[:, :M].double().sum(dim=0).cpu()
     want = (x.double().cpu() ** 2).sum(dim=1)
     assert ((total - want).abs() <= 1e-5 * want + 1e-30).all()
     normed = x.double().cpu() / torch.sqrt((x.double().cpu() ** 2).mean(dim=1, keepdim=True) + eps) * nw.double()
