@@ -46,15 +46,18 @@ int picolm_gemm_tiled_splitk(const void* A, const void* W, void* C, int c_dt, in
                              int64_t ldw, int64_t ldc, int epilogue, int variant, int splits, float* ws,
                              hipStream_t stream);
 
-// A decode step's products with an RMSNorm split between them, up to 16 rows.  A product with the
-// accumulating epilogue (skinny variant 0/1) can prepare the norm that follows: next_h[M][ldc] =
-// bf16(x * next_w) and next_ssq[next_parts][16] partial sums of x^2 (next_parts >= ceil(N / 16)).
-// A product whose input rows are such a next_h takes ssq[n_parts][16], the norm's row length and
-// eps and multiplies its sums by 1 / sqrt(sum / len + eps).  tiled != 0: tile variant 12 or 13.
+// A decode step's products with an RMSNorm split between them.  A product with the accumulating
+// epilogue can prepare the norm that follows: next_h[M][ldc] = bf16(x * next_w) and
+// next_ssq[next_parts][rows], one row of partial sums of x^2 per workgroup.  A product whose input
+// rows are such a next_h takes ssq[n_parts][rows], the norm's row length and eps and multiplies
+// its sums by 1 / sqrt(sum / len + eps).  Up to 16 rows (rows = 16): skinny variant 0/1 (either
+// role), 7, or tiled != 0 with tile variant 12/13 (taking only).  17 to 64 rows (rows = 64): tiled,
+// variant 12; cut along K (splits > 1, ws of splits * M * N floats, N a multiple of 1024) either
+// role, uncut taking only.
 int picolm_gemm_linked(const void* A, const void* W, void* C, int c_dt, int M, int N, int K, int64_t lda,
-                       int64_t ldw, int64_t ldc, int epilogue, int tiled, int variant, const float* next_w,
-                       void* next_h, float* next_ssq, int next_parts, const float* ssq, int n_parts,
-                       int norm_len, float eps, hipStream_t stream);
+                       int64_t ldw, int64_t ldc, int epilogue, int tiled, int variant, int splits, float* ws,
+                       const float* next_w, void* next_h, float* next_ssq, int next_parts, const float* ssq,
+                       int n_parts, int norm_len, float eps, int rows, hipStream_t stream);
 
 int picolm_attn_prefill_tile_rows(void);
 int picolm_attn_prefill_generic(const void* q, const void* k_pages, const void* v_pages, void* out,

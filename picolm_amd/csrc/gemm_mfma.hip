@@ -42,44 +42,46 @@ __device__ __forceinline__ float silu_mul(float g, float u) { return g / (1.0f +
 struct NormLink {
     const float* next_w;    // producer: weights of the norm that follows [N], or null
     bf16_t* next_h;         //   [M][ld of C] what the next product reads
-    float* next_ssq;        //   [next_parts][16] partial sums of x^2, one row of 16 per workgroup
+    float* next_ssq;        //   [next_parts][rows] partial sums of x^2, one row per workgroup
     int next_parts;
-    const float* ssq;       // consumer: the partial sums a producer left [n_parts][16], or null
+    const float* ssq;       // consumer: the partial sums a producer left [n_parts][rows], or null
     int n_parts;
     float inv_len, eps;     //   1 / row length of the norm, its eps
+    int rows;               // 16 (products of up to 16 rows) or 64: rows that the sums are kept for
 };
 
-// Consumer side.  `begin` has every thread ask for its share of the partial sums (row tid % 16,
-// every (THREADS/16)-th part) before the main loop; `finish` adds them up in a fixed order and
-// leaves the 16 row factors in LDS.  Both are called by all THREADS threads of the workgroup.
+// Consumer side.  `begin` has every thread ask for its share of the partial sums (row tid % rows,
+// every (THREADS/rows)-th part) before the main loop; `finish` adds them up in a fixed order and
+// leaves the row factors in LDS.  Both are called by all THREADS threads of the workgroup.
 template <int THREADS>
 __device__ __forceinline__ float row_scale_begin(const NormLink& k, int M) {
     float mine = 0.f;
     if (k.ssq) {
-        const int m = threadIdx.x % 16;
+        const int m = threadIdx.x % k.rows, stride = THREADS / k.rows;
         if (m < M) {
             // eight loads are asked for before the first is added: one trip to memory, not eight
-            constexpr int STRIDE = THREADS / 16;
-            for (int p0 = threadIdx.x / 16; p0 < k.n_parts; p0 += 8 * STRIDE) {
+            for (int p0 = threadIdx.x / k.rows; p0 < k.n_parts; p0 += 8 * stride) {
                 float v[8];
 #pragma unroll
-                for (int i = 0; i < 8; ++i) v[i] = k.ssq[(size_t)min(p0 + i * STRIDE, k.n_parts - 1) * 16 + m];
+                for (int i = 0; i < 8; ++i) v[i] = k.ssq[(size_t)min(p0 + i * stride, k.n_parts - 1) * k.rows + m];
 #pragma unroll
-                for (int i = 0; i < 8; ++i) mine += p0 + i * STRIDE < k.n_parts ? v[i] : 0.f;
+                for (int i = 0; i < 8; ++i) mine += p0 + i * stride < k.n_parts ? v[i] : 0.f;
             }
         }
     }
     return mine;
 }
 template <int THREADS>
-__device__ __forceinline__ void row_scale_finish(const NormLink& k, float mine, float (&scratch)[THREADS / 64][16],
-                                                 float (&scale)[16]) {
+__device__ __forceinline__ void row_scale_finish(const NormLink& k, float mine, float (&scratch)[THREADS / 64][64],
+                                                 float (&scale)[64]) {
     if (!k.ssq) return;          // uniform over the workgroup
-    mine += __shfl_xor(mine, 16, WAVE);
-    mine += __shfl_xor(mine, 32, WAVE);
-    if (threadIdx.x % 64 < 16) scratch[threadIdx.x / 64][threadIdx.x % 16] = mine;
+    if (k.rows == 16) {          // four lanes of a wave share a row
+        mine += __shfl_xor(mine, 16, WAVE);
+        mine += __shfl_xor(mine, 32, WAVE);
+    }
+    if ((int)(threadIdx.x % 64) < k.rows) scratch[threadIdx.x / 64][threadIdx.x % 64] = mine;
     __syncthreads();
-    if (threadIdx.x < 16) {
+    if ((int)threadIdx.x < k.rows) {
         float total = 0.f;
 #pragma unroll
         for (int w = 0; w < THREADS / 64; ++w) total += scratch[w][threadIdx.x];
@@ -99,7 +101,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const bf16_t* _
                                                                  TC* __restrict__ C, int M, int N, int K,
                                                                  int64_t lda, int64_t ldw, int64_t ldc, NormLink link) {
     extern __shared__ float red[];      // [WAVES][NT][MT][4][64]
-    __shared__ float link_scratch[WAVES][16], link_scale[16];
+    __shared__ float link_scratch[WAVES][64], link_scale[64];
     const float link_mine = row_scale_begin<WAVES * 64>(link, M);
     const int wave = threadIdx.x / 64, lane = threadIdx.x % 64;
     const int r16 = lane % 16, q = lane / 16;
@@ -236,7 +238,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const bf16_t* _
         if (wave < 4 && lane < 16) link_scratch[wave][lane] = next_sq;
         __syncthreads();
         if (threadIdx.x < 16)
-            link.next_ssq[(size_t)blockIdx.x * 16 + threadIdx.x] =
+            link.next_ssq[(size_t)blockIdx.x * link.rows + threadIdx.x] =
                 link_scratch[0][threadIdx.x] + link_scratch[1][threadIdx.x] + link_scratch[2][threadIdx.x] + link_scratch[3][threadIdx.x];
     }
 }
@@ -246,7 +248,8 @@ static int launch_skinny(const void* A, const void* W, void* C, int c_dt, int M,
                          int64_t ldw, int64_t ldc, int epi, hipStream_t stream, NormLink link = NormLink{}) {
     PICOLM_REQUIRE(!link.next_w || (MT == 1 && NT == 1 && WAVES == 8 && epi == 1 && link.next_parts >= ceil_div(N, 16)),
                    "gemm_skinny: only the 16x16 tile with the accumulating epilogue prepares a norm");
-    PICOLM_REQUIRE(!link.ssq || M <= 16, "gemm_skinny: a norm's statistics are taken for up to 16 rows, got %d", M);
+    PICOLM_REQUIRE((!link.ssq && !link.next_w) || (M <= 16 && link.rows == 16),
+                   "gemm_skinny: a split norm goes with up to 16 rows here, got %d", M);
     dim3 grid(ceil_div(N, 16 * NT)), block(WAVES * 64);
     const size_t lds = sizeof(float) * WAVES * NT * MT * 4 * 64;
     const bf16_t* a = (const bf16_t*)A;
@@ -287,7 +290,7 @@ __global__ __launch_bounds__(512) void gemm_skinny_resident_kernel(const bf16_t*
                                                                    int64_t lda, int64_t ldw, int64_t ldc, NormLink link) {
     constexpr int WAVES = 8;
     __shared__ float red[2][WAVES][4][64];
-    __shared__ float link_scratch[WAVES][16], link_scale[16];
+    __shared__ float link_scratch[WAVES][64], link_scale[64];
     const float link_mine = row_scale_begin<WAVES * 64>(link, M);
     const int wave = threadIdx.x / 64, lane = threadIdx.x % 64;
     const int r16 = lane % 16, q = lane / 16;
@@ -373,6 +376,7 @@ template <int STEPS>
 static int launch_skinny_resident(const void* A, const void* W, void* C, int c_dt, int M, int N, int K, int64_t lda,
                                   int64_t ldw, int64_t ldc, int epi, hipStream_t stream, NormLink link = NormLink{}) {
     PICOLM_REQUIRE(!link.next_w, "gemm_skinny: the resident variant prepares no norm");
+    PICOLM_REQUIRE(!link.ssq || link.rows == 16, "gemm_skinny: a split norm goes with up to 16 rows here");
     PICOLM_REQUIRE(M <= 16 && K % SK_KSTEP == 0 && K <= STEPS * 8 * SK_KSTEP,
                    "gemm_skinny: the resident variant takes M <= 16 and K a multiple of %d up to %d, got M=%d K=%d",
                    SK_KSTEP, STEPS * 8 * SK_KSTEP, M, K);
@@ -701,7 +705,7 @@ __global__ __launch_bounds__(64 * WN * WM) void gemm_direct_kernel(const bf16_t*
                                                                    int64_t lda, int64_t ldw, int64_t ldc,
                                                                    int tiles_m, int tiles_n, int64_t c_split_stride,
                                                                    NormLink link) {
-    __shared__ float link_scratch[WN * WM][16], link_scale[16];
+    __shared__ float link_scratch[WN * WM][64], link_scale[64];
     const float link_mine = row_scale_begin<64 * WN * WM>(link, M);
     // K here is the length of one split: workgroup row y of the grid takes columns y*K .. of A
     // and W and writes its sums to C + y * c_split_stride
@@ -861,7 +865,7 @@ __global__ __launch_bounds__(64 * WN * WM) void gemm_direct_kernel(const bf16_t*
             for (int e = 0; e < 16; ++e) {
                 const int m = m0 + wm + 32 * j + 8 * (e / 4) + 4 * kq + e % 4;
                 float v = acc[i][j][e];
-                if (link.ssq && m < 16) v *= link_scale[m];      // (the host admits this for M <= 16 only)
+                if (link.ssq && m < link.rows) v *= link_scale[m];     // (one row of tiles: the host sees to that)
                 if (EPI == 2) {
                     const float up = __shfl_xor(v, 1, WAVE);
                     if (m < M && (l32 & 1) == 0 && n + 1 < N) C[(int64_t)m * ldc + n / 2] = from_f32<TC>(silu_mul(v, up));
@@ -879,9 +883,9 @@ static int launch_direct(const void* A, const void* W, void* C, int c_dt, int M,
                          int64_t ldw, int64_t ldc, int epilogue, hipStream_t stream, int splits = 1,
                          int64_t c_split_stride = 0, NormLink link = NormLink{}) {
     PICOLM_REQUIRE(!link.next_w, "gemm_tiled: the tiled kernels prepare no norm");
-    PICOLM_REQUIRE(!link.ssq || (M <= 16 && splits == 1),
-                   "gemm_tiled: a norm's statistics are taken for up to 16 rows of an uncut product");
     constexpr int BN = 32 * TN * WN, BM = 32 * TM * WM;
+    PICOLM_REQUIRE(!link.ssq || (M <= link.rows && M <= BM && splits == 1 && (link.rows == 16 || link.rows == 64)),
+                   "gemm_tiled: a norm's statistics are taken for one row of tiles of an uncut product");
     PICOLM_REQUIRE(splits >= 1 && K % (BK * splits) == 0,
                    "gemm_tiled: K = %d is no multiple of %d times %d splits, which this variant needs", K, BK, splits);
     PICOLM_REQUIRE((int64_t)BN * ldw < (1ll << 30) && (int64_t)BM * lda < (1ll << 30),
@@ -922,36 +926,72 @@ static int launch_direct(const void* A, const void* W, void* C, int c_dt, int M,
 // A product with few output tiles is cut along K so that every CU has a workgroup: split z
 // writes its partial sums to ws[z][M][N]; the kernel below adds the splits in order (the same
 // order every time) and applies the epilogue.
+// With a split norm (NormLink) N is a multiple of 1024, so that the 1024 values of a workgroup lie
+// in one row: as the consumer it multiplies the sums by the row's factor; as the producer (epilogue
+// 1) it leaves bf16(x * w) and one partial sum of x^2 per workgroup.
 template <int EPI, typename TC>
 __global__ __launch_bounds__(256) void splitk_reduce_kernel(const float* __restrict__ ws, TC* __restrict__ C, int M, int N,
-                                                            int64_t ldc, int splits) {
-    constexpr int PER = EPI == 2 ? 2 : 1;
+                                                            int64_t ldc, int splits, NormLink link) {
+    __shared__ float wave_sq[4];
     const int64_t i = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) * 4;      // four floats of a row
-    if (i >= (int64_t)M * N) return;
-    const int m = (int)(i / N), n = (int)(i % N);        // N is a multiple of 4 (the host sees to that)
+    const bool inside = i < (int64_t)M * N;      // (always, with a split norm)
+    const int m = inside ? (int)(i / N) : 0, n = inside ? (int)(i % N) : 0;      // N is a multiple of 4 (the host sees to that)
     f32x4 sum = {0.f, 0.f, 0.f, 0.f};
-    for (int z = 0; z < splits; ++z) sum += *(const f32x4*)(ws + (int64_t)z * M * N + i);
-    if (EPI == 2) {
-        TC* p = C + (int64_t)m * ldc + n / 2;
-        p[0] = from_f32<TC>(silu_mul(sum[0], sum[1]));
-        p[1] = from_f32<TC>(silu_mul(sum[2], sum[3]));
-    } else {
-        TC* p = C + (int64_t)m * ldc + n;
+    if (inside)
+        for (int z = 0; z < splits; ++z) sum += *(const f32x4*)(ws + (int64_t)z * M * N + i);
+    if (link.ssq) {
+        float total = 0.f;      // (eight loads asked for at a time, as in row_scale_begin)
+        for (int p0 = 0; p0 < link.n_parts; p0 += 8) {
+            float v[8];
 #pragma unroll
-        for (int e = 0; e < 4; ++e) p[e] = from_f32<TC>(EPI == 1 ? to_f32<TC>(p[e]) + sum[e] : sum[e]);
+            for (int e = 0; e < 8; ++e) v[e] = link.ssq[(size_t)min(p0 + e, link.n_parts - 1) * link.rows + m];
+#pragma unroll
+            for (int e = 0; e < 8; ++e) total += p0 + e < link.n_parts ? v[e] : 0.f;
+        }
+        sum *= 1.0f / sqrtf(total * link.inv_len + link.eps);
     }
-    (void)PER;
+    float sq = 0.f;
+    if (inside) {
+        if (EPI == 2) {
+            TC* p = C + (int64_t)m * ldc + n / 2;
+            p[0] = from_f32<TC>(silu_mul(sum[0], sum[1]));
+            p[1] = from_f32<TC>(silu_mul(sum[2], sum[3]));
+        } else {
+            TC* p = C + (int64_t)m * ldc + n;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const float x = EPI == 1 ? to_f32<TC>(p[e]) + sum[e] : sum[e];
+                p[e] = from_f32<TC>(x);
+                if (EPI == 1 && link.next_w) {
+                    link.next_h[(int64_t)m * ldc + n + e] = f32_to_bf16_bits(x * link.next_w[n + e]);
+                    sq += x * x;
+                }
+            }
+        }
+    }
+    if (EPI == 1 && link.next_w) {
+#pragma unroll
+        for (int o = 32; o > 0; o >>= 1) sq += __shfl_xor(sq, o, WAVE);
+        if (threadIdx.x % 64 == 0) wave_sq[threadIdx.x / 64] = sq;
+        __syncthreads();
+        if (threadIdx.x == 0)
+            link.next_ssq[(size_t)(blockIdx.x % (N / 1024)) * link.rows + m] = wave_sq[0] + wave_sq[1] + wave_sq[2] + wave_sq[3];
+    }
 }
 
 static int launch_splitk_reduce(const float* ws, void* C, int c_dt, int M, int N, int64_t ldc, int splits, int epilogue,
-                                hipStream_t stream) {
+                                hipStream_t stream, NormLink link = NormLink{}) {
+    PICOLM_REQUIRE((!link.ssq && !link.next_w) || (N % 1024 == 0 && M <= link.rows && (link.rows == 16 || link.rows == 64)),
+                   "gemm_splitk: a split norm needs N (%d) in multiples of 1024 and up to %d rows", N, link.rows);
+    PICOLM_REQUIRE(!link.next_w || (epilogue == 1 && link.next_parts >= N / 1024),
+                   "gemm_splitk: only the accumulating epilogue prepares a norm");
     const int64_t quads = (int64_t)M * N / 4;
     dim3 grid((unsigned)ceil_div64(quads, 256)), block(256);
-    if (epilogue == 0 && c_dt == PICOLM_F32) splitk_reduce_kernel<0, float><<<grid, block, 0, stream>>>(ws, (float*)C, M, N, ldc, splits);
-    else if (epilogue == 0 && c_dt == PICOLM_BF16) splitk_reduce_kernel<0, bf16_t><<<grid, block, 0, stream>>>(ws, (bf16_t*)C, M, N, ldc, splits);
-    else if (epilogue == 1 && c_dt == PICOLM_F32) splitk_reduce_kernel<1, float><<<grid, block, 0, stream>>>(ws, (float*)C, M, N, ldc, splits);
-    else if (epilogue == 2 && c_dt == PICOLM_BF16) splitk_reduce_kernel<2, bf16_t><<<grid, block, 0, stream>>>(ws, (bf16_t*)C, M, N, ldc, splits);
-    else if (epilogue == 2 && c_dt == PICOLM_F32) splitk_reduce_kernel<2, float><<<grid, block, 0, stream>>>(ws, (float*)C, M, N, ldc, splits);
+    if (epilogue == 0 && c_dt == PICOLM_F32) splitk_reduce_kernel<0, float><<<grid, block, 0, stream>>>(ws, (float*)C, M, N, ldc, splits, link);
+    else if (epilogue == 0 && c_dt == PICOLM_BF16) splitk_reduce_kernel<0, bf16_t><<<grid, block, 0, stream>>>(ws, (bf16_t*)C, M, N, ldc, splits, link);
+    else if (epilogue == 1 && c_dt == PICOLM_F32) splitk_reduce_kernel<1, float><<<grid, block, 0, stream>>>(ws, (float*)C, M, N, ldc, splits, link);
+    else if (epilogue == 2 && c_dt == PICOLM_BF16) splitk_reduce_kernel<2, bf16_t><<<grid, block, 0, stream>>>(ws, (bf16_t*)C, M, N, ldc, splits, link);
+    else if (epilogue == 2 && c_dt == PICOLM_F32) splitk_reduce_kernel<2, float><<<grid, block, 0, stream>>>(ws, (float*)C, M, N, ldc, splits, link);
     else PICOLM_REQUIRE(false, "gemm_splitk: unsupported epilogue %d with output dtype %d", epilogue, c_dt);
     PICOLM_LAUNCH_CHECK("gemm_splitk_reduce");
     return 0;
@@ -1032,21 +1072,34 @@ extern "C" int picolm_gemm_tiled_splitk(const void* A, const void* W, void* C, i
     return launch_splitk_reduce(ws, C, c_dt, M, N, ldc, splits, epilogue, stream);
 }
 
-// The products of a decode step with a norm split between them (see NormLink): `variant` as in
-// picolm_gemm_skinny (0, 1, 7) or, with tiled != 0, a tile variant of picolm_gemm_tiled that
-// loads straight into LDS (12, 13).  next_*: this product (epilogue 1, skinny variant 0 or 1)
-// prepares the norm that follows; ssq, n_parts, norm_len, eps: this product's input rows are
-// the next_h of a product that prepared their norm.  Up to 16 rows.
+// The products of a decode step with a norm split between them (see NormLink).  Up to 16 rows:
+// `variant` as in picolm_gemm_skinny (0, 1, 7) or, with tiled != 0, tile variant 12 or 13; rows = 16.
+// 17 to 64 rows: tiled, variant 12, rows = 64; with splits > 1 (ws as in picolm_gemm_tiled_splitk)
+// the kernel that adds the parts takes either role and N must be a multiple of 1024; uncut, the
+// tile kernel can only take a prepared norm's statistics.
+// next_*: this product (epilogue 1) prepares the norm that follows: next_h[M][ldc] and
+// next_ssq[next_parts][rows], one row of partial sums per workgroup (ceil(N/16) of the skinny
+// kernel, N/1024 of the adding kernel).  ssq, n_parts, norm_len, eps: this product's input rows
+// are the next_h of a product that prepared their norm.
 extern "C" int picolm_gemm_linked(const void* A, const void* W, void* C, int c_dt, int M, int N, int K, int64_t lda,
-                                  int64_t ldw, int64_t ldc, int epilogue, int tiled, int variant,
-                                  const float* next_w, void* next_h, float* next_ssq, int next_parts,
-                                  const float* ssq, int n_parts, int norm_len, float eps, hipStream_t stream) {
+                                  int64_t ldw, int64_t ldc, int epilogue, int tiled, int variant, int splits,
+                                  float* ws, const float* next_w, void* next_h, float* next_ssq, int next_parts,
+                                  const float* ssq, int n_parts, int norm_len, float eps, int rows,
+                                  hipStream_t stream) {
     if (check_mfma_operands("gemm_linked", A, W, M, N, K, lda, ldw, ldc, epilogue, c_dt)) return -1;
-    PICOLM_REQUIRE(M <= 16, "gemm_linked: up to 16 rows, got %d", M);
+    PICOLM_REQUIRE((rows == 16 || rows == 64) && M <= rows, "gemm_linked: %d rows with sums kept for %d", M, rows);
     PICOLM_REQUIRE(!next_w || (next_h && next_ssq && next_parts > 0), "gemm_linked: an incomplete description of the next norm");
     PICOLM_REQUIRE(!ssq || (n_parts > 0 && norm_len > 0), "gemm_linked: an incomplete description of the norm's statistics");
+    PICOLM_REQUIRE(splits >= 1 && splits <= 64, "gemm_linked: %d splits", splits);
     if (M == 0) return 0;
-    NormLink link = {next_w, (bf16_t*)next_h, next_ssq, next_parts, ssq, n_parts, norm_len > 0 ? 1.0f / (float)norm_len : 0.f, eps};
+    NormLink link = {next_w, (bf16_t*)next_h, next_ssq, next_parts, ssq, n_parts, norm_len > 0 ? 1.0f / (float)norm_len : 0.f, eps, rows};
+    if (tiled && splits > 1) {
+        PICOLM_REQUIRE(variant == 12 && ws != nullptr && ((uintptr_t)ws & 15) == 0 && N % 4 == 0,
+                       "gemm_linked: a cut product needs tile variant 12, a workspace and N in multiples of 4");
+        const int rc = launch_direct<1, 2, 4, 1, 64, 3>(A, W, ws, PICOLM_F32, M, N, K, lda, ldw, N, 0, stream, splits, (int64_t)M * N);
+        if (rc) return rc;
+        return launch_splitk_reduce(ws, C, c_dt, M, N, ldc, splits, epilogue, stream, link);
+    }
     if (tiled) {
         switch (variant) {
             case 12: return launch_direct<1, 2, 4, 1, 64, 3>(A, W, C, c_dt, M, N, K, lda, ldw, ldc, epilogue, stream, 1, 0, link);

@@ -329,31 +329,63 @@ def mfma_gemm_takes(a, w, c, epilogue: int) -> bool:
     return True
 
 
-LINKED_NORM_MAX_M = 16
+def medium_gemm_splits(M: int, N: int, K: int) -> int:
+    """Into how many parts along K a product of 17..64 rows is cut: its tiles hold 128 weight
+    rows each, and every CU should have one."""
+    tiles = (N + 127) // 128
+    if tiles >= 200 or N % 4:
+        return 1
+    s = 8
+    while s > 1 and (tiles * s > 320 or K % (64 * s) or s * M * N > SPLITK_WS_FLOATS):
+        s //= 2
+    return s
 
 
-def linked_norm_parts(N: int) -> int:
-    """Partial sums per row that a product of N output columns leaves for the norm that follows."""
-    return (N + 15) // 16
+LINKED_NORM_MAX_M = 64
 
 
-def gemm_links_norms(a, w, c, epilogue: int) -> bool:
-    """Whether the product for these operands can take part in a norm split between two products
-    (prepare the next one with the accumulating epilogue, or take a prepared one's statistics):
-    the matrix-core kernels for up to 16 rows."""
-    return a.shape[0] <= LINKED_NORM_MAX_M and a.dim() == 2 and mfma_gemm_takes(a, w, c, epilogue)
+def linked_norm_rows(M: int) -> int:
+    """Rows that the partial sums of a split norm are kept for in a step of M rows."""
+    return 16 if M <= 16 else 64
+
+
+def linked_norm_parts(M: int, N: int) -> int:
+    """Partial sums per row that a product of M rows and N output columns leaves for the norm
+    that follows: one per workgroup of the kernel that finishes the rows."""
+    return (N + 15) // 16 if M <= 16 else N // 1024
+
+
+def gemm_links_norms(a, w, c, epilogue: int, prepares: bool) -> bool:
+    """Whether the product for these operands can take part in a norm split between two products:
+    prepare the next one (with the accumulating epilogue), or else take a prepared one's
+    statistics.  Up to 16 rows every matrix-core product can do both.  For 17 to 64 rows the
+    kernel that adds the parts of a product cut along K does either for N in multiples of 1024,
+    and the tile kernel of an uncut product can take the statistics."""
+    if a.dim() != 2 or a.shape[0] > LINKED_NORM_MAX_M or not mfma_gemm_takes(a, w, c, epilogue):
+        return False
+    M, N, K = a.shape[0], w.shape[0], a.shape[1]
+    if M <= 16:
+        return True
+    if K % 64:
+        return False
+    cut = medium_gemm_splits(M, N, K) > 1
+    return (cut and N % 1024 == 0) if prepares else (not cut or N % 1024 == 0)
 
 
 def gemm_linked(a, w, c, epilogue: int, prepare=None, prepared=None) -> None:
     """The product of a decode step next to an RMSNorm that is split between two products.
 
-    prepare = (norm weights f32 [N], h_out bf16 [M, N], ssq_out f32 [parts, 16]): with the
+    prepare = (norm weights f32 [N], h_out bf16 [M, N], ssq_out f32 [parts, rows]): with the
     accumulating epilogue, also leave h_out = bf16(c * weights) and the partial sums of c^2.
-    prepared = (ssq f32 [parts, 16], row length of the norm, eps): `a` is such an h_out; the sums
-    are multiplied by 1 / sqrt(sum(x^2) / length + eps)."""
+    prepared = (ssq f32 [parts, rows], row length of the norm, eps): `a` is such an h_out; the
+    sums are multiplied by 1 / sqrt(sum(x^2) / length + eps).  rows and parts as
+    linked_norm_rows / linked_norm_parts say for the step's M."""
     M, N, K = _gemm_shapes(a, w, c, epilogue)
-    if not gemm_links_norms(a, w, c, epilogue):
-        raise KernelError(f"gemm_linked: a {tuple(a.shape)} {a.dtype}, w {tuple(w.shape)} {w.dtype} are not taken")
+    for role, prepares in ((prepare, True), (prepared, False)):
+        if role is not None and not gemm_links_norms(a, w, c, epilogue, prepares):
+            raise KernelError(f"gemm_linked: a {tuple(a.shape)} {a.dtype}, w {tuple(w.shape)} {w.dtype} cannot "
+                              f"{'prepare a norm' if prepares else 'take a prepared norm'}")
+    rows = linked_norm_rows(M)
     nw = nh = nssq = ssq = None
     next_parts = n_parts = norm_len = 0
     eps = 0.0
@@ -365,32 +397,24 @@ def gemm_linked(a, w, c, epilogue: int, prepare=None, prepared=None) -> None:
         _dev("gemm_linked.h_out", nh, torch.bfloat16, 2)
         _dev("gemm_linked.ssq_out", nssq, torch.float32, 2)
         next_parts = nssq.shape[0]
-        if nw.numel() != N or tuple(nh.shape) != (M, N) or nssq.shape[1] != 16 or next_parts < linked_norm_parts(N):
+        if nw.numel() != N or tuple(nh.shape) != (M, N) or nssq.shape[1] != rows or next_parts != linked_norm_parts(M, N):
             raise KernelError("gemm_linked: the buffers for the next norm do not fit the product")
     if prepared is not None:
         ssq, norm_len, eps = prepared
         _dev("gemm_linked.ssq", ssq, torch.float32, 2)
         n_parts = ssq.shape[0]
-        if ssq.shape[1] != 16 or norm_len != K:
+        if ssq.shape[1] != rows or norm_len != K:
             raise KernelError("gemm_linked: the statistics are not those of this product's input rows")
-    tiled, variant = 0, 0
-    if prepare is None and M > 4 and K % 64 == 0 and 16384 <= N <= 128 * 256:
+    tiled, variant, splits, ws = 0, 0, 1, None
+    if M > 16:
+        tiled, variant, splits = 1, 12, medium_gemm_splits(M, N, K)          # as in gemm()
+        ws = splitk_workspace(a.device) if splits > 1 else None
+    elif prepare is None and M > 4 and K % 64 == 0 and 16384 <= N <= 128 * 256:
         tiled, variant = 1, 13          # as in gemm()
     _check(lib().picolm_gemm_linked(_ptr(a), _ptr(w), _ptr(c), dt_of(c), M, N, K, c_int64(K), c_int64(K),
-                                    c_int64(c.shape[1]), epilogue, tiled, variant, _ptr(nw), _ptr(nh), _ptr(nssq), next_parts,
-                                    _ptr(ssq), n_parts, int(norm_len), c_float(eps), _stream()))
-
-
-def medium_gemm_splits(M: int, N: int, K: int) -> int:
-    """Into how many parts along K a product of 17..64 rows is cut: its tiles hold 128 weight
-    rows each, and every CU should have one."""
-    tiles = (N + 127) // 128
-    if tiles >= 200 or N % 4:
-        return 1
-    s = 8
-    while s > 1 and (tiles * s > 320 or K % (64 * s) or s * M * N > SPLITK_WS_FLOATS):
-        s //= 2
-    return s
+                                    c_int64(c.shape[1]), epilogue, tiled, variant, splits, _ptr(ws),
+                                    _ptr(nw), _ptr(nh), _ptr(nssq), next_parts,
+                                    _ptr(ssq), n_parts, int(norm_len), c_float(eps), rows, _stream()))
 
 
 def gemm(a: torch.Tensor, w: torch.Tensor, c: torch.Tensor, epilogue: int = EPI_STORE) -> None:

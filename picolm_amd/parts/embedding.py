@@ -58,7 +58,7 @@ class LMHead(Part):
         if isinstance(h, NormedRows):
             rms = h.norm.rms_parameters()
             hp = h.prepared[0] if h.prepared is not None else None
-            if hp is not None and rms is not None and kernels.gemm_links_norms(hp, self.weight, logits, kernels.EPI_STORE):
+            if hp is not None and rms is not None and kernels.gemm_links_norms(hp, self.weight, logits, kernels.EPI_STORE, prepares=False):
                 kernels.gemm_linked(hp, self.weight, logits, kernels.EPI_STORE, None, (h.prepared[1], h.x.shape[1], rms[1]))
                 return logits
             h = h.tensor()

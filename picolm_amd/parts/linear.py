@@ -61,18 +61,19 @@ class Linear(Part):
         if isinstance(a, NormedRows):
             rms = a.norm.rms_parameters()
             h = a.prepared[0] if a.prepared is not None else None
-            if h is not None and rms is not None and kernels.gemm_links_norms(h, self.weight, out, epilogue):
+            if h is not None and rms is not None and kernels.gemm_links_norms(h, self.weight, out, epilogue, prepares=False):
                 prepared = (a.prepared[1], a.x.shape[1], rms[1])
                 a = h
             else:
                 a = a.tensor()
         prepare = None
         nxt = ctx.norm_after if ctx is not None and epilogue == kernels.EPI_ACCUMULATE else None
-        if nxt is not None and nxt.rms_parameters() is not None and kernels.gemm_links_norms(a, self.weight, out, epilogue):
+        if nxt is not None and nxt.rms_parameters() is not None and kernels.gemm_links_norms(a, self.weight, out, epilogue, prepares=True):
             T, N = out.shape
             which = ctx.ws.flip("norm.prepared")
             prepare = (nxt.rms_parameters()[0], ctx.ws.get(f"norm.prepared.h{which}", (T, N), torch.bfloat16),
-                       ctx.ws.get(f"norm.prepared.ssq{which}", (kernels.linked_norm_parts(N), 16), torch.float32))
+                       ctx.ws.get(f"norm.prepared.ssq{which}", (kernels.linked_norm_parts(T, N), kernels.linked_norm_rows(T)),
+                                  torch.float32))
         if prepare is None and prepared is None:
             kernels.gemm(a, self.weight, out, epilogue)
             return
