@@ -89,10 +89,14 @@ int picolm_attn_prefill_mfma(const void* q, const void* k_pages, const void* v_p
                              const int32_t* cu_seqlens, const int32_t* page_table, int max_pages,
                              int ring_pages, int H, int G, int d, int window, float scale, hipStream_t stream);
 int picolm_attn_decode_mfma_waves(int n_seq, int H, int G);      // waves a decode workgroup will have
+// chunks_done: n_seq * G * ceil(H/G / 32) counters that are zero when the call starts and zero again
+// when its kernel has run: the workgroup that finishes a sequence's last chunk combines the chunks,
+// and no merge kernel runs.  Null: the merge kernel combines them.
 int picolm_attn_decode_mfma(const void* q, const void* k_pages, const void* v_pages, void* out, float* partial,
                             int n_seq, const int32_t* chunk_list, int n_chunks, int pages_per_chunk,
                             int max_splits, const int32_t* seq_pos0, const int32_t* page_table, int max_pages,
-                            int ring_pages, int H, int G, int d, int window, float scale, hipStream_t stream);
+                            int ring_pages, int H, int G, int d, int window, float scale, int32_t* chunks_done,
+                            hipStream_t stream);
 
 // Rotation, cache write and attention of a decode step in one launch: q, k, v of the new tokens are
 // the float rows qkv[n_seq][(H+2G)*d]; tok_page[i] is the physical page for sequence i's new key
@@ -102,7 +106,7 @@ int picolm_attn_decode_rope_mfma(const float* qkv, void* k_pages, void* v_pages,
                                  int max_splits, const int32_t* seq_pos0, const int32_t* page_table,
                                  int max_pages, int ring_pages, int H, int G, int d, int window, float scale,
                                  const float* cos_t, const float* sin_t, int style, const int32_t* tok_page,
-                                 hipStream_t stream);
+                                 int32_t* chunks_done, hipStream_t stream);
 
 int picolm_argmax_scratch_floats(int n_rows, int V);
 int picolm_argmax(const float* logits, int32_t* out, int n_rows, int V, int64_t ld, float* scratch,

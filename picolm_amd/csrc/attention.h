@@ -37,6 +37,10 @@ struct AttnArgs {
     const float* sin_t;
     const int32_t* tok_page;
     int rope_style;             // 0 pairs (2i, 2i+1), 1 pairs (i, i + d/2)
+    // decode, matrix-core kernel: one counter per (sequence, workgroup of heads), zero between
+    // launches.  With it the workgroup that finishes a sequence's last chunk combines the chunks
+    // itself and no merge kernel runs; null: the merge kernel does.
+    int32_t* chunks_done;
 };
 
 // What a decode workgroup has to do.  A sequence whose visible pages fit one chunk is finished by

@@ -352,6 +352,14 @@ __device__ __forceinline__ void rotated_q(const AttnArgs& a, const float* row, i
     }
 }
 
+// single accesses that every workgroup of the GPU sees alike
+__device__ __forceinline__ void store_agent(float* p, float v) {
+    __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ float load_agent(const float* p) {
+    return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
 template <int D, int DEC_WAVES>
 __global__ __launch_bounds__(DEC_WAVES * 64) __attribute__((amdgpu_waves_per_eu(2))) void attn_decode_mfma_kernel(AttnArgs a) {
     extern __shared__ float mrg[];       // [DEC_WAVES + 1][Rc][D + 2], then the new key and value [2][D]
@@ -503,15 +511,72 @@ __global__ __launch_bounds__(DEC_WAVES * 64) __attribute__((amdgpu_waves_per_eu(
         const int hq = g * R + chunk * 32 + q;
         if (work.n_chunks > 1) {
             float* po = a.partial + (((size_t)seq * a.H + hq) * a.max_splits + split) * (D + 2);
-            if (dcol == 0) {
-                po[0] = M * LN2;        // the merge kernel works with natural exponents
-                po[1] = L;
+            if (a.chunks_done) {        // read back by another workgroup of this launch
+                if (dcol == 0) {
+                    store_agent(po, M * LN2);
+                    store_agent(po + 1, L);
+                }
+                store_agent(po + 2 + dcol, acc);
+            } else {
+                if (dcol == 0) {
+                    po[0] = M * LN2;        // the merge kernel works with natural exponents
+                    po[1] = L;
+                }
+                po[2 + dcol] = acc;
             }
-            po[2 + dcol] = acc;
         } else {
             ((bf16_t*)a.out)[tok * a.H * D + (size_t)hq * D + dcol] = f32_to_bf16_bits(L > 0.f ? acc / L : 0.f);
         }
     }
+    if (work.n_chunks <= 1 || a.chunks_done == nullptr) return;       // (uniform over the workgroup)
+    // The chunks of a sequence finish in any order.  Each workgroup counts itself once its partial
+    // results have arrived in memory; the one that counts last reads them all back and writes the
+    // output, chunk by chunk in their order, so the sum does not depend on who it was.  The
+    // partial results are written and read as single accesses that are coherent over the whole GPU
+    // (they pass the L2 of the chiplet): a fence of that scope would write back and invalidate
+    // the whole L2 in every workgroup, which costs far more than the merge kernel it replaces.
+    __shared__ int i_am_last;
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");      // this thread's stores have been acknowledged
+    __syncthreads();
+    int32_t* counter = a.chunks_done + (size_t)seq * (a.G * chunks) + which;
+    if (tid == 0)
+        i_am_last = __hip_atomic_fetch_add(counter, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == work.n_chunks - 1;
+    __syncthreads();
+    if (!i_am_last) return;
+    const int n = work.n_chunks;
+    for (int idx = tid; idx < Rc * D; idx += DEC_WAVES * 64) {
+        const int q = idx / D, dcol = idx % D;
+        const int hq = g * R + chunk * 32 + q;
+        const float* p = a.partial + ((size_t)seq * a.H + hq) * a.max_splits * (D + 2);
+        float M = NEG_BIG, L = 0.f, acc = 0.f;
+        for (int i0 = 0; i0 < n; i0 += 8) {             // eight chunks are asked for at a time
+            float st[8], li[8], col[8];
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                const float* pe = p + (size_t)min(i0 + e, n - 1) * (D + 2);
+                st[e] = load_agent(pe);
+                li[e] = load_agent(pe + 1);
+                col[e] = load_agent(pe + 2 + dcol);
+            }
+            float m_new = M;
+#pragma unroll
+            for (int e = 0; e < 8; ++e)
+                if (i0 + e < n) m_new = fmaxf(m_new, st[e]);
+            const float keep = expf(M - m_new);
+            L *= keep;
+            acc *= keep;
+#pragma unroll
+            for (int e = 0; e < 8; ++e)
+                if (i0 + e < n) {
+                    const float f = expf(st[e] - m_new);
+                    L += f * li[e];
+                    acc += f * col[e];
+                }
+            M = m_new;
+        }
+        ((bf16_t*)a.out)[tok * a.H * D + (size_t)hq * D + dcol] = f32_to_bf16_bits(L > 0.f ? acc / L : 0.f);
+    }
+    if (tid == 0) *counter = 0;          // as the next launch expects it
 }
 
 // =============================================================================================
@@ -604,20 +669,20 @@ static int launch_decode_mfma(const AttnArgs& a, int n_seq, int n_chunks, hipStr
     else DEC_LAUNCH(128, 8)
 #undef DEC_LAUNCH
     PICOLM_LAUNCH_CHECK("attn_decode_mfma");
-    return a.max_splits > 1 ? picolm_attn_merge_launch(a, PICOLM_BF16, n_seq, stream) : 0;
+    return a.max_splits > 1 && !a.chunks_done ? picolm_attn_merge_launch(a, PICOLM_BF16, n_seq, stream) : 0;
 }
 
 extern "C" int picolm_attn_decode_mfma(const void* q, const void* k_pages, const void* v_pages, void* out,
                                        float* partial, int n_seq, const int32_t* chunk_list, int n_chunks,
                                        int pages_per_chunk, int max_splits, const int32_t* seq_pos0,
                                        const int32_t* page_table, int max_pages, int ring_pages, int H, int G,
-                                       int d, int window, float scale, hipStream_t stream) {
+                                       int d, int window, float scale, int32_t* chunks_done, hipStream_t stream) {
     if (check_sizes("attn_decode_mfma", H, G, d, max_pages, ring_pages)) return -1;
     if (check_decode_chunks("attn_decode_mfma", partial, chunk_list, n_chunks, pages_per_chunk, max_splits)) return -1;
     if (n_seq <= 0 || n_chunks <= 0) return 0;
     AttnArgs a = {q, k_pages, v_pages, out, partial, nullptr, nullptr, nullptr, seq_pos0, nullptr, nullptr,
                   page_table, max_pages, ring_pages, H, G, d, window, scale, 1, chunk_list, pages_per_chunk, max_splits,
-                  nullptr, nullptr, nullptr, nullptr, 0};
+                  nullptr, nullptr, nullptr, nullptr, 0, chunks_done};
     return launch_decode_mfma(a, n_seq, n_chunks, stream);
 }
 
@@ -630,7 +695,7 @@ extern "C" int picolm_attn_decode_rope_mfma(const float* qkv, void* k_pages, voi
                                             const int32_t* page_table, int max_pages, int ring_pages, int H,
                                             int G, int d, int window, float scale, const float* cos_t,
                                             const float* sin_t, int style, const int32_t* tok_page,
-                                            hipStream_t stream) {
+                                            int32_t* chunks_done, hipStream_t stream) {
     if (check_sizes("attn_decode_rope_mfma", H, G, d, max_pages, ring_pages)) return -1;
     if (check_decode_chunks("attn_decode_rope_mfma", partial, chunk_list, n_chunks, pages_per_chunk, max_splits)) return -1;
     PICOLM_REQUIRE(qkv && tok_page, "attn_decode_rope_mfma: needs the qkv rows and every token's page");
@@ -641,6 +706,6 @@ extern "C" int picolm_attn_decode_rope_mfma(const float* qkv, void* k_pages, voi
     if (n_seq <= 0 || n_chunks <= 0) return 0;
     AttnArgs a = {nullptr, k_pages, v_pages, out, partial, nullptr, nullptr, nullptr, seq_pos0, nullptr, nullptr,
                   page_table, max_pages, ring_pages, H, G, d, window, scale, 1, chunk_list, pages_per_chunk, max_splits,
-                  qkv, cos_t, sin_t, tok_page, style};
+                  qkv, cos_t, sin_t, tok_page, style, chunks_done};
     return launch_decode_mfma(a, n_seq, n_chunks, stream);
 }

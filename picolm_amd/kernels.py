@@ -450,14 +450,27 @@ def attn_prefill_mfma(q, k_pages, v_pages, out, batch, page_table, ring_pages, H
         page_table.shape[1], ring_pages, H, G, d, window, c_float(scale), _stream()))
 
 
+def attn_decode_counters(n_seq: int, H: int, G: int) -> int:
+    """Counters (int32, zero between launches) with which the matrix-core decode kernels combine
+    the chunks of a sequence themselves: one per sequence and workgroup of heads."""
+    return n_seq * G * ((H // G + 31) // 32)
+
+
+def _counters_check(chunks_done, n_seq, H, G):
+    if chunks_done is not None:
+        _i32("attn.chunks_done", chunks_done, attn_decode_counters(n_seq, H, G))
+
+
 def attn_decode_mfma(q, k_pages, v_pages, out, partial, n_seq, chunk_list, n_chunks, pages_per_chunk,
-                     max_splits, seq_pos0, page_table, ring_pages, H, G, d, window, scale) -> None:
+                     max_splits, seq_pos0, page_table, ring_pages, H, G, d, window, scale, chunks_done=None) -> None:
+    """chunks_done: see attn_decode_counters; None lets a second kernel combine the chunks."""
     _attn_check(q, k_pages, v_pages, out, page_table, H, G, d)
     _decode_check(q, partial, n_seq, chunk_list, n_chunks, pages_per_chunk, max_splits, seq_pos0, H, d)
+    _counters_check(chunks_done, n_seq, H, G)
     _check(lib().picolm_attn_decode_mfma(
         _ptr(q), _ptr(k_pages), _ptr(v_pages), _ptr(out), _ptr(partial if max_splits > 1 else None), n_seq,
         _ptr(chunk_list), n_chunks, pages_per_chunk, max_splits, _ptr(seq_pos0), _ptr(page_table),
-        page_table.shape[1], ring_pages, H, G, d, window, c_float(scale), _stream()))
+        page_table.shape[1], ring_pages, H, G, d, window, c_float(scale), _ptr(chunks_done), _stream()))
 
 
 def attn_decode_rope_takes(dtype: torch.dtype, d: int) -> bool:
@@ -466,10 +479,13 @@ def attn_decode_rope_takes(dtype: torch.dtype, d: int) -> bool:
 
 
 def attn_decode_rope(qkv, k_pages, v_pages, out, partial, n_seq, chunk_list, n_chunks, pages_per_chunk, max_splits,
-                     seq_pos0, page_table, ring_pages, H, G, d, window, scale, cos, sin, style, tok_page) -> None:
+                     seq_pos0, page_table, ring_pages, H, G, d, window, scale, cos, sin, style, tok_page,
+                     chunks_done=None) -> None:
     """A decode step's rotation, cache write and attention in one launch (bfloat16 cache, head
     sizes of the matrix-core kernels): `qkv` are the float rows [n_seq, (H+2G)d] of the new tokens,
-    `tok_page[i]` the physical page that takes sequence i's new key and value."""
+    `tok_page[i]` the physical page that takes sequence i's new key and value.  chunks_done: see
+    attn_decode_counters."""
+    _counters_check(chunks_done, n_seq, H, G)
     _dev("attn.qkv", qkv, torch.float32, 2)
     if qkv.shape[0] < n_seq or qkv.shape[1] != (H + 2 * G) * d:
         raise KernelError(f"attn_decode_rope: qkv {tuple(qkv.shape)} is not [>= {n_seq}, {(H + 2 * G) * d}]")
@@ -496,7 +512,7 @@ def attn_decode_rope(qkv, k_pages, v_pages, out, partial, n_seq, chunk_list, n_c
         _ptr(qkv), _ptr(k_pages), _ptr(v_pages), _ptr(out), _ptr(partial if max_splits > 1 else None), n_seq,
         _ptr(chunk_list), n_chunks, pages_per_chunk, max_splits, _ptr(seq_pos0), _ptr(page_table),
         page_table.shape[1], ring_pages, H, G, d, window, c_float(scale), _ptr(cos), _ptr(sin), style, _ptr(tok_page),
-        _stream()))
+        _ptr(chunks_done), _stream()))
 
 
 def attn_prefill(q, k_pages, v_pages, out, batch, page_table, ring_pages, H, G, d, window, scale) -> None:
@@ -510,13 +526,17 @@ def attn_prefill(q, k_pages, v_pages, out, batch, page_table, ring_pages, H, G, 
 
 
 def attn_decode(q, k_pages, v_pages, out, partial, n_seq, chunk_list, n_chunks, pages_per_chunk, max_splits,
-                seq_pos0, page_table, ring_pages, H, G, d, window, scale) -> None:
+                seq_pos0, page_table, ring_pages, H, G, d, window, scale, chunks_done=None) -> None:
     """Attention of one new token per sequence (row i of q is sequence i) over its cache pages.
     `chunk_list` is the step's work list, eight ints an entry behind a header entry: entry 1 + x
-    gives workgroup x `pages_per_chunk` pages of one sequence."""
-    fn = attn_decode_mfma if attn_mfma_takes(q, d) else attn_decode_generic
-    fn(q, k_pages, v_pages, out, partial, n_seq, chunk_list, n_chunks, pages_per_chunk, max_splits, seq_pos0,
-       page_table, ring_pages, H, G, d, window, scale)
+    gives workgroup x `pages_per_chunk` pages of one sequence.  chunks_done: counters for the
+    kernels that can combine a sequence's chunks themselves (attn_decode_counters)."""
+    if attn_mfma_takes(q, d):
+        attn_decode_mfma(q, k_pages, v_pages, out, partial, n_seq, chunk_list, n_chunks, pages_per_chunk, max_splits,
+                         seq_pos0, page_table, ring_pages, H, G, d, window, scale, chunks_done)
+    else:
+        attn_decode_generic(q, k_pages, v_pages, out, partial, n_seq, chunk_list, n_chunks, pages_per_chunk,
+                            max_splits, seq_pos0, page_table, ring_pages, H, G, d, window, scale)
 
 
 def sample(logits: torch.Tensor, out: torch.Tensor, temperature: float, top_k: int, top_p: float,

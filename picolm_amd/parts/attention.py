@@ -76,15 +76,16 @@ class Attention(Mixer):
             chunk_list, n_chunks, ppc, most = b.decode_chunks(*self.decode_geometry(ctx.dtype, b.n_seq), self.window,
                                                                group, table_host, ring)
             partial = ctx.ws.get("attn.partial", (b.n_seq * H * most * (d + 2),), torch.float32) if most > 1 else None
+            done = ctx.ws.zeros("attn.chunks_done", (kernels.attn_decode_counters(b.n_seq, H, G),), torch.int32) if most > 1 else None
             if writes and kernels.attn_decode_rope_takes(ctx.dtype, d):
                 # rotation (if the position encoding is one), cache write and attention in one launch
                 kernels.attn_decode_rope(qkv, k_pages, v_pages, out, partial, b.n_seq, chunk_list, n_chunks, ppc, most,
                                          b.seq_pos0, table, ring, H, G, d, self.window, self.scale, cos, sin, style,
-                                         tok_page)
+                                         tok_page, done)
             else:
                 kernels.rope_kv_store(qkv, q, kp, vp, cos, sin, style, b.tok_pos, tok_page, H, G, d)
                 kernels.attn_decode(q, k_pages, v_pages, out, partial, b.n_seq, chunk_list, n_chunks, ppc, most,
-                                    b.seq_pos0, table, ring, H, G, d, self.window, self.scale)
+                                    b.seq_pos0, table, ring, H, G, d, self.window, self.scale, done)
         elif self.window > 0 and ring < table.shape[1] and b.max_new > WINDOW_STEP_TOKENS:
             # a ring holds a window and one chunk: write and answer the step chunk by chunk
             for c in b.chunks(WINDOW_STEP_TOKENS):

@@ -51,6 +51,19 @@ class Workspace:
             self._bufs[name] = buf
         return buf[:nbytes].view(dtype).view(*shape)
 
+    def zeros(self, name: str, shape, dtype: torch.dtype) -> torch.Tensor:
+        """A buffer that is zero when first given out and that its users leave at zero (counters
+        that a kernel resets itself)."""
+        n = 1
+        for s in shape:
+            n *= int(s)
+        nbytes = n * torch.empty((), dtype=dtype).element_size()
+        buf = self._bufs.get(name)
+        if buf is None or buf.numel() < nbytes:
+            buf = torch.zeros(max(nbytes, 256), dtype=torch.uint8, device=self.device)
+            self._bufs[name] = buf
+        return buf[:nbytes].view(dtype).view(*shape)
+
     def flip(self, name: str) -> int:
         """0, 1, 0, 1, ... per name: for a pair of buffers used in turn."""
         self._flips[name] = 1 - self._flips.get(name, 1)

@@ -400,6 +400,18 @@ def test_attention_decode(dtype, H, G, d, pages_per_chunk, window, spare):
     ref = case.reference(window)
     err = np.abs(out.double().cpu().numpy() - ref).max()
     assert err <= tol(dtype, np.abs(ref).max()), err
+    # the same with the chunks combined by the attention kernel itself (kernels that cannot ignore
+    # the counters); twice, for the counters must be left at zero
+    done = torch.zeros(K().attn_decode_counters(b.n_seq, H, G), dtype=torch.int32, device=DEV)
+    for _ in range(2):
+        out.zero_()
+        partial.fill_(float("nan"))
+        K().attn_decode(case.q_dev, case.k_pages, case.v_pages, out, partial, b.n_seq, chunk_list, n_chunks,
+                        pages_per_chunk, most, b.seq_pos0, case.table, case.table.shape[1], H, G, d, window,
+                        1.0 / math.sqrt(d), done)
+        err = np.abs(out.double().cpu().numpy() - ref).max()
+        assert err <= tol(dtype, np.abs(ref).max()), err
+        assert not done.any()
 
 
 @pytest.mark.parametrize("d", [64, 128])
@@ -414,12 +426,22 @@ def test_attention_decode_many_sequences(d, pages_per_chunk):
     out = torch.zeros_like(case.q_dev)
     chunk_list, n_chunks, most = decode_work_list(case, 0, pages_per_chunk, spare=2)
     partial = torch.full((b.n_seq * H * most * (d + 2),), float("nan"), device=DEV)
-    K().attn_decode(case.q_dev, case.k_pages, case.v_pages, out, partial, b.n_seq, chunk_list, n_chunks,
-                    pages_per_chunk, most, b.seq_pos0, case.table, case.table.shape[1], H, G, d, 0,
-                    1.0 / math.sqrt(d))
+    done = torch.zeros(K().attn_decode_counters(b.n_seq, H, G), dtype=torch.int32, device=DEV)
     ref = case.reference(0)
-    err = np.abs(out.double().cpu().numpy() - ref).max()
-    assert err <= tol(torch.bfloat16, np.abs(ref).max()), err
+    outs = []
+    # the partial results hold NaN before every run: one that is read before it arrived shows
+    for counters in [None] + [done] * 12:
+        out.zero_()
+        partial.fill_(float("nan"))
+        K().attn_decode(case.q_dev, case.k_pages, case.v_pages, out, partial, b.n_seq, chunk_list, n_chunks,
+                        pages_per_chunk, most, b.seq_pos0, case.table, case.table.shape[1], H, G, d, 0,
+                        1.0 / math.sqrt(d), counters)
+        err = np.abs(out.double().cpu().numpy() - ref).max()
+        assert err <= tol(torch.bfloat16, np.abs(ref).max()), err
+        assert not done.any()
+        outs.append(out.clone())
+    for o in outs[2:]:
+        assert torch.equal(outs[1], o)            # whichever workgroup came last, the sum is the same
 
 
 @pytest.mark.parametrize("H,G,d", [(6, 6, 32), (8, 2, 64), (32, 8, 128), (40, 1, 64)])
@@ -462,11 +484,18 @@ def test_attention_decode_with_rotation_and_cache_write_inside(H, G, d, style, p
     chunk_list, n_chunks, most = decode_work_list(case, window, pages_per_chunk, spare=1)
     partial = torch.full((n * H * most * (d + 2),), float("nan"), device=DEV)
     dev = lambda t: None if style is None else torch.from_numpy(t).float().to(DEV)
-    K().attn_decode_rope(torch.from_numpy(qkv).to(DEV), case.k_pages, case.v_pages, out, partial, n, chunk_list, n_chunks,
-                         pages_per_chunk, most, b.seq_pos0, case.table, case.table.shape[1], H, G, d, window,
-                         1.0 / math.sqrt(d), dev(cos), dev(sin), 0 if style != "half" else 1, tok_page)
-    err = np.abs(out.double().cpu().numpy() - ref).max()
-    assert err <= tol(torch.bfloat16, np.abs(ref).max()), err
+    # with a second kernel combining the chunks, then with the attention kernel doing it itself
+    # (the second call finds the new tokens' rows written; it must give the same)
+    done = torch.zeros(K().attn_decode_counters(n, H, G), dtype=torch.int32, device=DEV)
+    for counters in (None, done):
+        out.zero_()
+        K().attn_decode_rope(torch.from_numpy(qkv).to(DEV), case.k_pages, case.v_pages, out, partial, n, chunk_list,
+                             n_chunks, pages_per_chunk, most, b.seq_pos0, case.table, case.table.shape[1], H, G, d,
+                             window, 1.0 / math.sqrt(d), dev(cos), dev(sin), 0 if style != "half" else 1, tok_page,
+                             counters)
+        err = np.abs(out.double().cpu().numpy() - ref).max()
+        assert err <= tol(torch.bfloat16, np.abs(ref).max()), err
+        assert not done.any()
     for i in range(n):
         pg, row = int(tok_page[i]), pos0[i] % PAGE
         assert torch.equal(case.k_pages[pg, :, row, :].cpu(), bf(k_ref[i]))
