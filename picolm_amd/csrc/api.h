@@ -59,6 +59,10 @@ int picolm_gemm_linked(const void* A, const void* W, void* C, int c_dt, int M, i
                        const float* next_w, void* next_h, float* next_ssq, int next_parts, const float* ssq,
                        int n_parts, int norm_len, float eps, int rows, hipStream_t stream);
 
+// Within a group's part of a page, K[64][d] and V^T[d][64] lie as plain arrays, except in bfloat16
+// pages of head size 32, 64 or 128: those are in the order of the matrix-core kernels' operands.
+// Fills k_idx[key * d + i] and v_idx[i * 64 + key] with the offsets of K[key][i] and V^T[i][key].
+int picolm_kv_page_order(int dt, int d, int32_t* k_idx, int32_t* v_idx);
 int picolm_attn_prefill_tile_rows(void);
 int picolm_attn_prefill_generic(const void* q, const void* k_pages, const void* v_pages, void* out,
                                 int dt, const int32_t* tile_seq, const int32_t* tile_q0, int n_tiles,

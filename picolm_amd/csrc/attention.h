@@ -6,8 +6,8 @@
 
 struct AttnArgs {
     const void* q;            // [T][H*d]
-    const void* k_pages;      // [n_pages][G][PAGE][d]
-    const void* v_pages;      // [n_pages][G][d][PAGE]
+    const void* k_pages;      // [n_pages][G][PAGE][d]     (within [PAGE][d] in the order of
+    const void* v_pages;      // [n_pages][G][d][PAGE]      k_page_offset / v_page_offset)
     void* out;                // [T][H*d]
     float* partial;           // decode: [n_seq][H][max_splits][d+2]
     const int32_t* tile_seq;  // prefill: sequence of each tile
@@ -42,6 +42,44 @@ struct AttnArgs {
     // itself and no merge kernel runs; null: the merge kernel does.
     int32_t* chunks_done;
 };
+
+// ---- the order of a page's elements ---------------------------------------------------------
+// A page holds, per KV group, the keys K[64][d] and the values transposed V^T[d][64].  Pages of
+// the vector-ALU kernels (32-bit, or head sizes the matrix-core kernels do not take) keep these
+// as plain arrays.  Pages of the matrix-core kernels (bfloat16, d = 32, 64, 128) keep their
+// 16-byte chunks in the order in which a wave takes them as MFMA operands, so that every
+// wave-wide load reads 1 KB of adjacent memory:
+//   K   chunk ((tile * d/16 + kstep) * 64 + lane): key 32*tile + key_of_row(lane % 32),
+//       elements 16*kstep + 8*(lane / 32) .. + 8
+//   V^T chunk (((tile * d/32 + dblock) * 2 + step) * 64 + lane): row 32*dblock + lane % 32,
+//       keys 32*tile + 16*step + 8*(lane / 32) .. + 8
+// Row i of an S^T tile holds key_of_row(i) of the tile's 32 keys.  The accumulator of a lane in
+// wave half h holds rows 8a + 4h + b (a = 0..3, b = 0..3) as element 4a + b; with this map they
+// are the keys 8h .. 8h+7 (elements 0..7) and 16+8h .. 16+8h+7 (elements 8..15): P^T for step ks
+// of the second MFMA is elements 8ks .. 8ks+7 as they are.
+__host__ __device__ __forceinline__ int key_of_row(int i) {
+    const int hh = (i >> 2) & 1, aa = i >> 3, bb = i & 3;
+    return 16 * (aa >> 1) + 8 * hh + 4 * (aa & 1) + bb;
+}
+__host__ __device__ __forceinline__ int row_of_key(int k) {
+    const int aa = 2 * (k >> 4) + ((k >> 2) & 1), hh = (k >> 3) & 1, bb = k & 3;
+    return 8 * aa + 4 * hh + bb;
+}
+// whether pages of this dtype and head size are in the matrix-core kernels' order
+__host__ __device__ __forceinline__ bool kv_pages_tiled(int dt, int d) {
+    return dt == PICOLM_BF16 && (d == 32 || d == 64 || d == 128);
+}
+// offset of K[key][i] and of V^T[i][key] within one group's part of a page
+__host__ __device__ __forceinline__ int k_page_offset(int key, int i, int d, bool tiled) {
+    if (!tiled) return key * d + i;
+    const int chunk = i >> 3;
+    return ((((key >> 5) * (d >> 4) + (chunk >> 1)) * 64 + (chunk & 1) * 32 + row_of_key(key & 31)) << 3) + (i & 7);
+}
+__host__ __device__ __forceinline__ int v_page_offset(int i, int key, int d, bool tiled) {
+    if (!tiled) return i * PAGE_TOKENS + key;
+    const int kc = key >> 3;      // eight keys: tile kc / 4, step (kc / 2) % 2, wave half kc % 2
+    return (((((kc >> 2) * (d >> 5) + (i >> 5)) * 2 + ((kc >> 1) & 1)) * 64 + (kc & 1) * 32 + (i & 31)) << 3) + (key & 7);
+}
 
 // What a decode workgroup has to do.  A sequence whose visible pages fit one chunk is finished by
 // its workgroup; otherwise every chunk leaves (max, sum, acc) in `partial` and the merge kernel

@@ -291,6 +291,7 @@ extern "C" int picolm_attn_prefill_generic(const void* q, const void* k_pages, c
                                            int H, int G, int d, int window, float scale,
                                            hipStream_t stream) {
     if (check_attn_sizes("attn_prefill", H, G, d, max_pages, ring_pages)) return -1;
+    PICOLM_REQUIRE(!kv_pages_tiled(dt, d), "attn_prefill: bfloat16 pages of head size %d are in the matrix-core kernels' order", d);
     PICOLM_REQUIRE(H <= 65535, "attn_prefill: %d heads exceed the grid", H);
     if (n_tiles <= 0) return 0;
     AttnArgs a = {q, k_pages, v_pages, out, nullptr, tile_seq, tile_q0, seq_slot, seq_pos0, seq_nnew,
@@ -311,6 +312,7 @@ extern "C" int picolm_attn_decode_generic(const void* q, const void* k_pages, co
                                           int max_pages, int ring_pages, int H, int G, int d, int window,
                                           float scale, hipStream_t stream) {
     if (check_attn_sizes("attn_decode", H, G, d, max_pages, ring_pages)) return -1;
+    PICOLM_REQUIRE(!kv_pages_tiled(dt, d), "attn_decode: bfloat16 pages of head size %d are in the matrix-core kernels' order", d);
     if (check_decode_chunks("attn_decode", partial, chunk_list, n_chunks, pages_per_chunk, max_splits)) return -1;
     PICOLM_REQUIRE(dt == PICOLM_F32 || dt == PICOLM_BF16, "attn_decode: unknown dtype %d", dt);
     if (n_seq <= 0 || n_chunks <= 0) return 0;
@@ -323,4 +325,18 @@ extern "C" int picolm_attn_decode_generic(const void* q, const void* k_pages, co
     const int rc = dt == PICOLM_F32 ? launch_attn<float>(a, grid, stream) : launch_attn<bf16_t>(a, grid, stream);
     if (rc) return rc;
     return max_splits > 1 ? picolm_attn_merge_launch(a, dt, n_seq, stream) : 0;
+}
+
+// The order of a page's elements, for code that fills or reads pages on the host: offsets of
+// K[key][i] (k_idx[key * d + i]) and of V^T[i][key] (v_idx[i * 64 + key]) within a group's part
+// of a page of this dtype and head size.
+extern "C" int picolm_kv_page_order(int dt, int d, int32_t* k_idx, int32_t* v_idx) {
+    PICOLM_REQUIRE(d > 0 && k_idx && v_idx, "kv_page_order: bad arguments");
+    const bool tiled = kv_pages_tiled(dt, d);
+    for (int key = 0; key < PAGE_TOKENS; ++key)
+        for (int i = 0; i < d; ++i) {
+            k_idx[key * d + i] = k_page_offset(key, i, d, tiled);
+            v_idx[i * PAGE_TOKENS + key] = v_page_offset(i, key, d, tiled);
+        }
+    return 0;
 }

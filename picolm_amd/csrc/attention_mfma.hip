@@ -5,7 +5,8 @@
 // one exchange with lane^32, and the rescaling of the output accumulator O^T = V^T P^T is a
 // per-lane scalar.  The rows of an S^T tile are a permutation of its 32 keys, chosen so that a
 // lane's 16 accumulator values are 16 consecutive keys; P^T then feeds the second MFMA
-// straight from registers, and V^T (values are cached transposed) is read 16 bytes at a time.
+// straight from registers.  The cache pages hold K and V^T in the order of the MFMA operands
+// (k_page_offset, v_page_offset), so that a wave-wide load of an operand reads 1 KB in a row.
 // Softmax statistics are float, in the base-2 domain: p = exp2(s*scale*log2e - m).
 //
 //   prefill: a workgroup of 4 waves shares K and V^T tiles of one page through LDS; a wave
@@ -34,15 +35,6 @@ __device__ __forceinline__ bf16x8 zero8() {
 #pragma unroll
     for (int i = 0; i < 8; ++i) z[i] = (__bf16)0.0f;
     return z;
-}
-// Row i of an S^T tile holds key_of_row(i) of the tile's 32 keys.  The accumulator of a lane in
-// wave half h holds rows 8a + 4h + b (a = 0..3, b = 0..3) as element 4a + b; with this map they
-// are the keys 8h .. 8h+7 (elements 0..7) and 16+8h .. 16+8h+7 (elements 8..15): P^T for step ks
-// of the second MFMA is elements 8ks .. 8ks+7 as they are, and the two halves of a wave read
-// adjacent 16-byte chunks of a V^T row.
-__device__ __forceinline__ int key_of_row(int i) {
-    const int hh = (i >> 2) & 1, aa = i >> 3, bb = i & 3;
-    return 16 * (aa >> 1) + 8 * hh + 4 * (aa & 1) + bb;
 }
 // key (within the tile) of accumulator element e of a lane in half h
 __device__ __forceinline__ int key_of_elem(int e, int h) { return 16 * (e >> 3) + 8 * h + (e & 7); }
@@ -157,17 +149,8 @@ __device__ __forceinline__ void attend_tile(const bf16x8 (&Qf)[D / 16], const bf
 }
 
 // =============================================================================================
-// LDS tiles of the prefill kernel.  K rows are D bf16 (for D = 128 a row spans all 64 banks), V^T
-// rows are 64 bf16 (half of the banks); the 16-byte chunks of a row are XOR-permuted so that the
-// 16 lanes served in one LDS cycle touch every bank once.
-template <int D>
-__device__ __forceinline__ int k_off(int row, int chunk) {
-    constexpr int KCH = D / 8;
-    constexpr int ROWS_PER_SPAN = KCH >= 16 ? 1 : 16 / KCH;      // rows that share a 256-byte bank span
-    return (row * KCH + (chunk ^ ((row / ROWS_PER_SPAN) % KCH))) * 8;
-}
-__device__ __forceinline__ int v_off(int row, int chunk) { return (row * 8 + (chunk ^ ((row >> 1) & 7))) * 8; }
-
+// LDS tiles of the prefill kernel: a page's K and V^T as they lie in the cache, that is in the
+// order of the MFMA operands: the 64 lanes of a wave read 64 adjacent 16-byte chunks.
 template <int D>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void attn_prefill_mfma_kernel(AttnArgs a, int HB, int tile_tokens) {
     constexpr int KCH = D / 8;                        // 16-byte chunks of a K row
@@ -233,26 +216,24 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void a
         // keys past the sequence's end may hold anything: their values are zeroed, without a branch
         const int n_keys = b_qlast - page * PAGE_TOKENS + 1;
 #pragma unroll
-        for (int i = 0; i < KP; ++i) {
-            const int idx = tid + 256 * i;
-            *(bf16x8*)(Ks + k_off<D>(idx / KCH, idx % KCH)) = kreg[i];
-        }
+        for (int i = 0; i < KP; ++i) *(bf16x8*)(Ks + (size_t)(tid + 256 * i) * 8) = kreg[i];
 #pragma unroll
         for (int i = 0; i < VP; ++i) {
             const int idx = tid + 256 * i;
-            const int c = idx % 8;
+            // chunk idx of V^T holds keys 32*tile + 16*step + 8*half .. + 8 (see v_page_offset)
+            const int key0 = 32 * (idx / (128 * (D / 32))) + 16 * ((idx / 64) % 2) + 8 * ((idx % 64) / 32);
             bf16x8 v = vreg[i];
 #pragma unroll
-            for (int e = 0; e < 8; ++e) v[e] = (8 * c + e < n_keys) ? v[e] : (__bf16)0.0f;
-            *(bf16x8*)(Vs + v_off(idx / 8, c)) = v;
+            for (int e = 0; e < 8; ++e) v[e] = (key0 + e < n_keys) ? v[e] : (__bf16)0.0f;
+            *(bf16x8*)(Vs + (size_t)idx * 8) = v;
         }
     };
     auto compute = [&](int stage, int page) {
         if (page < w_page_lo || page >= w_page_hi) return;
         const bf16_t* Ks = lds + stage * STAGE;
         const bf16_t* Vs = Ks + PAGE_TOKENS * D;
-        auto kop = [&](int t, int s) { return *(const bf16x8*)(Ks + k_off<D>(32 * t + key_of_row(l32), 2 * s + h)); };
-        auto vop = [&](int dt, int t, int ks) { return *(const bf16x8*)(Vs + v_off(32 * dt + l32, 4 * t + 2 * ks + h)); };
+        auto kop = [&](int t, int s) { return *(const bf16x8*)(Ks + ((t * (D / 16) + s) * 64 + lane) * 8); };
+        auto vop = [&](int dt, int t, int ks) { return *(const bf16x8*)(Vs + (((t * (D / 32) + dt) * 2 + ks) * 64 + lane) * 8); };
         // a page wholly before the wave's first query needs no mask (rows without a query are
         // never stored, whatever they hold)
         if (a.window <= 0 && page * PAGE_TOKENS + PAGE_TOKENS - 1 <= w_qfirst)
@@ -434,16 +415,17 @@ __global__ __launch_bounds__(DEC_WAVES * 64) __attribute__((amdgpu_waves_per_eu(
         if (key0 > key_max) break;                           // nothing of this tile, or of a later one, is visible
         const int next_phys = tt + DEC_WAVES < n_tiles ? page_of_tile(tt + DEC_WAVES) : 0;   // asked for before this tile's data
         const size_t base = (size_t)phys * page_elems + (size_t)g * PAGE_TOKENS * D;
-        const bf16_t* kp = (const bf16_t*)a.k_pages + base + 8 * h;
-        const bf16_t* vp = (const bf16_t*)a.v_pages + base + (size_t)l32 * PAGE_TOKENS + 8 * h;
+        // tile t of the group's part of a page: 32 * D elements of K, then of V^T, as operands
+        const bf16_t* kp = (const bf16_t*)a.k_pages + base + (size_t)t * 32 * D + lane * 8;
+        const bf16_t* vp = (const bf16_t*)a.v_pages + base + (size_t)t * 32 * D + lane * 8;
         const int n_keys = key_max - key0 + 1;               // >= 1; keys past it are not this sequence's, or not written yet
         bf16x8 Kf[D / 16], Vf[D / 32][2];
 #pragma unroll
-        for (int s = 0; s < D / 16; ++s) Kf[s] = ldg8(kp + (size_t)(32 * t + key_of_row(l32)) * D + 16 * s);
+        for (int s = 0; s < D / 16; ++s) Kf[s] = ldg8(kp + 512 * s);
 #pragma unroll
         for (int dt = 0; dt < D / 32; ++dt)
 #pragma unroll
-            for (int ks = 0; ks < 2; ++ks) Vf[dt][ks] = ldg8(vp + (size_t)(32 * dt) * PAGE_TOKENS + 32 * t + 16 * ks);
+            for (int ks = 0; ks < 2; ++ks) Vf[dt][ks] = ldg8(vp + 512 * (2 * dt + ks));
         if (n_keys < 32) {                                   // keys past the end may hold anything
 #pragma unroll
             for (int dt = 0; dt < D / 32; ++dt)
@@ -491,8 +473,8 @@ __global__ __launch_bounds__(DEC_WAVES * 64) __attribute__((amdgpu_waves_per_eu(
         if (chunk == 0 && tid < D) {                        // one workgroup of the group writes the cache
             const size_t base = (size_t)a.tok_page[seq] * page_elems + (size_t)g * PAGE_TOKENS * D;
             const int in_page = qpos % PAGE_TOKENS;
-            ((bf16_t*)a.k_pages)[base + (size_t)in_page * D + tid] = f32_to_bf16_bits(knew[tid]);
-            ((bf16_t*)a.v_pages)[base + (size_t)tid * PAGE_TOKENS + in_page] = f32_to_bf16_bits(vnew[tid]);
+            ((bf16_t*)a.k_pages)[base + k_page_offset(in_page, tid, D, true)] = f32_to_bf16_bits(knew[tid]);
+            ((bf16_t*)a.v_pages)[base + v_page_offset(tid, in_page, D, true)] = f32_to_bf16_bits(vnew[tid]);
         }
         __syncthreads();
     }

@@ -2,6 +2,7 @@
 // element-wise helpers.  One workgroup handles one row (token); all arithmetic is float.
 #include "common.h"
 #include "api.h"
+#include "attention.h"
 
 // ---- embedding: x[t][:] = table[tokens[t]][:] ------------------------------------------
 // picolm/model_core.c:1785-1786, :2758-2762: the row is converted to float, no scaling.
@@ -117,7 +118,7 @@ __global__ void rope_kv_store_kernel(const float* __restrict__ qkv, TC* __restri
                                      const float* __restrict__ cos_t, const float* __restrict__ sin_t,
                                      int style, const int32_t* __restrict__ tok_pos,
                                      const int32_t* __restrict__ tok_page, int H, int G, int d,
-                                     const int32_t* __restrict__ rows) {
+                                     const int32_t* __restrict__ rows, bool tiled) {
     const int t = rows ? rows[blockIdx.x] : blockIdx.x;      // `rows`: the token rows this launch handles
     const int pos = tok_pos[t];
     const int half = d / 2;
@@ -126,14 +127,11 @@ __global__ void rope_kv_store_kernel(const float* __restrict__ qkv, TC* __restri
     const float* s = sin_t ? sin_t + (size_t)pos * half : nullptr;
 
     // keys are [page][G][PAGE][d]; values are kept transposed, [page][G][d][PAGE], so that the
-    // attention kernels read eight consecutive keys of one column as one 16-byte chunk
-    size_t cache_row = 0, page_base = 0;
+    // attention kernels read eight consecutive keys of one column as one 16-byte chunk; within
+    // a group's [PAGE][d] the order is that of k_page_offset / v_page_offset
+    size_t page_base = 0;
     const int in_page = pos % PAGE_TOKENS;
-    if (k_pages) {
-        const int page = tok_page[t];
-        page_base = ((size_t)page * G) * PAGE_TOKENS * d;
-        cache_row = page_base + (size_t)in_page * d;
-    }
+    if (k_pages) page_base = ((size_t)tok_page[t] * G) * PAGE_TOKENS * d;
     // blockIdx.y takes ROPE_HEADS heads of the row: heads 0..H-1 are q, H..H+G-1 are k, then v
     const int head_lo = blockIdx.y * ROPE_HEADS, head_hi = min(head_lo + ROPE_HEADS, H + 2 * G);
     for (int head = head_lo; head < head_hi; ++head) {
@@ -153,16 +151,16 @@ __global__ void rope_kv_store_kernel(const float* __restrict__ qkv, TC* __restri
                     q[i0] = from_f32<TC>(y0);
                     q[i1] = from_f32<TC>(y1);
                 } else if (k_pages) {
-                    TC* k = k_pages + cache_row + (size_t)(head - H) * PAGE_TOKENS * d;
-                    k[i0] = from_f32<TC>(y0);
-                    k[i1] = from_f32<TC>(y1);
+                    TC* k = k_pages + page_base + (size_t)(head - H) * PAGE_TOKENS * d;
+                    k[k_page_offset(in_page, i0, d, tiled)] = from_f32<TC>(y0);
+                    k[k_page_offset(in_page, i1, d, tiled)] = from_f32<TC>(y1);
                 }
             }
         } else if (v_pages) {
             const int g = head - H - G;
             const float* vrow = row + (size_t)head * d;
             for (int i = threadIdx.x; i < d; i += blockDim.x)
-                v_pages[page_base + ((size_t)g * d + i) * PAGE_TOKENS + in_page] = from_f32<TC>(vrow[i]);
+                v_pages[page_base + (size_t)g * PAGE_TOKENS * d + v_page_offset(i, in_page, d, tiled)] = from_f32<TC>(vrow[i]);
         }
     }
 }
@@ -182,11 +180,11 @@ extern "C" int picolm_rope_kv_store(const float* qkv, void* q_out, void* k_pages
     if (dt == PICOLM_F32)
         rope_kv_store_kernel<float><<<grid, block, 0, stream>>>(
             qkv, (float*)q_out, (float*)k_pages, (float*)v_pages, cos_t, sin_t, style, tok_pos, tok_page,
-            H, G, d, rows);
+            H, G, d, rows, kv_pages_tiled(dt, d));
     else if (dt == PICOLM_BF16)
         rope_kv_store_kernel<bf16_t><<<grid, block, 0, stream>>>(
             qkv, (bf16_t*)q_out, (bf16_t*)k_pages, (bf16_t*)v_pages, cos_t, sin_t, style, tok_pos, tok_page,
-            H, G, d, rows);
+            H, G, d, rows, kv_pages_tiled(dt, d));
     else
         PICOLM_REQUIRE(false, "rope_kv_store: unknown dtype %d", dt);
     PICOLM_LAUNCH_CHECK("rope_kv_store");

@@ -42,7 +42,7 @@ def dir_entry_points():
     return ["picolm_abi_version", "picolm_device_check", "picolm_embed", "picolm_rmsnorm",
             "picolm_rope_kv_store", "picolm_silu_mul", "picolm_add_into", "picolm_gemm_generic",
             "picolm_attn_prefill_tile_rows", "picolm_attn_prefill_generic",
-            "picolm_attn_decode_generic", "picolm_argmax", "picolm_argmax_scratch_floats", "picolm_sample", "picolm_gemm_skinny", "picolm_gemm_tiled", "picolm_gemm_tiled_splitk", "picolm_gemm_linked",
+            "picolm_attn_decode_generic", "picolm_argmax", "picolm_argmax_scratch_floats", "picolm_sample", "picolm_gemm_skinny", "picolm_gemm_tiled", "picolm_gemm_tiled_splitk", "picolm_gemm_linked", "picolm_kv_page_order",
             "picolm_attn_mfma_takes", "picolm_attn_prefill_mfma_heads", "picolm_attn_prefill_mfma_tile_tokens",
             "picolm_attn_prefill_mfma", "picolm_attn_decode_mfma", "picolm_attn_decode_rope_mfma", "picolm_attn_decode_mfma_waves", "picolm_read_probe", "picolm_mfma_probe"]
 
@@ -153,6 +153,43 @@ def rope_kv_store(qkv, q_out, k_pages, v_pages, cos, sin, style: int, tok_pos, t
     _check(lib().picolm_rope_kv_store(
         _ptr(qkv), _ptr(q_out), _ptr(k_pages), _ptr(v_pages), dt_of(q_out), _ptr(cos), _ptr(sin), style,
         _ptr(tok_pos), _ptr(tok_page if k_pages is not None else None), n_launch, H, G, d, _ptr(rows), _stream()))
+
+
+_page_orders: dict = {}
+
+
+def kv_page_order(dtype: torch.dtype, d: int):
+    """Where K[key][i] and V^T[i][key] lie within a group's part of a cache page: two int64
+    tensors k_idx [64, d] and v_idx [d, 64] of element offsets.  Plain arrays, except in bfloat16
+    pages of the head sizes that the matrix-core kernels take: those hold their 16-byte chunks
+    in the order in which a wave loads them as MFMA operands."""
+    key = (dtype, d)
+    if key not in _page_orders:
+        import numpy as np
+        k_idx = np.empty(PAGE_TOKENS * d, np.int32)
+        v_idx = np.empty(PAGE_TOKENS * d, np.int32)
+        _check(lib().picolm_kv_page_order(_DT[dtype], d, k_idx.ctypes.data_as(c_void_p), v_idx.ctypes.data_as(c_void_p)))
+        _page_orders[key] = (torch.from_numpy(k_idx.astype(np.int64)).reshape(PAGE_TOKENS, d),
+                             torch.from_numpy(v_idx.astype(np.int64)).reshape(d, PAGE_TOKENS))
+    return _page_orders[key]
+
+
+def kv_pages_pack(k: torch.Tensor, v: torch.Tensor):
+    """Pages given as plain arrays k [pages, G, 64, d], v [pages, G, d, 64] in the order the
+    kernels keep them (same shapes and dtype)."""
+    k_idx, v_idx = kv_page_order(k.dtype, k.shape[-1])
+    kp, vp = torch.empty_like(k), torch.empty_like(v)
+    kp.view(*k.shape[:2], -1)[..., k_idx.reshape(-1).to(k.device)] = k.reshape(*k.shape[:2], -1)
+    vp.view(*v.shape[:2], -1)[..., v_idx.reshape(-1).to(v.device)] = v.reshape(*v.shape[:2], -1)
+    return kp, vp
+
+
+def kv_pages_unpack(k_pages: torch.Tensor, v_pages: torch.Tensor):
+    """The kernels' pages as plain arrays k [pages, G, 64, d], v [pages, G, d, 64]."""
+    k_idx, v_idx = kv_page_order(k_pages.dtype, k_pages.shape[-1])
+    k = k_pages.reshape(*k_pages.shape[:2], -1)[..., k_idx.reshape(-1).to(k_pages.device)].view(k_pages.shape)
+    v = v_pages.reshape(*v_pages.shape[:2], -1)[..., v_idx.reshape(-1).to(v_pages.device)].view(v_pages.shape)
+    return k, v
 
 
 def _check_pages(who, k_pages, v_pages, dtype, G, d):

@@ -330,8 +330,8 @@ class PagedCase:
                 m = min(PAGE, t - j * PAGE)
                 kp[pg, :, :m, :] = torch.from_numpy(self.k[i][j * PAGE:j * PAGE + m]).permute(1, 0, 2).float()
                 vp[pg, :, :, :m] = torch.from_numpy(self.v[i][j * PAGE:j * PAGE + m]).permute(1, 2, 0).float()
-        self.k_pages = kp.to(dtype).to(DEV)
-        self.v_pages = vp.to(dtype).to(DEV)
+        # plain arrays above; the kernels keep some pages in an order of their own
+        self.k_pages, self.v_pages = K().kv_pages_pack(kp.to(dtype).to(DEV), vp.to(dtype).to(DEV))
         self.table_host = table
         self.table = table.to(DEV)
         # what the kernel sees after rounding to its storage type
@@ -476,10 +476,12 @@ def test_attention_decode_with_rotation_and_cache_write_inside(H, G, d, style, p
     ref = case.reference(window)
     # poison the new tokens' cache rows
     tok_page = b.write_pages(0, case.table_host, case.table_host.shape[1])
+    k_plain, v_plain = K().kv_pages_unpack(case.k_pages, case.v_pages)
     for i in range(n):
         pg, row = int(tok_page[i]), pos0[i] % PAGE
-        case.k_pages[pg, :, row, :] = float("nan")
-        case.v_pages[pg, :, :, row] = float("nan")
+        k_plain[pg, :, row, :] = float("nan")
+        v_plain[pg, :, :, row] = float("nan")
+    case.k_pages, case.v_pages = K().kv_pages_pack(k_plain, v_plain)
     out = torch.zeros(n, H * d, dtype=torch.bfloat16, device=DEV)
     chunk_list, n_chunks, most = decode_work_list(case, window, pages_per_chunk, spare=1)
     partial = torch.full((n * H * most * (d + 2),), float("nan"), device=DEV)
@@ -496,10 +498,11 @@ def test_attention_decode_with_rotation_and_cache_write_inside(H, G, d, style, p
         err = np.abs(out.double().cpu().numpy() - ref).max()
         assert err <= tol(torch.bfloat16, np.abs(ref).max()), err
         assert not done.any()
+    k_plain, v_plain = K().kv_pages_unpack(case.k_pages, case.v_pages)
     for i in range(n):
         pg, row = int(tok_page[i]), pos0[i] % PAGE
-        assert torch.equal(case.k_pages[pg, :, row, :].cpu(), bf(k_ref[i]))
-        assert torch.equal(case.v_pages[pg, :, :, row].cpu(), bf(v_ref[i]))
+        assert torch.equal(k_plain[pg, :, row, :].cpu(), bf(k_ref[i]))
+        assert torch.equal(v_plain[pg, :, :, row].cpu(), bf(v_ref[i]))
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
@@ -531,6 +534,24 @@ def test_attention_finds_a_far_key(dtype):
 
 
 # ------------------------------------------------------------------------------------------ rope
+@pytest.mark.parametrize("d", [16, 32, 48, 64, 128, 256])
+def test_kv_page_order_is_a_permutation(d):
+    """Every element of a page has one place; 32-bit pages and head sizes outside the matrix-core
+    kernels' are plain arrays; packing and unpacking undo each other."""
+    for dtype in (torch.float32, torch.bfloat16):
+        k_idx, v_idx = K().kv_page_order(dtype, d)
+        assert sorted(k_idx.reshape(-1).tolist()) == list(range(PAGE * d))
+        assert sorted(v_idx.reshape(-1).tolist()) == list(range(PAGE * d))
+        plain = dtype == torch.float32 or d not in (32, 64, 128)
+        assert (k_idx.reshape(-1).tolist() == list(range(PAGE * d))) == plain
+        assert (v_idx.reshape(-1).tolist() == list(range(PAGE * d))) == plain
+        k = torch.randn(3, 2, PAGE, d).to(dtype).to(DEV)
+        v = torch.randn(3, 2, d, PAGE).to(dtype).to(DEV)
+        kp, vp = K().kv_pages_pack(k, v)
+        k2, v2 = K().kv_pages_unpack(kp, vp)
+        assert torch.equal(k, k2) and torch.equal(v, v2)
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("style", ["pairwise", "half"])
 def test_rope_kv_store(dtype, style):
@@ -559,6 +580,7 @@ def test_rope_kv_store(dtype, style):
     v_ref = x[:, H + G:]
     t_ = tol(dtype, 4.0)
     assert np.abs(q_out.double().cpu().numpy() - q_ref).max() <= t_
+    kp, vp = K().kv_pages_unpack(kp, vp)
     kp, vp, tab = kp.double().cpu().numpy(), vp.double().cpu().numpy(), table.cpu().numpy()
     seq_of = np.repeat(np.arange(2), n_new)
     for t in range(T):
