@@ -117,9 +117,13 @@ int picolm_argmax(const float* logits, int32_t* out, int n_rows, int V, int64_t 
                   hipStream_t stream);
 // rng_states[state_index ? state_index[row] : row] is one xorshift64 state per sequence,
 // advanced by one draw when temperature > 0.
+// With a top_k small enough the row is cut into slices for many workgroups, which need scratch
+// memory: picolm_sample_scratch_bytes says how much (0: this case is one workgroup per row and
+// needs none); `scratch` may be null, then one workgroup per row does all the work.
+int picolm_sample_scratch_bytes(int n_rows, int V, float temperature, int top_k);
 int picolm_sample(const float* logits, int64_t ld, int n_rows, int V, float temperature, int top_k,
                   float top_p, float min_p, uint64_t* rng_states, const int32_t* state_index,
-                  int32_t* out, hipStream_t stream);
+                  int32_t* out, void* scratch, int64_t scratch_bytes, hipStream_t stream);
 
 #ifdef __cplusplus
 }

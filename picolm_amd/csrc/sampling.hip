@@ -549,14 +549,388 @@ __global__ __launch_bounds__(SM_THREADS) void sample_kernel(const float* __restr
     }
 }
 
+// ---------------------------------------------------------------------------------------------
+// With a top_k of a few dozen (picolm's default is 40) everything after the first cut works on
+// those k elements and on the softmax denominator.  Then a row is cut into slices, one workgroup
+// each: a slice leaves its maximum, its sum of exp(l - maximum) and its own k first elements in
+// the descending order (the row's k first are among them); one workgroup per row then orders the
+// candidates exactly and runs picolm's pipeline (sampler.c:58-121) on the first k.
+#define SLICE_VALUES 4096
+#define SLICE_THREADS 256
+#define SLICE_PER_THREAD (SLICE_VALUES / SLICE_THREADS)
+#define PICK_THREADS 1024
+#define PICK_MAX_CANDIDATES 4096
+#define PICK_MAX_TOP 1024
+
+struct SliceOut {          // per row and slice
+    float* max;            // [rows][slices]
+    double* sum;           // [rows][slices]
+    int32_t* count;        // [rows][slices]  candidates the slice left (min(k, its size))
+    uint32_t* key;         // [rows][slices][k]
+    int32_t* idx;          // [rows][slices][k]
+};
+__host__ __device__ inline size_t slice_out_bytes(int n_rows, int n_slices, int k) {
+    const size_t per = (size_t)n_rows * n_slices;
+    return per * 8 + per * 8 + per * 8 + per * k * 4 + per * k * 4;      // every part a multiple of 8 bytes
+}
+__host__ __device__ inline SliceOut slice_out_at(void* scratch, int n_rows, int n_slices, int k) {
+    const size_t per = (size_t)n_rows * n_slices;
+    char* p = (char*)scratch;
+    SliceOut o;
+    o.sum = (double*)p;
+    o.max = (float*)(p + per * 8);
+    o.count = (int32_t*)(p + per * 16);
+    o.key = (uint32_t*)(p + per * 24);
+    o.idx = (int32_t*)(p + per * 24 + per * k * 4);
+    return o;
+}
+
+// One wave finds, in a histogram of 256 bins, the bin that holds the `remaining`-th element
+// counted from the highest bin down, and how many elements lie in the bins above it.  The bins
+// hold at least `remaining` elements.
+__device__ __forceinline__ void find_bin(const unsigned* hist, unsigned remaining, int lane, unsigned& sel_bin,
+                                         unsigned& sel_above, unsigned& sel_count) {
+    // lane L holds bins 4L .. 4L+3; `above` counts the elements of all higher bins
+    const unsigned b0 = hist[4 * lane], b1 = hist[4 * lane + 1], b2 = hist[4 * lane + 2], b3 = hist[4 * lane + 3];
+    const unsigned mine = b0 + b1 + b2 + b3;
+    unsigned incl = mine;          // sum over lanes >= this one
+#pragma unroll
+    for (int s = 1; s < WAVE; s <<= 1) {
+        const unsigned other = __shfl_down(incl, s, WAVE);
+        if (lane + s < WAVE) incl += other;
+    }
+    unsigned above = incl - mine;
+    if (above < remaining && remaining <= incl) {        // one lane: the crossing is in its bins
+        int bin = 4 * lane + 3;
+        if (above + b3 < remaining) {
+            above += b3;
+            bin = 4 * lane + 2;
+            if (above + b2 < remaining) {
+                above += b2;
+                bin = 4 * lane + 1;
+                if (above + b1 < remaining) {
+                    above += b1;
+                    bin = 4 * lane;
+                }
+            }
+        }
+        sel_bin = (unsigned)bin;
+        sel_above = above;
+        sel_count = hist[bin];
+    }
+}
+
+__global__ __launch_bounds__(SLICE_THREADS) void sample_slice_kernel(const float* __restrict__ logits, int64_t ld,
+                                                                     int V, int k, SliceOut o) {
+    __shared__ unsigned hist[256];
+    __shared__ float red_f[SLICE_THREADS / WAVE];
+    __shared__ double red_d[SLICE_THREADS / WAVE];
+    __shared__ unsigned red_u[SLICE_THREADS / WAVE];
+    __shared__ unsigned sel_bin, sel_above, sel_count, n_out;
+    const int tid = threadIdx.x, wave = tid / WAVE, lane = tid % WAVE;
+    const int n_slices = gridDim.x;
+    const size_t slot = (size_t)blockIdx.y * n_slices + blockIdx.x;
+    const float* row = logits + (int64_t)blockIdx.y * ld;
+    const int lo = blockIdx.x * SLICE_VALUES;
+    const int n = min(SLICE_VALUES, V - lo);
+    // a thread holds 16 adjacent values, so that threads in order hold indices in order
+    float v[SLICE_PER_THREAD];
+    uint32_t key[SLICE_PER_THREAD];
+    const int first = tid * SLICE_PER_THREAD;
+    float mx = -INFINITY;
+#pragma unroll
+    for (int j = 0; j < SLICE_PER_THREAD; ++j) {
+        const bool ok = first + j < n;
+        v[j] = ok ? row[lo + first + j] : -INFINITY;
+        key[j] = order_key(v[j]);
+        if (ok) mx = fmaxf(mx, v[j]);
+    }
+#pragma unroll
+    for (int s = WAVE / 2; s > 0; s >>= 1) mx = fmaxf(mx, __shfl_xor(mx, s, WAVE));
+    if (lane == 0) red_f[wave] = mx;
+    __syncthreads();
+    mx = red_f[0];
+#pragma unroll
+    for (int w = 1; w < SLICE_THREADS / WAVE; ++w) mx = fmaxf(mx, red_f[w]);
+    double sum = 0.0;
+#pragma unroll
+    for (int j = 0; j < SLICE_PER_THREAD; ++j)
+        if (first + j < n) sum += exp((double)v[j] - (double)mx);
+#pragma unroll
+    for (int s = WAVE / 2; s > 0; s >>= 1) sum += __shfl_xor(sum, s, WAVE);
+    if (lane == 0) red_d[wave] = sum;
+    __syncthreads();
+    if (tid == 0) {
+        double t = 0.0;
+        for (int w = 0; w < SLICE_THREADS / WAVE; ++w) t += red_d[w];
+        o.sum[slot] = t;
+        o.max[slot] = mx;
+        o.count[slot] = min(k, n);
+        n_out = 0;
+    }
+    uint32_t* out_key = o.key + slot * k;
+    int32_t* out_idx = o.idx + slot * k;
+    if (n <= k) {                         // every element is a candidate
+#pragma unroll
+        for (int j = 0; j < SLICE_PER_THREAD; ++j)
+            if (first + j < n) {
+                out_key[first + j] = key[j];
+                out_idx[first + j] = lo + first + j;
+            }
+        return;
+    }
+    // the key of the k-th element in descending order, eight bits at a time from the top
+    uint32_t prefix = 0;
+    unsigned remaining = (unsigned)k;      // how many of the elements that share `prefix` are taken
+    int low_bits = 0;                      // bits of the key below `prefix` when the search ends
+    for (int pass = 0; pass < 4; ++pass) {
+        const int shift = 24 - 8 * pass;
+        hist[tid] = 0;                     // (256 threads, 256 bins)
+        __syncthreads();
+#pragma unroll
+        for (int j = 0; j < SLICE_PER_THREAD; ++j)
+            if (first + j < n && (pass == 0 || (key[j] >> (shift + 8)) == prefix)) atomicAdd(&hist[(key[j] >> shift) & 255], 1u);
+        __syncthreads();
+        if (wave == 0) find_bin(hist, remaining, lane, sel_bin, sel_above, sel_count);
+        __syncthreads();
+        prefix = (prefix << 8) | sel_bin;
+        remaining -= sel_above;
+        const bool whole_bin = sel_count == remaining;      // all that share the prefix are taken
+        __syncthreads();
+        if (whole_bin) {
+            low_bits = shift;
+            break;
+        }
+    }
+    // everything above the k-th key, and of its equals the first `remaining` by index (if the
+    // search ended early, `kth` is the least key with the prefix and all its "equals" are taken)
+    const uint32_t kth = prefix;
+    unsigned equals = 0;
+#pragma unroll
+    for (int j = 0; j < SLICE_PER_THREAD; ++j) {
+        key[j] >>= low_bits;
+        equals += (first + j < n && key[j] == kth) ? 1u : 0u;
+    }
+    unsigned scan = equals;                // inclusive over the lanes of the wave
+#pragma unroll
+    for (int s = 1; s < WAVE; s <<= 1) {
+        const unsigned other = __shfl_up(scan, s, WAVE);
+        if (lane >= s) scan += other;
+    }
+    if (lane == WAVE - 1) red_u[wave] = scan;
+    __syncthreads();
+    unsigned before = scan - equals;       // equals in threads before this one
+    for (int w = 0; w < wave; ++w) before += red_u[w];
+#pragma unroll
+    for (int j = 0; j < SLICE_PER_THREAD; ++j) {
+        if (first + j >= n) continue;
+        bool take = key[j] > kth;
+        if (key[j] == kth) take = before++ < remaining;
+        if (take) {
+            const unsigned pos = atomicAdd(&n_out, 1u);      // exactly k of them
+            out_key[pos] = order_key(v[j]);
+            out_idx[pos] = lo + first + j;
+        }
+    }
+}
+
+// A candidate as one number whose descending order is the pipeline's: the logit's key above,
+// the token id below, inverted so that of equal logits the lower id comes first.  0: no candidate.
+__device__ __forceinline__ uint64_t candidate(uint32_t key, int idx) {
+    return ((uint64_t)key << 32) | (uint32_t)(0x7fffffff - idx);
+}
+__device__ __forceinline__ uint32_t candidate_key(uint64_t c) { return (uint32_t)(c >> 32); }
+__device__ __forceinline__ int candidate_idx(uint64_t c) { return 0x7fffffff - (int)(uint32_t)c; }
+
+struct PickShared {
+    uint64_t cand[PICK_MAX_CANDIDATES];
+    uint64_t unordered[PICK_MAX_TOP];
+    uint64_t top[PICK_MAX_TOP];
+    double z_part[PICK_THREADS];       // a slice's share of the softmax denominator
+};
+
+__global__ __launch_bounds__(PICK_THREADS) void sample_pick_kernel(SliceOut o, int n_slices, int k, float temperature,
+                                                                   float top_p, float min_p,
+                                                                   uint64_t* __restrict__ rng_states,
+                                                                   const int32_t* __restrict__ state_index,
+                                                                   int32_t* __restrict__ out) {
+    __shared__ PickShared sm;
+    __shared__ unsigned hist[256];
+    __shared__ unsigned sel_bin, sel_above, sel_count;
+    __shared__ int n_valid, n_gathered;
+    const int tid = threadIdx.x;
+    const size_t slot0 = (size_t)blockIdx.x * n_slices;
+    const int n_slots = n_slices * k;
+    const int n_padded = (n_slots + 3) & ~3;
+    // asked for early: the generator's state, and the slices' maxima and sums
+    const int sidx = state_index ? state_index[blockIdx.x] : blockIdx.x;
+    const uint64_t state = tid == 0 ? rng_states[sidx] : 0;
+    float s_max = -INFINITY;
+    double s_sum = 0.0;
+    if (tid < n_slices) {                                  // (n_slices * k <= 4096 and k >= 1)
+        s_max = o.max[slot0 + tid];
+        s_sum = o.sum[slot0 + tid];
+    }
+    if (tid == 0) n_valid = n_gathered = 0;
+    __syncthreads();
+    int mine = 0;
+    for (int c = tid; c < n_padded; c += PICK_THREADS) {
+        const int s = c / k, j = c % k;
+        const bool ok = c < n_slots && j < o.count[slot0 + s];
+        sm.cand[c] = ok ? candidate(o.key[(slot0 + s) * k + j], o.idx[(slot0 + s) * k + j]) : 0ull;
+        mine += ok ? 1 : 0;
+    }
+    if (mine) atomicAdd(&n_valid, mine);
+    __syncthreads();
+    const int n_top = min(k, n_valid);
+    // the k-th candidate in descending order, eight bits at a time from the top
+    uint64_t kth = 1;                          // (every candidate is at least 1)
+    if (n_valid > k) {
+        uint64_t prefix = 0;
+        unsigned remaining = (unsigned)k;
+        for (int pass = 0; pass < 8; ++pass) {
+            const int shift = 56 - 8 * pass;
+            if (tid < 256) hist[tid] = 0;
+            __syncthreads();
+            for (int c = tid; c < n_slots; c += PICK_THREADS) {
+                const uint64_t me = sm.cand[c];
+                if (me != 0ull && (pass == 0 || (me >> (shift + 8)) == prefix)) atomicAdd(&hist[(unsigned)(me >> shift) & 255u], 1u);
+            }
+            __syncthreads();
+            if (tid < WAVE) find_bin(hist, remaining, tid, sel_bin, sel_above, sel_count);
+            __syncthreads();
+            prefix = (prefix << 8) | sel_bin;
+            remaining -= sel_above;
+            const bool whole_bin = sel_count == remaining;      // all that share the prefix are taken
+            __syncthreads();
+            if (whole_bin) {
+                prefix <<= shift;
+                break;
+            }
+        }
+        kth = prefix;
+    }
+    // the first k, gathered in any order, then put in order: a candidate's place is the number
+    // of greater ones among them
+    for (int c = tid; c < n_slots; c += PICK_THREADS) {
+        const uint64_t me = sm.cand[c];
+        if (me != 0ull && me >= kth) sm.unordered[atomicAdd(&n_gathered, 1)] = me;
+    }
+    __syncthreads();
+    for (int c = tid; c < n_top; c += PICK_THREADS) {
+        const uint64_t me = sm.unordered[c];
+        int rank = 0;
+        for (int j = 0; j < n_top; ++j) rank += sm.unordered[j] > me ? 1 : 0;
+        sm.top[rank] = me;
+    }
+    __syncthreads();
+    // the candidates' place now holds the weights of the first k: exp(l - max), exp((l - max) / T)
+    double* w_plain = (double*)sm.cand;
+    double* w_temp = w_plain + PICK_MAX_TOP;
+    // the row's maximum is the first candidate's logit; every thread weighs candidates and slices
+    const double lmax = (double)key_value(candidate_key(sm.top[0]));
+    const double inv_t = 1.0 / (double)temperature;
+    for (int j = tid; j < n_top; j += PICK_THREADS) {
+        const double x = (double)key_value(candidate_key(sm.top[j])) - lmax;
+        w_plain[j] = exp(x);
+        w_temp[j] = exp(x * inv_t);
+    }
+    if (tid < n_slices) sm.z_part[tid] = s_sum * exp((double)s_max - lmax);
+    __syncthreads();
+    if (tid != 0) return;
+    double Z = 0.0;                                                // the softmax denominator
+    for (int s = 0; s < n_slices; ++s) Z += sm.z_part[s];
+    const int top_token = candidate_idx(sm.top[0]);
+    int kept = n_top;                                              // sampler.c:70-73
+    if (top_p < 1.0f) {                                            // sampler.c:76-82
+        const double target = (double)top_p * Z;
+        double cum = 0.0;
+        bool hit = false;
+        for (int j0 = 0; j0 < n_top && !hit; j0 += 8) {            // eight weights are read at a time
+            double w[8];
+#pragma unroll
+            for (int e = 0; e < 8; ++e) w[e] = w_plain[min(j0 + e, n_top - 1)];
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                cum += w[e];
+                if (!hit && j0 + e < n_top && cum >= target) {
+                    kept = j0 + e + 1;
+                    hit = true;
+                }
+            }
+        }
+    }
+    if (min_p > 0.0f && kept > 1) {                                // sampler.c:85-95
+        int m = 0;
+        while (m < kept && w_plain[m] >= (double)min_p) ++m;
+        kept = m > 0 ? m : 1;                                      // keep at least the top token
+    }
+    // sampler.c:98-121
+    double W = 0.0;
+    for (int j0 = 0; j0 < kept; j0 += 8) {
+        double w[8];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) w[e] = w_temp[min(j0 + e, kept - 1)];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) W += j0 + e < kept ? w[e] : 0.0;
+    }
+    const uint64_t x = xorshift64(state);
+    const float rnd = (float)(x >> 11) / 9007199254740992.0f;      // sampler.c:19-21
+    const double target = (double)rnd * W;
+    int chosen = top_token;
+    double cum = 0.0;
+    bool hit = false;
+    for (int j0 = 0; j0 < kept && !hit; j0 += 8) {
+        double w[8];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) w[e] = w_temp[min(j0 + e, kept - 1)];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            cum += w[e];
+            if (!hit && j0 + e < kept && cum > target) {
+                chosen = candidate_idx(sm.top[j0 + e]);
+                hit = true;
+            }
+        }
+    }
+    out[blockIdx.x] = chosen;
+    rng_states[sidx] = x;
+}
+
+// Whether the sliced kernels take this case, and the scratch memory they need then (0: they do not).
+extern "C" int picolm_sample_scratch_bytes(int n_rows, int V, float temperature, int top_k) {
+    if (!(temperature > 0.0f) || top_k <= 0 || top_k >= V || top_k > PICK_MAX_TOP || n_rows <= 0) return 0;
+    const int n_slices = ceil_div(V, SLICE_VALUES);
+    if ((int64_t)n_slices * top_k > PICK_MAX_CANDIDATES || n_slices > PICK_THREADS) return 0;
+    const size_t bytes = slice_out_bytes(n_rows, n_slices, top_k);
+    return bytes < (1u << 30) ? (int)bytes : 0;
+}
+
+// `scratch`: picolm_sample_scratch_bytes(...) bytes of device memory, 8-byte aligned, or null;
+// without it, or where that function says 0, one workgroup per row does all the work.
 extern "C" int picolm_sample(const float* logits, int64_t ld, int n_rows, int V, float temperature,
                              int top_k, float top_p, float min_p, uint64_t* rng_states,
-                             const int32_t* state_index, int32_t* out, hipStream_t stream) {
+                             const int32_t* state_index, int32_t* out, void* scratch, int64_t scratch_bytes,
+                             hipStream_t stream) {
     PICOLM_REQUIRE(n_rows >= 0 && V > 0 && ld >= V, "sample: bad sizes rows=%d V=%d ld=%lld", n_rows, V,
                    (long long)ld);
     PICOLM_REQUIRE(temperature <= 0.0f || rng_states != nullptr, "sample: a temperature needs generator states");
     PICOLM_REQUIRE(top_p > 0.0f || temperature <= 0.0f, "sample: top_p must be positive, got %g", top_p);
     if (n_rows == 0) return 0;
+    const int need = picolm_sample_scratch_bytes(n_rows, V, temperature, top_k);
+    if (need > 0 && scratch != nullptr && n_rows <= 65535) {
+        PICOLM_REQUIRE(scratch_bytes >= need && ((uintptr_t)scratch & 7) == 0,
+                       "sample: the scratch buffer holds %lld bytes, %lld are needed (8-byte aligned)",
+                       (long long)scratch_bytes, (long long)need);
+        const int n_slices = ceil_div(V, SLICE_VALUES);
+        const SliceOut o = slice_out_at(scratch, n_rows, n_slices, top_k);
+        sample_slice_kernel<<<dim3(n_slices, n_rows), dim3(SLICE_THREADS), 0, stream>>>(logits, ld, V, top_k, o);
+        PICOLM_LAUNCH_CHECK("sample");
+        sample_pick_kernel<<<dim3(n_rows), dim3(PICK_THREADS), 0, stream>>>(o, n_slices, top_k, temperature, top_p,
+                                                                           min_p, rng_states, state_index, out);
+        PICOLM_LAUNCH_CHECK("sample");
+        return 0;
+    }
     sample_kernel<<<dim3(n_rows), dim3(SM_THREADS), 0, stream>>>(logits, ld, V, temperature, top_k, top_p, min_p,
                                                                rng_states, state_index, out);
     PICOLM_LAUNCH_CHECK("sample");

@@ -42,7 +42,7 @@ def dir_entry_points():
     return ["picolm_abi_version", "picolm_device_check", "picolm_embed", "picolm_rmsnorm",
             "picolm_rope_kv_store", "picolm_silu_mul", "picolm_add_into", "picolm_gemm_generic",
             "picolm_attn_prefill_tile_rows", "picolm_attn_prefill_generic",
-            "picolm_attn_decode_generic", "picolm_argmax", "picolm_argmax_scratch_floats", "picolm_sample", "picolm_gemm_skinny", "picolm_gemm_tiled", "picolm_gemm_tiled_splitk", "picolm_gemm_linked", "picolm_kv_page_order",
+            "picolm_attn_decode_generic", "picolm_argmax", "picolm_argmax_scratch_floats", "picolm_sample", "picolm_sample_scratch_bytes", "picolm_gemm_skinny", "picolm_gemm_tiled", "picolm_gemm_tiled_splitk", "picolm_gemm_linked", "picolm_kv_page_order",
             "picolm_attn_mfma_takes", "picolm_attn_prefill_mfma_heads", "picolm_attn_prefill_mfma_tile_tokens",
             "picolm_attn_prefill_mfma", "picolm_attn_decode_mfma", "picolm_attn_decode_rope_mfma", "picolm_attn_decode_mfma_waves", "picolm_read_probe", "picolm_mfma_probe"]
 
@@ -576,9 +576,16 @@ def attn_decode(q, k_pages, v_pages, out, partial, n_seq, chunk_list, n_chunks, 
                             max_splits, seq_pos0, page_table, ring_pages, H, G, d, window, scale)
 
 
+def sample_scratch_bytes(n_rows: int, V: int, temperature: float, top_k: int) -> int:
+    """Scratch memory with which `sample` spreads a row over many workgroups (0: it cannot)."""
+    return lib().picolm_sample_scratch_bytes(n_rows, V, c_float(temperature), int(top_k))
+
+
 def sample(logits: torch.Tensor, out: torch.Tensor, temperature: float, top_k: int, top_p: float,
-           min_p: float, rng_states: torch.Tensor | None, state_index: torch.Tensor | None) -> None:
-    """One token per row of `logits`; `rng_states` (int64 bits of xorshift64 states) advance."""
+           min_p: float, rng_states: torch.Tensor | None, state_index: torch.Tensor | None,
+           scratch: torch.Tensor | None = None) -> None:
+    """One token per row of `logits`; `rng_states` (int64 bits of xorshift64 states) advance.
+    `scratch` (uint8, sample_scratch_bytes): without it one workgroup per row does all the work."""
     _dev("sample.logits", logits, torch.float32, 2)
     n, V = logits.shape
     _i32("sample.out", out, n)
@@ -588,8 +595,11 @@ def sample(logits: torch.Tensor, out: torch.Tensor, temperature: float, top_k: i
             _i32("sample.state_index", state_index, n)
         elif rng_states.numel() < n:
             raise KernelError("sample: fewer generator states than rows")
+    if scratch is not None:
+        _dev("sample.scratch", scratch, torch.uint8)
     _check(lib().picolm_sample(_ptr(logits), c_int64(V), n, V, c_float(temperature), int(top_k), c_float(top_p),
-                               c_float(min_p), _ptr(rng_states), _ptr(state_index), _ptr(out), _stream()))
+                               c_float(min_p), _ptr(rng_states), _ptr(state_index), _ptr(out), _ptr(scratch),
+                               c_int64(scratch.numel() if scratch is not None else 0), _stream()))
 
 
 def read_probe(src: torch.Tensor, sink: torch.Tensor, blocks: int = 4096, unroll4: bool = True) -> None:

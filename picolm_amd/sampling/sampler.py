@@ -27,6 +27,9 @@ class Sampler:
         if self.device.type == "cuda":
             self._host_out = self._host_out.pin_memory()
         self._scratch = None
+        self._sample_scratch = None
+        self._idx_of = None                   # the sequence indices that `_idx` holds
+        self._idx = None
 
     def sample(self, logits: torch.Tensor, sequence_indices) -> list[int]:
         """`logits[i]` belongs to sequence `sequence_indices[i]`; returns one token each."""
@@ -39,8 +42,15 @@ class Sampler:
                 self._scratch = torch.empty(need, dtype=torch.float32, device=self.device)
             kernels.argmax(logits, out, self._scratch)
         else:
-            idx = torch.tensor(list(sequence_indices), dtype=torch.int32).to(self.device)
-            kernels.sample(logits, out, p.temperature, p.top_k, p.top_p, p.min_p, self.states, idx)
+            seqs = list(sequence_indices)
+            if seqs != self._idx_of:          # the same batch step after step: one upload
+                self._idx = torch.tensor(seqs, dtype=torch.int32).to(self.device)
+                self._idx_of = seqs
+            need = kernels.sample_scratch_bytes(n, logits.shape[1], p.temperature, p.top_k)
+            if need and (self._sample_scratch is None or self._sample_scratch.numel() < need):
+                self._sample_scratch = torch.empty(need, dtype=torch.uint8, device=self.device)
+            kernels.sample(logits, out, p.temperature, p.top_k, p.top_p, p.min_p, self.states, self._idx,
+                           self._sample_scratch if need else None)
         host = self._host_out[:n]
         host.copy_(out, non_blocking=True)
         torch.cuda.current_stream().synchronize()

@@ -602,7 +602,8 @@ def test_argmax_first_maximum():
 
 @pytest.mark.parametrize("V,scale", [(131, 1.0), (5000, 0.5), (128256, 1.0)])
 @pytest.mark.parametrize("opts", [(0.8, 0, 1.0, 0.0), (0.8, 40, 0.9, 0.05), (1.3, 0, 0.7, 0.0), (0.5, 7, 1.0, 0.2),
-                                  (1.0, 0, 1.0, 0.3), (0.0, 0, 1.0, 0.0)])
+                                  (1.0, 0, 1.0, 0.3), (0.0, 0, 1.0, 0.0), (0.9, 1000, 0.95, 0.0), (1.0, 1, 1.0, 0.0),
+                                  (0.7, 130, 1.0, 0.0), (1.1, 40, 1.0, 0.0)])
 def test_sampler_equals_plain(V, scale, opts):
     from picolm_amd.sampling import Sampler, SamplingParams, stream_state
     T, k, p, mp = opts
@@ -620,6 +621,38 @@ def test_sampler_equals_plain(V, scale, opts):
         for i in range(n):
             want, states[i] = SP.sample(logits[i], T, k, p, mp, states[i])
             assert got[i] == want, (i, got[i], want)
+
+
+@pytest.mark.parametrize("V", [131, 4096, 4097, 9000, 128256])
+def test_sampler_sliced_and_one_workgroup_kernels_agree(V):
+    """With a small top_k a row is cut into slices for many workgroups; one workgroup per row does
+    the same work without scratch memory.  Both must draw the same tokens from the same states:
+    rows with all logits equal, many equal, a dominant one, equal values across a slice's border."""
+    k = K()
+    rng = np.random.default_rng(V)
+    n = 6
+    logits = rng.standard_normal((n, V)).astype(np.float32)
+    logits[0, :] = -1.5
+    logits[1, ::3] = 2.0
+    logits[2, V // 2] = 30.0
+    logits[3, max(0, min(V, 4096) - 20):min(V, 4096 + 20)] = 3.25
+    lg = torch.from_numpy(logits).to(DEV)
+    for T, top_k, top_p, min_p in ((0.8, 40, 0.9, 0.05), (1.0, 5, 1.0, 0.0), (0.6, 64, 0.5, 0.0), (1.5, 100, 1.0, 0.01)):
+        if top_k >= V:
+            continue
+        need = k.sample_scratch_bytes(n, V, T, top_k)
+        assert need > 0
+        scratch = torch.empty(need, dtype=torch.uint8, device=DEV)
+        st_a = torch.arange(1, n + 1, dtype=torch.int64, device=DEV) * 2654435761
+        st_b = st_a.clone()
+        out_a = torch.zeros(n, dtype=torch.int32, device=DEV)
+        out_b = torch.zeros(n, dtype=torch.int32, device=DEV)
+        for _ in range(8):
+            k.sample(lg, out_a, T, top_k, top_p, min_p, st_a, None, scratch)
+            k.sample(lg, out_b, T, top_k, top_p, min_p, st_b, None, None)
+            assert out_a.tolist() == out_b.tolist(), (V, T, top_k, top_p, min_p)
+            assert torch.equal(st_a, st_b)
+    assert k.sample_scratch_bytes(n, V, 0.0, 40) == 0 and k.sample_scratch_bytes(n, V, 0.8, 0) == 0
 
 
 def test_sampler_streams_do_not_depend_on_the_batch():
