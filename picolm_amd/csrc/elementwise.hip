@@ -72,10 +72,11 @@ __global__ __launch_bounds__(NORM_THREADS) void rmsnorm_kernel(const float* __re
         for (int j = 0; j < NORM_REGS; ++j) {
             const int idx = threadIdx.x + j * NORM_THREADS;
             if (idx < nv) {
-                o[4 * idx + 0] = from_f32<TO>((v[j].x * scale) * ww[j].x);
-                o[4 * idx + 1] = from_f32<TO>((v[j].y * scale) * ww[j].y);
-                o[4 * idx + 2] = from_f32<TO>((v[j].z * scale) * ww[j].z);
-                o[4 * idx + 3] = from_f32<TO>((v[j].w * scale) * ww[j].w);
+                // one store of four values (D % 4 == 0 and the rows of `out` are dense, so it is aligned)
+                struct alignas(4 * sizeof(TO)) Four { TO a, b, c, d; };
+                Four f = {from_f32<TO>((v[j].x * scale) * ww[j].x), from_f32<TO>((v[j].y * scale) * ww[j].y),
+                          from_f32<TO>((v[j].z * scale) * ww[j].z), from_f32<TO>((v[j].w * scale) * ww[j].w)};
+                ((Four*)o)[idx] = f;
             }
         }
         return;
@@ -93,6 +94,8 @@ extern "C" int picolm_rmsnorm(const float* x, const float* w, void* out, int out
                               const int32_t* rows, int n_rows, int D, float eps,
                               hipStream_t stream) {
     PICOLM_REQUIRE(n_rows >= 0 && D > 0, "rmsnorm: bad sizes rows=%d D=%d", n_rows, D);
+    PICOLM_REQUIRE(D % 4 != 0 || ((((uintptr_t)x | (uintptr_t)w) & 15) == 0 && ((uintptr_t)out & 15) == 0),
+                   "rmsnorm: rows of a multiple of four values are read and written four at a time and must be 16-byte aligned");
     if (n_rows == 0) return 0;
     dim3 grid(n_rows), block(NORM_THREADS);
     if (out_dt == PICOLM_F32)
@@ -132,35 +135,45 @@ __global__ void rope_kv_store_kernel(const float* __restrict__ qkv, TC* __restri
     size_t page_base = 0;
     const int in_page = pos % PAGE_TOKENS;
     if (k_pages) page_base = ((size_t)tok_page[t] * G) * PAGE_TOKENS * d;
-    // blockIdx.y takes ROPE_HEADS heads of the row: heads 0..H-1 are q, H..H+G-1 are k, then v
-    const int head_lo = blockIdx.y * ROPE_HEADS, head_hi = min(head_lo + ROPE_HEADS, H + 2 * G);
-    for (int head = head_lo; head < head_hi; ++head) {
-        if (head < H + G) {
-            for (int i = threadIdx.x; i < half; i += blockDim.x) {
-                const int i0 = style == 0 ? 2 * i : i;
-                const int i1 = style == 0 ? 2 * i + 1 : i + half;
-                const float x0 = row[head * d + i0], x1 = row[head * d + i1];
-                float y0 = x0, y1 = x1;
-                if (c) {
-                    const float cc = c[i], ss = s[i];
-                    y0 = x0 * cc - x1 * ss;
-                    y1 = x0 * ss + x1 * cc;
-                }
-                if (head < H) {
-                    TC* q = q_out + (size_t)t * H * d + head * d;
-                    q[i0] = from_f32<TC>(y0);
-                    q[i1] = from_f32<TC>(y1);
-                } else if (k_pages) {
+    // blockIdx.y takes ROPE_HEADS heads of the row: heads 0..H-1 are q, H..H+G-1 are k, then v.
+    // A thread takes pair i of every head: all the heads' values are asked for before the first
+    // is used, and a value head goes the same way as a key head without a rotation.
+    const int head_lo = blockIdx.y * ROPE_HEADS, n_heads = H + 2 * G;
+    for (int i = threadIdx.x; i < half; i += blockDim.x) {
+        const int i0 = style == 0 ? 2 * i : i;
+        const int i1 = style == 0 ? 2 * i + 1 : i + half;
+        float x0[ROPE_HEADS], x1[ROPE_HEADS];
+#pragma unroll
+        for (int hh = 0; hh < ROPE_HEADS; ++hh) {
+            const int head = min(head_lo + hh, n_heads - 1);
+            x0[hh] = row[head * d + i0];
+            x1[hh] = row[head * d + i1];
+        }
+        const float cc = c ? c[i] : 1.0f, ss = c ? s[i] : 0.0f;
+#pragma unroll
+        for (int hh = 0; hh < ROPE_HEADS; ++hh) {
+            const int head = head_lo + hh;
+            if (head >= n_heads) break;
+            float y0 = x0[hh], y1 = x1[hh];
+            if (c && head < H + G) {
+                y0 = x0[hh] * cc - x1[hh] * ss;
+                y1 = x0[hh] * ss + x1[hh] * cc;
+            }
+            if (head < H) {
+                TC* q = q_out + (size_t)t * H * d + head * d;
+                q[i0] = from_f32<TC>(y0);
+                q[i1] = from_f32<TC>(y1);
+            } else if (head < H + G) {
+                if (k_pages) {
                     TC* k = k_pages + page_base + (size_t)(head - H) * PAGE_TOKENS * d;
                     k[k_page_offset(in_page, i0, d, tiled)] = from_f32<TC>(y0);
                     k[k_page_offset(in_page, i1, d, tiled)] = from_f32<TC>(y1);
                 }
+            } else if (v_pages) {
+                TC* v = v_pages + page_base + (size_t)(head - H - G) * PAGE_TOKENS * d;
+                v[v_page_offset(i0, in_page, d, tiled)] = from_f32<TC>(y0);
+                v[v_page_offset(i1, in_page, d, tiled)] = from_f32<TC>(y1);
             }
-        } else if (v_pages) {
-            const int g = head - H - G;
-            const float* vrow = row + (size_t)head * d;
-            for (int i = threadIdx.x; i < d; i += blockDim.x)
-                v_pages[page_base + (size_t)g * PAGE_TOKENS * d + v_page_offset(i, in_page, d, tiled)] = from_f32<TC>(vrow[i]);
         }
     }
 }
