@@ -152,7 +152,8 @@ __device__ __forceinline__ void attend_tile(const bf16x8 (&Qf)[D / 16], const bf
 // LDS tiles of the prefill kernel: a page's K and V^T as they lie in the cache, that is in the
 // order of the MFMA operands: the 64 lanes of a wave read 64 adjacent 16-byte chunks.
 template <int D>
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void attn_prefill_mfma_kernel(AttnArgs a, int HB, int tile_tokens) {
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void attn_prefill_mfma_kernel(AttnArgs a, int HB, int tile_tokens,
+                                                                                                        int n_tiles, int n_cus) {
     constexpr int KCH = D / 8;                        // 16-byte chunks of a K row
     constexpr int KP = PAGE_TOKENS * KCH / 256;       // K chunks a thread stages per page
     constexpr int VP = D * 8 / 256;                   // V^T chunks a thread stages per page
@@ -162,10 +163,19 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void a
     const int l32 = lane % 32, h = lane / 32;
     const int R = a.H / a.G;
     const int head_chunks = (R + HB - 1) / HB;
-    // long tiles first: the last tiles of a sequence see the most keys
-    const int tile_id = gridDim.x - 1 - blockIdx.x;
+    // The host lists the tiles with the fewest keys first.  Work items (tile, group of heads) are
+    // handed out longest first, in rounds of one workgroup per CU, and every other round runs
+    // backwards: the workgroups that share a CU from the start (a CU holds two) then have a long
+    // and a short tile, where the same order in every round would pair the longest with each other.
+    const int per_tile = a.G * head_chunks;
+    const int total = n_tiles * per_tile;
+    const int round0 = (int)(blockIdx.x / n_cus) * n_cus, in_round = blockIdx.x - round0;
+    const int round_size = min(n_cus, total - round0);
+    const int item = round0 + (((blockIdx.x / n_cus) & 1) ? round_size - 1 - in_round : in_round);
+    const int tile_id = n_tiles - 1 - item / per_tile;
+    const int which = item % per_tile;
     const int seq = a.tile_seq[tile_id], q0 = a.tile_q0[tile_id];
-    const int g = blockIdx.y / head_chunks, chunk = blockIdx.y % head_chunks;
+    const int g = which / head_chunks, chunk = which % head_chunks;
     const int head_local = chunk * HB + wave % HB;
     const int tb = wave / HB;
     const int nnew = a.seq_nnew[seq], pos0 = a.seq_pos0[seq];
@@ -592,14 +602,22 @@ extern "C" int picolm_attn_prefill_mfma(const void* q, const void* k_pages, cons
     const int HB = picolm_attn_prefill_mfma_heads(H, G);
     const int tile_tokens = 32 * (4 / HB);
     const int head_chunks = ceil_div(H / G, HB);
-    PICOLM_REQUIRE(G * head_chunks <= 65535, "attn_prefill_mfma: %d head groups exceed the grid", G * head_chunks);
     AttnArgs a = {q, k_pages, v_pages, out, nullptr, tile_seq, tile_q0, seq_slot, seq_pos0, seq_nnew,
                   cu_seqlens, page_table, max_pages, ring_pages, H, G, d, window, scale, 0, nullptr, 0, 1,
                   nullptr, nullptr, nullptr, nullptr, 0};
-    dim3 grid(n_tiles, G * head_chunks), block(256);
+    PICOLM_REQUIRE((int64_t)n_tiles * G * head_chunks < (1ll << 31), "attn_prefill_mfma: too many workgroups");
+    static int n_cus = 0;
+    if (n_cus == 0) {
+        int dev = 0;
+        hipDeviceProp_t prop;
+        PICOLM_REQUIRE(hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess,
+                       "attn_prefill_mfma: cannot read the device's properties");
+        n_cus = prop.multiProcessorCount > 0 ? prop.multiProcessorCount : 1;
+    }
+    dim3 grid(n_tiles * G * head_chunks), block(256);
     const size_t lds = 2 * 2 * (size_t)PAGE_TOKENS * d * sizeof(bf16_t);       // two stages of K and V^T
-    if (d == 32) attn_prefill_mfma_kernel<32><<<grid, block, lds, stream>>>(a, HB, tile_tokens);
-    else if (d == 64) attn_prefill_mfma_kernel<64><<<grid, block, lds, stream>>>(a, HB, tile_tokens);
+    if (d == 32) attn_prefill_mfma_kernel<32><<<grid, block, lds, stream>>>(a, HB, tile_tokens, n_tiles, n_cus);
+    else if (d == 64) attn_prefill_mfma_kernel<64><<<grid, block, lds, stream>>>(a, HB, tile_tokens, n_tiles, n_cus);
     else {
         static bool raised = false;
         if (!raised) {
@@ -608,7 +626,7 @@ extern "C" int picolm_attn_prefill_mfma(const void* q, const void* k_pages, cons
             PICOLM_REQUIRE(e == hipSuccess, "attn_prefill_mfma: cannot raise the LDS limit: %s", hipGetErrorString(e));
             raised = true;
         }
-        attn_prefill_mfma_kernel<128><<<grid, block, lds, stream>>>(a, HB, tile_tokens);
+        attn_prefill_mfma_kernel<128><<<grid, block, lds, stream>>>(a, HB, tile_tokens, n_tiles, n_cus);
     }
     PICOLM_LAUNCH_CHECK("attn_prefill_mfma");
     return 0;

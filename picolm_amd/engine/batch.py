@@ -93,11 +93,13 @@ class StepBatch:
     def prefill_tiles(self, rows_per_tile: int):
         """(tile_seq, tile_q0, n_tiles) on the device: tiles of `rows_per_tile` new tokens."""
         if rows_per_tile not in self._tiles:
-            seqs, q0s = [], []
+            tiles = []
             for i, n in enumerate(self.n_new):
                 for q0 in range(0, n, rows_per_tile):
-                    seqs.append(i)
-                    q0s.append(q0)
+                    tiles.append((self.pos0[i] + min(q0 + rows_per_tile, n), i, q0))
+            tiles.sort()          # by the keys a tile sees: the kernels hand out the longest first
+            seqs = [t[1] for t in tiles]
+            q0s = [t[2] for t in tiles]
             flat = torch.tensor(seqs + q0s, dtype=torch.int32).to(self._device)
             self._tiles[rows_per_tile] = (flat[:len(seqs)], flat[len(seqs):], len(seqs))
         return self._tiles[rows_per_tile]
@@ -200,6 +202,7 @@ class _Chunk:
     def __init__(self, parent: StepBatch, seqs, lo, n_new, first_rows):
         self.n_seq = len(seqs)
         self.n_new = n_new
+        self.pos0 = [parent.pos0[i] + lo for i in seqs]
         self.max_new = max(n_new)
         self.is_decode = False
         rows = np.concatenate([np.arange(r, r + n, dtype=np.int32) for r, n in zip(first_rows, n_new)])
@@ -208,7 +211,7 @@ class _Chunk:
         self._tiles = {}
         StepBatch._upload(self, {
             "seq_slot": np.asarray([parent.slots[i] for i in seqs], dtype=np.int32),
-            "seq_pos0": np.asarray([parent.pos0[i] + lo for i in seqs], dtype=np.int32),
+            "seq_pos0": np.asarray(self.pos0, dtype=np.int32),
             "seq_nnew": np.asarray(n_new, dtype=np.int32),
             "cu_seqlens": np.asarray(first_rows, dtype=np.int32),
             "rows": rows,

@@ -167,3 +167,16 @@ def test_decode_batch_looks_pages_up_again_when_the_cache_changed():
     table += 100
     b.fill([0, 1], [13, 73], [1, 1])                    # no version given: never the short way
     assert pages.tolist() == [200, 209]
+
+
+def test_prefill_tiles_are_listed_by_the_keys_they_see():
+    """Fewest keys first (the kernels hand out the longest first); every tile once."""
+    b = StepBatch([0, 1, 2], [100, 0, 5], [[1] * 70, [1] * 200, [1] * 33], [[], [], []], 10, "cpu")
+    seq, q0, n = b.prefill_tiles(32)
+    tiles = list(zip(seq.tolist(), q0.tolist()))
+    assert n == 3 + 7 + 2 and sorted(tiles) == sorted((i, q) for i, m in enumerate([70, 200, 33]) for q in range(0, m, 32))
+    ends = [[100, 0, 5][i] + min(q + 32, [70, 200, 33][i]) for i, q in tiles]
+    assert ends == sorted(ends)
+    for c in b.chunks(64):                       # a step cut along positions lists its own tiles
+        seq_c, q0_c, n_c = c.prefill_tiles(32)
+        assert n_c == sum((m + 31) // 32 for m in c.n_new)
