@@ -173,7 +173,8 @@ def decode_chunk_list(slots, pos0, window: int, pages_per_chunk: int, table_host
     """(entries [n][8] int32, most chunks of one sequence): every sequence's visible pages
     (those of its last `window` keys, or all) cut into runs of `pages_per_chunk`.  An entry is
     {sequence, which chunk, position of the new token, slot, physical pages of the chunk's first
-    four pages or -1}; the kernels derive each chunk's pages from the same arithmetic."""
+    four pages or -1}; the kernels derive each chunk's pages from the same arithmetic.  The
+    entries come in no particular order of sequences: every entry says whose it is."""
     pos = np.asarray(pos0, dtype=np.int64)
     slot = np.asarray(slots, dtype=np.int64)
     first = (np.maximum(0, pos - window + 1) if window > 0 else np.zeros_like(pos)) // PAGE_TOKENS
@@ -181,6 +182,11 @@ def decode_chunk_list(slots, pos0, window: int, pages_per_chunk: int, table_host
     n = (end - first + pages_per_chunk - 1) // pages_per_chunk
     seq = np.repeat(np.arange(len(pos), dtype=np.int64), n)
     idx = np.arange(int(n.sum())) - np.repeat(np.cumsum(n) - n, n)
+    # the chunks with the most pages first: workgroups are handed out in the list's order, and
+    # the short last chunks of the sequences then fill the gaps at the end
+    n_pages = np.minimum(end[seq] - first[seq] - idx * pages_per_chunk, pages_per_chunk)
+    order = np.argsort(-n_pages, kind="stable")
+    seq, idx = seq[order], idx[order]
     entries = np.empty((len(seq), CHUNK_ENTRY_INTS), dtype=np.int32)
     entries[:, 0] = seq
     entries[:, 1] = idx
