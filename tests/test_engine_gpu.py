@@ -21,7 +21,7 @@ pytestmark = pytest.mark.gpu
 DEV = "cuda:0"
 
 LENGTHS = {"A": [33, 47, 64, 65, 100, 128], "B": [33, 40, 64, 129, 200, 256], "C": [34, 63, 65, 128, 190, 300],
-           "D": [33, 50, 64, 127, 130, 260]}
+           "D": [33, 50, 64, 127, 130, 260], "E": [33, 64, 70, 129, 200, 320]}
 
 
 def tolerance(dtype, ref):
@@ -47,7 +47,7 @@ def requests_and_truth(folders):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("which", ["A", "B", "C", "D"])
+@pytest.mark.parametrize("which", ["A", "B", "C", "D", "E"])
 def test_replay_whole_tail_and_batches(which, dtype, folders, requests_and_truth, tmp_path):
     reqs, truth = requests_and_truth[which]
     one_batch = sum((len(r) + 63) // 64 for r in reqs[3:]) * 64          # room for the larger batch only
@@ -104,6 +104,32 @@ def test_replay_reports_a_full_cache(folders, tmp_path):
 def session(folder, dtype, max_tokens=2048, **kw):
     from picolm_amd.engine import Session, load_model
     return Session(load_model(folder, dtype=dtype), max_tokens=max_tokens, **kw)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("which,n_seq", [("E", 20), ("E", 64), ("D", 33)])
+def test_a_wide_batch_decodes_like_its_sequences_alone(which, n_seq, dtype, folders):
+    """Decode batches of 17 to 64 sequences take kernels of their own (tiles of 64 rows cut along
+    K, the norm split between the products where the widths allow).  Unequal prompts, six steps,
+    every sequence's logits against the plain implementation of that sequence alone."""
+    d = folders[which]
+    V = tiny.read_config(d)["vocab_size"]
+    rng = np.random.default_rng(n_seq)
+    lens = [int(x) for x in rng.integers(3, 90, size=n_seq)]
+    n_dec = 6
+    seqs = [tiny.random_tokens(rng, n + n_dec, V) for n in lens]
+    truth = [tiny.plain_logits(d, q) for q in seqs]
+    s = session(d, dtype, max_tokens=n_seq * 192, n_slots=n_seq)
+    slots = s.begin(n_seq)
+    got = s.step(slots, [q[:n] for q, n in zip(seqs, lens)]).double().cpu().numpy()
+    for i, n in enumerate(lens):
+        assert np.abs(got[i] - truth[i][n - 1]).max() <= tolerance(dtype, truth[i]), ("prompt", i)
+    for j in range(n_dec):
+        got = s.step(slots, [[q[n + j]] for q, n in zip(seqs, lens)]).double().cpu().numpy()
+        for i, n in enumerate(lens):
+            err = np.abs(got[i] - truth[i][n + j]).max()
+            assert err <= tolerance(dtype, truth[i]), (which, dtype, "step", j, "sequence", i, err)
+    s.release(slots)
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])

@@ -44,8 +44,20 @@ TINY_D = dict(
     eos_token_id=1, rope_style="half")
 TINY_D_WEIGHTS = dict(seed=3, std=0.04, norm_sigma=0.3)
 
+# a fifth with the head size and grouping of the large checkpoints (128, four query heads a KV
+# head) and a width of 1024: the kernels at the sizes they have there, and the norm that decode
+# batches of 17 to 64 rows split between the products around it
+TINY_E = dict(
+    architectures=["LlamaForCausalLM"], hidden_size=1024, intermediate_size=1536, num_attention_heads=8,
+    num_key_value_heads=2, num_hidden_layers=2, vocab_size=1031, head_dim=128, rms_norm_eps=1e-5,
+    rope_theta=500000.0,
+    rope_scaling=dict(rope_type="llama3", factor=8.0, low_freq_factor=1.0, high_freq_factor=4.0,
+                      original_max_position_embeddings=128),
+    tie_word_embeddings=False, max_position_embeddings=1024, eos_token_id=2, rope_style="half")
+TINY_E_WEIGHTS = dict(seed=4, std=0.03, norm_sigma=0.2)
+
 CONFIGS = {"A": (TINY_A, TINY_A_WEIGHTS), "B": (TINY_B, TINY_B_WEIGHTS), "C": (TINY_C, TINY_C_WEIGHTS),
-           "D": (TINY_D, TINY_D_WEIGHTS)}
+           "D": (TINY_D, TINY_D_WEIGHTS), "E": (TINY_E, TINY_E_WEIGHTS)}
 
 
 def make_model_dir(tmp_path, which: str, dtype: str = "bfloat16") -> str:
