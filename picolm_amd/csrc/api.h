@@ -54,6 +54,9 @@ int picolm_gemm_tiled_splitk(const void* A, const void* W, void* C, int c_dt, in
 // role), 7, or tiled != 0 with tile variant 12/13 (taking only).  17 to 64 rows (rows = 64): tiled,
 // variant 12; cut along K (splits > 1, ws of splits * M * N floats, N a multiple of 1024) either
 // role, uncut taking only.
+// More than 64 rows (rows = a multiple of 64 of at least M, sums for every row): the tiled product
+// by shape, either role; picolm_gemm_tiled_norm_parts gives the shares it leaves (0: it cannot).
+int picolm_gemm_tiled_norm_parts(int M, int N, int K);
 int picolm_gemm_linked(const void* A, const void* W, void* C, int c_dt, int M, int N, int K, int64_t lda,
                        int64_t ldw, int64_t ldc, int epilogue, int tiled, int variant, int splits, float* ws,
                        const float* next_w, void* next_h, float* next_ssq, int next_parts, const float* ssq,

@@ -15,6 +15,7 @@
 //
 // The order of the K summation inside an MFMA does not matter, so a lane's 8-element chunk
 // may come from any K offset as long as both operands use the same offset.
+#include <type_traits>
 #include "common.h"
 #include "api.h"
 
@@ -50,17 +51,18 @@ struct NormLink {
     int rows;               // 16 (products of up to 16 rows) or 64: rows that the sums are kept for
 };
 
-// Consumer side.  `begin` has every thread ask for its share of the partial sums (row tid % rows,
-// every (THREADS/rows)-th part) before the main loop; `finish` adds them up in a fixed order and
-// leaves the row factors in LDS.  Both are called by all THREADS threads of the workgroup.
+// Consumer side.  `begin` has every thread ask for its share of the partial sums (row
+// m0 + tid % tile_rows, every (THREADS/tile_rows)-th part) before the main loop; `finish` adds
+// them up in a fixed order and leaves the factors of the tile's rows in LDS.  Both are called by
+// all THREADS threads of the workgroup; tile_rows is a power of two of at most THREADS.
 template <int THREADS>
-__device__ __forceinline__ float row_scale_begin(const NormLink& k, int M) {
+__device__ __forceinline__ float row_scale_begin(const NormLink& k, int M, int m0, int tile_rows) {
     float mine = 0.f;
     if (k.ssq) {
-        const int m = threadIdx.x % k.rows, stride = THREADS / k.rows;
+        const int m = m0 + threadIdx.x % tile_rows, stride = THREADS / tile_rows;
         if (m < M) {
             // eight loads are asked for before the first is added: one trip to memory, not eight
-            for (int p0 = threadIdx.x / k.rows; p0 < k.n_parts; p0 += 8 * stride) {
+            for (int p0 = threadIdx.x / tile_rows; p0 < k.n_parts; p0 += 8 * stride) {
                 float v[8];
 #pragma unroll
                 for (int i = 0; i < 8; ++i) v[i] = k.ssq[(size_t)min(p0 + i * stride, k.n_parts - 1) * k.rows + m];
@@ -71,20 +73,15 @@ __device__ __forceinline__ float row_scale_begin(const NormLink& k, int M) {
     }
     return mine;
 }
-template <int THREADS>
-__device__ __forceinline__ void row_scale_finish(const NormLink& k, float mine, float (&scratch)[THREADS / 64][64],
-                                                 float (&scale)[64]) {
+template <int THREADS, int SCALES>
+__device__ __forceinline__ void row_scale_finish(const NormLink& k, float mine, int tile_rows, float (&scratch)[THREADS],
+                                                 float (&scale)[SCALES]) {
     if (!k.ssq) return;          // uniform over the workgroup
-    if (k.rows == 16) {          // four lanes of a wave share a row
-        mine += __shfl_xor(mine, 16, WAVE);
-        mine += __shfl_xor(mine, 32, WAVE);
-    }
-    if ((int)(threadIdx.x % 64) < k.rows) scratch[threadIdx.x / 64][threadIdx.x % 64] = mine;
+    scratch[threadIdx.x] = mine;             // [share][row of the tile]
     __syncthreads();
-    if ((int)threadIdx.x < k.rows) {
+    if ((int)threadIdx.x < tile_rows) {
         float total = 0.f;
-#pragma unroll
-        for (int w = 0; w < THREADS / 64; ++w) total += scratch[w][threadIdx.x];
+        for (int g = 0; g < THREADS / tile_rows; ++g) total += scratch[g * tile_rows + threadIdx.x];
         scale[threadIdx.x] = 1.0f / sqrtf(total * k.inv_len + k.eps);
     }
     __syncthreads();
@@ -101,8 +98,8 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const bf16_t* _
                                                                  TC* __restrict__ C, int M, int N, int K,
                                                                  int64_t lda, int64_t ldw, int64_t ldc, NormLink link) {
     extern __shared__ float red[];      // [WAVES][NT][MT][4][64]
-    __shared__ float link_scratch[WAVES][64], link_scale[64];
-    const float link_mine = row_scale_begin<WAVES * 64>(link, M);
+    __shared__ float link_scratch[WAVES * 64], link_scale[16];
+    const float link_mine = row_scale_begin<WAVES * 64>(link, M, 0, 16);
     const int wave = threadIdx.x / 64, lane = threadIdx.x % 64;
     const int r16 = lane % 16, q = lane / 16;
     const int n_base = blockIdx.x * (16 * NT);
@@ -184,7 +181,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const bf16_t* _
 #pragma unroll
             for (int r = 0; r < 4; ++r) red[(((wave * NT + t) * MT + u) * 4 + r) * 64 + lane] = acc[t][u][r];
     __syncthreads();
-    row_scale_finish<WAVES * 64>(link, link_mine, link_scratch, link_scale);
+    row_scale_finish<WAVES * 64>(link, link_mine, 16, link_scratch, link_scale);
     constexpr int PER_WAVE = NT * MT * 4 * 64;
     constexpr int STEP = (EPI == 2) ? 2 : 1;
     float next_sq = 0.f;                // producer side: x^2 of the value this thread finishes (MT = NT = 1 only)
@@ -235,11 +232,11 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const bf16_t* _
         next_sq += __shfl_xor(next_sq, 16, WAVE);
         next_sq += __shfl_xor(next_sq, 32, WAVE);
         __syncthreads();                    // link_scratch may still be read as the consumer's
-        if (wave < 4 && lane < 16) link_scratch[wave][lane] = next_sq;
+        if (wave < 4 && lane < 16) link_scratch[wave * 16 + lane] = next_sq;
         __syncthreads();
         if (threadIdx.x < 16)
             link.next_ssq[(size_t)blockIdx.x * link.rows + threadIdx.x] =
-                link_scratch[0][threadIdx.x] + link_scratch[1][threadIdx.x] + link_scratch[2][threadIdx.x] + link_scratch[3][threadIdx.x];
+                link_scratch[threadIdx.x] + link_scratch[16 + threadIdx.x] + link_scratch[32 + threadIdx.x] + link_scratch[48 + threadIdx.x];
     }
 }
 
@@ -290,8 +287,8 @@ __global__ __launch_bounds__(512) void gemm_skinny_resident_kernel(const bf16_t*
                                                                    int64_t lda, int64_t ldw, int64_t ldc, NormLink link) {
     constexpr int WAVES = 8;
     __shared__ float red[2][WAVES][4][64];
-    __shared__ float link_scratch[WAVES][64], link_scale[64];
-    const float link_mine = row_scale_begin<WAVES * 64>(link, M);
+    __shared__ float link_scratch[WAVES * 64], link_scale[16];
+    const float link_mine = row_scale_begin<WAVES * 64>(link, M, 0, 16);
     const int wave = threadIdx.x / 64, lane = threadIdx.x % 64;
     const int r16 = lane % 16, q = lane / 16;
     const int n_full = K / SK_KSTEP;            // K is a whole number of steps (the host sees to that)
@@ -358,7 +355,7 @@ __global__ __launch_bounds__(512) void gemm_skinny_resident_kernel(const bf16_t*
     const int stride = gridDim.x;
     int tile = blockIdx.x;
     fetch(w0, min(tile, n_tiles - 1));
-    row_scale_finish<WAVES * 64>(link, link_mine, link_scratch, link_scale);
+    row_scale_finish<WAVES * 64>(link, link_mine, 16, link_scratch, link_scale);
     while (tile < n_tiles) {
         fetch(w1, min(tile + stride, n_tiles - 1));
         __builtin_amdgcn_sched_barrier(0);      // the next tile is asked for before this one is waited for
@@ -686,6 +683,13 @@ template <int BK>
 __device__ __forceinline__ int swizzled_chunk(int row, int chunk) {
     return BK == 32 ? chunk ^ ((row >> 2) & 3) : chunk ^ ((row >> 1) & 7);
 }
+// A pointer that is the same in every lane, said so that it lies in scalar registers whatever
+// the compiler made of the arithmetic that led to it.
+__device__ __forceinline__ const void* same_in_every_lane(const void* p) {
+    const uint64_t v = (uint64_t)p;
+    const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v), hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
+    return (const void*)(((uint64_t)hi << 32) | lo);
+}
 __device__ __forceinline__ void load_16_bytes_to_lds(unsigned byte_offset, const void* base, unsigned lds_address) {
     asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dwordx4 %0, %1"
                  :
@@ -705,8 +709,10 @@ __global__ __launch_bounds__(64 * WN * WM) void gemm_direct_kernel(const bf16_t*
                                                                    int64_t lda, int64_t ldw, int64_t ldc,
                                                                    int tiles_m, int tiles_n, int64_t c_split_stride,
                                                                    NormLink link) {
-    __shared__ float link_scratch[WN * WM][64], link_scale[64];
-    const float link_mine = row_scale_begin<64 * WN * WM>(link, M);
+    // the rows of the tile that a split norm keeps factors for: the sums' own 16 or 64 in a decode
+    // step (one row of tiles), else all of the tile's
+    __shared__ float link_scratch[64 * WN * WM], link_scale[32 * TM * WM > 64 ? 32 * TM * WM : 64];
+    __shared__ float next_sums[EPI == 1 ? WN * 32 * TM * WM : 1];
     // K here is the length of one split: workgroup row y of the grid takes columns y*K .. of A
     // and W and writes its sums to C + y * c_split_stride
     A += (int64_t)blockIdx.y * K;
@@ -732,6 +738,8 @@ __global__ __launch_bounds__(64 * WN * WM) void gemm_direct_kernel(const bf16_t*
     const int band_w = min(band, tiles_n - b * band);
     const int tn = b * band + in_b % band_w, tm = in_b / band_w;
     const int n0 = tn * BN, m0 = tm * BM;
+    const int link_rows = link.rows <= 64 ? link.rows : BM;
+    const float link_mine = row_scale_begin<64 * WN * WM>(link, M, m0, link_rows);
 
     const int tid = threadIdx.x, wave = tid / 64, lane = tid % 64;
     const int wn = (wave % WN) * (32 * TN), wm = (wave / WN) * (32 * TM);
@@ -767,8 +775,8 @@ __global__ __launch_bounds__(64 * WN * WM) void gemm_direct_kernel(const bf16_t*
         const unsigned to = lds_wave + stage * (STAGE * 2);
         step += first_step;
         if (step >= n_steps) step -= n_steps;
-        const bf16_t* wsrc = w_tile + step * BK;
-        const bf16_t* asrc = a_tile + step * BK;
+        const void* wsrc = same_in_every_lane(w_tile + step * BK);
+        const void* asrc = same_in_every_lane(a_tile + step * BK);
 #pragma unroll
         for (int j = 0; j < W_LOADS; ++j) load_16_bytes_to_lds(w_off[j], wsrc, to + j * (NW * RG * BK * 2));
 #pragma unroll
@@ -855,25 +863,113 @@ __global__ __launch_bounds__(64 * WN * WM) void gemm_direct_kernel(const bf16_t*
         stage = next_stage;
     }
     wait_for_loads<0>();
-    row_scale_finish<64 * WN * WM>(link, link_mine, link_scratch, link_scale);
+    row_scale_finish<64 * WN * WM>(link, link_mine, link_rows, link_scratch, link_scale);
+    // A product that adds into the residual rows can prepare the norm that follows (NormLink):
+    // next_h = bf16(x * w) beside the new rows, and the tile's share of every row's sum of x^2.
+    const bool prepares = EPI == 1 && link.next_w != nullptr;
+    // The tile goes out in one of two ways: a tile that lies wholly inside C (most do) without a
+    // test per element, a tile on the edge with them.  FULL is a type that says which.
+    auto write_tile = [&](auto FULL) __attribute__((always_inline)) {
+        constexpr bool full = decltype(FULL)::value;
+        // element (i, j, e) of a lane is row r0 + 32j + 8(e/4) + e%4, column c0 + 32i of the tile
+        const int r0 = wm + 4 * kq, c0 = wn + l32;
+        TC* corner = C + (int64_t)m0 * ldc + (EPI == 2 ? n0 / 2 : n0);       // (n0 is even)
+        bf16_t* hcorner = prepares ? link.next_h + (int64_t)m0 * ldc + n0 : nullptr;
+        const unsigned ld = (unsigned)ldc;       // offsets within a tile fit 32 bits (the host sees to that)
+        float next_w[TN];
 #pragma unroll
-    for (int i = 0; i < TN; ++i) {
-        const int n = n0 + wn + 32 * i + l32;
+        for (int i = 0; i < TN; ++i) next_w[i] = prepares && (full || n0 + c0 + 32 * i < N) ? link.next_w[n0 + c0 + 32 * i] : 0.f;
 #pragma unroll
         for (int j = 0; j < TM; ++j) {
+            // what this product adds to: 32 rows' values are all asked for before the first is used
+            float before[EPI == 1 ? TN : 1][16];
+            if (EPI == 1) {
 #pragma unroll
-            for (int e = 0; e < 16; ++e) {
-                const int m = m0 + wm + 32 * j + 8 * (e / 4) + 4 * kq + e % 4;
-                float v = acc[i][j][e];
-                if (link.ssq && m < link.rows) v *= link_scale[m];     // (one row of tiles: the host sees to that)
-                if (EPI == 2) {
-                    const float up = __shfl_xor(v, 1, WAVE);
-                    if (m < M && (l32 & 1) == 0 && n + 1 < N) C[(int64_t)m * ldc + n / 2] = from_f32<TC>(silu_mul(v, up));
-                } else if (m < M && n < N) {
-                    TC* p = C + (int64_t)m * ldc + n;
-                    *p = from_f32<TC>(EPI == 1 ? to_f32<TC>(*p) + v : v);
+                for (int i = 0; i < TN; ++i)
+#pragma unroll
+                    for (int e = 0; e < 16; ++e) {
+                        const int r = r0 + 32 * j + 8 * (e / 4) + e % 4, c = c0 + 32 * i;
+                        const bool in = full || (m0 + r < M && n0 + c < N);
+                        before[i][e] = in ? to_f32<TC>(corner[(unsigned)r * ld + c]) : 0.f;
+                    }
+            }
+            float sq[16];               // this lane's share of 16 rows' sums of x^2
+#pragma unroll
+            for (int e = 0; e < 16; ++e) sq[e] = 0.f;
+#pragma unroll
+            for (int i = 0; i < TN; ++i) {
+                const int c = c0 + 32 * i;
+                const bool c_in = full || n0 + c < N;
+                unsigned hv[16];            // bf16(x * w) of this lane's 16 rows
+#pragma unroll
+                for (int e = 0; e < 16; ++e) {
+                    const int r = r0 + 32 * j + 8 * (e / 4) + e % 4;
+                    const bool r_in = full || m0 + r < M;
+                    float v = acc[i][j][e];
+                    if (link.ssq && r_in) v *= link_scale[r];
+                    hv[e] = 0;
+                    if (EPI == 2) {
+                        const float up = __shfl_xor(v, 1, WAVE);
+                        if (r_in && (l32 & 1) == 0 && (full || n0 + c + 1 < N))
+                            corner[(unsigned)r * ld + c / 2] = from_f32<TC>(silu_mul(v, up));
+                    } else if (r_in && c_in) {
+                        const float x = EPI == 1 ? before[EPI == 1 ? i : 0][e] + v : v;
+                        corner[(unsigned)r * ld + c] = from_f32<TC>(x);
+                        if (prepares) {
+                            hv[e] = f32_to_bf16_bits(x * next_w[i]);
+                            sq[e] += x * x;
+                        }
+                    }
+                }
+                if (prepares) {
+                    // Two lanes side by side hold two adjacent columns of 16 rows each: they swap
+                    // half of them, so that each writes two columns of 8 rows, four bytes a store
+                    // (N and the row stride are even: the host sees to that).
+                    const int odd = l32 & 1;
+#pragma unroll
+                    for (int e = 0; e < 16; e += 2) {
+                        const unsigned send = odd ? hv[e] : hv[e + 1];
+                        const unsigned recv = (unsigned)__shfl_xor((int)send, 1, WAVE);
+                        const int ee = e + odd;                 // the row this lane writes
+                        const int r = r0 + 32 * j + 8 * (ee / 4) + ee % 4;
+                        const unsigned lo = odd ? recv : hv[e], hi = odd ? hv[e + 1] : recv;
+                        if (full || (m0 + r < M && n0 + c - odd + 1 < N))
+                            *(unsigned*)(hcorner + (unsigned)r * ld + (c - odd)) = (lo & 0xffffu) | (hi << 16);
+                    }
                 }
             }
+            if (prepares) {
+                // The 16 rows' sums over the wave's columns, that is over the 32 lanes that hold
+                // them.  Lanes that differ in one bit swap half of what they still hold and add,
+                // four times: then a lane holds one row, the one its low four bits spell, summed
+                // over 16 lanes; the lane 16 further on holds the rest of it.
+#pragma unroll
+                for (int half = 8; half >= 1; half /= 2) {
+                    const int bit = 8 / half;               // 1, 2, 4, 8
+                    const bool upper = (l32 & bit) != 0;    // this lane keeps the upper half
+#pragma unroll
+                    for (int k = 0; k < half; ++k) {
+                        const float recv = __shfl_xor(upper ? sq[k] : sq[k + half], bit, WAVE);
+                        sq[k] = (upper ? sq[k + half] : sq[k]) + recv;
+                    }
+                }
+                const float t = sq[0] + __shfl_xor(sq[0], 16, WAVE);
+                const int e = 8 * (l32 & 1) + 4 * ((l32 >> 1) & 1) + 2 * ((l32 >> 2) & 1) + ((l32 >> 3) & 1);
+                if (l32 < 16) next_sums[(wave % WN) * BM + r0 + 32 * j + 8 * (e / 4) + e % 4] = t;
+            }
+
+        }
+    };
+    if (m0 + BM <= M && n0 + BN <= N) write_tile(std::true_type{});
+    else write_tile(std::false_type{});
+    if (EPI == 1 && prepares) {       // (uniform over the workgroup)
+        // ... then over the waves side by side, in a fixed order
+        __syncthreads();
+        for (int r = tid; r < BM; r += 64 * WN * WM) {
+            float t = 0.f;
+#pragma unroll
+            for (int w = 0; w < WN; ++w) t += next_sums[w * BM + r];
+            if (m0 + r < M) link.next_ssq[(size_t)tn * link.rows + m0 + r] = t;
         }
     }
 }
@@ -882,10 +978,17 @@ template <int TN, int TM, int WN, int WM, int BK, int NS>
 static int launch_direct(const void* A, const void* W, void* C, int c_dt, int M, int N, int K, int64_t lda,
                          int64_t ldw, int64_t ldc, int epilogue, hipStream_t stream, int splits = 1,
                          int64_t c_split_stride = 0, NormLink link = NormLink{}) {
-    PICOLM_REQUIRE(!link.next_w, "gemm_tiled: the tiled kernels prepare no norm");
     constexpr int BN = 32 * TN * WN, BM = 32 * TM * WM;
-    PICOLM_REQUIRE(!link.ssq || (M <= link.rows && M <= BM && splits == 1 && (link.rows == 16 || link.rows == 64)),
-                   "gemm_tiled: a norm's statistics are taken for one row of tiles of an uncut product");
+    // sums kept for 16 or 64 rows belong to a decode step, which has one row of tiles; otherwise
+    // they are kept for every row
+    PICOLM_REQUIRE((!link.ssq && !link.next_w) ||
+                       (splits == 1 && M <= link.rows && (link.rows > 64 || ((link.rows == 16 || link.rows == 64) && M <= BM))),
+                   "gemm_tiled: a split norm goes with an uncut product and sums for every row (%d rows, sums for %d)", M, link.rows);
+    PICOLM_REQUIRE((int64_t)BM * ldc < (1ll << 29), "gemm_tiled: a row stride of %lld overflows the tile's 32-bit offsets", (long long)ldc);
+    PICOLM_REQUIRE(!link.next_w || (N % 2 == 0 && ldc % 2 == 0 && ((uintptr_t)link.next_h & 3) == 0),
+                   "gemm_tiled: preparing a norm writes pairs of columns: N and the row stride must be even");
+    PICOLM_REQUIRE(!link.next_w || (epilogue == 1 && link.next_parts >= ceil_div(N, BN)),
+                   "gemm_tiled: only the accumulating epilogue prepares a norm, one share of the sums per column of tiles");
     PICOLM_REQUIRE(splits >= 1 && K % (BK * splits) == 0,
                    "gemm_tiled: K = %d is no multiple of %d times %d splits, which this variant needs", K, BK, splits);
     PICOLM_REQUIRE((int64_t)BN * ldw < (1ll << 30) && (int64_t)BM * lda < (1ll << 30),
@@ -1004,43 +1107,75 @@ static int launch_splitk_reduce(const float* ws, void* C, int c_dt, int M, int N
 //   batches of up to 64 or 32 rows, where the weights stream once and K may be split.
 // Tiles staged through registers (any K that is a multiple of 8):
 //   1: 128x128 (4 waves), 4: 256x256 (8 waves).
+// The tile variant for a product by its shape.  Every variant moves about the same bytes a second
+// from L2 into LDS, so the largest tile wins once its workgroups fill most of the 256 CUs.
+// n_first > 0: the first n_first columns of 256x256 tiles go to variant 9 and the rest to variant
+// 10: a last round that fills half of the CUs or less costs nearly a whole round, and the 256x128
+// tile gives those columns twice the workgroups.
+static int tiled_plan(int M, int N, int K, int& n_first) {
+    n_first = 0;
+    const int tiles_m = ceil_div(M, 256), tiles_n = ceil_div(N, 256);
+    const int64_t t256 = (int64_t)tiles_m * tiles_n;
+    const int64_t t128m = (int64_t)ceil_div(M, 128) * tiles_n;
+    if (K % 64 != 0) return t256 >= 512 ? 4 : 1;
+    const int64_t whole = t256 / 256 * 256, left = t256 - whole;
+    const int first = (int)(whole / tiles_m);
+    const int64_t rest = (int64_t)(tiles_n - first) * ceil_div(M, 128);
+    if (whole > 0 && left > 0 && left <= 160 && first > 0 && rest <= 288) {
+        n_first = first;
+        return 9;
+    }
+    return t256 >= 192 ? 9 : t128m >= 192 ? 10 : 11;
+}
+
+// Shares of a row's sum of squares that the tiled product of this shape leaves when it prepares a
+// norm (one per column of tiles), or 0 if its kernel cannot take part in a split norm.
+extern "C" int picolm_gemm_tiled_norm_parts(int M, int N, int K) {
+    int n_first;
+    const int variant = tiled_plan(M, N, K, n_first);
+    return variant == 9 || variant == 10 ? ceil_div(N, 256) : variant == 11 ? ceil_div(N, 128) : 0;
+}
+
+static int gemm_tiled_linked(const void* A, const void* W, void* C, int c_dt, int M, int N, int K, int64_t lda,
+                             int64_t ldw, int64_t ldc, int epilogue, int variant, hipStream_t stream, NormLink link);
+
 extern "C" int picolm_gemm_tiled(const void* A, const void* W, void* C, int c_dt, int M, int N, int K,
                                  int64_t lda, int64_t ldw, int64_t ldc, int epilogue, int variant,
                                  hipStream_t stream) {
     if (check_mfma_operands("gemm_tiled", A, W, M, N, K, lda, ldw, ldc, epilogue, c_dt)) return -1;
     if (M == 0) return 0;
+    return gemm_tiled_linked(A, W, C, c_dt, M, N, K, lda, ldw, ldc, epilogue, variant, stream, NormLink{});
+}
+
+static int gemm_tiled_linked(const void* A, const void* W, void* C, int c_dt, int M, int N, int K, int64_t lda,
+                             int64_t ldw, int64_t ldc, int epilogue, int variant, hipStream_t stream, NormLink link) {
     if (variant == 0) {
-        // Every variant moves about the same bytes a second from L2 into LDS, so the largest
-        // tile wins once its workgroups fill most of the 256 CUs.
-        const int tiles_m = ceil_div(M, 256), tiles_n = ceil_div(N, 256);
-        const int64_t t256 = (int64_t)tiles_m * tiles_n;
-        const int64_t t128m = (int64_t)ceil_div(M, 128) * tiles_n;
-        if (K % 64 == 0) {
-            // A last round that fills half of the CUs or less costs nearly a whole round: those
-            // columns of tiles go to the 256x128 tile instead, which gives them twice the workgroups.
-            const int64_t whole = t256 / 256 * 256, left = t256 - whole;
-            const int n_first = (int)(whole / tiles_m);
-            const int64_t rest = (int64_t)(tiles_n - n_first) * ceil_div(M, 128);
-            if (whole > 0 && left > 0 && left <= 160 && n_first > 0 && rest <= 288) {
-                const int N1 = n_first * 256;
-                const size_t c_item = c_dt == PICOLM_F32 ? 4 : 2;
-                const int rc = picolm_gemm_tiled(A, W, C, c_dt, M, N1, K, lda, ldw, ldc, epilogue, 9, stream);
-                if (rc) return rc;
-                return picolm_gemm_tiled(A, (const bf16_t*)W + (int64_t)N1 * ldw,
-                                         (char*)C + c_item * (epilogue == 2 ? N1 / 2 : N1), c_dt, M, N - N1, K, lda,
-                                         ldw, ldc, epilogue, 10, stream);
+        int n_first;
+        variant = tiled_plan(M, N, K, n_first);
+        if (n_first > 0) {
+            const int N1 = n_first * 256;
+            const size_t c_item = c_dt == PICOLM_F32 ? 4 : 2;
+            const int rc = gemm_tiled_linked(A, W, C, c_dt, M, N1, K, lda, ldw, ldc, epilogue, 9, stream, link);
+            if (rc) return rc;
+            if (link.next_w) {          // the second launch goes on where the first one's columns end
+                link.next_w += N1;
+                link.next_h += N1;
+                link.next_ssq += (size_t)n_first * link.rows;
+                link.next_parts -= n_first;
             }
-            variant = t256 >= 192 ? 9 : t128m >= 192 ? 10 : 11;
-        } else {
-            variant = t256 >= 512 ? 4 : 1;
+            return gemm_tiled_linked(A, (const bf16_t*)W + (int64_t)N1 * ldw,
+                                     (char*)C + c_item * (epilogue == 2 ? N1 / 2 : N1), c_dt, M, N - N1, K, lda, ldw,
+                                     ldc, epilogue, 10, stream, link);
         }
     }
+    if (link.ssq || link.next_w)
+        PICOLM_REQUIRE(variant >= 9 && variant <= 11, "gemm_tiled: tile variant %d takes no part in a split norm", variant);
     switch (variant) {
         case 1: return launch_tiled<2, 2, 2, 2, 2>(A, W, C, c_dt, M, N, K, lda, ldw, ldc, epilogue, stream);
         case 4: return launch_tiled<2, 4, 4, 2, 1>(A, W, C, c_dt, M, N, K, lda, ldw, ldc, epilogue, stream);
-        case 9: return launch_direct<2, 4, 4, 2, 64, 2>(A, W, C, c_dt, M, N, K, lda, ldw, ldc, epilogue, stream);
-        case 10: return launch_direct<2, 2, 4, 2, 64, 3>(A, W, C, c_dt, M, N, K, lda, ldw, ldc, epilogue, stream);
-        case 11: return launch_direct<2, 2, 2, 2, 64, 4>(A, W, C, c_dt, M, N, K, lda, ldw, ldc, epilogue, stream);
+        case 9: return launch_direct<2, 4, 4, 2, 64, 2>(A, W, C, c_dt, M, N, K, lda, ldw, ldc, epilogue, stream, 1, 0, link);
+        case 10: return launch_direct<2, 2, 4, 2, 64, 3>(A, W, C, c_dt, M, N, K, lda, ldw, ldc, epilogue, stream, 1, 0, link);
+        case 11: return launch_direct<2, 2, 2, 2, 64, 4>(A, W, C, c_dt, M, N, K, lda, ldw, ldc, epilogue, stream, 1, 0, link);
         case 12: return launch_direct<1, 2, 4, 1, 64, 3>(A, W, C, c_dt, M, N, K, lda, ldw, ldc, epilogue, stream);
         case 13: return launch_direct<1, 1, 4, 1, 64, 4>(A, W, C, c_dt, M, N, K, lda, ldw, ldc, epilogue, stream);
     }
@@ -1074,6 +1209,9 @@ extern "C" int picolm_gemm_tiled_splitk(const void* A, const void* W, void* C, i
 
 // The products of a decode step with a norm split between them (see NormLink).  Up to 16 rows:
 // `variant` as in picolm_gemm_skinny (0, 1, 7) or, with tiled != 0, tile variant 12 or 13; rows = 16.
+// More than 64 rows (a prefill step): tiled, rows = a multiple of 64 of at least M, the tile
+// variant by shape; either role, one share of the sums per column of tiles
+// (picolm_gemm_tiled_norm_parts).
 // 17 to 64 rows: tiled, variant 12, rows = 64; with splits > 1 (ws as in picolm_gemm_tiled_splitk)
 // the kernel that adds the parts takes either role and N must be a multiple of 1024; uncut, the
 // tile kernel can only take a prepared norm's statistics.
@@ -1087,12 +1225,17 @@ extern "C" int picolm_gemm_linked(const void* A, const void* W, void* C, int c_d
                                   const float* ssq, int n_parts, int norm_len, float eps, int rows,
                                   hipStream_t stream) {
     if (check_mfma_operands("gemm_linked", A, W, M, N, K, lda, ldw, ldc, epilogue, c_dt)) return -1;
-    PICOLM_REQUIRE((rows == 16 || rows == 64) && M <= rows, "gemm_linked: %d rows with sums kept for %d", M, rows);
+    PICOLM_REQUIRE((rows == 16 || rows == 64 || (rows > 64 && rows % 64 == 0)) && M <= rows,
+                   "gemm_linked: %d rows with sums kept for %d", M, rows);
     PICOLM_REQUIRE(!next_w || (next_h && next_ssq && next_parts > 0), "gemm_linked: an incomplete description of the next norm");
     PICOLM_REQUIRE(!ssq || (n_parts > 0 && norm_len > 0), "gemm_linked: an incomplete description of the norm's statistics");
     PICOLM_REQUIRE(splits >= 1 && splits <= 64, "gemm_linked: %d splits", splits);
     if (M == 0) return 0;
     NormLink link = {next_w, (bf16_t*)next_h, next_ssq, next_parts, ssq, n_parts, norm_len > 0 ? 1.0f / (float)norm_len : 0.f, eps, rows};
+    if (rows > 64) {            // a prefill step: the tile variants by shape, sums for every row
+        PICOLM_REQUIRE(tiled && splits == 1, "gemm_linked: more than 64 rows take the uncut tiled product");
+        return gemm_tiled_linked(A, W, C, c_dt, M, N, K, lda, ldw, ldc, epilogue, 0, stream, link);
+    }
     if (tiled && splits > 1) {
         PICOLM_REQUIRE(variant == 12 && ws != nullptr && ((uintptr_t)ws & 15) == 0 && N % 4 == 0,
                        "gemm_linked: a cut product needs tile variant 12, a workspace and N in multiples of 4");

@@ -42,7 +42,7 @@ def dir_entry_points():
     return ["picolm_abi_version", "picolm_device_check", "picolm_embed", "picolm_rmsnorm",
             "picolm_rope_kv_store", "picolm_silu_mul", "picolm_add_into", "picolm_gemm_generic",
             "picolm_attn_prefill_tile_rows", "picolm_attn_prefill_generic",
-            "picolm_attn_decode_generic", "picolm_argmax", "picolm_argmax_scratch_floats", "picolm_sample", "picolm_sample_scratch_bytes", "picolm_gemm_skinny", "picolm_gemm_tiled", "picolm_gemm_tiled_splitk", "picolm_gemm_linked", "picolm_kv_page_order",
+            "picolm_attn_decode_generic", "picolm_argmax", "picolm_argmax_scratch_floats", "picolm_sample", "picolm_sample_scratch_bytes", "picolm_gemm_skinny", "picolm_gemm_tiled", "picolm_gemm_tiled_splitk", "picolm_gemm_linked", "picolm_gemm_tiled_norm_parts", "picolm_kv_page_order",
             "picolm_attn_mfma_takes", "picolm_attn_prefill_mfma_heads", "picolm_attn_prefill_mfma_tile_tokens",
             "picolm_attn_prefill_mfma", "picolm_attn_decode_mfma", "picolm_attn_decode_rope_mfma", "picolm_attn_decode_mfma_waves", "picolm_read_probe", "picolm_mfma_probe"]
 
@@ -378,18 +378,24 @@ def medium_gemm_splits(M: int, N: int, K: int) -> int:
     return s
 
 
-LINKED_NORM_MAX_M = 64
+LINKED_NORM_MAX_M = 1 << 30      # (a switch for measurements: rows above it take the norm's own kernel)
 
 
 def linked_norm_rows(M: int) -> int:
-    """Rows that the partial sums of a split norm are kept for in a step of M rows."""
-    return 16 if M <= 16 else 64
+    """Rows that the partial sums of a split norm are kept for in a step of M rows: 16 or 64 in
+    a decode step, every row (in whole 64s) otherwise."""
+    return 16 if M <= 16 else 64 if M <= 64 else (M + 63) // 64 * 64
 
 
-def linked_norm_parts(M: int, N: int) -> int:
-    """Partial sums per row that a product of M rows and N output columns leaves for the norm
-    that follows: one per workgroup of the kernel that finishes the rows."""
-    return (N + 15) // 16 if M <= 16 else N // 1024
+def linked_norm_parts(M: int, N: int, K: int) -> int:
+    """Partial sums per row that a product of M rows, N output columns and K input columns leaves
+    for the norm that follows: one per workgroup (or column of tiles) of the kernel that finishes
+    the rows.  0: that kernel cannot."""
+    if M <= 16:
+        return (N + 15) // 16
+    if M <= 64:
+        return N // 1024
+    return lib().picolm_gemm_tiled_norm_parts(M, N, K)
 
 
 def gemm_links_norms(a, w, c, epilogue: int, prepares: bool) -> bool:
@@ -397,7 +403,8 @@ def gemm_links_norms(a, w, c, epilogue: int, prepares: bool) -> bool:
     prepare the next one (with the accumulating epilogue), or else take a prepared one's
     statistics.  Up to 16 rows every matrix-core product can do both.  For 17 to 64 rows the
     kernel that adds the parts of a product cut along K does either for N in multiples of 1024,
-    and the tile kernel of an uncut product can take the statistics."""
+    and the tile kernel of an uncut product can take the statistics.  Above that the tile kernels
+    whose tiles go straight into LDS (K in multiples of 64) do both."""
     if a.dim() != 2 or a.shape[0] > LINKED_NORM_MAX_M or not mfma_gemm_takes(a, w, c, epilogue):
         return False
     M, N, K = a.shape[0], w.shape[0], a.shape[1]
@@ -405,6 +412,8 @@ def gemm_links_norms(a, w, c, epilogue: int, prepares: bool) -> bool:
         return True
     if K % 64:
         return False
+    if M > 64:
+        return linked_norm_parts(M, N, K) > 0
     cut = medium_gemm_splits(M, N, K) > 1
     return (cut and N % 1024 == 0) if prepares else (not cut or N % 1024 == 0)
 
@@ -434,7 +443,7 @@ def gemm_linked(a, w, c, epilogue: int, prepare=None, prepared=None) -> None:
         _dev("gemm_linked.h_out", nh, torch.bfloat16, 2)
         _dev("gemm_linked.ssq_out", nssq, torch.float32, 2)
         next_parts = nssq.shape[0]
-        if nw.numel() != N or tuple(nh.shape) != (M, N) or nssq.shape[1] != rows or next_parts != linked_norm_parts(M, N):
+        if nw.numel() != N or tuple(nh.shape) != (M, N) or nssq.shape[1] != rows or next_parts != linked_norm_parts(M, N, K):
             raise KernelError("gemm_linked: the buffers for the next norm do not fit the product")
     if prepared is not None:
         ssq, norm_len, eps = prepared
@@ -443,7 +452,9 @@ def gemm_linked(a, w, c, epilogue: int, prepare=None, prepared=None) -> None:
         if ssq.shape[1] != rows or norm_len != K:
             raise KernelError("gemm_linked: the statistics are not those of this product's input rows")
     tiled, variant, splits, ws = 0, 0, 1, None
-    if M > 16:
+    if M > 64:
+        tiled = 1                       # the tile variant by shape, as in gemm()
+    elif M > 16:
         tiled, variant, splits = 1, 12, medium_gemm_splits(M, N, K)          # as in gemm()
         ws = splitk_workspace(a.device) if splits > 1 else None
     elif prepare is None and M > 4 and K % 64 == 0 and 16384 <= N <= 128 * 256:

@@ -72,7 +72,7 @@ class Linear(Part):
             T, N = out.shape
             which = ctx.ws.flip("norm.prepared")
             prepare = (nxt.rms_parameters()[0], ctx.ws.get(f"norm.prepared.h{which}", (T, N), torch.bfloat16),
-                       ctx.ws.get(f"norm.prepared.ssq{which}", (kernels.linked_norm_parts(T, N), kernels.linked_norm_rows(T)),
+                       ctx.ws.get(f"norm.prepared.ssq{which}", (kernels.linked_norm_parts(T, N, a.shape[1]), kernels.linked_norm_rows(T)),
                                   torch.float32))
         if prepare is None and prepared is None:
             kernels.gemm(a, self.weight, out, epilogue)

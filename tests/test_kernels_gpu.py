@@ -190,7 +190,7 @@ def test_gemm_with_a_norm_split_between_two_products(M, D):
     nw = 1.0 + 0.3 * torch.randn(D, generator=g)
     x = x0.clone().to(DEV)
     h = torch.full((M, D), float("nan"), dtype=torch.bfloat16, device=DEV)
-    ssq = torch.full((K().linked_norm_parts(M, D), 16), float("nan"), device=DEV)
+    ssq = torch.full((K().linked_norm_parts(M, D, K1), 16), float("nan"), device=DEV)
     K().gemm_linked(a1.to(DEV), w1.to(DEV), x, 1, prepare=(nw.to(DEV), h, ssq))
     x_ref = x0.double() + a1.double() @ w1.double().T
     assert (x.double().cpu() - x_ref).abs().max() <= tol(torch.float32, x_ref.abs().max().item()) + 1e-2 * 0
@@ -229,7 +229,7 @@ def test_gemm_with_a_norm_split_between_two_products_of_a_wide_decode_batch(M, D
     assert k.gemm_links_norms(a1.to(DEV), w1.to(DEV), x0.to(DEV), 1, prepares=True)
     x = x0.clone().to(DEV)
     h = torch.full((M, D), float("nan"), dtype=torch.bfloat16, device=DEV)
-    ssq = torch.full((k.linked_norm_parts(M, D), k.linked_norm_rows(M)), float("nan"), device=DEV)
+    ssq = torch.full((k.linked_norm_parts(M, D, K1), k.linked_norm_rows(M)), float("nan"), device=DEV)
     assert tuple(ssq.shape) == (D // 1024, 64)
     k.gemm_linked(a1.to(DEV), w1.to(DEV), x, 1, prepare=(nw.to(DEV), h, ssq))
     x_ref = x0.double() + a1.double() @ w1.double().T
@@ -257,6 +257,45 @@ def test_gemm_with_a_norm_split_between_two_products_of_a_wide_decode_batch(M, D
         k.gemm_linked(h, w3, c3, 0, prepared=(ssq, D, eps))
     assert not k.gemm_links_norms(h, torch.zeros(128 * 200, D, dtype=torch.bfloat16, device=DEV),
                                   torch.zeros(M, 128 * 200, device=DEV), 1, prepares=True)     # uncut: no preparing
+
+
+@pytest.mark.parametrize("M,D", [(65, 1024), (300, 1024), (2048, 1024), (65, 4352), (300, 4352), (2048, 10240)])
+def test_gemm_with_a_norm_split_between_two_products_of_a_prefill_step(M, D):
+    """More than 64 rows: the tile kernels keep sums for every row, one share per column of tiles;
+    10240 columns at 2048 rows are two launches with different tiles, which must meet without a seam."""
+    k = K()
+    g = torch.Generator().manual_seed(M * 31 + D)
+    eps, K1 = 1e-5, 256
+    x0 = torch.randn(M, D, generator=g) * (10.0 ** torch.arange(M).remainder(5).sub(2).float())[:, None]
+    a1 = torch.randn(M, K1, generator=g).to(torch.bfloat16)
+    w1 = (torch.randn(D, K1, generator=g) * 0.05).to(torch.bfloat16)
+    nw = 1.0 + 0.3 * torch.randn(D, generator=g)
+    x = x0.clone().to(DEV)
+    assert k.gemm_links_norms(a1.to(DEV), w1.to(DEV), x, 1, prepares=True)
+    h = torch.full((M, D), float("nan"), dtype=torch.bfloat16, device=DEV)
+    parts, rows = k.linked_norm_parts(M, D, K1), k.linked_norm_rows(M)
+    assert parts > 0 and rows >= M and rows % 64 == 0
+    ssq = torch.full((parts, rows), float("nan"), device=DEV)
+    k.gemm_linked(a1.to(DEV), w1.to(DEV), x, 1, prepare=(nw.to(DEV), h, ssq))
+    x_ref = x0.double() + a1.double() @ w1.double().T
+    assert (x.double().cpu() - x_ref).abs().max() <= tol(torch.float32, x_ref.abs().max().item())
+    assert torch.equal(h.cpu(), (x.cpu() * nw).to(torch.bfloat16))          # from the very values it stored
+    total = ssq[:, :M].double().sum(dim=0).cpu()
+    want = (x.double().cpu() ** 2).sum(dim=1)
+    assert ((total - want).abs() <= 1e-5 * want + 1e-30).all()
+    normed = x.double().cpu() / torch.sqrt((x.double().cpu() ** 2).mean(dim=1, keepdim=True) + eps) * nw.double()
+    for N2 in (384, 3072 + 6):
+        w2 = (torch.randn(N2, D, generator=g) * 0.1).to(torch.bfloat16)
+        for epi, cdt in ((0, torch.float32), (2, torch.bfloat16), (1, torch.float32)):
+            c = torch.randn(M, N2 // 2 if epi == 2 else N2, generator=g).to(cdt).to(DEV)
+            assert k.gemm_links_norms(h, w2.to(DEV), c, epi, prepares=False)
+            ref = gemm_ref(normed, w2, epi, c.clone())
+            k.gemm_linked(h, w2.to(DEV), c, epi, prepared=(ssq, D, eps))
+            err = (c.double().cpu() - ref).abs().max().item()
+            assert err <= tol(torch.bfloat16, ref.abs().max().item()), (M, D, N2, epi, err)
+    # K no multiple of 64: the older tiles, which take no part
+    assert not k.gemm_links_norms(torch.zeros(M, 72, dtype=torch.bfloat16, device=DEV),
+                                  torch.zeros(D, 72, dtype=torch.bfloat16, device=DEV), x, 1, prepares=True)
 
 
 def test_gemm_tiled_splits_a_partial_last_round():
