@@ -96,17 +96,21 @@ template <int MT, int NT, int WAVES, int EPI, typename TC>
 __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const bf16_t* __restrict__ A,
                                                                  const bf16_t* __restrict__ W,
                                                                  TC* __restrict__ C, int M, int N, int K,
-                                                                 int64_t lda, int64_t ldw, int64_t ldc, NormLink link) {
+                                                                 int64_t lda, int64_t ldw, int64_t ldc, NormLink link,
+                                                                 int rows_per_wg) {
     extern __shared__ float red[];      // [WAVES][NT][MT][4][64]
     __shared__ float link_scratch[WAVES * 64], link_scale[16];
     const float link_mine = row_scale_begin<WAVES * 64>(link, M, 0, 16);
     const int wave = threadIdx.x / 64, lane = threadIdx.x % 64;
     const int r16 = lane % 16, q = lane / 16;
-    const int n_base = blockIdx.x * (16 * NT);
+    // A workgroup takes rows_per_wg weight rows (at most 16 * NT): a number that need not fill
+    // its last tile of 16, so that the host can size the launch to the CUs.  Lanes of rows it does
+    // not have read its last row again, which costs no traffic, and their sums are not stored.
+    const int n_base = blockIdx.x * rows_per_wg;
 
     const bf16_t* wrow[NT];
 #pragma unroll
-    for (int t = 0; t < NT; ++t) wrow[t] = W + (int64_t)min(n_base + t * 16 + r16, N - 1) * ldw;
+    for (int t = 0; t < NT; ++t) wrow[t] = W + (int64_t)min(n_base + min(t * 16 + r16, rows_per_wg - 1), N - 1) * ldw;
     const bf16_t* arow[MT];
     bool mvalid[MT];
 #pragma unroll
@@ -207,7 +211,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const bf16_t* _
         }
         const int n = n_base + t * 16 + 4 * (l / 16) + r;
         const int m = u * 16 + l % 16;
-        if (m >= M || n >= N) continue;
+        if (m >= M || n >= N || t * 16 + 4 * (l / 16) + r >= rows_per_wg) continue;
         if (link.ssq) {
             s0 *= link_scale[m];
             s1 *= link_scale[m];
@@ -242,12 +246,15 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const bf16_t* _
 
 template <int MT, int NT, int WAVES>
 static int launch_skinny(const void* A, const void* W, void* C, int c_dt, int M, int N, int K, int64_t lda,
-                         int64_t ldw, int64_t ldc, int epi, hipStream_t stream, NormLink link = NormLink{}) {
+                         int64_t ldw, int64_t ldc, int epi, hipStream_t stream, NormLink link = NormLink{},
+                         int rows_per_wg = 16 * NT) {
     PICOLM_REQUIRE(!link.next_w || (MT == 1 && NT == 1 && WAVES == 8 && epi == 1 && link.next_parts >= ceil_div(N, 16)),
                    "gemm_skinny: only the 16x16 tile with the accumulating epilogue prepares a norm");
     PICOLM_REQUIRE((!link.ssq && !link.next_w) || (M <= 16 && link.rows == 16),
                    "gemm_skinny: a split norm goes with up to 16 rows here, got %d", M);
-    dim3 grid(ceil_div(N, 16 * NT)), block(WAVES * 64);
+    PICOLM_REQUIRE(rows_per_wg >= 2 && rows_per_wg <= 16 * NT && rows_per_wg % 2 == 0 && (!link.next_w || rows_per_wg == 16),
+                   "gemm_skinny: %d weight rows a workgroup do not fit %d tiles of 16", rows_per_wg, NT);
+    dim3 grid(ceil_div(N, rows_per_wg)), block(WAVES * 64);
     const size_t lds = sizeof(float) * WAVES * NT * MT * 4 * 64;
     const bf16_t* a = (const bf16_t*)A;
     const bf16_t* w = (const bf16_t*)W;
@@ -261,7 +268,7 @@ static int launch_skinny(const void* A, const void* W, void* C, int c_dt, int M,
                            hipGetErrorString(e));                                                       \
             raised = lds;                                                                               \
         }                                                                                               \
-        gemm_skinny_kernel<MT, NT, WAVES, EPI, TC><<<grid, block, lds, stream>>>(a, w, (TC*)C, M, N, K, lda, ldw, ldc, link); \
+        gemm_skinny_kernel<MT, NT, WAVES, EPI, TC><<<grid, block, lds, stream>>>(a, w, (TC*)C, M, N, K, lda, ldw, ldc, link, rows_per_wg); \
     }
     if (epi == 0 && c_dt == PICOLM_F32) SK_LAUNCH(0, float)
     else if (epi == 0 && c_dt == PICOLM_BF16) SK_LAUNCH(0, bf16_t)
@@ -412,6 +419,46 @@ static int check_mfma_operands(const char* who, const void* A, const void* W, in
 
 // variant: 0 picks by shape; 1..6 name (MT,NT,WAVES) combinations for tuning and tests, 7 is
 // the variant with resident activations
+// Weight rows a workgroup of the 16-row kernel takes: 16, or, where the workgroups of that size
+// would leave a last round of the CUs mostly empty, the multiple of 8 up to 64 with which the
+// launch takes the fewest rows per CU (6144 rows on 256 CUs: 24 rows each instead of 16 in one
+// and a half rounds).
+static int n_compute_units() {
+    static int n_cus = 0;
+    if (n_cus == 0) {
+        int dev = 0;
+        hipDeviceProp_t prop;
+        n_cus = hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess && prop.multiProcessorCount > 0
+                    ? prop.multiProcessorCount : 256;
+    }
+    return n_cus;
+}
+static int skinny_rows_per_wg(int N) {
+    const int cus = n_compute_units();
+    int best = 16;
+    int64_t best_cost = (int64_t)ceil_div(ceil_div(N, 16), cus) * 16 * 4;
+    for (int rows = 24; rows <= 64; rows += 8) {
+        // rounds of the CUs times what a workgroup moves; the rows that its last tile reads a
+        // second time cost no memory traffic but a quarter of their share of load instructions
+        const int padded = (rows + 15) / 16 * 16;
+        const int64_t cost = (int64_t)ceil_div(ceil_div(N, rows), cus) * (4 * rows + (padded - rows));
+        if (cost < best_cost) {
+            best = rows;
+            best_cost = cost;
+        }
+    }
+    return best;
+}
+template <int MT>
+static int launch_skinny_sized(const void* A, const void* W, void* C, int c_dt, int M, int N, int K, int64_t lda,
+                               int64_t ldw, int64_t ldc, int epi, hipStream_t stream, NormLink link) {
+    const int rows = link.next_w ? 16 : skinny_rows_per_wg(N);
+    if (rows <= 16) return launch_skinny<MT, 1, 8>(A, W, C, c_dt, M, N, K, lda, ldw, ldc, epi, stream, link, rows);
+    if (rows <= 32) return launch_skinny<MT, 2, 8>(A, W, C, c_dt, M, N, K, lda, ldw, ldc, epi, stream, link, rows);
+    if (rows <= 48) return launch_skinny<MT, 3, 8>(A, W, C, c_dt, M, N, K, lda, ldw, ldc, epi, stream, link, rows);
+    return launch_skinny<MT, 4, 8>(A, W, C, c_dt, M, N, K, lda, ldw, ldc, epi, stream, link, rows);
+}
+
 extern "C" int picolm_gemm_skinny(const void* A, const void* W, void* C, int c_dt, int M, int N, int K,
                                   int64_t lda, int64_t ldw, int64_t ldc, int epilogue, int variant,
                                   hipStream_t stream) {
@@ -426,7 +473,8 @@ extern "C" int picolm_gemm_skinny(const void* A, const void* W, void* C, int c_d
         else variant = M <= 16 ? 1 : (M <= 32 ? 3 : (N >= 8192 ? 6 : 5));
     }
     switch (variant) {
-        case 1: return launch_skinny<1, 1, 8>(A, W, C, c_dt, M, N, K, lda, ldw, ldc, epilogue, stream);
+        case 1: return launch_skinny_sized<1>(A, W, C, c_dt, M, N, K, lda, ldw, ldc, epilogue, stream, NormLink{});
+        case 8: return launch_skinny<1, 1, 8>(A, W, C, c_dt, M, N, K, lda, ldw, ldc, epilogue, stream);      // 16 rows a workgroup
         case 2: return launch_skinny<1, 2, 8>(A, W, C, c_dt, M, N, K, lda, ldw, ldc, epilogue, stream);
         case 3: return launch_skinny<2, 1, 8>(A, W, C, c_dt, M, N, K, lda, ldw, ldc, epilogue, stream);
         case 4: return launch_skinny<2, 2, 8>(A, W, C, c_dt, M, N, K, lda, ldw, ldc, epilogue, stream);
@@ -1252,7 +1300,7 @@ extern "C" int picolm_gemm_linked(const void* A, const void* W, void* C, int c_d
     }
     if (variant == 0) variant = (M > 4 && N >= 16384 && K % SK_KSTEP == 0 && K <= 4 * 8 * SK_KSTEP && !next_w) ? 7 : 1;
     switch (variant) {
-        case 1: return launch_skinny<1, 1, 8>(A, W, C, c_dt, M, N, K, lda, ldw, ldc, epilogue, stream, link);
+        case 1: return launch_skinny_sized<1>(A, W, C, c_dt, M, N, K, lda, ldw, ldc, epilogue, stream, link);
         case 7: return launch_skinny_resident<4>(A, W, C, c_dt, M, N, K, lda, ldw, ldc, epilogue, stream, link);
     }
     PICOLM_REQUIRE(false, "gemm_linked: skinny variant %d cannot take part in a split norm", variant);
