@@ -107,11 +107,12 @@ def session(folder, dtype, max_tokens=2048, **kw):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("which,n_seq", [("E", 20), ("E", 64), ("D", 33)])
+@pytest.mark.parametrize("which,n_seq", [("E", 20), ("E", 64), ("D", 33), ("E", 100)])
 def test_a_wide_batch_decodes_like_its_sequences_alone(which, n_seq, dtype, folders):
     """Decode batches of 17 to 64 sequences take kernels of their own (tiles of 64 rows cut along
-    K, the norm split between the products where the widths allow).  Unequal prompts, six steps,
-    every sequence's logits against the plain implementation of that sequence alone."""
+    K, the norm split between the products where the widths allow), and more than 64 the prefill's.
+    Unequal prompts, six steps, every sequence's logits against the plain implementation of that
+    sequence alone."""
     d = folders[which]
     V = tiny.read_config(d)["vocab_size"]
     rng = np.random.default_rng(n_seq)
