@@ -145,10 +145,31 @@ __device__ __forceinline__ double weight_of(const RowInfo& r, float l, int mode)
     return exp(mode == 1 ? x * r.inv_t : x);
 }
 
+// Every thread of the workgroup visits its share of the row: f(index, logit).  A row that starts
+// on a 16-byte boundary is read four values a load, several loads in flight.
+template <typename F>
+__device__ __forceinline__ void for_each_logit(const RowInfo& r, F f) {
+    const int tid = threadIdx.x;
+    int done = 0;
+    if (((uintptr_t)r.row & 15) == 0) {
+        const float4* p = (const float4*)r.row;
+        const int n4 = r.V / 4;
+#pragma unroll 4
+        for (int j = tid; j < n4; j += SM_THREADS) {
+            const float4 v = p[j];
+            f(4 * j, v.x);
+            f(4 * j + 1, v.y);
+            f(4 * j + 2, v.z);
+            f(4 * j + 3, v.w);
+        }
+        done = 4 * n4;
+    }
+    for (int i = done + tid; i < r.V; i += SM_THREADS) f(i, r.row[i]);
+}
+
 struct SampleShared {
     double hist_w[256];
     unsigned hist_c[256];
-    double red_d[SM_WAVES];
     unsigned red_u[SM_WAVES];
     int list_idx[SM_LIST];
     uint32_t list_key[SM_LIST];
@@ -158,6 +179,7 @@ struct SampleShared {
     unsigned n_list;
     int chosen;
     double base_w;
+    double target;
     unsigned base_c;
     Prefix res;
     unsigned res_count;
@@ -166,16 +188,6 @@ struct SampleShared {
     int bcast_i;
 };
 
-__device__ double block_sum_f64(double v, SampleShared& sm) {
-#pragma unroll
-    for (int o = WAVE / 2; o > 0; o >>= 1) v += __shfl_xor(v, o, WAVE);
-    __syncthreads();
-    if (threadIdx.x % WAVE == 0) sm.red_d[threadIdx.x / WAVE] = v;
-    __syncthreads();
-    double t = 0.0;
-    for (int i = 0; i < SM_WAVES; ++i) t += sm.red_d[i];
-    return t;
-}
 __device__ unsigned block_max_u32(unsigned v, SampleShared& sm) {
 #pragma unroll
     for (int o = WAVE / 2; o > 0; o >>= 1) v = max(v, (unsigned)__shfl_xor((int)v, o, WAVE));
@@ -246,9 +258,12 @@ __device__ int nth_tie(const RowInfo& r, uint32_t k, Prefix within, unsigned t, 
 // element where the sum crosses `target` (strict: sum > target, else sum >= target) or the
 // count reaches `limit`.  Leaves in sm.res the prefix ending at that element, in sm.res_count
 // its size, in sm.found whether a crossing happened (otherwise the prefix is `within`).
-__device__ void descend(const RowInfo& r, int mode, Prefix within, unsigned limit, double target,
+// The target is `fraction` times the sum of all weights of `within`, which the first histogram
+// gives (its buckets in ascending order): no pass of its own for the sum.
+__device__ void descend(const RowInfo& r, int mode, Prefix within, unsigned limit, double fraction,
                         bool strict, SampleShared& sm) {
     const int tid = threadIdx.x;
+    double target = 0.0;
     uint32_t prefix_q = 0;
     int bits = 0;
     if (tid == 0) {
@@ -263,17 +278,25 @@ __device__ void descend(const RowInfo& r, int mode, Prefix within, unsigned limi
             sm.hist_c[tid] = 0;
         }
         __syncthreads();
-        for (int i = tid; i < r.V; i += SM_THREADS) {
-            const float l = r.row[i];
+        for_each_logit(r, [&](int i, float l) {
             const uint32_t k = order_key(l);
-            if (!in_prefix(k, i, within)) continue;
+            if (!in_prefix(k, i, within)) return;
             const uint32_t q = quant24(r, l);
-            if (level > 0 && (q >> (shift + 8)) != prefix_q) continue;
+            if (level > 0 && (q >> (shift + 8)) != prefix_q) return;
             const int b = (q >> shift) & 255;
             atomicAdd(&sm.hist_c[b], 1u);
             if (mode != 2) unsafeAtomicAdd(&sm.hist_w[b], weight_of(r, l, mode));
-        }
+        });
         __syncthreads();
+        if (level == 0) {
+            if (tid == 0) {
+                double total = 0.0;
+                for (int b = 0; b < 256; ++b) total += sm.hist_w[b];
+                sm.target = fraction * total;
+            }
+            __syncthreads();
+            target = sm.target;
+        }
         if (tid == 0) {
             double cw = sm.base_w;
             unsigned cc = sm.base_c;
@@ -320,17 +343,16 @@ __device__ void descend(const RowInfo& r, int mode, Prefix within, unsigned limi
     if (bucket_count <= SM_LIST) {
         if (tid == 0) sm.n_list = 0;
         __syncthreads();
-        for (int i = tid; i < r.V; i += SM_THREADS) {
-            const float l = r.row[i];
+        for_each_logit(r, [&](int i, float l) {
             const uint32_t k = order_key(l);
-            if (!in_prefix(k, i, within)) continue;
-            if ((quant24(r, l) >> qshift) != prefix_q) continue;
+            if (!in_prefix(k, i, within)) return;
+            if ((quant24(r, l) >> qshift) != prefix_q) return;
             const unsigned pos = atomicAdd(&sm.n_list, 1u);
             if (pos < SM_LIST) {
                 sm.list_idx[pos] = i;
                 sm.list_key[pos] = k;
             }
-        }
+        });
         __syncthreads();
         const unsigned n = min(sm.n_list, (unsigned)SM_LIST);
         if ((unsigned)tid < n) {
@@ -459,14 +481,13 @@ __global__ __launch_bounds__(SM_THREADS) void sample_kernel(const float* __restr
     // maximum (first index) and minimum
     float best = -INFINITY, lo = INFINITY;
     int best_i = 0x7fffffff;
-    for (int i = tid; i < V; i += SM_THREADS) {
-        const float v = r.row[i];
+    for_each_logit(r, [&](int i, float v) {      // (a thread's indices come in ascending order)
         if (v > best || best_i == 0x7fffffff) {
             best = v;
             best_i = i;
         }
         lo = fminf(lo, v);
-    }
+    });
 #pragma unroll
     for (int o = WAVE / 2; o > 0; o >>= 1) {
         const float ov = __shfl_xor(best, o, WAVE);
@@ -507,24 +528,17 @@ __global__ __launch_bounds__(SM_THREADS) void sample_kernel(const float* __restr
     const unsigned k_limit = (top_k > 0 && top_k < V) ? (unsigned)top_k : (unsigned)V;   // sampler.c:70-73
     const bool use_p = top_p < 1.0f;
     if (use_p || k_limit < (unsigned)V) {                          // sampler.c:76-82
-        double Z = 0.0;
-        if (use_p) {
-            double z = 0.0;
-            for (int i = tid; i < V; i += SM_THREADS) z += weight_of(r, r.row[i], 0);
-            Z = block_sum_f64(z, sm);
-        }
-        descend(r, use_p ? 0 : 2, PREFIX_ALL, k_limit, (double)top_p * Z, false, sm);
+        descend(r, use_p ? 0 : 2, PREFIX_ALL, k_limit, (double)top_p, false, sm);
         kept = sm.res;
         kept_n = sm.res_count;
         __syncthreads();
     }
     if (min_p > 0.0f && kept_n > 1) {                              // sampler.c:85-95
         unsigned kmin = 0xffffffffu;
-        for (int i = tid; i < V; i += SM_THREADS) {
-            const float l = r.row[i];
+        for_each_logit(r, [&](int i, float l) {
             const uint32_t k = order_key(l);
             if (in_prefix(k, i, kept) && weight_of(r, l, 0) >= (double)min_p) kmin = min(kmin, k);
-        }
+        });
         const unsigned any = block_sum_u32(kmin != 0xffffffffu ? 1u : 0u, sm);
         kmin = block_min_u32(kmin, sm);
         if (any == 0)
@@ -533,16 +547,10 @@ __global__ __launch_bounds__(SM_THREADS) void sample_kernel(const float* __restr
             kept = Prefix{kmin, 0x7fffffff};
     }
     // sampler.c:98-121: weights p^(1/T) over the kept ones, a uniform r, the first running sum > r
-    double wsum = 0.0;
-    for (int i = tid; i < V; i += SM_THREADS) {
-        const float l = r.row[i];
-        if (in_prefix(order_key(l), i, kept)) wsum += weight_of(r, l, 1);
-    }
-    const double W = block_sum_f64(wsum, sm);
     const int sidx = state_index ? state_index[blockIdx.x] : blockIdx.x;
     const uint64_t x = xorshift64(rng_states[sidx]);
     const float rnd = (float)(x >> 11) / 9007199254740992.0f;      // sampler.c:19-21
-    descend(r, 1, kept, 0xffffffffu, (double)rnd * W, true, sm);
+    descend(r, 1, kept, 0xffffffffu, (double)rnd, true, sm);
     if (tid == 0) {
         out[blockIdx.x] = (sm.found && sm.res.idx != 0x7fffffff) ? sm.res.idx : top_token;
         rng_states[sidx] = x;
