@@ -120,9 +120,10 @@ class Session:
         for t in tokens:
             if not 0 <= t < self.vocab_size:
                 raise StepError(f"token id {t} is outside the vocabulary of {self.vocab_size}")
-        # unless a sequence starts a page (or runs out of room), every new token stays in its sequence's last page
-        if not all(p % PAGE_TOKENS for p in pos0) or max(pos0) >= self.cache.max_seq_len:
-            self.cache.reserve_many(slots, [p + 1 for p in pos0])
+        # unless a sequence starts a page (or runs out of room), its new token stays in its last page
+        grow = [(s, p + 1) for s, p in zip(slots, pos0) if p % PAGE_TOKENS == 0 or p >= self.cache.max_seq_len]
+        if grow:
+            self.cache.reserve_many([s for s, _ in grow], [n for _, n in grow])
             self.cache.flush()
         geometry = self._decode_geometry.get(len(slots))
         if geometry is None:
