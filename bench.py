@@ -61,6 +61,8 @@ def main() -> int:
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 / 64 points and the prefill")
     ap.add_argument("--prefill-only", action="store_true", help="run only the 2,048-token prefill (for profiling)")
     ap.add_argument("--batch-only", action="store_true", help="run only the decode at --batch (for profiling)")
+    ap.add_argument("--sampling", choices=["greedy", "picolm"], default="greedy",
+                    help="greedy (the measured default) or picolm's command-line defaults: temperature 0.8, top_k 40, top_p 0.9, min_p 0.05")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py measures one GPU; --gpus {args.gpus} is not supported by this single-GPU library")
@@ -71,6 +73,7 @@ def main() -> int:
     from picolm_amd import LlamaConfig
     from picolm_amd.engine import Session, random_model
     from picolm_amd.sampling import Sampler, SamplingParams
+    from picolm_amd.sampling.params import CLI_DEFAULTS
 
     full_layers = LLAMA31_8B["num_hidden_layers"]
     cfg_dict = dict(LLAMA31_8B)
@@ -89,7 +92,7 @@ def main() -> int:
         prompts = [[int(t) for t in rng.integers(0, cfg.vocab_size, size=n)] for n in lens]
         pages = sum((min(n + steps + warmup + 1, CONTEXT) + 63) // 64 for n in lens)
         sess = Session(model, max_tokens=pages * 64, max_seq_len=CONTEXT, n_slots=batch)
-        sampler = Sampler(SamplingParams(), batch, dev)
+        sampler = Sampler(CLI_DEFAULTS if args.sampling == "picolm" else SamplingParams(), batch, dev)
         slots = sess.begin(batch)
         # prompts go in one at a time here only to bound the workspace of this harness
         rows = []
@@ -152,7 +155,7 @@ def main() -> int:
             "rope_theta": cfg.rope_theta, "rope_scaling": "llama3 factor 8 low 1 high 4 original 8192",
             "rms_norm_eps": cfg.rms_norm_eps, "tied": cfg.tie_word_embeddings, "global_batch": args.batch,
             "seq_len": CONTEXT, "prompt_lengths": "uniform[128,2048]", "mean_context": round(ctx_tokens / args.batch, 1),
-            "parallelism": "single GPU",
+            "sampling": args.sampling, "parallelism": "single GPU",
         },
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBS, 4)},
