@@ -378,9 +378,6 @@ def medium_gemm_splits(M: int, N: int, K: int) -> int:
     return s
 
 
-LINKED_NORM_MAX_M = 1 << 30      # (a switch for measurements: rows above it take the norm's own kernel)
-
-
 def linked_norm_rows(M: int) -> int:
     """Rows that the partial sums of a split norm are kept for in a step of M rows: 16 or 64 in
     a decode step, every row (in whole 64s) otherwise."""
@@ -405,7 +402,7 @@ def gemm_links_norms(a, w, c, epilogue: int, prepares: bool) -> bool:
     kernel that adds the parts of a product cut along K does either for N in multiples of 1024,
     and the tile kernel of an uncut product can take the statistics.  Above that the tile kernels
     whose tiles go straight into LDS (K in multiples of 64) do both."""
-    if a.dim() != 2 or a.shape[0] > LINKED_NORM_MAX_M or not mfma_gemm_takes(a, w, c, epilogue):
+    if a.dim() != 2 or not mfma_gemm_takes(a, w, c, epilogue):
         return False
     M, N, K = a.shape[0], w.shape[0], a.shape[1]
     if M <= 16:
