@@ -63,6 +63,9 @@ def main() -> int:
     ap.add_argument("--batch-only", action="store_true", help="run only the decode at --batch (for profiling)")
     ap.add_argument("--sampling", choices=["greedy", "picolm"], default="greedy",
                     help="greedy (the measured default) or picolm's command-line defaults: temperature 0.8, top_k 40, top_p 0.9, min_p 0.05")
+    ap.add_argument("--steps-ahead", type=int, choices=[0, 1], default=1,
+                    help="1 (the generation loop's way): the next step is launched before this step's tokens are "
+                         "read on the host; 0: the host reads every step's tokens first")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py measures one GPU; --gpus {args.gpus} is not supported by this single-GPU library")
@@ -101,16 +104,28 @@ def main() -> int:
         logits = torch.cat(rows)
         idx = list(range(batch))
 
-        def one_step(lg):
-            toks = sampler.sample(lg, idx)
-            return sess.step(slots, [[t] for t in toks])
+        if args.steps_ahead:
+            # as the generation loop runs: a step takes its tokens on the device from the draw
+            # before it, and the host reads a step's tokens while the next step runs
+            def one_step(pending):
+                lg = sess.step_tokens_on_device(slots, pending.on_device())
+                nxt = sampler.launch(lg, idx)
+                pending.wait()
+                return nxt
 
+            state = sampler.launch(logits, idx)
+        else:
+            def one_step(lg):
+                toks = sampler.sample(lg, idx)
+                return sess.step(slots, [[t] for t in toks])
+
+            state = logits
         for _ in range(warmup):
-            logits = one_step(logits)
+            state = one_step(state)
         torch.cuda.synchronize()
         t = time.perf_counter()
         for _ in range(steps):
-            logits = one_step(logits)
+            state = one_step(state)
         torch.cuda.synchronize()
         dt = time.perf_counter() - t
         ctx = sum(sess.length(s) for s in slots) - batch * steps / 2.0     # mean live context over the timed steps
@@ -155,7 +170,7 @@ def main() -> int:
             "rope_theta": cfg.rope_theta, "rope_scaling": "llama3 factor 8 low 1 high 4 original 8192",
             "rms_norm_eps": cfg.rms_norm_eps, "tied": cfg.tie_word_embeddings, "global_batch": args.batch,
             "seq_len": CONTEXT, "prompt_lengths": "uniform[128,2048]", "mean_context": round(ctx_tokens / args.batch, 1),
-            "sampling": args.sampling, "parallelism": "single GPU",
+            "sampling": args.sampling, "steps_ahead": args.steps_ahead, "parallelism": "single GPU",
         },
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBS, 4)},

@@ -140,7 +140,13 @@ class Cache:
         """Bring the device page tables up to date (rows of slots that got pages)."""
         for g in self.kv:
             for s in sorted(g.dirty):
-                g.table[s].copy_(g.table_host[s], non_blocking=False)
+                row = g.table_host[s]
+                if g.table.device.type == "cuda":
+                    # through a pinned copy of the row and without waiting for the GPU (a step may
+                    # still be running); torch keeps the pinned block until the transfer has run
+                    g.table[s].copy_(row.pin_memory(), non_blocking=True)
+                else:
+                    g.table[s].copy_(row)
             g.dirty.clear()
 
     def bytes(self) -> int:

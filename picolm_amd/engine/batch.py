@@ -253,8 +253,14 @@ class DecodeBatch:
         off = (off + 3) // 4 * 4                    # what follows is read 16 bytes at a time
         self._used, self._size = off, off + (reserve_ints + 3) // 4 * 4
         self._device = torch.device(device)
-        self._host = self._host_block(self._size)
+        self._host = torch.zeros(self._size, dtype=torch.int32)
         self._dev = torch.zeros(self._size, dtype=torch.int32, device=device)
+        # The block goes to the device through one of two pinned copies, in turn, and the copy does
+        # not wait: a step can be handed to the GPU while the one before it still runs.  A pinned
+        # copy is written again only after the transfer that read it has ended.
+        self._pinned = [self._host_block(self._size), self._host_block(self._size)] if self._device.type == "cuda" else []
+        self._sent = [None, None]
+        self._turn = 0
         h = self._host.numpy()
         ar = np.arange(n + 1, dtype=np.int32)
         self._np = {k: h[o:o + s] for k, (o, s) in self._spans.items()}
@@ -286,9 +292,11 @@ class DecodeBatch:
         own = self._host_block(n_ints)
         return own.numpy(), torch.zeros(n_ints, dtype=torch.int32, device=self._device), own
 
-    def fill(self, slots, pos0, tokens, cache_version=None) -> None:
+    def fill(self, slots, pos0, tokens, cache_version=None, tokens_on_device=None) -> None:
         """`cache_version`: the cache's counter of slot and page changes; while it stands still
-        (and is given), what the last fill looked up in the page tables still holds."""
+        (and is given), what the last fill looked up in the page tables still holds.
+        `tokens_on_device`: an int32 tensor with the step's tokens, in place of `tokens`: the
+        host need not know them yet (they may come from a sampling kernel that has not run)."""
         # between page boundaries only the positions move: the lists and pages stay as they are
         same_pages = (cache_version is not None and cache_version == self._cache_version
                       and list(slots) == self.slots and len(pos0) == len(self.pos0)
@@ -298,7 +306,8 @@ class DecodeBatch:
         self._np["seq_slot"][:] = slots
         self._np["seq_pos0"][:] = pos0
         self._np["tok_pos"][:] = pos0
-        self._np["tokens"][:] = tokens
+        if tokens_on_device is None:
+            self._np["tokens"][:] = tokens
         for key in self._lists:
             if same_pages and key[0] == 0:          # (a window's first page can move on any step)
                 self._lists[key][0].reshape(-1, CHUNK_ENTRY_INTS)[1:1 + self._live[key], 2] += 1
@@ -307,10 +316,26 @@ class DecodeBatch:
         if not same_pages:
             for group in self._pages:
                 self._fill_pages(group)
-        self._dev.copy_(self._host, non_blocking=False)
+        self._send()
+        if tokens_on_device is not None:
+            self.tokens.copy_(tokens_on_device)
         for host, dev, *_, own in list(self._lists.values()) + list(self._pages.values()):
             if own is not None:
                 dev.copy_(own, non_blocking=False)
+
+    def _send(self) -> None:
+        if not self._pinned:
+            self._dev.copy_(self._host)
+            return
+        t = self._turn
+        self._turn ^= 1
+        if self._sent[t] is None:
+            self._sent[t] = torch.cuda.Event()
+        else:
+            self._sent[t].synchronize()
+        self._pinned[t].copy_(self._host)
+        self._dev.copy_(self._pinned[t], non_blocking=True)
+        self._sent[t].record()
 
     def _fill_pages(self, group: int) -> None:
         host, dev, table_host, ring_pages, own = self._pages[group]

@@ -28,8 +28,8 @@ class _DecodeGraph:
         self.logits = None
         self.uses = 0
 
-    def run(self, s: "Session", slots, pos0, tokens) -> torch.Tensor:
-        self.batch.fill(slots, pos0, tokens, s.cache.version)
+    def run(self, s: "Session", slots, pos0, tokens, tokens_on_device=None) -> torch.Tensor:
+        self.batch.fill(slots, pos0, tokens, s.cache.version, tokens_on_device)
         self.uses += 1
         if self.graph is not None:
             self.graph.replay()
@@ -114,10 +114,28 @@ class Session:
             self.cache.set_length(s, p + n)
         return logits
 
-    def _decode_step(self, slots, pos0, tokens) -> torch.Tensor:
+    def step_tokens_on_device(self, slots, tokens: torch.Tensor) -> torch.Tensor:
+        """One more token for each sequence, the tokens being an int32 tensor on the device that
+        the host need not have seen: what a sampling kernel wrote, or will have written when the
+        step runs.  Nothing here waits for the GPU, so the step can be handed over while the one
+        that produces its tokens still runs.  The tokens must lie inside the vocabulary (a
+        sampler's do); logits as from `step`, one row a sequence."""
+        slots = list(slots)
+        for s in slots:
+            if not self.cache.slots.is_live(s):
+                raise StepError(f"slot {s} is not live")
+        device = torch.device(self.model.runtime.device)
+        if tokens.dtype != torch.int32 or tokens.shape != (len(slots),) or tokens.device.type != device.type:
+            raise StepError(f"tokens on the device: expected int32 [{len(slots)}] on {device}, "
+                            f"got {tokens.dtype} {tuple(tokens.shape)} on {tokens.device}")
+        if not (self.graphs and slots):
+            return self.step(slots, [[t] for t in tokens.tolist()])
+        return self._decode_step(slots, [self.cache.length(s) for s in slots], None, tokens)
+
+    def _decode_step(self, slots, pos0, tokens, tokens_on_device=None) -> torch.Tensor:
         if len(set(slots)) != len(slots):
             raise StepError("a slot appears twice in one step")
-        for t in tokens:
+        for t in tokens or ():
             if not 0 <= t < self.vocab_size:
                 raise StepError(f"token id {t} is outside the vocabulary of {self.vocab_size}")
         # unless a sequence starts a page (or runs out of room), its new token stays in its last page
@@ -133,7 +151,7 @@ class Session:
         g = self._decode_graphs.get(key)
         if g is None:
             g = self._decode_graphs[key] = _DecodeGraph(self, len(slots), ppc)
-        logits = g.run(self, slots, pos0, tokens)
+        logits = g.run(self, slots, pos0, tokens, tokens_on_device)
         for s, p in zip(slots, pos0):
             self.cache.set_length(s, p + 1)
         return logits

@@ -10,6 +10,12 @@ ended its slots are released and the next batch starts in them.
 The loop only decides; it never looks inside logits.  `stepper` needs begin(n) -> slots,
 step(slots, tokens) -> logits rows, release(slots), `capacity` (longest sequence) and
 fits(lengths) -> bool; `make_sampler(n)` returns an object with sample(logits, indices).
+
+A stepper with step_ahead(slots, tokens on the device) and a sampler with launch(logits,
+indices) -> pending tokens (on_device(rows), wait()) are driven one step ahead: the next step is
+handed to the GPU before this step's tokens have reached the host, so that the GPU does not
+stand still while the host decides.  The decisions and the tokens are the same; a sequence that
+a stop token ends has by then been stepped once more, and that step's token is dropped.
 """
 from __future__ import annotations
 
@@ -95,6 +101,9 @@ class GenerationLoop:
             self.stats.steps += 1
             live = list(ids)
             t0 = self.clock()
+            if hasattr(st, "step_ahead") and hasattr(sampler, "launch"):
+                self._decode_one_ahead(sampler, logits, live, slot_of, length, results, max_new_tokens, on_token)
+                live = []
             while live:
                 tokens = sampler.sample(logits, live)
                 nxt = []
@@ -128,6 +137,49 @@ class GenerationLoop:
         finally:
             if slot_of:
                 st.release(list(slot_of.values()))
+
+    def _decode_one_ahead(self, sampler, logits, ids, slot_of, length, results, max_new_tokens, on_token) -> None:
+        """The decode loop of `_run_batch` with the next step launched before this step's tokens
+        are read.  Whether a sequence ends by its count of tokens or at the cache's capacity is
+        known without its token; only a stop token is found out one step late."""
+        st = self.stepper
+        rows = list(ids)                   # the sequences that the pending tokens belong to, row by row
+        pending = sampler.launch(logits, rows)
+        ended = set()
+        while rows:
+            ahead = [i for i in rows if i not in ended and len(results[i].tokens) + 1 < max_new_tokens
+                     and length[i] + 1 <= st.capacity]
+            next_pending = None
+            if ahead:
+                pick = None if ahead == rows else [rows.index(i) for i in ahead]
+                logits = st.step_ahead([slot_of[i] for i in ahead], pending.on_device(pick))
+                self.stats.steps += 1
+                for i in ahead:
+                    length[i] += 1
+                next_pending = sampler.launch(logits, ahead)
+            goes_on = set(ahead)
+            now_ended = []
+            for i, tok in zip(rows, pending.wait()):
+                if i in ended:             # stepped once more before its stop token was seen
+                    continue
+                tok = int(tok)
+                results[i].tokens.append(tok)
+                self.stats.generated_tokens += 1
+                if on_token:
+                    on_token(i, tok)
+                if tok in self.stop_ids:
+                    results[i].finish = "stop"
+                elif i in goes_on:
+                    continue
+                else:
+                    results[i].finish = "length" if len(results[i].tokens) >= max_new_tokens else "capacity"
+                now_ended.append(i)
+            if now_ended:
+                # a step that is still running for one of these reads and writes that sequence's
+                # own pages only, and whatever uses them next comes after it in the stream
+                st.release([slot_of.pop(i) for i in now_ended])
+                ended.update(now_ended)
+            rows, pending = ahead, next_pending
 
 
 # ---------------------------------------------------------------------------------------------
@@ -175,6 +227,9 @@ class SessionStepper:
 
     def step(self, slots, tokens):
         return self.session.step(slots, tokens)
+
+    def step_ahead(self, slots, tokens_on_device):
+        return self.session.step_tokens_on_device(slots, tokens_on_device)
 
     def release(self, slots):
         self.session.release(slots)

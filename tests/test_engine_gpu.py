@@ -376,3 +376,58 @@ def test_a_batch_that_continues_where_another_stopped(which, folders):
     for i, t in enumerate(second):
         ref = tiny.plain_logits(d, t)[-1]
         assert np.abs(got[i] - ref).max() <= tolerance("bfloat16", ref)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_steps_with_tokens_on_the_device_equal_steps_with_tokens_from_the_host(dtype, folders):
+    """A decode step may take its tokens from device memory (what the sampler wrote) so that the
+    host can hand it over before it has read them.  Several such steps in a row, each launched
+    before the one before it has been waited for, across a page boundary and with a sequence
+    leaving the batch: the same logits, bit for bit, as steps fed from the host."""
+    from picolm_amd.sampling import Sampler, SamplingParams
+    d = folders["D"]
+    V = tiny.read_config(d)["vocab_size"]
+    rng = np.random.default_rng(21)
+    prompts = [tiny.random_tokens(rng, n, V) for n in (61, 5, 120)]
+
+    def run(on_device):
+        s = session(d, dtype, max_tokens=1024)
+        sampler = Sampler(SamplingParams(), 3, DEV)
+        slots = s.begin(3)
+        logits = s.step(slots, prompts)
+        seen, live = [], [0, 1, 2]
+        pending = sampler.launch(logits, live)
+        for j in range(8):
+            if j == 5:                       # the second sequence leaves
+                pick, live = [0, 2], [0, 2]
+            else:
+                pick = None
+            if on_device:
+                logits = s.step_tokens_on_device([slots[i] for i in live], pending.on_device(pick))
+            else:
+                toks = pending.wait()
+                toks = toks if pick is None else [toks[r] for r in pick]
+                logits = s.step([slots[i] for i in live], [[t] for t in toks])
+            seen.append(logits.clone())
+            pending = sampler.launch(logits, live)
+        torch.cuda.synchronize()
+        assert [s.length(x) for x in slots] == [61 + 8, 5 + 5, 120 + 8]
+        return seen
+
+    a, b = run(True), run(False)
+    for x, y in zip(a, b):
+        assert torch.equal(x, y)
+
+
+def test_tokens_on_the_device_are_checked(folders):
+    from picolm_amd.engine import StepError
+    s = session(folders["A"], "float32")
+    slots = s.begin(2)
+    s.step(slots, [[1, 2], [3]])
+    with pytest.raises(StepError, match="int32"):
+        s.step_tokens_on_device(slots, torch.zeros(2, dtype=torch.int64, device=DEV))
+    with pytest.raises(StepError, match="int32"):
+        s.step_tokens_on_device(slots, torch.zeros(3, dtype=torch.int32, device=DEV))
+    s.release([slots[1]])
+    with pytest.raises(StepError, match="not live"):
+        s.step_tokens_on_device(slots, torch.zeros(2, dtype=torch.int32, device=DEV))

@@ -139,3 +139,60 @@ def test_a_failing_step_releases_the_batch():
     with pytest.raises(RuntimeError):
         loop.run([[1], [2]], 3)
     assert st.length == {} and len(st.free) == 4
+
+
+# -- one step ahead ---------------------------------------------------------------------------
+class AheadStepper(ScriptedStepper):
+    """Also takes the tokens of a step before the host has looked at them."""
+
+    def step_ahead(self, slots, tokens_on_device):
+        assert len(tokens_on_device) == len(slots)
+        return self.step(slots, [[t] for t in tokens_on_device])
+
+
+class _Pending:
+    def __init__(self, tokens, sampler):
+        self.tokens, self.sampler, self.waited = tokens, sampler, False
+
+    def on_device(self, rows=None):
+        return list(self.tokens) if rows is None else [self.tokens[r] for r in rows]
+
+    def wait(self):
+        assert not self.waited
+        self.waited = True
+        self.sampler.unread -= 1
+        return list(self.tokens)
+
+
+class AheadSampler(ScriptedSampler):
+    def launch(self, logits, indices):
+        self.unread = getattr(self, "unread", 0) + 1
+        assert self.unread <= 2, "more than two draws whose tokens the host has not read"
+        return _Pending(self.sample(logits, indices), self)
+
+
+@pytest.mark.parametrize("case", range(40))
+def test_one_step_ahead_decides_as_the_plain_loop(case):
+    """Random requests, stops, limits and a small capacity: the loop that launches the next step
+    before it reads this step's tokens produces the same tokens and endings, uses slots the same
+    way, and steps a sequence at most once beyond its stop token."""
+    import random
+    rnd = random.Random(case)
+    n = rnd.randint(1, 7)
+    prompts = [[10 + i] + [5] * rnd.randint(0, 6) for i in range(n)]
+    max_new = rnd.randint(1, 9)
+    capacity = rnd.choice([8, 10, 1000])
+    stop_at = {10 + i: len(prompts[i]) + rnd.randint(0, 8) for i in range(n) if rnd.random() < 0.6}
+    kw = dict(n_slots=rnd.randint(1, 4), capacity=capacity, batch_size=rnd.randint(1, 4))
+    plain, st0, sm0, loop0 = run(prompts, max_new, stop_at, **kw)
+    st = AheadStepper(n_slots=kw["n_slots"], capacity=capacity)
+    sm = AheadSampler(stop_at)
+    loop = GenerationLoop(st, lambda k: sm, stop_ids=[9], batch_size=kw["batch_size"])
+    ahead = loop.run(prompts, max_new)
+    assert [(r.tokens, r.finish) for r in ahead] == [(r.tokens, r.finish) for r in plain]
+    assert not st.length and sorted(st.free) == list(range(kw["n_slots"]))
+    assert loop.stats.generated_tokens == loop0.stats.generated_tokens
+    stopped = sum(r.finish == "stop" for r in plain)
+    assert loop0.stats.steps <= loop.stats.steps
+    tokens_stepped = lambda s: sum(sum(e[2]) for e in s.log if e[0] == "step")
+    assert tokens_stepped(st0) <= tokens_stepped(st) <= tokens_stepped(st0) + stopped
