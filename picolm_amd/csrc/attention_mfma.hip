@@ -41,6 +41,11 @@ __device__ __forceinline__ int key_of_elem(int e, int h) { return 16 * (e >> 3) 
 
 __device__ __forceinline__ __bf16 to_bf16(float f) { return (__bf16)f; }      // the hardware's round-to-nearest-even
 
+// 2^x as the hardware's one instruction.  exp2f() wraps it in a range check and two scalings so
+// that results below 2^-126 come out as denormals; a probability that small adds nothing to a sum
+// of float probabilities whose largest is near 1, and zero is as good.
+__device__ __forceinline__ float exp2_flushing(float x) { return __builtin_amdgcn_exp2f(x); }
+
 // One page of one wave: scores, online softmax, and the update of O^T.  KOP(t, s) returns the
 // K operand of tile t, k-step s; VOP(dt, t, ks) the V^T operand of column block dt.
 template <int D, bool MASKED, typename KOP, typename VOP>
@@ -76,7 +81,7 @@ __device__ __forceinline__ void attend_page(const bf16x8 (&Qf)[D / 16], f32x16 (
     // arithmetic; probabilities may reach 2^LAZY_MAX_STEP instead of 1 meanwhile.
     const bool grow = mx > m_run + LAZY_MAX_STEP;
     const float m_new = grow ? mx : m_run;
-    const float alpha = grow ? exp2f(m_run - m_new) : 1.0f;
+    const float alpha = grow ? exp2_flushing(m_run - m_new) : 1.0f;
     const bool rescale = __any(grow);
     float sum = 0.f;
     bf16x8 Pf[2][2];
@@ -84,7 +89,7 @@ __device__ __forceinline__ void attend_page(const bf16x8 (&Qf)[D / 16], f32x16 (
     for (int t = 0; t < 2; ++t)
 #pragma unroll
         for (int e = 0; e < 16; ++e) {
-            const float p = (!MASKED || S[t][e] > 0.5f * NEG_BIG) ? exp2f(fmaf(S[t][e], scale2, -m_new)) : 0.f;
+            const float p = (!MASKED || S[t][e] > 0.5f * NEG_BIG) ? exp2_flushing(fmaf(S[t][e], scale2, -m_new)) : 0.f;
             sum += p;
             Pf[t][e / 8][e % 8] = to_bf16(p);
         }
@@ -126,12 +131,12 @@ __device__ __forceinline__ void attend_tile(const bf16x8 (&Qf)[D / 16], const bf
     }
     mx = fmaxf(mx, __shfl_xor(mx, 32, WAVE));
     const float m_new = fmaxf(m_run, mx);
-    const float alpha = exp2f(m_run - m_new);
+    const float alpha = exp2_flushing(m_run - m_new);
     float sum = 0.f;
     bf16x8 Pf[2];
 #pragma unroll
     for (int e = 0; e < 16; ++e) {
-        const float p = S[e] > 0.5f * NEG_BIG ? exp2f(S[e] - m_new) : 0.f;
+        const float p = S[e] > 0.5f * NEG_BIG ? exp2_flushing(S[e] - m_new) : 0.f;
         sum += p;
         Pf[e / 8][e % 8] = to_bf16(p);
     }
