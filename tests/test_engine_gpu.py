@@ -431,3 +431,42 @@ def test_tokens_on_the_device_are_checked(folders):
     s.release([slots[1]])
     with pytest.raises(StepError, match="not live"):
         s.step_tokens_on_device(slots, torch.zeros(2, dtype=torch.int32, device=DEV))
+
+
+def test_generation_one_step_ahead_equals_generation_step_by_step(folders):
+    """The entry point drives a session one step ahead (the next step is launched before this
+    step's tokens are read).  With stops, a token limit and several batches in a small cache it
+    returns what a loop that reads every step's tokens first returns, with recorded steps and
+    without them."""
+    from picolm_amd.engine import Session, load_model
+    from picolm_amd.generation import GenerationLoop, SessionStepper
+    from picolm_amd.sampling import Sampler, SamplingParams
+    d = folders["D"]
+    V = tiny.read_config(d)["vocab_size"]
+    model = load_model(d, dtype="float32")
+    rng = np.random.default_rng(31)
+    prompts = [tiny.random_tokens(rng, n, V) for n in (3, 70, 20, 64, 9, 33)]
+    params = SamplingParams(temperature=0.9, top_k=50, top_p=0.95, seed=5)
+
+    class StepByStep:
+        """A stepper without step_ahead: the loop then reads every step's tokens first."""
+
+        def __init__(self, session):
+            self._inner = SessionStepper(session)
+            self.capacity = self._inner.capacity
+            self.begin, self.step, self.release, self.fits = (self._inner.begin, self._inner.step,
+                                                              self._inner.release, self._inner.fits)
+
+    def run(stepper_type, graphs, stop_ids):
+        s = Session(model, max_tokens=4 * 192, graphs=graphs)
+        loop = GenerationLoop(stepper_type(s), lambda n: Sampler(params, n, DEV), stop_ids, batch_size=3)
+        out = loop.run(prompts, 40)
+        assert s.cache.slots.n_free == s.cache.slots.n_slots
+        return [(r.tokens, r.finish) for r in out]
+
+    free = run(SessionStepper, True, ())
+    stops = [free[1][0][5], free[4][0][17]]
+    want = run(SessionStepper, True, stops)
+    assert any(f == "stop" for _, f in want) and any(f == "length" for _, f in want)
+    assert run(SessionStepper, False, stops) == want
+    assert run(StepByStep, True, stops) == want
