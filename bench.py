@@ -63,6 +63,8 @@ def main() -> int:
     ap.add_argument("--batch-only", action="store_true", help="run only the decode at --batch (for profiling)")
     ap.add_argument("--sampling", choices=["greedy", "picolm"], default="greedy",
                     help="greedy (the measured default) or picolm's command-line defaults: temperature 0.8, top_k 40, top_p 0.9, min_p 0.05")
+    ap.add_argument("--prefill-tokens", type=int, default=PREFILL_TOKENS,
+                    help="with --prefill-only: a prompt of another length than the 2,048 of the record")
     ap.add_argument("--steps-ahead", type=int, choices=[0, 1], default=1,
                     help="1 (the generation loop's way): the next step is launched before this step's tokens are "
                          "read on the host; 0: the host reads every step's tokens first")
@@ -135,7 +137,7 @@ def main() -> int:
         return batch * steps / dt, dt / steps, ctx
 
     def prefill_run(T: int, reps: int = 3):
-        sess = Session(model, max_tokens=T + 64, max_seq_len=CONTEXT, n_slots=1)
+        sess = Session(model, max_tokens=T + 64, max_seq_len=max(CONTEXT, T + 64), n_slots=1)
         toks = [int(t) for t in rng.integers(0, cfg.vocab_size, size=T)]
         times = []
         for _ in range(reps + 1):
@@ -151,8 +153,8 @@ def main() -> int:
         return float(np.median(times[1:]))
 
     if args.prefill_only:
-        sec = prefill_run(PREFILL_TOKENS)
-        print(json.dumps({"prefill_ms": round(sec * 1e3, 3), "tokens": PREFILL_TOKENS, "layers": cfg.num_hidden_layers}))
+        sec = prefill_run(args.prefill_tokens)
+        print(json.dumps({"prefill_ms": round(sec * 1e3, 3), "tokens": args.prefill_tokens, "layers": cfg.num_hidden_layers}))
         return 0
     tok_s, s_per_step, ctx_tokens = decode_run(args.batch, args.steps, args.warmup)
     step_bytes = weight_bytes(cfg) + ctx_tokens * kv_bytes_per_token(cfg)

@@ -156,15 +156,22 @@ __device__ __forceinline__ void attend_tile(const bf16x8 (&Qf)[D / 16], const bf
 // =============================================================================================
 // LDS tiles of the prefill kernel: a page's K and V^T as they lie in the cache, that is in the
 // order of the MFMA operands: the 64 lanes of a wave read 64 adjacent 16-byte chunks.
-template <int D>
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void attn_prefill_mfma_kernel(AttnArgs a, int HB, int tile_tokens,
-                                                                                                        int n_tiles, int n_cus) {
+//
+// HALVES = 2: eight waves in two halves of four.  Both halves have the same queries and heads and
+// each takes every other page of the keys, with LDS stages of its own; at the end the second half
+// hands its sums and softmax statistics to the first through LDS.  The longest tiles, which set
+// the kernel's time when a prompt gives each CU only a tile or two, then take half as long.
+template <int D, int HALVES>
+__global__ __launch_bounds__(256 * HALVES) __attribute__((amdgpu_waves_per_eu(2))) void attn_prefill_mfma_kernel(AttnArgs a, int HB, int tile_tokens,
+                                                                                                                 int n_tiles, int n_cus) {
     constexpr int KCH = D / 8;                        // 16-byte chunks of a K row
     constexpr int KP = PAGE_TOKENS * KCH / 256;       // K chunks a thread stages per page
     constexpr int VP = D * 8 / 256;                   // V^T chunks a thread stages per page
     constexpr int STAGE = 2 * PAGE_TOKENS * D;        // K tile + V^T tile, in bf16
-    extern __shared__ __attribute__((aligned(16))) bf16_t lds[];      // two stages
-    const int tid = threadIdx.x, wave = tid / WAVE, lane = tid % WAVE;
+    extern __shared__ __attribute__((aligned(16))) bf16_t lds_all[];      // two stages for each half
+    const int half = threadIdx.x / 256;
+    bf16_t* lds = lds_all + half * (2 * STAGE);
+    const int tid = threadIdx.x % 256, wave = tid / WAVE, lane = tid % WAVE;      // (within the half)
     const int l32 = lane % 32, h = lane / 32;
     const int R = a.H / a.G;
     const int head_chunks = (R + HB - 1) / HB;
@@ -174,9 +181,12 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void a
     // and a short tile, where the same order in every round would pair the longest with each other.
     const int per_tile = a.G * head_chunks;
     const int total = n_tiles * per_tile;
+    // (with HALVES = 2 a CU holds one workgroup at a time and takes the next when it is done:
+    // longest first as it is)
     const int round0 = (int)(blockIdx.x / n_cus) * n_cus, in_round = blockIdx.x - round0;
     const int round_size = min(n_cus, total - round0);
-    const int item = round0 + (((blockIdx.x / n_cus) & 1) ? round_size - 1 - in_round : in_round);
+    const int item = HALVES == 2 ? (int)blockIdx.x
+                                 : round0 + (((blockIdx.x / n_cus) & 1) ? round_size - 1 - in_round : in_round);
     const int tile_id = n_tiles - 1 - item / per_tile;
     const int which = item % per_tile;
     const int seq = a.tile_seq[tile_id], q0 = a.tile_q0[tile_id];
@@ -257,21 +267,52 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void a
             attend_page<D, true>(Qf, O, m_run, l_run, page * PAGE_TOKENS, qpos, q_ok, a.window, scale2, h, kop, vop);
     };
 
-    fetch(page_lo);
-    stash(0, page_lo);
+    // a half's pages: page_lo + half, then every HALVES-th; both halves go round the loop alike
+    const int n_rounds = (page_hi - page_lo + HALVES - 1) / HALVES;
+    auto page_of = [&](int round) { return page_lo + HALVES * round + half; };
+    if (page_of(0) < page_hi) {
+        fetch(page_of(0));
+        stash(0, page_of(0));
+    }
     __syncthreads();
     int cur = 0;
-    for (int page = page_lo; page + 1 < page_hi; ++page) {
-        fetch(page + 1);                          // in flight while this page is attended to
+    for (int round = 0; round + 1 < n_rounds; ++round) {
+        const int page = page_of(round), next = page_of(round + 1);
+        if (next < page_hi) fetch(next);          // in flight while this page is attended to
         __builtin_amdgcn_sched_barrier(0);
         compute(cur, page);
         __builtin_amdgcn_sched_barrier(0);
-        stash(cur ^ 1, page + 1);
+        if (next < page_hi) stash(cur ^ 1, next);
         __syncthreads();
         cur ^= 1;
     }
-    compute(cur, page_hi - 1);
+    if (page_of(n_rounds - 1) < page_hi) compute(cur, page_of(n_rounds - 1));
 
+    if (HALVES == 2) {
+        // The second half's O^T, reference point and sum of each lane go to the first half's lane
+        // of the same place through LDS (the stages are read out by now): value v of all lanes of a
+        // wave side by side.
+        __syncthreads();
+        float* hand = (float*)lds_all + (size_t)wave * (D / 32 * 16 + 2) * WAVE + lane;
+        if (half == 1) {
+#pragma unroll
+            for (int dt = 0; dt < D / 32; ++dt)
+#pragma unroll
+                for (int e = 0; e < 16; ++e) hand[(dt * 16 + e) * WAVE] = O[dt][e];
+            hand[(D / 32 * 16) * WAVE] = m_run;
+            hand[(D / 32 * 16 + 1) * WAVE] = l_run;
+        }
+        __syncthreads();
+        if (half == 1) return;
+        const float m_other = hand[(D / 32 * 16) * WAVE], l_other = hand[(D / 32 * 16 + 1) * WAVE];
+        const float m_both = fmaxf(m_run, m_other);
+        const float mine = exp2_flushing(m_run - m_both), other = exp2_flushing(m_other - m_both);
+        l_run = l_run * mine + l_other * other;
+#pragma unroll
+        for (int dt = 0; dt < D / 32; ++dt)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) O[dt][e] = O[dt][e] * mine + hand[(dt * 16 + e) * WAVE] * other;
+    }
     if (!q_ok) return;
     const float inv = l_run > 0.f ? 1.0f / l_run : 0.f;
     bf16_t* o = (bf16_t*)a.out + tok * a.H * D + (size_t)head * D;
@@ -619,20 +660,32 @@ extern "C" int picolm_attn_prefill_mfma(const void* q, const void* k_pages, cons
                        "attn_prefill_mfma: cannot read the device's properties");
         n_cus = prop.multiProcessorCount > 0 ? prop.multiProcessorCount : 1;
     }
-    dim3 grid(n_tiles * G * head_chunks), block(256);
-    const size_t lds = 2 * 2 * (size_t)PAGE_TOKENS * d * sizeof(bf16_t);       // two stages of K and V^T
-    if (d == 32) attn_prefill_mfma_kernel<32><<<grid, block, lds, stream>>>(a, HB, tile_tokens, n_tiles, n_cus);
-    else if (d == 64) attn_prefill_mfma_kernel<64><<<grid, block, lds, stream>>>(a, HB, tile_tokens, n_tiles, n_cus);
-    else {
-        static bool raised = false;
-        if (!raised) {
-            hipError_t e = hipFuncSetAttribute((const void*)attn_prefill_mfma_kernel<128>,
-                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-            PICOLM_REQUIRE(e == hipSuccess, "attn_prefill_mfma: cannot raise the LDS limit: %s", hipGetErrorString(e));
-            raised = true;
-        }
-        attn_prefill_mfma_kernel<128><<<grid, block, lds, stream>>>(a, HB, tile_tokens, n_tiles, n_cus);
+    // Up to a tile for each of a CU's two places the longest tile sets the time, and eight waves
+    // that share its pages halve it (measured at head size 128: 43 -> 33 us for 1,024 tokens, 85 -> 75
+    // for 2,048); with more tiles the CUs even out by themselves and two independent workgroups a CU
+    // overlap better than eight waves in step (219 against 243 us for 4,096 tokens).
+    const int halves = (int64_t)n_tiles * G * head_chunks <= 2 * (int64_t)n_cus ? 2 : 1;
+    dim3 grid(n_tiles * G * head_chunks), block(256 * halves);
+    const size_t lds = halves * 2 * 2 * (size_t)PAGE_TOKENS * d * sizeof(bf16_t);       // two stages of K and V^T a half
+#define PREFILL_LAUNCH(D, HALVES)                                                                             \
+    {                                                                                                         \
+        static size_t raised = 48 * 1024;                                                                     \
+        if (lds > raised) {                                                                                   \
+            hipError_t e = hipFuncSetAttribute((const void*)attn_prefill_mfma_kernel<D, HALVES>,              \
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);         \
+            PICOLM_REQUIRE(e == hipSuccess, "attn_prefill_mfma: cannot raise the LDS limit: %s",              \
+                           hipGetErrorString(e));                                                             \
+            raised = lds;                                                                                     \
+        }                                                                                                     \
+        attn_prefill_mfma_kernel<D, HALVES><<<grid, block, lds, stream>>>(a, HB, tile_tokens, n_tiles, n_cus); \
     }
+    if (d == 32 && halves == 2) PREFILL_LAUNCH(32, 2)
+    else if (d == 64 && halves == 2) PREFILL_LAUNCH(64, 2)
+    else if (halves == 2) PREFILL_LAUNCH(128, 2)
+    else if (d == 32) PREFILL_LAUNCH(32, 1)
+    else if (d == 64) PREFILL_LAUNCH(64, 1)
+    else PREFILL_LAUNCH(128, 1)
+#undef PREFILL_LAUNCH
     PICOLM_LAUNCH_CHECK("attn_prefill_mfma");
     return 0;
 }

@@ -410,6 +410,24 @@ def test_attention_prefill(dtype, H, G, d, window):
     assert err <= tol(dtype, np.abs(ref).max()), err
 
 
+@pytest.mark.parametrize("H,G,d,old,new", [(64, 16, 32, [0, 100], [700, 400]), (32, 16, 64, [0, 37], [1500, 640])])
+def test_attention_prefill_with_more_tiles_than_places(H, G, d, old, new):
+    """Up to two workgroups a CU the matrix-core kernel runs eight waves, in two halves that share
+    a tile's pages; with more tiles than that four waves.  The other prefill tests are small and
+    take the first way, this one is large enough (more than 512 workgroups) for the second."""
+    case = PagedCase(H, G, d, old, new, torch.bfloat16, seed=H + d)
+    b = case.batch()
+    heads = 4 if H // G >= 3 else H // G              # heads of a group that share a workgroup
+    n_tiles = sum(-(-n // (32 * (4 // heads))) for n in new)
+    assert n_tiles * G * -(-(H // G) // heads) > 512
+    out = torch.zeros_like(case.q_dev)
+    K().attn_prefill(case.q_dev, case.k_pages, case.v_pages, out, b, case.table, case.table.shape[1], H, G, d,
+                     0, 1.0 / math.sqrt(d))
+    ref = case.reference(0)
+    err = np.abs(out.double().cpu().numpy() - ref).max()
+    assert err <= tol(torch.bfloat16, np.abs(ref).max()), err
+
+
 def decode_work_list(case, window, pages_per_chunk, spare=0):
     """The work list the engine would build, with room for `spare` more entries behind it (a
     recorded step's list has room for full-length sequences): those hold garbage."""
