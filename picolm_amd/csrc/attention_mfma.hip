@@ -226,8 +226,10 @@ __global__ __launch_bounds__(256 * HALVES) __attribute__((amdgpu_waves_per_eu(2)
     const size_t page_elems = (size_t)a.G * PAGE_TOKENS * D;
 
     bf16x8 kreg[KP], vreg[VP];
-    auto fetch = [&](int page) {
-        const size_t base = (size_t)pt[page % a.ring_pages] * page_elems + (size_t)g * PAGE_TOKENS * D;
+    // (where a page lies is asked a round ahead of its loads, which would otherwise wait for it)
+    auto place_of = [&](int page) { return pt[page % a.ring_pages]; };
+    auto fetch = [&](int place) {
+        const size_t base = (size_t)place * page_elems + (size_t)g * PAGE_TOKENS * D;
         const bf16_t* kp = (const bf16_t*)a.k_pages + base;
         const bf16_t* vp = (const bf16_t*)a.v_pages + base;
 #pragma unroll
@@ -270,23 +272,26 @@ __global__ __launch_bounds__(256 * HALVES) __attribute__((amdgpu_waves_per_eu(2)
     // a half's pages: page_lo + half, then every HALVES-th; both halves go round the loop alike
     const int n_rounds = (page_hi - page_lo + HALVES - 1) / HALVES;
     auto page_of = [&](int round) { return page_lo + HALVES * round + half; };
-    if (page_of(0) < page_hi) {
-        fetch(page_of(0));
-        stash(0, page_of(0));
-    }
+    // (A half whose turn has no page left stages the tile's last page again and attends to
+    // nothing: loads and stores without conditions around them keep the waits for them apart from
+    // the matrix products.)
+    fetch(place_of(min(page_of(0), page_hi - 1)));
+    int next_place = place_of(min(page_of(1), page_hi - 1));
+    stash(0, min(page_of(0), page_hi - 1));
     __syncthreads();
     int cur = 0;
     for (int round = 0; round + 1 < n_rounds; ++round) {
-        const int page = page_of(round), next = page_of(round + 1);
-        if (next < page_hi) fetch(next);          // in flight while this page is attended to
+        const int next = min(page_of(round + 1), page_hi - 1);
+        fetch(next_place);                        // in flight while this page is attended to
+        next_place = place_of(min(page_of(round + 2), page_hi - 1));
         __builtin_amdgcn_sched_barrier(0);
-        compute(cur, page);
+        compute(cur, page_of(round));
         __builtin_amdgcn_sched_barrier(0);
-        if (next < page_hi) stash(cur ^ 1, next);
+        stash(cur ^ 1, next);
         __syncthreads();
         cur ^= 1;
     }
-    if (page_of(n_rounds - 1) < page_hi) compute(cur, page_of(n_rounds - 1));
+    compute(cur, page_of(n_rounds - 1));          // (past the tile's pages: nothing)
 
     if (HALVES == 2) {
         // The second half's O^T, reference point and sum of each lane go to the first half's lane
