@@ -65,6 +65,9 @@ def main() -> int:
                     help="greedy (the measured default) or picolm's command-line defaults: temperature 0.8, top_k 40, top_p 0.9, min_p 0.05")
     ap.add_argument("--prefill-tokens", type=int, default=PREFILL_TOKENS,
                     help="with --prefill-only: a prompt of another length than the 2,048 of the record")
+    ap.add_argument("--prompt-range", default="128,2048",
+                    help="prompt lengths of the decode runs, uniform in LO,HI (the record's are 128,2048)")
+    ap.add_argument("--context", type=int, default=CONTEXT, help="longest sequence the cache is laid out for")
     ap.add_argument("--steps-ahead", type=int, choices=[0, 1], default=1,
                     help="1 (the generation loop's way): the next step is launched before this step's tokens are "
                          "read on the host; 0: the host reads every step's tokens first")
@@ -91,12 +94,14 @@ def main() -> int:
     torch.cuda.synchronize()
     print(f"[bench] model of {cfg.num_hidden_layers} layers ready in {time.time() - t0:.1f}s", file=sys.stderr, flush=True)
     rng = np.random.default_rng(0)
+    prompt_lo, prompt_hi = (int(x) for x in args.prompt_range.split(","))
+    context = args.context
 
     def decode_run(batch: int, steps: int, warmup: int):
-        lens = [int(x) for x in rng.integers(128, 2049, size=batch)]
+        lens = [int(x) for x in rng.integers(prompt_lo, prompt_hi + 1, size=batch)]
         prompts = [[int(t) for t in rng.integers(0, cfg.vocab_size, size=n)] for n in lens]
-        pages = sum((min(n + steps + warmup + 1, CONTEXT) + 63) // 64 for n in lens)
-        sess = Session(model, max_tokens=pages * 64, max_seq_len=CONTEXT, n_slots=batch)
+        pages = sum((min(n + steps + warmup + 1, context) + 63) // 64 for n in lens)
+        sess = Session(model, max_tokens=pages * 64, max_seq_len=context, n_slots=batch)
         sampler = Sampler(CLI_DEFAULTS if args.sampling == "picolm" else SamplingParams(), batch, dev)
         slots = sess.begin(batch)
         # prompts go in one at a time here only to bound the workspace of this harness
@@ -137,7 +142,7 @@ def main() -> int:
         return batch * steps / dt, dt / steps, ctx
 
     def prefill_run(T: int, reps: int = 3):
-        sess = Session(model, max_tokens=T + 64, max_seq_len=max(CONTEXT, T + 64), n_slots=1)
+        sess = Session(model, max_tokens=T + 64, max_seq_len=max(context, T + 64), n_slots=1)
         toks = [int(t) for t in rng.integers(0, cfg.vocab_size, size=T)]
         times = []
         for _ in range(reps + 1):
@@ -164,14 +169,14 @@ def main() -> int:
         "value": round(tok_s, 2), "unit": "tok/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(s_per_step * 1e3, 4), "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": "bf16",
-        "data": "synthetic: random bf16 weights N(0,0.02), seeded uniform-random token ids, prompt lengths uniform in [128,2048]",
+        "data": f"synthetic: random bf16 weights N(0,0.02), seeded uniform-random token ids, prompt lengths uniform in [{prompt_lo},{prompt_hi}]",
         "config": {
             "model": "Llama-3.1-8B shape", "layers": cfg.num_hidden_layers, "layers_of_shape": full_layers,
             "hidden": cfg.hidden_size, "heads": cfg.num_attention_heads, "kv_heads": cfg.num_key_value_heads,
             "head_dim": cfg.head_dim, "intermediate": cfg.intermediate_size, "vocab": cfg.vocab_size,
             "rope_theta": cfg.rope_theta, "rope_scaling": "llama3 factor 8 low 1 high 4 original 8192",
             "rms_norm_eps": cfg.rms_norm_eps, "tied": cfg.tie_word_embeddings, "global_batch": args.batch,
-            "seq_len": CONTEXT, "prompt_lengths": "uniform[128,2048]", "mean_context": round(ctx_tokens / args.batch, 1),
+            "seq_len": context, "prompt_lengths": f"uniform[{prompt_lo},{prompt_hi}]", "mean_context": round(ctx_tokens / args.batch, 1),
             "sampling": args.sampling, "steps_ahead": args.steps_ahead, "parallelism": "single GPU",
         },
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",

@@ -55,11 +55,12 @@ int picolm_gemm_tiled_splitk(const void* A, const void* W, void* C, int c_dt, in
 // variant 12; cut along K (splits > 1, ws of splits * M * N floats, N a multiple of 1024) either
 // role, uncut taking only.
 // More than 64 rows (rows = a multiple of 64 of at least M, sums for every row): the tiled product
-// by shape, either role; picolm_gemm_tiled_norm_parts gives the shares it leaves (0: it cannot).
-int picolm_gemm_tiled_norm_parts(int M, int N, int K);
+// by shape, either role, cut along K when ws (ws_floats floats) is given and the shape has tiles for
+// half of the CUs or fewer; picolm_gemm_tiled_norm_parts gives the shares it leaves (0: it cannot).
+int picolm_gemm_tiled_norm_parts(int M, int N, int K, int64_t ws_floats);
 int picolm_gemm_linked(const void* A, const void* W, void* C, int c_dt, int M, int N, int K, int64_t lda,
                        int64_t ldw, int64_t ldc, int epilogue, int tiled, int variant, int splits, float* ws,
-                       const float* next_w, void* next_h, float* next_ssq, int next_parts, const float* ssq,
+                       int64_t ws_floats, const float* next_w, void* next_h, float* next_ssq, int next_parts, const float* ssq,
                        int n_parts, int norm_len, float eps, int rows, hipStream_t stream);
 
 // Within a group's part of a page, K[64][d] and V^T[d][64] lie as plain arrays, except in bfloat16

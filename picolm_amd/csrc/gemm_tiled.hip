@@ -289,8 +289,8 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(const float* __restr
 }
 
 static int launch_splitk_reduce(const float* ws, void* C, int c_dt, int M, int N, int64_t ldc, int splits, int epilogue,
-                                hipStream_t stream, NormLink link = NormLink{}) {
-    PICOLM_REQUIRE((!link.ssq && !link.next_w) || (N % 1024 == 0 && M <= link.rows && (link.rows == 16 || link.rows == 64)),
+                                hipStream_t stream, NormLink link) {
+    PICOLM_REQUIRE((!link.ssq && !link.next_w) || (N % 1024 == 0 && M <= link.rows),
                    "gemm_splitk: a split norm needs N (%d) in multiples of 1024 and up to %d rows", N, link.rows);
     PICOLM_REQUIRE(!link.next_w || (epilogue == 1 && link.next_parts >= N / 1024),
                    "gemm_splitk: only the accumulating epilogue prepares a norm");
@@ -334,16 +334,36 @@ static int tiled_plan(int M, int N, int K, int& n_first) {
     return t256 >= 192 ? 9 : t128m >= 192 ? 10 : 11;
 }
 
+// A short prompt's product with a narrow output has tiles for half of the CUs or fewer (512 rows
+// and 4096 columns: 128 tiles of 128x128).  Given room for the parts' sums it is cut along K like
+// a wide decode batch's, into 2 or 4, and the adding kernel applies the epilogue.  The cut depends
+// on the shape and the room alone, not on whether a norm is split around the product: the shares
+// of a norm's sums (N / 1024 of the adding kernel) must be known before the call.
+static int tiled_splits(int M, int N, int K, int variant, int64_t ws_floats) {
+    if (variant < 9 || variant > 11 || N % 1024 != 0) return 1;
+    const int bn = variant == 11 ? 128 : 256, bm = variant == 9 ? 256 : 128;
+    const int64_t tiles = (int64_t)ceil_div(M, bm) * ceil_div(N, bn);
+    if (tiles > 128) return 1;
+    int s = 4;
+    while (s > 1 && (tiles * s > 320 || K % (64 * s) != 0 || (int64_t)s * M * N > ws_floats)) s /= 2;
+    return s;
+}
+
 // Shares of a row's sum of squares that the tiled product of this shape leaves when it prepares a
-// norm (one per column of tiles), or 0 if its kernel cannot take part in a split norm.
-extern "C" int picolm_gemm_tiled_norm_parts(int M, int N, int K) {
+// norm (one per column of tiles, or per 1024 columns if the product is cut along K, which it is
+// when a workspace of ws_floats floats allows it), or 0 if its kernel cannot take part in a split norm.
+extern "C" int picolm_gemm_tiled_norm_parts(int M, int N, int K, int64_t ws_floats) {
     int n_first;
     const int variant = tiled_plan(M, N, K, n_first);
+    if (n_first == 0 && tiled_splits(M, N, K, variant, ws_floats) > 1) return N / 1024;
     return variant == 9 || variant == 10 ? ceil_div(N, 256) : variant == 11 ? ceil_div(N, 128) : 0;
 }
 
+static int launch_splitk_reduce(const float* ws, void* C, int c_dt, int M, int N, int64_t ldc, int splits, int epilogue,
+                                hipStream_t stream, NormLink link);
 static int gemm_tiled_linked(const void* A, const void* W, void* C, int c_dt, int M, int N, int K, int64_t lda,
-                             int64_t ldw, int64_t ldc, int epilogue, int variant, hipStream_t stream, NormLink link);
+                             int64_t ldw, int64_t ldc, int epilogue, int variant, hipStream_t stream, NormLink link,
+                             float* ws = nullptr, int64_t ws_floats = 0);
 
 extern "C" int picolm_gemm_tiled(const void* A, const void* W, void* C, int c_dt, int M, int N, int K,
                                  int64_t lda, int64_t ldw, int64_t ldc, int epilogue, int variant,
@@ -354,10 +374,19 @@ extern "C" int picolm_gemm_tiled(const void* A, const void* W, void* C, int c_dt
 }
 
 static int gemm_tiled_linked(const void* A, const void* W, void* C, int c_dt, int M, int N, int K, int64_t lda,
-                             int64_t ldw, int64_t ldc, int epilogue, int variant, hipStream_t stream, NormLink link) {
+                             int64_t ldw, int64_t ldc, int epilogue, int variant, hipStream_t stream, NormLink link,
+                             float* ws, int64_t ws_floats) {
     if (variant == 0) {
         int n_first;
         variant = tiled_plan(M, N, K, n_first);
+        const int splits = n_first == 0 && ws != nullptr ? tiled_splits(M, N, K, variant, ws_floats) : 1;
+        if (splits > 1) {
+            PICOLM_REQUIRE(((uintptr_t)ws & 15) == 0, "gemm_tiled: the workspace of a cut product must be 16-byte aligned");
+            const int rc = picolm_gemm_direct_prefill_(variant, A, W, ws, PICOLM_F32, M, N, K, lda, ldw, N, 0, stream, splits,
+                                                       (int64_t)M * N, NormLink{});
+            if (rc) return rc;
+            return launch_splitk_reduce(ws, C, c_dt, M, N, ldc, splits, epilogue, stream, link);
+        }
         if (n_first > 0) {
             const int N1 = n_first * 256;
             const size_t c_item = c_dt == PICOLM_F32 ? 4 : 2;
@@ -410,14 +439,14 @@ extern "C" int picolm_gemm_tiled_splitk(const void* A, const void* W, void* C, i
         default: PICOLM_REQUIRE(false, "gemm_splitk: variant %d cannot split K", variant);
     }
     if (rc) return rc;
-    return launch_splitk_reduce(ws, C, c_dt, M, N, ldc, splits, epilogue, stream);
+    return launch_splitk_reduce(ws, C, c_dt, M, N, ldc, splits, epilogue, stream, NormLink{});
 }
 
 // The products of a decode step with a norm split between them (see NormLink).  Up to 16 rows:
 // `variant` as in picolm_gemm_skinny (0, 1, 7) or, with tiled != 0, tile variant 12 or 13; rows = 16.
 // More than 64 rows (a prefill step): tiled, rows = a multiple of 64 of at least M, the tile
-// variant by shape; either role, one share of the sums per column of tiles
-// (picolm_gemm_tiled_norm_parts).
+// variant by shape, cut along K if ws is given and the shape has few tiles; either role, the
+// shares of the sums as picolm_gemm_tiled_norm_parts says for the same ws_floats.
 // 17 to 64 rows: tiled, variant 12, rows = 64; with splits > 1 (ws as in picolm_gemm_tiled_splitk)
 // the kernel that adds the parts takes either role and N must be a multiple of 1024; uncut, the
 // tile kernel can only take a prepared norm's statistics.
@@ -427,7 +456,7 @@ extern "C" int picolm_gemm_tiled_splitk(const void* A, const void* W, void* C, i
 // are the next_h of a product that prepared their norm.
 extern "C" int picolm_gemm_linked(const void* A, const void* W, void* C, int c_dt, int M, int N, int K, int64_t lda,
                                   int64_t ldw, int64_t ldc, int epilogue, int tiled, int variant, int splits,
-                                  float* ws, const float* next_w, void* next_h, float* next_ssq, int next_parts,
+                                  float* ws, int64_t ws_floats, const float* next_w, void* next_h, float* next_ssq, int next_parts,
                                   const float* ssq, int n_parts, int norm_len, float eps, int rows,
                                   hipStream_t stream) {
     if (check_mfma_operands("gemm_linked", A, W, M, N, K, lda, ldw, ldc, epilogue, c_dt)) return -1;
@@ -440,9 +469,10 @@ extern "C" int picolm_gemm_linked(const void* A, const void* W, void* C, int c_d
     NormLink link = {next_w, (bf16_t*)next_h, next_ssq, next_parts, ssq, n_parts, norm_len > 0 ? 1.0f / (float)norm_len : 0.f, eps, rows};
     if (rows > 64) {            // a prefill step: the tile variants by shape, sums for every row
         PICOLM_REQUIRE(tiled && splits == 1, "gemm_linked: more than 64 rows take the uncut tiled product");
-        return gemm_tiled_linked(A, W, C, c_dt, M, N, K, lda, ldw, ldc, epilogue, 0, stream, link);
+        return gemm_tiled_linked(A, W, C, c_dt, M, N, K, lda, ldw, ldc, epilogue, 0, stream, link, ws, ws_floats);
     }
     if (tiled && splits > 1) {
+        PICOLM_REQUIRE((int64_t)splits * M * N <= ws_floats, "gemm_linked: %d splits of %d x %d exceed the workspace", splits, M, N);
         PICOLM_REQUIRE(variant == 12 && ws != nullptr && ((uintptr_t)ws & 15) == 0 && N % 4 == 0,
                        "gemm_linked: a cut product needs tile variant 12, a workspace and N in multiples of 4");
         const int rc = launch_direct<1, 2, 4, 1, 64, 3>(A, W, ws, PICOLM_F32, M, N, K, lda, ldw, N, 0, stream, splits, (int64_t)M * N);

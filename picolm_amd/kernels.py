@@ -393,7 +393,7 @@ def linked_norm_parts(M: int, N: int, K: int) -> int:
         return (N + 15) // 16
     if M <= 64:
         return N // 1024
-    return lib().picolm_gemm_tiled_norm_parts(M, N, K)
+    return lib().picolm_gemm_tiled_norm_parts(M, N, K, c_int64(SPLITK_WS_FLOATS))
 
 
 def gemm_links_norms(a, w, c, epilogue: int, prepares: bool) -> bool:
@@ -451,7 +451,8 @@ def gemm_linked(a, w, c, epilogue: int, prepare=None, prepared=None) -> None:
             raise KernelError("gemm_linked: the statistics are not those of this product's input rows")
     tiled, variant, splits, ws = 0, 0, 1, None
     if M > 64:
-        tiled = 1                       # the tile variant by shape, as in gemm()
+        tiled = 1                       # the tile variant by shape, cut along K where it has few tiles
+        ws = splitk_workspace(a.device)
     elif M > 16:
         tiled, variant, splits = 1, 12, medium_gemm_splits(M, N, K)          # as in gemm()
         ws = splitk_workspace(a.device) if splits > 1 else None
@@ -459,6 +460,7 @@ def gemm_linked(a, w, c, epilogue: int, prepare=None, prepared=None) -> None:
         tiled, variant = 1, 13          # as in gemm()
     _check(lib().picolm_gemm_linked(_ptr(a), _ptr(w), _ptr(c), dt_of(c), M, N, K, c_int64(K), c_int64(K),
                                     c_int64(c.shape[1]), epilogue, tiled, variant, splits, _ptr(ws),
+                                    c_int64(SPLITK_WS_FLOATS),
                                     _ptr(nw), _ptr(nh), _ptr(nssq), next_parts,
                                     _ptr(ssq), n_parts, int(norm_len), c_float(eps), rows, _stream()))
 
@@ -468,7 +470,7 @@ def gemm(a: torch.Tensor, w: torch.Tensor, c: torch.Tensor, epilogue: int = EPI_
     if mfma_gemm_takes(a, w, c, epilogue):
         M, N, K = a.shape[0], w.shape[0], a.shape[1]
         if M > SKINNY_MAX_M:
-            gemm_tiled(a, w, c, epilogue)
+            gemm_linked(a, w, c, epilogue)          # (no norm around it: the tiled product, cut along K if short)
         elif M > 16 and K % 64 == 0:
             # a decode batch too wide to re-read its activations for every 16 weight rows: tiles
             # of 128 weight rows through LDS, cut along K where there are few of them

@@ -175,6 +175,20 @@ def test_gemm_medium_batches_pick_their_splits():
             run_gemm(K().gemm, M, N, Kd, epi, torch.bfloat16, torch.bfloat16, cdt)
 
 
+def test_gemm_of_a_short_prompt_is_cut_along_k():
+    """More than 64 rows but tiles for half of the CUs or fewer (a short prompt's products into
+    the model's width): the tiled product is cut along K like a wide decode batch's.  Every
+    epilogue against the plain product, with and without the cut (N no multiple of 1024: uncut)."""
+    k = K()
+    ws = k.SPLITK_WS_FLOATS
+    assert k.lib().picolm_gemm_tiled_norm_parts(512, 4096, 4096, k.c_int64(ws)) == 4           # cut: N / 1024
+    assert k.lib().picolm_gemm_tiled_norm_parts(512, 4096, 4096, k.c_int64(0)) == 32          # no room: per column of tiles
+    assert k.lib().picolm_gemm_tiled_norm_parts(2048, 4096, 4096, k.c_int64(ws)) == 16        # enough tiles
+    for M, N, Kd in ((512, 4096, 4096), (300, 1024, 512), (65, 2048, 14336 // 7), (512, 4096 + 8, 1024), (200, 2048, 64 * 3)):
+        for epi, cdt in ((0, torch.float32), (2, torch.bfloat16), (1, torch.float32), (0, torch.bfloat16)):
+            run_gemm(k.gemm, M, N, Kd, epi, torch.bfloat16, torch.bfloat16, cdt)
+
+
 @pytest.mark.parametrize("M", [1, 8, 16])
 @pytest.mark.parametrize("D", [48, 256, 4096])
 def test_gemm_with_a_norm_split_between_two_products(M, D):
