@@ -331,7 +331,7 @@ static int tiled_plan(int M, int N, int K, int& n_first) {
         n_first = first;
         return 9;
     }
-    return t256 >= 192 ? 9 : t128m >= 192 ? 10 : 11;
+    return t256 >= 144 ? 9 : t128m >= 144 ? 10 : 11;
 }
 
 // A short prompt's product with a narrow output has tiles for half of the CUs or fewer (512 rows
@@ -349,13 +349,31 @@ static int tiled_splits(int M, int N, int K, int variant, int64_t ws_floats) {
     return s;
 }
 
+// The variant, the cut along K and the two-launch plan for a shape.  Where the 128x128 tiles are
+// too many to cut but the 256x128 ones are few and K is long (a prompt of 768 tokens into the
+// model's width from the feed-forward's), the larger tile cut in two is the faster (measured
+// 103 against 114 us at 768 x 4096 x 14336; with K = 4096 the smaller tile uncut wins).
+static void tiled_choice(int M, int N, int K, int64_t ws_floats, int& variant, int& splits, int& n_first) {
+    variant = tiled_plan(M, N, K, n_first);
+    splits = 1;
+    if (n_first > 0) return;
+    splits = tiled_splits(M, N, K, variant, ws_floats);
+    if (splits == 1 && variant == 11 && K >= 8192) {
+        const int s10 = tiled_splits(M, N, K, 10, ws_floats);
+        if (s10 > 1) {
+            variant = 10;
+            splits = s10;
+        }
+    }
+}
+
 // Shares of a row's sum of squares that the tiled product of this shape leaves when it prepares a
 // norm (one per column of tiles, or per 1024 columns if the product is cut along K, which it is
 // when a workspace of ws_floats floats allows it), or 0 if its kernel cannot take part in a split norm.
 extern "C" int picolm_gemm_tiled_norm_parts(int M, int N, int K, int64_t ws_floats) {
-    int n_first;
-    const int variant = tiled_plan(M, N, K, n_first);
-    if (n_first == 0 && tiled_splits(M, N, K, variant, ws_floats) > 1) return N / 1024;
+    int variant, splits, n_first;
+    tiled_choice(M, N, K, ws_floats, variant, splits, n_first);
+    if (splits > 1) return N / 1024;
     return variant == 9 || variant == 10 ? ceil_div(N, 256) : variant == 11 ? ceil_div(N, 128) : 0;
 }
 
@@ -377,9 +395,8 @@ static int gemm_tiled_linked(const void* A, const void* W, void* C, int c_dt, in
                              int64_t ldw, int64_t ldc, int epilogue, int variant, hipStream_t stream, NormLink link,
                              float* ws, int64_t ws_floats) {
     if (variant == 0) {
-        int n_first;
-        variant = tiled_plan(M, N, K, n_first);
-        const int splits = n_first == 0 && ws != nullptr ? tiled_splits(M, N, K, variant, ws_floats) : 1;
+        int n_first, splits;
+        tiled_choice(M, N, K, ws != nullptr ? ws_floats : 0, variant, splits, n_first);
         if (splits > 1) {
             PICOLM_REQUIRE(((uintptr_t)ws & 15) == 0, "gemm_tiled: the workspace of a cut product must be 16-byte aligned");
             const int rc = picolm_gemm_direct_prefill_(variant, A, W, ws, PICOLM_F32, M, N, K, lda, ldw, N, 0, stream, splits,

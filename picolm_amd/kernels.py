@@ -332,7 +332,7 @@ def gemm_tiled(a, w, c, epilogue: int = EPI_STORE, variant: int = 0) -> None:
                                    c_int64(c.shape[1]), epilogue, variant, _stream()))
 
 
-SPLITK_WS_FLOATS = 4 << 20        # 16 MB of partial sums: splits * M * N may not exceed it
+SPLITK_WS_FLOATS = 8 << 20        # 32 MB of partial sums: splits * M * N may not exceed it
 _splitk_ws: dict = {}
 
 
