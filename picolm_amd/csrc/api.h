@@ -52,7 +52,7 @@ int picolm_gemm_tiled_splitk(const void* A, const void* W, void* C, int c_dt, in
 // rows are such a next_h takes ssq[n_parts][rows], the norm's row length and eps and multiplies
 // its sums by 1 / sqrt(sum / len + eps).  Up to 16 rows (rows = 16): skinny variant 0/1 (either
 // role), 7, or tiled != 0 with tile variant 12/13 (taking only).  17 to 64 rows (rows = 64): tiled,
-// variant 12; cut along K (splits > 1, ws of splits * M * N floats, N a multiple of 1024) either
+// variant 12 (13 up to 32 rows); cut along K (splits > 1, ws of splits * M * N floats, N a multiple of 1024) either
 // role, uncut taking only.
 // More than 64 rows (rows = a multiple of 64 of at least M, sums for every row): the tiled product
 // by shape, either role, cut along K when ws (ws_floats floats) is given and the shape has tiles for

@@ -464,7 +464,7 @@ extern "C" int picolm_gemm_tiled_splitk(const void* A, const void* W, void* C, i
 // More than 64 rows (a prefill step): tiled, rows = a multiple of 64 of at least M, the tile
 // variant by shape, cut along K if ws is given and the shape has few tiles; either role, the
 // shares of the sums as picolm_gemm_tiled_norm_parts says for the same ws_floats.
-// 17 to 64 rows: tiled, variant 12, rows = 64; with splits > 1 (ws as in picolm_gemm_tiled_splitk)
+// 17 to 64 rows: tiled, variant 12 (13 up to 32 rows), rows = 64; with splits > 1 (ws as in picolm_gemm_tiled_splitk)
 // the kernel that adds the parts takes either role and N must be a multiple of 1024; uncut, the
 // tile kernel can only take a prepared norm's statistics.
 // next_*: this product (epilogue 1) prepares the norm that follows: next_h[M][ldc] and
@@ -490,9 +490,11 @@ extern "C" int picolm_gemm_linked(const void* A, const void* W, void* C, int c_d
     }
     if (tiled && splits > 1) {
         PICOLM_REQUIRE((int64_t)splits * M * N <= ws_floats, "gemm_linked: %d splits of %d x %d exceed the workspace", splits, M, N);
-        PICOLM_REQUIRE(variant == 12 && ws != nullptr && ((uintptr_t)ws & 15) == 0 && N % 4 == 0,
-                       "gemm_linked: a cut product needs tile variant 12, a workspace and N in multiples of 4");
-        const int rc = launch_direct<1, 2, 4, 1, 64, 3>(A, W, ws, PICOLM_F32, M, N, K, lda, ldw, N, 0, stream, splits, (int64_t)M * N);
+        PICOLM_REQUIRE((variant == 12 || (variant == 13 && M <= 32)) && ws != nullptr && ((uintptr_t)ws & 15) == 0 && N % 4 == 0,
+                       "gemm_linked: a cut product needs tile variant 12 (or 13 up to 32 rows), a workspace and N in multiples of 4");
+        const int rc = variant == 12
+            ? launch_direct<1, 2, 4, 1, 64, 3>(A, W, ws, PICOLM_F32, M, N, K, lda, ldw, N, 0, stream, splits, (int64_t)M * N)
+            : launch_direct<1, 1, 4, 1, 64, 4>(A, W, ws, PICOLM_F32, M, N, K, lda, ldw, N, 0, stream, splits, (int64_t)M * N);
         if (rc) return rc;
         return launch_splitk_reduce(ws, C, c_dt, M, N, ldc, splits, epilogue, stream, link);
     }

@@ -367,6 +367,12 @@ def mfma_gemm_takes(a, w, c, epilogue: int) -> bool:
     return True
 
 
+def medium_gemm_variant(M: int) -> int:
+    """The tile variant for a decode batch of 17 to 64 rows: tiles of 128 weight rows by 64
+    activation rows, or by 32 where that is enough (measured 5 to 9 % faster there)."""
+    return 13 if M <= 32 else 12
+
+
 def medium_gemm_splits(M: int, N: int, K: int) -> int:
     """Into how many parts along K a product of 17..64 rows is cut: its tiles hold 128 weight
     rows each, and every CU should have one."""
@@ -454,7 +460,7 @@ def gemm_linked(a, w, c, epilogue: int, prepare=None, prepared=None) -> None:
         tiled = 1                       # the tile variant by shape, cut along K where it has few tiles
         ws = splitk_workspace(a.device)
     elif M > 16:
-        tiled, variant, splits = 1, 12, medium_gemm_splits(M, N, K)          # as in gemm()
+        tiled, variant, splits = 1, medium_gemm_variant(M), medium_gemm_splits(M, N, K)          # as in gemm()
         ws = splitk_workspace(a.device) if splits > 1 else None
     elif prepare is None and M > 4 and K % 64 == 0 and 16384 <= N <= 128 * 256:
         tiled, variant = 1, 13          # as in gemm()
@@ -474,7 +480,7 @@ def gemm(a: torch.Tensor, w: torch.Tensor, c: torch.Tensor, epilogue: int = EPI_
         elif M > 16 and K % 64 == 0:
             # a decode batch too wide to re-read its activations for every 16 weight rows: tiles
             # of 128 weight rows through LDS, cut along K where there are few of them
-            gemm_tiled_splitk(a, w, c, epilogue, 12, medium_gemm_splits(M, N, K))
+            gemm_tiled_splitk(a, w, c, epilogue, medium_gemm_variant(M), medium_gemm_splits(M, N, K))
         elif M > 4 and K % 64 == 0 and 16384 <= N <= 128 * 256:
             # several rows and one round of 128-row tiles for the CUs: the tiles share the
             # activations through LDS (more rounds suit the skinny kernel's resident variant better)
