@@ -247,7 +247,14 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(const float* __restr
     const int m = inside ? (int)(i / N) : 0, n = inside ? (int)(i % N) : 0;      // N is a multiple of 4 (the host sees to that)
     f32x4 sum = {0.f, 0.f, 0.f, 0.f};
     if (inside)
-        for (int z = 0; z < splits; ++z) sum += *(const f32x4*)(ws + (int64_t)z * M * N + i);
+        for (int z0 = 0; z0 < splits; z0 += 8) {      // eight parts asked for at a time, added in order
+            f32x4 part[8];
+#pragma unroll
+            for (int e = 0; e < 8; ++e) part[e] = *(const f32x4*)(ws + (int64_t)min(z0 + e, splits - 1) * M * N + i);
+#pragma unroll
+            for (int e = 0; e < 8; ++e)
+                if (z0 + e < splits) sum += part[e];
+        }
     if (link.ssq) {
         float total = 0.f;      // (eight loads asked for at a time, as in row_scale_begin)
         for (int p0 = 0; p0 < link.n_parts; p0 += 8) {
