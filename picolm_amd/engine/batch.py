@@ -19,6 +19,16 @@ class StepError(ValueError):
     """A step that cannot run: a dead slot, a token outside the vocabulary, no room."""
 
 
+def _to_device(host: torch.Tensor, device) -> torch.Tensor:
+    """A copy of a small host array on the device that does not make the host wait for the GPU (a
+    plain copy from pageable memory waits for everything the stream still has to do, and a prefill
+    step asks for such arrays after its first kernels are on their way): through pinned memory,
+    which torch keeps until the transfer has run."""
+    if torch.device(device).type != "cuda":
+        return host.to(device)
+    return host.pin_memory().to(device, non_blocking=True)
+
+
 class StepBatch:
     def __init__(self, slots, pos0, new_tokens, want, vocab_size: int, device):
         """slots[i]: cache slot of sequence i; pos0[i]: tokens it holds; new_tokens[i]: its
@@ -85,7 +95,7 @@ class StepBatch:
             flat[off:off + len(v)] = v
             spans[k] = (off, n)
             off += n
-        dev = torch.from_numpy(flat).to(self._device)
+        dev = _to_device(torch.from_numpy(flat), self._device)
         for k, (o, n) in spans.items():
             setattr(self, k, dev[o:o + n])
 
@@ -100,7 +110,7 @@ class StepBatch:
             tiles.sort()          # by the keys a tile sees: the kernels hand out the longest first
             seqs = [t[1] for t in tiles]
             q0s = [t[2] for t in tiles]
-            flat = torch.tensor(seqs + q0s, dtype=torch.int32).to(self._device)
+            flat = _to_device(torch.tensor(seqs + q0s, dtype=torch.int32), self._device)
             self._tiles[rows_per_tile] = (flat[:len(seqs)], flat[len(seqs):], len(seqs))
         return self._tiles[rows_per_tile]
 
@@ -121,7 +131,7 @@ class StepBatch:
         key and value (device int32 [T])."""
         if group not in self._write_pages:
             pages = token_pages(self._host["tok_seq"], self._host["tok_pos"], self.slots, table_host, ring_pages)
-            self._write_pages[group] = torch.from_numpy(pages).to(self._device)
+            self._write_pages[group] = _to_device(torch.from_numpy(pages), self._device)
         return self._write_pages[group]
 
     def decode_chunks(self, blocks_per_chunk: int, max_pages_per_chunk: int, window: int, group: int, table_host,
@@ -133,7 +143,7 @@ class StepBatch:
         if key not in self._chunks:
             ppc = decode_pages_per_chunk(self.pos0, blocks_per_chunk, max_pages_per_chunk)
             entries, most = decode_chunk_list(self.slots, self.pos0, window, ppc, table_host, ring_pages)
-            self._chunks[key] = (torch.from_numpy(with_header(entries, len(entries))).to(self._device), len(entries),
+            self._chunks[key] = (_to_device(torch.from_numpy(with_header(entries, len(entries))), self._device), len(entries),
                                  ppc, most)
         return self._chunks[key]
 

@@ -59,7 +59,14 @@ def require_device() -> None:
     _check(lib().picolm_device_check())
 
 
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+
+
 def _stream() -> c_void_p:
+    """torch's current stream on the current device (asked for at every launch: a graph is
+    recorded on a stream of its own)."""
+    if _raw_stream is not None:           # the same handle without building a Stream object
+        return c_void_p(_raw_stream(torch.cuda.current_device()))
     return c_void_p(torch.cuda.current_stream().cuda_stream)
 
 

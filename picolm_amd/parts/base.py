@@ -39,17 +39,26 @@ class Workspace:
         self.device = device
         self._bufs: dict[str, torch.Tensor] = {}
         self._flips: dict[str, int] = {}
+        self._views: dict[tuple, tuple] = {}      # (name, shape, dtype) -> (buffer, view of it)
 
     def get(self, name: str, shape, dtype: torch.dtype) -> torch.Tensor:
+        key = (name, tuple(shape), dtype)
+        hit = self._views.get(key)
+        if hit is not None and hit[0] is self._bufs.get(name):
+            return hit[1]                       # the same request as before: the same view
         n = 1
         for s in shape:
             n *= int(s)
-        nbytes = n * torch.empty((), dtype=dtype).element_size()
+        nbytes = n * dtype.itemsize
         buf = self._bufs.get(name)
         if buf is None or buf.numel() < nbytes:
             buf = torch.empty(max(nbytes, 256), dtype=torch.uint8, device=self.device)
             self._bufs[name] = buf
-        return buf[:nbytes].view(dtype).view(*shape)
+        view = buf[:nbytes].view(dtype).view(*shape)
+        if len(self._views) >= 4096:            # (a long run of steps of ever new sizes)
+            self._views.clear()
+        self._views[key] = (buf, view)
+        return view
 
     def zeros(self, name: str, shape, dtype: torch.dtype) -> torch.Tensor:
         """A buffer that is zero when first given out and that its users leave at zero (counters
@@ -57,7 +66,7 @@ class Workspace:
         n = 1
         for s in shape:
             n *= int(s)
-        nbytes = n * torch.empty((), dtype=dtype).element_size()
+        nbytes = n * dtype.itemsize
         buf = self._bufs.get(name)
         if buf is None or buf.numel() < nbytes:
             buf = torch.zeros(max(nbytes, 256), dtype=torch.uint8, device=self.device)
