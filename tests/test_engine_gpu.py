@@ -212,7 +212,7 @@ def test_greedy_generation_through_the_entry_point(dtype, folders):
     from picolm_amd.generation import generate
     d = folders["A"]
     rng = np.random.default_rng(0)
-    prompts = [tiny.random_tokens(rng, n, 256) for n in (5, 11, 17)]       # BASELINE's tiny workload: 8 greedy steps
+    prompts = [tiny.random_tokens(rng, n, 256) for n in (5, 11, 17)]       # three prompts of unequal length, 8 greedy steps
     model = load_model(d, dtype=dtype)
     got = generate(model, prompts, max_new_tokens=8, stop_ids=())
     for p, r in zip(prompts, got):
