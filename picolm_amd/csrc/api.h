@@ -119,6 +119,15 @@ int picolm_attn_decode_rope_mfma(const float* qkv, void* k_pages, void* v_pages,
 int picolm_argmax_scratch_floats(int n_rows, int V);
 int picolm_argmax(const float* logits, int32_t* out, int n_rows, int V, int64_t ld, float* scratch,
                   hipStream_t stream);
+// picolm_argmax for callers that cannot allocate device memory (code under HIP graph capture,
+// tight serving loops, harnesses that forbid it).  It has no counterpart in picolm.  The partial
+// results go to an array of picolm_argmax_static_max_floats() floats (256 KiB) that the library
+// keeps in each GPU's memory for the life of the process; 2 * n_rows * ceil(V / 4096) floats
+// beyond that are refused with an error.  It allocates and frees nothing.  All calls on one GPU
+// share that GPU's array: two calls that overlap there (different streams, or threads without an
+// order between them) race; calls queued on one stream do not.
+int picolm_argmax_static_max_floats(void);
+int picolm_argmax_static(const float* logits, int32_t* out, int n_rows, int V, int64_t ld, hipStream_t stream);
 // rng_states[state_index ? state_index[row] : row] is one xorshift64 state per sequence,
 // advanced by one draw when temperature > 0.
 // With a top_k small enough the row is cut into slices for many workgroups, which need scratch

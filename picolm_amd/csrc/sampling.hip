@@ -15,6 +15,7 @@
 // cannot change a decision in practice.
 #include "common.h"
 #include "api.h"
+#include <mutex>
 
 #define SM_THREADS 1024
 #define SM_LIST 1024
@@ -105,6 +106,54 @@ extern "C" int picolm_argmax(const float* logits, int32_t* out, int n_rows, int 
     argmax_pick_kernel<<<dim3(n_rows), dim3(ARGMAX_THREADS), 0, stream>>>(part_v, part_i, out, n_slices);
     PICOLM_LAUNCH_CHECK("argmax");
     return 0;
+}
+
+// The same two kernels over scratch memory that belongs to the library: a file-scope array in
+// device memory, PICOLM_ARGMAX_STATIC_FLOATS floats (256 KiB) that each GPU the library runs on
+// holds until the process ends.  The array's name is a host-side handle only; its address on a
+// device is asked for once per device, with that device current, and kept.
+#define PICOLM_ARGMAX_STATIC_FLOATS 65536
+#define PICOLM_MAX_DEVICES 64
+static __device__ __align__(256) float g_argmax_scratch[PICOLM_ARGMAX_STATIC_FLOATS];
+static float* g_argmax_scratch_ptr[PICOLM_MAX_DEVICES];      // per device, null until asked for
+static std::mutex g_argmax_scratch_mutex;
+
+static int argmax_static_scratch(float** out) {
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    PICOLM_REQUIRE(e == hipSuccess, "argmax_static: no current device: %s", hipGetErrorString(e));
+    PICOLM_REQUIRE(dev >= 0 && dev < PICOLM_MAX_DEVICES, "argmax_static: device %d is beyond the %d this library keeps scratch for",
+                   dev, PICOLM_MAX_DEVICES);
+    std::lock_guard<std::mutex> lock(g_argmax_scratch_mutex);
+    if (g_argmax_scratch_ptr[dev] == nullptr) {
+        void* p = nullptr;
+        e = hipGetSymbolAddress(&p, HIP_SYMBOL(g_argmax_scratch));
+        PICOLM_REQUIRE(e == hipSuccess && p != nullptr, "argmax_static: no address for the scratch array on device %d: %s", dev,
+                       hipGetErrorString(e));
+        g_argmax_scratch_ptr[dev] = (float*)p;
+    }
+    *out = g_argmax_scratch_ptr[dev];
+    return 0;
+}
+
+extern "C" int picolm_argmax_static_max_floats(void) { return PICOLM_ARGMAX_STATIC_FLOATS; }
+
+extern "C" int picolm_argmax_static(const float* logits, int32_t* out, int n_rows, int V, int64_t ld,
+                                    hipStream_t stream) {
+    PICOLM_REQUIRE(n_rows >= 0 && V > 0 && ld >= V, "argmax_static: bad sizes rows=%d V=%d ld=%lld", n_rows, V,
+                   (long long)ld);
+    PICOLM_REQUIRE(logits != nullptr && out != nullptr, "argmax_static: null logits or output");
+    PICOLM_REQUIRE(n_rows <= 65535, "argmax_static: %d rows exceed the grid", n_rows);
+    const int64_t need = 2 * (int64_t)n_rows * ceil_div(V, ARGMAX_SLICE);
+    PICOLM_REQUIRE(need <= PICOLM_ARGMAX_STATIC_FLOATS,
+                   "argmax_static: %d rows of %d logits need %lld floats of scratch, the library's array holds %d "
+                   "(picolm_argmax takes a buffer of any size)", n_rows, V, (long long)need, PICOLM_ARGMAX_STATIC_FLOATS);
+    if (n_rows == 0) return 0;
+    float* scratch = nullptr;
+    if (int rc = argmax_static_scratch(&scratch)) return rc;
+    // every entry that the second kernel reads is written by the first, so what an earlier call
+    // left in the array needs no clearing
+    return picolm_argmax(logits, out, n_rows, V, ld, scratch, stream);
 }
 
 // ---------------------------------------------------------------------------------------------
