@@ -126,6 +126,11 @@ class Cache:
 
     def reserve_many(self, slots, lengths) -> None:
         """All or nothing for a whole batch."""
+        for s, n in zip(slots, lengths):
+            if not self.slots.is_live(s):
+                raise CacheError(f"slot {s} is not live")
+            if n > self.max_seq_len:
+                raise CacheFull(f"a sequence of {n} tokens exceeds the cache's {self.max_seq_len}")
         for g in self.kv:
             need = sum(g.book.missing(s, n) for s, n in zip(slots, lengths))
             if need > g.book.pool.n_free:

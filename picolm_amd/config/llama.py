@@ -13,6 +13,9 @@ import os
 from dataclasses import dataclass, field
 
 
+MAX_HEAD_DIM = 256
+
+
 class ConfigError(ValueError):
     """A config.json that cannot describe a model; the message names the key."""
 
@@ -106,7 +109,13 @@ class LlamaConfig:
         D = integer("hidden_size")
         if H <= 0:
             raise ConfigError("num_attention_heads: must be positive")
-        head_dim = integer("head_dim", 0) or (D // H)
+        head_dim = integer("head_dim", 0)
+        if not head_dim:
+            # picolm divides without a check (picolm/safetensors.c:75-76); a width that the heads
+            # do not divide would give every head a silently smaller size
+            if D % H:
+                raise ConfigError(f"hidden_size: {D} is not divisible by num_attention_heads = {H}, and head_dim is not given")
+            head_dim = D // H
         eps = float(d.get("rms_norm_eps") or 0.0) or 1e-6          # safetensors.c:77-78
         theta = float(d.get("rope_theta") or 0.0)
         if theta <= 0.0:
@@ -161,6 +170,10 @@ class LlamaConfig:
                 f"num_attention_heads {self.num_attention_heads}")
         if self.head_dim % 2 != 0:
             raise ConfigError(f"head_dim: {self.head_dim} is odd; rotation needs pairs")
+        if self.head_dim > MAX_HEAD_DIM:
+            # picolm's bound too (picolm/model_attention.c:163); here it is what a tile of the
+            # attention kernels holds, and it is refused when the configuration is read
+            raise ConfigError(f"head_dim: {self.head_dim} exceeds {MAX_HEAD_DIM}, the largest head the attention kernels take")
         if not (self.rms_norm_eps > 0.0):
             raise ConfigError("rms_norm_eps: must be positive")
         if self.rope_style not in _ROPE_STYLES:

@@ -63,6 +63,23 @@ int picolm_gemm_linked(const void* A, const void* W, void* C, int c_dt, int M, i
                        int64_t ws_floats, const float* next_w, void* next_h, float* next_ssq, int next_parts, const float* ssq,
                        int n_parts, int norm_len, float eps, int rows, hipStream_t stream);
 
+// The product a layer asks for: picks the kernel for the operands' types and sizes (linear.hip).
+// Row-major contiguous A[M][K], W[N][K], C[M][N] (N/2 with the gated epilogue 2).  next_*: with
+// the accumulating epilogue 1, also prepare the RMSNorm that follows (next_h[M][N] bf16, next_ssq
+// [next_parts][rows] with rows = picolm_linear_norm_rows(M), next_parts =
+// picolm_linear_norm_parts(M, N, K)); ssq, n_parts, norm_len, eps: A is such a next_h.  Either
+// role needs picolm_linear_links_norms to say yes.  ws: picolm_linear_workspace_floats() floats for
+// products cut along K, or null.
+int64_t picolm_linear_workspace_floats(void);
+int picolm_linear_norm_rows(int M);
+int picolm_linear_medium_splits(int M, int N, int K);    // parts along K of a product of 17..64 rows
+int picolm_linear_norm_parts(int M, int N, int K);
+int picolm_linear_links_norms(const void* a, int a_dt, const void* w, int w_dt, int c_dt, int M, int N, int K,
+                              int epilogue, int prepares);
+int picolm_linear(const void* A, int a_dt, const void* W, int w_dt, void* C, int c_dt, int M, int N, int K, int epilogue,
+                  const float* next_w, void* next_h, float* next_ssq, int next_parts, const float* ssq, int n_parts,
+                  int norm_len, float eps, float* ws, hipStream_t stream);
+
 // Within a group's part of a page, K[64][d] and V^T[d][64] lie as plain arrays, except in bfloat16
 // pages of head size 32, 64 or 128: those are in the order of the matrix-core kernels' operands.
 // Fills k_idx[key * d + i] and v_idx[i * 64 + key] with the offsets of K[key][i] and V^T[i][key].

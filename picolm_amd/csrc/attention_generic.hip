@@ -1,5 +1,6 @@
-// Attention over the paged cache on the vector ALU, for any head size that is a multiple of
-// 16 (up to 256), any number of heads and groups, float or bf16 storage.  One kernel serves
+// Attention over the paged cache on the vector ALU, for any head size up to 256 (a size that is
+// no multiple of 16 leaves the last of a row's column groups partly empty), any number of heads
+// and groups, float or bf16 storage.  One kernel serves
 // both kinds of step: a tile is up to 16 "rows" that share one KV head.
 //   prefill: rows = consecutive new tokens of one sequence, for one query head;
 //   decode : rows = the query heads of one KV group, for a sequence's single new token,
@@ -86,7 +87,7 @@ __global__ __launch_bounds__(AT_THREADS) void attn_tile_kernel(AttnArgs a) {
     }
     // PV ownership: thread -> (row pr, column group pc), columns pc + 16*j
     const int pr = tid / 16, pc = tid % 16;
-    const int n_cg = d / 16;
+    const int n_cg = pc < d ? (d - pc + 15) / 16 : 0;      // this thread's columns pc + 16*j below d
     float acc[AT_MAX_D / 16];
 #pragma unroll
     for (int j = 0; j < AT_MAX_D / 16; ++j) acc[j] = 0.f;
@@ -266,8 +267,7 @@ int check_decode_chunks(const char* who, const float* partial, const int32_t* ch
 
 static int check_attn_sizes(const char* who, int H, int G, int d, int max_pages, int ring_pages) {
     PICOLM_REQUIRE(H > 0 && G > 0 && H % G == 0, "%s: %d heads do not split over %d groups", who, H, G);
-    PICOLM_REQUIRE(d >= 16 && d % 16 == 0 && d <= AT_MAX_D,
-                   "%s: head size %d is not a multiple of 16 in [16, %d]", who, d, AT_MAX_D);
+    PICOLM_REQUIRE(d >= 1 && d <= AT_MAX_D, "%s: head size %d is not in [1, %d]", who, d, AT_MAX_D);
     PICOLM_REQUIRE(max_pages > 0 && ring_pages > 0 && ring_pages <= max_pages,
                    "%s: bad page table geometry max_pages=%d ring_pages=%d", who, max_pages, ring_pages);
     return 0;

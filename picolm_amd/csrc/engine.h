@@ -1,0 +1,171 @@
+// The engine behind a C ABI: a cache with a slot per sequence, the step function and a generation
+// loop, for a model given as a launch program.
+//
+// picolm's counterpart is model_load / model_forward / model_forward_prefill / model_free
+// (picolm/model.h:504-551) and sampler_init / sampler_sample (picolm/sampler.h:14-16): one
+// sequence, one architecture's layer order written out in C.  Here the layer order is data.  A
+// model is a flat list of operations over named row buffers (a "program"), which the parts of a
+// model emit once (picolm_amd/parts/*.py, `emit`); the engine owns everything that changes from
+// step to step: slots and pages, the step's index arrays, the workspace, recorded decode steps.
+// Weights stay with the caller, as device pointers inside the operations.
+//
+// Every function returns 0 or a negative code and leaves a message for picolm_last_error().
+// Nothing here waits for the GPU unless it says so; work is queued on the stream that is passed
+// in, and all calls on one engine must use one stream (or be ordered by the caller).  An engine is
+// used by one thread at a time.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+// return codes beside -1 (bad argument) and -2 (a launch failed)
+#define PICOLM_ERR_STEP (-10)        // a step that cannot run: a dead slot, a token outside the vocabulary
+#define PICOLM_ERR_CACHE_FULL (-11)  // no free slot or page, or a sequence longer than the cache takes
+#define PICOLM_ERR_CACHE (-12)       // a slot freed twice, a slot that does not exist
+#define PICOLM_ERR_DEVICE (-13)      // the HIP runtime refused something
+
+enum { PICOLM_OP_EMBED = 1, PICOLM_OP_RMSNORM = 2, PICOLM_OP_LINEAR = 3, PICOLM_OP_ATTENTION = 4 };
+// which rows of the step an operation covers: every new token's, or only those whose logits are wanted
+enum { PICOLM_ROWS_STEP = 0, PICOLM_ROWS_WANTED = 1 };
+
+// A row buffer of the workspace: `row_bytes` bytes for each of the step's rows of that kind.
+typedef struct {
+    int32_t row_bytes;
+    int32_t rows;            // PICOLM_ROWS_STEP or PICOLM_ROWS_WANTED
+    int32_t dtype;           // PICOLM_F32 (0) or PICOLM_BF16 (1)
+} picolm_buffer;
+
+// One operation.  Buffers are indices into the program's buffers.  Fields an operation does not
+// use are zero.
+//   EMBED      out[t] = weight[tokens[t]] widened to float          weight [n][k] of weight_dt
+//   RMSNORM    out = in / sqrt(mean(in^2) + eps) * weight           weight float [k]; in float
+//   LINEAR     out (=, +=, = silu-gated) in weight^T                weight [n][k]; epilogue 0, 1, 2
+//              in_norm_weight: `in` is scratch and the input is rmsnorm(in_norm_x) with that weight
+//              and in_norm_eps; the engine either runs the norm into `in` or, where the kernels
+//              can, lets the product before and this one compute it between them.
+//              out_norm_weight (epilogue 1): the rmsnorm that meets `out` next, so that this
+//              product can prepare it; out_norm_when = 1: only in steps that want every row.
+//   ATTENTION  in: float rows [(H + 2G) d] of q, k, v; rotates q and k (cos_table, sin_table
+//              [table_positions][d/2], null for none; rope_style 0 pairs (2i, 2i+1), 1 pairs
+//              (i, i + d/2)), writes k and v to cache entry (kv_group, kv_entry) unless
+//              kv_writes = 0, attends over the cache; out [H d]; q_buffer: scratch [H d].
+typedef struct {
+    int32_t kind, rows;
+    int32_t in, out;
+    const void* weight;
+    int32_t weight_dt, n, k, epilogue;
+    float eps;
+    const float* in_norm_weight;
+    float in_norm_eps;
+    int32_t in_norm_x;
+    const float* out_norm_weight;
+    float out_norm_eps;
+    int32_t out_norm_when;
+    int32_t n_heads, n_kv_heads, head_dim, window;
+    float scale;
+    const float* cos_table;
+    const float* sin_table;
+    int32_t rope_style, table_positions;
+    int32_t kv_group, kv_entry, kv_writes, q_buffer;
+} picolm_op;
+
+// Keys and values of `n_entries` layer calls that need the same kind of cache.
+typedef struct {
+    int32_t n_entries, n_kv_heads, head_dim, window;
+} picolm_kv_group;
+
+// Fixed-size state per sequence for `n_entries` layer calls, zeroed when a slot is given out.
+typedef struct {
+    int32_t n_entries;
+    int64_t bytes_per_slot;
+} picolm_state_group;
+
+typedef struct {
+    int32_t dtype;           // PICOLM_BF16: serving precision; PICOLM_F32: true 32-bit
+    int32_t vocab_size;
+    const picolm_op* ops;
+    int32_t n_ops;
+    const picolm_buffer* buffers;
+    int32_t n_buffers;
+    int32_t logits_buffer;   // float rows [vocab_size], PICOLM_ROWS_WANTED
+    const picolm_kv_group* kv_groups;
+    int32_t n_kv_groups;
+    const picolm_state_group* state_groups;
+    int32_t n_state_groups;
+} picolm_program;
+
+#define PICOLM_ENGINE_NO_GRAPHS 1    // launch every decode step's kernels one by one
+#define PICOLM_ENGINE_HOST_ONLY 2    // books and index arrays only, no device memory: steps plan but do not run
+
+typedef struct picolm_engine picolm_engine;
+
+// max_tokens: the most tokens live sequences hold together, each sequence's count rounded up to
+// pages of 64; max_seq_len: the longest one sequence may get; n_slots: 0 gives one per page.
+// The program is copied; the weights and tables it points to must outlive the engine.
+int picolm_engine_create(const picolm_program* program, int64_t max_tokens, int32_t max_seq_len, int32_t n_slots,
+                         int32_t flags, picolm_engine** out);
+void picolm_engine_destroy(picolm_engine* e);
+
+int picolm_engine_slot_alloc(picolm_engine* e, int32_t* slot, hipStream_t stream);
+int picolm_engine_slot_free(picolm_engine* e, int32_t slot);
+int picolm_engine_slot_length(picolm_engine* e, int32_t slot);      // tokens the slot holds, negative: not live
+
+// One step.  Sequence i lives in slots[i] and brings n_new[i] >= 1 tokens, packed in `tokens`
+// (host memory) in the order of the sequences; they are appended at the slot's length.  The
+// sequences of a step either all bring prompts (any lengths) or one token each.  want_counts[i]
+// indices into sequence i's new tokens are listed, packed, in `want`; want_counts null: each
+// sequence's last token.  *logits: float [*n_rows][vocab] in device memory that the engine owns,
+// valid until the next step of this engine, in the order of the sequences and of `want`.  A
+// refused step (PICOLM_ERR_STEP, PICOLM_ERR_CACHE_FULL) leaves every sequence where it was.
+int picolm_engine_step(picolm_engine* e, int32_t n_seq, const int32_t* slots, const int32_t* n_new,
+                       const int32_t* tokens, const int32_t* want_counts, const int32_t* want, float** logits,
+                       int32_t* n_rows, hipStream_t stream);
+// One more token for each sequence, the tokens lying in device memory (what a sampling kernel
+// wrote, or will have written when the step runs); they must lie inside the vocabulary.
+int picolm_engine_step_device_tokens(picolm_engine* e, int32_t n_seq, const int32_t* slots, const int32_t* tokens_dev,
+                                     float** logits, hipStream_t stream);
+
+// Sampling options with picolm's meanings (picolm/sampler.h:6-12): temperature <= 0 is greedy,
+// top_k 0 is off, top_p 1 and min_p 0 are off, seed 0 becomes 42.
+typedef struct {
+    float temperature;
+    int32_t top_k;
+    float top_p, min_p;
+    uint64_t seed;
+} picolm_sampling;
+
+// The generation loop (picolm/picolm.c:1502-1610) over batches of unequal prompts: prompts of a
+// batch in one step, then one token each; a sequence ends with a stop token (recorded), after
+// max_new tokens, or at the cache's capacity, leaves the batch and gives its slot back; batches of
+// up to batch_size requests follow each other until all are done.  prompts: packed token ids,
+// prompt_lens[i] >= 1 each.  out_tokens: [n_prompts][max_new]; out_counts[i] tokens were made;
+// out_finish[i]: 1 stop token, 2 length, 3 capacity.  It waits for the GPU once a step.
+int picolm_engine_generate(picolm_engine* e, int32_t n_prompts, const int32_t* prompts, const int32_t* prompt_lens,
+                           int32_t max_new, const picolm_sampling* sampling, const int32_t* stop_ids, int32_t n_stop,
+                           int32_t batch_size, int32_t* out_tokens, int32_t* out_counts, int32_t* out_finish,
+                           hipStream_t stream);
+
+// ---- what the engine holds, for bindings and tests ---------------------------------------------
+// what: 0 max_seq_len, 1 n_slots, 2 free slots, 3 free tokens (pages free in the tightest group
+// times 64), 4 recorded decode steps, 5 pages of a sequence's table row, 6 bytes of device memory
+// held, 7 the counter that moves when a slot or page changes hands
+int64_t picolm_engine_info(picolm_engine* e, int32_t what);
+// keys [n_pages][G][64][d] and values [n_pages][G][d][64] of one cache entry (device memory)
+int picolm_engine_kv_entry(picolm_engine* e, int32_t group, int32_t entry, void** k, void** v, int64_t* n_pages);
+// state [n_slots][bytes_per_slot] of one entry (device memory)
+int picolm_engine_state_entry(picolm_engine* e, int32_t group, int32_t entry, void** state, int64_t* bytes_per_slot);
+// the pages a slot holds in a group, in logical order; returns their number (negative: error)
+int picolm_engine_slot_pages(picolm_engine* e, int32_t group, int32_t slot, int32_t* pages, int32_t capacity);
+int picolm_engine_free_pages(picolm_engine* e, int32_t group);
+// One of the index arrays of the step planned last, by name, from the host's copy: "seq_slot",
+// "seq_pos0", "seq_nnew", "cu_seqlens", "tok_pos", "tok_seq", "tokens", "want_rows",
+// "write_pages.<group>", "chunks.<group>" (the decode work list with its header),
+// "tiles.<rows>.seq", "tiles.<rows>.q0".  Returns the number of ints (negative: no such array).
+int picolm_engine_step_array(picolm_engine* e, const char* name, int32_t* out, int32_t capacity);
+
+#ifdef __cplusplus
+}
+#endif

@@ -114,7 +114,7 @@ class DecoderModel:
         kernels.require_device()
         check_specs(source, self.tensor_specs())
         self.runtime = runtime
-        fetch = WeightFetcher(source, runtime.device)
+        fetch = WeightFetcher(source, runtime.device, runtime.dtype)
         for p in self.parts():
             p.load_all(fetch, runtime)
         return self
@@ -126,6 +126,38 @@ class DecoderModel:
         for b in self.blocks:
             b.mixer.prepare(self.runtime, cache.max_seq_len)
         return cache
+
+    # -- the model as a launch program --------------------------------------------------------
+    def program(self):
+        """The model as the flat list of operations that the engine in the library walks
+        (engine/program.py), or None when a part has no such operations: then `step` below runs
+        it part by part.  The mixers must have been prepared (`new_cache` does that) for the
+        positions the engine will see."""
+        from .program import CannotEmit, ProgramBuilder
+        if self.runtime is None:
+            raise StepError("the model has no weights loaded")
+        b = ProgramBuilder(self.runtime.dtype)
+        try:
+            for part in (self.embedding, self.head, *self.blocks):
+                if not callable(getattr(part, "emit", None)):
+                    raise CannotEmit(f"{type(part).__name__} has no operations of the engine's")
+            final = self.final_norm.norm_ref() if hasattr(self.final_norm, "norm_ref") else None
+            if final is None:
+                raise CannotEmit(f"{type(self.final_norm).__name__} has no operations of the engine's")
+            x = self.embedding.emit(b)
+            for i, (call, binding) in enumerate(zip(self.order, self.bindings)):
+                b.binding = binding
+                if i + 1 < len(self.order):
+                    nxt = getattr(self.blocks[self.order[i + 1].block], "first_norm", lambda: None)()
+                    after = nxt.norm_ref() if nxt is not None and hasattr(nxt, "norm_ref") else None
+                    self.blocks[call.block].emit(b, x, after, 0)
+                else:       # the final norm meets every row only in steps that want every row's logits
+                    self.blocks[call.block].emit(b, x, final, 1)
+            b.binding = None
+            self.head.emit(b, final, x)
+        except CannotEmit:
+            return None
+        return b.finish(self.head.V, self.cache_spec)
 
     # -- the step ---------------------------------------------------------------------------
     def step(self, cache: Cache, batch: StepBatch, workspace: Workspace) -> torch.Tensor:

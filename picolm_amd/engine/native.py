@@ -1,0 +1,251 @@
+"""The Python face of the engine in libpicolm_hip.so (csrc/engine.h): a launch program goes in,
+slots, steps and generation come out as single calls.  Everything a step needs lives in the
+library (the books of the cache, the step's index arrays, the workspace, recorded decode steps);
+this file only converts arguments and wraps the memory the library hands back as tensors.
+"""
+from __future__ import annotations
+
+import ctypes
+from ctypes import byref, c_int32, c_int64, c_void_p
+
+import numpy as np
+import torch
+
+from .. import kernels
+from ..cache.slots import CacheError, CacheFull
+from . import program as P
+from .batch import StepError
+
+_declared = False
+
+
+def _lib():
+    global _declared
+    lib = kernels.lib()
+    if not _declared:
+        P.declare(lib)
+        _declared = True
+    return lib
+
+
+def _raise(rc: int):
+    msg = kernels.lib().picolm_last_error().decode("utf-8", "replace")
+    if rc == P.ERR_STEP:
+        raise StepError(msg)
+    if rc == P.ERR_CACHE_FULL:
+        raise CacheFull(msg)
+    if rc == P.ERR_CACHE:
+        raise CacheError(msg)
+    raise kernels.KernelError(msg)
+
+
+class _DeviceMemory:
+    """Memory that the library owns, for torch to look at (never to free)."""
+
+    def __init__(self, ptr: int, nbytes: int):
+        self.__cuda_array_interface__ = {"shape": (nbytes,), "typestr": "|u1", "data": (ptr, False), "version": 2}
+
+
+def device_view(ptr: int, shape, dtype: torch.dtype, device) -> torch.Tensor:
+    n = dtype.itemsize
+    for s in shape:
+        n *= int(s)
+    if n == 0 or not ptr:
+        return torch.empty(tuple(shape), dtype=dtype, device=device)
+    return torch.as_tensor(_DeviceMemory(ptr, n), device=device).view(dtype).view(*shape)
+
+
+def _i32(values) -> np.ndarray:
+    return np.ascontiguousarray(values, dtype=np.int32)
+
+
+class _SlotCount:
+    def __init__(self, engine):
+        self._e = engine
+        self.n_slots = engine.info(1)
+
+    @property
+    def n_free(self) -> int:
+        return self._e.info(2)
+
+    def is_live(self, slot: int) -> bool:
+        return self._e.length(slot) >= 0
+
+
+class _KVEntries:
+    """keys [entry][page][G][64][d] and values [entry][page][G][d][64] of one cache group, as the
+    library keeps them."""
+
+    def __init__(self, engine, group: int, spec, dtype, device):
+        k, v, n = c_void_p(), c_void_p(), c_int64()
+        rc = _lib().picolm_engine_kv_entry(engine.handle, group, 0, byref(k), byref(v), byref(n))
+        if rc:
+            _raise(rc)
+        G, d = spec.n_kv_heads, spec.head_dim
+        self.spec = spec
+        self.k = device_view(k.value, (spec.n_entries, n.value, G, kernels.PAGE_TOKENS, d), dtype, device)
+        self.v = device_view(v.value, (spec.n_entries, n.value, G, d, kernels.PAGE_TOKENS), dtype, device)
+
+
+class EngineCache:
+    """What generation and the tests ask of a cache, answered by the library's books."""
+
+    def __init__(self, engine, cache_spec, dtype, device):
+        self._e = engine
+        self.spec = cache_spec
+        self.dtype = dtype
+        self.device = torch.device(device)
+        self.max_seq_len = engine.info(0)
+        self.n_slots = engine.info(1)
+        self.max_pages = engine.info(5)
+        self.slots = _SlotCount(engine)
+        self.kv = [_KVEntries(engine, gi, g, dtype, device) for gi, g in enumerate(cache_spec.kv_groups)]
+
+    def length(self, slot: int) -> int:
+        return max(self._e.length(slot), 0)
+
+    def free_tokens(self) -> int:
+        return self._e.info(3)
+
+    def bytes(self) -> int:
+        return self._e.info(6)
+
+    @property
+    def version(self) -> int:
+        return self._e.info(7)
+
+
+class NativeEngine:
+    def __init__(self, built: P.BuiltProgram, max_tokens: int, max_seq_len: int, n_slots: int | None, device,
+                 graphs: bool = True, host_only: bool = False):
+        self.program = built                      # keeps the weights and tables alive
+        self.device = torch.device(device)
+        self.vocab_size = built.struct.vocab_size
+        flags = (0 if graphs else P.ENGINE_NO_GRAPHS) | (P.ENGINE_HOST_ONLY if host_only else 0)
+        h = c_void_p()
+        rc = _lib().picolm_engine_create(byref(built.struct), int(max_tokens), int(max_seq_len), int(n_slots or 0), flags,
+                                         byref(h))
+        if rc:
+            _raise(rc)
+        self.handle = h
+        self.host_only = host_only
+        self._views: dict = {}
+
+    def _stream(self):
+        return None if self.host_only else kernels._stream()
+
+    def close(self) -> None:
+        if getattr(self, "handle", None):
+            _lib().picolm_engine_destroy(self.handle)
+            self.handle = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+    # -- books -----------------------------------------------------------------------------
+    def info(self, what: int) -> int:
+        return int(_lib().picolm_engine_info(self.handle, what))
+
+    def slot_alloc(self) -> int:
+        s = c_int32()
+        rc = _lib().picolm_engine_slot_alloc(self.handle, byref(s), self._stream())
+        if rc:
+            _raise(rc)
+        return s.value
+
+    def slot_free(self, slot: int) -> None:
+        rc = _lib().picolm_engine_slot_free(self.handle, int(slot))
+        if rc:
+            _raise(rc)
+
+    def length(self, slot: int) -> int:
+        return _lib().picolm_engine_slot_length(self.handle, int(slot))
+
+    def slot_pages(self, group: int, slot: int) -> list[int]:
+        out = np.zeros(max(self.info(5), 1), dtype=np.int32)
+        n = _lib().picolm_engine_slot_pages(self.handle, group, slot, out.ctypes.data, len(out))
+        if n < 0:
+            _raise(n)
+        return out[:n].tolist()
+
+    def free_pages(self, group: int) -> int:
+        return _lib().picolm_engine_free_pages(self.handle, group)
+
+    def recorded_steps(self) -> int:
+        return self.info(4)
+
+    def step_array(self, name: str) -> np.ndarray:
+        n = _lib().picolm_engine_step_array(self.handle, name.encode(), None, 0)
+        if n < 0:
+            _raise(n)
+        out = np.zeros(max(n, 1), dtype=np.int32)
+        _lib().picolm_engine_step_array(self.handle, name.encode(), out.ctypes.data, n)
+        return out[:n]
+
+    # -- steps -----------------------------------------------------------------------------
+    def _logits(self, ptr, rows: int) -> torch.Tensor:
+        key = (ptr, rows)
+        t = self._views.get(key)
+        if t is None:
+            if len(self._views) >= 256:
+                self._views.clear()
+            t = self._views[key] = device_view(ptr, (rows, self.vocab_size), torch.float32, self.device)
+        return t
+
+    def step(self, slots, new_tokens, want=None) -> torch.Tensor | None:
+        """As Session.step; None from an engine without device memory."""
+        n = len(slots)
+        if not (len(new_tokens) == n and (want is None or len(want) == n)):
+            raise StepError("slots, tokens and wanted rows differ in length")
+        if n == 0:
+            raise StepError("a step needs at least one sequence")
+        n_new = _i32([len(t) for t in new_tokens])
+        flat = np.concatenate([np.asarray(t, dtype=np.int64).reshape(-1) for t in new_tokens]) if n_new.sum() else np.zeros(0, np.int64)
+        if flat.size and (flat.min() < 0 or flat.max() >= self.vocab_size):
+            bad = int(flat[(flat < 0) | (flat >= self.vocab_size)][0])
+            raise StepError(f"token id {bad} is outside the vocabulary of {self.vocab_size}")
+        tokens = _i32(flat)
+        sl = _i32(list(slots))
+        counts = idx = None
+        if want is not None:
+            counts = _i32([len(w) for w in want])
+            idx = _i32([j for w in want for j in w]) if counts.sum() else np.zeros(1, np.int32)
+        logits, rows = c_void_p(), c_int32()
+        rc = _lib().picolm_engine_step(self.handle, n, sl.ctypes.data, n_new.ctypes.data, tokens.ctypes.data,
+                                       counts.ctypes.data if counts is not None else None,
+                                       idx.ctypes.data if idx is not None else None, byref(logits), byref(rows), self._stream())
+        if rc:
+            _raise(rc)
+        if not logits.value:
+            return None if rows.value else torch.empty((0, self.vocab_size), dtype=torch.float32, device=self.device)
+        return self._logits(logits.value, rows.value)
+
+    def step_device_tokens(self, slots, tokens: torch.Tensor) -> torch.Tensor:
+        sl = _i32(list(slots))
+        logits = c_void_p()
+        rc = _lib().picolm_engine_step_device_tokens(self.handle, len(sl), sl.ctypes.data, tokens.data_ptr(), byref(logits),
+                                                     kernels._stream())
+        if rc:
+            _raise(rc)
+        return self._logits(logits.value, len(sl))
+
+    def generate(self, prompts, max_new_tokens: int, params, stop_ids=(), batch_size: int = 64):
+        """The library's own generation loop; returns (tokens of each request, finish reasons)."""
+        n = len(prompts)
+        lens = _i32([len(p) for p in prompts])
+        flat = _i32(np.concatenate([np.asarray(p, dtype=np.int64) for p in prompts])) if n and lens.sum() else np.zeros(1, np.int32)
+        stops = _i32(list(stop_ids)) if len(stop_ids) else np.zeros(1, np.int32)
+        out = np.zeros((max(n, 1), max(max_new_tokens, 1)), dtype=np.int32)
+        counts = np.zeros(max(n, 1), dtype=np.int32)
+        finish = np.zeros(max(n, 1), dtype=np.int32)
+        sp = P.Sampling(params.temperature, params.top_k, params.top_p, params.min_p, int(params.seed) & ((1 << 64) - 1))
+        rc = _lib().picolm_engine_generate(self.handle, n, flat.ctypes.data, lens.ctypes.data, int(max_new_tokens), byref(sp),
+                                           stops.ctypes.data, len(stop_ids), int(batch_size), out.ctypes.data, counts.ctypes.data,
+                                           finish.ctypes.data, kernels._stream())
+        if rc:
+            _raise(rc)
+        reasons = {0: "", 1: "stop", 2: "length", 3: "capacity"}
+        return [out[i, :counts[i]].tolist() for i in range(n)], [reasons[int(f)] for f in finish[:n]]

@@ -3,6 +3,12 @@
 `begin` gives each new sequence a slot, `step` runs a batch of them from the cache and
 returns logits at the wanted rows, `release` gives slots and pages back.  A step never
 runs tokens it was not given: the prompt once, then one token each.
+
+A model whose parts all emit operations of a launch program (`DecoderModel.program`) is stepped
+by the engine in the library: the cache's books, the step's index arrays, the workspace and the
+recorded decode steps live there, and a step is one call (picolm's model_forward and
+model_forward_prefill are such calls too, picolm/model.h:538-539).  A model with a part that
+only has a Python `forward` is stepped part by part from here, with the same kernels.
 """
 from __future__ import annotations
 
@@ -56,13 +62,30 @@ class _DecodeGraph:
 
 class Session:
     def __init__(self, model: DecoderModel, max_tokens: int, max_seq_len: int | None = None,
-                 n_slots: int | None = None, graphs: bool = True):
+                 n_slots: int | None = None, graphs: bool = True, native: bool | None = None):
+        """`native`: None steps in the library when the model's parts allow it, False steps from
+        Python part by part, True insists on the library."""
         if model.runtime is None:
             raise StepError("the model has no weights loaded")
         self.model = model
+        self.vocab_size = model.head.V
+        self.engine = None
+        if native is not False:
+            limit = getattr(model.config, "max_position_embeddings", None) or max_tokens
+            seq_len = min(max_seq_len or limit, limit)
+            for b in model.blocks:          # tables for every position the cache can hold
+                b.mixer.prepare(model.runtime, min(seq_len, (max_tokens + PAGE_TOKENS - 1) // PAGE_TOKENS * PAGE_TOKENS))
+            built = model.program()
+            if built is not None:
+                from .native import EngineCache, NativeEngine
+                self.engine = NativeEngine(built, max_tokens, seq_len, n_slots, model.runtime.device, graphs=graphs)
+                self.cache = EngineCache(self.engine, model.cache_spec, model.runtime.dtype, model.runtime.device)
+                self.graphs = graphs
+                return
+            if native:
+                raise StepError("a part of this model has no operations of the engine's; it is stepped from Python")
         self.cache: Cache = model.new_cache(max_tokens, max_seq_len, n_slots)
         self.workspace = Workspace(model.runtime.device)
-        self.vocab_size = model.head.V
         # decode steps replay recorded HIP graphs when every part's launches depend on device
         # memory only (a part says so with `graph_safe`)
         self.graphs = graphs and model.graph_safe()
@@ -72,19 +95,26 @@ class Session:
     # -- slots -------------------------------------------------------------------------------
     def begin(self, n: int = 1) -> list[int]:
         """Slots for `n` new sequences; on failure none is kept."""
+        alloc = self.engine.slot_alloc if self.engine is not None else self.cache.alloc_slot
         got = []
         try:
             for _ in range(n):
-                got.append(self.cache.alloc_slot())
+                got.append(alloc())
         except CacheFull:
-            for s in got:
-                self.cache.free_slot(s)
+            self.release(got)
             raise
         return got
 
     def release(self, slots) -> None:
+        free = self.engine.slot_free if self.engine is not None else self.cache.free_slot
         for s in slots:
-            self.cache.free_slot(s)
+            free(s)
+
+    def recorded_steps(self) -> int:
+        """Decode steps (by batch size and chunking) that replay a recorded HIP graph."""
+        if self.engine is not None:
+            return self.engine.recorded_steps()
+        return sum(g.graph is not None for g in self._decode_graphs.values())
 
     def length(self, slot: int) -> int:
         return self.cache.length(slot)
@@ -97,6 +127,8 @@ class Session:
         sequences and of `want`; the tensor is workspace memory, valid until the next step.
         """
         slots = list(slots)
+        if self.engine is not None:
+            return self.engine.step(slots, new_tokens, want)
         for s in slots:
             if not self.cache.slots.is_live(s):
                 raise StepError(f"slot {s} is not live")
@@ -121,13 +153,15 @@ class Session:
         that produces its tokens still runs.  The tokens must lie inside the vocabulary (a
         sampler's do); logits as from `step`, one row a sequence."""
         slots = list(slots)
-        for s in slots:
-            if not self.cache.slots.is_live(s):
-                raise StepError(f"slot {s} is not live")
         device = torch.device(self.model.runtime.device)
         if tokens.dtype != torch.int32 or tokens.shape != (len(slots),) or tokens.device.type != device.type:
             raise StepError(f"tokens on the device: expected int32 [{len(slots)}] on {device}, "
                             f"got {tokens.dtype} {tuple(tokens.shape)} on {tokens.device}")
+        if self.engine is not None:
+            return self.engine.step_device_tokens(slots, tokens.contiguous())
+        for s in slots:
+            if not self.cache.slots.is_live(s):
+                raise StepError(f"slot {s} is not live")
         if not (self.graphs and slots):
             return self.step(slots, [[t] for t in tokens.tolist()])
         return self._decode_step(slots, [self.cache.length(s) for s in slots], None, tokens)

@@ -44,7 +44,9 @@ def dir_entry_points():
             "picolm_attn_prefill_tile_rows", "picolm_attn_prefill_generic",
             "picolm_attn_decode_generic", "picolm_argmax", "picolm_argmax_scratch_floats", "picolm_sample", "picolm_sample_scratch_bytes", "picolm_gemm_skinny", "picolm_gemm_tiled", "picolm_gemm_tiled_splitk", "picolm_gemm_linked", "picolm_gemm_tiled_norm_parts", "picolm_kv_page_order",
             "picolm_attn_mfma_takes", "picolm_attn_prefill_mfma_heads", "picolm_attn_prefill_mfma_tile_tokens",
-            "picolm_attn_prefill_mfma", "picolm_attn_decode_mfma", "picolm_attn_decode_rope_mfma", "picolm_attn_decode_mfma_waves", "picolm_read_probe", "picolm_mfma_probe"]
+            "picolm_attn_prefill_mfma", "picolm_attn_decode_mfma", "picolm_attn_decode_rope_mfma", "picolm_attn_decode_mfma_waves", "picolm_read_probe", "picolm_mfma_probe",
+            "picolm_linear", "picolm_linear_norm_rows", "picolm_linear_norm_parts", "picolm_linear_links_norms",
+            "picolm_linear_medium_splits", "picolm_argmax_static", "picolm_argmax_static_max_floats"]
 
 
 def _check(rc: int) -> None:
@@ -361,76 +363,40 @@ def gemm_tiled_splitk(a, w, c, epilogue: int, variant: int, splits: int) -> None
                                           c_int64(c.shape[1]), epilogue, variant, splits, _ptr(ws), _stream()))
 
 
-def mfma_gemm_takes(a, w, c, epilogue: int) -> bool:
-    """Whether the matrix-core kernels accept these operands; otherwise the float kernel runs."""
-    if a.dtype != torch.bfloat16 or w.dtype != torch.bfloat16:
-        return False
-    if a.shape[1] % 8 != 0 or a.data_ptr() % 16 or w.data_ptr() % 16:
-        return False
-    if epilogue == EPI_STORE:
-        return True
-    if epilogue == EPI_ACCUMULATE:
-        return c.dtype == torch.float32
-    return True
-
-
-def medium_gemm_variant(M: int) -> int:
-    """The tile variant for a decode batch of 17 to 64 rows: tiles of 128 weight rows by 64
-    activation rows, or by 32 where that is enough (measured 5 to 9 % faster there)."""
-    return 13 if M <= 32 else 12
-
-
 def medium_gemm_splits(M: int, N: int, K: int) -> int:
     """Into how many parts along K a product of 17..64 rows is cut: its tiles hold 128 weight
     rows each, and every CU should have one."""
-    tiles = (N + 127) // 128
-    if tiles >= 200 or N % 4:
-        return 1
-    s = 8
-    while s > 1 and (tiles * s > 320 or K % (64 * s) or s * M * N > SPLITK_WS_FLOATS):
-        s //= 2
-    return s
+    return lib().picolm_linear_medium_splits(M, N, K)
 
 
 def linked_norm_rows(M: int) -> int:
     """Rows that the partial sums of a split norm are kept for in a step of M rows: 16 or 64 in
     a decode step, every row (in whole 64s) otherwise."""
-    return 16 if M <= 16 else 64 if M <= 64 else (M + 63) // 64 * 64
+    return lib().picolm_linear_norm_rows(M)
 
 
 def linked_norm_parts(M: int, N: int, K: int) -> int:
     """Partial sums per row that a product of M rows, N output columns and K input columns leaves
     for the norm that follows: one per workgroup (or column of tiles) of the kernel that finishes
     the rows.  0: that kernel cannot."""
-    if M <= 16:
-        return (N + 15) // 16
-    if M <= 64:
-        return N // 1024
-    return lib().picolm_gemm_tiled_norm_parts(M, N, K, c_int64(SPLITK_WS_FLOATS))
+    return lib().picolm_linear_norm_parts(M, N, K)
 
 
 def gemm_links_norms(a, w, c, epilogue: int, prepares: bool) -> bool:
     """Whether the product for these operands can take part in a norm split between two products:
     prepare the next one (with the accumulating epilogue), or else take a prepared one's
-    statistics.  Up to 16 rows every matrix-core product can do both.  For 17 to 64 rows the
-    kernel that adds the parts of a product cut along K does either for N in multiples of 1024,
-    and the tile kernel of an uncut product can take the statistics.  Above that the tile kernels
-    whose tiles go straight into LDS (K in multiples of 64) do both."""
-    if a.dim() != 2 or not mfma_gemm_takes(a, w, c, epilogue):
+    statistics.  The library decides (picolm_linear_links_norms): it depends on the operands'
+    types and on which kernel their sizes get."""
+    if a.dim() != 2 or a.dtype not in _DT or w.dtype not in _DT or c.dtype not in _DT:
         return False
-    M, N, K = a.shape[0], w.shape[0], a.shape[1]
-    if M <= 16:
-        return True
-    if K % 64:
-        return False
-    if M > 64:
-        return linked_norm_parts(M, N, K) > 0
-    cut = medium_gemm_splits(M, N, K) > 1
-    return (cut and N % 1024 == 0) if prepares else (not cut or N % 1024 == 0)
+    return bool(lib().picolm_linear_links_norms(_ptr(a), dt_of(a), _ptr(w), dt_of(w), dt_of(c), a.shape[0], w.shape[0],
+                                                a.shape[1], epilogue, int(prepares)))
 
 
 def gemm_linked(a, w, c, epilogue: int, prepare=None, prepared=None) -> None:
-    """The product of a decode step next to an RMSNorm that is split between two products.
+    """c (=, +=, = silu-gated) a @ w.T through the kernel that the library picks for the operands'
+    types and sizes (picolm_linear), optionally next to an RMSNorm that is split between two
+    products.
 
     prepare = (norm weights f32 [N], h_out bf16 [M, N], ssq_out f32 [parts, rows]): with the
     accumulating epilogue, also leave h_out = bf16(c * weights) and the partial sums of c^2.
@@ -438,64 +404,32 @@ def gemm_linked(a, w, c, epilogue: int, prepare=None, prepared=None) -> None:
     sums are multiplied by 1 / sqrt(sum(x^2) / length + eps).  rows and parts as
     linked_norm_rows / linked_norm_parts say for the step's M."""
     M, N, K = _gemm_shapes(a, w, c, epilogue)
-    for role, prepares in ((prepare, True), (prepared, False)):
-        if role is not None and not gemm_links_norms(a, w, c, epilogue, prepares):
-            raise KernelError(f"gemm_linked: a {tuple(a.shape)} {a.dtype}, w {tuple(w.shape)} {w.dtype} cannot "
-                              f"{'prepare a norm' if prepares else 'take a prepared norm'}")
     rows = linked_norm_rows(M)
     nw = nh = nssq = ssq = None
     next_parts = n_parts = norm_len = 0
     eps = 0.0
     if prepare is not None:
         nw, nh, nssq = prepare
-        if epilogue != EPI_ACCUMULATE:
-            raise KernelError("gemm_linked: only the accumulating epilogue prepares a norm")
         _dev("gemm_linked.norm_weight", nw, torch.float32, 1)
         _dev("gemm_linked.h_out", nh, torch.bfloat16, 2)
         _dev("gemm_linked.ssq_out", nssq, torch.float32, 2)
         next_parts = nssq.shape[0]
-        if nw.numel() != N or tuple(nh.shape) != (M, N) or nssq.shape[1] != rows or next_parts != linked_norm_parts(M, N, K):
+        if nw.numel() != N or tuple(nh.shape) != (M, N) or nssq.shape[1] != rows:
             raise KernelError("gemm_linked: the buffers for the next norm do not fit the product")
     if prepared is not None:
         ssq, norm_len, eps = prepared
         _dev("gemm_linked.ssq", ssq, torch.float32, 2)
         n_parts = ssq.shape[0]
-        if ssq.shape[1] != rows or norm_len != K:
+        if ssq.shape[1] != rows:
             raise KernelError("gemm_linked: the statistics are not those of this product's input rows")
-    tiled, variant, splits, ws = 0, 0, 1, None
-    if M > 64:
-        tiled = 1                       # the tile variant by shape, cut along K where it has few tiles
-        ws = splitk_workspace(a.device)
-    elif M > 16:
-        tiled, variant, splits = 1, medium_gemm_variant(M), medium_gemm_splits(M, N, K)          # as in gemm()
-        ws = splitk_workspace(a.device) if splits > 1 else None
-    elif prepare is None and M > 4 and K % 64 == 0 and 16384 <= N <= 128 * 256:
-        tiled, variant = 1, 13          # as in gemm()
-    _check(lib().picolm_gemm_linked(_ptr(a), _ptr(w), _ptr(c), dt_of(c), M, N, K, c_int64(K), c_int64(K),
-                                    c_int64(c.shape[1]), epilogue, tiled, variant, splits, _ptr(ws),
-                                    c_int64(SPLITK_WS_FLOATS),
-                                    _ptr(nw), _ptr(nh), _ptr(nssq), next_parts,
-                                    _ptr(ssq), n_parts, int(norm_len), c_float(eps), rows, _stream()))
+    _check(lib().picolm_linear(_ptr(a), dt_of(a), _ptr(w), dt_of(w), _ptr(c), dt_of(c), M, N, K, epilogue,
+                               _ptr(nw), _ptr(nh), _ptr(nssq), next_parts, _ptr(ssq), n_parts, int(norm_len), c_float(eps),
+                               _ptr(splitk_workspace(a.device)), _stream()))
 
 
 def gemm(a: torch.Tensor, w: torch.Tensor, c: torch.Tensor, epilogue: int = EPI_STORE) -> None:
-    """The product the engine calls: picks the kernel for the operands' types and sizes."""
-    if mfma_gemm_takes(a, w, c, epilogue):
-        M, N, K = a.shape[0], w.shape[0], a.shape[1]
-        if M > SKINNY_MAX_M:
-            gemm_linked(a, w, c, epilogue)          # (no norm around it: the tiled product, cut along K if short)
-        elif M > 16 and K % 64 == 0:
-            # a decode batch too wide to re-read its activations for every 16 weight rows: tiles
-            # of 128 weight rows through LDS, cut along K where there are few of them
-            gemm_tiled_splitk(a, w, c, epilogue, medium_gemm_variant(M), medium_gemm_splits(M, N, K))
-        elif M > 4 and K % 64 == 0 and 16384 <= N <= 128 * 256:
-            # several rows and one round of 128-row tiles for the CUs: the tiles share the
-            # activations through LDS (more rounds suit the skinny kernel's resident variant better)
-            gemm_tiled_splitk(a, w, c, epilogue, 13, 1)
-        else:
-            gemm_skinny(a, w, c, epilogue)
-    else:
-        gemm_generic(a, w, c, epilogue)
+    """The product the engine calls: the library picks the kernel for the operands' types and sizes."""
+    gemm_linked(a, w, c, epilogue)
 
 
 def attn_mfma_takes(q: torch.Tensor, d: int) -> bool:

@@ -19,6 +19,9 @@ from .position import NoPosition, PositionEncoding
 import torch
 
 
+MAX_HEAD_DIM = 256      # what a tile of the vector-ALU attention kernel holds in LDS
+
+
 class Attention(Mixer):
     graph_safe = True      # launches depend on device memory only
     takes_normed_rows = True   # the input goes to a Linear unchanged
@@ -28,8 +31,8 @@ class Attention(Mixer):
                  names=("q_proj.weight", "k_proj.weight", "v_proj.weight", "o_proj.weight")):
         if n_heads % n_kv_heads:
             raise ValueError(f"{n_heads} heads do not split over {n_kv_heads} KV heads")
-        if head_dim % 16 or not 16 <= head_dim <= 256:
-            raise ValueError(f"head size {head_dim}: the attention kernels take multiples of 16 up to 256")
+        if not 1 <= head_dim <= MAX_HEAD_DIM:
+            raise ValueError(f"head size {head_dim}: the attention kernels take 1 to {MAX_HEAD_DIM}")
         self.H, self.G, self.d = n_heads, n_kv_heads, head_dim
         self.window = int(window)
         self.scale = float(scale) if scale is not None else 1.0 / math.sqrt(head_dim)   # model_core.c:2077
@@ -51,6 +54,24 @@ class Attention(Mixer):
 
     def prepare(self, runtime: Runtime, max_positions: int) -> None:
         self.position.prepare(runtime, max_positions)
+
+    def emit(self, b, norm, x: int, out_norm=None, out_norm_when: int = 0) -> None:
+        """x += o(attention(rotate(q, k), v)) with q, k, v = W norm(x), as operations of a launch
+        program.  The engine runs rotations (or no position encoding) and keeps all keys."""
+        from ..engine.program import CannotEmit
+        from .position import RotaryEmbedding
+        if type(self) is not Attention or type(self.position) not in (RotaryEmbedding, NoPosition):
+            raise CannotEmit("an attention or position encoding of another kind than the engine runs")
+        if self.window:
+            raise CannotEmit("the engine keeps all keys; a window of them is stepped from Python")
+        H, G, d = self.H, self.G, self.d
+        h = b.buffer("norm.out", self.qkv.in_size, b.dtype)
+        qkv = b.buffer("attn.qkv", (H + 2 * G) * d, torch.float32)
+        self.qkv.emit(b, h, qkv, kernels.EPI_STORE, in_norm=norm, in_norm_x=x)
+        q = b.buffer("attn.q", H * d, b.dtype)
+        out = b.buffer("attn.out", H * d, b.dtype)
+        b.attention(qkv, q, out, H, G, d, self.window, self.scale, self.position.rotary_tables())
+        self.o.emit(b, out, x, kernels.EPI_ACCUMULATE, out_norm=out_norm, out_norm_when=out_norm_when)
 
     def forward(self, ctx: StepContext, h, residual) -> None:
         b = ctx.batch

@@ -152,6 +152,10 @@ class StepContext:
 
 
 class Part:
+    """`emit`, where a part has it, appends the part's work to a launch program (engine/program.py)
+    instead of running it: a model whose parts all have it is stepped by the library in one call.
+    A part that only has `forward` is run from Python, and so is every model that contains one."""
+
     def tensor_specs(self) -> list[TensorSpec]:
         return []
 

@@ -21,6 +21,28 @@ class PreNormBlock(Block):
         have it prepared (see NormedRows)."""
         return self.mixer_norm
 
+    def emit(self, b, x: int, after=None, after_when: int = 0) -> None:
+        """The block as operations of a launch program over the residual rows in buffer `x`;
+        `after`: the norm that meets x after this block (after_when = 1: only in steps that want
+        every row's logits), so that the block's last product can prepare it."""
+        from ..engine.program import CannotEmit
+        if type(self) is not PreNormBlock:
+            raise CannotEmit(f"{type(self).__name__} changes what PreNormBlock does")
+        for part in (self.mixer, self.ffn):
+            if part is not None and not callable(getattr(part, "emit", None)):
+                raise CannotEmit(f"{type(part).__name__} has no operations of the engine's")
+        n1 = self.mixer_norm.norm_ref() if hasattr(self.mixer_norm, "norm_ref") else None
+        if n1 is None:
+            raise CannotEmit(f"{type(self.mixer_norm).__name__} has no operations of the engine's")
+        if self.ffn is None:
+            self.mixer.emit(b, n1, x, after, after_when)
+            return
+        if not hasattr(self.ffn_norm, "norm_ref"):
+            raise CannotEmit(f"{type(self.ffn_norm).__name__} has no operations of the engine's")
+        n2 = self.ffn_norm.norm_ref()
+        self.mixer.emit(b, n1, x, n2, 0)
+        self.ffn.emit(b, n2, x, after, after_when)
+
     def forward(self, ctx: StepContext, x) -> None:
         """x += mixer(norm(x)); x += ffn(norm(x))."""
         after = ctx.norm_after_block                # the norm that meets x after this block, if the caller knows it

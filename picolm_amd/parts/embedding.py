@@ -25,6 +25,15 @@ class TokenEmbedding(Part):
         t = fetch.get(self.name)
         self.table = (t.to(torch.float32) if runtime.is_f32 else t).contiguous()
 
+    def emit(self, b) -> int:
+        """The lookup as an operation of a launch program; returns the buffer of the residual rows."""
+        from ..engine.program import CannotEmit
+        if type(self) is not TokenEmbedding or self.table is None:
+            raise CannotEmit(f"{type(self).__name__} is no plain embedding with a loaded table")
+        x = b.buffer("residual", self.D, torch.float32)
+        b.embed(self.table, x)
+        return x
+
     def forward(self, ctx: StepContext, tokens: torch.Tensor, n_tokens: int) -> torch.Tensor:
         x = ctx.ws.get("residual", (n_tokens, self.D), torch.float32)
         kernels.embed(self.table, tokens, x)
@@ -51,6 +60,16 @@ class LMHead(Part):
             self.weight = (t.to(torch.float32) if runtime.is_f32 else t).contiguous()
 
     takes_normed_rows = True   # the input goes to the product unchanged
+
+    def emit(self, b, norm, x: int) -> None:
+        """logits = W norm(x) on the wanted rows, as an operation of a launch program."""
+        from ..engine.program import ROWS_WANTED, CannotEmit
+        if type(self) is not LMHead or self.weight is None:
+            raise CannotEmit(f"{type(self).__name__} is no plain head with loaded weights")
+        h = b.buffer("norm.final", self.D, b.dtype, ROWS_WANTED)
+        logits = b.buffer("logits", self.V, torch.float32, ROWS_WANTED)
+        b.linear(self.weight, h, logits, kernels.EPI_STORE, rows=ROWS_WANTED, in_norm=norm, in_norm_x=x)
+        b.logits_buffer = logits
 
     def forward(self, ctx: StepContext, h) -> torch.Tensor:
         """h: the final hidden rows, or NormedRows of them."""

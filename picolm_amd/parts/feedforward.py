@@ -22,6 +22,17 @@ class SwiGLU(FeedForward):
     def children(self):
         return [self.gate_up, self.down]
 
+    def emit(self, b, norm, x: int, out_norm=None, out_norm_when: int = 0) -> None:
+        """x += down(silu(gate h) * (up h)) with h = norm(x), as operations of a launch program."""
+        import torch
+        from ..engine.program import CannotEmit
+        if type(self) is not SwiGLU:
+            raise CannotEmit(f"{type(self).__name__} changes what SwiGLU does")
+        h = b.buffer("norm.out", self.D, b.dtype)
+        act = b.buffer("ffn.act", self.F, b.dtype)
+        self.gate_up.emit(b, h, act, kernels.EPI_SWIGLU, in_norm=norm, in_norm_x=x)
+        self.down.emit(b, act, x, kernels.EPI_ACCUMULATE, out_norm=out_norm, out_norm_when=out_norm_when)
+
     def forward(self, ctx: StepContext, h, residual) -> None:
         act = ctx.ws.get("ffn.act", (h.shape[0], self.F), ctx.dtype)
         self.gate_up.forward(h, act, kernels.EPI_SWIGLU)

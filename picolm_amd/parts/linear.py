@@ -52,6 +52,14 @@ class Linear(Part):
             w = ws[0] if len(ws) == 1 else torch.cat(ws, dim=0)
         self.weight = w.contiguous()
 
+    def emit(self, b, inp: int, out: int, epilogue: int = kernels.EPI_STORE, **norms) -> None:
+        """The same product as an operation of a launch program; `norms` as ProgramBuilder.linear
+        takes them (the norm of the input, the norm that meets the output next)."""
+        from ..engine.program import CannotEmit
+        if type(self) is not Linear or self.weight is None:
+            raise CannotEmit(f"{type(self).__name__} is no plain Linear with loaded weights")
+        b.linear(self.weight, inp, out, epilogue, **norms)
+
     def forward(self, a, out: torch.Tensor, epilogue: int = kernels.EPI_STORE, ctx=None) -> None:
         """out (=, +=, = silu-gated) a W^T.  `a` is a tensor, or NormedRows: rows whose norm the
         products compute between them.  With `ctx` and the accumulating epilogue, the norm that

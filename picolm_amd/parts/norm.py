@@ -33,6 +33,13 @@ class RMSNorm(Norm):
     def rms_parameters(self):
         return self.weight, self.eps
 
+    def norm_ref(self):
+        """This norm as a launch program's operations carry it."""
+        from ..engine.program import CannotEmit, NormRef
+        if type(self) is not RMSNorm or self.weight is None:
+            raise CannotEmit(f"{type(self).__name__} is no plain RMSNorm with loaded weights")
+        return NormRef(self.weight, self.eps)
+
     def forward(self, ctx: StepContext, x, rows=None, n_rows=None, out_name="norm.out"):
         n = x.shape[0] if rows is None else (n_rows if n_rows is not None else rows.numel())
         out = ctx.ws.get(out_name, (n, self.size), ctx.dtype)

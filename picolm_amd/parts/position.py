@@ -39,10 +39,15 @@ class RotaryEmbedding(PositionEncoding):
         self.head_dim, self.theta, self.scaling, self.style = head_dim, float(theta), scaling, style
         self.cos = self.sin = None
         self.n_positions = 0
+        self._handed_out = []       # earlier, shorter tables: recorded steps hold their addresses
 
     def prepare(self, runtime: Runtime, max_positions: int) -> None:
         if self.cos is not None and self.n_positions >= max_positions and self.cos.device == runtime.device:
             return
+        if self.cos is not None:
+            # a recorded decode step keeps the raw addresses of the tables it was recorded with and
+            # no reference to them: tables that were handed out are kept for the part's lifetime
+            self._handed_out.append((self.cos, self.sin))
         inv = rotary_inv_freq(self.head_dim, self.theta, self.scaling).to(torch.float32)
         pos = torch.arange(max_positions, dtype=torch.float32)
         ang = pos[:, None] * inv[None, :]                     # float32 product

@@ -5,8 +5,10 @@ a `model.language_model.` name up as `model.` too (:170-183), checks presence on
 only (:509-512) and never checks a shape.  Here every tensor a model declares is checked,
 and all faults are reported together in one `WeightsError`.
 
-Storage policy: bfloat16 stays bfloat16, 32-bit floats stay 32-bit, float16 is rounded to
-bfloat16 (the engine has no float16 arithmetic), integer tables become int32.
+Storage policy: bfloat16 stays bfloat16, 32-bit floats stay 32-bit, integer tables become
+int32.  The engine has no float16 arithmetic (picolm keeps such tensors as they are,
+picolm/safetensors.c:163-164): in the 32-bit runtime a float16 tensor is widened to float32,
+which is exact; in the bfloat16 runtime it is rounded to bfloat16, which drops three bits.
 """
 from __future__ import annotations
 
@@ -19,6 +21,9 @@ import torch
 from .safetensors_io import SafetensorsError, SafetensorsFile
 
 _RENAMES = (("model.language_model.", "model."),)
+# buffers that older checkpoints of this family carry and that are no parameters: picolm binds
+# tensors by name and never looks at the rest (picolm/safetensors.c:242-277)
+_IGNORED_SUFFIXES = ("rotary_emb.inv_freq",)
 
 
 class WeightsError(ValueError):
@@ -60,11 +65,14 @@ def canonical_name(name: str) -> str:
     return name
 
 
-def stored_dtype(dtype: torch.dtype, kind: str = "float") -> torch.dtype | None:
-    """The dtype a tensor is kept in, or None if the engine cannot hold it."""
+def stored_dtype(dtype: torch.dtype, kind: str = "float", runtime_dtype: torch.dtype | None = None) -> torch.dtype | None:
+    """The dtype a tensor is kept in by a runtime of `runtime_dtype`, or None if the engine
+    cannot hold it."""
     if kind == "int":
         return torch.int32 if dtype in (torch.int32, torch.int64, torch.int16, torch.int8, torch.uint8) else None
-    if dtype in (torch.bfloat16, torch.float16):
+    if dtype == torch.float16:
+        return torch.float32 if runtime_dtype == torch.float32 else torch.bfloat16
+    if dtype == torch.bfloat16:
         return torch.bfloat16
     if dtype == torch.float32:
         return torch.float32
@@ -144,7 +152,7 @@ def check_specs(source, specs: list[TensorSpec]) -> None:
         wanted[s.name] = s
     have = set(source.names())
     missing = [n for n, s in wanted.items() if n not in have and not s.optional]
-    unexpected = sorted(have - set(wanted))
+    unexpected = sorted(n for n in have - set(wanted) if not n.endswith(_IGNORED_SUFFIXES))
     wrong_shape, wrong_dtype = [], []
     for n, s in wanted.items():
         if n not in have:
@@ -161,9 +169,10 @@ def check_specs(source, specs: list[TensorSpec]) -> None:
 class WeightFetcher:
     """Hands checked tensors to the parts, in their kept dtype, on the target device."""
 
-    def __init__(self, source, device):
+    def __init__(self, source, device, runtime_dtype: torch.dtype | None = None):
         self.source = source
         self.device = device
+        self.runtime_dtype = runtime_dtype
         self._have = set(source.names())
 
     def has(self, name: str) -> bool:
@@ -171,7 +180,7 @@ class WeightFetcher:
 
     def get(self, name: str, kind: str = "float") -> torch.Tensor:
         t = self.source.tensor(name)
-        dt = stored_dtype(t.dtype, kind)
+        dt = stored_dtype(t.dtype, kind, self.runtime_dtype)
         if dt is None:
             raise WeightsError(self.source.source, wrong_dtype=[(name, str(t.dtype))])
         t = t.to(device=self.device, non_blocking=False)

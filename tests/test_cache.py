@@ -134,3 +134,19 @@ def test_random_walk_keeps_the_books_balanced():
                 assert len(g.book.pages[s]) == want
         assert sorted(live) == c.slots.live_slots()
         assert c.slots.n_free + len(live) == c.n_slots
+
+
+def test_a_refused_batch_leaves_the_books_as_they_were():
+    c = make_cache(max_tokens=64 * 20, n_slots=4, max_seq_len=64 * 4)
+    a, b = c.alloc_slot(), c.alloc_slot()
+    free = [g.book.pool.n_free for g in c.kv]
+    with pytest.raises(CacheFull):
+        c.reserve_many([a, b], [100, 64 * 4 + 1])          # the last sequence is too long: nothing may grow
+    assert [g.book.pool.n_free for g in c.kv] == free
+    assert all(len(g.book.pages[a]) == 0 for g in c.kv)
+    c.free_slot(b)
+    with pytest.raises(CacheError, match="not live"):
+        c.reserve_many([a, b], [100, 10])                  # a dead slot behind a good one
+    assert [g.book.pool.n_free for g in c.kv] == free
+    c.reserve_many([a], [100])
+    assert all(len(g.book.pages[a]) == g.book.need(100) for g in c.kv)

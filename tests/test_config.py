@@ -115,3 +115,15 @@ def test_model_structure_comes_from_the_configuration():
         assert len(g) == 1 and g[0].n_entries == c.num_hidden_layers and g[0].n_kv_heads == c.num_key_value_heads
         written = [s for s in specs.values() if s.init is not None]
         assert len(written) == 2 + 9 * c.num_hidden_layers + (0 if c.tie_word_embeddings else 1)
+
+
+def test_head_size_limits_are_named_when_the_configuration_is_read():
+    d = dict(architectures=["LlamaForCausalLM"], hidden_size=100, intermediate_size=96, num_attention_heads=6,
+             num_hidden_layers=1, vocab_size=50)
+    with pytest.raises(ConfigError, match="hidden_size.*not divisible.*num_attention_heads"):
+        LlamaConfig.from_dict(d)                                   # picolm would floor to 16 silently
+    assert LlamaConfig.from_dict(dict(d, head_dim=20)).head_dim == 20     # given: no division takes place
+    assert LlamaConfig.from_dict(dict(d, num_attention_heads=5)).head_dim == 20      # any even size, not only 16s
+    with pytest.raises(ConfigError, match="head_dim.*256"):
+        LlamaConfig.from_dict(dict(d, head_dim=320))
+    assert LlamaConfig.from_dict(dict(d, head_dim=256)).head_dim == 256

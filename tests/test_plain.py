@@ -108,6 +108,24 @@ def test_llama3_scaling_properties():
         assert abs(scaled_over_base(edge * (1 - 1e-9)) - scaled_over_base(edge * (1 + 1e-9))) < 1e-6
     assert np.isclose(scaled_over_base(10.0), 1.0) and np.isclose(scaled_over_base(100.0), 1 / 8)
     assert 1 / 8 < scaled_over_base(32.0) < 1.0
+    # the blend is linear in original/wavelength, not in the wavelength: at wavelength 32 that ratio
+    # is 2, a third of the way from low = 1 to high = 4, so the weight of the unscaled frequency
+    # is 1/3 and the result (2/3)/8 + 1/3 = 5/12; a blend linear in the wavelength would weigh it
+    # (64 - 32) / (64 - 16) = 2/3 and give 17/24
+    assert np.isclose(scaled_over_base(32.0), 5 / 12, rtol=1e-12)
+    assert np.isclose(scaled_over_base(48.0), (1 - 1 / 9) / 8 + 1 / 9, rtol=1e-12)      # ratio 4/3: weight 1/9
+
+
+def test_the_engine_tables_use_the_same_frequencies():
+    # the product's own routine (it runs on the host) against the plain one and the hand value
+    from picolm_amd.config import LlamaConfig
+    from picolm_amd.parts.position import rotary_inv_freq
+    cfg = LlamaConfig.from_dict(dict(tiny.TINY_B))
+    got = rotary_inv_freq(32, 500000.0, cfg.rope_scaling).numpy()
+    want = P.rope_inv_freq(32, 500000.0, tiny.TINY_B["rope_scaling"])
+    assert np.allclose(got, want, rtol=1e-14)
+    theta = (32.0 / (2 * math.pi)) ** 2
+    assert np.isclose(float(rotary_inv_freq(4, theta, cfg.rope_scaling)[1] / rotary_inv_freq(4, theta)[1]), 5 / 12, rtol=1e-12)
 
 
 # ---------------------------------------------------------------------------------------- attention
@@ -198,13 +216,57 @@ def test_whole_model_structure():
     assert np.allclose(P.forward(w, cfg, toks, start_pos=17), full)
 
 
+def test_each_half_of_a_layer_has_its_own_norm():
+    """One token, one layer: softmax over the single visible key is 1, so the mixer's output is
+    W_o applied to the value heads (each repeated for its query heads), and the whole layer can be
+    written out by hand.  The two norms get different constant weights a and b: swapping them, or
+    using one for both halves, changes the result."""
+    rng = np.random.default_rng(21)
+    D, F, V, H, G, d = 6, 5, 7, 2, 1, 4
+    a, b, c = 0.5, 3.0, 1.25
+    cfg = dict(num_hidden_layers=1, num_attention_heads=H, num_key_value_heads=G, head_dim=d, rms_norm_eps=1e-5,
+               rope_theta=100.0)
+    p = "model.layers.0."
+    w = {"model.embed_tokens.weight": rng.standard_normal((V, D)), "model.norm.weight": np.full(D, c),
+         p + "input_layernorm.weight": np.full(D, a), p + "post_attention_layernorm.weight": np.full(D, b),
+         p + "self_attn.q_proj.weight": rng.standard_normal((H * d, D)),
+         p + "self_attn.k_proj.weight": rng.standard_normal((G * d, D)),
+         p + "self_attn.v_proj.weight": rng.standard_normal((G * d, D)),
+         p + "self_attn.o_proj.weight": rng.standard_normal((D, H * d)),
+         p + "mlp.gate_proj.weight": rng.standard_normal((F, D)), p + "mlp.up_proj.weight": rng.standard_normal((F, D)),
+         p + "mlp.down_proj.weight": rng.standard_normal((D, F)), "lm_head.weight": rng.standard_normal((V, D))}
+
+    def unit(x):
+        return x / math.sqrt(float(x @ x) / D + 1e-5)
+
+    def by_hand(first, second):
+        x = w["model.embed_tokens.weight"][3]
+        v = w[p + "self_attn.v_proj.weight"] @ (first * unit(x))
+        x = x + w[p + "self_attn.o_proj.weight"] @ np.concatenate([v] * (H // G))
+        h = second * unit(x)
+        g, u = w[p + "mlp.gate_proj.weight"] @ h, w[p + "mlp.up_proj.weight"] @ h
+        x = x + w[p + "mlp.down_proj.weight"] @ (g / (1.0 + np.exp(-g)) * u)
+        return w["lm_head.weight"] @ (c * unit(x))
+
+    got = P.forward(w, cfg, [3])[0]
+    assert np.allclose(got, by_hand(a, b), rtol=1e-12)
+    assert not np.allclose(got, by_hand(b, a), rtol=1e-3)
+    assert not np.allclose(got, by_hand(a, a), rtol=1e-3) and not np.allclose(got, by_hand(b, b), rtol=1e-3)
+
+
 # ---------------------------------------------------------------------------------------- sampler
 def test_xorshift64_known_value_and_uniform():
     assert SP.xorshift64(1) == 1082269761                    # 1 -> 8193 -> 8257 -> 8257 ^ (8257 << 17)
     assert SP.init_state(0) == 42 and SP.init_state(5) == 5
+    # (float)(x >> 11) / (float)(1 << 53), sampler.c:19-21: the 53-bit integer is rounded to the 24
+    # bits of a float before the division.  Expected values from exact integer arithmetic: state
+    # 42 gives x >> 11 = 22194729, which is odd beyond 2^24 and rounds to 22194728
     r, s = SP.rand_float(42)
-    assert s == SP.xorshift64(42) and 0.0 <= r <= 1.0
-    assert r == float(np.float32(np.float32(s >> 11) / np.float32(2.0 ** 53)))
+    assert s == 45454805674 and s >> 11 == 22194729
+    assert r == float.fromhex("0x1.52aa28p-29") == 22194728 / 2.0 ** 53
+    r, s = SP.rand_float(0x123456789ABCDEF)
+    assert s == 4550888344034083252 and s >> 11 == 2222113449235392
+    assert r == float.fromhex("0x1.f94006p-3") == 2222113402388480 / 2.0 ** 53     # not 2222113449235392 / 2^53
 
 
 def test_sampler_special_cases():

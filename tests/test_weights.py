@@ -11,7 +11,7 @@ import torch
 import tiny
 from picolm_amd import LlamaConfig, write_random_model
 from picolm_amd.engine import build_from_config_dict, tensor_specs_for
-from picolm_amd.weights import (Checkpoint, SafetensorsError, SafetensorsFile, TensorDict, WeightFetcher, WeightsError,
+from picolm_amd.weights import (Checkpoint, SafetensorsError, SafetensorsFile, TensorDict, WeightFetcher, WeightsError, stored_dtype,
                                 check_specs, random_tensors, write_safetensors)
 
 
@@ -132,6 +132,29 @@ def test_storage_policy_and_aliases(tmp_path):
     assert f.get("model.b").dtype == torch.float32               # stored in 32-bit, stays so
     assert f.get("model.c").dtype == torch.bfloat16
     assert f.get("model.idx", kind="int").dtype == torch.int32
+    # the 32-bit runtime widens float16 exactly instead (picolm keeps float16 as it is,
+    # safetensors.c:163-164); everything else is kept as above
+    third = torch.tensor([1 / 3, 0.1], dtype=torch.float16)
+    write_safetensors(str(tmp_path / "m" / "model.safetensors"), dict(t, **{"model.language_model.a": third}))
+    f32 = WeightFetcher(Checkpoint(str(tmp_path / "m")), "cpu", torch.float32)
+    assert f32.get("model.a").dtype == torch.float32 and torch.equal(f32.get("model.a"), third.float())
+    assert f32.get("model.c").dtype == torch.bfloat16 and f32.get("model.b").dtype == torch.float32
+    bf = WeightFetcher(Checkpoint(str(tmp_path / "m")), "cpu", torch.bfloat16)
+    assert bf.get("model.a").dtype == torch.bfloat16 and not torch.equal(bf.get("model.a").float(), third.float())
+    assert stored_dtype(torch.float16, "float", torch.float32) == torch.float32
+    assert stored_dtype(torch.float16, "float", torch.bfloat16) == torch.bfloat16 == stored_dtype(torch.float16)
+
+
+def test_buffers_that_are_no_parameters_are_ignored():
+    cfg = LlamaConfig.from_dict(tiny.TINY_A)
+    specs = tensor_specs_for(cfg)
+    t = dict(random_tensors(specs, 0))
+    t["model.layers.0.self_attn.rotary_emb.inv_freq"] = torch.ones(8)      # older checkpoints carry these
+    check_specs(TensorDict(t), specs)
+    t["model.layers.0.self_attn.rotary_emb.other"] = torch.ones(8)
+    with pytest.raises(WeightsError) as e:
+        check_specs(TensorDict(t), specs)
+    assert e.value.unexpected == ["model.layers.0.self_attn.rotary_emb.other"]
 
 
 def test_sharded_folder(tmp_path):
