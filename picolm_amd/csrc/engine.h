@@ -142,7 +142,10 @@ typedef struct {
 // max_new tokens, or at the cache's capacity, leaves the batch and gives its slot back; batches of
 // up to batch_size requests follow each other until all are done.  prompts: packed token ids,
 // prompt_lens[i] >= 1 each.  out_tokens: [n_prompts][max_new]; out_counts[i] tokens were made;
-// out_finish[i]: 1 stop token, 2 length, 3 capacity.  It waits for the GPU once a step.
+// out_finish[i]: 1 stop token, 2 length, 3 capacity.  It waits for the GPU once a step.  Prompts
+// of a batch that together exceed the step's token budget (16,384 unless set otherwise; it sizes
+// the workspace) go in as several steps, each appending to what the slots hold.
+int picolm_engine_set_prefill_step_tokens(picolm_engine* e, int32_t tokens);
 int picolm_engine_generate(picolm_engine* e, int32_t n_prompts, const int32_t* prompts, const int32_t* prompt_lens,
                            int32_t max_new, const picolm_sampling* sampling, const int32_t* stop_ids, int32_t n_stop,
                            int32_t batch_size, int32_t* out_tokens, int32_t* out_counts, int32_t* out_finish,

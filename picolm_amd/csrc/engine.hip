@@ -356,6 +356,7 @@ struct picolm_engine {
     void* gen_scratch = nullptr;
     size_t gen_scratch_bytes = 0;
     int gen_rows = 0;
+    int prefill_step_tokens = 16384;       // most tokens of one prefill step of the generation loop
     bool host_only() const { return (flags & PICOLM_ENGINE_HOST_ONLY) != 0; }
 };
 
@@ -1258,6 +1259,12 @@ extern "C" int picolm_engine_step_array(picolm_engine* e, const char* name, int3
     return s.n;
 }
 
+extern "C" int picolm_engine_set_prefill_step_tokens(picolm_engine* e, int32_t tokens) {
+    E_REQUIRE(-1, e && tokens >= 64, "prefill_step_tokens: at least one page of 64 tokens");
+    e->prefill_step_tokens = tokens;
+    return 0;
+}
+
 // ---- generation ------------------------------------------------------------------------------------
 // Initial xorshift64 state of sequence `index`: sequence 0 has picolm's single stream
 // (`seed ? seed : 42`, picolm/sampler.c:43); the others are offset so that a sequence's draws do
@@ -1377,43 +1384,78 @@ extern "C" int picolm_engine_generate(picolm_engine* e, int32_t n_prompts, const
             first += n;
             continue;
         }
-        std::vector<int32_t> sl(n), nn(n);
-        for (int i = 0; i < n; ++i) {
-            sl[i] = slot_of[ids[i]];
-            nn[i] = prompt_lens[ids[i]];
-        }
+        // what a sampled token means for its request: recorded; the request goes on or ends and
+        // gives its slot back at once
+        std::vector<int> last_token(n_prompts, 0);
+        auto accept = [&](int i, int tok) {
+            out_tokens[(int64_t)i * max_new + out_counts[i]++] = tok;
+            last_token[i] = tok;
+            if (is_stop(tok)) out_finish[i] = 1;
+            else if (out_counts[i] >= max_new) out_finish[i] = 2;
+            else if (length[i] + 1 > e->max_seq_len) out_finish[i] = 3;
+            else return true;
+            (void)picolm_engine_slot_free(e, slot_of[i]);
+            slot_of[i] = -1;
+            return false;
+        };
+        // the prompts: one step if they fit the step's token budget, else several, each giving every
+        // unfinished prompt an equal share in whole pages; a prompt's last step gives its first token
+        std::vector<int> done(n, 0), live;
+        std::vector<int32_t> sl, nn, toks, counts, idx;
         float* logits = nullptr;
-        rc = picolm_engine_step(e, n, sl.data(), nn.data(), prompts + start[first], nullptr, nullptr, &logits, nullptr, stream);
-        std::vector<int> live = ids;
-        while (!rc && !live.empty()) {
-            rc = gen_sample(e, logits, live, sampling, stream);
-            if (rc) break;
-            std::vector<int> next;
-            std::vector<int32_t> toks;
-            for (size_t x = 0; x < live.size(); ++x) {
-                const int i = live[x], tok = e->gen_tokens_host[x];
-                out_tokens[(int64_t)i * max_new + out_counts[i]++] = tok;
-                if (is_stop(tok)) out_finish[i] = 1;
-                else if (out_counts[i] >= max_new) out_finish[i] = 2;
-                else if (length[i] + 1 > e->max_seq_len) out_finish[i] = 3;
-                else {
-                    next.push_back(i);
-                    toks.push_back(tok);
-                    continue;
+        int64_t total = 0;
+        for (int i = 0; i < n; ++i) total += prompt_lens[ids[i]];
+        while (!rc) {
+            std::vector<int> left;
+            for (int i = 0; i < n; ++i)
+                if (done[i] < prompt_lens[ids[i]]) left.push_back(i);
+            if (left.empty()) break;
+            const int budget = e->prefill_step_tokens;
+            const int share = total <= budget ? (1 << 30) : std::max(64, budget / (int)left.size() / 64 * 64);
+            int64_t room = total <= budget ? total : std::max<int64_t>(budget, 64 * (int64_t)left.size());
+            sl.clear(), nn.clear(), toks.clear(), counts.clear(), idx.clear();
+            std::vector<int> ending;
+            for (int i : left) {
+                const int id = ids[i];
+                const int take = (int)std::min<int64_t>(std::min(prompt_lens[id] - done[i], share), room);
+                if (take <= 0) continue;
+                sl.push_back(slot_of[id]);
+                nn.push_back(take);
+                toks.insert(toks.end(), prompts + start[id] + done[i], prompts + start[id] + done[i] + take);
+                done[i] += take;
+                room -= take;
+                const bool ends = done[i] == prompt_lens[id];
+                counts.push_back(ends ? 1 : 0);
+                if (ends) {
+                    idx.push_back(take - 1);
+                    ending.push_back(id);
                 }
-                // sequences that ended give their slots back at once; the rest go on
-                (void)picolm_engine_slot_free(e, slot_of[i]);
-                slot_of[i] = -1;
             }
-            live = next;
-            if (live.empty()) break;
+            if (idx.empty()) idx.push_back(0);
+            rc = picolm_engine_step(e, (int)sl.size(), sl.data(), nn.data(), toks.data(), counts.data(), idx.data(), &logits, nullptr, stream);
+            if (rc || ending.empty()) continue;
+            rc = gen_sample(e, logits, ending, sampling, stream);
+            for (size_t x = 0; !rc && x < ending.size(); ++x)
+                if (accept(ending[x], e->gen_tokens_host[x])) live.push_back(ending[x]);
+        }
+        std::sort(live.begin(), live.end());
+        while (!rc && !live.empty()) {
             sl.resize(live.size());
             nn.assign(live.size(), 1);
+            toks.resize(live.size());
             for (size_t x = 0; x < live.size(); ++x) {
                 sl[x] = slot_of[live[x]];
+                toks[x] = last_token[live[x]];
                 length[live[x]] += 1;
             }
             rc = picolm_engine_step(e, (int)live.size(), sl.data(), nn.data(), toks.data(), nullptr, nullptr, &logits, nullptr, stream);
+            if (rc) break;
+            rc = gen_sample(e, logits, live, sampling, stream);
+            if (rc) break;
+            std::vector<int> next;
+            for (size_t x = 0; x < live.size(); ++x)
+                if (accept(live[x], e->gen_tokens_host[x])) next.push_back(live[x]);
+            live = next;
         }
         release_all();
         if (rc) return rc;

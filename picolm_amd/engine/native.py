@@ -232,8 +232,13 @@ class NativeEngine:
             _raise(rc)
         return self._logits(logits.value, len(sl))
 
-    def generate(self, prompts, max_new_tokens: int, params, stop_ids=(), batch_size: int = 64):
+    def generate(self, prompts, max_new_tokens: int, params, stop_ids=(), batch_size: int = 64,
+                 prefill_step_tokens: int | None = None):
         """The library's own generation loop; returns (tokens of each request, finish reasons)."""
+        if prefill_step_tokens is not None:
+            rc = _lib().picolm_engine_set_prefill_step_tokens(self.handle, int(prefill_step_tokens))
+            if rc:
+                _raise(rc)
         n = len(prompts)
         lens = _i32([len(p) for p in prompts])
         flat = _i32(np.concatenate([np.asarray(p, dtype=np.int64) for p in prompts])) if n and lens.sum() else np.zeros(1, np.int32)

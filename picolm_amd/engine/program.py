@@ -181,6 +181,8 @@ def declare(lib) -> None:
     lib.picolm_engine_step_device_tokens.argtypes = [E, c_int32, c_void_p, c_void_p, POINTER(c_void_p), c_void_p]
     lib.picolm_engine_generate.argtypes = [E, c_int32, c_void_p, c_void_p, c_int32, POINTER(Sampling), c_void_p, c_int32,
                                            c_int32, c_void_p, c_void_p, c_void_p, c_void_p]
+    lib.picolm_engine_set_prefill_step_tokens.argtypes = [E, c_int32]
+    lib.picolm_engine_set_prefill_step_tokens.restype = ctypes.c_int
     lib.picolm_engine_info.argtypes = [E, c_int32]
     lib.picolm_engine_info.restype = c_int64
     lib.picolm_engine_kv_entry.argtypes = [E, c_int32, c_int32, POINTER(c_void_p), POINTER(c_void_p), POINTER(c_int64)]

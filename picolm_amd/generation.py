@@ -183,9 +183,38 @@ class GenerationLoop:
 
 
 # ---------------------------------------------------------------------------------------------
+PREFILL_STEP_TOKENS = 16384        # most tokens of one prefill step: what sizes the step's workspace
+
+
+def prefill_steps(lengths, budget: int = PREFILL_STEP_TOKENS):
+    """How a batch of prompts of these lengths goes through the model: a list of steps, each a list
+    of (sequence, first token, count).  Prompts that fit the budget together are one step (picolm
+    prefills a prompt in one call too, picolm/picolm.c:1502-1530).  Otherwise every step gives each
+    unfinished sequence an equal share of the budget, in whole cache pages, and a sequence joins
+    the later steps with what it has left, appended to what its slot already holds."""
+    lengths = [int(n) for n in lengths]
+    if sum(lengths) <= budget:
+        return [[(i, 0, n) for i, n in enumerate(lengths)]]
+    done = [0] * len(lengths)
+    steps = []
+    while any(d < n for d, n in zip(done, lengths)):
+        left = [i for i, n in enumerate(lengths) if done[i] < n]
+        share = max(64, budget // len(left) // 64 * 64)
+        step, room = [], max(budget, 64 * len(left))
+        for i in left:
+            take = min(lengths[i] - done[i], share, room)
+            if take <= 0:
+                continue
+            step.append((i, done[i], take))
+            done[i] += take
+            room -= take
+        steps.append(step)
+    return steps
+
+
 def generate(model_or_session, prompts, max_new_tokens: int = 256, params: SamplingParams | None = None,
              stop_ids=None, batch_size: int = 64, max_tokens: int | None = None, on_token=None,
-             return_stats: bool = False):
+             return_stats: bool = False, prefill_step_tokens: int = PREFILL_STEP_TOKENS):
     """The Python entry point: token ids in, generated token ids out.
 
     `model_or_session`: a loaded model (a session sized for the work is made) or a Session.
@@ -209,7 +238,7 @@ def generate(model_or_session, prompts, max_new_tokens: int = 256, params: Sampl
     if stop_ids is None:
         stop_ids = getattr(session.model.config, "eos_token_ids", ())
     device = session.model.runtime.device
-    loop = GenerationLoop(SessionStepper(session), lambda n: Sampler(params, n, device), stop_ids, batch_size,
+    loop = GenerationLoop(SessionStepper(session, prefill_step_tokens), lambda n: Sampler(params, n, device), stop_ids, batch_size,
                           sync=lambda: torch.cuda.synchronize(device))
     out = loop.run(prompts, max_new_tokens, on_token)
     return (out, loop.stats) if return_stats else out
@@ -218,15 +247,29 @@ def generate(model_or_session, prompts, max_new_tokens: int = 256, params: Sampl
 class SessionStepper:
     """The face of a Session that the loop needs."""
 
-    def __init__(self, session):
+    def __init__(self, session, prefill_step_tokens: int = PREFILL_STEP_TOKENS):
         self.session = session
         self.capacity = session.cache.max_seq_len
+        self.prefill_step_tokens = prefill_step_tokens
 
     def begin(self, n):
         return self.session.begin(n)
 
     def step(self, slots, tokens):
-        return self.session.step(slots, tokens)
+        """The last row's logits of every sequence.  Prompts beyond the budget of one step go in as
+        several steps (`prefill_steps`); each sequence's row is kept from the step that ends it."""
+        plan = prefill_steps([len(t) for t in tokens], self.prefill_step_tokens)
+        if len(plan) == 1:
+            return self.session.step(slots, tokens)
+        import torch
+        out = torch.empty((len(slots), self.session.vocab_size), dtype=torch.float32, device=self.session.model.runtime.device)
+        for step in plan:
+            ends = [i for i, first, count in step if first + count == len(tokens[i])]
+            logits = self.session.step([slots[i] for i, _, _ in step], [tokens[i][first:first + count] for i, first, count in step],
+                                       [[count - 1] if first + count == len(tokens[i]) else [] for i, first, count in step])
+            if ends:
+                out[torch.tensor(ends, device=out.device)] = logits
+        return out
 
     def step_ahead(self, slots, tokens_on_device):
         return self.session.step_tokens_on_device(slots, tokens_on_device)

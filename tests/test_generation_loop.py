@@ -196,3 +196,20 @@ def test_one_step_ahead_decides_as_the_plain_loop(case):
     assert loop0.stats.steps <= loop.stats.steps
     tokens_stepped = lambda s: sum(sum(e[2]) for e in s.log if e[0] == "step")
     assert tokens_stepped(st0) <= tokens_stepped(st) <= tokens_stepped(st0) + stopped
+
+
+def test_prompts_are_cut_into_steps_within_the_token_budget():
+    from picolm_amd.generation import prefill_steps
+    assert prefill_steps([10, 20, 30], 100) == [[(0, 0, 10), (1, 0, 20), (2, 0, 30)]]      # they fit: one step
+    lens = [300, 50, 1000, 64, 1]
+    steps = prefill_steps(lens, 512)
+    seen = [0] * len(lens)
+    for st in steps:
+        assert sum(c for _, _, c in st) <= 512
+        assert len({i for i, _, _ in st}) == len(st)                     # a sequence is in a step once
+        for i, first, count in st:
+            assert first == seen[i] and count > 0                        # each goes on where it stopped
+            assert first % 64 == 0                                       # in whole pages until its end
+            seen[i] += count
+    assert seen == lens
+    assert len(prefill_steps([100] * 40, 64)) == 2                       # more sequences than the budget has pages: a page each

@@ -364,3 +364,97 @@ def test_toy_feed_forward_with_routing():
     ref = np.stack([P.swiglu(x[t:t + 1], w[f"f.experts.{c}.gate_proj.weight"], w[f"f.experts.{c}.up_proj.weight"],
                              w[f"f.experts.{c}.down_proj.weight"])[0] for t, c in enumerate(choice)])
     assert np.abs(res.double().cpu().numpy() - ref).max() <= tol(torch.bfloat16, ref)
+
+
+# ------------------------------------------------------------------------------------------- a window's ring, lap after lap
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("window", [40, 100])
+def test_a_window_of_keys_through_several_laps_of_its_ring(dtype, window, tmp_path):
+    """A decoder whose attention keeps a window of keys: its cache group is a ring of pages per
+    slot.  A prompt longer than one chunk, then decoding far past the ring's first lap, launched
+    step by step and replayed from the recording; every step against the plain implementation
+    with the same window.  (Such a model is stepped from Python: the engine keeps all keys.)"""
+    from picolm_amd import LlamaConfig
+    from picolm_amd.engine import DecoderModel, Session
+    from picolm_amd.parts import (Attention, LMHead, PreNormBlock, RMSNorm, RotaryEmbedding, Runtime, SwiGLU, TokenEmbedding)
+    from picolm_amd.weights import Checkpoint, write_random_model
+    cfgd = dict(tiny.TINY_C, max_position_embeddings=1024, num_hidden_layers=2)
+    cfg = LlamaConfig.from_dict(cfgd)
+    d = write_random_model(cfg, str(tmp_path / "m"), seed=6, std=0.08, norm_sigma=0.1)
+    D = cfg.hidden_size
+    rotary = RotaryEmbedding(cfg.head_dim, cfg.rope_theta, None, cfg.rope_style)
+    blocks = [PreNormBlock(RMSNorm(f"model.layers.{l}.input_layernorm.weight", D, cfg.rms_norm_eps),
+                           Attention(f"model.layers.{l}.self_attn.", D, cfg.num_attention_heads, cfg.num_key_value_heads,
+                                     cfg.head_dim, position=rotary, window=window),
+                           RMSNorm(f"model.layers.{l}.post_attention_layernorm.weight", D, cfg.rms_norm_eps),
+                           SwiGLU(f"model.layers.{l}.mlp.", D, cfg.intermediate_size)) for l in range(2)]
+    emb = TokenEmbedding("model.embed_tokens.weight", cfg.vocab_size, D)
+    model = DecoderModel(cfg, emb, blocks, RMSNorm("model.norm.weight", D, cfg.rms_norm_eps),
+                         LMHead("lm_head.weight", cfg.vocab_size, D, emb, False))
+    ck = Checkpoint(d)
+    model.load(ck, Runtime(DEV, dtype))
+    ck.close()
+    rng = np.random.default_rng(window)
+    n_prompt, n_all = 300, 640
+    toks = tiny.random_tokens(rng, n_all, cfg.vocab_size)
+    ref = P.forward(tiny.read_weights_f64(d), dict(tiny.read_config(d), window=window), toks)
+    for graphs in (False, True):
+        s = Session(model, max_tokens=2048, graphs=graphs)
+        assert s.engine is None                                   # a window is stepped from Python
+        ring = s.cache.kv[0].ring_pages
+        assert ring < s.cache.max_pages and 64 * ring < n_all - 64      # decoding laps the ring more than once
+        [a] = s.begin(1)
+        got = s.step([a], [toks[:n_prompt]], [list(range(n_prompt))]).double().cpu().numpy()
+        assert np.abs(got - ref[:n_prompt]).max() <= tol(dtype, ref)
+        for j in range(n_prompt, n_all):
+            got = s.step([a], [[toks[j]]]).double().cpu().numpy()
+            err = np.abs(got[0] - ref[j]).max()
+            assert err <= tol(dtype, ref), (window, dtype, "graphs", graphs, "position", j, err)
+        assert (s.recorded_steps() > 0) == graphs
+        assert len(s.cache.kv[0].book.pages[a]) == ring           # the slot never holds more than its ring
+        s.release([a])
+
+
+@pytest.mark.parametrize("window", [40, 60])
+def test_the_edge_of_a_window_in_decode_steps_past_the_first_lap(window):
+    """One head whose query, key and value are the input row itself.  Two rows stand out: their
+    keys score far above all others for every later query, so a decode step's output is that
+    row's value while the row is inside the window and small once it has left.  The last step
+    that sees it has it exactly at position - window + 1; the next one must drop it, also when its
+    page of the ring has meanwhile been written again."""
+    from picolm_amd.engine.batch import StepBatch
+    from picolm_amd.parts import Attention
+    from picolm_amd.weights import TensorDict, WeightFetcher
+    d = 16
+    eye = torch.eye(d)
+    part = Attention("a.", d, 1, 1, d, window=window)
+    from picolm_amd.cache.kv import window_ring_pages
+    ring = window_ring_pages(window)
+    n_prompt, n_all = 300, 64 * ring + 5 + window + 8          # (the harness's cache takes sequences of 512)
+    rt, ctx = harness(torch.float32, part.cache_requests(), [1], [0], [n_all], max_tokens=1024)
+    assert ctx.cache.kv[0].ring_pages == ring and n_all <= 512
+    part.load_all(WeightFetcher(TensorDict({f"a.{n}_proj.weight": eye.clone() for n in "qkvo"}), DEV), rt)
+    rng = np.random.default_rng(window)
+    u = np.zeros(d)
+    u[3] = 1.0
+    h = rng.standard_normal((n_all, d)) * 0.05
+    h[:, 3] = 1.0                                  # every query looks along u
+    big = [305, 64 * ring + 5]                     # one in the first lap, one just after the ring has wrapped; never both in a window
+    for j in big:
+        h[j] = 60.0 * u                            # score 60 / 4 = 15 against about 0.25 for the others
+    ref = P.causal_attention(h[:, None, :], h[:, None, :], h[:, None, :], window)[:, 0, :]
+    ctx.batch = StepBatch([1], [0], [[0] * n_prompt], [[]], 10, DEV)
+    res = torch.zeros(n_prompt, d, device=DEV)
+    part.forward(ctx, torch.from_numpy(h[:n_prompt]).float().to(DEV), res)
+    assert np.abs(res.double().cpu().numpy() - ref[:n_prompt]).max() <= 1e-4
+    for p in range(n_prompt, n_all):
+        ctx.batch = StepBatch([1], [p], [[0]], [[]], 10, DEV)
+        res = torch.zeros(1, d, device=DEV)
+        part.forward(ctx, torch.from_numpy(h[p:p + 1]).float().to(DEV), res)
+        out = res.double().cpu().numpy()[0]
+        assert np.abs(out - ref[p]).max() <= 1e-4, p
+        for j in big:
+            if p == j + window - 1:
+                assert out[3] > 50.0, (p, "the key at position - window + 1 is visible")
+            if p == j + window:
+                assert out[3] < 2.0, (p, "the key at position - window is dropped")
