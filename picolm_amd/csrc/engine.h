@@ -99,6 +99,7 @@ typedef struct {
 
 #define PICOLM_ENGINE_NO_GRAPHS 1    // launch every decode step's kernels one by one
 #define PICOLM_ENGINE_HOST_ONLY 2    // books and index arrays only, no device memory: steps plan but do not run
+#define PICOLM_ENGINE_TIME_OPS 4     // an event before and after every operation (decode steps are then launched, not replayed)
 
 typedef struct picolm_engine picolm_engine;
 
@@ -150,6 +151,13 @@ int picolm_engine_generate(picolm_engine* e, int32_t n_prompts, const int32_t* p
                            int32_t max_new, const picolm_sampling* sampling, const int32_t* stop_ids, int32_t n_stop,
                            int32_t batch_size, int32_t* out_tokens, int32_t* out_counts, int32_t* out_finish,
                            hipStream_t stream);
+
+// With PICOLM_ENGINE_TIME_OPS: the GPU time in milliseconds since the last call, summed by class
+// of operation: ms[0] embedding and norms of their own, ms[1] the layers' products (with the norms
+// and partial sums that belong to them), ms[2] the head's product, ms[3] attention (with rotation
+// and the cache write).  Waits for the GPU.  picolm prints such figures for its layers itself
+// (picolm/picolm.c:305-317).
+int picolm_engine_op_times(picolm_engine* e, double* ms);
 
 // ---- what the engine holds, for bindings and tests ---------------------------------------------
 // what: 0 max_seq_len, 1 n_slots, 2 free slots, 3 free tokens (pages free in the tightest group

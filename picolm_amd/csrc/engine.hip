@@ -348,6 +348,14 @@ struct picolm_engine {
     std::map<std::pair<int, int>, std::unique_ptr<DecodeGraph>> graphs;
     hipStream_t capture_stream = nullptr;
     const StepPlan* last_plan = nullptr;
+    // timing by class of operation (PICOLM_ENGINE_TIME_OPS): an event before and after each one
+    struct TimedOp {
+        int cls;
+        hipEvent_t before, after;
+    };
+    std::vector<TimedOp> timed;
+    std::vector<hipEvent_t> spare_events;
+    bool timing() const { return (flags & PICOLM_ENGINE_TIME_OPS) != 0; }
     // generation
     int32_t* gen_tokens_dev = nullptr;
     int32_t* gen_tokens_host = nullptr;    // pinned
@@ -565,6 +573,11 @@ extern "C" void picolm_engine_destroy(picolm_engine* e) {
     if (e->gen_index) (void)hipFree(e->gen_index);
     if (e->gen_scratch) (void)hipFree(e->gen_scratch);
     e->stager.destroy();
+    for (auto& t : e->timed) {
+        (void)hipEventDestroy(t.before);
+        (void)hipEventDestroy(t.after);
+    }
+    for (auto ev : e->spare_events) (void)hipEventDestroy(ev);
     if (e->capture_stream) (void)hipStreamDestroy(e->capture_stream);
     delete e;
 }
@@ -1008,10 +1021,23 @@ static int run_attention(Run& r, const picolm_op& o) {
 
 // embedding -> the layer calls -> final norm on the wanted rows -> head
 // (picolm/model_core.c:1785, :1799-2210, :2213, :2220), as the program lists them.
+static int timing_event(picolm_engine* e, hipEvent_t* ev, hipStream_t stream) {
+    if (!e->spare_events.empty()) {
+        *ev = e->spare_events.back();
+        e->spare_events.pop_back();
+    } else {
+        HIP_TRY(hipEventCreate(ev));
+    }
+    HIP_TRY(hipEventRecord(*ev, stream));
+    return 0;
+}
+
 static int run_program(picolm_engine* e, const StepPlan& p, Workspace& w, hipStream_t stream) {
     Run r{e, p, w, stream, Prepared()};
     for (const picolm_op& o : e->ops) {
         if (o.rows == PICOLM_ROWS_WANTED && p.n_want == 0) continue;
+        hipEvent_t before = nullptr;
+        if (e->timing()) TRY(timing_event(e, &before, stream));
         switch (o.kind) {
             case PICOLM_OP_EMBED:
                 TRY(picolm_embed(o.weight, o.weight_dt, p.at(p.tokens), (float*)r.buf(o.out), p.T, o.k, o.n, stream));
@@ -1026,7 +1052,28 @@ static int run_program(picolm_engine* e, const StepPlan& p, Workspace& w, hipStr
             case PICOLM_OP_LINEAR: TRY(run_linear(r, o)); break;
             case PICOLM_OP_ATTENTION: TRY(run_attention(r, o)); break;
         }
+        if (e->timing()) {
+            hipEvent_t after = nullptr;
+            TRY(timing_event(e, &after, stream));
+            const int cls = o.kind == PICOLM_OP_LINEAR ? (o.rows == PICOLM_ROWS_WANTED ? 2 : 1) : o.kind == PICOLM_OP_ATTENTION ? 3 : 0;
+            e->timed.push_back({cls, before, after});
+        }
     }
+    return 0;
+}
+
+extern "C" int picolm_engine_op_times(picolm_engine* e, double* ms) {
+    E_REQUIRE(-1, e && ms && e->timing(), "op_times: the engine was not made with PICOLM_ENGINE_TIME_OPS");
+    for (int c = 0; c < 4; ++c) ms[c] = 0.0;
+    for (auto& t : e->timed) {
+        HIP_TRY(hipEventSynchronize(t.after));
+        float dt = 0.f;
+        HIP_TRY(hipEventElapsedTime(&dt, t.before, t.after));
+        ms[t.cls] += dt;
+        e->spare_events.push_back(t.before);
+        e->spare_events.push_back(t.after);
+    }
+    e->timed.clear();
     return 0;
 }
 
@@ -1079,7 +1126,7 @@ static int decode_step(picolm_engine* e, const std::vector<int>& slots, const st
             TRY(workspace_ensure(e, g.ws, p, most));
             TRY(run_program(e, p, g.ws, stream));
             g.logits = (float*)(g.ws.base + g.ws.offsets[e->logits_buffer]);
-            if (g.uses >= 2 && !(e->flags & PICOLM_ENGINE_NO_GRAPHS)) {
+            if (g.uses >= 2 && !(e->flags & (PICOLM_ENGINE_NO_GRAPHS | PICOLM_ENGINE_TIME_OPS))) {
                 // the sizes have been seen and the workspace is allocated: record the same launches
                 // (recording runs nothing; this step's result came from the launches above)
                 hipGraph_t graph = nullptr;

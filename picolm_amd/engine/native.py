@@ -117,11 +117,11 @@ class EngineCache:
 
 class NativeEngine:
     def __init__(self, built: P.BuiltProgram, max_tokens: int, max_seq_len: int, n_slots: int | None, device,
-                 graphs: bool = True, host_only: bool = False):
+                 graphs: bool = True, host_only: bool = False, time_ops: bool = False):
         self.program = built                      # keeps the weights and tables alive
         self.device = torch.device(device)
         self.vocab_size = built.struct.vocab_size
-        flags = (0 if graphs else P.ENGINE_NO_GRAPHS) | (P.ENGINE_HOST_ONLY if host_only else 0)
+        flags = (0 if graphs else P.ENGINE_NO_GRAPHS) | (P.ENGINE_HOST_ONLY if host_only else 0) | (P.ENGINE_TIME_OPS if time_ops else 0)
         h = c_void_p()
         rc = _lib().picolm_engine_create(byref(built.struct), int(max_tokens), int(max_seq_len), int(n_slots or 0), flags,
                                          byref(h))
@@ -176,6 +176,14 @@ class NativeEngine:
 
     def recorded_steps(self) -> int:
         return self.info(4)
+
+    def op_times(self) -> dict:
+        """GPU milliseconds since the last call by class of operation (an engine made with time_ops)."""
+        ms = (ctypes.c_double * 4)()
+        rc = _lib().picolm_engine_op_times(self.handle, ms)
+        if rc:
+            _raise(rc)
+        return {"other": ms[0], "products": ms[1], "head": ms[2], "attention": ms[3]}
 
     def step_array(self, name: str) -> np.ndarray:
         n = _lib().picolm_engine_step_array(self.handle, name.encode(), None, 0)

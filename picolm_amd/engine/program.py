@@ -17,7 +17,7 @@ F32, BF16 = 0, 1
 _DT = {torch.float32: F32, torch.bfloat16: BF16}
 OP_EMBED, OP_RMSNORM, OP_LINEAR, OP_ATTENTION = 1, 2, 3, 4
 ROWS_STEP, ROWS_WANTED = 0, 1
-ENGINE_NO_GRAPHS, ENGINE_HOST_ONLY = 1, 2
+ENGINE_NO_GRAPHS, ENGINE_HOST_ONLY, ENGINE_TIME_OPS = 1, 2, 4
 ERR_STEP, ERR_CACHE_FULL, ERR_CACHE, ERR_DEVICE = -10, -11, -12, -13
 
 
@@ -183,6 +183,8 @@ def declare(lib) -> None:
                                            c_int32, c_void_p, c_void_p, c_void_p, c_void_p]
     lib.picolm_engine_set_prefill_step_tokens.argtypes = [E, c_int32]
     lib.picolm_engine_set_prefill_step_tokens.restype = ctypes.c_int
+    lib.picolm_engine_op_times.argtypes = [E, c_void_p]
+    lib.picolm_engine_op_times.restype = ctypes.c_int
     lib.picolm_engine_info.argtypes = [E, c_int32]
     lib.picolm_engine_info.restype = c_int64
     lib.picolm_engine_kv_entry.argtypes = [E, c_int32, c_int32, POINTER(c_void_p), POINTER(c_void_p), POINTER(c_int64)]

@@ -62,9 +62,10 @@ class _DecodeGraph:
 
 class Session:
     def __init__(self, model: DecoderModel, max_tokens: int, max_seq_len: int | None = None,
-                 n_slots: int | None = None, graphs: bool = True, native: bool | None = None):
+                 n_slots: int | None = None, graphs: bool = True, native: bool | None = None, time_ops: bool = False):
         """`native`: None steps in the library when the model's parts allow it, False steps from
-        Python part by part, True insists on the library."""
+        Python part by part, True insists on the library.  `time_ops` (library only): GPU time is
+        kept by class of operation (`engine.op_times()`), and decode steps are launched one by one."""
         if model.runtime is None:
             raise StepError("the model has no weights loaded")
         self.model = model
@@ -78,7 +79,7 @@ class Session:
             built = model.program()
             if built is not None:
                 from .native import EngineCache, NativeEngine
-                self.engine = NativeEngine(built, max_tokens, seq_len, n_slots, model.runtime.device, graphs=graphs)
+                self.engine = NativeEngine(built, max_tokens, seq_len, n_slots, model.runtime.device, graphs=graphs, time_ops=time_ops)
                 self.cache = EngineCache(self.engine, model.cache_spec, model.runtime.dtype, model.runtime.device)
                 self.graphs = graphs
                 return
