@@ -91,7 +91,12 @@ def main(argv=None) -> int:
     model = load_model(args.model, dtype=args.dtype)
     cfg = model.config
     if not prompts:
-        prompts = [[cfg.bos_token_id]]                 # picolm starts from BOS without a prompt (picolm.c:1532-1535)
+        # picolm starts from BOS without a prompt (picolm.c:1532-1535); an architecture whose
+        # configuration names no start token needs a prompt
+        bos = getattr(cfg, "bos_token_id", None)
+        if bos is None:
+            raise SystemExit("no prompt given, and this model's configuration names no start token (bos_token_id)")
+        prompts = [[int(bos)]]
     context = args.context or cfg.max_position_embeddings
     per = sorted((pages_for(min(len(p) + args.max_tokens, context)) for p in prompts), reverse=True)
     session = Session(model, max_tokens=max(1, sum(per[:args.batch])) * PAGE_TOKENS, max_seq_len=context)

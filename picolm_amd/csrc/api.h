@@ -27,9 +27,6 @@ int picolm_rope_kv_store(const float* qkv, void* q_out, void* k_pages, void* v_p
                          const float* cos_t, const float* sin_t, int style, const int32_t* tok_pos,
                          const int32_t* tok_page /* physical cache page of every token */, int T, int H, int G,
                          int d, const int32_t* rows /* null: rows 0..T-1 */, hipStream_t stream);
-int picolm_silu_mul(const void* gu, int in_dt, void* out, int out_dt, int64_t n_pairs,
-                    hipStream_t stream);
-int picolm_add_into(float* y, const void* x, int x_dt, int64_t n, hipStream_t stream);
 
 int picolm_gemm_generic(const void* A, int a_dt, const void* W, int w_dt, void* C, int c_dt, int M,
                         int N, int K, int64_t lda, int64_t ldw, int64_t ldc, int epilogue,

@@ -203,50 +203,3 @@ extern "C" int picolm_rope_kv_store(const float* qkv, void* q_out, void* k_pages
     PICOLM_LAUNCH_CHECK("rope_kv_store");
     return 0;
 }
-
-// ---- silu(gate) * up on separate or interleaved inputs ------------------------------------
-// picolm/tensor.c:3306-3315 and :3325: g/(1+expf(-g)) * u.  `gu` holds rows of 2F values with
-// gate j at 2j and up j at 2j+1.
-template <typename TI, typename TO>
-__global__ void silu_mul_kernel(const TI* __restrict__ gu, TO* __restrict__ out, int64_t n_pairs) {
-    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (i >= n_pairs) return;
-    const float g = to_f32<TI>(gu[2 * i]), u = to_f32<TI>(gu[2 * i + 1]);
-    out[i] = from_f32<TO>(g / (1.0f + expf(-g)) * u);
-}
-
-extern "C" int picolm_silu_mul(const void* gu, int in_dt, void* out, int out_dt, int64_t n_pairs,
-                               hipStream_t stream) {
-    if (n_pairs <= 0) return 0;
-    dim3 block(256), grid((unsigned)ceil_div64(n_pairs, 256));
-    if (in_dt == PICOLM_F32 && out_dt == PICOLM_F32)
-        silu_mul_kernel<float, float><<<grid, block, 0, stream>>>((const float*)gu, (float*)out, n_pairs);
-    else if (in_dt == PICOLM_F32 && out_dt == PICOLM_BF16)
-        silu_mul_kernel<float, bf16_t><<<grid, block, 0, stream>>>((const float*)gu, (bf16_t*)out, n_pairs);
-    else if (in_dt == PICOLM_BF16 && out_dt == PICOLM_BF16)
-        silu_mul_kernel<bf16_t, bf16_t><<<grid, block, 0, stream>>>((const bf16_t*)gu, (bf16_t*)out, n_pairs);
-    else
-        PICOLM_REQUIRE(false, "silu_mul: unsupported dtypes %d -> %d", in_dt, out_dt);
-    PICOLM_LAUNCH_CHECK("silu_mul");
-    return 0;
-}
-
-// ---- y += x (float residual) ---------------------------------------------------------------
-template <typename TI>
-__global__ void add_into_kernel(float* __restrict__ y, const TI* __restrict__ x, int64_t n) {
-    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (i < n) y[i] += to_f32<TI>(x[i]);
-}
-
-extern "C" int picolm_add_into(float* y, const void* x, int x_dt, int64_t n, hipStream_t stream) {
-    if (n <= 0) return 0;
-    dim3 block(256), grid((unsigned)ceil_div64(n, 256));
-    if (x_dt == PICOLM_F32)
-        add_into_kernel<float><<<grid, block, 0, stream>>>(y, (const float*)x, n);
-    else if (x_dt == PICOLM_BF16)
-        add_into_kernel<bf16_t><<<grid, block, 0, stream>>>(y, (const bf16_t*)x, n);
-    else
-        PICOLM_REQUIRE(false, "add_into: unknown dtype %d", x_dt);
-    PICOLM_LAUNCH_CHECK("add_into");
-    return 0;
-}

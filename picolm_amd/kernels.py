@@ -40,7 +40,7 @@ def lib():
 
 def dir_entry_points():
     return ["picolm_abi_version", "picolm_device_check", "picolm_embed", "picolm_rmsnorm",
-            "picolm_rope_kv_store", "picolm_silu_mul", "picolm_add_into", "picolm_gemm_generic",
+            "picolm_rope_kv_store", "picolm_gemm_generic",
             "picolm_attn_prefill_tile_rows", "picolm_attn_prefill_generic",
             "picolm_attn_decode_generic", "picolm_argmax", "picolm_argmax_scratch_floats", "picolm_sample", "picolm_sample_scratch_bytes", "picolm_gemm_skinny", "picolm_gemm_tiled", "picolm_gemm_tiled_splitk", "picolm_gemm_linked", "picolm_gemm_tiled_norm_parts", "picolm_kv_page_order",
             "picolm_attn_mfma_takes", "picolm_attn_prefill_mfma_heads", "picolm_attn_prefill_mfma_tile_tokens",
@@ -209,22 +209,6 @@ def _check_pages(who, k_pages, v_pages, dtype, G, d):
         raise KernelError(f"{who}: k_pages {tuple(k_pages.shape)} is not [pages, {G}, {PAGE_TOKENS}, {d}]")
     if tuple(v_pages.shape[1:]) != (G, d, PAGE_TOKENS) or v_pages.shape[0] != k_pages.shape[0]:
         raise KernelError(f"{who}: v_pages {tuple(v_pages.shape)} is not [{k_pages.shape[0]}, {G}, {d}, {PAGE_TOKENS}]")
-
-
-def silu_mul(gu: torch.Tensor, out: torch.Tensor) -> None:
-    _dev("silu_mul.gu", gu, (torch.float32, torch.bfloat16))
-    _dev("silu_mul.out", out, (torch.float32, torch.bfloat16))
-    if gu.numel() != 2 * out.numel():
-        raise KernelError("silu_mul: input must hold two values per output")
-    _check(lib().picolm_silu_mul(_ptr(gu), dt_of(gu), _ptr(out), dt_of(out), c_int64(out.numel()), _stream()))
-
-
-def add_into(y: torch.Tensor, x: torch.Tensor) -> None:
-    _dev("add_into.y", y, torch.float32)
-    _dev("add_into.x", x, (torch.float32, torch.bfloat16))
-    if x.numel() != y.numel():
-        raise KernelError("add_into: sizes differ")
-    _check(lib().picolm_add_into(_ptr(y), _ptr(x), dt_of(x), c_int64(y.numel()), _stream()))
 
 
 def gemm_generic(a: torch.Tensor, w: torch.Tensor, c: torch.Tensor, epilogue: int = EPI_STORE) -> None:

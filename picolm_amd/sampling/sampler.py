@@ -81,7 +81,12 @@ class PendingTokens:
         """The tokens as an int32 tensor on the device; `rows` picks some of them, in that order."""
         if rows is None:
             return self._device
-        return self._device[torch.tensor(list(rows), dtype=torch.int64).to(self._device.device)]
+        # the picked rows' indices go up through pinned memory without waiting for the GPU (torch
+        # keeps the pinned block until the copy has run); the gather is queued behind the draw
+        idx = torch.tensor(list(rows), dtype=torch.int64)
+        if self._device.is_cuda:
+            idx = idx.pin_memory().to(self._device.device, non_blocking=True)
+        return self._device.index_select(0, idx)
 
     def wait(self) -> list[int]:
         if self._arrived is not None:

@@ -1,6 +1,6 @@
 """Plain, slow Llama decoder in NumPy float64: whole sequences, no cache, one function a part.
 
-Written from the formulas of whoreson/picolm (cited as file:line under /root/reference/picolm).
+Written from the formulas of whoreson/picolm (cited as file:line of its picolm/ folder).
 It shares no code with picolm_amd: tests compare the engine against it.
 The llama3 frequency scaling is not in the reference; its definition here follows the
 parameter names of the model's config.json (`rope_scaling`).

@@ -54,20 +54,6 @@ def test_rmsnorm(out_dtype, T, D, eps):
     assert torch.equal(out2[0], out[T - 1]) and torch.equal(out2[1], out[0])
 
 
-def test_silu_mul_and_add():
-    g = torch.Generator().manual_seed(2)
-    gu = torch.randn(7, 2 * 33, generator=g).to(DEV)
-    out = torch.empty(7, 33, device=DEV)
-    K().silu_mul(gu, out)
-    ref = P.silu(gu[:, 0::2].double().cpu().numpy()) * gu[:, 1::2].double().cpu().numpy()
-    assert np.abs(out.double().cpu().numpy() - ref).max() < 1e-6
-    y = torch.randn(5, 9, generator=g).to(DEV)
-    x = torch.randn(5, 9, generator=g).to(torch.bfloat16).to(DEV)
-    want = y + x.float()
-    K().add_into(y, x)
-    assert torch.equal(y, want)
-
-
 # ------------------------------------------------------------------------------------------ gemm
 def gemm_ref(a, w, epi, c0):
     y = a.double().cpu() @ w.double().cpu().T
