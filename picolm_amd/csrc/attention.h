@@ -98,10 +98,12 @@ __device__ __forceinline__ int decode_first_page(int window, int qpos) {
 __device__ __forceinline__ bool decode_work(const AttnArgs& a, int per_entry, DecodeWork& w, int& which) {
     const int entry = blockIdx.x / per_entry;
     which = blockIdx.x % per_entry;
-    // the count is one scalar load for the whole workgroup: those past it leave at once
-    if (entry >= a.chunk_list[0]) return false;
+    // The count of entries in use and this workgroup's entry are asked for together (the list has
+    // room for every workgroup of the launch): one trip to memory, not two.  Workgroups past the
+    // count leave at once.
     const int4* e = (const int4*)a.chunk_list + 2 * ((size_t)entry + 1);
     const int4 e0 = e[0], e1 = e[1];
+    if (entry >= a.chunk_list[0]) return false;
     w.seq = e0.x;
     w.split = e0.y;
     w.qpos = e0.z;
