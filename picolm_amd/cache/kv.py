@@ -2,7 +2,8 @@
 live sequence, and fixed-size per-sequence state beside them.
 
 Layout of one KV group: K is [entry][page][kv_head][PAGE_TOKENS][head_dim] and V is kept
-transposed, [entry][page][kv_head][head_dim][PAGE_TOKENS]; an entry is one layer call's cache.  A slot's row of the group's page table maps logical page
+transposed, [entry][page][kv_head][head_dim][PAGE_TOKENS] (with a size of its own where a mixer's values
+are not as wide as its keys); an entry is one layer call's cache.  A slot's row of the group's page table maps logical page
 j (tokens 64j .. 64j+63) to a page; a group that keeps a window of keys maps j modulo its
 ring.  picolm's cache is [kv_layer][pos][G*d] for its one sequence, indexed through
 kv_layer_ordinal (picolm/model_core.c:734-739, :668-681, :1880-1883); the per-layer-call
@@ -25,6 +26,11 @@ class KVGroupSpec:
     n_kv_heads: int
     head_dim: int
     window: int = 0            # 0: all keys are kept; w > 0: the last w keys
+    v_head_dim: int = 0        # size of a value where it is not that of a key
+
+    @property
+    def value_dim(self) -> int:
+        return self.v_head_dim or self.head_dim
 
 
 @dataclass(frozen=True)
@@ -59,13 +65,13 @@ class KVGroup:
         self.book = PagedGroupBook(n_pages, n_slots, self.ring_pages if spec.window > 0 else 0)
         n = max(n_pages, 1)
         self.k = torch.zeros((spec.n_entries, n, spec.n_kv_heads, PAGE_TOKENS, spec.head_dim), dtype=dtype, device=device)
-        self.v = torch.zeros((spec.n_entries, n, spec.n_kv_heads, spec.head_dim, PAGE_TOKENS), dtype=dtype, device=device)
+        self.v = torch.zeros((spec.n_entries, n, spec.n_kv_heads, spec.value_dim, PAGE_TOKENS), dtype=dtype, device=device)
         self.table_host = torch.zeros((n_slots, max_pages), dtype=torch.int32)
         self.table = torch.zeros((n_slots, max_pages), dtype=torch.int32, device=device)
         self.dirty: set[int] = set()
 
     def bytes(self) -> int:
-        return 2 * self.k.numel() * self.k.element_size()
+        return (self.k.numel() + self.v.numel()) * self.k.element_size()
 
 
 class Cache:

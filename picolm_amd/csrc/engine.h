@@ -72,9 +72,11 @@ typedef struct {
     int32_t kv_group, kv_entry, kv_writes, q_buffer;
 } picolm_op;
 
-// Keys and values of `n_entries` layer calls that need the same kind of cache.
+// Keys and values of `n_entries` layer calls that need the same kind of cache.  v_head_dim: the
+// size of a value where it is not that of a key (0: the same); the attention operation here takes
+// one size for both.
 typedef struct {
-    int32_t n_entries, n_kv_heads, head_dim, window;
+    int32_t n_entries, n_kv_heads, head_dim, window, v_head_dim;
 } picolm_kv_group;
 
 // Fixed-size state per sequence for `n_entries` layer calls, zeroed when a slot is given out.

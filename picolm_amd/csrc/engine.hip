@@ -493,6 +493,9 @@ extern "C" int picolm_engine_create(const picolm_program* program, int64_t max_t
         g.spec = program->kv_groups[gi];
         E_REQUIRE(-1, g.spec.n_entries > 0 && g.spec.n_kv_heads > 0 && g.spec.head_dim > 0 && g.spec.window == 0,
                   "engine: cache group %d is ill-formed (this engine keeps all keys, no windows)", gi);
+        E_REQUIRE(-1, g.spec.v_head_dim == 0 || g.spec.v_head_dim == g.spec.head_dim,
+                  "engine: cache group %d has keys of %d and values of %d: the attention operation takes one size for both", gi,
+                  g.spec.head_dim, g.spec.v_head_dim);
         g.max_pages = g.ring_pages = e->max_pages;
         g.n_pages = (int)std::min<int64_t>(n_pages, (int64_t)e->n_slots * e->max_pages);
         g.pool.init(g.n_pages);

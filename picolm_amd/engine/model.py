@@ -87,7 +87,7 @@ class DecoderModel:
                 state_counts[g] += 1
             self.bindings.append(CacheBinding(kv, st, writes=True))
         self.cache_spec = CacheSpec(
-            [KVGroupSpec(n, k.n_kv_heads, k.head_dim, k.window) for k, n in zip(kv_keys, kv_counts)],
+            [KVGroupSpec(n, k.n_kv_heads, k.head_dim, k.window, k.v_head_dim) for k, n in zip(kv_keys, kv_counts)],
             [StateGroupSpec(n, tuple(k.shape), k.dtype) for k, n in zip(state_keys, state_counts)])
 
     def graph_safe(self) -> bool:

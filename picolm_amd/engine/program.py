@@ -40,7 +40,8 @@ class Op(Structure):
 
 
 class KVGroup(Structure):
-    _fields_ = [("n_entries", c_int32), ("n_kv_heads", c_int32), ("head_dim", c_int32), ("window", c_int32)]
+    _fields_ = [("n_entries", c_int32), ("n_kv_heads", c_int32), ("head_dim", c_int32), ("window", c_int32),
+                ("v_head_dim", c_int32)]
 
 
 class StateGroup(Structure):
@@ -150,7 +151,7 @@ class BuiltProgram:
         self.keep = list(b.keep)
         self.ops = (Op * len(b.ops))(*b.ops)
         self.buffers = (Buffer * len(b._specs))(*[Buffer(*s) for s in b._specs])
-        kv = [KVGroup(g.n_entries, g.n_kv_heads, g.head_dim, g.window) for g in cache_spec.kv_groups]
+        kv = [KVGroup(g.n_entries, g.n_kv_heads, g.head_dim, g.window, g.v_head_dim) for g in cache_spec.kv_groups]
         st = []
         for g in cache_spec.state_groups:
             n = g.dtype.itemsize

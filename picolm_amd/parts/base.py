@@ -84,10 +84,20 @@ class Workspace:
 
 @dataclass(frozen=True)
 class KVRequest:
-    """A mixer's need for keys and values of each token."""
+    """A mixer's need for keys and values of each token.  `head_dim` is the size of a key;
+    `v_head_dim` that of a value where it differs (0: the same)."""
     n_kv_heads: int
     head_dim: int
     window: int = 0
+    v_head_dim: int = 0
+
+    def __post_init__(self):
+        if self.v_head_dim == self.head_dim:        # one way to say "the same": requests compare equal
+            object.__setattr__(self, "v_head_dim", 0)
+
+    @property
+    def value_dim(self) -> int:
+        return self.v_head_dim or self.head_dim
 
 
 @dataclass(frozen=True)

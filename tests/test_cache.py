@@ -66,6 +66,16 @@ def test_cache_shapes_and_groups():
     assert c.max_seq_len == 320 and c.max_pages == 5
 
 
+def test_values_of_another_size_than_keys():
+    from picolm_amd.parts import KVRequest
+    assert KVRequest(2, 16, 0, 16) == KVRequest(2, 16) and KVRequest(2, 16).value_dim == 16
+    assert KVRequest(2, 16, 0, 24) != KVRequest(2, 16) and KVRequest(2, 16, 0, 24).value_dim == 24
+    c = Cache(CacheSpec([KVGroupSpec(1, 2, 16, 0, 24)], []), 128, 128, torch.float32, "cpu", 2)
+    (g,) = c.kv
+    assert tuple(g.k.shape) == (1, 2, 2, 64, 16) and tuple(g.v.shape) == (1, 2, 2, 24, 64)
+    assert g.bytes() == 4 * 2 * 2 * 64 * (16 + 24) == c.bytes()
+
+
 def test_reserve_is_all_or_nothing_and_lengths_are_per_slot():
     c = make_cache()
     a, b = c.alloc_slot(), c.alloc_slot()

@@ -22,7 +22,7 @@ def harness(dtype, requests, slots, pos0, new_lens, n_slots=4, max_tokens=1024):
     from picolm_amd.engine.batch import StepBatch
     from picolm_amd.parts import CacheBinding, Runtime, StepContext, Workspace
     kv_req, st_req = requests
-    spec = CacheSpec([KVGroupSpec(1, kv_req.n_kv_heads, kv_req.head_dim, kv_req.window)] if kv_req else [],
+    spec = CacheSpec([KVGroupSpec(1, kv_req.n_kv_heads, kv_req.head_dim, kv_req.window, kv_req.v_head_dim)] if kv_req else [],
                      [StateGroupSpec(1, tuple(st_req.shape), st_req.dtype)] if st_req else [])
     rt = Runtime(DEV, dtype)
     cache = Cache(spec, max_tokens, 512, dtype, DEV, n_slots)
@@ -266,6 +266,114 @@ def test_toy_architecture_with_a_stateful_mixer(tmp_path):
             live = [i for i in live if pos[i] < len(reqs[i])]
     finally:
         unregister_architecture("ToyRunningMeanLM")
+
+
+def test_toy_mixer_whose_values_are_wider_than_its_keys(tmp_path):
+    """A one-head attention defined here with keys of 16 and values of 24: the cache gives its
+    group keys and values of their own sizes.  Whole prompts as an unequal batch, then the same
+    requests cut into a prompt and single tokens in slots that were used before."""
+    from picolm_amd.cache.slots import PAGE_TOKENS
+    from picolm_amd.config import register_architecture, unregister_architecture
+    from picolm_amd.engine import DecoderModel, Session, load_model
+    from picolm_amd.parts import KVRequest, LMHead, Mixer, PreNormBlock, RMSNorm, SwiGLU, TokenEmbedding
+    from picolm_amd.weights import TensorSpec, write_random_model
+    DK, DV = 16, 24
+
+    class ToyConfig:
+        def __init__(self, d):
+            self.d = dict(d)
+            self.hidden_size, self.vocab_size, self.intermediate_size = d["hidden_size"], d["vocab_size"], d["intermediate_size"]
+            self.max_position_embeddings = d["max_position_embeddings"]
+            self.torch_dtype = "bfloat16"
+            self.eos_token_ids = ()
+
+        def to_dict(self):
+            return dict(self.d)
+
+    class NarrowKeys(Mixer):
+        def __init__(self, prefix, D):
+            self.prefix, self.D, self.w = prefix, D, {}
+
+        def tensor_specs(self):
+            return [TensorSpec(self.prefix + "q", (DK, self.D)), TensorSpec(self.prefix + "k", (DK, self.D)),
+                    TensorSpec(self.prefix + "v", (DV, self.D)), TensorSpec(self.prefix + "o", (self.D, DV))]
+
+        def load(self, fetch, runtime):
+            self.w = {n: fetch.get(self.prefix + n).float() for n in "qkvo"}
+
+        def cache_requests(self):
+            return KVRequest(1, DK, 0, DV), None
+
+        def forward(self, ctx, h, residual):
+            k_pages, v_pages, table, _ = ctx.kv()          # [page][1][64][DK], [page][1][DV][64]
+            assert k_pages.shape[-1] == DK and v_pages.shape[-2] == DV
+            b, row = ctx.batch, 0
+            for slot, p0, n in zip(b.slots, b.pos0, b.n_new):
+                x = h[row:row + n].float()
+                q, k, v = x @ self.w["q"].T, x @ self.w["k"].T, x @ self.w["v"].T
+                pos = torch.arange(p0 + n, device=x.device)
+                page, at = table[slot, pos // PAGE_TOKENS].long(), pos % PAGE_TOKENS
+                k_pages[page[p0:], 0, at[p0:]] = k.to(k_pages.dtype)
+                v_pages[page[p0:], 0, :, at[p0:]] = v.to(v_pages.dtype)
+                keys, values = k_pages[page, 0, at].float(), v_pages[page, 0, :, at].float()
+                s = q @ keys.T / math.sqrt(DK)
+                s = s.masked_fill(pos[None, :] > pos[p0:, None], float("-inf"))
+                residual[row:row + n] += (torch.softmax(s, dim=-1) @ values) @ self.w["o"].T
+                row += n
+
+    def build(cfg):
+        D = cfg.hidden_size
+        emb = TokenEmbedding("emb.weight", cfg.vocab_size, D)
+        blocks = [PreNormBlock(RMSNorm(f"l{i}.norm1.weight", D, 1e-5), NarrowKeys(f"l{i}.mix.", D),
+                               RMSNorm(f"l{i}.norm2.weight", D, 1e-5), SwiGLU(f"l{i}.ffn.", D, cfg.intermediate_size)) for i in range(2)]
+        return DecoderModel(cfg, emb, blocks, RMSNorm("final.weight", D, 1e-5),
+                            LMHead("head.weight", cfg.vocab_size, D, emb, tied=True))
+
+    register_architecture("ToyNarrowKeysLM", ToyConfig, build)
+    try:
+        cfg = ToyConfig(dict(architectures=["ToyNarrowKeysLM"], hidden_size=40, vocab_size=77, intermediate_size=56,
+                             max_position_embeddings=256))
+        d = write_random_model(cfg, str(tmp_path / "toy"), seed=5, std=0.3)
+        model = load_model(d, dtype="float32")
+        (group,) = model.cache_spec.kv_groups
+        assert (group.n_entries, group.head_dim, group.value_dim) == (2, DK, DV)
+        assert model.program() is None            # a part without `emit`: stepped part by part
+        w = tiny.read_weights_f64(d)
+
+        def plain(tokens):
+            x = w["emb.weight"][tokens]
+            n = len(tokens)
+            for i in range(2):
+                hh = P.rmsnorm(x, w[f"l{i}.norm1.weight"], 1e-5)
+                q, k, v = (hh @ w[f"l{i}.mix.{c}"].T for c in "qkv")
+                s = q @ k.T / math.sqrt(DK)
+                s[np.triu_indices(n, 1)] = -np.inf
+                p = np.exp(s - s.max(axis=1, keepdims=True))
+                x = x + (p / p.sum(axis=1, keepdims=True)) @ v @ w[f"l{i}.mix.o"].T
+                x = x + P.swiglu(P.rmsnorm(x, w[f"l{i}.norm2.weight"], 1e-5), w[f"l{i}.ffn.gate_proj.weight"],
+                                 w[f"l{i}.ffn.up_proj.weight"], w[f"l{i}.ffn.down_proj.weight"])
+            return P.rmsnorm(x, w["final.weight"], 1e-5) @ w["emb.weight"].T
+        rng = np.random.default_rng(8)
+        reqs = [tiny.random_tokens(rng, n, 77) for n in (70, 3, 130)]
+        truth = [plain(r) for r in reqs]
+        s = Session(model, max_tokens=512, n_slots=3)
+        assert s.cache.kv[0].k.shape[-1] == DK and s.cache.kv[0].v.shape[-2] == DV
+        slots = s.begin(3)
+        got = s.step(slots, reqs, [list(range(len(r))) for r in reqs]).double().cpu().numpy()
+        assert np.abs(got - np.concatenate(truth)).max() < 1e-4
+        s.release(slots)
+        slots = s.begin(3)
+        cut = [60, 1, 126]
+        s.step(slots, [r[:c] for r, c in zip(reqs, cut)])
+        pos, live = dict(zip(range(3), cut)), [0, 1, 2]
+        while live:
+            out = s.step([slots[i] for i in live], [[reqs[i][pos[i]]] for i in live]).double().cpu().numpy()
+            for k, i in enumerate(live):
+                assert np.abs(out[k] - truth[i][pos[i]]).max() < 1e-4
+                pos[i] += 1
+            live = [i for i in live if pos[i] < len(reqs[i])]
+    finally:
+        unregister_architecture("ToyNarrowKeysLM")
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
