@@ -28,6 +28,15 @@ int picolm_rope_kv_store(const float* qkv, void* q_out, void* k_pages, void* v_p
                          const int32_t* tok_page /* physical cache page of every token */, int T, int H, int G,
                          int d, const int32_t* rows /* null: rows 0..T-1 */, hipStream_t stream);
 
+// Keys (rotated) and values of a prefill step into the cache, over the attention kernel's tiles
+// (tile t: up to tile_tokens new tokens of sequence tile_seq[t] from its tile_q0[t]-th on); q is
+// left alone.  d in multiples of 4.
+int picolm_kv_store_tiles(const float* qkv, void* k_pages, void* v_pages, int dt, const float* cos_t,
+                          const float* sin_t, int style, const int32_t* tile_seq, const int32_t* tile_q0, int n_tiles,
+                          int tile_tokens, const int32_t* seq_slot, const int32_t* seq_pos0, const int32_t* seq_nnew,
+                          const int32_t* cu_seqlens, const int32_t* page_table, int max_pages, int ring_pages, int H,
+                          int G, int d, hipStream_t stream);
+
 int picolm_gemm_generic(const void* A, int a_dt, const void* W, int w_dt, void* C, int c_dt, int M,
                         int N, int K, int64_t lda, int64_t ldw, int64_t ldc, int epilogue,
                         hipStream_t stream);
@@ -110,6 +119,15 @@ int picolm_attn_prefill_mfma(const void* q, const void* k_pages, const void* v_p
                              const int32_t* seq_slot, const int32_t* seq_pos0, const int32_t* seq_nnew,
                              const int32_t* cu_seqlens, const int32_t* page_table, int max_pages,
                              int ring_pages, int H, int G, int d, int window, float scale, hipStream_t stream);
+// The same with q taken from the float rows qkv[T][(H+2G)*d] and rotated inside the kernel (tables
+// as in picolm_rope_kv_store, both null for no rotation); the step's keys and values must be in
+// the cache already.
+int picolm_attn_prefill_rope_mfma(const float* qkv, const void* k_pages, const void* v_pages, void* out,
+                                  const int32_t* tile_seq, const int32_t* tile_q0, int n_tiles,
+                                  const int32_t* seq_slot, const int32_t* seq_pos0, const int32_t* seq_nnew,
+                                  const int32_t* cu_seqlens, const int32_t* page_table, int max_pages,
+                                  int ring_pages, int H, int G, int d, int window, float scale,
+                                  const float* cos_t, const float* sin_t, int style, hipStream_t stream);
 int picolm_attn_decode_mfma_waves(int n_seq, int H, int G);      // waves a decode workgroup will have
 // chunks_done: n_seq * G * ceil(H/G / 32) counters that are zero when the call starts and zero again
 // when its kernel has run: the workgroup that finishes a sequence's last chunk combines the chunks,

@@ -153,6 +153,59 @@ __device__ __forceinline__ void attend_tile(const bf16x8 (&Qf)[D / 16], const bf
     }
 }
 
+// A lane's share of a query row as MFMA operands, taken from the float row that the qkv product
+// left and rotated by the position's table row on the way (cos_t null: only rounded).  k-step s of
+// a lane in wave half h covers elements 16s + 8h .. + 8.
+template <int D>
+__device__ __forceinline__ void rotated_q(const AttnArgs& a, const float* row, int pos, int h, bool ok, bf16x8 (&Qf)[D / 16]) {
+    const float* c = a.cos_t ? a.cos_t + (size_t)pos * (D / 2) : nullptr;
+    const float* sn = a.sin_t ? a.sin_t + (size_t)pos * (D / 2) : nullptr;
+#pragma unroll
+    for (int s = 0; s < D / 16; ++s) Qf[s] = zero8();
+    if (!ok) return;
+    if (!c) {
+#pragma unroll
+        for (int s = 0; s < D / 16; ++s) {
+            const f32x4 x0 = *(const f32x4*)(row + 16 * s + 8 * h), x1 = *(const f32x4*)(row + 16 * s + 8 * h + 4);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                Qf[s][e] = to_bf16(x0[e]);
+                Qf[s][4 + e] = to_bf16(x1[e]);
+            }
+        }
+    } else if (a.rope_style == 0) {
+#pragma unroll
+        for (int s = 0; s < D / 16; ++s) {
+            const int d0 = 16 * s + 8 * h;
+            const f32x4 x0 = *(const f32x4*)(row + d0), x1 = *(const f32x4*)(row + d0 + 4);
+            const f32x4 cc = *(const f32x4*)(c + d0 / 2), ss = *(const f32x4*)(sn + d0 / 2);
+            Qf[s][0] = to_bf16(x0[0] * cc[0] - x0[1] * ss[0]);
+            Qf[s][1] = to_bf16(x0[0] * ss[0] + x0[1] * cc[0]);
+            Qf[s][2] = to_bf16(x0[2] * cc[1] - x0[3] * ss[1]);
+            Qf[s][3] = to_bf16(x0[2] * ss[1] + x0[3] * cc[1]);
+            Qf[s][4] = to_bf16(x1[0] * cc[2] - x1[1] * ss[2]);
+            Qf[s][5] = to_bf16(x1[0] * ss[2] + x1[1] * cc[2]);
+            Qf[s][6] = to_bf16(x1[2] * cc[3] - x1[3] * ss[3]);
+            Qf[s][7] = to_bf16(x1[2] * ss[3] + x1[3] * cc[3]);
+        }
+    } else {
+#pragma unroll
+        for (int s = 0; s < D / 32; ++s) {
+            const int d0 = 16 * s + 8 * h;          // below d/2; its partner is d0 + d/2, k-step s + D/32 of this lane
+#pragma unroll
+            for (int half4 = 0; half4 < 2; ++half4) {
+                const f32x4 lo = *(const f32x4*)(row + d0 + 4 * half4), hi = *(const f32x4*)(row + d0 + D / 2 + 4 * half4);
+                const f32x4 cc = *(const f32x4*)(c + d0 + 4 * half4), ss = *(const f32x4*)(sn + d0 + 4 * half4);
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    Qf[s][4 * half4 + e] = to_bf16(lo[e] * cc[e] - hi[e] * ss[e]);
+                    Qf[s + D / 32][4 * half4 + e] = to_bf16(lo[e] * ss[e] + hi[e] * cc[e]);
+                }
+            }
+        }
+    }
+}
+
 // =============================================================================================
 // LDS tiles of the prefill kernel: a page's K and V^T as they lie in the cache, that is in the
 // order of the MFMA operands: the 64 lanes of a wave read 64 adjacent 16-byte chunks.
@@ -210,11 +263,6 @@ __global__ __launch_bounds__(256 * HALVES) __attribute__((amdgpu_waves_per_eu(2)
     const int w_page_hi = w_active ? w_qlast / PAGE_TOKENS + 1 : 0;
 
     bf16x8 Qf[D / 16];
-    {
-        const bf16_t* qp = (const bf16_t*)a.q + tok * a.H * D + (size_t)head * D + 8 * h;
-#pragma unroll
-        for (int s = 0; s < D / 16; ++s) Qf[s] = q_ok ? ldg8(qp + 16 * s) : zero8();
-    }
     f32x16 O[D / 32];
 #pragma unroll
     for (int dt = 0; dt < D / 32; ++dt)
@@ -277,6 +325,14 @@ __global__ __launch_bounds__(256 * HALVES) __attribute__((amdgpu_waves_per_eu(2)
     // the matrix products.)
     fetch(place_of(min(page_of(0), page_hi - 1)));
     int next_place = place_of(min(page_of(1), page_hi - 1));
+    // the queries, while the first page is on its way
+    if (a.qkv) {        // the float rows of the qkv product: rotated here, no rotated copy of q in memory
+        rotated_q<D>(a, a.qkv + tok * (size_t)(a.H + 2 * a.G) * D + (size_t)head * D, qpos, h, q_ok, Qf);
+    } else {
+        const bf16_t* qp = (const bf16_t*)a.q + tok * a.H * D + (size_t)head * D + 8 * h;
+#pragma unroll
+        for (int s = 0; s < D / 16; ++s) Qf[s] = q_ok ? ldg8(qp + 16 * s) : zero8();
+    }
     stash(0, min(page_of(0), page_hi - 1));
     __syncthreads();
     int cur = 0;
@@ -344,56 +400,6 @@ __global__ __launch_bounds__(256 * HALVES) __attribute__((amdgpu_waves_per_eu(2)
 // round key and value to bfloat16 as the cache holds them, put them into the merge below as one
 // more partial result (score, weight 1, value), and one of them writes them to the cache for
 // later steps.  The cache row of the new token is not read in this step.
-template <int D>
-__device__ __forceinline__ void rotated_q(const AttnArgs& a, const float* row, int pos, int h, bool ok, bf16x8 (&Qf)[D / 16]) {
-    const float* c = a.cos_t ? a.cos_t + (size_t)pos * (D / 2) : nullptr;
-    const float* sn = a.sin_t ? a.sin_t + (size_t)pos * (D / 2) : nullptr;
-#pragma unroll
-    for (int s = 0; s < D / 16; ++s) Qf[s] = zero8();
-    if (!ok) return;
-    if (!c) {
-#pragma unroll
-        for (int s = 0; s < D / 16; ++s) {
-            const f32x4 x0 = *(const f32x4*)(row + 16 * s + 8 * h), x1 = *(const f32x4*)(row + 16 * s + 8 * h + 4);
-#pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                Qf[s][e] = to_bf16(x0[e]);
-                Qf[s][4 + e] = to_bf16(x1[e]);
-            }
-        }
-    } else if (a.rope_style == 0) {
-#pragma unroll
-        for (int s = 0; s < D / 16; ++s) {
-            const int d0 = 16 * s + 8 * h;
-            const f32x4 x0 = *(const f32x4*)(row + d0), x1 = *(const f32x4*)(row + d0 + 4);
-            const f32x4 cc = *(const f32x4*)(c + d0 / 2), ss = *(const f32x4*)(sn + d0 / 2);
-            Qf[s][0] = to_bf16(x0[0] * cc[0] - x0[1] * ss[0]);
-            Qf[s][1] = to_bf16(x0[0] * ss[0] + x0[1] * cc[0]);
-            Qf[s][2] = to_bf16(x0[2] * cc[1] - x0[3] * ss[1]);
-            Qf[s][3] = to_bf16(x0[2] * ss[1] + x0[3] * cc[1]);
-            Qf[s][4] = to_bf16(x1[0] * cc[2] - x1[1] * ss[2]);
-            Qf[s][5] = to_bf16(x1[0] * ss[2] + x1[1] * cc[2]);
-            Qf[s][6] = to_bf16(x1[2] * cc[3] - x1[3] * ss[3]);
-            Qf[s][7] = to_bf16(x1[2] * ss[3] + x1[3] * cc[3]);
-        }
-    } else {
-#pragma unroll
-        for (int s = 0; s < D / 32; ++s) {
-            const int d0 = 16 * s + 8 * h;          // below d/2; its partner is d0 + d/2, k-step s + D/32 of this lane
-#pragma unroll
-            for (int half4 = 0; half4 < 2; ++half4) {
-                const f32x4 lo = *(const f32x4*)(row + d0 + 4 * half4), hi = *(const f32x4*)(row + d0 + D / 2 + 4 * half4);
-                const f32x4 cc = *(const f32x4*)(c + d0 + 4 * half4), ss = *(const f32x4*)(sn + d0 + 4 * half4);
-#pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                    Qf[s][4 * half4 + e] = to_bf16(lo[e] * cc[e] - hi[e] * ss[e]);
-                    Qf[s + D / 32][4 * half4 + e] = to_bf16(lo[e] * ss[e] + hi[e] * cc[e]);
-                }
-            }
-        }
-    }
-}
-
 // single accesses that every workgroup of the GPU sees alike
 __device__ __forceinline__ void store_agent(float* p, float v) {
     __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -642,20 +648,11 @@ extern "C" int picolm_attn_prefill_mfma_tile_tokens(int H, int G) {
     return 32 * (4 / picolm_attn_prefill_mfma_heads(H, G));
 }
 
-extern "C" int picolm_attn_prefill_mfma(const void* q, const void* k_pages, const void* v_pages, void* out,
-                                        const int32_t* tile_seq, const int32_t* tile_q0, int n_tiles,
-                                        const int32_t* seq_slot, const int32_t* seq_pos0,
-                                        const int32_t* seq_nnew, const int32_t* cu_seqlens,
-                                        const int32_t* page_table, int max_pages, int ring_pages, int H, int G,
-                                        int d, int window, float scale, hipStream_t stream) {
-    if (check_sizes("attn_prefill_mfma", H, G, d, max_pages, ring_pages)) return -1;
-    if (n_tiles <= 0) return 0;
+static int launch_prefill_mfma(AttnArgs a, int n_tiles, hipStream_t stream) {
+    const int H = a.H, G = a.G, d = a.d;
     const int HB = picolm_attn_prefill_mfma_heads(H, G);
     const int tile_tokens = 32 * (4 / HB);
     const int head_chunks = ceil_div(H / G, HB);
-    AttnArgs a = {q, k_pages, v_pages, out, nullptr, tile_seq, tile_q0, seq_slot, seq_pos0, seq_nnew,
-                  cu_seqlens, page_table, max_pages, ring_pages, H, G, d, window, scale, 0, nullptr, 0, 1,
-                  nullptr, nullptr, nullptr, nullptr, 0};
     PICOLM_REQUIRE((int64_t)n_tiles * G * head_chunks < (1ll << 31), "attn_prefill_mfma: too many workgroups");
     static int n_cus = 0;
     if (n_cus == 0) {
@@ -693,6 +690,42 @@ extern "C" int picolm_attn_prefill_mfma(const void* q, const void* k_pages, cons
 #undef PREFILL_LAUNCH
     PICOLM_LAUNCH_CHECK("attn_prefill_mfma");
     return 0;
+}
+
+extern "C" int picolm_attn_prefill_mfma(const void* q, const void* k_pages, const void* v_pages, void* out,
+                                        const int32_t* tile_seq, const int32_t* tile_q0, int n_tiles,
+                                        const int32_t* seq_slot, const int32_t* seq_pos0,
+                                        const int32_t* seq_nnew, const int32_t* cu_seqlens,
+                                        const int32_t* page_table, int max_pages, int ring_pages, int H, int G,
+                                        int d, int window, float scale, hipStream_t stream) {
+    if (check_sizes("attn_prefill_mfma", H, G, d, max_pages, ring_pages)) return -1;
+    if (n_tiles <= 0) return 0;
+    AttnArgs a = {q, k_pages, v_pages, out, nullptr, tile_seq, tile_q0, seq_slot, seq_pos0, seq_nnew,
+                  cu_seqlens, page_table, max_pages, ring_pages, H, G, d, window, scale, 0, nullptr, 0, 1,
+                  nullptr, nullptr, nullptr, nullptr, 0};
+    return launch_prefill_mfma(a, n_tiles, stream);
+}
+
+// The same with the queries taken from the float rows qkv[T][(H+2G)*d] of the step and rotated on
+// their way into the kernel (cos_t, sin_t [positions][d/2], both null: no rotation; style as in
+// picolm_rope_kv_store): no rotated copy of q is written or read.  The keys and values of the
+// step's tokens must be in the cache already (picolm_rope_kv_store with q_out null).
+extern "C" int picolm_attn_prefill_rope_mfma(const float* qkv, const void* k_pages, const void* v_pages, void* out,
+                                             const int32_t* tile_seq, const int32_t* tile_q0, int n_tiles,
+                                             const int32_t* seq_slot, const int32_t* seq_pos0,
+                                             const int32_t* seq_nnew, const int32_t* cu_seqlens,
+                                             const int32_t* page_table, int max_pages, int ring_pages, int H, int G,
+                                             int d, int window, float scale, const float* cos_t, const float* sin_t,
+                                             int style, hipStream_t stream) {
+    if (check_sizes("attn_prefill_rope_mfma", H, G, d, max_pages, ring_pages)) return -1;
+    PICOLM_REQUIRE(qkv != nullptr && ((uintptr_t)qkv & 15) == 0, "attn_prefill_rope_mfma: the qkv rows must be 16-byte aligned");
+    PICOLM_REQUIRE((cos_t == nullptr) == (sin_t == nullptr), "attn_prefill_rope_mfma: need both tables or none");
+    PICOLM_REQUIRE(style == 0 || style == 1, "attn_prefill_rope_mfma: unknown pairing %d", style);
+    if (n_tiles <= 0) return 0;
+    AttnArgs a = {nullptr, k_pages, v_pages, out, nullptr, tile_seq, tile_q0, seq_slot, seq_pos0, seq_nnew,
+                  cu_seqlens, page_table, max_pages, ring_pages, H, G, d, window, scale, 0, nullptr, 0, 1,
+                  qkv, cos_t, sin_t, nullptr, style};
+    return launch_prefill_mfma(a, n_tiles, stream);
 }
 
 int check_decode_chunks(const char* who, const float* partial, const int32_t* chunk_list, int n_chunks,

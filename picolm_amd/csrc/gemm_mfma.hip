@@ -339,7 +339,7 @@ static int launch_skinny_resident(const void* A, const void* W, void* C, int c_d
 // would leave a last round of the CUs mostly empty, the multiple of 8 up to 64 with which the
 // launch takes the fewest rows per CU (6144 rows on 256 CUs: 24 rows each instead of 16 in one
 // and a half rounds).
-static int skinny_rows_per_wg(int N) {
+static int skinny_rows_per_wg(int N, int M) {
     const int cus = n_compute_units();
     int best = 16;
     int64_t best_cost = (int64_t)ceil_div(ceil_div(N, 16), cus) * 16 * 4;
@@ -348,7 +348,10 @@ static int skinny_rows_per_wg(int N) {
         // second time cost no memory traffic but a quarter of their share of load instructions
         const int padded = (rows + 15) / 16 * 16;
         const int64_t cost = (int64_t)ceil_div(ceil_div(N, rows), cus) * (4 * rows + (padded - rows));
-        if (cost < best_cost) {
+        // as cheap with fewer, larger workgroups: every workgroup reads all the activations, so with
+        // many rows the fewer win (12288 x 4096: 22 against 26 us at 16 rows), with one row the more
+        // (20 against 22 us)
+        if (cost < best_cost || (cost == best_cost && M > 8)) {
             best = rows;
             best_cost = cost;
         }
@@ -358,7 +361,7 @@ static int skinny_rows_per_wg(int N) {
 template <int MT>
 static int launch_skinny_sized(const void* A, const void* W, void* C, int c_dt, int M, int N, int K, int64_t lda,
                                int64_t ldw, int64_t ldc, int epi, hipStream_t stream, NormLink link) {
-    const int rows = link.next_w ? 16 : skinny_rows_per_wg(N);
+    const int rows = link.next_w ? 16 : skinny_rows_per_wg(N, M);
     if (rows <= 16) return launch_skinny<MT, 1, 8>(A, W, C, c_dt, M, N, K, lda, ldw, ldc, epi, stream, link, rows);
     if (rows <= 32) return launch_skinny<MT, 2, 8>(A, W, C, c_dt, M, N, K, lda, ldw, ldc, epi, stream, link, rows);
     if (rows <= 48) return launch_skinny<MT, 3, 8>(A, W, C, c_dt, M, N, K, lda, ldw, ldc, epi, stream, link, rows);

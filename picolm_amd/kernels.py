@@ -141,11 +141,14 @@ def rope_kv_store(qkv, q_out, k_pages, v_pages, cos, sin, style: int, tok_pos, t
     T = qkv.shape[0]
     if qkv.shape[1] != (H + 2 * G) * d:
         raise KernelError(f"rope: qkv has {qkv.shape[1]} columns, (H+2G)d = {(H + 2 * G) * d}")
-    _dev("rope.q_out", q_out, (torch.float32, torch.bfloat16), 2)
-    if tuple(q_out.shape) != (T, H * d):
-        raise KernelError(f"rope: q_out {tuple(q_out.shape)} is not {(T, H * d)}")
+    if q_out is None and k_pages is None:
+        raise KernelError("rope: neither q nor the cache to write")
+    if q_out is not None:
+        _dev("rope.q_out", q_out, (torch.float32, torch.bfloat16), 2)
+        if tuple(q_out.shape) != (T, H * d):
+            raise KernelError(f"rope: q_out {tuple(q_out.shape)} is not {(T, H * d)}")
     if k_pages is not None:
-        _check_pages("rope", k_pages, v_pages, q_out.dtype, G, d)
+        _check_pages("rope", k_pages, v_pages, q_out.dtype if q_out is not None else k_pages.dtype, G, d)
         _i32("rope.tok_page", tok_page, T)
     if cos is not None:
         _dev("rope.cos", cos, torch.float32, 2)
@@ -160,7 +163,7 @@ def rope_kv_store(qkv, q_out, k_pages, v_pages, cos, sin, style: int, tok_pos, t
         if n_launch > T:
             raise KernelError("rope: more rows listed than there are")
     _check(lib().picolm_rope_kv_store(
-        _ptr(qkv), _ptr(q_out), _ptr(k_pages), _ptr(v_pages), dt_of(q_out), _ptr(cos), _ptr(sin), style,
+        _ptr(qkv), _ptr(q_out), _ptr(k_pages), _ptr(v_pages), dt_of(q_out if q_out is not None else k_pages), _ptr(cos), _ptr(sin), style,
         _ptr(tok_pos), _ptr(tok_page if k_pages is not None else None), n_launch, H, G, d, _ptr(rows), _stream()))
 
 
@@ -427,6 +430,56 @@ def attn_prefill_mfma(q, k_pages, v_pages, out, batch, page_table, ring_pages, H
         _ptr(q), _ptr(k_pages), _ptr(v_pages), _ptr(out), _ptr(tile_seq), _ptr(tile_q0), n_tiles,
         _ptr(batch.seq_slot), _ptr(batch.seq_pos0), _ptr(batch.seq_nnew), _ptr(batch.cu_seqlens), _ptr(page_table),
         page_table.shape[1], ring_pages, H, G, d, window, c_float(scale), _stream()))
+
+
+def kv_store_tiles(qkv, k_pages, v_pages, cos, sin, style: int, batch, page_table, ring_pages: int, H: int, G: int, d: int) -> None:
+    """Keys (rotated) and values of a prefill step's tokens into the cache, over the tiles of the
+    matrix-core attention kernel; q is left to that kernel (attn_prefill_rope)."""
+    _dev("kv_store.qkv", qkv, torch.float32, 2)
+    if qkv.shape[1] != (H + 2 * G) * d or qkv.shape[0] < batch.T:
+        raise KernelError(f"kv_store_tiles: qkv {tuple(qkv.shape)} is not [{batch.T}, {(H + 2 * G) * d}]")
+    _check_pages("kv_store_tiles", k_pages, v_pages, k_pages.dtype, G, d)
+    _dev("kv_store.page_table", page_table, torch.int32, 2)
+    if cos is not None:
+        _dev("kv_store.cos", cos, torch.float32, 2)
+        _dev("kv_store.sin", sin, torch.float32, 2)
+        if cos.shape[1] != d // 2 or sin.shape != cos.shape or cos.shape[0] < batch.max_len:
+            raise KernelError(f"kv_store_tiles: tables {tuple(cos.shape)} do not cover {batch.max_len} positions of d/2 = {d // 2}")
+    tile_tokens = lib().picolm_attn_prefill_mfma_tile_tokens(H, G)
+    tile_seq, tile_q0, n_tiles = batch.prefill_tiles(tile_tokens)
+    _check(lib().picolm_kv_store_tiles(
+        _ptr(qkv), _ptr(k_pages), _ptr(v_pages), dt_of(k_pages), _ptr(cos), _ptr(sin), style, _ptr(tile_seq), _ptr(tile_q0),
+        n_tiles, tile_tokens, _ptr(batch.seq_slot), _ptr(batch.seq_pos0), _ptr(batch.seq_nnew), _ptr(batch.cu_seqlens),
+        _ptr(page_table), page_table.shape[1], ring_pages, H, G, d, _stream()))
+
+
+def attn_prefill_rope_takes(dtype: torch.dtype, d: int) -> bool:
+    """Whether the prefill attention that rotates q itself takes this case."""
+    return dtype == torch.bfloat16 and bool(lib().picolm_attn_mfma_takes(d))
+
+
+def attn_prefill_rope(qkv, k_pages, v_pages, out, batch, page_table, ring_pages, H, G, d, window, scale, cos, sin, style) -> None:
+    """attn_prefill_mfma with q taken from the float rows qkv [T, (H+2G)d] and rotated inside the
+    kernel (cos, sin None: no rotation).  The step's keys and values must be in the cache already
+    (rope_kv_store with q_out None)."""
+    _dev("attn.qkv", qkv, torch.float32, 2)
+    if qkv.shape[1] != (H + 2 * G) * d or qkv.shape[0] < batch.T:
+        raise KernelError(f"attn_prefill_rope: qkv {tuple(qkv.shape)} is not [{batch.T}, {(H + 2 * G) * d}]")
+    _dev("attn.out", out, torch.bfloat16, 2)
+    if tuple(out.shape) != (qkv.shape[0], H * d):
+        raise KernelError(f"attn_prefill_rope: out {tuple(out.shape)} is not {(qkv.shape[0], H * d)}")
+    _check_pages("attn_prefill_rope", k_pages, v_pages, torch.bfloat16, G, d)
+    _dev("attn.page_table", page_table, torch.int32, 2)
+    if cos is not None:
+        _dev("attn.cos", cos, torch.float32, 2)
+        _dev("attn.sin", sin, torch.float32, 2)
+        if cos.shape[1] != d // 2 or sin.shape != cos.shape or cos.shape[0] < batch.max_len:
+            raise KernelError(f"attn_prefill_rope: tables {tuple(cos.shape)} do not cover {batch.max_len} positions of d/2 = {d // 2}")
+    tile_seq, tile_q0, n_tiles = batch.prefill_tiles(lib().picolm_attn_prefill_mfma_tile_tokens(H, G))
+    _check(lib().picolm_attn_prefill_rope_mfma(
+        _ptr(qkv), _ptr(k_pages), _ptr(v_pages), _ptr(out), _ptr(tile_seq), _ptr(tile_q0), n_tiles,
+        _ptr(batch.seq_slot), _ptr(batch.seq_pos0), _ptr(batch.seq_nnew), _ptr(batch.cu_seqlens), _ptr(page_table),
+        page_table.shape[1], ring_pages, H, G, d, window, c_float(scale), _ptr(cos), _ptr(sin), style, _stream()))
 
 
 def attn_decode_counters(n_seq: int, H: int, G: int) -> int:

@@ -428,6 +428,61 @@ def test_attention_prefill_with_more_tiles_than_places(H, G, d, old, new):
     assert err <= tol(torch.bfloat16, np.abs(ref).max()), err
 
 
+@pytest.mark.parametrize("H,G,d", [(6, 6, 32), (8, 2, 64), (32, 8, 128), (40, 1, 64)])
+@pytest.mark.parametrize("style", ["pairwise", "half", None])
+@pytest.mark.parametrize("window", [0, 70])
+def test_attention_prefill_with_rotation_inside(H, G, d, style, window):
+    """The prefill step of the matrix-core path: the rotation kernel writes only keys and values
+    (no rotated copy of q), and the attention kernel takes q unrotated in float and rotates it on
+    the way in.  New tokens that start a sequence, continue one inside a page and across pages;
+    their cache rows hold NaN beforehand."""
+    old, new = [0, 0, 5, 130], [1, 200, 67, 33]
+    case = PagedCase(H, G, d, old, new, torch.bfloat16, seed=H + d)
+    b = case.batch()
+    T = sum(new)
+    rng = np.random.default_rng(11)
+    qkv = rng.standard_normal((T, (H + 2 * G) * d)).astype(np.float32)
+    inv = P.rope_inv_freq(d, 10000.0)
+    positions = np.concatenate([np.arange(o, o + n) for o, n in zip(old, new)])
+    cos, sin = P.rope_tables(np.arange(256), inv)
+    x = qkv.astype(np.float64).reshape(T, H + 2 * G, d)
+    if style is None:
+        q_ref, k_ref = x[:, :H], x[:, H:H + G]
+    else:
+        c, s = P.rope_tables(positions, inv)
+        q_ref, k_ref = P.apply_rope(x[:, :H], c, s, style), P.apply_rope(x[:, H:H + G], c, s, style)
+    v_ref = x[:, H + G:]
+    bf = lambda t: torch.from_numpy(np.ascontiguousarray(t)).to(torch.bfloat16)
+    row = 0
+    for i, (o, n) in enumerate(zip(old, new)):
+        case.q[i][o:] = bf(q_ref[row:row + n]).double().numpy()
+        case.k[i][o:] = bf(k_ref[row:row + n]).double().numpy()
+        case.v[i][o:] = bf(v_ref[row:row + n]).double().numpy()
+        row += n
+    ref = case.reference(window)
+    tok_page = b.write_pages(0, case.table_host, case.table_host.shape[1])
+    k_plain, v_plain = K().kv_pages_unpack(case.k_pages, case.v_pages)
+    for t in range(T):
+        k_plain[int(tok_page[t]), :, positions[t] % PAGE, :] = float("nan")
+        v_plain[int(tok_page[t]), :, :, positions[t] % PAGE] = float("nan")
+    case.k_pages, case.v_pages = K().kv_pages_pack(k_plain, v_plain)
+    dev = lambda t: None if style is None else torch.from_numpy(t).float().to(DEV)
+    st = 0 if style != "half" else 1
+    qkv_dev = torch.from_numpy(qkv).to(DEV)
+    K().kv_store_tiles(qkv_dev, case.k_pages, case.v_pages, dev(cos), dev(sin), st, b, case.table, case.table.shape[1], H, G, d)
+    out = torch.zeros(T, H * d, dtype=torch.bfloat16, device=DEV)
+    K().attn_prefill_rope(qkv_dev, case.k_pages, case.v_pages, out, b, case.table, case.table.shape[1], H, G, d, window,
+                          1.0 / math.sqrt(d), dev(cos), dev(sin), st)
+    err = np.abs(out.double().cpu().numpy() - ref).max()
+    assert err <= tol(torch.bfloat16, np.abs(ref).max()), err
+    k_plain, v_plain = K().kv_pages_unpack(case.k_pages, case.v_pages)
+    for t in range(T):
+        pg, r = int(tok_page[t]), positions[t] % PAGE
+        # (a key rotated in 32-bit and one rotated in 64-bit may round to neighbouring bfloat16 values)
+        assert np.abs(k_plain[pg, :, r, :].double().cpu().numpy() - k_ref[t]).max() <= tol(torch.bfloat16, 4.0)
+        assert torch.equal(v_plain[pg, :, :, r].cpu(), bf(v_ref[t]))
+
+
 def decode_work_list(case, window, pages_per_chunk, spare=0):
     """The work list the engine would build, with room for `spare` more entries behind it (a
     recorded step's list has room for full-length sequences): those hold garbage."""
@@ -644,6 +699,14 @@ def test_rope_kv_store(dtype, style):
         pg = tab[slots[seq_of[t]], positions[t] // PAGE]
         assert np.abs(kp[pg, :, positions[t] % PAGE, :] - k_ref[t]).max() <= t_
         assert np.abs(vp[pg, :, :, positions[t] % PAGE] - v_ref[t]).max() <= t_
+    # the kernel that writes only keys and values, tile by tile (values in runs of eight keys where
+    # the tokens fill one: the first sequence starts at 61, the second at 0)
+    kp2 = torch.zeros(6, G, PAGE, d, dtype=dtype, device=DEV)
+    vp2 = torch.zeros(6, G, d, PAGE, dtype=dtype, device=DEV)
+    K().kv_store_tiles(torch.from_numpy(qkv).to(DEV), kp2, vp2, torch.from_numpy(cos).float().to(DEV),
+                       torch.from_numpy(sin).float().to(DEV), 0 if style == "pairwise" else 1, b, table, 2, H, G, d)
+    kp2, vp2 = K().kv_pages_unpack(kp2, vp2)
+    assert np.abs(kp2.double().cpu().numpy() - kp).max() <= t_ and np.array_equal(vp2.double().cpu().numpy(), vp)
 
 
 # ------------------------------------------------------------------------------------------ sampling
