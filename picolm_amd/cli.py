@@ -8,6 +8,10 @@ prompt, and several lines make a batch.  Timings go to standard error in picolm'
   picolm <model_dir> [-p "1 5 17"] [-n 256] [-t 0.8] [-k 40] [--top-p 0.9] [--min-p 0.05]
          [-s 42] [-c CONTEXT] [--dtype bfloat16|float32] [--batch-file FILE] [--batch N]
   picolm --random-model OUT_DIR --config CONFIG.json [-s SEED] [--std 0.02] [--norm-sigma 0]
+  picolm <model_dir> --benchmark [-p ...] [-n N]         prompt and generation again and again
+  picolm <model_dir> --benchmark-ctx [-p ...] [-n N] [-c CONTEXT]     speed over a growing context (CSV)
+  picolm --gpu-diff S I O | --gpu-attn-diff N_TOK N_HEADS N_KV_HEADS HEAD_DIM     kernels against slow ones
+  picolm <model_dir> --list-tensors | --list-kv
 """
 from __future__ import annotations
 
@@ -48,6 +52,16 @@ def build_parser() -> argparse.ArgumentParser:
     ap.add_argument("--std", type=float, default=0.02)
     ap.add_argument("--norm-sigma", type=float, default=0.0)
     ap.add_argument("--list-tensors", action="store_true", help="list the model folder's tensors and exit")
+    ap.add_argument("--list-kv", action="store_true", help="list the model folder's metadata entries and exit")
+    ap.add_argument("--gpu-diff", nargs=3, type=int, metavar=("S", "I", "O"),
+                    help="diff the product kernels (matrix cores, 32-bit, float64 on the host) on random input: S rows, I inputs, O outputs")
+    ap.add_argument("--gpu-attn-diff", nargs=4, type=int, metavar=("N_TOK", "N_HEADS", "N_KV_HEADS", "HEAD_DIM"),
+                    help="diff the attention kernels (bfloat16, 32-bit, float64 on the host) on random q, k, v")
+    ap.add_argument("--benchmark-ctx", action="store_true",
+                    help="prefill and generation speed at growing context sizes: -p is appended and answered over the cached "
+                         "context, then -n tokens are generated, until -c is full; CSV ctx_size,prefill_tok/s,gen_tok/s")
+    ap.add_argument("--benchmark", action="store_true", help="continuous benchmark loop (Ctrl-C to stop)")
+    ap.add_argument("--benchmark-iterations", type=int, default=0, help="stop --benchmark after this many rounds (0: never)")
     return ap
 
 
@@ -63,6 +77,12 @@ def main(argv=None) -> int:
         write_random_model(cfg, args.random_model, seed=args.seed, std=args.std, norm_sigma=args.norm_sigma)
         print(args.random_model)
         return 0
+    if args.gpu_diff:              # stand-alone kernel checks: no model needed (picolm.c:950-963)
+        from .diagnostics import gpu_diff
+        return gpu_diff(*args.gpu_diff, seed=args.seed)
+    if args.gpu_attn_diff:
+        from .diagnostics import gpu_attn_diff
+        return gpu_attn_diff(*args.gpu_attn_diff, seed=args.seed)
     if not args.model:
         build_parser().print_usage(sys.stderr)
         print("No model folder specified", file=sys.stderr)
@@ -74,6 +94,9 @@ def main(argv=None) -> int:
             dt, shape = ck.info(n)
             print(f"{n}\t{list(shape)}\t{str(dt).replace('torch.', '')}")
         return 0
+    if args.list_kv:
+        from .diagnostics import list_kv
+        return list_kv(args.model)
     if args.batch_file:
         with open(args.batch_file) as f:
             lines = [l for l in f.read().splitlines() if l.strip()]
@@ -98,9 +121,16 @@ def main(argv=None) -> int:
             raise SystemExit("no prompt given, and this model's configuration names no start token (bos_token_id)")
         prompts = [[int(bos)]]
     context = args.context or cfg.max_position_embeddings
+    params = SamplingParams(args.temperature, args.top_k, args.top_p, args.min_p, args.seed)
+    if args.benchmark or args.benchmark_ctx:        # one sequence, speed only (picolm.c:969-976, :1311)
+        from . import diagnostics
+        context = min(context, cfg.max_position_embeddings)
+        session = Session(model, max_tokens=pages_for(context) * PAGE_TOKENS, max_seq_len=context, n_slots=1)
+        if args.benchmark_ctx:
+            return diagnostics.benchmark_ctx(session, prompts[0], args.max_tokens, context, params)
+        return diagnostics.benchmark(session, prompts[0], args.max_tokens, params, args.benchmark_iterations)
     per = sorted((pages_for(min(len(p) + args.max_tokens, context)) for p in prompts), reverse=True)
     session = Session(model, max_tokens=max(1, sum(per[:args.batch])) * PAGE_TOKENS, max_seq_len=context)
-    params = SamplingParams(args.temperature, args.top_k, args.top_p, args.min_p, args.seed)
     results, stats = generate(session, prompts, args.max_tokens, params, batch_size=args.batch, return_stats=True)
     if args.json:
         print(json.dumps({"tokens": [r.tokens for r in results], "finish": [r.finish for r in results],

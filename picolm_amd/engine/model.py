@@ -119,6 +119,17 @@ class DecoderModel:
             p.load_all(fetch, runtime)
         return self
 
+    def weight_bytes(self) -> int:
+        """Bytes of the declared tensors at the runtime's element size: about what a decode step reads."""
+        size = self.runtime.dtype.itemsize if self.runtime is not None else 2
+        total = 0
+        for spec in self.tensor_specs():
+            n = 1
+            for d in spec.shape:
+                n *= int(d)
+            total += n * size
+        return total
+
     def new_cache(self, max_tokens: int, max_seq_len: int | None = None, n_slots: int | None = None) -> Cache:
         limit = getattr(self.config, "max_position_embeddings", None) or max_tokens
         max_seq_len = min(max_seq_len or limit, limit)

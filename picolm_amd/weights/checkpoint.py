@@ -109,6 +109,13 @@ class Checkpoint:
     def names(self):
         return list(self._where)
 
+    def metadata(self) -> dict:
+        """What the files' headers carry beside tensors (`__metadata__`), all files together."""
+        out = {}
+        for sf in self._files:
+            out.update({str(k): v for k, v in sf.metadata.items()})
+        return out
+
     def info(self, name):
         sf, n = self._where[name]
         return sf.info(n)

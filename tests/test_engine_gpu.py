@@ -299,6 +299,29 @@ def test_command_line(folders, tmp_path):
     assert "model.layers.0.self_attn.q_proj.weight\t[96, 80]\tbfloat16" in ls.stdout
 
 
+def test_command_line_checks_and_speed_runs(folders, capsys):
+    """picolm's --gpu-diff, --gpu-attn-diff, --benchmark-ctx and --benchmark, run in this process."""
+    from picolm_amd import cli
+    # products: a decode batch, a wide decode batch, a prompt (three kernels of the matrix-core path)
+    for S, I, O in ((8, 512, 1024), (40, 1024, 520), (300, 192, 1031)):
+        assert cli.main(["--gpu-diff", str(S), str(I), str(O)]) == 0
+    err = capsys.readouterr().err
+    assert err.count("PASS") == 3 and "matrix-core kernel against float64" in err
+    # attention: a head size of the matrix-core kernels, and one that only the plain kernels take
+    assert cli.main(["--gpu-attn-diff", "200", "8", "2", "64"]) == 0
+    assert cli.main(["--gpu-attn-diff", "70", "6", "3", "20", "-s", "5"]) == 0
+    assert capsys.readouterr().err.count("PASS") == 2
+    d = folders["A"]
+    assert cli.main([d, "--benchmark-ctx", "-p", "5 6 7 8 9", "-n", "11", "-c", "100", "-t", "0"]) == 0
+    rows = [l for l in capsys.readouterr().err.splitlines() if l and l[0].isdigit()]
+    # 16 tokens a step into a context of 100: steps at 0, 16, ..., 80
+    assert [int(r.split(",")[0]) for r in rows] == list(range(0, 96, 16)) and all(float(x) > 0 for r in rows for x in r.split(",")[1:])
+    assert cli.main([d, "--benchmark", "--benchmark-iterations", "2", "-p", "5 6 7", "-n", "9", "-t", "0.7"]) == 0
+    err = capsys.readouterr().err
+    assert "--- Iteration 2" in err and "--- Iteration 3" not in err
+    assert err.count("Prefill: 3 tokens") == 2 and err.count("Generation: 9 tokens") == 2
+
+
 def test_missing_tensor_is_reported_when_loading(folders, tmp_path):
     from safetensors.torch import load_file, save_file
     from picolm_amd import WeightsError

@@ -175,3 +175,15 @@ def test_sharded_folder(tmp_path):
     assert torch.equal(ck.tensor(names[9]), t[names[9]])
     with pytest.raises(SafetensorsError, match="no model.safetensors"):
         Checkpoint(str(tmp_path))
+
+
+def test_list_kv_prints_the_folders_metadata(tmp_path, capsys):
+    """picolm's --list-kv (picolm/picolm.c:187): here config.json's entries and the safetensors metadata."""
+    from picolm_amd import LlamaConfig, cli, write_random_model
+    d = write_random_model(LlamaConfig.from_dict(tiny.TINY_A), str(tmp_path / "m"), seed=1)
+    assert cli.main([d, "--list-kv"]) == 0
+    out = capsys.readouterr().out.splitlines()
+    assert f"config.hidden_size = {tiny.TINY_A['hidden_size']}" in out
+    assert 'config.architectures = ["LlamaForCausalLM"]' in out
+    assert out == sorted(out, key=lambda l: (not l.startswith("config."), l))
+
