@@ -122,6 +122,7 @@ int picolm_attn_prefill_mfma(const void* q, const void* k_pages, const void* v_p
 // The same with q taken from the float rows qkv[T][(H+2G)*d] and rotated inside the kernel (tables
 // as in picolm_rope_kv_store, both null for no rotation); the step's keys and values must be in
 // the cache already.
+int picolm_attn_prefill_rotates_q(int T);      // whether a step of T tokens should take this way (long prompts gain, short ones lose)
 int picolm_attn_prefill_rope_mfma(const float* qkv, const void* k_pages, const void* v_pages, void* out,
                                   const int32_t* tile_seq, const int32_t* tile_q0, int n_tiles,
                                   const int32_t* seq_slot, const int32_t* seq_pos0, const int32_t* seq_nnew,

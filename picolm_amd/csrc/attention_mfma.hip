@@ -706,6 +706,14 @@ extern "C" int picolm_attn_prefill_mfma(const void* q, const void* k_pages, cons
     return launch_prefill_mfma(a, n_tiles, stream);
 }
 
+// Whether a prefill step of T tokens should let the attention kernel rotate q itself
+// (picolm_kv_store_tiles + picolm_attn_prefill_rope_mfma) rather than read a rotated copy
+// (picolm_rope_kv_store + picolm_attn_prefill_mfma).  Without the copy a layer of 2,048 tokens
+// takes 84 us for the two kernels instead of 94, one of 8,192 tokens 4 % less; but a short prompt
+// has few workgroups, each of which then rotates its queries before it can start, where the
+// rotation kernel spreads that over the GPU: 24 us against 17 at 128 tokens, 32 against 30 at 512.
+extern "C" int picolm_attn_prefill_rotates_q(int T) { return T >= 1024; }
+
 // The same with the queries taken from the float rows qkv[T][(H+2G)*d] of the step and rotated on
 // their way into the kernel (cos_t, sin_t [positions][d/2], both null: no rotation; style as in
 // picolm_rope_kv_store): no rotated copy of q is written or read.  The keys and values of the

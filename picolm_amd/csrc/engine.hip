@@ -1011,7 +1011,7 @@ static int run_attention(Run& r, const picolm_op& o) {
     }
     const TileList* tl = p.tiles_of(mfma ? picolm_attn_prefill_mfma_tile_tokens(H, G) : picolm_attn_prefill_tile_rows());
     E_REQUIRE(-1, tl != nullptr, "attention: the step has no tiles of the height this kernel takes");
-    if (mfma) {         // keys and values go to the cache; the attention kernel rotates q on its way in
+    if (mfma && picolm_attn_prefill_rotates_q(p.T)) {      // keys and values go to the cache; the attention kernel rotates q on its way in
         if (writes)
             TRY(picolm_kv_store_tiles(qkv, k_pages, v_pages, dt, o.cos_table, o.sin_table, o.rope_style, p.at(tl->seq), p.at(tl->q0), tl->n,
                                       tl->rows_per_tile, p.at(p.seq_slot), p.at(p.seq_pos0), p.at(p.seq_nnew), p.at(p.cu_seqlens),
@@ -1022,6 +1022,10 @@ static int run_attention(Run& r, const picolm_op& o) {
     }
     TRY(picolm_rope_kv_store(qkv, q, writes ? k_pages : nullptr, writes ? v_pages : nullptr, dt, o.cos_table, o.sin_table, o.rope_style,
                              p.at(p.tok_pos), tok_page, p.T, H, G, d, nullptr, r.stream));
+    if (mfma)
+        return picolm_attn_prefill_mfma(q, k_pages, v_pages, out, p.at(tl->seq), p.at(tl->q0), tl->n, p.at(p.seq_slot), p.at(p.seq_pos0),
+                                        p.at(p.seq_nnew), p.at(p.cu_seqlens), g.table_dev, g.max_pages, g.ring_pages, H, G, d, o.window,
+                                        o.scale, r.stream);
     return picolm_attn_prefill_generic(q, k_pages, v_pages, out, dt, p.at(tl->seq), p.at(tl->q0), tl->n, p.at(p.seq_slot),
                                        p.at(p.seq_pos0), p.at(p.seq_nnew), p.at(p.cu_seqlens), g.table_dev, g.max_pages, g.ring_pages, H,
                                        G, d, o.window, o.scale, r.stream);

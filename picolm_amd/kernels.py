@@ -453,9 +453,12 @@ def kv_store_tiles(qkv, k_pages, v_pages, cos, sin, style: int, batch, page_tabl
         _ptr(page_table), page_table.shape[1], ring_pages, H, G, d, _stream()))
 
 
-def attn_prefill_rope_takes(dtype: torch.dtype, d: int) -> bool:
-    """Whether the prefill attention that rotates q itself takes this case."""
-    return dtype == torch.bfloat16 and bool(lib().picolm_attn_mfma_takes(d))
+def attn_prefill_rope_takes(dtype: torch.dtype, d: int, T: int | None = None) -> bool:
+    """Whether the prefill attention that rotates q itself takes this case and, given the step's
+    number of tokens, whether the library would take that way (long prompts gain by it)."""
+    if not (dtype == torch.bfloat16 and bool(lib().picolm_attn_mfma_takes(d))):
+        return False
+    return T is None or bool(lib().picolm_attn_prefill_rotates_q(int(T)))
 
 
 def attn_prefill_rope(qkv, k_pages, v_pages, out, batch, page_table, ring_pages, H, G, d, window, scale, cos, sin, style) -> None:

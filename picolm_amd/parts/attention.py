@@ -113,7 +113,7 @@ class Attention(Mixer):
                 kernels.rope_kv_store(qkv, q, kp, vp, cos, sin, style, b.tok_pos, tok_page, H, G, d,
                                       rows=c.rows, n_rows=c.n_rows)
                 kernels.attn_prefill(q, k_pages, v_pages, out, c, table, ring, H, G, d, self.window, self.scale)
-        elif kernels.attn_prefill_rope_takes(ctx.dtype, d):
+        elif kernels.attn_prefill_rope_takes(ctx.dtype, d, T):
             # keys and values go to the cache; the attention kernel rotates q on its way in
             if writes:
                 kernels.kv_store_tiles(qkv, kp, vp, cos, sin, style, b, table, ring, H, G, d)

@@ -526,6 +526,39 @@ def test_steps_that_append_several_tokens_to_what_a_slot_holds(which, dtype, fol
     s.release(slots)
 
 
+@pytest.mark.parametrize("native", [True, False])
+@pytest.mark.parametrize("which", ["D", "E"])
+def test_a_prefill_step_of_a_thousand_tokens_and_more(which, native, folders):
+    """From 1,024 tokens a step on, the matrix-core path writes no rotated copy of q: the attention
+    kernel rotates q itself and a tile-wise kernel writes keys and values.  Prompts that make
+    such a step together, one of them continued from what its slot holds; then decode steps, which
+    read what that kernel wrote.  In the library's step and in the one from Python."""
+    d = folders[which]
+    cfg = tiny.read_config(d)
+    rng = np.random.default_rng(77)
+    limit = cfg["max_position_embeddings"]
+    lens = [min(700, limit - 8), 420]
+    while sum(lens) - 37 < 1024:
+        lens.append(300)
+    n = len(lens)
+    seqs = [tiny.random_tokens(rng, m + 4, cfg["vocab_size"]) for m in lens]
+    truth = [tiny.plain_logits(d, q) for q in seqs]
+    s = session(d, "bfloat16", max_tokens=2048, native=native)
+    slots = s.begin(n)
+    s.step([slots[1]], [seqs[1][:37]])                       # the second prompt's first 37 tokens are held already
+    first = [0, 37] + [0] * (n - 2)
+    want = [[0, 5, m - f - 1] for m, f in zip(lens, first)]
+    got = s.step(slots, [q[f:m] for q, f, m in zip(seqs, first, lens)], want).double().cpu().numpy()
+    for i in range(n):
+        for k, j in enumerate(want[i]):
+            assert np.abs(got[3 * i + k] - truth[i][first[i] + j]).max() <= tolerance("bfloat16", truth[i]), (i, j)
+    for j in range(4):
+        got = s.step(slots, [[q[m + j]] for q, m in zip(seqs, lens)]).double().cpu().numpy()
+        for i in range(n):
+            assert np.abs(got[i] - truth[i][lens[i] + j]).max() <= tolerance("bfloat16", truth[i]), (i, "step", j)
+    s.release(slots)
+
+
 @pytest.mark.parametrize("stored", ["float32", "float16"])
 def test_folders_stored_in_other_types_than_bfloat16(stored, tmp_path):
     """A folder stored in 32-bit keeps its weights in 32-bit in both runtimes (the bfloat16 runtime
