@@ -16,12 +16,9 @@ typedef uint16_t bf16_t;
 __device__ __forceinline__ float bf16_bits_to_f32(bf16_t v) {
     return __uint_as_float(((uint32_t)v) << 16);
 }
-// Round to nearest, ties to even; NaN stays NaN.
+// Round to nearest, ties to even; NaN stays NaN.  (The conversion is one instruction on gfx950.)
 __device__ __forceinline__ bf16_t f32_to_bf16_bits(float f) {
-    uint32_t u = __float_as_uint(f);
-    if ((u & 0x7fffffffu) > 0x7f800000u) return (bf16_t)((u >> 16) | 0x40u);
-    u += 0x7fffu + ((u >> 16) & 1u);
-    return (bf16_t)(u >> 16);
+    return __builtin_bit_cast(bf16_t, (__bf16)f);
 }
 
 template <typename T> __device__ __forceinline__ float to_f32(T v);

@@ -16,6 +16,9 @@
 // The loads are inline assembly so that the wait for "all but the newest steps" (s_waitcnt
 // vmcnt(n)) stays as written: the compiler, when it knows of such loads, waits for all of them
 // before any LDS read.  M0 carries the LDS address of a wave's 1 KB; nothing else here uses M0.
+#ifndef SPREAD_FROM
+#define SPREAD_FROM 4
+#endif
 template <int BK>
 __device__ __forceinline__ int swizzled_chunk(int row, int chunk) {
     return BK == 32 ? chunk ^ ((row >> 2) & 3) : chunk ^ ((row >> 1) & 7);
@@ -38,6 +41,15 @@ __device__ __forceinline__ void wait_for_loads() {      // vmcnt(N), other count
     static_assert(N_OUTSTANDING < 64, "vmcnt has six bits");
     __builtin_amdgcn_s_waitcnt((N_OUTSTANDING & 15) | (7 << 4) | (15 << 8) | ((N_OUTSTANDING >> 4) << 14));
 }
+
+// The value that the lane named by a permutation of each four lanes holds (DPP quad_perm:
+// 0xB1 the lane beside, 0x4E the lane two further on).
+template <int QUAD_PERM>
+__device__ __forceinline__ float swap_lanes(float v) {
+    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), QUAD_PERM, 0xf, 0xf, true));
+}
+__device__ __forceinline__ void store_pair(float* p, float a, float b) { *(float2*)p = make_float2(a, b); }
+__device__ __forceinline__ void store_pair(bf16_t* p, bf16_t a, bf16_t b) { *(unsigned*)p = (unsigned)a | ((unsigned)b << 16); }
 
 template <int TN, int TM, int WN, int WM, int BK, int NS, int EPI, typename TC>
 __global__ __launch_bounds__(64 * WN * WM) void gemm_direct_kernel(const bf16_t* __restrict__ A,
@@ -131,6 +143,7 @@ __global__ __launch_bounds__(64 * WN * WM) void gemm_direct_kernel(const bf16_t*
     // Fragments of k-slice g+1 are read from LDS while the MFMAs of slice g run; the wait, the
     // barrier and the next loads of a step sit in the middle of the last slice of the step before.
     constexpr int KS = BK / 16;
+    constexpr bool SPREAD = TN * TM >= SPREAD_FROM;      // the prefill's tiles
     static_assert(KS % 2 == 0, "fragment sets alternate by slice");
     bf16x8 wf[2][TN], af[2][TM];
     auto read_frags = [&](int stage, int ks, bf16x8 (&w)[TN], bf16x8 (&a)[TM]) {
@@ -180,6 +193,35 @@ __global__ __launch_bounds__(64 * WN * WM) void gemm_direct_kernel(const bf16_t*
                     __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
                 }
                 __builtin_amdgcn_sched_barrier(0);
+            } else if (SPREAD) {
+                // The last slice begins with the wait and the barrier; the next loads follow one
+                // by one between its MFMAs, each pinned where it is written: a burst of loads
+                // holds up the MFMAs behind it while the memory pipeline takes them in.
+                __builtin_amdgcn_sched_barrier(0);
+                wait_for_loads<(W_LOADS + A_LOADS) * (NS - 2)>();
+                __syncthreads();
+                __builtin_amdgcn_sched_barrier(0);
+                const unsigned to = lds_wave + stage * (STAGE * 2);
+                int step = min(it + NS, n_steps - 1) + first_step;
+                if (step >= n_steps) step -= n_steps;
+                const void* wsrc = same_in_every_lane(w_tile + step * BK);
+                const void* asrc = same_in_every_lane(a_tile + step * BK);
+                read_frags(next_stage, 0, wf[0], af[0]);       // past the last step: a stage of repeats
+                __builtin_amdgcn_sched_barrier(0);
+                constexpr int NL = W_LOADS + A_LOADS, NM = TN * TM, PER = (NL + NM - 1) / NM;
+#pragma unroll
+                for (int m = 0; m < NM; ++m) {
+                    const int i = m / TM, j = m % TM;
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[ks & 1][j], wf[ks & 1][i], acc[i][j], 0, 0, 0);
+                    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                    for (int q = 0; q < PER; ++q) {
+                        const int l = m * PER + q;
+                        if (l < W_LOADS) load_16_bytes_to_lds(w_off[l], wsrc, to + l * (NW * RG * BK * 2));
+                        else if (l < NL) load_16_bytes_to_lds(a_off[l - W_LOADS], asrc, to + (BN * BK * 2) + (l - W_LOADS) * (NW * RG * BK * 2));
+                    }
+                    __builtin_amdgcn_sched_barrier(0);
+                }
             } else {
                 multiply(wf[ks & 1], af[ks & 1], 0, TN / 2);
                 __builtin_amdgcn_sched_barrier(0);
@@ -216,6 +258,54 @@ __global__ __launch_bounds__(64 * WN * WM) void gemm_direct_kernel(const bf16_t*
         float next_w[TN];
 #pragma unroll
         for (int i = 0; i < TN; ++i) next_w[i] = prepares && (full || n0 + c0 + 32 * i < N) ? link.next_w[n0 + c0 + 32 * i] : 0.f;
+        if constexpr (EPI == 2) {
+            // Two lanes side by side hold a gate column and its up column, 16 rows each.  They
+            // swap half (DPP, no LDS): then the even lane has gate and up of its first eight rows
+            // and the odd lane of its last eight, so that each value of the output is computed
+            // once.  A second swap with the lane two further on, which holds the next output
+            // column, leaves every lane two adjacent columns of four rows: four bytes a store.
+            const int odd = l32 & 1, upper = (l32 >> 1) & 1;
+            const int r0 = wm + 4 * kq + 16 * odd + 8 * upper;         // first of this lane's four rows in a block of 32
+            const int oc = (wn >> 1) + ((l32 >> 2) << 1);              // lower of its two output columns, less 16 i
+            TC* corner = C + (int64_t)m0 * ldc + n0 / 2;
+            const unsigned ld = (unsigned)ldc;
+            const bool paired = (ldc & 1) == 0 && ((uintptr_t)C & (2 * sizeof(TC) - 1)) == 0;     // (n0 / 2 is even)
+#pragma unroll
+            for (int j = 0; j < TM; ++j)
+#pragma unroll
+                for (int i = 0; i < TN; ++i) {
+                    float o[8];
+#pragma unroll
+                    for (int k = 0; k < 8; ++k) {
+                        const float lo = acc[i][j][k], hi = acc[i][j][k + 8];
+                        const float recv = swap_lanes<0xB1>(odd ? lo : hi);      // with the lane beside
+                        float g = odd ? recv : lo, u = odd ? hi : recv;
+                        if (link.ssq) {
+                            const int r = wm + 4 * kq + 32 * j + 16 * odd + 8 * (k / 4) + k % 4;
+                            const float sc = (full || m0 + r < M) ? link_scale[r] : 0.f;
+                            g *= sc;
+                            u *= sc;
+                        }
+                        o[k] = silu_mul(g, u);
+                    }
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) {
+                        const float recv = swap_lanes<0x4E>(upper ? o[q] : o[q + 4]);   // with the lane two further
+                        const float c_lo = upper ? recv : o[q], c_hi = upper ? o[q + 4] : recv;
+                        const int r = r0 + 32 * j + q, c = oc + 16 * i;
+                        if (!full && m0 + r >= M) continue;
+                        TC* p = corner + (unsigned)r * ld + c;
+                        const bool in_lo = full || n0 / 2 + c < N / 2, in_hi = full || n0 / 2 + c + 1 < N / 2;
+                        if (paired && in_hi) {
+                            store_pair(p, from_f32<TC>(c_lo), from_f32<TC>(c_hi));
+                        } else {
+                            if (in_lo) p[0] = from_f32<TC>(c_lo);
+                            if (in_hi) p[1] = from_f32<TC>(c_hi);
+                        }
+                    }
+                }
+            return;
+        }
 #pragma unroll
         for (int j = 0; j < TM; ++j) {
             // what this product adds to: 32 rows' values are all asked for before the first is used

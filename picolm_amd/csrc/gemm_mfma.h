@@ -17,7 +17,12 @@ __device__ __forceinline__ bf16x8 zero_chunk() {
     for (int i = 0; i < 8; ++i) z[i] = (__bf16)0.0f;
     return z;
 }
-__device__ __forceinline__ float silu_mul(float g, float u) { return g / (1.0f + expf(-g)) * u; }
+// silu(g) * u with the hardware's 2^x and 1/x (an ulp each: far below the bfloat16 rounding of
+// the products these kernels serve; the 32-bit path has its own formula in gemm_generic.hip).
+// 2^x of a large x is inf and its reciprocal 0, so a very negative gate gives -0, as it should.
+__device__ __forceinline__ float silu_mul(float g, float u) {
+    return g * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(g * -1.4426950408889634f)) * u;
+}
 
 // =============================================================================================
 // a norm split between two products
