@@ -16,6 +16,7 @@
 //            (columns = the query heads of one KV group); the 4 waves of a workgroup take
 //            pages in turn and merge through LDS; split-K partials go to a buffer that the
 //            merge kernel of the generic path combines.
+#include <utility>
 #include "common.h"
 #include "api.h"
 #include "attention.h"
@@ -46,67 +47,150 @@ __device__ __forceinline__ __bf16 to_bf16(float f) { return (__bf16)f; }      //
 // of float probabilities whose largest is near 1, and zero is as good.
 __device__ __forceinline__ float exp2_flushing(float x) { return __builtin_amdgcn_exp2f(x); }
 
-// One page of one wave: scores, online softmax, and the update of O^T.  KOP(t, s) returns the
-// K operand of tile t, k-step s; VOP(dt, t, ks) the V^T operand of column block dt.
+
+// A value's maximum or sum over a lane and the lane 32 further on (or back): one swap of the
+// wave's halves (both results of it hold the lower half's value and the upper half's), no LDS.
+__device__ __forceinline__ float max_of_halves(float v) {
+    const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+}
+__device__ __forceinline__ float sum_of_halves(float v) {
+    const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+}
+
+// The softmax of one S^T tile (32 keys) of a wave in pieces, so that the pieces can be written
+// between the matrix products of another tile: mask and maximum of some elements; then the
+// reference point of the exponentials; then the probabilities of some elements, as operands of
+// the second product; then the sum.
+struct TileSoftmax {
+    float mx, m_new, alpha, sum;
+    bool rescale;
+};
+template <bool MASKED>
+__device__ __forceinline__ void softmax_mask_max(f32x16& S, int e0, int n, int key0, int qpos, bool q_ok, int window, int h, TileSoftmax& t) {
+#pragma unroll
+    for (int e = e0; e < e0 + n; ++e) {
+        if (MASKED) {
+            const int key = key0 + key_of_elem(e, h);
+            const bool vis = q_ok && key <= qpos && (window <= 0 || qpos - key < window);
+            S[e] = vis ? S[e] : NEG_BIG;
+        }                               // else every key of the page is visible to every query of the wave
+        t.mx = fmaxf(t.mx, S[e]);
+    }
+}
+// m_run is the reference point of the exponentials, not necessarily the maximum: it follows the
+// maximum only when that has grown by more than LAZY_MAX_STEP (in powers of two), so that most
+// tiles leave it alone and O^T need not be rescaled.  The result is the same in exact arithmetic;
+// probabilities may reach 2^LAZY_MAX_STEP instead of 1 meanwhile.  The scores stay unscaled (the
+// scale is positive, so their order is that of the scaled ones): the scale goes into the
+// exponent's multiply-add.
+__device__ __forceinline__ void softmax_reference(TileSoftmax& t, float m_run, float scale2) {
+    const float mx = max_of_halves(t.mx) * scale2;
+    const bool grow = mx > m_run + LAZY_MAX_STEP;
+    t.m_new = grow ? mx : m_run;
+    t.alpha = grow ? exp2_flushing(m_run - t.m_new) : 1.0f;
+    t.rescale = __any(grow);
+    t.sum = 0.f;
+}
+template <bool MASKED>
+__device__ __forceinline__ void softmax_exp(const f32x16& S, int e0, int n, float scale2, TileSoftmax& t, bf16x8 (&Pf)[2]) {
+#pragma unroll
+    for (int e = e0; e < e0 + n; ++e) {
+        const float p = (!MASKED || S[e] > 0.5f * NEG_BIG) ? exp2_flushing(fmaf(S[e], scale2, -t.m_new)) : 0.f;
+        t.sum += p;
+        Pf[e / 8][e % 8] = to_bf16(p);
+    }
+}
+__device__ __forceinline__ void softmax_finish(TileSoftmax& t, float& m_run, float& l_run) {
+    l_run = l_run * t.alpha + sum_of_halves(t.sum);
+    m_run = t.m_new;
+}
+
+// v *= alpha, every element in the register it is in.  (Written as plain C++ the compiler gives
+// the product registers of its own and copies all of O^T, on the path that does not rescale too.)
+__device__ __forceinline__ void scale_in_place(f32x16& v, float alpha) {
+#pragma unroll
+    for (int e = 0; e < 16; ++e) {
+        float x = v[e];
+        asm volatile("v_mul_f32 %0, %1, %0" : "+v"(x) : "v"(alpha));
+        v[e] = x;
+    }
+}
+
+// One page of one wave: scores, online softmax, and the update of O^T, a tile of 32 keys at a
+// time, with one tile's softmax (vector ALU) written between the other tile's products (matrix
+// cores) and held there, so that a wave keeps both busy: S1 = K1 Q^T beside softmax(S0), then
+// O^T += V0^T P0^T beside softmax(S1).  KOP(t, s) returns the K operand of tile t, k-step s;
+// VOP(dt, t, ks) the V^T operand of column block dt.
 template <int D, bool MASKED, typename KOP, typename VOP>
 __device__ __forceinline__ void attend_page(const bf16x8 (&Qf)[D / 16], f32x16 (&O)[D / 32], float& m_run,
                                             float& l_run, int key0, int qpos, bool q_ok, int window,
                                             float scale2, int h, KOP kop, VOP vop) {
-    f32x16 S[2];
+    constexpr int NP = D / 16;                  // products of a tile, in either role
+    static_assert(NP % 2 == 0 && 16 % (NP / 2) == 0, "the softmax's pieces go between the products");
+    constexpr int PIECE = 16 / (NP / 2);        // elements per piece: half of the products see the maximum, half the exponentials
+    f32x16 S0, S1;
 #pragma unroll
-    for (int t = 0; t < 2; ++t) {
+    for (int e = 0; e < 16; ++e) S0[e] = 0.f, S1[e] = 0.f;
+    // (every operand is asked for two products early and held there: the compiler, left alone,
+    // asks for all of a tile's operands at once and runs out of registers)
+    bf16x8 ahead = kop(0, 0), ahead2 = kop(0, 1);
 #pragma unroll
-        for (int e = 0; e < 16; ++e) S[t][e] = 0.f;
-#pragma unroll
-        for (int s = 0; s < D / 16; ++s) S[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kop(t, s), Qf[s], S[t], 0, 0, 0);
+    for (int s = 0; s < NP; ++s) {
+        const bf16x8 now = ahead;
+        ahead = ahead2;
+        ahead2 = s + 2 < NP ? kop(0, s + 2) : kop(1, s + 2 - NP);
+        S0 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(now, Qf[s], S0, 0, 0, 0);
+        __builtin_amdgcn_sched_barrier(0);
     }
-    float mx = NEG_BIG;
+    TileSoftmax t;
+    bf16x8 P0[2], P1[2];
+    t.mx = NEG_BIG;
+    __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-    for (int t = 0; t < 2; ++t)
+    for (int s = 0; s < NP; ++s) {
+        const bf16x8 now = ahead;
+        ahead = ahead2;
+        ahead2 = s + 2 < NP ? kop(1, s + 2) : vop((s + 2 - NP) / 2, 0, (s + 2 - NP) % 2);
+        S1 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(now, Qf[s], S1, 0, 0, 0);
+        __builtin_amdgcn_sched_barrier(0);
+        if (s < NP / 2) softmax_mask_max<MASKED>(S0, PIECE * s, PIECE, key0, qpos, q_ok, window, h, t);
+        if (s == NP / 2 - 1) softmax_reference(t, m_run, scale2);
+        if (s >= NP / 2) softmax_exp<MASKED>(S0, PIECE * (s - NP / 2), PIECE, scale2, t, P0);
+        __builtin_amdgcn_sched_barrier(0);
+    }
+    softmax_finish(t, m_run, l_run);
+    if (t.rescale) {
 #pragma unroll
-        for (int e = 0; e < 16; ++e) {
-            if (MASKED) {
-                const int key = key0 + 32 * t + key_of_elem(e, h);
-                const bool vis = q_ok && key <= qpos && (window <= 0 || qpos - key < window);
-                S[t][e] = vis ? S[t][e] : NEG_BIG;
-            }                               // else every key of the page is visible to every query of the wave
-            mx = fmaxf(mx, S[t][e]);
-        }
-    // the scores stay unscaled (the scale is positive, so their order is that of the scaled ones):
-    // the scale goes into the exponent's multiply-add below
-    mx = fmaxf(mx, __shfl_xor(mx, 32, WAVE)) * scale2;
-    // m_run is the reference point of the exponentials, not necessarily the maximum: it follows
-    // the maximum only when that has grown by more than LAZY_MAX_STEP (in powers of two), so that
-    // most pages leave it alone and O^T need not be rescaled.  The result is the same in exact
-    // arithmetic; probabilities may reach 2^LAZY_MAX_STEP instead of 1 meanwhile.
-    const bool grow = mx > m_run + LAZY_MAX_STEP;
-    const float m_new = grow ? mx : m_run;
-    const float alpha = grow ? exp2_flushing(m_run - m_new) : 1.0f;
-    const bool rescale = __any(grow);
-    float sum = 0.f;
-    bf16x8 Pf[2][2];
+        for (int dt = 0; dt < D / 32; ++dt) scale_in_place(O[dt], t.alpha);
+    }
+    t.mx = NEG_BIG;
+    __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-    for (int t = 0; t < 2; ++t)
+    for (int s = 0; s < NP; ++s) {
+        const bf16x8 now = ahead;
+        ahead = ahead2;
+        ahead2 = s + 2 < NP ? vop((s + 2) / 2, 0, (s + 2) % 2) : vop((s + 2 - NP) / 2, 1, (s + 2 - NP) % 2);
+        O[s / 2] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(now, P0[s % 2], O[s / 2], 0, 0, 0);
+        __builtin_amdgcn_sched_barrier(0);
+        if (s < NP / 2) softmax_mask_max<MASKED>(S1, PIECE * s, PIECE, key0 + 32, qpos, q_ok, window, h, t);
+        if (s == NP / 2 - 1) softmax_reference(t, m_run, scale2);
+        if (s >= NP / 2) softmax_exp<MASKED>(S1, PIECE * (s - NP / 2), PIECE, scale2, t, P1);
+        __builtin_amdgcn_sched_barrier(0);
+    }
+    softmax_finish(t, m_run, l_run);
+    if (t.rescale) {
 #pragma unroll
-        for (int e = 0; e < 16; ++e) {
-            const float p = (!MASKED || S[t][e] > 0.5f * NEG_BIG) ? exp2_flushing(fmaf(S[t][e], scale2, -m_new)) : 0.f;
-            sum += p;
-            Pf[t][e / 8][e % 8] = to_bf16(p);
-        }
-    sum += __shfl_xor(sum, 32, WAVE);
-    l_run = l_run * alpha + sum;
-    m_run = m_new;
+        for (int dt = 0; dt < D / 32; ++dt) scale_in_place(O[dt], t.alpha);
+    }
 #pragma unroll
-    for (int dt = 0; dt < D / 32; ++dt) {
-        if (rescale) {
-#pragma unroll
-            for (int e = 0; e < 16; ++e) O[dt][e] *= alpha;
-        }
-#pragma unroll
-        for (int t = 0; t < 2; ++t)
-#pragma unroll
-            for (int ks = 0; ks < 2; ++ks)
-                O[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vop(dt, t, ks), Pf[t][ks], O[dt], 0, 0, 0);
+    for (int s = 0; s < NP; ++s) {
+        const bf16x8 now = ahead;
+        ahead = ahead2;
+        if (s + 2 < NP) ahead2 = vop((s + 2) / 2, 1, (s + 2) % 2);
+        O[s / 2] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(now, P1[s % 2], O[s / 2], 0, 0, 0);
+        __builtin_amdgcn_sched_barrier(0);
     }
 }
 
@@ -217,14 +301,12 @@ __device__ __forceinline__ void rotated_q(const AttnArgs& a, const float* row, i
 template <int D, int HALVES>
 __global__ __launch_bounds__(256 * HALVES) __attribute__((amdgpu_waves_per_eu(2))) void attn_prefill_mfma_kernel(AttnArgs a, int HB, int tile_tokens,
                                                                                                                  int n_tiles, int n_cus) {
-    constexpr int KCH = D / 8;                        // 16-byte chunks of a K row
-    constexpr int KP = PAGE_TOKENS * KCH / 256;       // K chunks a thread stages per page
-    constexpr int VP = D * 8 / 256;                   // V^T chunks a thread stages per page
+    constexpr int LOADS = D / 32;                     // KB of a page's K (and of its V^T) that a wave brings in
     constexpr int STAGE = 2 * PAGE_TOKENS * D;        // K tile + V^T tile, in bf16
-    extern __shared__ __attribute__((aligned(16))) bf16_t lds_all[];      // two stages for each half
-    const int half = threadIdx.x / 256;
+    extern __shared__ __attribute__((aligned(1024))) bf16_t lds_all[];    // two stages for each half
+    const int half = __builtin_amdgcn_readfirstlane(threadIdx.x / 256);
     bf16_t* lds = lds_all + half * (2 * STAGE);
-    const int tid = threadIdx.x % 256, wave = tid / WAVE, lane = tid % WAVE;      // (within the half)
+    const int tid = threadIdx.x % 256, wave = __builtin_amdgcn_readfirstlane(tid / WAVE), lane = tid % WAVE;      // (within the half)
     const int l32 = lane % 32, h = lane / 32;
     const int R = a.H / a.G;
     const int head_chunks = (R + HB - 1) / HB;
@@ -273,57 +355,76 @@ __global__ __launch_bounds__(256 * HALVES) __attribute__((amdgpu_waves_per_eu(2)
     const int32_t* pt = a.page_table + (size_t)a.seq_slot[seq] * a.max_pages;
     const size_t page_elems = (size_t)a.G * PAGE_TOKENS * D;
 
-    bf16x8 kreg[KP], vreg[VP];
-    // (where a page lies is asked a round ahead of its loads, which would otherwise wait for it)
-    auto place_of = [&](int page) { return pt[page % a.ring_pages]; };
-    auto fetch = [&](int place) {
+    // A page's K and V^T go from the cache straight into LDS: as they lie in the cache they are in
+    // the order of the MFMA operands, so a wave copies whole kilobytes (wave w of a half the KB
+    // w, w + 4, ..).  Where a page lies is asked a round ahead of its loads, which would otherwise
+    // wait for it.
+    auto place_of = [&](int page) { return __builtin_amdgcn_readfirstlane(pt[page % a.ring_pages]); };
+    const unsigned lds_wave = __builtin_amdgcn_readfirstlane(
+        (unsigned)(size_t)(__attribute__((address_space(3))) bf16_t*)lds + wave * 1024);
+    const unsigned lane_bytes = lane * 16;
+    auto fetch = [&](int stage, int place) {
         const size_t base = (size_t)place * page_elems + (size_t)g * PAGE_TOKENS * D;
-        const bf16_t* kp = (const bf16_t*)a.k_pages + base;
-        const bf16_t* vp = (const bf16_t*)a.v_pages + base;
+        const char* kp = (const char*)((const bf16_t*)a.k_pages + base) + wave * 1024;
+        const char* vp = (const char*)((const bf16_t*)a.v_pages + base) + wave * 1024;
+        const unsigned to = lds_wave + stage * (STAGE * 2);
 #pragma unroll
-        for (int i = 0; i < KP; ++i) kreg[i] = ldg8(kp + (size_t)(tid + 256 * i) * 8);
+        for (int i = 0; i < LOADS; ++i) load_16_bytes_to_lds(lane_bytes, same_in_every_lane(kp + i * 4096), to + i * 4096);
 #pragma unroll
-        for (int i = 0; i < VP; ++i) vreg[i] = ldg8(vp + (size_t)(tid + 256 * i) * 8);
+        for (int i = 0; i < LOADS; ++i)
+            load_16_bytes_to_lds(lane_bytes, same_in_every_lane(vp + i * 4096), to + PAGE_TOKENS * D * 2 + i * 4096);
     };
-    auto stash = [&](int stage, int page) {
-        bf16_t* Ks = lds + stage * STAGE;
-        bf16_t* Vs = Ks + PAGE_TOKENS * D;
-        // keys past the sequence's end may hold anything: their values are zeroed, without a branch
+    // What a wave has brought in is in LDS; before the others may read it, the values of keys past
+    // the sequence's end, which may hold anything, are zeroed (their probabilities are zero, but
+    // zero times anything is not).  Only a tile's last page has such keys.
+    auto landed = [&](int stage, int page) {
+        wait_for_loads<0>();
         const int n_keys = b_qlast - page * PAGE_TOKENS + 1;
+        if (n_keys < PAGE_TOKENS) {
+            bf16_t* Vs = lds + stage * STAGE + PAGE_TOKENS * D;
 #pragma unroll
-        for (int i = 0; i < KP; ++i) *(bf16x8*)(Ks + (size_t)(tid + 256 * i) * 8) = kreg[i];
+            for (int i = 0; i < LOADS; ++i) {
+                const int idx = tid + 256 * i;
+                // chunk idx of V^T holds keys 32*tile + 16*step + 8*half .. + 8 (see v_page_offset)
+                const int key0 = 32 * (idx / (128 * (D / 32))) + 16 * ((idx / 64) % 2) + 8 * ((idx % 64) / 32);
+                bf16x8 v = *(const bf16x8*)(Vs + (size_t)idx * 8);
 #pragma unroll
-        for (int i = 0; i < VP; ++i) {
-            const int idx = tid + 256 * i;
-            // chunk idx of V^T holds keys 32*tile + 16*step + 8*half .. + 8 (see v_page_offset)
-            const int key0 = 32 * (idx / (128 * (D / 32))) + 16 * ((idx / 64) % 2) + 8 * ((idx % 64) / 32);
-            bf16x8 v = vreg[i];
-#pragma unroll
-            for (int e = 0; e < 8; ++e) v[e] = (key0 + e < n_keys) ? v[e] : (__bf16)0.0f;
-            *(bf16x8*)(Vs + (size_t)idx * 8) = v;
+                for (int e = 0; e < 8; ++e) v[e] = (key0 + e < n_keys) ? v[e] : (__bf16)0.0f;
+                *(bf16x8*)(Vs + (size_t)idx * 8) = v;
+            }
         }
+        __syncthreads();
+    };
+    auto operands = [&](int stage) {
+        const bf16_t* Ks = lds + stage * STAGE;
+        const bf16_t* Vs = Ks + PAGE_TOKENS * D;
+        return std::make_pair(
+            [=](int t, int s) { return *(const bf16x8*)(Ks + ((t * (D / 16) + s) * 64 + lane) * 8); },
+            [=](int dt, int t, int ks) { return *(const bf16x8*)(Vs + (((t * (D / 32) + dt) * 2 + ks) * 64 + lane) * 8); });
+    };
+    // a page wholly before the tile's first query: every wave attends to all of it (rows
+    // without a query are never stored, whatever they hold)
+    auto compute_plain = [&](int stage, int page) {
+        const auto op = operands(stage);
+        attend_page<D, false>(Qf, O, m_run, l_run, page * PAGE_TOKENS, qpos, q_ok, a.window, scale2, h, op.first, op.second);
     };
     auto compute = [&](int stage, int page) {
         if (page < w_page_lo || page >= w_page_hi) return;
-        const bf16_t* Ks = lds + stage * STAGE;
-        const bf16_t* Vs = Ks + PAGE_TOKENS * D;
-        auto kop = [&](int t, int s) { return *(const bf16x8*)(Ks + ((t * (D / 16) + s) * 64 + lane) * 8); };
-        auto vop = [&](int dt, int t, int ks) { return *(const bf16x8*)(Vs + (((t * (D / 32) + dt) * 2 + ks) * 64 + lane) * 8); };
-        // a page wholly before the wave's first query needs no mask (rows without a query are
-        // never stored, whatever they hold)
+        const auto op = operands(stage);
+        // a page wholly before the wave's first query needs no mask
         if (a.window <= 0 && page * PAGE_TOKENS + PAGE_TOKENS - 1 <= w_qfirst)
-            attend_page<D, false>(Qf, O, m_run, l_run, page * PAGE_TOKENS, qpos, q_ok, a.window, scale2, h, kop, vop);
+            attend_page<D, false>(Qf, O, m_run, l_run, page * PAGE_TOKENS, qpos, q_ok, a.window, scale2, h, op.first, op.second);
         else
-            attend_page<D, true>(Qf, O, m_run, l_run, page * PAGE_TOKENS, qpos, q_ok, a.window, scale2, h, kop, vop);
+            attend_page<D, true>(Qf, O, m_run, l_run, page * PAGE_TOKENS, qpos, q_ok, a.window, scale2, h, op.first, op.second);
     };
 
     // a half's pages: page_lo + half, then every HALVES-th; both halves go round the loop alike
     const int n_rounds = (page_hi - page_lo + HALVES - 1) / HALVES;
     auto page_of = [&](int round) { return page_lo + HALVES * round + half; };
-    // (A half whose turn has no page left stages the tile's last page again and attends to
-    // nothing: loads and stores without conditions around them keep the waits for them apart from
-    // the matrix products.)
-    fetch(place_of(min(page_of(0), page_hi - 1)));
+    // (A half whose turn has no page left brings in the tile's last page again and attends to
+    // nothing: loads without conditions around them keep the waits for them apart from the matrix
+    // products.)
+    fetch(0, place_of(min(page_of(0), page_hi - 1)));
     int next_place = place_of(min(page_of(1), page_hi - 1));
     // the queries, while the first page is on its way
     if (a.qkv) {        // the float rows of the qkv product: rotated here, no rotated copy of q in memory
@@ -333,18 +434,30 @@ __global__ __launch_bounds__(256 * HALVES) __attribute__((amdgpu_waves_per_eu(2)
 #pragma unroll
         for (int s = 0; s < D / 16; ++s) Qf[s] = q_ok ? ldg8(qp + 16 * s) : zero8();
     }
-    stash(0, min(page_of(0), page_hi - 1));
-    __syncthreads();
-    int cur = 0;
-    for (int round = 0; round + 1 < n_rounds; ++round) {
+    landed(0, min(page_of(0), page_hi - 1));
+    int cur = 0, round = 0;
+    // The rounds whose pages lie wholly before the tile's first query, most of a long prompt's,
+    // have a loop of their own with one path through it: in the general loop below, where a wave
+    // may skip a page or mask it, the compiler moves all of O^T between registers twice a page.
+    const int plain_rounds = a.window > 0 ? 0 : min(n_rounds - 1, max(0, (b_qfirst / PAGE_TOKENS - page_lo) / HALVES));
+    for (; round < plain_rounds; ++round) {
         const int next = min(page_of(round + 1), page_hi - 1);
-        fetch(next_place);                        // in flight while this page is attended to
+        fetch(cur ^ 1, next_place);               // in flight while this page is attended to
+        next_place = place_of(min(page_of(round + 2), page_hi - 1));
+        __builtin_amdgcn_sched_barrier(0);
+        compute_plain(cur, page_of(round));
+        __builtin_amdgcn_sched_barrier(0);
+        landed(cur ^ 1, next);
+        cur ^= 1;
+    }
+    for (; round + 1 < n_rounds; ++round) {
+        const int next = min(page_of(round + 1), page_hi - 1);
+        fetch(cur ^ 1, next_place);
         next_place = place_of(min(page_of(round + 2), page_hi - 1));
         __builtin_amdgcn_sched_barrier(0);
         compute(cur, page_of(round));
         __builtin_amdgcn_sched_barrier(0);
-        stash(cur ^ 1, next);
-        __syncthreads();
+        landed(cur ^ 1, next);
         cur ^= 1;
     }
     compute(cur, page_of(n_rounds - 1));          // (past the tile's pages: nothing)

@@ -29,6 +29,31 @@ template <typename T> __device__ __forceinline__ T from_f32(float v);
 template <> __device__ __forceinline__ float from_f32<float>(float v) { return v; }
 template <> __device__ __forceinline__ bf16_t from_f32<bf16_t>(float v) { return f32_to_bf16_bits(v); }
 
+// ---- loads from global memory straight into LDS ------------------------------------------
+// global_load_lds_dwordx4: the 64 lanes of a wave bring 16 bytes each to 1 KB of LDS in a row, with
+// no staging registers and no LDS store instructions.  Inline assembly, so that a wait for "all
+// but the newest loads" (s_waitcnt vmcnt(n)) stays as written: the compiler, when it knows of such
+// loads, waits for all of them before any LDS read.  M0 carries the LDS address of the wave's 1 KB.
+// A pointer that is the same in every lane, said so that it lies in scalar registers whatever
+// the compiler made of the arithmetic that led to it.
+__device__ __forceinline__ const void* same_in_every_lane(const void* p) {
+    const uint64_t v = (uint64_t)p;
+    const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v), hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
+    return (const void*)(((uint64_t)hi << 32) | lo);
+}
+__device__ __forceinline__ void load_16_bytes_to_lds(unsigned byte_offset, const void* base, unsigned lds_address) {
+    asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dwordx4 %0, %1"
+                 :
+                 : "v"(byte_offset), "s"(base), "s"(lds_address)
+                 : "memory");
+}
+template <int N_OUTSTANDING>
+__device__ __forceinline__ void wait_for_loads() {      // vmcnt(N), other counters untouched
+    static_assert(N_OUTSTANDING < 64, "vmcnt has six bits");
+    __builtin_amdgcn_s_waitcnt((N_OUTSTANDING & 15) | (7 << 4) | (15 << 8) | ((N_OUTSTANDING >> 4) << 14));
+}
+
+
 // ---- reductions ---------------------------------------------------------------------
 __device__ __forceinline__ float wave_sum(float v) {
 #pragma unroll

@@ -23,25 +23,6 @@ template <int BK>
 __device__ __forceinline__ int swizzled_chunk(int row, int chunk) {
     return BK == 32 ? chunk ^ ((row >> 2) & 3) : chunk ^ ((row >> 1) & 7);
 }
-// A pointer that is the same in every lane, said so that it lies in scalar registers whatever
-// the compiler made of the arithmetic that led to it.
-__device__ __forceinline__ const void* same_in_every_lane(const void* p) {
-    const uint64_t v = (uint64_t)p;
-    const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v), hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
-    return (const void*)(((uint64_t)hi << 32) | lo);
-}
-__device__ __forceinline__ void load_16_bytes_to_lds(unsigned byte_offset, const void* base, unsigned lds_address) {
-    asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dwordx4 %0, %1"
-                 :
-                 : "v"(byte_offset), "s"(base), "s"(lds_address)
-                 : "memory");
-}
-template <int N_OUTSTANDING>
-__device__ __forceinline__ void wait_for_loads() {      // vmcnt(N), other counters untouched
-    static_assert(N_OUTSTANDING < 64, "vmcnt has six bits");
-    __builtin_amdgcn_s_waitcnt((N_OUTSTANDING & 15) | (7 << 4) | (15 << 8) | ((N_OUTSTANDING >> 4) << 14));
-}
-
 // The value that the lane named by a permutation of each four lanes holds (DPP quad_perm:
 // 0xB1 the lane beside, 0x4E the lane two further on).
 template <int QUAD_PERM>
