@@ -225,17 +225,21 @@ def main() -> int:
                    for b, u in ((2048, False), (1024, False), (512, True)))
         mfma = max(kernels.mfma_probe(fsink, b, 2000) / timed(lambda b=b: kernels.mfma_probe(fsink, b, 2000)) / 1e12
                    for b in (512, 1024, 2048))
+        # the same loop on operands like real data: the power limit then sets the clock
+        mfma_real = max(kernels.mfma_probe(fsink, b, 16000, True) / timed(lambda b=b: kernels.mfma_probe(fsink, b, 16000, True)) / 1e12
+                        for b in (512, 1024, 2048))
         del src
         torch.cuda.empty_cache()
-        return read, mfma
+        return read, mfma, mfma_real
 
     def kernel_classes(n_seq: int):
         """Each class of kernels against the nominal peak and against the measured ceiling, from
         events around every operation of launched (not replayed) steps."""
-        read_gbs, mfma_tflops = ceilings()
+        read_gbs, mfma_tflops, mfma_real_tflops = ceilings()
         n = 12
         _, _, ctx, ops = decode_run(n_seq, n, 3, time_ops=True)
-        out = {"read_ceiling_gbs": round(read_gbs, 1), "mfma_ceiling_tflops": round(mfma_tflops, 1), "decode_batch": n_seq}
+        out = {"read_ceiling_gbs": round(read_gbs, 1), "mfma_ceiling_tflops": round(mfma_tflops, 1),
+               "mfma_ceiling_random_operands_tflops": round(mfma_real_tflops, 1), "decode_batch": n_seq}
 
         def put(name, achieved, unit, ceiling, peak):
             out[f"{name}_{unit}"] = round(achieved, 1)
@@ -247,6 +251,7 @@ def main() -> int:
         pre = prefill_run(PREFILL_TOKENS, time_ops=True)
         put("prefill_products", product_flops(cfg, PREFILL_TOKENS) / (pre["products"] * 1e-3) / 1e12, "tflops", mfma_tflops, PEAK_TFLOPS["bf16"])
         put("prefill_attention", attention_flops(cfg, PREFILL_TOKENS) / (pre["attention"] * 1e-3) / 1e12, "tflops", mfma_tflops, PEAK_TFLOPS["bf16"])
+        out["prefill_products_of_ceiling_random_operands"] = round(out["prefill_products_tflops"] / mfma_real_tflops, 4)
         return out
 
     if args.prefill_only:

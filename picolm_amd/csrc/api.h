@@ -16,8 +16,10 @@ int picolm_device_check(void);     // 0 if the current device is a gfx950
 // reads `bytes` from `src` once; for bandwidth measurements
 int picolm_read_probe(const void* src, size_t bytes, void* sink, int blocks, int unroll4, hipStream_t stream);
 
-// runs blocks*4 waves of `iters` x 8 MFMAs (32x32x16 bf16) on registers; for MFMA-rate measurements
-int picolm_mfma_probe(void* sink, int blocks, int iters, hipStream_t stream);
+// runs blocks*4 waves of `iters` x 8 MFMAs (32x32x16 bf16) on registers, on small integers or
+// (random_operands != 0) on pseudo-random values of the size of real data, which the GPU's power
+// limit slows down; for MFMA-rate measurements
+int picolm_mfma_probe(void* sink, int blocks, int iters, int random_operands, hipStream_t stream);
 
 int picolm_embed(const void* table, int table_dt, const int32_t* tokens, float* x, int T, int D,
                  int V, hipStream_t stream);

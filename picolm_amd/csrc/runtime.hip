@@ -61,13 +61,30 @@ extern "C" int picolm_read_probe(const void* src, size_t bytes, void* sink, int 
 // registers (no memory traffic), for the measurement harness's "achievable" MFMA rate.
 typedef __attribute__((ext_vector_type(8))) __bf16 probe_bf16x8;
 typedef __attribute__((ext_vector_type(16))) float probe_f32x16;
+// RANDOM: the operands are pseudo-random values of about the size of activations and weights, a
+// different pair of registers for each of a wave's eight products (as in a tile product's wave:
+// four operands one way, two the other).  With such operands the multipliers and adders switch as
+// they do on real data, and the GPU's power limit, not the matrix cores' issue rate, sets the clock:
+// this is the rate a real product can hope for.  With small integers (RANDOM = false) the same
+// loop runs near the nominal peak.
+template <bool RANDOM>
 __global__ __launch_bounds__(256) void mfma_probe_kernel(float* __restrict__ sink, int iters) {
-    probe_bf16x8 a, b;
+    probe_bf16x8 a[4], b[2];
+    unsigned seed = threadIdx.x * 2654435761u + blockIdx.x * 40503u + 12345u;
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
-        a[i] = (__bf16)(float)(threadIdx.x % 7);
-        b[i] = (__bf16)(float)(threadIdx.x % 5);
-    }
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            seed = seed * 1664525u + 1013904223u;
+            a[j][i] = RANDOM ? (__bf16)(((int)(seed >> 8) % 8192 - 4096) * (1.0f / 2048.0f)) : (__bf16)(float)(threadIdx.x % 7);
+        }
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            seed = seed * 1664525u + 1013904223u;
+            b[j][i] = RANDOM ? (__bf16)(((int)(seed >> 8) % 8192 - 4096) * (0.02f / 2048.0f)) : (__bf16)(float)(threadIdx.x % 5);
+        }
     probe_f32x16 acc[8];
 #pragma unroll
     for (int t = 0; t < 8; ++t)
@@ -75,7 +92,7 @@ __global__ __launch_bounds__(256) void mfma_probe_kernel(float* __restrict__ sin
         for (int e = 0; e < 16; ++e) acc[t][e] = 0.f;
     for (int it = 0; it < iters; ++it) {
 #pragma unroll
-        for (int t = 0; t < 8; ++t) acc[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, acc[t], 0, 0, 0);
+        for (int t = 0; t < 8; ++t) acc[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[t % 4], b[t / 4], acc[t], 0, 0, 0);
     }
     float s = 0.f;
 #pragma unroll
@@ -84,9 +101,10 @@ __global__ __launch_bounds__(256) void mfma_probe_kernel(float* __restrict__ sin
 }
 
 // flops done: blocks * 4 waves * iters * 8 * 32768
-extern "C" int picolm_mfma_probe(void* sink, int blocks, int iters, hipStream_t stream) {
+extern "C" int picolm_mfma_probe(void* sink, int blocks, int iters, int random_operands, hipStream_t stream) {
     PICOLM_REQUIRE(blocks > 0 && iters > 0, "mfma_probe: bad sizes");
-    mfma_probe_kernel<<<dim3(blocks), dim3(256), 0, stream>>>((float*)sink, iters);
+    if (random_operands) mfma_probe_kernel<true><<<dim3(blocks), dim3(256), 0, stream>>>((float*)sink, iters);
+    else mfma_probe_kernel<false><<<dim3(blocks), dim3(256), 0, stream>>>((float*)sink, iters);
     PICOLM_LAUNCH_CHECK("mfma_probe");
     return 0;
 }

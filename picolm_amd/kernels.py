@@ -608,8 +608,9 @@ def read_probe(src: torch.Tensor, sink: torch.Tensor, blocks: int = 4096, unroll
     _check(lib().picolm_read_probe(_ptr(src), ctypes.c_size_t(nbytes - nbytes % 16), _ptr(sink), blocks, int(unroll4), _stream()))
 
 
-def mfma_probe(sink: torch.Tensor, blocks: int, iters: int) -> float:
-    """Queue a compute-only MFMA kernel; returns the flops it performs."""
+def mfma_probe(sink: torch.Tensor, blocks: int, iters: int, random_operands: bool = False) -> float:
+    """Queue a compute-only MFMA kernel (on small integers, or on pseudo-random values that make
+    the GPU draw the power real data does); returns the flops it performs."""
     _dev("mfma_probe.sink", sink, torch.float32)
-    _check(lib().picolm_mfma_probe(_ptr(sink), blocks, iters, _stream()))
+    _check(lib().picolm_mfma_probe(_ptr(sink), blocks, iters, int(random_operands), _stream()))
     return blocks * 4 * iters * 8 * 32768.0
