@@ -9,8 +9,10 @@
 // (k_page_offset, v_page_offset), so that a wave-wide load of an operand reads 1 KB in a row.
 // Softmax statistics are float, in the base-2 domain: p = exp2(s*scale*log2e - m).
 //
-//   prefill: a workgroup of 4 waves shares K and V^T tiles of one page through LDS; a wave
-//            owns 32 new tokens of one query head; with grouped heads the waves of a
+//   prefill: a workgroup of 4 waves shares K and V^T tiles of one page through LDS, where they
+//            arrive straight from the cache (global_load_lds_dwordx4); a wave owns 32 new tokens
+//            of one query head and takes a page as two tiles of 32 keys, one tile's softmax
+//            written between the other tile's products; with grouped heads the waves of a
 //            workgroup take different heads of the group, so a page is loaded once per group.
 //   decode : a wave streams its own pages straight from global memory into MFMA operands
 //            (columns = the query heads of one KV group); the 4 waves of a workgroup take

@@ -318,7 +318,9 @@ def test_gemm_tiled_direct_to_lds(variant):
     """The variants whose tiles go from global memory straight into LDS: K in whole steps of 64,
     fewer steps than stages, many steps (every stage is reused), ragged M and N."""
     for M, N, Kd in ((300, 530, 1024), (70, 260, 64), (513, 100, 192), (9, 700, 128), (257, 258, 2048)):
-        for epi, cdt in ((0, torch.float32), (2, torch.bfloat16), (1, torch.float32), (0, torch.bfloat16)):
+        # (the gated epilogue stores pairs of columns where the output's rows are an even number of
+        # values long, N = 260, 100, 700, and single values otherwise; in either type)
+        for epi, cdt in ((0, torch.float32), (2, torch.bfloat16), (1, torch.float32), (0, torch.bfloat16), (2, torch.float32)):
             run_gemm(K().gemm_tiled, M, N, Kd, epi, torch.bfloat16, torch.bfloat16, cdt, variant=variant)
     with pytest.raises(Exception, match="multiple"):
         run_gemm(K().gemm_tiled, 70, 64, 72, 0, torch.bfloat16, torch.bfloat16, torch.float32, variant=variant)
