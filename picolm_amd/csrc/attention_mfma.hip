@@ -587,27 +587,45 @@ __global__ __launch_bounds__(DEC_WAVES * 64) __attribute__((amdgpu_waves_per_eu(
     // tile tt of the chunk: keys 32*tt .. 32*tt+31 counted from the chunk's first page
     const int n_tiles = 2 * (page_hi - page_lo);
     auto page_of_tile = [&](int tt) {                       // the first eight tiles' pages came with the entry
+        if (tt >= n_tiles) return 0;
         if (tt >= 8) return pt[(page_lo + tt / 2) % a.ring_pages];
         return tt < 2 ? work.phys[0] : tt < 4 ? work.phys[1] : tt < 6 ? work.phys[2] : work.phys[3];
     };
-    int phys = page_of_tile(wave);
-    for (int tt = wave; tt < n_tiles; tt += DEC_WAVES) {
-        const int page = page_lo + tt / 2, t = tt & 1;
-        const int key0 = page * PAGE_TOKENS + 32 * t;
-        if (key0 > key_max) break;                           // nothing of this tile, or of a later one, is visible
-        const int next_phys = tt + DEC_WAVES < n_tiles ? page_of_tile(tt + DEC_WAVES) : 0;   // asked for before this tile's data
-        const size_t base = (size_t)phys * page_elems + (size_t)g * PAGE_TOKENS * D;
-        // tile t of the group's part of a page: 32 * D elements of K, then of V^T, as operands
-        const bf16_t* kp = (const bf16_t*)a.k_pages + base + (size_t)t * 32 * D + lane * 8;
-        const bf16_t* vp = (const bf16_t*)a.v_pages + base + (size_t)t * 32 * D + lane * 8;
-        const int n_keys = key_max - key0 + 1;               // >= 1; keys past it are not this sequence's, or not written yet
-        bf16x8 Kf[D / 16], Vf[D / 32][2];
+    // whether anything of tile tt is visible (if not, nothing of a later one is either)
+    auto visible = [&](int tt) { return tt < n_tiles && (page_lo + tt / 2) * PAGE_TOKENS + 32 * (tt & 1) <= key_max; };
+    // tile t of the group's part of a page: 32 * D elements of K, then of V^T, as operands
+    auto tile_offset = [&](int tt, int phys) {
+        return (size_t)phys * page_elems + (size_t)g * PAGE_TOKENS * D + (size_t)(tt & 1) * 32 * D + lane * 8;
+    };
+    // A wave takes tiles wave, wave + DEC_WAVES, ..  The keys of its next tile are asked for before
+    // it attends to this one, and this tile's values when its keys are already there: the scores and
+    // the softmax run while the values are on their way.  The page of the tile after the next is
+    // looked up a round ahead of its loads.
+    bf16x8 Kf[D / 16], Kn[D / 16], Vf[D / 32][2];
+    int tt = wave;
+    bool have = visible(tt);
+    int phys = page_of_tile(tt), phys_next = page_of_tile(tt + DEC_WAVES);
+    if (have) {
+        const bf16_t* kp = (const bf16_t*)a.k_pages + tile_offset(tt, phys);
 #pragma unroll
         for (int s = 0; s < D / 16; ++s) Kf[s] = ldg8(kp + 512 * s);
+    }
+    while (have) {
+        const int key0 = (page_lo + tt / 2) * PAGE_TOKENS + 32 * (tt & 1);
+        const int n_keys = key_max - key0 + 1;               // >= 1; keys past it are not this sequence's, or not written yet
+        const bf16_t* vp = (const bf16_t*)a.v_pages + tile_offset(tt, phys);
 #pragma unroll
         for (int dt = 0; dt < D / 32; ++dt)
 #pragma unroll
             for (int ks = 0; ks < 2; ++ks) Vf[dt][ks] = ldg8(vp + 512 * (2 * dt + ks));
+        const int tn = tt + DEC_WAVES;
+        const bool have_next = visible(tn);
+        const int phys_after = page_of_tile(tn + DEC_WAVES);
+        if (have_next) {
+            const bf16_t* kp = (const bf16_t*)a.k_pages + tile_offset(tn, phys_next);
+#pragma unroll
+            for (int s = 0; s < D / 16; ++s) Kn[s] = ldg8(kp + 512 * s);
+        }
         if (n_keys < 32) {                                   // keys past the end may hold anything
 #pragma unroll
             for (int dt = 0; dt < D / 32; ++dt)
@@ -620,7 +638,12 @@ __global__ __launch_bounds__(DEC_WAVES * 64) __attribute__((amdgpu_waves_per_eu(
                 }
         }
         attend_tile<D>(Qf, Kf, Vf, O, m_run, l_run, key0, key_max, qpos, q_ok, a.window, scale2, h);
-        phys = next_phys;
+#pragma unroll
+        for (int s = 0; s < D / 16; ++s) Kf[s] = Kn[s];
+        tt = tn;
+        have = have_next;
+        phys = phys_next;
+        phys_next = phys_after;
     }
     // merge the waves
     float* mine = mrg + (size_t)wave * Rc * (D + 2);
