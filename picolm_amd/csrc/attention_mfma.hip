@@ -567,7 +567,7 @@ __global__ __launch_bounds__(DEC_WAVES * 64) __attribute__((amdgpu_waves_per_eu(
                 knew[i0] = (float)to_bf16(y0);
                 knew[i1] = (float)to_bf16(y1);
             }
-            if (tid >= 64 && tid < 64 + D) vnew[tid - 64] = (float)to_bf16(vrow[tid - 64]);
+            for (int i = tid; i < D; i += DEC_WAVES * 64) vnew[i] = (float)to_bf16(vrow[i]);
         }
     } else {
         const bf16_t* qp = (const bf16_t*)a.q + tok * a.H * D + (size_t)head * D + 8 * h;
