@@ -105,6 +105,9 @@ def main() -> int:
     ap.add_argument("--prompt-range", default="",
                     help="prompt lengths of the decode runs, uniform in LO,HI (default: the shape's, 128,2048 for the 8B shape)")
     ap.add_argument("--context", type=int, default=CONTEXT, help="longest sequence the cache is laid out for")
+    ap.add_argument("--weight-std", type=float, default=None,
+                    help="standard deviation of the random weights (default: the shape's); 0 makes every operand of "
+                         "every product zero, which shows what the GPU's power limit costs the same kernels on real data")
     ap.add_argument("--steps-ahead", type=int, choices=[0, 1], default=1,
                     help="1 (the generation loop's way): the next step is launched before this step's tokens are "
                          "read on the host; 0: the host reads every step's tokens first")
@@ -132,6 +135,8 @@ def main() -> int:
     cfg = LlamaConfig.from_dict(cfg_dict)
     dev = torch.device("cuda:0")
     t0 = time.time()
+    if args.weight_std is not None:
+        shape = dict(shape, std=args.weight_std)
     model = random_model(cfg, seed=0, std=shape["std"], dtype="bfloat16", device=dev)
     torch.cuda.synchronize()
     print(f"[bench] {shape['name']}: {cfg.num_hidden_layers} layers, {weight_bytes(cfg) / 1e9:.1f} GB of weights ready in "
