@@ -315,7 +315,7 @@ static int launch_splitk_reduce(const float* ws, void* C, int c_dt, int M, int N
 
 // variant 0 picks by shape.  Tiles loaded straight into LDS (K a multiple of 64):
 //   9: 256x256, 8 waves, two stages of 64 columns;  10: 256(n)x128(m), 8 waves, three stages;
-//   11: 128x128, 4 waves, four stages;
+//   11: 128x128, 4 waves, four stages;  14: 192(n)x256(m), 8 waves, two stages;
 //   12: 128(n)x64(m), 4 waves, three stages;  13: 128(n)x32(m), 4 waves, four stages: for decode
 //   batches of up to 64 or 32 rows, where the weights stream once and K may be split.
 // Tiles staged through registers (any K that is a multiple of 8):
@@ -325,7 +325,7 @@ static int launch_splitk_reduce(const float* ws, void* C, int c_dt, int M, int N
 // n_first > 0: the first n_first columns of 256x256 tiles go to variant 9 and the rest to variant
 // 10: a last round that fills half of the CUs or less costs nearly a whole round, and the 256x128
 // tile gives those columns twice the workgroups.
-static int tiled_plan(int M, int N, int K, int& n_first) {
+static int tiled_plan_256(int M, int N, int K, int& n_first) {
     n_first = 0;
     const int tiles_m = ceil_div(M, 256), tiles_n = ceil_div(N, 256);
     const int64_t t256 = (int64_t)tiles_m * tiles_n;
@@ -339,6 +339,31 @@ static int tiled_plan(int M, int N, int K, int& n_first) {
         return 9;
     }
     return t256 >= 144 ? 9 : t128m >= 144 ? 10 : 11;
+}
+// Where N is a whole number of 192 columns (the qkv product of 32 + 8 + 8 heads of 128), tiles of
+// 192 columns by 256 rows (variant 14) may fill the CUs' rounds better than 256 x 256: 2,048 rows of
+// 6,144 columns are 192 tiles of the one kind, three quarters of a round, and exactly 256 of the
+// other.  The plans are compared by their rounds weighted with the tile's size (a 256 x 128 tile
+// does a little more than half the work of a 256 x 256 tile's time, a 192-column tile three
+// quarters and a little); measured at 1,024 to 16,384 rows of the qkv shape, the rule takes the
+// faster plan everywhere (15 % at 1,536 rows, 6 % at 2,048, 5 % at 3,072 and 6,144).
+static int tiled_plan(int M, int N, int K, int& n_first) {
+    const int variant = tiled_plan_256(M, N, K, n_first);
+    if (K % 64 != 0 || N % 192 != 0 || variant == 11) return variant;
+    const int tiles_m = ceil_div(M, 256);
+    const int64_t t256 = (int64_t)tiles_m * ceil_div(N, 256), t192 = (int64_t)tiles_m * (N / 192);
+    double cost;
+    if (n_first > 0)
+        cost = (double)(t256 / 256) + 0.55 * (double)ceil_div64((int64_t)(ceil_div(N, 256) - n_first) * ceil_div(M, 128), 256);
+    else if (variant == 9)
+        cost = (double)ceil_div64(t256, 256);
+    else
+        cost = 0.55 * (double)ceil_div64((int64_t)ceil_div(M, 128) * ceil_div(N, 256), 256);
+    if (t192 >= 144 && 0.77 * (double)ceil_div64(t192, 256) <= cost) {
+        n_first = 0;
+        return 14;
+    }
+    return variant;
 }
 
 // A short prompt's product with a narrow output has tiles for half of the CUs or fewer (512 rows
@@ -381,7 +406,7 @@ extern "C" int picolm_gemm_tiled_norm_parts(int M, int N, int K, int64_t ws_floa
     int variant, splits, n_first;
     tiled_choice(M, N, K, ws_floats, variant, splits, n_first);
     if (splits > 1) return N / 1024;
-    return variant == 9 || variant == 10 ? ceil_div(N, 256) : variant == 11 ? ceil_div(N, 128) : 0;
+    return variant == 9 || variant == 10 ? ceil_div(N, 256) : variant == 11 ? ceil_div(N, 128) : variant == 14 ? ceil_div(N, 192) : 0;
 }
 
 static int launch_splitk_reduce(const float* ws, void* C, int c_dt, int M, int N, int64_t ldc, int splits, int epilogue,
@@ -428,13 +453,14 @@ static int gemm_tiled_linked(const void* A, const void* W, void* C, int c_dt, in
         }
     }
     if (link.ssq || link.next_w)
-        PICOLM_REQUIRE(variant >= 9 && variant <= 11, "gemm_tiled: tile variant %d takes no part in a split norm", variant);
+        PICOLM_REQUIRE((variant >= 9 && variant <= 11) || variant == 14, "gemm_tiled: tile variant %d takes no part in a split norm", variant);
     switch (variant) {
         case 1: return launch_tiled<2, 2, 2, 2, 2>(A, W, C, c_dt, M, N, K, lda, ldw, ldc, epilogue, stream);
         case 4: return launch_tiled<2, 4, 4, 2, 1>(A, W, C, c_dt, M, N, K, lda, ldw, ldc, epilogue, stream);
         case 9: return picolm_gemm_direct_prefill_(9, A, W, C, c_dt, M, N, K, lda, ldw, ldc, epilogue, stream, 1, 0, link);
         case 10: return picolm_gemm_direct_prefill_(10, A, W, C, c_dt, M, N, K, lda, ldw, ldc, epilogue, stream, 1, 0, link);
         case 11: return picolm_gemm_direct_prefill_(11, A, W, C, c_dt, M, N, K, lda, ldw, ldc, epilogue, stream, 1, 0, link);
+        case 14: return picolm_gemm_direct_prefill_(14, A, W, C, c_dt, M, N, K, lda, ldw, ldc, epilogue, stream, 1, 0, link);
         case 12: return launch_direct<1, 2, 4, 1, 64, 3>(A, W, C, c_dt, M, N, K, lda, ldw, ldc, epilogue, stream);
         case 13: return launch_direct<1, 1, 4, 1, 64, 4>(A, W, C, c_dt, M, N, K, lda, ldw, ldc, epilogue, stream);
     }

@@ -259,10 +259,11 @@ def test_gemm_with_a_norm_split_between_two_products_of_a_wide_decode_batch(M, D
                                   torch.zeros(M, 128 * 200, device=DEV), 1, prepares=True)     # uncut: no preparing
 
 
-@pytest.mark.parametrize("M,D", [(65, 1024), (300, 1024), (2048, 1024), (65, 4352), (300, 4352), (2048, 10240)])
+@pytest.mark.parametrize("M,D", [(65, 1024), (300, 1024), (2048, 1024), (65, 4352), (300, 4352), (2048, 10240), (1536, 6144)])
 def test_gemm_with_a_norm_split_between_two_products_of_a_prefill_step(M, D):
     """More than 64 rows: the tile kernels keep sums for every row, one share per column of tiles;
-    10240 columns at 2048 rows are two launches with different tiles, which must meet without a seam."""
+    10240 columns at 2048 rows are two launches with different tiles, which must meet without a seam;
+    6144 columns at 1536 or 2048 rows take the tiles of 192 columns, in either role."""
     k = K()
     g = torch.Generator().manual_seed(M * 31 + D)
     eps, K1 = 1e-5, 256
@@ -284,7 +285,7 @@ def test_gemm_with_a_norm_split_between_two_products_of_a_prefill_step(M, D):
     want = (x.double().cpu() ** 2).sum(dim=1)
     assert ((total - want).abs() <= 1e-5 * want + 1e-30).all()
     normed = x.double().cpu() / torch.sqrt((x.double().cpu() ** 2).mean(dim=1, keepdim=True) + eps) * nw.double()
-    for N2 in (384, 3072 + 6):
+    for N2 in (384, 3072 + 6) + ((6144,) if (M, D) == (2048, 1024) else ()):
         w2 = (torch.randn(N2, D, generator=g) * 0.1).to(torch.bfloat16)
         for epi, cdt in ((0, torch.float32), (2, torch.bfloat16), (1, torch.float32)):
             c = torch.randn(M, N2 // 2 if epi == 2 else N2, generator=g).to(cdt).to(DEV)
@@ -296,6 +297,13 @@ def test_gemm_with_a_norm_split_between_two_products_of_a_prefill_step(M, D):
     # K no multiple of 64: the older tiles, which take no part
     assert not k.gemm_links_norms(torch.zeros(M, 72, dtype=torch.bfloat16, device=DEV),
                                   torch.zeros(D, 72, dtype=torch.bfloat16, device=DEV), x, 1, prepares=True)
+
+
+def test_gemm_tiles_of_192_columns_where_they_fill_the_rounds_better():
+    """1536 rows of 6144 columns: 144 tiles of 256 x 256 or 192 of 192 columns; the plan takes the latter."""
+    for epi, cdt in ((0, torch.float32), (2, torch.bfloat16), (1, torch.float32)):
+        run_gemm(K().gemm_tiled, 1536, 6144, 128, epi, torch.bfloat16, torch.bfloat16, cdt)
+        run_gemm(K().gemm_tiled, 1500, 6144, 64, epi, torch.bfloat16, torch.bfloat16, cdt)
 
 
 def test_gemm_tiled_splits_a_partial_last_round():
@@ -313,7 +321,7 @@ def test_gemm_tiled_block_tiles(variant):
             run_gemm(K().gemm_tiled, M, N, Kd, epi, torch.bfloat16, torch.bfloat16, cdt, variant=variant)
 
 
-@pytest.mark.parametrize("variant", [9, 10, 11, 12, 13])
+@pytest.mark.parametrize("variant", [9, 10, 11, 12, 13, 14])
 def test_gemm_tiled_direct_to_lds(variant):
     """The variants whose tiles go from global memory straight into LDS: K in whole steps of 64,
     fewer steps than stages, many steps (every stage is reused), ragged M and N."""
