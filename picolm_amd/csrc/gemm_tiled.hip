@@ -315,7 +315,7 @@ static int launch_splitk_reduce(const float* ws, void* C, int c_dt, int M, int N
 
 // variant 0 picks by shape.  Tiles loaded straight into LDS (K a multiple of 64):
 //   9: 256x256, 8 waves, two stages of 64 columns;  10: 256(n)x128(m), 8 waves, three stages;
-//   11: 128x128, 4 waves, four stages;  14: 192(n)x256(m), 8 waves, two stages;
+//   11: 128x128, 4 waves, four stages;  14: 192(n)x256(m), 15: 320(n)x256(m), 8 waves, two stages;
 //   12: 128(n)x64(m), 4 waves, three stages;  13: 128(n)x32(m), 4 waves, four stages: for decode
 //   batches of up to 64 or 32 rows, where the weights stream once and K may be split.
 // Tiles staged through registers (any K that is a multiple of 8):
@@ -343,15 +343,15 @@ static int tiled_plan_256(int M, int N, int K, int& n_first) {
 // Where N is a whole number of 192 columns (the qkv product of 32 + 8 + 8 heads of 128), tiles of
 // 192 columns by 256 rows (variant 14) may fill the CUs' rounds better than 256 x 256: 2,048 rows of
 // 6,144 columns are 192 tiles of the one kind, three quarters of a round, and exactly 256 of the
-// other.  The plans are compared by their rounds weighted with the tile's size (a 256 x 128 tile
+// other.  Likewise 320 columns (variant 15) for 10,240 (64 + 8 + 8 heads): 320 tiles or 256.  The plans are compared by their rounds weighted with the tile's size (a 256 x 128 tile
 // does a little more than half the work of a 256 x 256 tile's time, a 192-column tile three
 // quarters and a little); measured at 1,024 to 16,384 rows of the qkv shape, the rule takes the
 // faster plan everywhere (15 % at 1,536 rows, 6 % at 2,048, 5 % at 3,072 and 6,144).
-static int tiled_plan(int M, int N, int K, int& n_first) {
+static int tiled_plan(int M, int N, int K, int epilogue, int& n_first) {
     const int variant = tiled_plan_256(M, N, K, n_first);
-    if (K % 64 != 0 || N % 192 != 0 || variant == 11) return variant;
+    if (K % 64 != 0 || variant == 11) return variant;
     const int tiles_m = ceil_div(M, 256);
-    const int64_t t256 = (int64_t)tiles_m * ceil_div(N, 256), t192 = (int64_t)tiles_m * (N / 192);
+    const int64_t t256 = (int64_t)tiles_m * ceil_div(N, 256);
     double cost;
     if (n_first > 0)
         cost = (double)(t256 / 256) + 0.55 * (double)ceil_div64((int64_t)(ceil_div(N, 256) - n_first) * ceil_div(M, 128), 256);
@@ -359,11 +359,23 @@ static int tiled_plan(int M, int N, int K, int& n_first) {
         cost = (double)ceil_div64(t256, 256);
     else
         cost = 0.55 * (double)ceil_div64((int64_t)ceil_div(M, 128) * ceil_div(N, 256), 256);
-    if (t192 >= 144 && 0.77 * (double)ceil_div64(t192, 256) <= cost) {
-        n_first = 0;
-        return 14;
+    // tiles of 192 or 320 columns (variants 14, 15) where the columns are a whole number of them:
+    // their rounds times the width's share of 256, a little more for the narrow tile and a little
+    // less for the wide one, which moves fewer bytes per flop (1.35 against 1.22 PFLOP/s at 8,192
+    // rows of 10,240 columns).  The wide tile's sums fill the registers: not with the epilogue that
+    // adds to what is there, which needs room of its own.
+    int best = variant;
+    for (int width : {192, 320}) {
+        if (N % width != 0 || (width == 320 && epilogue == 1)) continue;
+        const int64_t t = (int64_t)tiles_m * (N / width);
+        const double c = (width == 192 ? 1.03 : 0.93) * width / 256.0 * (double)ceil_div64(t, 256);
+        if (t >= 144 && c <= cost) {
+            cost = c;
+            best = width == 192 ? 14 : 15;
+        }
     }
-    return variant;
+    if (best != variant) n_first = 0;
+    return best;
 }
 
 // A short prompt's product with a narrow output has tiles for half of the CUs or fewer (512 rows
@@ -385,8 +397,8 @@ static int tiled_splits(int M, int N, int K, int variant, int64_t ws_floats) {
 // too many to cut but the 256x128 ones are few and K is long (a prompt of 768 tokens into the
 // model's width from the feed-forward's), the larger tile cut in two is the faster (measured
 // 103 against 114 us at 768 x 4096 x 14336; with K = 4096 the smaller tile uncut wins).
-static void tiled_choice(int M, int N, int K, int64_t ws_floats, int& variant, int& splits, int& n_first) {
-    variant = tiled_plan(M, N, K, n_first);
+static void tiled_choice(int M, int N, int K, int epilogue, int64_t ws_floats, int& variant, int& splits, int& n_first) {
+    variant = tiled_plan(M, N, K, epilogue, n_first);
     splits = 1;
     if (n_first > 0) return;
     splits = tiled_splits(M, N, K, variant, ws_floats);
@@ -404,9 +416,9 @@ static void tiled_choice(int M, int N, int K, int64_t ws_floats, int& variant, i
 // when a workspace of ws_floats floats allows it), or 0 if its kernel cannot take part in a split norm.
 extern "C" int picolm_gemm_tiled_norm_parts(int M, int N, int K, int64_t ws_floats) {
     int variant, splits, n_first;
-    tiled_choice(M, N, K, ws_floats, variant, splits, n_first);
+    tiled_choice(M, N, K, 1, ws_floats, variant, splits, n_first);       // the product that prepares a norm adds to the rows
     if (splits > 1) return N / 1024;
-    return variant == 9 || variant == 10 ? ceil_div(N, 256) : variant == 11 ? ceil_div(N, 128) : variant == 14 ? ceil_div(N, 192) : 0;
+    return variant == 9 || variant == 10 ? ceil_div(N, 256) : variant == 11 ? ceil_div(N, 128) : variant == 14 ? ceil_div(N, 192) : variant == 15 ? ceil_div(N, 320) : 0;
 }
 
 static int launch_splitk_reduce(const float* ws, void* C, int c_dt, int M, int N, int64_t ldc, int splits, int epilogue,
@@ -428,7 +440,7 @@ static int gemm_tiled_linked(const void* A, const void* W, void* C, int c_dt, in
                              float* ws, int64_t ws_floats) {
     if (variant == 0) {
         int n_first, splits;
-        tiled_choice(M, N, K, ws != nullptr ? ws_floats : 0, variant, splits, n_first);
+        tiled_choice(M, N, K, epilogue, ws != nullptr ? ws_floats : 0, variant, splits, n_first);
         if (splits > 1) {
             PICOLM_REQUIRE(((uintptr_t)ws & 15) == 0, "gemm_tiled: the workspace of a cut product must be 16-byte aligned");
             const int rc = picolm_gemm_direct_prefill_(variant, A, W, ws, PICOLM_F32, M, N, K, lda, ldw, N, 0, stream, splits,
@@ -453,7 +465,7 @@ static int gemm_tiled_linked(const void* A, const void* W, void* C, int c_dt, in
         }
     }
     if (link.ssq || link.next_w)
-        PICOLM_REQUIRE((variant >= 9 && variant <= 11) || variant == 14, "gemm_tiled: tile variant %d takes no part in a split norm", variant);
+        PICOLM_REQUIRE((variant >= 9 && variant <= 11) || variant == 14 || variant == 15, "gemm_tiled: tile variant %d takes no part in a split norm", variant);
     switch (variant) {
         case 1: return launch_tiled<2, 2, 2, 2, 2>(A, W, C, c_dt, M, N, K, lda, ldw, ldc, epilogue, stream);
         case 4: return launch_tiled<2, 4, 4, 2, 1>(A, W, C, c_dt, M, N, K, lda, ldw, ldc, epilogue, stream);
@@ -461,6 +473,7 @@ static int gemm_tiled_linked(const void* A, const void* W, void* C, int c_dt, in
         case 10: return picolm_gemm_direct_prefill_(10, A, W, C, c_dt, M, N, K, lda, ldw, ldc, epilogue, stream, 1, 0, link);
         case 11: return picolm_gemm_direct_prefill_(11, A, W, C, c_dt, M, N, K, lda, ldw, ldc, epilogue, stream, 1, 0, link);
         case 14: return picolm_gemm_direct_prefill_(14, A, W, C, c_dt, M, N, K, lda, ldw, ldc, epilogue, stream, 1, 0, link);
+        case 15: return picolm_gemm_direct_prefill_(15, A, W, C, c_dt, M, N, K, lda, ldw, ldc, epilogue, stream, 1, 0, link);
         case 12: return launch_direct<1, 2, 4, 1, 64, 3>(A, W, C, c_dt, M, N, K, lda, ldw, ldc, epilogue, stream);
         case 13: return launch_direct<1, 1, 4, 1, 64, 4>(A, W, C, c_dt, M, N, K, lda, ldw, ldc, epilogue, stream);
     }

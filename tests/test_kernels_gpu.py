@@ -299,11 +299,15 @@ def test_gemm_with_a_norm_split_between_two_products_of_a_prefill_step(M, D):
                                   torch.zeros(D, 72, dtype=torch.bfloat16, device=DEV), x, 1, prepares=True)
 
 
-def test_gemm_tiles_of_192_columns_where_they_fill_the_rounds_better():
-    """1536 rows of 6144 columns: 144 tiles of 256 x 256 or 192 of 192 columns; the plan takes the latter."""
+def test_gemm_tiles_of_192_and_320_columns_where_they_fill_the_rounds_better():
+    """1536 rows of 6144 columns: 144 tiles of 256 x 256 or 192 of 192 columns; 2048 rows of 10240
+    columns: 320 tiles or 256 of 320 columns; the plan takes the latter in both cases (the wide
+    tile not with the adding epilogue)."""
     for epi, cdt in ((0, torch.float32), (2, torch.bfloat16), (1, torch.float32)):
         run_gemm(K().gemm_tiled, 1536, 6144, 128, epi, torch.bfloat16, torch.bfloat16, cdt)
         run_gemm(K().gemm_tiled, 1500, 6144, 64, epi, torch.bfloat16, torch.bfloat16, cdt)
+        run_gemm(K().gemm_tiled, 2048, 10240, 128, epi, torch.bfloat16, torch.bfloat16, cdt)
+        run_gemm(K().gemm_tiled, 2000, 10240, 64, epi, torch.bfloat16, torch.bfloat16, cdt)
 
 
 def test_gemm_tiled_splits_a_partial_last_round():
@@ -321,7 +325,7 @@ def test_gemm_tiled_block_tiles(variant):
             run_gemm(K().gemm_tiled, M, N, Kd, epi, torch.bfloat16, torch.bfloat16, cdt, variant=variant)
 
 
-@pytest.mark.parametrize("variant", [9, 10, 11, 12, 13, 14])
+@pytest.mark.parametrize("variant", [9, 10, 11, 12, 13, 14, 15])
 def test_gemm_tiled_direct_to_lds(variant):
     """The variants whose tiles go from global memory straight into LDS: K in whole steps of 64,
     fewer steps than stages, many steps (every stage is reused), ragged M and N."""
