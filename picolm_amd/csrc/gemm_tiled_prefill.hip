@@ -1,5 +1,5 @@
-// The prefill's tile variants 10 and 11 of the kernel in gemm_direct.h (variant 9 has a file of
-// its own), apart from the others so that they compile side by side.
+// The prefill's tile variants 10, 11, 14 and 15 of the kernel in gemm_direct.h (variant 9 has a
+// file of its own), apart from the others so that they compile side by side.
 #include "gemm_direct.h"
 
 int picolm_gemm_direct_prefill_(int variant, const void* A, const void* W, void* C, int c_dt, int M, int N, int K,
