@@ -111,6 +111,9 @@ int picolm_gemm_skinny_linked_(const void* A, const void* W, void* C, int c_dt, 
 int picolm_gemm_direct_prefill_(int variant, const void* A, const void* W, void* C, int c_dt, int M, int N, int K,
                                 int64_t lda, int64_t ldw, int64_t ldc, int epilogue, hipStream_t stream, int splits,
                                 int64_t c_split_stride, NormLink link);
+int picolm_gemm_direct_wide_(int variant, const void* A, const void* W, void* C, int c_dt, int M, int N, int K,
+                             int64_t lda, int64_t ldw, int64_t ldc, int epilogue, hipStream_t stream, int splits,
+                             int64_t c_split_stride, NormLink link);
 int picolm_gemm_direct_256x256_(const void* A, const void* W, void* C, int c_dt, int M, int N, int K, int64_t lda,
                                 int64_t ldw, int64_t ldc, int epilogue, hipStream_t stream, int splits,
                                 int64_t c_split_stride, NormLink link);
