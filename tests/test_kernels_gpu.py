@@ -659,6 +659,105 @@ def test_attention_finds_a_far_key(dtype):
             assert np.abs(got[h] - case.v[0][target, h // 2]).max() < 2e-2
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_attention_over_pages_beyond_four_gigabytes(dtype):
+    """A cache of a large batch of long sequences: the pages of this case lie more than 2^32 bytes
+    (and more than 2^31 elements) into the key and value arrays.  An offset computed in 32 bits
+    anywhere (the table's page times the page's size) reads or writes somewhere else."""
+    H, G, d = 32, 8, 128
+    page_bytes = G * PAGE * d * (4 if dtype == torch.float32 else 2)
+    base = (1 << 32) // page_bytes + 777
+    case = PagedCase(H, G, d, [0, 130, 650], [70, 33, 1], dtype, seed=5)
+
+    def moved(pages):
+        big = torch.empty((base + pages.shape[0],) + tuple(pages.shape[1:]), dtype=dtype, device=DEV)
+        big[:64].fill_(float("nan"))          # where a truncated offset of these pages would land
+        big[base:] = pages
+        return big
+    k_big, v_big = moved(case.k_pages), moved(case.v_pages)
+    table_host = case.table_host + base
+    table = table_host.to(DEV)
+    b = case.batch()
+    ref = case.reference(0)
+    out = torch.zeros_like(case.q_dev)
+    K().attn_prefill(case.q_dev, k_big, v_big, out, b, table, table.shape[1], H, G, d, 0, 1.0 / math.sqrt(d))
+    err = np.abs(out.double().cpu().numpy() - ref).max()
+    assert err <= tol(dtype, np.abs(ref).max()), err
+    # the last sequence alone as a decode step, its chunks combined by the kernel and by the merge kernel
+    from picolm_amd.engine.batch import StepBatch, decode_chunk_list, with_header
+    slot, pos0 = int(case.slots[2]), 650
+    db = StepBatch([slot], [pos0], [[0]], [[]], 10, DEV)
+    q1 = case.q_dev[-1:].contiguous()
+    for pages_per_chunk in (16, 2):
+        entries, most = decode_chunk_list(db.slots, db.pos0, 0, pages_per_chunk, table_host, table_host.shape[1])
+        chunk_list = torch.from_numpy(with_header(entries, len(entries))).to(DEV)
+        partial = torch.full((H * most * (d + 2),), float("nan"), device=DEV)
+        done = torch.zeros(K().attn_decode_counters(1, H, G), dtype=torch.int32, device=DEV)
+        for counters in (None, done):
+            out1 = torch.zeros_like(q1)
+            args = (q1, k_big, v_big, out1, partial, 1, chunk_list, len(entries), pages_per_chunk, most, db.seq_pos0,
+                    table, table.shape[1], H, G, d, 0, 1.0 / math.sqrt(d))
+            K().attn_decode(*args) if counters is None else K().attn_decode(*args, counters)
+            err = np.abs(out1.double().cpu().numpy() - ref[-1:]).max()
+            assert err <= tol(dtype, np.abs(ref).max()), (pages_per_chunk, err)
+    if dtype == torch.bfloat16:
+        # the decode step's one launch: rotation, cache write and attention; the new token's row must land
+        # in its page up there, and the output must be that of the sequence with this last token
+        rng = np.random.default_rng(2)
+        qkv1 = rng.standard_normal((1, (H + 2 * G) * d)).astype(np.float32)
+        inv = P.rope_inv_freq(d, 10000.0)
+        cos, sin = P.rope_tables(np.arange(800), inv)
+        c, s_ = P.rope_tables(np.asarray([pos0]), inv)
+        x = qkv1.astype(np.float64).reshape(1, H + 2 * G, d)
+        bf = lambda t: torch.from_numpy(np.ascontiguousarray(t)).to(torch.bfloat16)
+        q_new, k_new, v_new = P.apply_rope(x[:, :H], c, s_, "half")[0], P.apply_rope(x[:, H:H + G], c, s_, "half")[0], x[0, H + G:]
+        case.q[2][-1], case.k[2][-1], case.v[2][-1] = (bf(t).double().numpy() for t in (q_new, k_new, v_new))
+        ref1 = P.causal_attention(case.q[2], case.k[2], case.v[2], 0)[-1:].reshape(1, H * d)
+        tok_page = db.write_pages(0, table_host, table_host.shape[1])
+        assert int(tok_page[0]) >= base
+        entries, most = decode_chunk_list(db.slots, db.pos0, 0, 4, table_host, table_host.shape[1])
+        chunk_list = torch.from_numpy(with_header(entries, len(entries))).to(DEV)
+        partial = torch.full((H * most * (d + 2),), float("nan"), device=DEV)
+        out1 = torch.zeros(1, H * d, dtype=dtype, device=DEV)
+        K().attn_decode_rope(torch.from_numpy(qkv1).to(DEV), k_big, v_big, out1, partial, 1, chunk_list, len(entries), 4,
+                             most, db.seq_pos0, table, table.shape[1], H, G, d, 0, 1.0 / math.sqrt(d),
+                             torch.from_numpy(cos).float().to(DEV), torch.from_numpy(sin).float().to(DEV), 1, tok_page, done)
+        err = np.abs(out1.double().cpu().numpy() - ref1).max()
+        assert err <= tol(dtype, np.abs(ref1).max()), err
+        pg = int(tok_page[0])
+        kp, vp = K().kv_pages_unpack(k_big[pg:pg + 1], v_big[pg:pg + 1])
+        assert torch.equal(kp[0, :, pos0 % PAGE, :].cpu(), bf(k_new)) and torch.equal(vp[0, :, :, pos0 % PAGE].cpu(), bf(v_new))
+    # writing keys and values there: both kernels, read back through the plain order
+    rng = np.random.default_rng(1)
+    T = sum(case.lens_new)
+    qkv = torch.from_numpy(rng.standard_normal((T, (H + 2 * G) * d)).astype(np.float32)).to(DEV)
+    inv = P.rope_inv_freq(d, 1000.0)
+    cos, sin = (torch.from_numpy(x).float().to(DEV) for x in P.rope_tables(np.arange(800), inv))
+    positions = np.concatenate([np.arange(p, p + n) for p, n in zip(case.lens_old, case.lens_new)])
+    c, s_ = P.rope_tables(positions, inv)
+    x = qkv.double().cpu().numpy().reshape(T, H + 2 * G, d)
+    k_ref, v_ref = P.apply_rope(x[:, H:H + G], c, s_, "half"), x[:, H + G:]
+    seq_of = np.repeat(np.arange(3), case.lens_new)
+    tab = table_host.numpy()
+    for which in ("rope_kv_store", "kv_store_tiles"):
+        k_big[base:].zero_()
+        v_big[base:].zero_()
+        if which == "rope_kv_store":
+            q_out = torch.zeros(T, H * d, dtype=dtype, device=DEV)
+            K().rope_kv_store(qkv, q_out, k_big, v_big, cos, sin, 1, b.tok_pos,
+                              b.write_pages(0, table_host, table_host.shape[1]), H, G, d)
+        else:
+            K().kv_store_tiles(qkv, k_big, v_big, cos, sin, 1, b, table, table.shape[1], H, G, d)
+        kp, vp = K().kv_pages_unpack(k_big[base:], v_big[base:])
+        kp, vp = kp.double().cpu().numpy(), vp.double().cpu().numpy()
+        for t in range(T):
+            pg = tab[case.slots[seq_of[t]], positions[t] // PAGE] - base
+            assert np.abs(kp[pg, :, positions[t] % PAGE, :] - k_ref[t]).max() <= tol(dtype, 4.0), (which, t)
+            assert np.abs(vp[pg, :, :, positions[t] % PAGE] - v_ref[t]).max() <= tol(dtype, 4.0), (which, t)
+    del k_big, v_big
+    torch.cuda.empty_cache()
+
+
 # ------------------------------------------------------------------------------------------ rope
 @pytest.mark.parametrize("d", [16, 32, 48, 64, 128, 256])
 def test_kv_page_order_is_a_permutation(d):
