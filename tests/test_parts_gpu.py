@@ -268,6 +268,102 @@ def test_toy_architecture_with_a_stateful_mixer(tmp_path):
         unregister_architecture("ToyRunningMeanLM")
 
 
+@pytest.mark.parametrize("native", [True, False])
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_layer_order_names_a_block_twice_and_lets_a_call_read_anothers_cache(dtype, native, tmp_path):
+    """The order of layers is data.  Three blocks of the library's own parts run as four calls:
+    block 0, block 1, block 0 again (the same weights, keys and values of its own) and block 2,
+    whose attention writes nothing and reads the keys and values that the call of block 1 left
+    (its own k and v projections are loaded and unused).  Whole prompts as an unequal batch, then
+    token by token from a cut, in the library's step and in the one from Python, against the
+    plain functions."""
+    from picolm_amd.config import LlamaConfig, register_architecture, unregister_architecture
+    from picolm_amd.engine import DecoderModel, LayerCall, Session, load_model
+    from picolm_amd.parts import Attention, LMHead, PreNormBlock, RMSNorm, RotaryEmbedding, SwiGLU, TokenEmbedding
+    from picolm_amd.weights import write_random_model
+
+    def build(cfg):
+        D = cfg.hidden_size
+        rotary = RotaryEmbedding(cfg.head_dim, cfg.rope_theta, cfg.rope_scaling, cfg.rope_style)
+        blocks = []
+        for l in range(3):
+            q = f"model.layers.{l}."
+            blocks.append(PreNormBlock(RMSNorm(q + "input_layernorm.weight", D, cfg.rms_norm_eps),
+                                       Attention(q + "self_attn.", D, cfg.num_attention_heads, cfg.num_key_value_heads,
+                                                 cfg.head_dim, position=rotary),
+                                       RMSNorm(q + "post_attention_layernorm.weight", D, cfg.rms_norm_eps),
+                                       SwiGLU(q + "mlp.", D, cfg.intermediate_size)))
+        emb = TokenEmbedding("model.embed_tokens.weight", cfg.vocab_size, D)
+        return DecoderModel(cfg, emb, blocks, RMSNorm("model.norm.weight", D, cfg.rms_norm_eps),
+                            LMHead("lm_head.weight", cfg.vocab_size, D, emb, True),
+                            order=[0, 1, 0, LayerCall(2, reads_cache_of=1)])
+
+    name = "ToyOrderLM"
+    register_architecture(name, LlamaConfig.from_dict, build)
+    try:
+        c = dict(architectures=[name], hidden_size=192, num_attention_heads=6, num_key_value_heads=2, head_dim=32,
+                 intermediate_size=272, num_hidden_layers=3, vocab_size=301, rms_norm_eps=1e-5, rope_theta=10000.0,
+                 max_position_embeddings=512, tie_word_embeddings=True, torch_dtype="bfloat16")
+        cfg = LlamaConfig.from_dict(c)
+        d = write_random_model(cfg, str(tmp_path / "order"), seed=11, std=0.06)
+        model = load_model(d, dtype=dtype)
+        assert [g.n_entries for g in model.cache_spec.kv_groups] == [3]      # four calls, three of them own an entry
+        w = tiny.read_weights_f64(d)
+        pc = dict(c, rope_style=cfg.rope_style)
+        H, G, hd = 6, 2, 32
+
+        def plain(tokens):
+            T = len(tokens)
+            pos = np.arange(T)
+            x = w["model.embed_tokens.weight"][np.asarray(tokens)]
+            kept = {}
+            for call, (l, reads) in enumerate([(0, None), (1, None), (0, None), (2, 1)]):
+                q_ = f"model.layers.{l}."
+                h = P.rmsnorm(x, w[q_ + "input_layernorm.weight"], 1e-5)
+                if reads is None:
+                    x = x + P.attention_block(h, w, q_ + "self_attn.", pc, pos)
+                    inv = P.rope_inv_freq(hd, 10000.0)
+                    cos, sin = P.rope_tables(pos, inv)
+                    kept[call] = (P.apply_rope((h @ w[q_ + "self_attn.k_proj.weight"].T).reshape(T, G, hd), cos, sin, cfg.rope_style),
+                                  (h @ w[q_ + "self_attn.v_proj.weight"].T).reshape(T, G, hd))
+                else:
+                    inv = P.rope_inv_freq(hd, 10000.0)
+                    cos, sin = P.rope_tables(pos, inv)
+                    qq = P.apply_rope((h @ w[q_ + "self_attn.q_proj.weight"].T).reshape(T, H, hd), cos, sin, cfg.rope_style)
+                    a = P.causal_attention(qq, kept[reads][0], kept[reads][1]).reshape(T, H * hd)
+                    x = x + a @ w[q_ + "self_attn.o_proj.weight"].T
+                h = P.rmsnorm(x, w[q_ + "post_attention_layernorm.weight"], 1e-5)
+                x = x + P.swiglu(h, w[q_ + "mlp.gate_proj.weight"], w[q_ + "mlp.up_proj.weight"], w[q_ + "mlp.down_proj.weight"])
+            return P.rmsnorm(x, w["model.norm.weight"], 1e-5) @ w["model.embed_tokens.weight"].T
+
+        rng = np.random.default_rng(3)
+        reqs = [tiny.random_tokens(rng, n, 301) for n in (150, 9, 70)]
+        truth = [plain(r) for r in reqs]
+        tol_ = lambda t: tiny.tolerance(dtype, t, tiny.spread(192, 0.06))
+        s = Session(model, max_tokens=1024, n_slots=3, native=native)
+        assert (s.engine is not None) == native
+        slots = s.begin(3)
+        got = s.step(slots, reqs, [list(range(len(r))) for r in reqs]).double().cpu().numpy()
+        row = 0
+        for r, t in zip(reqs, truth):
+            assert np.abs(got[row:row + len(r)] - t).max() <= tol_(t)
+            row += len(r)
+        s.release(slots)
+        slots = s.begin(3)                                        # the slots again, from a cut, token by token
+        cut = [130, 1, 60]
+        s.step(slots, [r[:c_] for r, c_ in zip(reqs, cut)])
+        pos = dict(zip(range(3), cut))
+        live = [0, 1, 2]
+        while live:
+            out = s.step([slots[i] for i in live], [[reqs[i][pos[i]]] for i in live]).double().cpu().numpy()
+            for k, i in enumerate(live):
+                assert np.abs(out[k] - truth[i][pos[i]]).max() <= tol_(truth[i]), (i, pos[i])
+                pos[i] += 1
+            live = [i for i in live if pos[i] < len(reqs[i])]
+    finally:
+        unregister_architecture(name)
+
+
 def test_toy_mixer_whose_values_are_wider_than_its_keys(tmp_path):
     """A one-head attention defined here with keys of 16 and values of 24: the cache gives its
     group keys and values of their own sizes.  Whole prompts as an unequal batch, then the same
