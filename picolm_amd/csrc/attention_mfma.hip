@@ -33,6 +33,19 @@ typedef __attribute__((ext_vector_type(4))) float f32x4;
 #define LAZY_MAX_STEP 8.0f
 
 __device__ __forceinline__ bf16x8 ldg8(const bf16_t* p) { return *(const bf16x8*)p; }
+// N chunks of a tile of keys or values, 512 elements apart (a wave's load is one contiguous KB).
+// `once`: no other workgroup of the launch reads them, so they are marked non-temporal and pass the
+// caches without displacing anything (a sweep over memory is a seventh faster that way).
+template <int N>
+__device__ __forceinline__ void load_tile_chunks(bf16x8 (&dst)[N], const bf16_t* p, bool once) {
+    if (once) {
+#pragma unroll
+        for (int s = 0; s < N; ++s) dst[s] = __builtin_nontemporal_load((const bf16x8*)(p + 512 * s));
+    } else {
+#pragma unroll
+        for (int s = 0; s < N; ++s) dst[s] = ldg8(p + 512 * s);
+    }
+}
 __device__ __forceinline__ bf16x8 zero8() {
     bf16x8 z;
 #pragma unroll
@@ -602,29 +615,22 @@ __global__ __launch_bounds__(DEC_WAVES * 64) __attribute__((amdgpu_waves_per_eu(
     // the softmax run while the values are on their way.  The page of the tile after the next is
     // looked up a round ahead of its loads.
     bf16x8 Kf[D / 16], Kn[D / 16], Vf[D / 32][2];
+    const bool once = chunks == 1;        // all heads of the group are here: nobody else reads these keys and values
     int tt = wave;
     bool have = visible(tt);
     int phys = page_of_tile(tt), phys_next = page_of_tile(tt + DEC_WAVES);
     if (have) {
-        const bf16_t* kp = (const bf16_t*)a.k_pages + tile_offset(tt, phys);
-#pragma unroll
-        for (int s = 0; s < D / 16; ++s) Kf[s] = ldg8(kp + 512 * s);
+        load_tile_chunks(Kf, (const bf16_t*)a.k_pages + tile_offset(tt, phys), once);
     }
     while (have) {
         const int key0 = (page_lo + tt / 2) * PAGE_TOKENS + 32 * (tt & 1);
         const int n_keys = key_max - key0 + 1;               // >= 1; keys past it are not this sequence's, or not written yet
-        const bf16_t* vp = (const bf16_t*)a.v_pages + tile_offset(tt, phys);
-#pragma unroll
-        for (int dt = 0; dt < D / 32; ++dt)
-#pragma unroll
-            for (int ks = 0; ks < 2; ++ks) Vf[dt][ks] = ldg8(vp + 512 * (2 * dt + ks));
+        load_tile_chunks((bf16x8(&)[D / 16])Vf, (const bf16_t*)a.v_pages + tile_offset(tt, phys), once);
         const int tn = tt + DEC_WAVES;
         const bool have_next = visible(tn);
         const int phys_after = page_of_tile(tn + DEC_WAVES);
         if (have_next) {
-            const bf16_t* kp = (const bf16_t*)a.k_pages + tile_offset(tn, phys_next);
-#pragma unroll
-            for (int s = 0; s < D / 16; ++s) Kn[s] = ldg8(kp + 512 * s);
+            load_tile_chunks(Kn, (const bf16_t*)a.k_pages + tile_offset(tn, phys_next), once);
         }
         if (n_keys < 32) {                                   // keys past the end may hold anything
 #pragma unroll

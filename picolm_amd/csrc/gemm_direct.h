@@ -97,6 +97,7 @@ __global__ __launch_bounds__(64 * WN * WM) void gemm_direct_kernel(const bf16_t*
     // memory channels would take all the traffic.  With several rows of tiles the tiles that share
     // a slice must stay in step, so that one of them finds it in L2.
     const int n_steps = K / BK;
+    const bool stream_w = tiles_m == 1;       // with one row of tiles every weight is read once: past the caches
     const int first_step = tiles_m == 1 ? (int)(((unsigned)tile * 5u + blockIdx.y * 3u) % (unsigned)n_steps) : 0;
     auto issue = [&](int stage, int step) {
         const unsigned to = lds_wave + stage * (STAGE * 2);
@@ -104,8 +105,13 @@ __global__ __launch_bounds__(64 * WN * WM) void gemm_direct_kernel(const bf16_t*
         if (step >= n_steps) step -= n_steps;
         const void* wsrc = same_in_every_lane(w_tile + step * BK);
         const void* asrc = same_in_every_lane(a_tile + step * BK);
+        if (stream_w) {
 #pragma unroll
-        for (int j = 0; j < W_LOADS; ++j) load_16_bytes_to_lds(w_off[j], wsrc, to + j * (NW * RG * BK * 2));
+            for (int j = 0; j < W_LOADS; ++j) stream_16_bytes_to_lds(w_off[j], wsrc, to + j * (NW * RG * BK * 2));
+        } else {
+#pragma unroll
+            for (int j = 0; j < W_LOADS; ++j) load_16_bytes_to_lds(w_off[j], wsrc, to + j * (NW * RG * BK * 2));
+        }
 #pragma unroll
         for (int j = 0; j < A_LOADS; ++j) load_16_bytes_to_lds(a_off[j], asrc, to + (BN * BK * 2) + j * (NW * RG * BK * 2));
     };

@@ -11,6 +11,8 @@ typedef __attribute__((ext_vector_type(4))) float f32x4;
 typedef __attribute__((ext_vector_type(16))) float f32x16;
 
 __device__ __forceinline__ bf16x8 load_chunk(const bf16_t* p) { return *(const bf16x8*)p; }
+// a chunk of a matrix that this launch reads once: a non-temporal load (see stream_16_bytes_to_lds)
+__device__ __forceinline__ bf16x8 stream_chunk(const bf16_t* p) { return __builtin_nontemporal_load((const bf16x8*)p); }
 __device__ __forceinline__ bf16x8 zero_chunk() {
     bf16x8 z;
 #pragma unroll
