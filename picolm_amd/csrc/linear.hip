@@ -5,8 +5,8 @@
 // picolm/quant.c:4957-4968); here the number of rows decides as well:
 //   not bf16 x bf16, or K no multiple of 8      the float kernel on the vector ALU
 //   up to 16 rows                               skinny: weights streamed once into MFMA operands
-//                                               (tiles of 128 weight rows through LDS for 5..16
-//                                               rows and one round of such tiles)
+//                                               (tiles of 128 weight rows through LDS where there
+//                                               are 128 such tiles and more)
 //   17 to 64 rows                               128-row weight tiles through LDS, cut along K
 //                                               when there are fewer tiles than CUs
 //   more than 64 rows                           the prefill's tile variants by shape
@@ -116,9 +116,13 @@ extern "C" int picolm_linear(const void* A, int a_dt, const void* W, int w_dt, v
         return picolm_gemm_linked(A, W, C, c_dt, M, N, K, K, K, ldc, epilogue, 1, variant, splits, splits > 1 ? ws : nullptr,
                                   ws_floats, next_w, next_h, next_ssq, next_parts, ssq, n_parts, norm_len, eps, rows, stream);
     }
-    // several rows and one round of 128-row tiles for the CUs: the tiles share the activations
-    // through LDS (more rounds suit the skinny kernel's resident variant better)
-    const bool one_round = M > 4 && M <= 16 && K % 64 == 0 && N >= 16384 && N <= 128 * 256;
+    // enough weight rows for half a round and more of 128-row tiles: the tile kernel, whose loads
+    // cover whole lines, streams the weights past the caches (measured with weights from memory,
+    // 28,672 x 4,096: 37.0 us against the skinny kernel's 40.2 at one row, 37.2 against 43.7 at
+    // eight; 57,344 x 8,192: 142 against 164 and 144 against 177; 12,288 rows, 96 tiles, are
+    // better off skinny: 19 against 26 us).  One to four rows of many rounds (a vocabulary) stay
+    // skinny: 165 against 167 us for 128,256 rows.
+    const bool one_round = M <= 16 && K % 64 == 0 && N >= 16384 && (M > 4 || N <= 512 * 128);
     if (!linked) {
         if (one_round) return picolm_gemm_tiled_splitk(A, W, C, c_dt, M, N, K, K, K, ldc, epilogue, 13, 1, nullptr, stream);
         return picolm_gemm_skinny(A, W, C, c_dt, M, N, K, K, K, ldc, epilogue, 0, stream);
