@@ -226,8 +226,8 @@ def main() -> int:
                 torch.cuda.synchronize()
                 out.append(start.elapsed_time(stop) * 1e-3)
             return float(np.median(out))
-        read = max((4 << 30) / timed(lambda b=b, u=u: kernels.read_probe(src, sink, b, u)) / 1e9
-                   for b, u in ((2048, False), (1024, False), (512, True)))
+        read = max(kernels.read_probe(src, sink, b) / timed(lambda b=b: kernels.read_probe(src, sink, b)) / 1e9
+                   for b in (2048, 1024, 512))
         mfma = max(kernels.mfma_probe(fsink, b, 2000) / timed(lambda b=b: kernels.mfma_probe(fsink, b, 2000)) / 1e12
                    for b in (512, 1024, 2048))
         # the same loop on operands like real data: the power limit then sets the clock

@@ -13,8 +13,10 @@ const char* picolm_last_error(void);
 int picolm_abi_version(void);
 int picolm_device_check(void);     // 0 if the current device is a gfx950
 
-// reads `bytes` from `src` once; for bandwidth measurements
-int picolm_read_probe(const void* src, size_t bytes, void* sink, int blocks, int unroll4, hipStream_t stream);
+// Sweeps `src` once, each workgroup a contiguous share in whole rounds of 32 KB (picolm_read_probe_bytes
+// says how many bytes that reads), with non-temporal loads if `streaming`; for bandwidth measurements.
+int picolm_read_probe(const void* src, size_t bytes, void* sink, int blocks, int streaming, hipStream_t stream);
+size_t picolm_read_probe_bytes(size_t bytes, int blocks);
 
 // runs blocks*4 waves of `iters` x 8 MFMAs (32x32x16 bf16) on registers, on small integers or
 // (random_operands != 0) on pseudo-random values of the size of real data, which the GPU's power

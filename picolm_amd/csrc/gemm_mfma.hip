@@ -84,17 +84,21 @@ __device__ __forceinline__ void skinny_finish(f32x4 (&acc)[NT][MT], float* red, 
             C[(int64_t)m * ldc + n] = from_f32<TC>(s0);
         }
     }
-    if (EPI == 1 && MT == 1 && NT == 1 && link.next_w) {
-        // this workgroup's 16 columns of every row: lanes l, l+16, l+32, l+48 of the first four
-        // waves hold them (r = wave); rows past M and columns past N added nothing
+    if (EPI == 1 && MT == 1 && NT * 4 <= WAVES && link.next_w) {
+        // Every thread of the first 4 NT waves has finished one value (the loop above ran once for
+        // it).  Tile t's 16 columns of every row: lanes l, l+16, l+32, l+48 of waves 4t .. 4t+3 hold
+        // them (r = wave % 4); rows past M and columns past N added nothing.  One share of the sums
+        // per tile of 16 columns: share blockIdx.x * NT + t (the workgroup has 16 NT rows).
         next_sq += __shfl_xor(next_sq, 16, WAVE);
         next_sq += __shfl_xor(next_sq, 32, WAVE);
         __syncthreads();                    // link_scratch may still be read as the consumer's
-        if (wave < 4 && lane < 16) link_scratch[wave * 16 + lane] = next_sq;
+        if (wave < 4 * NT && lane < 16) link_scratch[wave * 16 + lane] = next_sq;
         __syncthreads();
-        if (threadIdx.x < 16)
-            link.next_ssq[(size_t)blockIdx.x * link.rows + threadIdx.x] =
-                link_scratch[threadIdx.x] + link_scratch[16 + threadIdx.x] + link_scratch[32 + threadIdx.x] + link_scratch[48 + threadIdx.x];
+        if (threadIdx.x < 16 * NT) {
+            const int t = threadIdx.x / 16, m = threadIdx.x % 16;
+            const float* part = link_scratch + t * 64 + m;
+            link.next_ssq[((size_t)blockIdx.x * NT + t) * link.rows + m] = part[0] + part[16] + part[32] + part[48];
+        }
     }
 }
 
@@ -310,7 +314,7 @@ __global__ __launch_bounds__(512) void gemm_skinny_staged_kernel(const bf16_t* _
 
 // Whether the staged kernel takes a product, and with how many stages a wave.
 static int skinny_staged_stages(int M, int K, int rows_per_wg) {
-    if (M > 16 || K % SKS_KSTEP || rows_per_wg % 8 || rows_per_wg > 32) return 0;
+    if (M > 16 || K % SKS_KSTEP || rows_per_wg % 8 || rows_per_wg > 48) return 0;
     const int per_step = (rows_per_wg + 7) / 8 + (M + 7) / 8;
     int stages = (SKS_LDS_BYTES - 4096) / 8 / (per_step * 1024);      // (the kernel has 2 KB of its own)
     if (stages > 8) stages = 8;
@@ -322,8 +326,8 @@ static int launch_skinny_staged(const void* A, const void* W, void* C, int c_dt,
                                 int64_t ldw, int64_t ldc, int epi, hipStream_t stream, NormLink link, int rows_per_wg) {
     const int stages = skinny_staged_stages(M, K, rows_per_wg);
     PICOLM_REQUIRE(stages > 0 && rows_per_wg <= 16 * NT, "gemm_skinny: the staged kernel does not take M=%d K=%d with %d rows a workgroup", M, K, rows_per_wg);
-    PICOLM_REQUIRE(!link.next_w || (NT == 1 && epi == 1 && rows_per_wg == 16 && link.next_parts >= ceil_div(N, 16)),
-                   "gemm_skinny: only the 16x16 tile with the accumulating epilogue prepares a norm");
+    PICOLM_REQUIRE(!link.next_w || (NT <= 2 && epi == 1 && rows_per_wg == 16 * NT && link.next_parts >= ceil_div(N, 16)),
+                   "gemm_skinny: whole tiles of 16 weight rows with the accumulating epilogue prepare a norm");
     PICOLM_REQUIRE((!link.ssq && !link.next_w) || link.rows == 16, "gemm_skinny: a split norm goes with up to 16 rows here");
     PICOLM_REQUIRE(64 * ldw * 2 < (1ll << 31) && 16 * lda * 2 < (1ll << 31), "gemm_skinny: row strides %lld / %lld overflow 32-bit offsets",
                    (long long)lda, (long long)ldw);
@@ -531,7 +535,8 @@ static int skinny_rows_per_wg(int N, int M) {
         // as cheap with fewer, larger workgroups: every workgroup reads all the activations, so with
         // many rows the fewer win (12288 x 4096: 22 against 26 us at 16 rows), with one row the more
         // (20 against 22 us)
-        if (cost < best_cost || (cost == best_cost && M > 8)) {
+        // (and one round of up to 32 rows a workgroup is what the staged kernel takes)
+        if (cost < best_cost || (cost == best_cost && (M > 8 || (rows <= 32 && ceil_div(N, rows) <= cus)))) {
             best = rows;
             best_cost = cost;
         }
@@ -541,13 +546,18 @@ static int skinny_rows_per_wg(int N, int M) {
 template <int MT>
 static int launch_skinny_sized(const void* A, const void* W, void* C, int c_dt, int M, int N, int K, int64_t lda,
                                int64_t ldw, int64_t ldc, int epi, hipStream_t stream, NormLink link, bool staged = true) {
-    const int rows = link.next_w ? 16 : skinny_rows_per_wg(N, M);
+    // a product that prepares a norm leaves one share of its sums per 16 weight rows, so its
+    // workgroups take whole tiles: 16 rows, or 32 where that makes one round of the CUs out of two
+    const int cus = n_compute_units();
+    const bool two_tiles = N % 32 == 0 && ceil_div(N, 16) > cus && N / 32 <= cus && skinny_staged_stages(M, K, 32) > 0;
+    const int rows = link.next_w ? (staged && MT == 1 && two_tiles ? 32 : 16) : skinny_rows_per_wg(N, M);
     // The staged kernel where every CU has at most one workgroup: its stages fill the LDS, so that a
     // second round of workgroups would wait for the first to leave (12,288 rows as 512 workgroups: 22
     // us against 19; a vocabulary of 128,256 rows: 183 against 165).
     if (staged && MT == 1 && skinny_staged_stages(M, K, rows) > 0 && ceil_div(N, rows) <= n_compute_units()) {
         if (rows <= 16) return launch_skinny_staged<1>(A, W, C, c_dt, M, N, K, lda, ldw, ldc, epi, stream, link, rows);
-        return launch_skinny_staged<2>(A, W, C, c_dt, M, N, K, lda, ldw, ldc, epi, stream, link, rows);
+        if (rows <= 32) return launch_skinny_staged<2>(A, W, C, c_dt, M, N, K, lda, ldw, ldc, epi, stream, link, rows);
+        return launch_skinny_staged<3>(A, W, C, c_dt, M, N, K, lda, ldw, ldc, epi, stream, link, rows);
     }
     if (rows <= 16) return launch_skinny<MT, 1, 8>(A, W, C, c_dt, M, N, K, lda, ldw, ldc, epi, stream, link, rows);
     if (rows <= 32) return launch_skinny<MT, 2, 8>(A, W, C, c_dt, M, N, K, lda, ldw, ldc, epi, stream, link, rows);

@@ -32,6 +32,7 @@ def lib():
         l.picolm_last_error.restype = ctypes.c_char_p
         for name in dir_entry_points():
             getattr(l, name).restype = c_int
+        l.picolm_read_probe_bytes.restype = ctypes.c_size_t
         if l.picolm_abi_version() != 1:
             raise KernelError("libpicolm_hip.so has another ABI version; rebuild it")
         _lib = l
@@ -600,12 +601,15 @@ def sample(logits: torch.Tensor, out: torch.Tensor, temperature: float, top_k: i
                                c_int64(scratch.numel() if scratch is not None else 0), _stream()))
 
 
-def read_probe(src: torch.Tensor, sink: torch.Tensor, blocks: int = 4096, unroll4: bool = True) -> None:
-    """Sweep `src` once with a plain read kernel (for bandwidth measurements)."""
+def read_probe(src: torch.Tensor, sink: torch.Tensor, blocks: int = 2048, streaming: bool = True) -> int:
+    """Queue one sweep over `src` (each workgroup a contiguous share; non-temporal loads if
+    `streaming`, as the kernels load what a launch reads once); returns the bytes it reads."""
     _dev("read_probe.src", src)
     _dev("read_probe.sink", sink, torch.int32)
     nbytes = src.numel() * src.element_size()
-    _check(lib().picolm_read_probe(_ptr(src), ctypes.c_size_t(nbytes - nbytes % 16), _ptr(sink), blocks, int(unroll4), _stream()))
+    nbytes -= nbytes % 16
+    _check(lib().picolm_read_probe(_ptr(src), ctypes.c_size_t(nbytes), _ptr(sink), blocks, int(streaming), _stream()))
+    return int(lib().picolm_read_probe_bytes(ctypes.c_size_t(nbytes), blocks))
 
 
 def mfma_probe(sink: torch.Tensor, blocks: int, iters: int, random_operands: bool = False) -> float:

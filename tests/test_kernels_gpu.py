@@ -176,12 +176,13 @@ def test_gemm_of_a_short_prompt_is_cut_along_k():
 
 
 @pytest.mark.parametrize("M", [1, 8, 16])
-@pytest.mark.parametrize("D", [48, 256, 4096])
+@pytest.mark.parametrize("D", [48, 256, 4096, 8192])
 def test_gemm_with_a_norm_split_between_two_products(M, D):
     """The product that finishes rows of the residual stream prepares the RMSNorm that follows
     (bf16(x * w) and partial sums of x^2), the next product applies 1 / sqrt(mean(x^2) + eps) to
     its sums: together they must give norm-then-product.  Rows of very different size, so that a
-    factor taken from the wrong row shows; every kernel that can be the consumer."""
+    factor taken from the wrong row shows; every kernel that can be the consumer.  (A width of
+    8,192 makes two rounds of 16-row workgroups: the producer then takes 32 rows a workgroup.)"""
     g = torch.Generator().manual_seed(M * 31 + D)
     eps, K1 = 1e-5, 192
     x0 = torch.randn(M, D, generator=g) * (10.0 ** torch.arange(M).remainder(5).sub(2).float())[:, None]
