@@ -99,6 +99,24 @@ def test_gemm_skinny(M, N, Kd):
         run_gemm(K().gemm_skinny, M, N, Kd, epi, torch.bfloat16, torch.bfloat16, cdt)
 
 
+@pytest.mark.parametrize("M", [1, 5, 8, 9, 16])
+@pytest.mark.parametrize("N,Kd", [(100, 128), (16, 64), (4096, 4096), (6144, 1024), (8192, 576), (10240, 512), (4090, 14336)])
+def test_gemm_skinny_through_stages_of_a_waves_own(M, N, Kd):
+    """One round of workgroups of 16, 24, 32 or 40 weight rows with K in multiples of 64: weights
+    and activations go through LDS stages of each wave (three to eight of them, by the rows of both).
+    Few slices of K (some waves have none), many (a wave goes round its stages several times), a
+    last workgroup with fewer rows than the others; and the older kernel must give the same sums."""
+    for epi, cdt in ((0, torch.float32), (0, torch.bfloat16), (1, torch.float32), (2, torch.bfloat16)):
+        run_gemm(K().gemm_skinny, M, N, Kd, epi, torch.bfloat16, torch.bfloat16, cdt)
+    g = torch.Generator().manual_seed(N + M)
+    a = torch.randn(M, Kd, generator=g).to(torch.bfloat16).to(DEV)
+    w = (torch.randn(N, Kd, generator=g) * 0.1).to(torch.bfloat16).to(DEV)
+    c1, c2 = torch.zeros(M, N, device=DEV), torch.zeros(M, N, device=DEV)
+    K().gemm_skinny(a, w, c1, 0)
+    K().gemm_skinny(a, w, c2, 0, variant=9)          # never staged
+    assert (c1 - c2).abs().max().item() <= 1e-5 * c2.abs().max().item()
+
+
 @pytest.mark.parametrize("variant", [1, 2, 3, 4, 5, 6])
 def test_gemm_skinny_variants(variant):
     M = {1: 16, 2: 13, 3: 32, 4: 21, 5: 64, 6: 50}[variant]
