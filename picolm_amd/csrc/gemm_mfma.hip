@@ -22,6 +22,46 @@
 // =============================================================================================
 #define SK_KSTEP 128      // K elements one wave consumes per step: 4 MFMAs of 32
 
+// The values a thread of a skinny product's workgroup finishes, one per pass of the epilogue's
+// loop: value v = ((t*MT + u)*4 + r)*64 + l is row m = 16 u + l % 16, column n_base + 16 t +
+// 4 (l / 16) + r (the gated epilogue takes r and r + 1 together).
+template <int MT, int NT, int WAVES, int EPI>
+struct SkinnyValues {
+    static constexpr int PER_WAVE = NT * MT * 4 * 64;
+    static constexpr int STEP = (EPI == 2) ? 2 : 1;
+    static constexpr int PASSES = (PER_WAVE / STEP + WAVES * 64 - 1) / (WAVES * 64);
+    // where pass p's value lies: false if this thread has none there
+    __device__ static bool place(int pass, int M, int N, int n_base, int rows_per_wg, int& idx, int& m, int& n) {
+        const int v = threadIdx.x + pass * (WAVES * 64);
+        if (v >= PER_WAVE / STEP) return false;
+        const int l = v % 64;
+        const int r = EPI == 2 ? 2 * ((v / 64) % 2) : (v / 64) % 4;
+        const int tu = EPI == 2 ? v / 128 : v / 256;
+        const int u = tu % MT, t = tu / MT;
+        idx = ((t * MT + u) * 4 + r) * 64 + l;
+        n = n_base + t * 16 + 4 * (l / 16) + r;
+        m = u * 16 + l % 16;
+        return m < M && n < N && t * 16 + 4 * (l / 16) + r < rows_per_wg;
+    }
+    float before[PASSES], next_w[PASSES];      // (accumulating epilogue) what the sums are added to, the next norm's weight
+};
+// Asked for before the main loop, so that the epilogue does not wait a trip to memory for them.
+template <int MT, int NT, int WAVES, int EPI, typename TC>
+__device__ __forceinline__ SkinnyValues<MT, NT, WAVES, EPI> skinny_prefetch(const TC* __restrict__ C, int M, int N, int64_t ldc,
+                                                                            const NormLink& link, int n_base, int rows_per_wg) {
+    SkinnyValues<MT, NT, WAVES, EPI> pre;
+#pragma unroll
+    for (int pass = 0; pass < pre.PASSES; ++pass) {
+        pre.before[pass] = pre.next_w[pass] = 0.f;
+        int idx, m, n;
+        if (EPI == 1 && pre.place(pass, M, N, n_base, rows_per_wg, idx, m, n)) {
+            pre.before[pass] = to_f32<TC>(C[(int64_t)m * ldc + n]);
+            if (link.next_w) pre.next_w[pass] = link.next_w[n];
+        }
+    }
+    return pre;
+}
+
 // What the waves of a skinny product's workgroup have summed over their shares of K comes together
 // here: through LDS (red: a wave's NT * MT * 256 floats start wave_stride floats apart), in a fixed
 // order, then the epilogue.  Called by all threads.
@@ -29,7 +69,7 @@ template <int MT, int NT, int WAVES, int EPI, typename TC>
 __device__ __forceinline__ void skinny_finish(f32x4 (&acc)[NT][MT], float* red, int wave_stride, TC* __restrict__ C, int M, int N,
                                               int64_t ldc, const NormLink& link, float link_mine,
                                               float (&link_scratch)[WAVES * 64], float (&link_scale)[16], int n_base,
-                                              int rows_per_wg) {
+                                              int rows_per_wg, const SkinnyValues<MT, NT, WAVES, EPI>& pre) {
     const int wave = threadIdx.x / 64, lane = threadIdx.x % 64;
     // reduce over the waves
 #pragma unroll
@@ -40,32 +80,17 @@ __device__ __forceinline__ void skinny_finish(f32x4 (&acc)[NT][MT], float* red, 
             for (int r = 0; r < 4; ++r) red[(size_t)wave * wave_stride + ((t * MT + u) * 4 + r) * 64 + lane] = acc[t][u][r];
     __syncthreads();
     row_scale_finish<WAVES * 64>(link, link_mine, 16, link_scratch, link_scale);
-    constexpr int PER_WAVE = NT * MT * 4 * 64;
-    constexpr int STEP = (EPI == 2) ? 2 : 1;
-    float next_sq = 0.f;                // producer side: x^2 of the value this thread finishes (MT = NT = 1 only)
-    // value v = ((t*MT + u)*4 + r)*64 + l ; the gated epilogue takes r and r+1 together
-    for (int v = threadIdx.x; v < PER_WAVE / STEP; v += WAVES * 64) {
-        int l, r, tu;
-        if (EPI == 2) {
-            l = v % 64;
-            r = 2 * ((v / 64) % 2);
-            tu = v / 128;
-        } else {
-            l = v % 64;
-            r = (v / 64) % 4;
-            tu = v / 256;
-        }
-        const int u = tu % MT, t = tu / MT;
-        const int idx = ((t * MT + u) * 4 + r) * 64 + l;
+    float next_sq = 0.f;                // producer side: x^2 of the value this thread finishes (one pass only)
+#pragma unroll
+    for (int pass = 0; pass < pre.PASSES; ++pass) {
+        int idx, m, n;
+        if (!pre.place(pass, M, N, n_base, rows_per_wg, idx, m, n)) continue;
         float s0 = 0.f, s1 = 0.f;
 #pragma unroll
         for (int w = 0; w < WAVES; ++w) {
             s0 += red[(size_t)w * wave_stride + idx];
             if (EPI == 2) s1 += red[(size_t)w * wave_stride + idx + 64];
         }
-        const int n = n_base + t * 16 + 4 * (l / 16) + r;
-        const int m = u * 16 + l % 16;
-        if (m >= M || n >= N || t * 16 + 4 * (l / 16) + r >= rows_per_wg) continue;
         if (link.ssq) {
             s0 *= link_scale[m];
             s1 *= link_scale[m];
@@ -73,11 +98,10 @@ __device__ __forceinline__ void skinny_finish(f32x4 (&acc)[NT][MT], float* red, 
         if (EPI == 2) {
             C[(int64_t)m * ldc + n / 2] = from_f32<TC>(silu_mul(s0, s1));
         } else if (EPI == 1) {
-            TC* p = C + (int64_t)m * ldc + n;
-            const float x = to_f32<TC>(*p) + s0;
-            *p = from_f32<TC>(x);
+            const float x = pre.before[pass] + s0;
+            C[(int64_t)m * ldc + n] = from_f32<TC>(x);
             if (link.next_w) {
-                link.next_h[(int64_t)m * ldc + n] = f32_to_bf16_bits(x * link.next_w[n]);
+                link.next_h[(int64_t)m * ldc + n] = f32_to_bf16_bits(x * pre.next_w[pass]);
                 next_sq = x * x;
             }
         } else {
@@ -117,6 +141,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const bf16_t* _
     // its last tile of 16, so that the host can size the launch to the CUs.  Lanes of rows it does
     // not have read its last row again, which costs no traffic, and their sums are not stored.
     const int n_base = blockIdx.x * rows_per_wg;
+    const auto pre = skinny_prefetch<MT, NT, WAVES, EPI, TC>(C, M, N, ldc, link, n_base, rows_per_wg);
 
     const bf16_t* wrow[NT];
 #pragma unroll
@@ -188,7 +213,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const bf16_t* _
         multiply(0);
     }
     skinny_finish<MT, NT, WAVES, EPI, TC>(acc, red, NT * MT * 4 * 64, C, M, N, ldc, link, link_mine, link_scratch, link_scale, n_base,
-                                          rows_per_wg);
+                                          rows_per_wg, pre);
 }
 
 // ---- skinny, weights and activations staged through LDS -----------------------------------------
@@ -229,6 +254,7 @@ __global__ __launch_bounds__(512) void gemm_skinny_staged_kernel(const bf16_t* _
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / 64), lane = threadIdx.x % 64;
     const int r16 = lane % 16, q = lane / 16;
     const int n_base = blockIdx.x * rows_per_wg;
+    const auto pre = skinny_prefetch<1, NT, 8, EPI, TC>(C, M, N, ldc, link, n_base, rows_per_wg);
     // kilobytes (loads of a wave) that a step brings in: eight weight rows each, eight activation rows each
     const int w_loads = (rows_per_wg + 7) / 8, a_loads = (M + 7) / 8;
     const int stage_bytes = (w_loads + a_loads) * 1024;
@@ -309,7 +335,7 @@ __global__ __launch_bounds__(512) void gemm_skinny_staged_kernel(const bf16_t* _
     }
     // each wave leaves its sums in its own stages, which only it has read
     skinny_finish<1, NT, 8, EPI, TC>(acc, (float*)staged_lds, n_stages * stage_bytes / 4, C, M, N, ldc, link, link_mine, link_scratch,
-                                     link_scale, n_base, rows_per_wg);
+                                     link_scale, n_base, rows_per_wg, pre);
 }
 
 // Whether the staged kernel takes a product, and with how many stages a wave.
