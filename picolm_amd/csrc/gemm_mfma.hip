@@ -421,130 +421,7 @@ static int launch_skinny(const void* A, const void* W, void* C, int c_dt, int M,
     return 0;
 }
 
-// ---- skinny, with the activations resident ---------------------------------------------------
-// For M <= 16 and K <= STEPS * 1024: a wave keeps the activation chunks of its K slices in
-// registers for the whole launch and a workgroup walks over many tiles of 16 weight rows, with
-// the next tile's weights in flight while the current one is multiplied and reduced.  The
-// activations are read once per workgroup instead of once per tile, and the gap between tiles
-// (the reduction through LDS, the epilogue) no longer leaves the memory pipe empty.
-template <int STEPS, int EPI, typename TC>
-__global__ __launch_bounds__(512) void gemm_skinny_resident_kernel(const bf16_t* __restrict__ A,
-                                                                   const bf16_t* __restrict__ W,
-                                                                   TC* __restrict__ C, int M, int N, int K,
-                                                                   int64_t lda, int64_t ldw, int64_t ldc, NormLink link) {
-    constexpr int WAVES = 8;
-    __shared__ float red[2][WAVES][4][64];
-    __shared__ float link_scratch[WAVES * 64], link_scale[16];
-    const float link_mine = row_scale_begin<WAVES * 64>(link, M, 0, 16);
-    const int wave = threadIdx.x / 64, lane = threadIdx.x % 64;
-    const int r16 = lane % 16, q = lane / 16;
-    const int n_full = K / SK_KSTEP;            // K is a whole number of steps (the host sees to that)
-    const int n_tiles = (N + 15) / 16;
-
-    bf16x8 av[STEPS][4];
-    int koff[STEPS];                            // element offset of this lane's first chunk of step i
-#pragma unroll
-    for (int i = 0; i < STEPS; ++i) {
-        const int s = wave + i * WAVES;
-        const bool valid = s < n_full && r16 < M;
-        koff[i] = min(s, n_full - 1) * SK_KSTEP + q * 8;      // a step past the end reads the last one; its activations are zero
-#pragma unroll
-        for (int j = 0; j < 4; ++j)
-            av[i][j] = valid ? load_chunk(A + (int64_t)r16 * lda + koff[i] + 32 * j) : zero_chunk();
-    }
-    auto fetch = [&](bf16x8 (&wv)[STEPS][4], int tile) {
-        const bf16_t* wrow = W + (int64_t)min(tile * 16 + r16, N - 1) * ldw;
-#pragma unroll
-        for (int i = 0; i < STEPS; ++i)
-#pragma unroll
-            for (int j = 0; j < 4; ++j) wv[i][j] = load_chunk(wrow + koff[i] + 32 * j);
-    };
-    auto finish = [&](const bf16x8 (&wv)[STEPS][4], int tile, int buf) {
-        f32x4 acc = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-        for (int i = 0; i < STEPS; ++i)
-#pragma unroll
-            for (int j = 0; j < 4; ++j) acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wv[i][j], av[i][j], acc, 0, 0, 0);
-#pragma unroll
-        for (int r = 0; r < 4; ++r) red[buf][wave][r][lane] = acc[r];
-        __syncthreads();
-        // value (r, l): n = 16*tile + 4*(l/16) + r, m = l%16; the gated epilogue takes r and r+1 together
-        constexpr int STEP = (EPI == 2) ? 2 : 1;
-        const int v = threadIdx.x;
-        if (v < 256 / STEP) {
-            const int l = v % 64, r = EPI == 2 ? 2 * (v / 64) : v / 64;
-            float s0 = 0.f, s1 = 0.f;
-#pragma unroll
-            for (int w = 0; w < WAVES; ++w) {
-                s0 += red[buf][w][r][l];
-                if (EPI == 2) s1 += red[buf][w][r + 1][l];
-            }
-            const int n = tile * 16 + 4 * (l / 16) + r, m = l % 16;
-            if (m < M && n < N) {
-                if (link.ssq) {
-                    s0 *= link_scale[m];
-                    s1 *= link_scale[m];
-                }
-                if (EPI == 2) {
-                    C[(int64_t)m * ldc + n / 2] = from_f32<TC>(silu_mul(s0, s1));
-                } else if (EPI == 1) {
-                    TC* p = C + (int64_t)m * ldc + n;
-                    *p = from_f32<TC>(to_f32<TC>(*p) + s0);
-                } else {
-                    C[(int64_t)m * ldc + n] = from_f32<TC>(s0);
-                }
-            }
-        }
-    };
-    // two register sets of weights and two LDS buffers alternate, so that one barrier a tile is
-    // enough; tiles past the end read the last tile again and are not finished
-    bf16x8 w0[STEPS][4], w1[STEPS][4];
-    const int stride = gridDim.x;
-    int tile = blockIdx.x;
-    fetch(w0, min(tile, n_tiles - 1));
-    row_scale_finish<WAVES * 64>(link, link_mine, 16, link_scratch, link_scale);
-    while (tile < n_tiles) {
-        fetch(w1, min(tile + stride, n_tiles - 1));
-        __builtin_amdgcn_sched_barrier(0);      // the next tile is asked for before this one is waited for
-        finish(w0, tile, 0);
-        tile += stride;
-        if (tile >= n_tiles) break;
-        fetch(w0, min(tile + stride, n_tiles - 1));
-        __builtin_amdgcn_sched_barrier(0);
-        finish(w1, tile, 1);
-        tile += stride;
-    }
-}
-
-template <int STEPS>
-static int launch_skinny_resident(const void* A, const void* W, void* C, int c_dt, int M, int N, int K, int64_t lda,
-                                  int64_t ldw, int64_t ldc, int epi, hipStream_t stream, NormLink link = NormLink{}) {
-    PICOLM_REQUIRE(!link.next_w, "gemm_skinny: the resident variant prepares no norm");
-    PICOLM_REQUIRE(!link.ssq || link.rows == 16, "gemm_skinny: a split norm goes with up to 16 rows here");
-    PICOLM_REQUIRE(M <= 16 && K % SK_KSTEP == 0 && K <= STEPS * 8 * SK_KSTEP,
-                   "gemm_skinny: the resident variant takes M <= 16 and K a multiple of %d up to %d, got M=%d K=%d",
-                   SK_KSTEP, STEPS * 8 * SK_KSTEP, M, K);
-    // one workgroup a CU; the same number of tiles for every workgroup where that is possible
-    const int n_tiles = ceil_div(N, 16);
-    const int rounds = ceil_div(n_tiles, 256);
-    dim3 grid(ceil_div(n_tiles, rounds)), block(512);
-    const bf16_t* a = (const bf16_t*)A;
-    const bf16_t* w = (const bf16_t*)W;
-#define SR_LAUNCH(EPI, TC) \
-    gemm_skinny_resident_kernel<STEPS, EPI, TC><<<grid, block, 0, stream>>>(a, w, (TC*)C, M, N, K, lda, ldw, ldc, link);
-    if (epi == 0 && c_dt == PICOLM_F32) SR_LAUNCH(0, float)
-    else if (epi == 0 && c_dt == PICOLM_BF16) SR_LAUNCH(0, bf16_t)
-    else if (epi == 1 && c_dt == PICOLM_F32) SR_LAUNCH(1, float)
-    else if (epi == 2 && c_dt == PICOLM_BF16) SR_LAUNCH(2, bf16_t)
-    else if (epi == 2 && c_dt == PICOLM_F32) SR_LAUNCH(2, float)
-    else PICOLM_REQUIRE(false, "gemm_skinny: unsupported epilogue %d with output dtype %d", epi, c_dt);
-#undef SR_LAUNCH
-    PICOLM_LAUNCH_CHECK("gemm_skinny");
-    return 0;
-}
-
-// variant: 0 picks by shape; 1..6 name (MT,NT,WAVES) combinations for tuning and tests, 7 is
-// the variant with resident activations
+// variant: 0 picks by shape; 1..6 name (MT,NT,WAVES) combinations for tuning and tests, 9 is 1 without the staged kernel
 // Weight rows a workgroup of the 16-row kernel takes: 16, or, where the workgroups of that size
 // would leave a last round of the CUs mostly empty, the multiple of 8 up to 64 with which the
 // launch takes the fewest rows per CU (6144 rows on 256 CUs: 24 rows each instead of 16 in one
@@ -597,13 +474,7 @@ extern "C" int picolm_gemm_skinny(const void* A, const void* W, void* C, int c_d
     if (check_mfma_operands("gemm_skinny", A, W, M, N, K, lda, ldw, ldc, epilogue, c_dt)) return -1;
     PICOLM_REQUIRE(M <= 64, "gemm_skinny: M=%d exceeds 64", M);
     if (M == 0) return 0;
-    if (variant == 0) {
-        // many tiles a CU and several rows: the resident variant reads the activations once and
-        // keeps the memory pipe full between tiles (a few rows cost little to re-read, and then
-        // several workgroups a CU hide more latency); few tiles: one workgroup a tile
-        if (M > 4 && M <= 16 && N >= 16384 && K % SK_KSTEP == 0 && K <= 4 * 8 * SK_KSTEP) variant = 7;
-        else variant = M <= 16 ? 1 : (M <= 32 ? 3 : (N >= 8192 ? 6 : 5));
-    }
+    if (variant == 0) variant = M <= 16 ? 1 : (M <= 32 ? 3 : (N >= 8192 ? 6 : 5));
     switch (variant) {
         case 1: return launch_skinny_sized<1>(A, W, C, c_dt, M, N, K, lda, ldw, ldc, epilogue, stream, NormLink{});
         case 9: return launch_skinny_sized<1>(A, W, C, c_dt, M, N, K, lda, ldw, ldc, epilogue, stream, NormLink{}, false);   // never staged
@@ -613,7 +484,6 @@ extern "C" int picolm_gemm_skinny(const void* A, const void* W, void* C, int c_d
         case 4: return launch_skinny<2, 2, 8>(A, W, C, c_dt, M, N, K, lda, ldw, ldc, epilogue, stream);
         case 5: return launch_skinny<4, 1, 8>(A, W, C, c_dt, M, N, K, lda, ldw, ldc, epilogue, stream);
         case 6: return launch_skinny<4, 2, 4>(A, W, C, c_dt, M, N, K, lda, ldw, ldc, epilogue, stream);
-        case 7: return launch_skinny_resident<4>(A, W, C, c_dt, M, N, K, lda, ldw, ldc, epilogue, stream);
     }
     PICOLM_REQUIRE(false, "gemm_skinny: unknown variant %d", variant);
 }
@@ -621,11 +491,6 @@ extern "C" int picolm_gemm_skinny(const void* A, const void* W, void* C, int c_d
 // The skinny side of picolm_gemm_linked (up to 16 rows).
 int picolm_gemm_skinny_linked_(const void* A, const void* W, void* C, int c_dt, int M, int N, int K, int64_t lda,
                                int64_t ldw, int64_t ldc, int epilogue, int variant, hipStream_t stream, NormLink link) {
-    const float* next_w = link.next_w;
-    if (variant == 0) variant = (M > 4 && N >= 16384 && K % SK_KSTEP == 0 && K <= 4 * 8 * SK_KSTEP && !next_w) ? 7 : 1;
-    switch (variant) {
-        case 1: return launch_skinny_sized<1>(A, W, C, c_dt, M, N, K, lda, ldw, ldc, epilogue, stream, link);
-        case 7: return launch_skinny_resident<4>(A, W, C, c_dt, M, N, K, lda, ldw, ldc, epilogue, stream, link);
-    }
+    if (variant == 0 || variant == 1) return launch_skinny_sized<1>(A, W, C, c_dt, M, N, K, lda, ldw, ldc, epilogue, stream, link);
     PICOLM_REQUIRE(false, "gemm_linked: skinny variant %d cannot take part in a split norm", variant);
 }

@@ -506,7 +506,7 @@ extern "C" int picolm_gemm_tiled_splitk(const void* A, const void* W, void* C, i
 }
 
 // The products of a decode step with a norm split between them (see NormLink).  Up to 16 rows:
-// `variant` as in picolm_gemm_skinny (0, 1, 7) or, with tiled != 0, tile variant 12 or 13; rows = 16.
+// `variant` as in picolm_gemm_skinny (0 or 1) or, with tiled != 0, tile variant 12 or 13; rows = 16.
 // More than 64 rows (a prefill step): tiled, rows = a multiple of 64 of at least M, the tile
 // variant by shape, cut along K if ws is given and the shape has few tiles; either role, the
 // shares of the sums as picolm_gemm_tiled_norm_parts says for the same ws_floats.

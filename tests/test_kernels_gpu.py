@@ -131,20 +131,6 @@ def test_gemm_tiled(M, N, Kd):
         run_gemm(K().gemm_tiled, M, N, Kd, epi, torch.bfloat16, torch.bfloat16, cdt)
 
 
-@pytest.mark.parametrize("M", [1, 8, 16])
-def test_gemm_skinny_resident_activations(M):
-    """The variant that keeps the activations in registers and walks over many tiles: fewer
-    tiles than workgroups, a ragged last tile, several tiles a workgroup (more than 256 tiles),
-    K below and at its limit."""
-    for N, Kd in ((530, 1024), (16 * 300 - 6, 128), (16 * 700 + 2, 4096), (48, 3968)):
-        for epi, cdt in ((0, torch.float32), (2, torch.bfloat16), (1, torch.float32), (0, torch.bfloat16)):
-            run_gemm(K().gemm_skinny, M, N, Kd, epi, torch.bfloat16, torch.bfloat16, cdt, variant=7)
-    with pytest.raises(Exception, match="resident"):
-        run_gemm(K().gemm_skinny, M, 64, 4096 + 128, 0, torch.bfloat16, torch.bfloat16, torch.float32, variant=7)
-    with pytest.raises(Exception, match="resident"):
-        run_gemm(K().gemm_skinny, M, 64, 1032, 0, torch.bfloat16, torch.bfloat16, torch.float32, variant=7)
-
-
 @pytest.mark.parametrize("variant,splits", [(12, 2), (12, 8), (13, 4), (11, 4), (9, 3)])
 def test_gemm_tiled_split_along_k(variant, splits):
     """K cut into parts whose partial sums a second kernel adds in order: every epilogue, ragged

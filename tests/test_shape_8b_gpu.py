@@ -2,9 +2,9 @@
 (hidden 4096, 32 heads over 8 KV heads of 128, intermediate 14336, the full vocabulary of 128,256,
 llama3 frequency scaling) with seeded random weights N(0, 0.02) made on the GPU.
 
-The kernels that only such sizes reach (256x256 prefill tiles, the skinny product that keeps its
-activations resident for a head of 128,256 rows, tiles of 128 weight rows for 5..16 rows, K of
-14,336) are checked here in the model: the bfloat16 engine against the 32-bit engine under every
+The kernels that only such sizes reach (256x256 prefill tiles, a head of 128,256 rows, tiles of
+128 weight rows for up to 16 activation rows, skinny products staged through LDS with K of 14,336)
+are checked here in the model: the bfloat16 engine against the 32-bit engine under every
 cutting of the work, and the 32-bit engine against the plain implementation on a short request.
 picolm checks its fast path against its plain one in the same way (picolm/picolm.c:1437-1463,
 warning above 1e-2)."""
