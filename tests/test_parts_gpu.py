@@ -523,6 +523,109 @@ def test_toy_position_encoding_that_is_no_rotation(dtype):
         assert np.abs(res.double().cpu().numpy() - want).max() <= tol(dtype, want)
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_toy_norm_that_is_no_rmsnorm(dtype, tmp_path):
+    """A norm of another kind, defined here: it subtracts the row's mean, divides by the standard
+    deviation and has a weight and a bias.  The products around a norm share an RMSNorm between
+    them in decode steps; this one says nothing of the kind (`rms_parameters` is None), so its
+    own `forward` must run wherever it stands: before the mixer, before the feed-forward, and as
+    the last norm of one block with an RMSNorm following in the next.  Prompts whole, then token by
+    token (where the sharing would happen), against the plain functions."""
+    from picolm_amd.config import LlamaConfig, register_architecture, unregister_architecture
+    from picolm_amd.engine import DecoderModel, Session, load_model
+    from picolm_amd.parts import Attention, LMHead, Norm, PreNormBlock, RMSNorm, RotaryEmbedding, SwiGLU, TokenEmbedding
+    from picolm_amd.weights import TensorSpec, write_random_model
+
+    class CenteredNorm(Norm):
+        def __init__(self, name, size, eps):
+            self.name, self.size, self.eps = name, size, eps
+            self.weight = self.bias = None
+
+        def tensor_specs(self):
+            return [TensorSpec(self.name + ".weight", (self.size,), init="ones"), TensorSpec(self.name + ".bias", (self.size,))]
+
+        def load(self, fetch, runtime):
+            self.weight = fetch.get(self.name + ".weight").float()
+            self.bias = fetch.get(self.name + ".bias").float()
+
+        def forward(self, ctx, x, rows=None, n_rows=None, out_name="norm.out"):
+            if rows is not None:
+                x = x[rows[:n_rows].long()] if n_rows is not None else x[rows.long()]
+            xc = x - x.mean(dim=1, keepdim=True)
+            y = xc * torch.rsqrt((xc * xc).mean(dim=1, keepdim=True) + self.eps) * self.weight + self.bias
+            return y.to(ctx.dtype)
+
+    def build(cfg):
+        D = cfg.hidden_size
+        rotary = RotaryEmbedding(cfg.head_dim, cfg.rope_theta, cfg.rope_scaling, cfg.rope_style)
+        blocks = []
+        for l in range(2):
+            q = f"model.layers.{l}."
+            first = CenteredNorm(q + "input_norm", D, 1e-5) if l == 0 else RMSNorm(q + "input_layernorm.weight", D, 1e-5)
+            second = RMSNorm(q + "post_attention_layernorm.weight", D, 1e-5) if l == 0 else CenteredNorm(q + "post_norm", D, 1e-5)
+            blocks.append(PreNormBlock(first, Attention(q + "self_attn.", D, cfg.num_attention_heads, cfg.num_key_value_heads,
+                                                        cfg.head_dim, position=rotary),
+                                       second, SwiGLU(q + "mlp.", D, cfg.intermediate_size)))
+        emb = TokenEmbedding("model.embed_tokens.weight", cfg.vocab_size, D)
+        return DecoderModel(cfg, emb, blocks, CenteredNorm("model.final_norm", D, 1e-5),
+                            LMHead("lm_head.weight", cfg.vocab_size, D, emb, True))
+
+    name = "ToyCenteredNormLM"
+    register_architecture(name, LlamaConfig.from_dict, build)
+    try:
+        c = dict(architectures=[name], hidden_size=128, num_attention_heads=4, num_key_value_heads=2, head_dim=32,
+                 intermediate_size=192, num_hidden_layers=2, vocab_size=211, rms_norm_eps=1e-5, rope_theta=10000.0,
+                 max_position_embeddings=256, tie_word_embeddings=True, torch_dtype="bfloat16")
+        cfg = LlamaConfig.from_dict(c)
+        d = write_random_model(cfg, str(tmp_path / "centered"), seed=5, std=0.08)
+        model = load_model(d, dtype=dtype)
+        w = tiny.read_weights_f64(d)
+        pc = dict(c, rope_style=cfg.rope_style)
+
+        def centered(x, n):
+            xc = x - x.mean(axis=1, keepdims=True)
+            return xc / np.sqrt((xc * xc).mean(axis=1, keepdims=True) + 1e-5) * w[n + ".weight"] + w[n + ".bias"]
+
+        def plain(tokens):
+            pos = np.arange(len(tokens))
+            x = w["model.embed_tokens.weight"][np.asarray(tokens)]
+            x = x + P.attention_block(centered(x, "model.layers.0.input_norm"), w, "model.layers.0.self_attn.", pc, pos)
+            h = P.rmsnorm(x, w["model.layers.0.post_attention_layernorm.weight"], 1e-5)
+            x = x + P.swiglu(h, w["model.layers.0.mlp.gate_proj.weight"], w["model.layers.0.mlp.up_proj.weight"], w["model.layers.0.mlp.down_proj.weight"])
+            h = P.rmsnorm(x, w["model.layers.1.input_layernorm.weight"], 1e-5)
+            x = x + P.attention_block(h, w, "model.layers.1.self_attn.", pc, pos)
+            h = centered(x, "model.layers.1.post_norm")
+            x = x + P.swiglu(h, w["model.layers.1.mlp.gate_proj.weight"], w["model.layers.1.mlp.up_proj.weight"], w["model.layers.1.mlp.down_proj.weight"])
+            return centered(x, "model.final_norm") @ w["model.embed_tokens.weight"].T
+
+        rng = np.random.default_rng(9)
+        reqs = [tiny.random_tokens(rng, n, 211) for n in (70, 5, 33)]
+        truth = [plain(r) for r in reqs]
+        tol_ = lambda t: tiny.tolerance(dtype, t, tiny.spread(128, 0.08))
+        s = Session(model, max_tokens=512, n_slots=3)
+        assert s.engine is None                       # a part the library has no operations for: stepped from Python
+        slots = s.begin(3)
+        got = s.step(slots, reqs, [list(range(len(r))) for r in reqs]).double().cpu().numpy()
+        row = 0
+        for r, t in zip(reqs, truth):
+            assert np.abs(got[row:row + len(r)] - t).max() <= tol_(t)
+            row += len(r)
+        s.release(slots)
+        slots = s.begin(3)
+        cut = [50, 2, 20]
+        s.step(slots, [r[:c_] for r, c_ in zip(reqs, cut)])
+        pos = dict(zip(range(3), cut))
+        live = [0, 1, 2]
+        while live:
+            out = s.step([slots[i] for i in live], [[reqs[i][pos[i]]] for i in live]).double().cpu().numpy()
+            for k, i in enumerate(live):
+                assert np.abs(out[k] - truth[i][pos[i]]).max() <= tol_(truth[i]), (i, pos[i])
+                pos[i] += 1
+            live = [i for i in live if pos[i] < len(reqs[i])]
+    finally:
+        unregister_architecture(name)
+
+
 def test_toy_feed_forward_with_routing():
     """A feed-forward defined here: two gated experts and a router that sends every row to the
     expert with the larger logit (router logits in float).  It is built from the library's Linear
