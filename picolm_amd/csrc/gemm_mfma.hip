@@ -438,7 +438,8 @@ static int skinny_rows_per_wg(int N, int M) {
         // as cheap with fewer, larger workgroups: every workgroup reads all the activations, so with
         // many rows the fewer win (12288 x 4096: 22 against 26 us at 16 rows), with one row the more
         // (20 against 22 us)
-        // (and one round of up to 32 rows a workgroup is what the staged kernel takes)
+        // (and one round of up to 32 rows a workgroup suits the staged kernel; with 48 rows it has
+        // three stages and is no better than two rounds of the other: 12288 x 4096, 21 against 19 us)
         if (cost < best_cost || (cost == best_cost && (M > 8 || (rows <= 32 && ceil_div(N, rows) <= cus)))) {
             best = rows;
             best_cost = cost;
