@@ -29,7 +29,10 @@ __device__ __forceinline__ float swap_lanes(float v) {
 __device__ __forceinline__ void store_pair(float* p, float a, float b) { *(float2*)p = make_float2(a, b); }
 __device__ __forceinline__ void store_pair(bf16_t* p, bf16_t a, bf16_t b) { *(unsigned*)p = (unsigned)a | ((unsigned)b << 16); }
 
-template <int TN, int TM, int WN, int WM, int BK, int NS, int EPI, typename TC>
+// STREAM_SPREAD: the weights' loads that are spread between the MFMAs are non-temporal (a launch
+// with one row of tiles, where every weight is read once).  A choice at compile time: made at run
+// time at each of those loads it costs the long prompts' products 1.6 %.
+template <int TN, int TM, int WN, int WM, int BK, int NS, int EPI, typename TC, bool STREAM_SPREAD = false>
 __global__ __launch_bounds__(64 * WN * WM) void gemm_direct_kernel(const bf16_t* __restrict__ A,
                                                                    const bf16_t* __restrict__ W,
                                                                    TC* __restrict__ C, int M, int N, int K,
@@ -97,8 +100,7 @@ __global__ __launch_bounds__(64 * WN * WM) void gemm_direct_kernel(const bf16_t*
     // memory channels would take all the traffic.  With several rows of tiles the tiles that share
     // a slice must stay in step, so that one of them finds it in L2.
     const int n_steps = K / BK;
-    // with one row of tiles every weight is read once: past the caches (the decode batches' tiles; in the
-    // prefill's, whose loads are spread between the MFMAs, the choice costs the long prompts 1.6 %)
+    // with one row of tiles every weight is read once: past the caches
     const bool stream_w = tiles_m == 1;
     const int first_step = tiles_m == 1 ? (int)(((unsigned)tile * 5u + blockIdx.y * 3u) % (unsigned)n_steps) : 0;
     auto issue = [&](int stage, int step) {
@@ -203,8 +205,10 @@ __global__ __launch_bounds__(64 * WN * WM) void gemm_direct_kernel(const bf16_t*
 #pragma unroll
                     for (int q = 0; q < PER; ++q) {
                         const int l = m * PER + q;
-                        if (l < W_LOADS) load_16_bytes_to_lds(w_off[l], wsrc, to + l * (NW * RG * BK * 2));
-                        else if (l < NL) load_16_bytes_to_lds(a_off[l - W_LOADS], asrc, to + (BN * BK * 2) + (l - W_LOADS) * (NW * RG * BK * 2));
+                        if (l < W_LOADS) {
+                            if constexpr (STREAM_SPREAD) stream_16_bytes_to_lds(w_off[l], wsrc, to + l * (NW * RG * BK * 2));
+                            else load_16_bytes_to_lds(w_off[l], wsrc, to + l * (NW * RG * BK * 2));
+                        } else if (l < NL) load_16_bytes_to_lds(a_off[l - W_LOADS], asrc, to + (BN * BK * 2) + (l - W_LOADS) * (NW * RG * BK * 2));
                     }
                     __builtin_amdgcn_sched_barrier(0);
                 }
@@ -387,7 +391,7 @@ __global__ __launch_bounds__(64 * WN * WM) void gemm_direct_kernel(const bf16_t*
     }
 }
 
-template <int TN, int TM, int WN, int WM, int BK, int NS>
+template <int TN, int TM, int WN, int WM, int BK, int NS, bool MAY_STREAM_SPREAD = false>
 static int launch_direct(const void* A, const void* W, void* C, int c_dt, int M, int N, int K, int64_t lda,
                          int64_t ldw, int64_t ldc, int epilogue, hipStream_t stream, int splits = 1,
                          int64_t c_split_stride = 0, NormLink link = NormLink{}) {
@@ -420,12 +424,19 @@ static int launch_direct(const void* A, const void* W, void* C, int c_dt, int M,
         if (lds > raised) {                                                                                \
             hipError_t e = hipFuncSetAttribute((const void*)gemm_direct_kernel<TN, TM, WN, WM, BK, NS, EPI, TC>, \
                                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);      \
+            if (e == hipSuccess && MAY_STREAM_SPREAD)                                                      \
+                e = hipFuncSetAttribute((const void*)gemm_direct_kernel<TN, TM, WN, WM, BK, NS, EPI, TC, MAY_STREAM_SPREAD>, \
+                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);             \
             PICOLM_REQUIRE(e == hipSuccess, "gemm_tiled: cannot raise the LDS limit: %s",                  \
                            hipGetErrorString(e));                                                          \
             raised = lds;                                                                                  \
         }                                                                                                  \
-        gemm_direct_kernel<TN, TM, WN, WM, BK, NS, EPI, TC><<<grid, block, lds, stream>>>(                 \
-            a, w, (TC*)C, M, N, k_len, lda, ldw, ldc, tiles_m, tiles_n, c_split_stride, link);             \
+        if (MAY_STREAM_SPREAD && tiles_m == 1)                                                             \
+            gemm_direct_kernel<TN, TM, WN, WM, BK, NS, EPI, TC, MAY_STREAM_SPREAD><<<grid, block, lds, stream>>>( \
+                a, w, (TC*)C, M, N, k_len, lda, ldw, ldc, tiles_m, tiles_n, c_split_stride, link);         \
+        else                                                                                               \
+            gemm_direct_kernel<TN, TM, WN, WM, BK, NS, EPI, TC><<<grid, block, lds, stream>>>(             \
+                a, w, (TC*)C, M, N, k_len, lda, ldw, ldc, tiles_m, tiles_n, c_split_stride, link);         \
     }
     if (epilogue == 0 && c_dt == PICOLM_F32) TD_LAUNCH(0, float)
     else if (epilogue == 0 && c_dt == PICOLM_BF16) TD_LAUNCH(0, bf16_t)

@@ -11,7 +11,7 @@ int picolm_gemm_direct_prefill_(int variant, const void* A, const void* W, void*
         case 10: return launch_direct<2, 2, 4, 2, 64, 3>(A, W, C, c_dt, M, N, K, lda, ldw, ldc, epilogue, stream, splits, c_split_stride, link);
         case 14:
         case 15: return picolm_gemm_direct_wide_(variant, A, W, C, c_dt, M, N, K, lda, ldw, ldc, epilogue, stream, splits, c_split_stride, link);
-        case 11: return launch_direct<2, 2, 2, 2, 64, 4>(A, W, C, c_dt, M, N, K, lda, ldw, ldc, epilogue, stream, splits, c_split_stride, link);
+        case 11: return launch_direct<2, 2, 2, 2, 64, 4, true>(A, W, C, c_dt, M, N, K, lda, ldw, ldc, epilogue, stream, splits, c_split_stride, link);
     }
     PICOLM_REQUIRE(false, "gemm_tiled: %d is no prefill tile variant", variant);
 }
