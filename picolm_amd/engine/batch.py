@@ -155,12 +155,13 @@ def token_pages(tok_seq, tok_pos, slots, table_host, ring_pages: int):
 
 
 def decode_pages_per_chunk(pos0, blocks_per_chunk: int, max_pages_per_chunk: int = 16, min_blocks: int = 160) -> int:
-    """Pages that one workgroup of the decode attention takes: the largest of 4, 8, 16 within
-    `max_pages_per_chunk` (a wave should not walk over too many tiles one after the other) that
-    still leaves `min_blocks` workgroups for the launch, which is most of the CUs; 4 (a page for
-    each of four waves) if none does.  Fewer, larger chunks mean fewer partial results to merge."""
+    """Pages that one workgroup of the decode attention takes: the largest of 4, 8, 16, 32, 64
+    within `max_pages_per_chunk` (what the kernel that will run was measured with) that still
+    leaves `min_blocks` workgroups for the launch, which is most of the CUs; 4 (a page for each of
+    four waves) if none does.  Fewer, larger chunks mean fewer partial results to merge and longer
+    streams a wave."""
     pages = [int(p) // PAGE_TOKENS + 1 for p in pos0]
-    for ppc in (16, 8):
+    for ppc in (64, 32, 16, 8):
         if ppc <= max_pages_per_chunk and sum((n + ppc - 1) // ppc for n in pages) * max(1, blocks_per_chunk) >= min_blocks:
             return ppc
     return 4

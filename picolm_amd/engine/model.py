@@ -100,7 +100,7 @@ class DecoderModel:
     def decode_geometry(self, n_seq: int) -> tuple[int, int]:
         """(workgroups per chunk, most pages a chunk should have) over the mixers that run a
         decode attention: the widest launch and the tightest limit size the step's work list."""
-        per_chunk, max_pages = 1, 16
+        per_chunk, max_pages = 1, 64
         for b in self.blocks:
             f = getattr(b.mixer, "decode_geometry", None)
             if f is not None:

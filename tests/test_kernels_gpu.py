@@ -545,6 +545,30 @@ def test_attention_decode(dtype, H, G, d, pages_per_chunk, window, spare):
         assert not done.any()
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("pages_per_chunk", [32, 64])
+def test_attention_decode_over_long_chunks(dtype, pages_per_chunk):
+    """Chunks of 32 and 64 pages, as long contexts get them: a wave walks over up to 16 tiles, most
+    of whose pages it looks up in the page table itself (a work list's entry carries four), and a
+    sequence of 64 pages is two chunks of 32 or one of 64; shorter sequences beside it."""
+    H, G, d = 8, 2, 128
+    pos0 = [4095, 2049, 70, 1984]
+    case = PagedCase(H, G, d, pos0, [1] * len(pos0), dtype, seed=pages_per_chunk)
+    b = case.batch()
+    ref = case.reference(0)
+    chunk_list, n_chunks, most = decode_work_list(case, 0, pages_per_chunk, spare=2)
+    partial = torch.full((b.n_seq * H * most * (d + 2),), float("nan"), device=DEV)
+    done = torch.zeros(K().attn_decode_counters(b.n_seq, H, G), dtype=torch.int32, device=DEV)
+    for counters in (None, done):
+        out = torch.zeros_like(case.q_dev)
+        args = (case.q_dev, case.k_pages, case.v_pages, out, partial, b.n_seq, chunk_list, n_chunks, pages_per_chunk, most,
+                b.seq_pos0, case.table, case.table.shape[1], H, G, d, 0, 1.0 / math.sqrt(d))
+        K().attn_decode(*args) if counters is None else K().attn_decode(*args, counters)
+        err = np.abs(out.double().cpu().numpy() - ref).max()
+        assert err <= tol(dtype, np.abs(ref).max()), err
+    assert not done.any()
+
+
 @pytest.mark.parametrize("d", [64, 128])
 @pytest.mark.parametrize("pages_per_chunk", [1, 4, 8])
 def test_attention_decode_many_sequences(d, pages_per_chunk):
