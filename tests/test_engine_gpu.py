@@ -146,6 +146,45 @@ def test_long_decoding_and_first_tokens(dtype, folders):
     assert s.length(a) == 400
 
 
+@pytest.mark.parametrize("native", [True, False])
+def test_decoding_at_contexts_of_thousands_of_tokens(native, tmp_path):
+    """Twelve sequences of about 5,000 tokens: enough pages for the decode attention to take chunks
+    of 64 (and, when most sequences have ended, 32 and 16), each sequence several chunks whose
+    partial results are merged.  All twelve are beginnings of one token sequence, so that one pass
+    of the plain implementation knows every logit; they differ in length, slot and pages."""
+    from picolm_amd import LlamaConfig, write_random_model
+    from picolm_amd.engine import Session, load_model
+    cfg = dict(architectures=["LlamaForCausalLM"], hidden_size=256, intermediate_size=344, num_attention_heads=8,
+               num_key_value_heads=8, num_hidden_layers=1, vocab_size=300, head_dim=32, rms_norm_eps=1e-5, rope_theta=10000.0,
+               tie_word_embeddings=False, max_position_embeddings=8192, torch_dtype="bfloat16")
+    d = write_random_model(LlamaConfig.from_dict(cfg), str(tmp_path / "long"), seed=21, std=0.05)
+    rng = np.random.default_rng(21)
+    toks = tiny.random_tokens(rng, 5010, 300)
+    truth = tiny.plain_logits(d, toks)
+    lens = [5000 - 37 * i for i in range(12)]
+    s = Session(load_model(d, dtype="bfloat16"), max_tokens=12 * 5120, native=native)
+    assert (s.engine is not None) == native
+    slots = s.begin(12)
+    got = s.step(slots, [toks[:n] for n in lens]).double().cpu().numpy()          # the prompts, all in one step
+    tol_ = tiny.tolerance("bfloat16", truth, tiny.spread(256, 0.05))
+    for i, n in enumerate(lens):
+        assert np.abs(got[i] - truth[n - 1]).max() <= tol_, ("prefill", i)
+    from picolm_amd.engine.batch import decode_pages_per_chunk
+    seen = set()
+    live = list(range(12))
+    for step in range(6):
+        if step == 2:
+            live = live[:8]                       # fewer sequences: shorter chunks
+        if step == 4:
+            live = live[:4]
+        pos = [lens[i] + step for i in live]
+        seen.add(decode_pages_per_chunk(pos, 8, 64))
+        got = s.step([slots[i] for i in live], [[toks[lens[i] + step]] for i in live]).double().cpu().numpy()
+        for k, i in enumerate(live):
+            assert np.abs(got[k] - truth[lens[i] + step]).max() <= tol_, (step, i)
+    assert seen == {64, 32, 16}
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_stale_cache_contents_change_nothing(dtype, folders):
     d = folders["B"]
