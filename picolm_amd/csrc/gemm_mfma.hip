@@ -223,7 +223,8 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const bf16_t* _
 // operands are read from there.  Whole lines are what lets the weights be marked non-temporal
 // (the kernel above asks for 64 bytes of 16 rows at a time, which such loads make slower), and
 // stages in LDS cost no registers, so that several steps of a wave are in flight: with 16 weight
-// rows and up to 8 activation rows six stages of 3 KB.  No barrier in the loop: a wave reads only
+// rows and up to 8 activation rows six stages of 3 KB (and with 48 and 16, two of 8 KB, which
+// still beat the kernel above: 12,288 x 4,096 at 16 rows 18.5 against 22.2 us).  No barrier in the loop: a wave reads only
 // what it loaded, when its own count of outstanding loads says that it has arrived.  All loads of
 // the loop are assembly for that count's sake, as in the tile kernel.
 #define SKS_KSTEP 64
@@ -345,7 +346,7 @@ static int skinny_staged_stages(int M, int K, int rows_per_wg) {
     int stages = (SKS_LDS_BYTES - 4096) / 8 / (per_step * 1024);      // (the kernel has 2 KB of its own)
     if (stages > 8) stages = 8;
     while (stages > 1 && (stages - 1) * per_step > 42) --stages;
-    return stages >= 3 ? stages : 0;
+    return stages >= 2 ? stages : 0;
 }
 template <int NT>
 static int launch_skinny_staged(const void* A, const void* W, void* C, int c_dt, int M, int N, int K, int64_t lda,
