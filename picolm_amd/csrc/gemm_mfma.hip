@@ -340,10 +340,11 @@ __global__ __launch_bounds__(512) void gemm_skinny_staged_kernel(const bf16_t* _
 }
 
 // Whether the staged kernel takes a product, and with how many stages a wave.
-static int skinny_staged_stages(int M, int K, int rows_per_wg) {
+// two_a_cu: half of the LDS, so that two workgroups share a CU
+static int skinny_staged_stages(int M, int K, int rows_per_wg, bool two_a_cu = false) {
     if (M > 16 || K % SKS_KSTEP || rows_per_wg % 8 || rows_per_wg > 48) return 0;
     const int per_step = (rows_per_wg + 7) / 8 + (M + 7) / 8;
-    int stages = (SKS_LDS_BYTES - 4096) / 8 / (per_step * 1024);      // (the kernel has 2 KB of its own)
+    int stages = ((two_a_cu ? SKS_LDS_BYTES / 2 : SKS_LDS_BYTES) - 4096) / 8 / (per_step * 1024);      // (the kernel has 2 KB of its own)
     if (stages > 8) stages = 8;
     while (stages > 1 && (stages - 1) * per_step > 42) --stages;
     return stages >= 2 ? stages : 0;
@@ -351,7 +352,7 @@ static int skinny_staged_stages(int M, int K, int rows_per_wg) {
 template <int NT>
 static int launch_skinny_staged(const void* A, const void* W, void* C, int c_dt, int M, int N, int K, int64_t lda,
                                 int64_t ldw, int64_t ldc, int epi, hipStream_t stream, NormLink link, int rows_per_wg) {
-    const int stages = skinny_staged_stages(M, K, rows_per_wg);
+    const int stages = skinny_staged_stages(M, K, rows_per_wg, ceil_div(N, rows_per_wg) > n_compute_units());
     PICOLM_REQUIRE(stages > 0 && rows_per_wg <= 16 * NT, "gemm_skinny: the staged kernel does not take M=%d K=%d with %d rows a workgroup", M, K, rows_per_wg);
     PICOLM_REQUIRE(!link.next_w || (NT <= 2 && epi == 1 && rows_per_wg == 16 * NT && link.next_parts >= ceil_div(N, 16)),
                    "gemm_skinny: whole tiles of 16 weight rows with the accumulating epilogue prepare a norm");
@@ -456,10 +457,11 @@ static int launch_skinny_sized(const void* A, const void* W, void* C, int c_dt, 
     const int cus = n_compute_units();
     const bool two_tiles = N % 32 == 0 && ceil_div(N, 16) > cus && N / 32 <= cus && skinny_staged_stages(M, K, 32) > 0;
     const int rows = link.next_w ? (staged && MT == 1 && two_tiles ? 32 : 16) : skinny_rows_per_wg(N, M);
-    // The staged kernel where every CU has at most one workgroup: its stages fill the LDS, so that a
-    // second round of workgroups would wait for the first to leave (12,288 rows as 512 workgroups: 22
-    // us against 19; a vocabulary of 128,256 rows: 183 against 165).
-    if (staged && MT == 1 && skinny_staged_stages(M, K, rows) > 0 && ceil_div(N, rows) <= n_compute_units()) {
+    // A launch of more workgroups than CUs gets half the LDS a workgroup, so that two share a CU and
+    // one's start and end overlap the other's loop (with all of it, a second round of workgroups
+    // waits for the first to leave: 12,288 rows as 512 workgroups took 22 us, 17.4 this way and 19
+    // in the kernel above; a vocabulary of 128,256 rows 183, 155 and 165).
+    if (staged && MT == 1 && skinny_staged_stages(M, K, rows, ceil_div(N, rows) > n_compute_units()) > 0) {
         if (rows <= 16) return launch_skinny_staged<1>(A, W, C, c_dt, M, N, K, lda, ldw, ldc, epi, stream, link, rows);
         if (rows <= 32) return launch_skinny_staged<2>(A, W, C, c_dt, M, N, K, lda, ldw, ldc, epi, stream, link, rows);
         return launch_skinny_staged<3>(A, W, C, c_dt, M, N, K, lda, ldw, ldc, epi, stream, link, rows);

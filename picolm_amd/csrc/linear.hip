@@ -120,9 +120,10 @@ extern "C" int picolm_linear(const void* A, int a_dt, const void* W, int w_dt, v
     // cover whole lines, streams the weights past the caches (measured with weights from memory,
     // 28,672 x 4,096: 37.0 us against the skinny kernel's 40.2 at one row, 37.2 against 43.7 at
     // eight; 57,344 x 8,192: 142 against 164 and 144 against 177; 12,288 rows, 96 tiles, are
-    // better off skinny: 19 against 26 us).  One to four rows of many rounds (a vocabulary) stay
-    // skinny: 165 against 167 us for 128,256 rows.
-    const bool one_round = M <= 16 && K % 64 == 0 && N >= 16384 && (M > 4 || N <= 512 * 128);
+    // better off skinny: 19 against 26 us).  Up to eight rows of many rounds (a vocabulary) stay
+    // skinny, two staged workgroups a CU: 155 against 167 us for 128,256 rows at one row, 154
+    // against 172 at eight.
+    const bool one_round = M <= 16 && K % 64 == 0 && N >= 16384 && (M > 8 || N <= 512 * 128);
     if (!linked) {
         if (one_round) return picolm_gemm_tiled_splitk(A, W, C, c_dt, M, N, K, K, K, ldc, epilogue, 13, 1, nullptr, stream);
         return picolm_gemm_skinny(A, W, C, c_dt, M, N, K, K, K, ldc, epilogue, 0, stream);
