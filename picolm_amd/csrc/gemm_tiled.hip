@@ -417,7 +417,8 @@ static void tiled_choice(int M, int N, int K, int epilogue, int64_t ws_floats, i
 extern "C" int picolm_gemm_tiled_norm_parts(int M, int N, int K, int64_t ws_floats) {
     int variant, splits, n_first;
     tiled_choice(M, N, K, 1, ws_floats, variant, splits, n_first);       // the product that prepares a norm adds to the rows
-    if (splits > 1) return N / 1024;
+    if (splits > 1) return N % 1024 ? 0 : N / 1024;      // the kernel that adds the parts takes 1024 columns a workgroup
+    if (N % 2) return 0;                                 // the tile kernels write the next rows in pairs of columns
     return variant == 9 || variant == 10 ? ceil_div(N, 256) : variant == 11 ? ceil_div(N, 128) : variant == 14 ? ceil_div(N, 192) : variant == 15 ? ceil_div(N, 320) : 0;
 }
 

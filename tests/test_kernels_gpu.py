@@ -302,6 +302,17 @@ def test_gemm_with_a_norm_split_between_two_products_of_a_prefill_step(M, D):
     # K no multiple of 64: the older tiles, which take no part
     assert not k.gemm_links_norms(torch.zeros(M, 72, dtype=torch.bfloat16, device=DEV),
                                   torch.zeros(D, 72, dtype=torch.bfloat16, device=DEV), x, 1, prepares=True)
+    # the answer beforehand and the kernels' own conditions agree at widths that some of them refuse
+    # (an odd one: the tiles write pairs of columns; cut along K, one that is no multiple of 1024):
+    # a yes runs, and an odd width gets a no
+    for width in (515, 1500, 1032):
+        a, w = torch.zeros(M, 512, dtype=torch.bfloat16, device=DEV), torch.zeros(width, 512, dtype=torch.bfloat16, device=DEV)
+        c = torch.zeros(M, width, device=DEV)
+        yes = k.gemm_links_norms(a, w, c, 1, prepares=True)
+        assert yes == (k.linked_norm_parts(M, width, 512) > 0) and not (yes and width % 2)
+        if yes:
+            k.gemm_linked(a, w, c, 1, prepare=(torch.ones(width, device=DEV), torch.empty(M, width, dtype=torch.bfloat16, device=DEV),
+                                               torch.empty(k.linked_norm_parts(M, width, 512), k.linked_norm_rows(M), device=DEV)))
 
 
 def test_gemm_tiles_of_192_and_320_columns_where_they_fill_the_rounds_better():
