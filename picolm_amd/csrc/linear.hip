@@ -30,14 +30,17 @@ static bool mfma_takes(const void* a, int a_dt, const void* w, int w_dt, int c_d
 static int medium_variant(int M) { return M <= 32 ? 13 : 12; }
 
 // Into how many parts along K a product of 17..64 rows is cut: its tiles hold 128 weight rows
-// each, and every CU should have one.
+// each, and every CU should have one; never a few more workgroups than CUs, whose last ones run
+// while most CUs wait (measured with weights from memory at 32 rows: 80 tiles, 10,240 x 8,192,
+// cut in two 36.7 us and in four 43.0; 40 tiles, 5,120 x 13,824, in four 33.6 and in eight 37.8;
+// 160 tiles, 20,480 x 4,096, uncut 31.6 and in two 41.7).
 extern "C" int picolm_linear_medium_splits(int M, int N, int K);
 static int medium_splits(int M, int N, int K) { return picolm_linear_medium_splits(M, N, K); }
 extern "C" int picolm_linear_medium_splits(int M, int N, int K) {
     const int tiles = (N + 127) / 128;
     if (tiles >= 200 || N % 4) return 1;
     int s = 8;
-    while (s > 1 && (tiles * s > 320 || K % (64 * s) || (int64_t)s * M * N > PICOLM_SPLITK_WS_FLOATS)) s /= 2;
+    while (s > 1 && (tiles * s > n_compute_units() || K % (64 * s) || (int64_t)s * M * N > PICOLM_SPLITK_WS_FLOATS)) s /= 2;
     return s;
 }
 
