@@ -48,6 +48,12 @@ SHAPES = {
                     num_key_value_heads=32, num_hidden_layers=32, vocab_size=32000, head_dim=128, rms_norm_eps=1e-5,
                     rope_theta=10000.0, rope_scaling=None, tie_word_embeddings=False, max_position_embeddings=4096,
                     eos_token_id=2, bos_token_id=1)),
+    "llama32-1b": dict(
+        name="Llama-3.2-1B shape", std=0.02, batch=8, steps=64, warmup=8, prompt_range=(128, 2048), points=(1, 64),
+        config=dict(architectures=["LlamaForCausalLM"], hidden_size=2048, intermediate_size=8192, num_attention_heads=32,
+                    num_key_value_heads=8, num_hidden_layers=16, vocab_size=128256, head_dim=64, rms_norm_eps=1e-5,
+                    rope_theta=500000.0, rope_scaling=dict(LLAMA3_SCALING, factor=32.0), tie_word_embeddings=True,
+                    max_position_embeddings=131072, eos_token_id=128001, bos_token_id=128000)),
     "llama31-70b": dict(
         name="Llama-3.1-70B shape", std=0.01, batch=8, steps=16, warmup=3, prompt_range=(128, 2048), points=(1,),
         config=dict(architectures=["LlamaForCausalLM"], hidden_size=8192, intermediate_size=28672, num_attention_heads=64,

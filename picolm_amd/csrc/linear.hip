@@ -125,8 +125,13 @@ extern "C" int picolm_linear(const void* A, int a_dt, const void* W, int w_dt, v
     // eight; 57,344 x 8,192: 142 against 164 and 144 against 177; 12,288 rows, 96 tiles, are
     // better off skinny: 19 against 26 us).  Up to eight rows of many rounds (a vocabulary) stay
     // skinny, two staged workgroups a CU: 155 against 167 us for 128,256 rows at one row, 154
-    // against 172 at eight.
-    const bool one_round = M <= 16 && K % 64 == 0 && N >= 16384 && (M > 8 || N <= 512 * 128);
+    // against 172 at eight; and so do up to eight rows of a product whose tiles reach little more
+    // than half of the CUs, unless K is long (16,384 x 2,048: 14.3 against 16.3 us at one row, 14.7
+    // against 16.9 at eight; x 4,096: 23.5 against 26.7 and 22.3 against 27.9; 18,432 x 4,096: 24.9
+    // against 27.7 and 24.4 against 28.4; 19,456 x 4,096: 27.0 against 27.6 and 26.1 against 28.9;
+    // 16,384 x 8,192: 48.6 against 47.2 and 52.1 against 48.8).
+    const bool one_round = M <= 16 && K % 64 == 0 && N >= 16384 &&
+                           (M > 8 || (N <= 512 * 128 && (N > 72 * n_compute_units() || K > 4096)));
     if (!linked) {
         if (one_round) return picolm_gemm_tiled_splitk(A, W, C, c_dt, M, N, K, K, K, ldc, epilogue, 13, 1, nullptr, stream);
         return picolm_gemm_skinny(A, W, C, c_dt, M, N, K, K, K, ldc, epilogue, 0, stream);
