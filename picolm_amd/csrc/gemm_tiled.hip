@@ -397,13 +397,14 @@ static int tiled_splits(int M, int N, int K, int variant, int64_t ws_floats) {
 // The variant, the cut along K and the two-launch plan for a shape.  Where the 128x128 tiles are
 // too many to cut but the 256x128 ones are few and K is long (a prompt of 768 tokens into the
 // model's width from the feed-forward's), the larger tile cut in two is the faster (measured
-// 103 against 114 us at 768 x 4096 x 14336; with K = 4096 the smaller tile uncut wins).
+// 103 against 114 us at 768 x 4096 x 14336 and 135 against 140 at 1024 rows; with K = 4096 the
+// smaller tile uncut wins, and with K = 8192 too: 76 against 82 us at 2048 x 2048 x 8192).
 static void tiled_choice(int M, int N, int K, int epilogue, int64_t ws_floats, int& variant, int& splits, int& n_first) {
     variant = tiled_plan(M, N, K, epilogue, n_first);
     splits = 1;
     if (n_first > 0) return;
     splits = tiled_splits(M, N, K, variant, ws_floats);
-    if (splits == 1 && variant == 11 && K >= 8192) {
+    if (splits == 1 && variant == 11 && K > 8192) {
         const int s10 = tiled_splits(M, N, K, 10, ws_floats);
         if (s10 > 1) {
             variant = 10;
