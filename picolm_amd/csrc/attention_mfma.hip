@@ -884,11 +884,15 @@ int check_decode_chunks(const char* who, const float* partial, const int32_t* ch
                         int pages_per_chunk, int max_splits);
 int picolm_attn_merge_launch(const AttnArgs& a, int dt, int n_seq, hipStream_t stream);
 
-// waves of a decode workgroup: eight give a short step for a few sequences; with many sequences
-// four waves, two workgroups a CU, move more bytes
+// waves of a decode workgroup: eight while every sequence's workgroups are at most two a CU of
+// 256 (a sequence's pages are a shorter chain for each wave); beyond that four waves move more
+// bytes.  Measured, eight against four waves a step: 256 workgroups 4.59 against 4.61 ms (8 KV
+// groups of head size 128, batch 32) and 1.41 against 1.53 (head size 64); 384: 5.16 against
+// 5.37; 512: 5.74 against 5.83, 1.78 against 1.80, and 3.98 against 3.96 (32 KV groups, batch
+// 16); 1,024: 8.77 against 8.64; 2,048: 8.37 against 7.81.
 extern "C" int picolm_attn_decode_mfma_waves(int n_seq, int H, int G) {
     const int chunks = ceil_div(H / (G > 0 ? G : 1), 32);
-    return (int64_t)n_seq * G * chunks >= 256 ? 4 : 8;
+    return (int64_t)n_seq * G * chunks > 512 ? 4 : 8;
 }
 
 static int launch_decode_mfma(const AttnArgs& a, int n_seq, int n_chunks, hipStream_t stream) {
