@@ -1,13 +1,13 @@
 #!/usr/bin/env python3
 """Decode and prefill throughput of a Llama shape on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--shape llama31-8b|llama2-7b|llama31-70b]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--shape llama31-8b|llama2-7b|llama31-70b|llama32-1b]
                     [--batch B] [--layers L]
 
 The default run is the Llama-3.1-8B shape at batch 8 and a context of up to 4,096; the other
 shapes are the other workloads the library is measured on (Llama-2-7B: batch 16, prompts of 64 to
 1,024 tokens, 256 greedy steps; Llama-3.1-70B: 80 layers with 141 GB of weights made on the GPU,
-decode at batch 8 and 1).  A step is one decode step of the generation loop's inner body: the model
+decode at batch 8 and 1; Llama-3.2-1B: head size 64 and a tied head, batch 8, 1 and 64).  A step is one decode step of the generation loop's inner body: the model
 step over the batch from the cache, the sampler, and the hand-over of the sampled tokens.  Weights
 are random bf16 made on the GPU, prompts are seeded uniform-random token ids; they go through the
 model as the generation loop sends them (one step, or the steps of its token budget).  Prints one
