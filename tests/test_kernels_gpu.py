@@ -159,6 +159,17 @@ def test_gemm_medium_batches_pick_their_splits():
     assert medium_gemm_splits(64, 4096, 14336) == 8
     assert medium_gemm_splits(64, 4096, 64 * 3) == 1         # K does not split evenly
     assert medium_gemm_splits(33, 130, 4096) == 1            # N no multiple of 4
+    # never a few more workgroups than CUs: 80 tiles in two parts, 160 tiles uncut, 40 tiles in four
+    cus = torch.cuda.get_device_properties(0).multi_processor_count
+    for N in (10240, 20480, 5120):
+        assert (N // 128) * medium_gemm_splits(32, N, 8192) <= cus < 2 * (N // 128) * medium_gemm_splits(32, N, 8192)
+
+
+def test_decode_attention_picks_eight_waves_up_to_two_workgroups_a_cu():
+    waves = K().lib().picolm_attn_decode_mfma_waves
+    assert waves(8, 32, 8) == 8 and waves(64, 32, 8) == 8            # 64 and 512 workgroups
+    assert waves(65, 32, 8) == 4 and waves(16, 32, 32) == 8 and waves(17, 32, 32) == 4
+    assert waves(4, 128, 2) == 8 and waves(512, 128, 2) == 4         # 64 heads a group: two workgroups each
     for M, N, Kd in ((64, 4096, 4096), (40, 6144, 1024), (17, 260, 192), (64, 28672 // 4, 512), (8, 16384 + 2, 128),
                      (5, 128 * 256, 64)):
         for epi, cdt in ((0, torch.float32), (2, torch.bfloat16), (1, torch.float32)):
