@@ -16,8 +16,8 @@
 //            workgroup take different heads of the group, so a page is loaded once per group.
 //   decode : a wave streams its own pages straight from global memory into MFMA operands
 //            (columns = the query heads of one KV group); the 4 waves of a workgroup take
-//            pages in turn and merge through LDS; split-K partials go to a buffer that the
-//            merge kernel of the generic path combines.
+//            pages in turn and merge through LDS; the chunks of a sequence leave partial
+//            results in a buffer, and the workgroup that finishes last adds them up itself.
 #include <utility>
 #include "common.h"
 #include "api.h"
