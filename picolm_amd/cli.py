@@ -108,7 +108,7 @@ def main(argv=None) -> int:
         lines = []
     prompts = [parse_ids(l) for l in lines]
 
-    from .cache.slots import PAGE_TOKENS, pages_for
+    from .cache import PAGE_TOKENS, pages_for
     from .engine import Session, load_model
     from .generation import generate
     model = load_model(args.model, dtype=args.dtype)

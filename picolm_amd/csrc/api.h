@@ -10,6 +10,9 @@ extern "C" {
 #endif
 
 const char* picolm_last_error(void);
+// leaves a message for picolm_last_error(): for code outside the library that fails a call of the
+// library's (an operation of the caller's inside an engine's program)
+void picolm_set_error_message(const char* message);
 int picolm_abi_version(void);
 int picolm_device_check(void);     // 0 if the current device is a gfx950
 

@@ -152,7 +152,9 @@ def load() -> ctypes.CDLL:
     if _LIB is None:
         path = _built_library() or build()
         try:
-            _LIB = ctypes.CDLL(path)
+            # (its symbols are visible to libraries loaded later: a part with kernels of its own, built
+            # elsewhere, may call the error channel)
+            _LIB = ctypes.CDLL(path, mode=ctypes.RTLD_GLOBAL)
         except OSError as e:
             raise BuildError(f"cannot load {path}: {e}") from None
     return _LIB

@@ -9,6 +9,13 @@
 // step to step: slots and pages, the step's index arrays, the workspace, recorded decode steps.
 // Weights stay with the caller, as device pointers inside the operations.
 //
+// A program is made by whoever knows the architecture: in this library the Python parts read
+// config.json, bind the checkpoint's tensors and emit it (picolm_amd/engine/model.py), so a C
+// caller starts at a built program, where picolm's starts at a file name (model_load).  The set
+// of operations is open: PICOLM_OP_CALL hands the running step to a function of the caller's, so
+// that a part with kernels of its own (a mixer with state, another norm, a routed feed-forward)
+// joins a program without a change to this header or to the engine.
+//
 // Every function returns 0 or a negative code and leaves a message for picolm_last_error().
 // Nothing here waits for the GPU unless it says so; work is queued on the stream that is passed
 // in, and all calls on one engine must use one stream (or be ordered by the caller).  An engine is
@@ -27,7 +34,7 @@ extern "C" {
 #define PICOLM_ERR_CACHE (-12)       // a slot freed twice, a slot that does not exist
 #define PICOLM_ERR_DEVICE (-13)      // the HIP runtime refused something
 
-enum { PICOLM_OP_EMBED = 1, PICOLM_OP_RMSNORM = 2, PICOLM_OP_LINEAR = 3, PICOLM_OP_ATTENTION = 4 };
+enum { PICOLM_OP_EMBED = 1, PICOLM_OP_RMSNORM = 2, PICOLM_OP_LINEAR = 3, PICOLM_OP_ATTENTION = 4, PICOLM_OP_CALL = 5 };
 // which rows of the step an operation covers: every new token's, or only those whose logits are wanted
 enum { PICOLM_ROWS_STEP = 0, PICOLM_ROWS_WANTED = 1 };
 
@@ -37,6 +44,53 @@ typedef struct {
     int32_t rows;            // PICOLM_ROWS_STEP or PICOLM_ROWS_WANTED
     int32_t dtype;           // PICOLM_F32 (0) or PICOLM_BF16 (1)
 } picolm_buffer;
+
+// What a called operation (PICOLM_OP_CALL) sees of the running step.  Everything is read-only for
+// it but the memory behind `out`, `extra` of buffers it writes, its cache entry and its state.
+// Host arrays are valid during the call; device memory until the step's work has run.
+typedef struct {
+    int32_t struct_bytes;        // sizeof(picolm_step_view) in the library that made it
+    int32_t dtype;               // the engine's: PICOLM_F32 or PICOLM_BF16
+    int32_t n_seq, n_tokens, n_wanted;
+    int32_t is_decode;           // every sequence brings one token
+    int32_t every_row_wanted;    // the wanted rows are the step's rows, in order
+    int32_t recording;           // the stream records (a decode step that will be replayed): the host arrays
+                                 // below hold this step's values and will not be seen again
+    const int32_t *slots, *pos0, *n_new;     // host, [n_seq]: cache slot, tokens held before the step, new tokens
+    // device int32 arrays: per sequence [n_seq] (cu_seqlens [n_seq + 1]), per token [n_tokens], wanted rows [n_wanted]
+    const int32_t *seq_slot, *seq_pos0, *seq_nnew, *cu_seqlens, *tok_pos, *tok_seq, *tokens, *want_rows;
+    int32_t rows;                // rows the operation covers: n_tokens or n_wanted
+    void *in, *out, *extra[4];   // the operation's buffers (null where it names none)
+    int32_t in_row_bytes, out_row_bytes, extra_row_bytes[4];
+    // the cache entry of the operation (PICOLM_CALL_KV): keys [n_pages][G][64][d], values [n_pages][G][dv][64]
+    void *k_pages, *v_pages;
+    const int32_t* page_table;   // device [n_slots][max_pages]; logical page j of a slot lies at column j % ring_pages
+    int32_t n_pages, max_pages, ring_pages, n_kv_heads, head_dim, v_head_dim, window, kv_writes;
+    const int32_t* write_pages;  // device [n_tokens]: the physical page that takes each new token's key and value
+    // with PICOLM_CALL_ATTENDS: the decode step's work list over that group's pages (see
+    // picolm_attn_decode_generic in api.h), or the prefill step's tiles of `tile_rows` new tokens
+    const int32_t* chunk_list;
+    int32_t n_chunks, pages_per_chunk, most_chunks;
+    float* partial;              // [n_seq][most_chunks][partial_floats] floats for partial results
+    int32_t* counters;           // zero when the call starts; whoever uses them leaves them at zero
+    const int32_t *tile_seq, *tile_q0;
+    int32_t n_tiles, tile_rows;
+    // the state entry of the operation (PICOLM_CALL_STATE): [n_slots][state_bytes_per_slot], zeroed when a slot is given out
+    void* state;
+    int64_t state_bytes_per_slot;
+    int32_t n_slots;
+    hipStream_t stream;          // queue the work here; do not wait for it
+} picolm_step_view;
+
+// Returns 0, or a negative code after picolm_set_error (or any message of its own: a non-zero
+// return fails the step with PICOLM_ERR_STEP unless it is one of the codes above).
+typedef int (*picolm_call_fn)(void* user, const picolm_step_view* view);
+
+#define PICOLM_CALL_RECORDABLE 1   // what it queues depends on device memory only (not on the view's host arrays,
+                                   // not on allocations of its own): a decode step that holds it may be recorded and replayed
+#define PICOLM_CALL_KV 2           // it uses the cache entry (kv_group, kv_entry); kv_writes as for ATTENTION
+#define PICOLM_CALL_ATTENDS 4      // with PICOLM_CALL_KV: it wants the decode work list and, with tile_rows > 0, the prefill tiles
+#define PICOLM_CALL_STATE 8        // it uses the state entry (state_group, state_entry)
 
 // One operation.  Buffers are indices into the program's buffers.  Fields an operation does not
 // use are zero.
@@ -52,6 +106,11 @@ typedef struct {
 //              [table_positions][d/2], null for none; rope_style 0 pairs (2i, 2i+1), 1 pairs
 //              (i, i + d/2)), writes k and v to cache entry (kv_group, kv_entry) unless
 //              kv_writes = 0, attends over the cache; out [H d]; q_buffer: scratch [H d].
+//              window > 0: only the last `window` keys are seen, and the group keeps a ring of pages.
+//   CALL       call(call_user, view) queues whatever it likes on the view's stream.  in, out and
+//              extra[] name buffers (-1 for none; out is required and decides the rows covered);
+//              call_flags as above; partial_floats: floats per sequence and chunk it wants at
+//              view->partial.
 typedef struct {
     int32_t kind, rows;
     int32_t in, out;
@@ -70,11 +129,18 @@ typedef struct {
     const float* sin_table;
     int32_t rope_style, table_positions;
     int32_t kv_group, kv_entry, kv_writes, q_buffer;
+    picolm_call_fn call;
+    void* call_user;
+    int32_t call_flags;
+    int32_t state_group, state_entry;
+    int32_t extra[4];
+    int32_t tile_rows, partial_floats;
 } picolm_op;
 
-// Keys and values of `n_entries` layer calls that need the same kind of cache.  v_head_dim: the
-// size of a value where it is not that of a key (0: the same); the attention operation here takes
-// one size for both.
+// Keys and values of `n_entries` layer calls that need the same kind of cache.  window > 0: the
+// group keeps the last `window` keys of a sequence in a ring of pages (enough for a window and a
+// prefill chunk of 256 tokens); 0: all keys.  v_head_dim: the size of a value where it is not that
+// of a key (0: the same); the ATTENTION operation takes one size for both, a called operation any.
 typedef struct {
     int32_t n_entries, n_kv_heads, head_dim, window, v_head_dim;
 } picolm_kv_group;
@@ -176,7 +242,9 @@ int picolm_engine_free_pages(picolm_engine* e, int32_t group);
 // One of the index arrays of the step planned last, by name, from the host's copy: "seq_slot",
 // "seq_pos0", "seq_nnew", "cu_seqlens", "tok_pos", "tok_seq", "tokens", "want_rows",
 // "write_pages.<group>", "chunks.<group>" (the decode work list with its header),
-// "tiles.<rows>.seq", "tiles.<rows>.q0".  Returns the number of ints (negative: no such array).
+// "tiles.<rows>.seq", "tiles.<rows>.q0", and of slice c of a prefill step for the groups that keep a
+// ring "window_chunk.<c>.seq_slot", ".seq_pos0", ".seq_nnew", ".first_row", ".rows", ".tiles.<rows>.seq",
+// ".tiles.<rows>.q0".  Returns the number of ints (negative: no such array).
 int picolm_engine_step_array(picolm_engine* e, const char* name, int32_t* out, int32_t capacity);
 
 #ifdef __cplusplus

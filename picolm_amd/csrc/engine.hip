@@ -13,6 +13,7 @@
 #include <map>
 #include <memory>
 #include <string>
+#include <tuple>
 #include <vector>
 
 #define E_REQUIRE(code, cond, ...)            \
@@ -84,19 +85,27 @@ struct SlotTable {
     bool is_live(int s) const { return s >= 0 && s < n_slots && live[s]; }
 };
 
+// New tokens of one sequence that a group with a window takes in at once: its ring holds a window
+// and one such chunk, so a longer prompt is written and answered chunk by chunk.
+static const int WINDOW_STEP_TOKENS = 256;
+
 struct KVGroup {
     picolm_kv_group spec;
     int max_pages = 0, ring_pages = 0, n_pages = 0;
     PagePool pool;
-    std::vector<std::vector<int>> pages;     // slot -> its pages in logical order
+    std::vector<std::vector<int>> pages;     // slot -> its pages in logical order (a ring: page j lies at j % ring_pages)
     std::vector<int32_t> table_host;         // [n_slots][max_pages]
     int32_t* table_dev = nullptr;
     char* k = nullptr;                       // [n_entries][n_pages][G][64][d]
-    char* v = nullptr;                       // [n_entries][n_pages][G][d][64]
-    size_t entry_bytes = 0;
+    char* v = nullptr;                       // [n_entries][n_pages][G][dv][64]
+    size_t k_entry_bytes = 0, v_entry_bytes = 0;
     std::vector<int> dirty;                  // slots whose table row changed since the last flush
-    int need(int n_tokens) const { return pages_for(n_tokens); }
+    int value_dim() const { return spec.v_head_dim ? spec.v_head_dim : spec.head_dim; }
+    bool is_ring() const { return ring_pages < max_pages; }
+    int need(int n_tokens) const { return std::min(pages_for(n_tokens), ring_pages); }
     int missing(int slot, int n_tokens) const { return std::max(0, need(n_tokens) - (int)pages[slot].size()); }
+    // the first page that a query at `pos` sees
+    int first_page(int pos) const { return spec.window > 0 ? std::max(0, pos - spec.window + 1) / PAGE_TOKENS : 0; }
 };
 
 struct StateGroup {
@@ -196,6 +205,18 @@ struct DecodeList {
     int n_chunks = 0;       // entries the launch covers
     int most = 1;           // chunks a sequence can have: stride of the partial results
 };
+// A slice of a prefill step along positions (new tokens lo .. lo + 255 of every sequence that has
+// them): it looks like a step of its own to the attention kernels.
+struct WindowChunk {
+    int n_seq = 0, n_rows = 0;
+    Span seq_slot, seq_pos0, seq_nnew, first_row, rows;
+    std::vector<TileList> tiles;
+    const TileList* tiles_of(int rows_per_tile) const {
+        for (auto& t : tiles)
+            if (t.rows_per_tile == rows_per_tile) return &t;
+        return nullptr;
+    }
+};
 
 // What the operations read of a step: sizes, and where each array lies in the int block.
 struct StepPlan {
@@ -206,6 +227,7 @@ struct StepPlan {
     std::vector<Span> write_pages;        // per KV group (n = 0: not needed)
     std::vector<DecodeList> lists;        // per KV group, decode steps
     std::vector<TileList> tiles;          // prefill steps
+    std::vector<WindowChunk> window_chunks;   // prefill steps of more than WINDOW_STEP_TOKENS a sequence, where a group keeps a ring
     int pages_per_chunk = 0;
     std::vector<int32_t> ints;            // the host's copy of the block
     const int32_t* dev = nullptr;         // the block on the device
@@ -238,11 +260,14 @@ static int decode_pages_per_chunk(const std::vector<int>& pos0, int blocks_per_c
     return 4;
 }
 
-// The work list of a decode step over one group's pages: every sequence's pages cut into runs of
-// `ppc`; an entry is {sequence, which chunk, position of the new token, slot, physical pages of
-// the chunk's first four pages or -1}.  The chunks with the most pages come first: workgroups are
-// handed out in the list's order, and the short last chunks then fill the gaps at the end.
+// The work list of a decode step over one group's pages: every sequence's visible pages (those of
+// its last `window` keys, or all) cut into runs of `ppc`; an entry is {sequence, which chunk,
+// position of the new token, slot, physical pages of the chunk's first four pages or -1}.  The
+// chunks with the most pages come first: workgroups are handed out in the list's order, and the
+// short last chunks then fill the gaps at the end.
 // Returns the number of entries written behind the header at `out`; *most: chunks of the longest.
+static int chunks_of(const KVGroup& g, int pos, int ppc) { return (pos / PAGE_TOKENS + 1 - g.first_page(pos) + ppc - 1) / ppc; }
+
 static int fill_chunk_list(int32_t* out, const std::vector<int>& slots, const std::vector<int>& pos0, int ppc,
                            const KVGroup& g, int* most) {
     struct Chunk {
@@ -251,10 +276,10 @@ static int fill_chunk_list(int32_t* out, const std::vector<int>& slots, const st
     std::vector<Chunk> chunks;
     int longest = 0;
     for (int i = 0; i < (int)slots.size(); ++i) {
-        const int end = pos0[i] / PAGE_TOKENS + 1;
-        const int n = (end + ppc - 1) / ppc;
+        const int first = g.first_page(pos0[i]), end = pos0[i] / PAGE_TOKENS + 1;
+        const int n = (end - first + ppc - 1) / ppc;
         longest = std::max(longest, n);
-        for (int c = 0; c < n; ++c) chunks.push_back({i, c, std::min(end - c * ppc, ppc)});
+        for (int c = 0; c < n; ++c) chunks.push_back({i, c, std::min(end - first - c * ppc, ppc)});
     }
     std::stable_sort(chunks.begin(), chunks.end(), [](const Chunk& a, const Chunk& b) { return a.n_pages > b.n_pages; });
     out[0] = (int)chunks.size();
@@ -262,13 +287,13 @@ static int fill_chunk_list(int32_t* out, const std::vector<int>& slots, const st
     for (size_t x = 0; x < chunks.size(); ++x) {
         const Chunk& c = chunks[x];
         int32_t* e = out + 8 * (x + 1);
-        const int slot = slots[c.seq], end = pos0[c.seq] / PAGE_TOKENS + 1;
+        const int slot = slots[c.seq], first = g.first_page(pos0[c.seq]), end = pos0[c.seq] / PAGE_TOKENS + 1;
         e[0] = c.seq;
         e[1] = c.idx;
         e[2] = pos0[c.seq];
         e[3] = slot;
         for (int w = 0; w < 4; ++w) {
-            const int page = c.idx * ppc + w;
+            const int page = first + c.idx * ppc + w;
             const bool inside = page < end && w < ppc;
             e[4 + w] = inside ? g.table_host[(size_t)slot * g.max_pages + page % g.ring_pages] : -1;
         }
@@ -301,9 +326,11 @@ struct Workspace {
     size_t prep_h[2] = {0, 0}, prep_ssq[2] = {0, 0}, partial = 0;
     int for_T = -1, for_want = -1, for_seq = -1, for_most = -1;
     int flip = 1;
+    int64_t generation = 0;            // moves when the memory does
 };
 
 struct Prepared {                      // a norm that the product before has prepared
+    const picolm_op* by = nullptr;
     const void* x = nullptr;
     const float* w = nullptr;
     float eps = 0.f;
@@ -312,13 +339,18 @@ struct Prepared {                      // a norm that the product before has pre
     int parts = 0;
 };
 
+// A decode step of one shape (sequences, pages a chunk, chunks a sequence): its block, and the
+// recording of its launches once it has been used twice.  All of them share one workspace (they
+// run on one stream, one after the other); a recording holds that workspace's addresses and is
+// dropped when it moves.
 struct DecodeGraph {
     DecodeBatch batch;
-    Workspace ws;
     hipGraphExec_t exec = nullptr;
+    int64_t ws_generation = -1;
     int uses = 0;
-    float* logits = nullptr;
+    int64_t last_used = 0;
 };
+static const size_t MAX_DECODE_SHAPES = 48;      // blocks and recordings kept; the least recently used goes first
 
 struct picolm_engine {
     int dtype = PICOLM_BF16, vocab = 0, flags = 0;
@@ -337,6 +369,7 @@ struct picolm_engine {
     std::vector<int> tile_rows;            // tile heights of the prefill kernels in use
     int decode_blocks_per_chunk = 1, decode_max_pages_per_chunk = 64;
     int counters_needed = 0;
+    bool recordable = true;                // every called operation says that its launches may be recorded
     size_t partial_floats_per_seq_chunk = 0;   // max over attention operations of H * (d + 2)
     int prep_n = 0;                        // widest output that prepares a norm
     // the running step
@@ -346,7 +379,9 @@ struct picolm_engine {
     Workspace ws;
     Stager stager;
     float* splitk_ws = nullptr;
-    std::map<std::pair<int, int>, std::unique_ptr<DecodeGraph>> graphs;
+    Workspace decode_ws;                   // of all decode steps over blocks that stay in place
+    std::map<std::tuple<int, int, int>, std::unique_ptr<DecodeGraph>> graphs;
+    int64_t decode_tick = 0;
     hipStream_t capture_stream = nullptr;
     const StepPlan* last_plan = nullptr;
     // timing by class of operation (PICOLM_ENGINE_TIME_OPS): an event before and after each one
@@ -440,7 +475,7 @@ static int check_program(const picolm_program* p, picolm_engine* e) {
             case PICOLM_OP_ATTENTION: {
                 const int H = o.n_heads, G = o.n_kv_heads, d = o.head_dim;
                 E_REQUIRE(-1, H > 0 && G > 0 && H % G == 0 && d >= 1 && d <= 256, "engine: operation %d (attention): %d heads, %d groups, size %d", i, H, G, d);
-                E_REQUIRE(-1, o.window == 0, "engine: operation %d: attention over a window of keys is not run by this engine", i);
+                E_REQUIRE(-1, o.window >= 0, "engine: operation %d: a window of %d keys", i, o.window);
                 E_REQUIRE(-1, buf_ok(o.in) && buf_ok(o.q_buffer) && o.rows == PICOLM_ROWS_STEP, "engine: operation %d (attention) is incomplete", i);
                 const picolm_buffer &in = p->buffers[o.in], &q = p->buffers[o.q_buffer];
                 E_REQUIRE(-1, in.dtype == PICOLM_F32 && in.row_bytes >= 4 * (H + 2 * G) * d, "engine: operation %d (attention) reads float rows of q, k, v", i);
@@ -451,10 +486,40 @@ static int check_program(const picolm_program* p, picolm_engine* e) {
                 const picolm_kv_group& g = p->kv_groups[o.kv_group];
                 E_REQUIRE(-1, o.kv_entry >= 0 && o.kv_entry < g.n_entries && g.n_kv_heads == G && g.head_dim == d && g.window == o.window,
                           "engine: operation %d does not fit its cache group", i);
+                E_REQUIRE(-1, g.v_head_dim == 0 || g.v_head_dim == d,
+                          "engine: operation %d: the attention operation takes keys and values of one size, its group has %d and %d", i, d,
+                          g.v_head_dim);
                 E_REQUIRE(-1, (o.cos_table == nullptr) == (o.sin_table == nullptr) && (o.rope_style == 0 || o.rope_style == 1) &&
                                   (!o.cos_table || d % 2 == 0),
                           "engine: operation %d: rotation needs both tables, a pairing of 0 or 1 and an even head size", i);
                 E_REQUIRE(-1, o.scale > 0.f, "engine: operation %d: scale %g", i, o.scale);
+                break;
+            }
+            case PICOLM_OP_CALL: {
+                E_REQUIRE(-1, o.call != nullptr, "engine: operation %d (call) has no function", i);
+                E_REQUIRE(-1, o.in == -1 || buf_ok(o.in), "engine: operation %d (call) reads buffer %d, there are %d", i, o.in, p->n_buffers);
+                for (int x = 0; x < 4; ++x) {
+                    E_REQUIRE(-1, o.extra[x] == -1 || buf_ok(o.extra[x]), "engine: operation %d (call) names buffer %d, there are %d", i,
+                              o.extra[x], p->n_buffers);
+                    E_REQUIRE(-1, o.extra[x] == -1 || p->buffers[o.extra[x]].rows == PICOLM_ROWS_STEP || o.rows == PICOLM_ROWS_WANTED,
+                              "engine: operation %d (call) over every row names a buffer of the wanted rows", i);
+                }
+                E_REQUIRE(-1, out.rows == o.rows, "engine: operation %d (call) writes a buffer of other rows than it covers", i);
+                E_REQUIRE(-1, o.in == -1 || p->buffers[o.in].rows == PICOLM_ROWS_STEP || o.rows == PICOLM_ROWS_WANTED,
+                          "engine: operation %d (call) over every row reads a buffer of the wanted rows", i);
+                if (o.call_flags & PICOLM_CALL_KV) {
+                    E_REQUIRE(-1, o.kv_group >= 0 && o.kv_group < p->n_kv_groups && o.kv_entry >= 0 &&
+                                      o.kv_entry < p->kv_groups[o.kv_group].n_entries && o.rows == PICOLM_ROWS_STEP,
+                              "engine: operation %d (call): cache entry (%d, %d)", i, o.kv_group, o.kv_entry);
+                } else {
+                    E_REQUIRE(-1, !(o.call_flags & PICOLM_CALL_ATTENDS), "engine: operation %d (call) wants a work list without a cache entry", i);
+                }
+                if (o.call_flags & PICOLM_CALL_STATE)
+                    E_REQUIRE(-1, o.state_group >= 0 && o.state_group < p->n_state_groups && o.state_entry >= 0 &&
+                                      o.state_entry < p->state_groups[o.state_group].n_entries,
+                              "engine: operation %d (call): state entry (%d, %d)", i, o.state_group, o.state_entry);
+                E_REQUIRE(-1, o.tile_rows >= 0 && o.partial_floats >= 0, "engine: operation %d (call): tile_rows %d, partial_floats %d", i,
+                          o.tile_rows, o.partial_floats);
                 break;
             }
             default: E_REQUIRE(-1, false, "engine: operation %d has unknown kind %d", i, o.kind);
@@ -492,20 +557,22 @@ extern "C" int picolm_engine_create(const picolm_program* program, int64_t max_t
     for (int gi = 0; gi < program->n_kv_groups; ++gi) {
         KVGroup& g = e->kv[gi];
         g.spec = program->kv_groups[gi];
-        E_REQUIRE(-1, g.spec.n_entries > 0 && g.spec.n_kv_heads > 0 && g.spec.head_dim > 0 && g.spec.window == 0,
-                  "engine: cache group %d is ill-formed (this engine keeps all keys, no windows)", gi);
-        E_REQUIRE(-1, g.spec.v_head_dim == 0 || g.spec.v_head_dim == g.spec.head_dim,
-                  "engine: cache group %d has keys of %d and values of %d: the attention operation takes one size for both", gi,
-                  g.spec.head_dim, g.spec.v_head_dim);
-        g.max_pages = g.ring_pages = e->max_pages;
-        g.n_pages = (int)std::min<int64_t>(n_pages, (int64_t)e->n_slots * e->max_pages);
+        E_REQUIRE(-1, g.spec.n_entries > 0 && g.spec.n_kv_heads > 0 && g.spec.head_dim > 0 && g.spec.window >= 0 && g.spec.v_head_dim >= 0,
+                  "engine: cache group %d is ill-formed", gi);
+        g.max_pages = e->max_pages;
+        // a window's ring: the window of the first query of a chunk of new tokens together with the
+        // whole chunk, which is written before its queries are answered
+        g.ring_pages = g.spec.window > 0 ? std::min(pages_for(g.spec.window - 1 + WINDOW_STEP_TOKENS) + 1, e->max_pages) : e->max_pages;
+        g.n_pages = (int)std::min<int64_t>(n_pages, (int64_t)e->n_slots * g.ring_pages);
         g.pool.init(g.n_pages);
         g.pages.assign(e->n_slots, {});
         g.table_host.assign((size_t)e->n_slots * g.max_pages, 0);
-        g.entry_bytes = (size_t)std::max(g.n_pages, 1) * g.spec.n_kv_heads * PAGE_TOKENS * g.spec.head_dim * dt_bytes(e->dtype);
+        const size_t page_rows = (size_t)std::max(g.n_pages, 1) * g.spec.n_kv_heads * PAGE_TOKENS * dt_bytes(e->dtype);
+        g.k_entry_bytes = page_rows * g.spec.head_dim;
+        g.v_entry_bytes = page_rows * g.value_dim();
         if (!e->host_only()) {
-            TRY(dev_alloc(e.get(), (void**)&g.k, g.entry_bytes * g.spec.n_entries, true));
-            TRY(dev_alloc(e.get(), (void**)&g.v, g.entry_bytes * g.spec.n_entries, true));
+            TRY(dev_alloc(e.get(), (void**)&g.k, g.k_entry_bytes * g.spec.n_entries, true));
+            TRY(dev_alloc(e.get(), (void**)&g.v, g.v_entry_bytes * g.spec.n_entries, true));
             TRY(dev_alloc(e.get(), (void**)&g.table_dev, g.table_host.size() * 4, true));
         }
     }
@@ -519,7 +586,22 @@ extern "C" int picolm_engine_create(const picolm_program* program, int64_t max_t
     }
     e->group_written.assign(e->kv.size(), 0);
     e->group_attended.assign(e->kv.size(), 0);
+    e->recordable = true;
     for (const picolm_op& o : e->ops) {
+        if (o.kind == PICOLM_OP_CALL) {
+            if (!(o.call_flags & PICOLM_CALL_RECORDABLE)) e->recordable = false;
+            if (!(o.call_flags & PICOLM_CALL_KV)) continue;
+            const KVGroup& g = e->kv[o.kv_group];
+            if (o.kv_writes) e->group_written[o.kv_group] = 1;
+            if (!(o.call_flags & PICOLM_CALL_ATTENDS)) continue;
+            e->group_attended[o.kv_group] = 1;
+            if (o.tile_rows > 0) add_unique(e->tile_rows, o.tile_rows);
+            e->decode_blocks_per_chunk = std::max(e->decode_blocks_per_chunk, g.spec.n_kv_heads);
+            e->decode_max_pages_per_chunk = std::min(e->decode_max_pages_per_chunk, 16);
+            e->counters_needed = std::max(e->counters_needed, e->n_slots * g.spec.n_kv_heads * 4);
+            e->partial_floats_per_seq_chunk = std::max(e->partial_floats_per_seq_chunk, (size_t)o.partial_floats);
+            continue;
+        }
         if (o.kind != PICOLM_OP_ATTENTION) continue;
         E_REQUIRE(-1, !o.cos_table || o.table_positions >= e->max_seq_len,
                   "engine: rotation tables for %d positions, the cache takes sequences of %d", o.table_positions, e->max_seq_len);
@@ -549,19 +631,23 @@ static void free_workspace(Workspace& w) {
     w.counters = nullptr;
 }
 
+static void free_decode_graph(picolm_engine* e, DecodeGraph& g) {
+    if (g.exec) (void)hipGraphExecDestroy(g.exec);
+    if (g.batch.dev) {
+        (void)hipFree(g.batch.dev);
+        e->device_bytes -= g.batch.plan.ints.size() * 4;
+    }
+    for (int t = 0; t < 2; ++t) {
+        if (g.batch.pinned[t]) (void)hipHostFree(g.batch.pinned[t]);
+        if (g.batch.sent[t]) (void)hipEventDestroy(g.batch.sent[t]);
+    }
+}
+
 extern "C" void picolm_engine_destroy(picolm_engine* e) {
     if (!e) return;
     if (!e->host_only()) (void)hipDeviceSynchronize();
-    for (auto& kvp : e->graphs) {
-        DecodeGraph& g = *kvp.second;
-        if (g.exec) (void)hipGraphExecDestroy(g.exec);
-        free_workspace(g.ws);
-        if (g.batch.dev) (void)hipFree(g.batch.dev);
-        for (int t = 0; t < 2; ++t) {
-            if (g.batch.pinned[t]) (void)hipHostFree(g.batch.pinned[t]);
-            if (g.batch.sent[t]) (void)hipEventDestroy(g.batch.sent[t]);
-        }
-    }
+    for (auto& kvp : e->graphs) free_decode_graph(e, *kvp.second);
+    free_workspace(e->decode_ws);
     for (KVGroup& g : e->kv) {
         if (g.k) (void)hipFree(g.k);
         if (g.v) (void)hipFree(g.v);
@@ -683,6 +769,31 @@ static void plan_write_pages(picolm_engine* e, StepPlan& p, const std::vector<in
     }
 }
 
+// The tiles of `rpt` new tokens of a prefill step (or of a slice of one), sorted by the keys a tile
+// sees: the kernels hand out the longest first.
+static TileList plan_tiles(StepPlan& p, const std::vector<int>& pos0, const std::vector<int>& n_new, int rpt) {
+    struct Tile {
+        int keys, seq, q0;
+    };
+    std::vector<Tile> tiles;
+    for (int i = 0; i < (int)n_new.size(); ++i)
+        for (int q0 = 0; q0 < n_new[i]; q0 += rpt) tiles.push_back({pos0[i] + std::min(q0 + rpt, n_new[i]), i, q0});
+    std::sort(tiles.begin(), tiles.end(), [](const Tile& a, const Tile& b) {
+        return a.keys != b.keys ? a.keys < b.keys : a.seq != b.seq ? a.seq < b.seq : a.q0 < b.q0;
+    });
+    std::vector<int32_t> seqs, q0s;
+    for (auto& t : tiles) {
+        seqs.push_back(t.seq);
+        q0s.push_back(t.q0);
+    }
+    TileList tl;
+    tl.rows_per_tile = rpt;
+    tl.n = (int)tiles.size();
+    tl.seq = put(p, seqs);
+    tl.q0 = put(p, q0s);
+    return tl;
+}
+
 // Builds the index arrays of a step that is not a recorded decode step.  The sequences and their
 // tokens have been checked, and the pages reserved.
 static void plan_step(picolm_engine* e, StepPlan& p, const std::vector<int>& slots, const std::vector<int>& pos0,
@@ -722,35 +833,44 @@ static void plan_step(picolm_engine* e, StepPlan& p, const std::vector<int>& slo
         for (size_t gi = 0; gi < e->kv.size(); ++gi) {
             if (!e->group_attended[gi]) continue;
             int n = 0;
-            for (int q : pos0) n += (q / PAGE_TOKENS + 1 + p.pages_per_chunk - 1) / p.pages_per_chunk;
+            for (int q : pos0) n += chunks_of(e->kv[gi], q, p.pages_per_chunk);
             DecodeList& l = p.lists[gi];
             l.span.n = 8 * (n + 1);
             l.span.off = p.take(l.span.n);
             l.n_chunks = fill_chunk_list(&p.ints[l.span.off], slots, pos0, p.pages_per_chunk, e->kv[gi], &l.most);
         }
     } else {
-        for (int rpt : e->tile_rows) {
-            struct Tile {
-                int keys, seq, q0;
-            };
-            std::vector<Tile> tiles;
-            for (int i = 0; i < p.n_seq; ++i)
-                for (int q0 = 0; q0 < n_new[i]; q0 += rpt) tiles.push_back({pos0[i] + std::min(q0 + rpt, n_new[i]), i, q0});
-            // by the keys a tile sees: the kernels hand out the longest first
-            std::sort(tiles.begin(), tiles.end(), [](const Tile& a, const Tile& b) {
-                return a.keys != b.keys ? a.keys < b.keys : a.seq != b.seq ? a.seq < b.seq : a.q0 < b.q0;
-            });
-            std::vector<int32_t> seqs, q0s;
-            for (auto& t : tiles) {
-                seqs.push_back(t.seq);
-                q0s.push_back(t.q0);
+        for (int rpt : e->tile_rows) p.tiles.push_back(plan_tiles(p, pos0, n_new, rpt));
+        bool rings = false;
+        for (size_t gi = 0; gi < e->kv.size(); ++gi) rings = rings || (e->group_attended[gi] && e->kv[gi].is_ring());
+        if (rings && p.max_new > WINDOW_STEP_TOKENS) {
+            // the step cut along positions: chunk c holds, of every sequence that has them, its new
+            // tokens c * 256 .. c * 256 + 255
+            for (int lo = 0; lo < p.max_new; lo += WINDOW_STEP_TOKENS) {
+                WindowChunk c;
+                std::vector<int32_t> sl, ps, nn, first, rows;
+                std::vector<int> cpos, cnew;
+                for (int i = 0; i < p.n_seq; ++i) {
+                    if (n_new[i] <= lo) continue;
+                    const int n = std::min(WINDOW_STEP_TOKENS, n_new[i] - lo);
+                    sl.push_back(slots[i]);
+                    ps.push_back(pos0[i] + lo);
+                    nn.push_back(n);
+                    first.push_back(cu[i] + lo);
+                    cpos.push_back(pos0[i] + lo);
+                    cnew.push_back(n);
+                    for (int j = 0; j < n; ++j) rows.push_back(cu[i] + lo + j);
+                }
+                c.n_seq = (int)sl.size();
+                c.n_rows = (int)rows.size();
+                c.seq_slot = put(p, sl);
+                c.seq_pos0 = put(p, ps);
+                c.seq_nnew = put(p, nn);
+                c.first_row = put(p, first);
+                c.rows = put(p, rows);
+                for (int rpt : e->tile_rows) c.tiles.push_back(plan_tiles(p, cpos, cnew, rpt));
+                p.window_chunks.push_back(c);
             }
-            TileList tl;
-            tl.rows_per_tile = rpt;
-            tl.n = (int)tiles.size();
-            tl.seq = put(p, seqs);
-            tl.q0 = put(p, q0s);
-            p.tiles.push_back(tl);
         }
     }
 }
@@ -773,7 +893,7 @@ static int upload_plan(picolm_engine* e, StepPlan& p, hipStream_t stream) {
 }
 
 // ---- recorded decode steps: the block that stays in place --------------------------------------
-static int decode_batch_init(picolm_engine* e, DecodeBatch& b, int n_seq, int ppc) {
+static int decode_batch_init(picolm_engine* e, DecodeBatch& b, int n_seq, int ppc, int most_chunks) {
     StepPlan& p = b.plan;
     p = StepPlan();
     p.n_seq = p.T = p.n_want = n_seq;
@@ -797,10 +917,11 @@ static int decode_batch_init(picolm_engine* e, DecodeBatch& b, int n_seq, int pp
     for (size_t gi = 0; gi < e->kv.size(); ++gi) {
         if (e->group_written[gi]) p.write_pages[gi] = put(p, zeros);
         if (e->group_attended[gi]) {
-            // a list of fixed capacity: every sequence at the cache's full length; entries not in
-            // use hold what an earlier step left, and the header says how many are
+            // a list of fixed capacity: every sequence with `most_chunks` chunks (or as many as the
+            // group's pages make); entries not in use hold what an earlier step left, and the
+            // header says how many are
             DecodeList& l = p.lists[gi];
-            l.most = (e->kv[gi].max_pages + ppc - 1) / ppc;
+            l.most = std::min(most_chunks, (e->kv[gi].ring_pages + ppc - 1) / ppc);
             l.n_chunks = n_seq * l.most;
             l.span.n = 8 * (l.n_chunks + 1);
             l.span.off = p.take(l.span.n);
@@ -843,11 +964,16 @@ static int decode_batch_fill(picolm_engine* e, DecodeBatch& b, const std::vector
         DecodeList& l = p.lists[gi];
         if (l.span.n) {
             int32_t* list = &p.ints[l.span.off];
-            if (same_pages) {
+            if (same_pages && g.spec.window == 0) {        // (a window's first page can move on any step)
                 for (int x = 0; x < b.live[gi]; ++x) list[8 * (x + 1) + 2] += 1;
             } else {
                 int chunks = 0;
-                for (int q : pos0) chunks += (q / PAGE_TOKENS + 1 + p.pages_per_chunk - 1) / p.pages_per_chunk;
+                for (int q : pos0) {
+                    E_REQUIRE(PICOLM_ERR_STEP, chunks_of(g, q, p.pages_per_chunk) <= l.most,
+                              "a decode step's work list was laid out for %d chunks a sequence, one needs %d", l.most,
+                              chunks_of(g, q, p.pages_per_chunk));
+                    chunks += chunks_of(g, q, p.pages_per_chunk);
+                }
                 E_REQUIRE(PICOLM_ERR_STEP, chunks <= l.n_chunks, "a decode step's work list holds %d chunks, %d are needed", l.n_chunks, chunks);
                 int most = 0;
                 b.live[gi] = fill_chunk_list(list, slots, pos0, p.pages_per_chunk, g, &most);
@@ -905,6 +1031,7 @@ static int workspace_ensure(picolm_engine* e, Workspace& w, const StepPlan& p, i
         w.cap = align_up(off + off / 8, 1 << 16);
         HIP_TRY(hipMalloc((void**)&w.base, w.cap));
         e->device_bytes += w.cap;
+        w.generation++;
     }
     w.for_T = p.T;
     w.for_want = p.n_want;
@@ -968,6 +1095,7 @@ static int run_linear(Run& r, const picolm_op& o) {
     TRY(picolm_linear(a, a_dt, o.weight, o.weight_dt, c, bo.dtype, M, o.n, o.k, o.epilogue, next_w, next_h, next_ssq, next_parts, ssq,
                       n_parts, norm_len, eps, e->splitk_ws, r.stream));
     if (next_w) {
+        r.prepared.by = &o;
         r.prepared.x = c;
         r.prepared.w = o.out_norm_weight;
         r.prepared.eps = o.out_norm_eps;
@@ -988,8 +1116,8 @@ static int run_attention(Run& r, const picolm_op& o) {
     const float* qkv = (const float*)r.buf(o.in);
     void* q = r.buf(o.q_buffer);
     void* out = r.buf(o.out);
-    char* k_pages = g.k + (size_t)o.kv_entry * g.entry_bytes;
-    char* v_pages = g.v + (size_t)o.kv_entry * g.entry_bytes;
+    char* k_pages = g.k + (size_t)o.kv_entry * g.k_entry_bytes;
+    char* v_pages = g.v + (size_t)o.kv_entry * g.v_entry_bytes;
     const bool writes = o.kv_writes != 0;
     const int32_t* tok_page = writes ? p.at(p.write_pages[o.kv_group]) : nullptr;
     const bool mfma = attn_on_matrix_cores(e, d);
@@ -1011,7 +1139,26 @@ static int run_attention(Run& r, const picolm_op& o) {
                                           l.most, p.at(p.seq_pos0), g.table_dev, g.max_pages, g.ring_pages, H, G, d, o.window, o.scale,
                                           r.stream);
     }
-    const TileList* tl = p.tiles_of(mfma ? picolm_attn_prefill_mfma_tile_tokens(H, G) : picolm_attn_prefill_tile_rows());
+    const int tile_rows = mfma ? picolm_attn_prefill_mfma_tile_tokens(H, G) : picolm_attn_prefill_tile_rows();
+    if (g.is_ring() && !p.window_chunks.empty()) {
+        // a ring holds a window and one chunk of new tokens: write and answer the step chunk by chunk
+        for (const WindowChunk& c : p.window_chunks) {
+            const TileList* ct = c.tiles_of(tile_rows);
+            E_REQUIRE(-1, ct != nullptr, "attention: the step has no tiles of the height this kernel takes");
+            TRY(picolm_rope_kv_store(qkv, q, writes ? k_pages : nullptr, writes ? v_pages : nullptr, dt, o.cos_table, o.sin_table,
+                                     o.rope_style, p.at(p.tok_pos), tok_page, c.n_rows, H, G, d, p.at(c.rows), r.stream));
+            if (mfma)
+                TRY(picolm_attn_prefill_mfma(q, k_pages, v_pages, out, p.at(ct->seq), p.at(ct->q0), ct->n, p.at(c.seq_slot), p.at(c.seq_pos0),
+                                             p.at(c.seq_nnew), p.at(c.first_row), g.table_dev, g.max_pages, g.ring_pages, H, G, d, o.window,
+                                             o.scale, r.stream));
+            else
+                TRY(picolm_attn_prefill_generic(q, k_pages, v_pages, out, dt, p.at(ct->seq), p.at(ct->q0), ct->n, p.at(c.seq_slot),
+                                                p.at(c.seq_pos0), p.at(c.seq_nnew), p.at(c.first_row), g.table_dev, g.max_pages,
+                                                g.ring_pages, H, G, d, o.window, o.scale, r.stream));
+        }
+        return 0;
+    }
+    const TileList* tl = p.tiles_of(tile_rows);
     E_REQUIRE(-1, tl != nullptr, "attention: the step has no tiles of the height this kernel takes");
     if (mfma && picolm_attn_prefill_rotates_q(p.T)) {      // keys and values go to the cache; the attention kernel rotates q on its way in
         if (writes)
@@ -1031,6 +1178,92 @@ static int run_attention(Run& r, const picolm_op& o) {
     return picolm_attn_prefill_generic(q, k_pages, v_pages, out, dt, p.at(tl->seq), p.at(tl->q0), tl->n, p.at(p.seq_slot),
                                        p.at(p.seq_pos0), p.at(p.seq_nnew), p.at(p.cu_seqlens), g.table_dev, g.max_pages, g.ring_pages, H,
                                        G, d, o.window, o.scale, r.stream);
+}
+
+// An operation of the caller's: it is handed what the engine knows of the step and queues its own
+// work on the step's stream (picolm's layer loop branches per layer kind in C instead,
+// picolm/model_core.c:1824-1839).
+static int run_call(Run& r, const picolm_op& o) {
+    picolm_engine* e = r.e;
+    const StepPlan& p = r.p;
+    picolm_step_view v;
+    memset(&v, 0, sizeof(v));
+    v.struct_bytes = (int32_t)sizeof(v);
+    v.dtype = e->dtype;
+    v.n_seq = p.n_seq;
+    v.n_tokens = p.T;
+    v.n_wanted = p.n_want;
+    v.is_decode = p.is_decode;
+    v.every_row_wanted = p.every_row;
+    v.recording = r.stream == e->capture_stream && e->capture_stream != nullptr;
+    v.slots = p.slots.data();
+    v.pos0 = p.pos0.data();
+    v.n_new = p.n_new.data();
+    v.seq_slot = p.at(p.seq_slot);
+    v.seq_pos0 = p.at(p.seq_pos0);
+    v.seq_nnew = p.at(p.seq_nnew);
+    v.cu_seqlens = p.at(p.cu_seqlens);
+    v.tok_pos = p.at(p.tok_pos);
+    v.tok_seq = p.at(p.tok_seq);
+    v.tokens = p.at(p.tokens);
+    v.want_rows = p.at(p.want_rows);
+    v.rows = o.rows == PICOLM_ROWS_STEP ? p.T : p.n_want;
+    if (o.in >= 0) {
+        v.in = r.buf(o.in);
+        v.in_row_bytes = e->buffers[o.in].row_bytes;
+    }
+    v.out = r.buf(o.out);
+    v.out_row_bytes = e->buffers[o.out].row_bytes;
+    for (int x = 0; x < 4; ++x)
+        if (o.extra[x] >= 0) {
+            v.extra[x] = r.buf(o.extra[x]);
+            v.extra_row_bytes[x] = e->buffers[o.extra[x]].row_bytes;
+        }
+    if (o.call_flags & PICOLM_CALL_KV) {
+        const KVGroup& g = e->kv[o.kv_group];
+        v.k_pages = g.k + (size_t)o.kv_entry * g.k_entry_bytes;
+        v.v_pages = g.v + (size_t)o.kv_entry * g.v_entry_bytes;
+        v.page_table = g.table_dev;
+        v.n_pages = std::max(g.n_pages, 1);
+        v.max_pages = g.max_pages;
+        v.ring_pages = g.ring_pages;
+        v.n_kv_heads = g.spec.n_kv_heads;
+        v.head_dim = g.spec.head_dim;
+        v.v_head_dim = g.value_dim();
+        v.window = g.spec.window;
+        v.kv_writes = o.kv_writes;
+        if (o.kv_writes) v.write_pages = p.at(p.write_pages[o.kv_group]);
+        if (o.call_flags & PICOLM_CALL_ATTENDS) {
+            if (p.is_decode) {
+                const DecodeList& l = p.lists[o.kv_group];
+                v.chunk_list = p.at(l.span);
+                v.n_chunks = l.n_chunks;
+                v.pages_per_chunk = p.pages_per_chunk;
+                v.most_chunks = l.most;
+                v.partial = l.most > 1 && o.partial_floats ? (float*)(r.w.base + r.w.partial) : nullptr;
+                v.counters = r.w.counters;
+            } else if (o.tile_rows > 0) {
+                const TileList* tl = p.tiles_of(o.tile_rows);
+                E_REQUIRE(-1, tl != nullptr, "call: the step has no tiles of %d rows", o.tile_rows);
+                v.tile_seq = p.at(tl->seq);
+                v.tile_q0 = p.at(tl->q0);
+                v.n_tiles = tl->n;
+                v.tile_rows = o.tile_rows;
+            }
+        }
+    }
+    if (o.call_flags & PICOLM_CALL_STATE) {
+        const StateGroup& sg = e->state[o.state_group];
+        v.state = sg.data + (size_t)o.state_entry * e->n_slots * sg.spec.bytes_per_slot;
+        v.state_bytes_per_slot = sg.spec.bytes_per_slot;
+    }
+    v.n_slots = e->n_slots;
+    v.stream = r.stream;
+    const int rc = o.call(o.call_user, &v);
+    if (rc == 0) return 0;
+    return rc == PICOLM_ERR_STEP || rc == PICOLM_ERR_CACHE_FULL || rc == PICOLM_ERR_CACHE || rc == PICOLM_ERR_DEVICE || rc == -1 || rc == -2
+               ? rc
+               : PICOLM_ERR_STEP;
 }
 
 // embedding -> the layer calls -> final norm on the wanted rows -> head
@@ -1065,7 +1298,12 @@ static int run_program(picolm_engine* e, const StepPlan& p, Workspace& w, hipStr
             }
             case PICOLM_OP_LINEAR: TRY(run_linear(r, o)); break;
             case PICOLM_OP_ATTENTION: TRY(run_attention(r, o)); break;
+            case PICOLM_OP_CALL: TRY(run_call(r, o)); break;
         }
+        // what a product prepared of a norm holds for the rows as they were: whoever writes them since
+        // (any operation but the product that just prepared it) makes it stale
+        if (r.prepared.x == r.buf(o.out) && !(o.kind == PICOLM_OP_LINEAR && r.prepared.by == &o)) r.prepared = Prepared();
+        if (o.kind == PICOLM_OP_CALL) r.prepared = Prepared();      // (it may write any of its buffers)
         if (e->timing()) {
             hipEvent_t after = nullptr;
             TRY(timing_event(e, &after, stream));
@@ -1115,40 +1353,61 @@ static int decode_step(picolm_engine* e, const std::vector<int>& slots, const st
     TRY(reserve_many(e, slots, lengths));
     TRY(flush_tables(e, stream));
     const int ppc = decode_pages_per_chunk(pos0, e->decode_blocks_per_chunk, e->decode_max_pages_per_chunk);
-    auto& slot = e->graphs[{n, ppc}];
+    // the step's shape: the chunks that the longest sequence needs, rounded up to a power of two, so
+    // that a launch covers what the live contexts need and not what the cache could hold
+    int need = 1, most_chunks = 1;
+    for (size_t gi = 0; gi < e->kv.size(); ++gi)
+        if (e->group_attended[gi])
+            for (int q : pos0) need = std::max(need, chunks_of(e->kv[gi], q, ppc));
+    while (most_chunks < need) most_chunks *= 2;
+    const auto key = std::make_tuple(n, ppc, most_chunks);
+    auto& slot = e->graphs[key];
     if (!slot) {
         slot.reset(new DecodeGraph);
-        const int rc = decode_batch_init(e, slot->batch, n, ppc);
+        const int rc = decode_batch_init(e, slot->batch, n, ppc, most_chunks);
         if (rc) {
-            e->graphs.erase({n, ppc});
+            e->graphs.erase(key);
             return rc;
         }
+        if (e->graphs.size() > MAX_DECODE_SHAPES) {
+            auto oldest = e->graphs.end();
+            for (auto it = e->graphs.begin(); it != e->graphs.end(); ++it)
+                if (it->first != key && (oldest == e->graphs.end() || it->second->last_used < oldest->second->last_used)) oldest = it;
+            if (!e->host_only()) HIP_TRY(hipStreamSynchronize(stream));      // its last step may still read its block
+            free_decode_graph(e, *oldest->second);
+            e->graphs.erase(oldest);
+        }
     }
-    DecodeGraph& g = *slot;
+    DecodeGraph& g = *e->graphs[key];
+    g.last_used = ++e->decode_tick;
     TRY(decode_batch_fill(e, g.batch, slots, pos0, tokens, stream));
     e->last_plan = &g.batch.plan;
     if (!e->host_only()) {
         const StepPlan& p = g.batch.plan;
+        Workspace& ws = e->decode_ws;
         if (tokens_dev)
             HIP_TRY(hipMemcpyAsync(g.batch.dev + p.tokens.off, tokens_dev, (size_t)n * 4, hipMemcpyDeviceToDevice, stream));
         g.uses++;
+        int most = 1;
+        for (auto& l : p.lists) most = std::max(most, l.most);
+        TRY(workspace_ensure(e, ws, p, most));
+        if (g.exec && g.ws_generation != ws.generation) {      // the workspace has moved since the recording
+            (void)hipGraphExecDestroy(g.exec);
+            g.exec = nullptr;
+        }
         if (g.exec) {
             HIP_TRY(hipGraphLaunch(g.exec, stream));
         } else {
-            int most = 1;
-            for (auto& l : p.lists) most = std::max(most, l.most);
-            TRY(workspace_ensure(e, g.ws, p, most));
-            TRY(run_program(e, p, g.ws, stream));
-            g.logits = (float*)(g.ws.base + g.ws.offsets[e->logits_buffer]);
-            if (g.uses >= 2 && !(e->flags & (PICOLM_ENGINE_NO_GRAPHS | PICOLM_ENGINE_TIME_OPS))) {
+            TRY(run_program(e, p, ws, stream));
+            if (g.uses >= 2 && e->recordable && !(e->flags & (PICOLM_ENGINE_NO_GRAPHS | PICOLM_ENGINE_TIME_OPS))) {
                 // the sizes have been seen and the workspace is allocated: record the same launches
                 // (recording runs nothing; this step's result came from the launches above)
                 hipGraph_t graph = nullptr;
-                const int flip = g.ws.flip;
+                const int flip = ws.flip;
                 HIP_TRY(hipStreamBeginCapture(e->capture_stream, hipStreamCaptureModeThreadLocal));
-                const int rc = run_program(e, p, g.ws, e->capture_stream);
+                const int rc = run_program(e, p, ws, e->capture_stream);
                 const hipError_t end = hipStreamEndCapture(e->capture_stream, &graph);
-                g.ws.flip = flip;
+                ws.flip = flip;
                 if (rc) {
                     if (graph) (void)hipGraphDestroy(graph);
                     return rc;
@@ -1157,9 +1416,10 @@ static int decode_step(picolm_engine* e, const std::vector<int>& slots, const st
                 const hipError_t inst = hipGraphInstantiate(&g.exec, graph, nullptr, nullptr, 0);
                 (void)hipGraphDestroy(graph);
                 HIP_TRY(inst);
+                g.ws_generation = ws.generation;
             }
         }
-        if (logits) *logits = g.logits;
+        if (logits) *logits = (float*)(ws.base + ws.offsets[e->logits_buffer]);
     }
     for (int i = 0; i < n; ++i) e->slots.length[slots[i]] = pos0[i] + 1;
     return 0;
@@ -1258,8 +1518,8 @@ extern "C" int picolm_engine_kv_entry(picolm_engine* e, int32_t group, int32_t e
     E_REQUIRE(-1, e && group >= 0 && group < (int)e->kv.size(), "kv_entry: no cache group %d", group);
     const KVGroup& g = e->kv[group];
     E_REQUIRE(-1, entry >= 0 && entry < g.spec.n_entries, "kv_entry: group %d has %d entries", group, g.spec.n_entries);
-    if (k) *k = g.k ? g.k + (size_t)entry * g.entry_bytes : nullptr;
-    if (v) *v = g.v ? g.v + (size_t)entry * g.entry_bytes : nullptr;
+    if (k) *k = g.k ? g.k + (size_t)entry * g.k_entry_bytes : nullptr;
+    if (v) *v = g.v ? g.v + (size_t)entry * g.v_entry_bytes : nullptr;
     if (n_pages) *n_pages = std::max(g.n_pages, 1);
     return 0;
 }
@@ -1307,6 +1567,27 @@ extern "C" int picolm_engine_step_array(picolm_engine* e, const char* name, int3
         const int g = atoi(n.c_str() + 7);
         found = g >= 0 && g < (int)p.lists.size() && p.lists[g].span.n > 0;
         if (found) s = p.lists[g].span;
+    } else if (n.rfind("window_chunk.", 0) == 0) {
+        // "window_chunk.<c>.<array>": a slice of a prefill step for the groups that keep a ring
+        const int c = atoi(n.c_str() + 13);
+        const size_t dot = n.find('.', 13);
+        found = c >= 0 && c < (int)p.window_chunks.size() && dot != std::string::npos;
+        if (found) {
+            const WindowChunk& wc = p.window_chunks[c];
+            const std::string what = n.substr(dot + 1);
+            if (what == "seq_slot") s = wc.seq_slot;
+            else if (what == "seq_pos0") s = wc.seq_pos0;
+            else if (what == "seq_nnew") s = wc.seq_nnew;
+            else if (what == "first_row") s = wc.first_row;
+            else if (what == "rows") s = wc.rows;
+            else if (what.rfind("tiles.", 0) == 0) {
+                const TileList* tl = wc.tiles_of(atoi(what.c_str() + 6));
+                found = tl != nullptr;
+                if (found) s = what.find(".seq") != std::string::npos ? tl->seq : tl->q0;
+            } else {
+                found = false;
+            }
+        }
     } else if (n.rfind("tiles.", 0) == 0) {
         const int rows = atoi(n.c_str() + 6);
         const TileList* tl = p.tiles_of(rows);

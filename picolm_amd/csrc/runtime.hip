@@ -15,7 +15,9 @@ void picolm_set_error(const char* fmt, ...) {
 
 extern "C" const char* picolm_last_error(void) { return g_error; }
 
-extern "C" int picolm_abi_version(void) { return 1; }
+extern "C" void picolm_set_error_message(const char* message) { picolm_set_error("%s", message ? message : ""); }
+
+extern "C" int picolm_abi_version(void) { return 2; }
 
 extern "C" int picolm_device_check(void) {
     int dev = 0;

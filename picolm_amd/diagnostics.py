@@ -62,12 +62,28 @@ def gpu_diff(S: int, I: int, O: int, seed: int = 42) -> int:
     return 0 if ok else 1
 
 
+class _OneSequence:
+    """The index arrays of a step that brings one sequence's first n tokens, as the attention
+    kernels read them (the engine plans such arrays for every step)."""
+
+    def __init__(self, n: int, dev):
+        i32 = lambda v: torch.tensor(v, dtype=torch.int32, device=dev)
+        self.n_seq, self.T, self.max_len = 1, n, n
+        self.seq_slot, self.seq_pos0, self.seq_nnew, self.cu_seqlens = i32([0]), i32([0]), i32([n]), i32([0, n])
+        self.tok_pos = torch.arange(n, dtype=torch.int32, device=dev)
+        self._dev = dev
+
+    def prefill_tiles(self, rows_per_tile: int):
+        q0 = list(range(0, self.T, rows_per_tile))          # in the order of the keys they see
+        return (torch.zeros(len(q0), dtype=torch.int32, device=self._dev), torch.tensor(q0, dtype=torch.int32, device=self._dev),
+                len(q0))
+
+
 def gpu_attn_diff(n_tok: int, H: int, G: int, d: int, seed: int = 42) -> int:
     """Causal attention of one sequence of n_tok new tokens over a fresh cache: the bfloat16 kernels
     (matrix cores where the head size allows) and the 32-bit kernels, against float64 on the host."""
     from . import kernels
-    from .cache.slots import PAGE_TOKENS
-    from .engine.batch import StepBatch
+    from .cache import PAGE_TOKENS
     if min(n_tok, H, G, d) < 1 or H % G or d % 2 or d > 256:
         raise SystemExit("--gpu-attn-diff n_tok n_heads n_kv_heads head_dim: heads in whole groups, an even head size up to 256")
     dev = _device()
@@ -79,7 +95,7 @@ def gpu_attn_diff(n_tok: int, H: int, G: int, d: int, seed: int = 42) -> int:
     _say(f"GPU attention diff: {n_tok} tokens, {H} heads on {G} groups of size {d}, seed {seed}")
     outs = {}
     for dtype in (torch.float32, torch.bfloat16):
-        batch = StepBatch([0], [0], [[0] * n_tok], [[]], 1, dev)
+        batch = _OneSequence(n_tok, dev)
         kp = torch.zeros(n_pages, G, PAGE_TOKENS, d, dtype=dtype, device=dev)
         vp = torch.zeros(n_pages, G, d, PAGE_TOKENS, dtype=dtype, device=dev)
         q = torch.zeros(n_tok, H * d, dtype=dtype, device=dev)

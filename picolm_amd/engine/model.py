@@ -1,4 +1,4 @@
-"""A decoder put together from parts, and its one step function.
+"""A decoder put together from parts, and its launch program.
 
 embedding -> the layer calls of `order` -> final norm on the wanted rows -> head
 (picolm/model_core.c:1785, :1799-2210, :2213, :2220).  `order` is data: a list of layer
@@ -15,10 +15,10 @@ from dataclasses import dataclass
 import torch
 
 from .. import kernels
-from ..cache import Cache, CacheSpec, KVGroupSpec, StateGroupSpec
-from ..parts.base import CacheBinding, Runtime, StepContext, Workspace
+from ..cache import CacheSpec, KVGroupSpec, StateGroupSpec
+from ..parts.base import CacheBinding, Runtime, Workspace
 from ..weights import WeightFetcher, check_specs
-from .batch import StepBatch, StepError
+from .errors import StepError
 
 
 @dataclass(frozen=True)
@@ -90,24 +90,6 @@ class DecoderModel:
             [KVGroupSpec(n, k.n_kv_heads, k.head_dim, k.window, k.v_head_dim) for k, n in zip(kv_keys, kv_counts)],
             [StateGroupSpec(n, tuple(k.shape), k.dtype) for k, n in zip(state_keys, state_counts)])
 
-    def graph_safe(self) -> bool:
-        """Whether a decode step's launches depend on device memory only, so that they can be
-        recorded once and replayed."""
-        def safe(p):
-            return getattr(p, "graph_safe", False) and all(safe(c) for c in p.children())
-        return all(safe(p) for p in self.parts())
-
-    def decode_geometry(self, n_seq: int) -> tuple[int, int]:
-        """(workgroups per chunk, most pages a chunk should have) over the mixers that run a
-        decode attention: the widest launch and the tightest limit size the step's work list."""
-        per_chunk, max_pages = 1, 64
-        for b in self.blocks:
-            f = getattr(b.mixer, "decode_geometry", None)
-            if f is not None:
-                p, m = f(self.runtime.dtype, n_seq)
-                per_chunk, max_pages = max(per_chunk, p), min(max_pages, m)
-        return per_chunk, max_pages
-
     # -- weights ----------------------------------------------------------------------------
     def load(self, source, runtime: Runtime) -> "DecoderModel":
         """Check `source` against every declared tensor, then bind."""
@@ -130,70 +112,37 @@ class DecoderModel:
             total += n * size
         return total
 
-    def new_cache(self, max_tokens: int, max_seq_len: int | None = None, n_slots: int | None = None) -> Cache:
-        limit = getattr(self.config, "max_position_embeddings", None) or max_tokens
-        max_seq_len = min(max_seq_len or limit, limit)
-        cache = Cache(self.cache_spec, max_tokens, max_seq_len, self.runtime.dtype, self.runtime.device, n_slots)
+    def prepare(self, max_positions: int) -> None:
+        """Let the mixers lay out what depends on the longest sequence (rotary tables)."""
         for b in self.blocks:
-            b.mixer.prepare(self.runtime, cache.max_seq_len)
-        return cache
+            b.mixer.prepare(self.runtime, max_positions)
 
     # -- the model as a launch program --------------------------------------------------------
     def program(self):
         """The model as the flat list of operations that the engine in the library walks
-        (engine/program.py), or None when a part has no such operations: then `step` below runs
-        it part by part.  The mixers must have been prepared (`new_cache` does that) for the
-        positions the engine will see."""
-        from .program import CannotEmit, ProgramBuilder
+        (engine/program.py): embedding -> the layer calls of `order` -> final norm on the wanted
+        rows -> head.  Every part emits what it is: operations of the engine's own, or a call of its
+        `forward`.  The mixers must have been prepared (`prepare`) for the positions the engine
+        will see."""
+        from .program import ROWS_WANTED, ProgramBuilder
+        from ..parts.block import norm_ref_of
         if self.runtime is None:
             raise StepError("the model has no weights loaded")
+        ws = Workspace(self.runtime.device)
+        for part in self.parts():
+            part.bind_runtime(self.runtime, ws)
         b = ProgramBuilder(self.runtime.dtype)
-        try:
-            for part in (self.embedding, self.head, *self.blocks):
-                if not callable(getattr(part, "emit", None)):
-                    raise CannotEmit(f"{type(part).__name__} has no operations of the engine's")
-            final = self.final_norm.norm_ref() if hasattr(self.final_norm, "norm_ref") else None
-            if final is None:
-                raise CannotEmit(f"{type(self.final_norm).__name__} has no operations of the engine's")
-            x = self.embedding.emit(b)
-            for i, (call, binding) in enumerate(zip(self.order, self.bindings)):
-                b.binding = binding
-                if i + 1 < len(self.order):
-                    nxt = getattr(self.blocks[self.order[i + 1].block], "first_norm", lambda: None)()
-                    after = nxt.norm_ref() if nxt is not None and hasattr(nxt, "norm_ref") else None
-                    self.blocks[call.block].emit(b, x, after, 0)
-                else:       # the final norm meets every row only in steps that want every row's logits
-                    self.blocks[call.block].emit(b, x, final, 1)
-            b.binding = None
-            self.head.emit(b, final, x)
-        except CannotEmit:
-            return None
-        return b.finish(self.head.V, self.cache_spec)
-
-    # -- the step ---------------------------------------------------------------------------
-    def step(self, cache: Cache, batch: StepBatch, workspace: Workspace) -> torch.Tensor:
-        """Run the batch's new tokens from the cache; logits [n_want, vocab] float32, a view
-        of workspace memory valid until the next step."""
-        ctx = StepContext(self.runtime, batch, cache, workspace)
-        x = self.embedding.forward(ctx, batch.tokens, batch.T)
-        # a block is told which norm meets the residual stream after it (the next block's first one,
-        # or the final norm when every row's logits are wanted), so that its last product can
-        # prepare that norm (see NormedRows)
-        every_row = getattr(batch, "wants_every_row", False)
+        x = self.embedding.emit(b)
         for i, (call, binding) in enumerate(zip(self.order, self.bindings)):
-            ctx.binding = binding
-            block = self.blocks[call.block]
+            b.binding = binding
+            # a block is told which norm meets the residual stream after it (the next block's first
+            # one, or the final norm when every row's logits are wanted), so that its last product
+            # can prepare that norm
             if i + 1 < len(self.order):
-                after = getattr(self.blocks[self.order[i + 1].block], "first_norm", lambda: None)()
+                nxt = self.blocks[self.order[i + 1].block].first_norm()
+                self.blocks[call.block].emit(b, x, norm_ref_of(nxt) if nxt is not None else None, 0)
             else:
-                after = self.final_norm if every_row and batch.n_want else None
-            ctx.norm_after_block = after
-            block.forward(ctx, x)
-        if batch.n_want == 0:
-            return workspace.get("logits", (0, self.head.V), torch.float32)
-        if every_row:
-            h = ctx.normed(self.final_norm, x, self.head)
-        else:
-            ctx.prepared_norm = None
-            h = self.final_norm.forward(ctx, x, rows=batch.want_rows, n_rows=batch.n_want, out_name="norm.final")
-        return self.head.forward(ctx, h)
+                self.blocks[call.block].emit(b, x, norm_ref_of(self.final_norm), 1)
+        b.binding = None
+        self.head.emit(b, self.final_norm.emit(b, x, ROWS_WANTED))
+        return b.finish(self.head.V, self.cache_spec)

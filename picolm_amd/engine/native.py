@@ -12,9 +12,10 @@ import numpy as np
 import torch
 
 from .. import kernels
-from ..cache.slots import CacheError, CacheFull
+from ..cache import CacheError, CacheFull, window_ring_pages
+from ..kernels import device_view
 from . import program as P
-from .batch import StepError
+from .errors import StepError
 
 _declared = False
 
@@ -28,7 +29,11 @@ def _lib():
     return lib
 
 
-def _raise(rc: int):
+def _raise(rc: int, failures=None):
+    if failures:            # a called Python operation raised: that exception, not its summary
+        exc = failures.pop()
+        del failures[:]
+        raise exc
     msg = kernels.lib().picolm_last_error().decode("utf-8", "replace")
     if rc == P.ERR_STEP:
         raise StepError(msg)
@@ -37,22 +42,6 @@ def _raise(rc: int):
     if rc == P.ERR_CACHE:
         raise CacheError(msg)
     raise kernels.KernelError(msg)
-
-
-class _DeviceMemory:
-    """Memory that the library owns, for torch to look at (never to free)."""
-
-    def __init__(self, ptr: int, nbytes: int):
-        self.__cuda_array_interface__ = {"shape": (nbytes,), "typestr": "|u1", "data": (ptr, False), "version": 2}
-
-
-def device_view(ptr: int, shape, dtype: torch.dtype, device) -> torch.Tensor:
-    n = dtype.itemsize
-    for s in shape:
-        n *= int(s)
-    if n == 0 or not ptr:
-        return torch.empty(tuple(shape), dtype=dtype, device=device)
-    return torch.as_tensor(_DeviceMemory(ptr, n), device=device).view(dtype).view(*shape)
 
 
 def _i32(values) -> np.ndarray:
@@ -83,8 +72,9 @@ class _KVEntries:
             _raise(rc)
         G, d = spec.n_kv_heads, spec.head_dim
         self.spec = spec
-        self.k = device_view(k.value, (spec.n_entries, n.value, G, kernels.PAGE_TOKENS, d), dtype, device)
-        self.v = device_view(v.value, (spec.n_entries, n.value, G, d, kernels.PAGE_TOKENS), dtype, device)
+        self.ring_pages = min(window_ring_pages(spec.window), engine.info(5)) if spec.window > 0 else engine.info(5)
+        self.k = device_view(k.value, (spec.n_entries, n.value, G, kernels.PAGE_TOKENS, d), dtype, device, engine._handle)
+        self.v = device_view(v.value, (spec.n_entries, n.value, G, spec.value_dim, kernels.PAGE_TOKENS), dtype, device, engine._handle)
 
 
 class EngineCache:
@@ -100,6 +90,15 @@ class EngineCache:
         self.max_pages = engine.info(5)
         self.slots = _SlotCount(engine)
         self.kv = [_KVEntries(engine, gi, g, dtype, device) for gi, g in enumerate(cache_spec.kv_groups)]
+        self.state = [self._state_entries(gi, g) for gi, g in enumerate(cache_spec.state_groups)]
+
+    def _state_entries(self, group: int, spec) -> torch.Tensor:
+        """[entry][slot][...] of one state group, as the library keeps it."""
+        ptr, nbytes = c_void_p(), c_int64()
+        rc = _lib().picolm_engine_state_entry(self._e.handle, group, 0, byref(ptr), byref(nbytes))
+        if rc:
+            _raise(rc)
+        return device_view(ptr.value, (spec.n_entries, self.n_slots, *spec.shape), spec.dtype, self.device, self._e._handle)
 
     def length(self, slot: int) -> int:
         return max(self._e.length(slot), 0)
@@ -115,6 +114,25 @@ class EngineCache:
         return self._e.info(7)
 
 
+class _Handle:
+    """Owns the engine in the library.  Tensors over the engine's memory keep it (and so that
+    memory) alive: logits or a cache view that outlive their session stay readable."""
+
+    def __init__(self, value):
+        self.value = value
+
+    def close(self) -> None:
+        if self.value:
+            _lib().picolm_engine_destroy(self.value)
+            self.value = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+
 class NativeEngine:
     def __init__(self, built: P.BuiltProgram, max_tokens: int, max_seq_len: int, n_slots: int | None, device,
                  graphs: bool = True, host_only: bool = False, time_ops: bool = False):
@@ -127,23 +145,21 @@ class NativeEngine:
                                          byref(h))
         if rc:
             _raise(rc)
-        self.handle = h
+        self._handle = _Handle(h)
         self.host_only = host_only
         self._views: dict = {}
 
     def _stream(self):
         return None if self.host_only else kernels._stream()
 
-    def close(self) -> None:
-        if getattr(self, "handle", None):
-            _lib().picolm_engine_destroy(self.handle)
-            self.handle = None
+    @property
+    def handle(self):
+        return self._handle.value
 
-    def __del__(self):
-        try:
-            self.close()
-        except Exception:
-            pass
+    def close(self) -> None:
+        """Destroys the engine now; tensors over its memory must not be used afterwards."""
+        self._views.clear()
+        self._handle.close()
 
     # -- books -----------------------------------------------------------------------------
     def info(self, what: int) -> int:
@@ -174,6 +190,21 @@ class NativeEngine:
     def free_pages(self, group: int) -> int:
         return _lib().picolm_engine_free_pages(self.handle, group)
 
+    def kv_pages(self, group: int) -> int:
+        """Pages that a cache group has in all."""
+        n = c_int64()
+        rc = _lib().picolm_engine_kv_entry(self.handle, group, 0, None, None, byref(n))
+        if rc:
+            _raise(rc)
+        return n.value
+
+    def state_bytes_per_slot(self, group: int) -> int:
+        n = c_int64()
+        rc = _lib().picolm_engine_state_entry(self.handle, group, 0, None, byref(n))
+        if rc:
+            _raise(rc)
+        return n.value
+
     def recorded_steps(self) -> int:
         return self.info(4)
 
@@ -200,7 +231,7 @@ class NativeEngine:
         if t is None:
             if len(self._views) >= 256:
                 self._views.clear()
-            t = self._views[key] = device_view(ptr, (rows, self.vocab_size), torch.float32, self.device)
+            t = self._views[key] = device_view(ptr, (rows, self.vocab_size), torch.float32, self.device, self._handle)
         return t
 
     def step(self, slots, new_tokens, want=None) -> torch.Tensor | None:
@@ -226,7 +257,7 @@ class NativeEngine:
                                        counts.ctypes.data if counts is not None else None,
                                        idx.ctypes.data if idx is not None else None, byref(logits), byref(rows), self._stream())
         if rc:
-            _raise(rc)
+            _raise(rc, self.program.failures)
         if not logits.value:
             return None if rows.value else torch.empty((0, self.vocab_size), dtype=torch.float32, device=self.device)
         return self._logits(logits.value, rows.value)
@@ -237,7 +268,7 @@ class NativeEngine:
         rc = _lib().picolm_engine_step_device_tokens(self.handle, len(sl), sl.ctypes.data, tokens.data_ptr(), byref(logits),
                                                      kernels._stream())
         if rc:
-            _raise(rc)
+            _raise(rc, self.program.failures)
         return self._logits(logits.value, len(sl))
 
     def generate(self, prompts, max_new_tokens: int, params, stop_ids=(), batch_size: int = 64,
@@ -259,6 +290,6 @@ class NativeEngine:
                                            stops.ctypes.data, len(stop_ids), int(batch_size), out.ctypes.data, counts.ctypes.data,
                                            finish.ctypes.data, kernels._stream())
         if rc:
-            _raise(rc)
+            _raise(rc, self.program.failures)
         reasons = {0: "", 1: "stop", 2: "length", 3: "capacity"}
         return [out[i, :counts[i]].tolist() for i in range(n)], [reasons[int(f)] for f in finish[:n]]

@@ -223,7 +223,7 @@ def generate(model_or_session, prompts, max_new_tokens: int = 256, params: Sampl
     """
     import torch
 
-    from .cache.slots import PAGE_TOKENS, pages_for
+    from .cache import PAGE_TOKENS, pages_for
     from .engine.session import Session
     from .sampling.sampler import Sampler
     params = params or SamplingParams()
@@ -278,8 +278,8 @@ class SessionStepper:
         self.session.release(slots)
 
     def fits(self, lengths) -> bool:
-        from .cache.slots import PAGE_TOKENS
-        from .cache.slots import pages_for
+        from .cache import PAGE_TOKENS
+        from .cache import pages_for
         c = self.session.cache
         if len(lengths) > c.slots.n_free:
             return False

@@ -33,7 +33,7 @@ def lib():
         for name in dir_entry_points():
             getattr(l, name).restype = c_int
         l.picolm_read_probe_bytes.restype = ctypes.c_size_t
-        if l.picolm_abi_version() != 1:
+        if l.picolm_abi_version() != 2:
             raise KernelError("libpicolm_hip.so has another ABI version; rebuild it")
         _lib = l
     return _lib
@@ -96,6 +96,25 @@ def _i32(name, t, n=None):
     if n is not None and t.numel() < n:
         raise KernelError(f"{name}: holds {t.numel()} entries, {n} are needed")
     return t
+
+
+class _DeviceMemory:
+    """Memory that the library owns, for torch to look at (never to free).  `owner`: whatever must
+    stay alive as long as a tensor over this memory does."""
+
+    def __init__(self, ptr: int, nbytes: int, owner=None):
+        self.__cuda_array_interface__ = {"shape": (nbytes,), "typestr": "|u1", "data": (ptr, False), "version": 2}
+        self.owner = owner
+
+
+def device_view(ptr: int, shape, dtype: torch.dtype, device, owner=None) -> torch.Tensor:
+    """A tensor over `ptr`, device memory that someone else owns."""
+    n = dtype.itemsize
+    for s in shape:
+        n *= int(s)
+    if n == 0 or not ptr:
+        return torch.empty(tuple(shape), dtype=dtype, device=device)
+    return torch.as_tensor(_DeviceMemory(ptr, n, owner), device=device).view(dtype).view(*shape)
 
 
 def dt_of(t: torch.Tensor) -> int:

@@ -1,15 +1,23 @@
 """What every part of a layer is: something that declares its tensors and its cache needs,
-loads them, and acts on rows of a step.  No part knows which model it is in; its sizes and
-constants are constructor parameters (picolm passes them as arguments too:
+loads them, and puts its work into a launch program.  No part knows which model it is in; its
+sizes and constants are constructor parameters (picolm passes them as arguments too:
 `rmsnorm(..., eps)` picolm/tensor.h:92, `rope(..., rope_type, half)` :102).
 
-Interfaces
-  Norm.forward(ctx, x[T,D] float32, rows=None)   -> h[n,D] in the compute dtype
-  PositionEncoding.rotary_tables(ctx)            -> (cos, sin, style) or None, and
+A part joins a model's program through `emit` (engine/program.py).  The built-in parts emit the
+engine's own operations.  A part that only defines `forward`, which runs its kernels (or torch
+operators) on the tensors it is handed, inherits an `emit` that wraps `forward` into a called
+operation: the engine hands it the running step, and it sees the step's rows, its cache entry and
+its state as tensors over the engine's memory.
+
+Interfaces (a new part implements `forward`, or `emit`, or both)
+  Norm.forward(ctx, x[T,D] float32, rows=None, n_rows=None) -> h[n,D] in the compute dtype
+  Norm.emit(b, x, rows) -> Rows                  the norm of buffer x as a part's input
+  PositionEncoding.rotary_tables()               -> (cos, sin, style) or None, and
   PositionEncoding.apply(ctx, qkv, H, G, d)      in place, when it is not a rotation
   Mixer.forward(ctx, h[T,D], residual[T,D] f32)  adds its output into `residual`
-  FeedForward.forward(ctx, h, residual)          adds its output into `residual`
-  Block.forward(ctx, x[T,D] f32)                 the arrangement of the four above
+  Mixer.emit(b, src: Rows, x, out_norm, out_norm_when)
+  FeedForward.forward / .emit                    the same
+  Block.emit(b, x, after, after_when)            the arrangement of the four above
 """
 from __future__ import annotations
 
@@ -17,6 +25,7 @@ from dataclasses import dataclass
 
 import torch
 
+from .. import kernels
 from ..weights import TensorSpec
 
 
@@ -32,13 +41,12 @@ class Runtime:
 
 
 class Workspace:
-    """Named scratch buffers that grow to the largest request and are reused by every
-    layer; nothing is allocated in a step whose sizes were seen before."""
+    """Named scratch buffers for parts that run from Python: they grow to the largest request and
+    are reused; nothing is allocated in a step whose sizes were seen before."""
 
     def __init__(self, device):
         self.device = device
         self._bufs: dict[str, torch.Tensor] = {}
-        self._flips: dict[str, int] = {}
         self._views: dict[tuple, tuple] = {}      # (name, shape, dtype) -> (buffer, view of it)
 
     def get(self, name: str, shape, dtype: torch.dtype) -> torch.Tensor:
@@ -59,24 +67,6 @@ class Workspace:
             self._views.clear()
         self._views[key] = (buf, view)
         return view
-
-    def zeros(self, name: str, shape, dtype: torch.dtype) -> torch.Tensor:
-        """A buffer that is zero when first given out and that its users leave at zero (counters
-        that a kernel resets itself)."""
-        n = 1
-        for s in shape:
-            n *= int(s)
-        nbytes = n * dtype.itemsize
-        buf = self._bufs.get(name)
-        if buf is None or buf.numel() < nbytes:
-            buf = torch.zeros(max(nbytes, 256), dtype=torch.uint8, device=self.device)
-            self._bufs[name] = buf
-        return buf[:nbytes].view(dtype).view(*shape)
-
-    def flip(self, name: str) -> int:
-        """0, 1, 0, 1, ... per name: for a pair of buffers used in turn."""
-        self._flips[name] = 1 - self._flips.get(name, 1)
-        return self._flips[name]
 
     def bytes(self) -> int:
         return sum(b.numel() for b in self._bufs.values())
@@ -116,55 +106,107 @@ class CacheBinding:
     writes: bool = True
 
 
-class StepContext:
-    """What a part sees of the step it runs in."""
+class StepArrays:
+    """The running step as a part that runs from Python sees it: host lists per sequence and the
+    engine's device arrays as int32 tensors (made when first asked for)."""
 
-    def __init__(self, runtime: Runtime, batch, cache, workspace: Workspace):
+    _DEVICE = {"seq_slot": "n_seq", "seq_pos0": "n_seq", "seq_nnew": "n_seq", "tok_pos": "T", "tok_seq": "T", "tokens": "T",
+               "want_rows": "n_want"}
+
+    def __init__(self, view, device):
+        self._view, self._device = view, device
+        self.n_seq, self.T, self.n_want = view.n_seq, view.n_tokens, view.n_wanted
+        self.is_decode = bool(view.is_decode)
+        self.wants_every_row = bool(view.every_row_wanted)
+        self.slots = view.slots[:self.n_seq]
+        self.pos0 = view.pos0[:self.n_seq]
+        self.n_new = view.n_new[:self.n_seq]
+        self.max_new = max(self.n_new)
+        self.max_len = max(p + n for p, n in zip(self.pos0, self.n_new))
+
+    def __getattr__(self, name):
+        if name == "cu_seqlens":
+            n = self.n_seq + 1
+        elif name in self._DEVICE:
+            n = getattr(self, self._DEVICE[name])
+        else:
+            raise AttributeError(name)
+        t = kernels.device_view(getattr(self._view, name), (max(n, 1),), torch.int32, self._device)[:n]
+        setattr(self, name, t)
+        return t
+
+    def write_pages(self) -> torch.Tensor:
+        """For every token of the step the physical page that takes its key and value (int32 [T])."""
+        if not self._view.write_pages:
+            raise ValueError("this layer call writes no keys and values")
+        return kernels.device_view(self._view.write_pages, (self.T,), torch.int32, self._device)
+
+
+class StepContext:
+    """What a part that runs from Python sees of the step it runs in."""
+
+    def __init__(self, runtime: Runtime, view, workspace: Workspace, state_request: StateRequest | None = None):
         self.runtime = runtime
-        self.batch = batch
-        self.cache = cache
+        self.view = view
         self.ws = workspace
-        self.binding: CacheBinding | None = None
-        # the norm that will be applied to the residual stream after the running part has added to
-        # it (set by the block; a Linear that adds into the stream may prepare it) and what such a
-        # Linear prepared (picked up by whoever applies that norm next)
-        self.norm_after: Norm | None = None
-        self.prepared_norm: NormedRows | None = None
-        self.norm_after_block: Norm | None = None      # set by the model for the block it calls
+        self.batch = StepArrays(view, runtime.device)
+        self.recording = bool(view.recording)
+        self._state_request = state_request
 
     @property
     def dtype(self) -> torch.dtype:
         return self.runtime.dtype
 
     def kv(self):
-        """(k_pages, v_pages, page_table, ring_pages) of the running layer call."""
-        gi, e = self.binding.kv
-        g = self.cache.kv[gi]
-        return g.k[e], g.v[e], g.table, g.ring_pages
+        """(k_pages [pages, G, 64, d], v_pages [pages, G, dv, 64], page_table [slots, max_pages],
+        ring_pages) of the running layer call."""
+        v = self.view
+        if not v.k_pages:
+            raise ValueError("this part asked for no keys and values (cache_requests)")
+        k = kernels.device_view(v.k_pages, (v.n_pages, v.n_kv_heads, kernels.PAGE_TOKENS, v.head_dim), self.dtype, self.runtime.device)
+        vv = kernels.device_view(v.v_pages, (v.n_pages, v.n_kv_heads, v.v_head_dim, kernels.PAGE_TOKENS), self.dtype, self.runtime.device)
+        table = kernels.device_view(v.page_table, (v.n_slots, v.max_pages), torch.int32, self.runtime.device)
+        return k, vv, table, v.ring_pages
 
-    def kv_host(self):
-        """(cache group index, the group's page table on the host) of the running layer call."""
-        gi, _ = self.binding.kv
-        return gi, self.cache.kv[gi].table_host
-
-    def normed(self, norm: "Norm", x: torch.Tensor, part=None):
-        """norm(x) for `part`: what a Linear prepared for this very norm and x if there is such a
-        thing and the part passes it on to a Linear, else the norm's own kernel."""
-        got, self.prepared_norm = self.prepared_norm, None
-        if got is not None and got.norm is norm and got.x is x:
-            return got if getattr(part, "takes_normed_rows", False) else got.tensor()
-        return norm.forward(self, x)
+    @property
+    def writes_cache(self) -> bool:
+        return bool(self.view.kv_writes)
 
     def state(self) -> torch.Tensor:
-        """[n_slots, ...] state of the running layer call; index it with batch.seq_slot."""
-        gi, e = self.binding.state
-        return self.cache.state[gi][e]
+        """[n_slots, ...] state of the running layer call; index it with batch.slots / batch.seq_slot."""
+        v, rq = self.view, self._state_request
+        if not v.state or rq is None:
+            raise ValueError("this part asked for no state (cache_requests)")
+        return kernels.device_view(v.state, (v.n_slots, *rq.shape), rq.dtype, self.runtime.device)
+
+
+def rows_view(ptr, rows: int, row_bytes: int, dtype: torch.dtype, device) -> torch.Tensor:
+    """A row buffer of the engine's as a tensor [rows, width]."""
+    return kernels.device_view(ptr, (rows, row_bytes // dtype.itemsize), dtype, device)
+
+
+def keeps_forward(part, cls) -> bool:
+    """Whether `part` still does in `forward` what `cls.emit` emits: a subclass that changes
+    `forward` and leaves `emit` alone has changed the work, and runs through `forward`."""
+    t = type(part)
+    return t.forward is cls.forward or t.emit is not cls.emit
+
+
+def forward_is_graph_safe(part, method: str = "forward") -> bool:
+    """Whether the class that defines the part's `forward` (or one derived from it) says
+    `graph_safe = True` itself: a subclass that writes a `forward` of its own does not inherit the
+    word of the class it changed."""
+    for cls in type(part).__mro__:
+        if cls.__dict__.get("graph_safe") is True:
+            return True
+        if method in cls.__dict__:
+            return False
+    return False
 
 
 class Part:
-    """`emit`, where a part has it, appends the part's work to a launch program (engine/program.py)
-    instead of running it: a model whose parts all have it is stepped by the library in one call.
-    A part that only has `forward` is run from Python, and so is every model that contains one."""
+    graph_safe = False      # True: what `forward` queues depends on device memory only and allocates nothing anew, so
+                            # that a decode step which holds it can be recorded once and replayed
 
     def tensor_specs(self) -> list[TensorSpec]:
         return []
@@ -186,41 +228,62 @@ class Part:
         for c in self.children():
             c.load_all(fetch, runtime)
 
+    def bind_runtime(self, runtime: Runtime, workspace: Workspace) -> None:
+        """Called before a model's program is emitted: where the part runs, and scratch memory
+        for the parts that run from Python."""
+        self._runtime, self._workspace = runtime, workspace
+        for c in self.children():
+            c.bind_runtime(runtime, workspace)
+
+    def _context(self, view, state_request=None) -> StepContext:
+        return StepContext(self._runtime, view, self._workspace, state_request)
+
+
+class on_stream:
+    """Runs the body with torch's current stream set to the stream of a step view (the engine
+    records decode steps on a stream of its own)."""
+
+    def __init__(self, view):
+        self._raw = view.stream or 0
+        self._guard = None
+
+    def __enter__(self):
+        if self._raw != (kernels._stream().value or 0):
+            self._guard = torch.cuda.stream(torch.cuda.ExternalStream(self._raw))
+            self._guard.__enter__()
+
+    def __exit__(self, *exc):
+        if self._guard is not None:
+            self._guard.__exit__(*exc)
+
 
 class Norm(Part):
+    size: int
+
     def forward(self, ctx: StepContext, x: torch.Tensor, rows: torch.Tensor | None = None,
                 n_rows: int | None = None) -> torch.Tensor:
         raise NotImplementedError
 
-    def rms_parameters(self):
-        """(float weights, eps) if this norm is y = x / sqrt(mean(x^2) + eps) * weights, which the
-        products around it can compute between them (see NormedRows); None otherwise."""
-        return None
+    def emit(self, b, x: int, rows: int = 0):
+        """This norm of the float rows in buffer `x` (of the step's rows, or with rows = 1 of the
+        rows whose logits are wanted) as the input of the part that follows: a `Rows`."""
+        from ..engine.program import ROWS_WANTED, Rows
+        width = b._specs[x][0] // 4
+        h = b.buffer("norm.final" if rows == ROWS_WANTED else "norm.out", width, b.dtype, rows)
+        dtype = b.dtype
 
-
-class NormedRows:
-    """norm(x) where the norm has not run as a kernel of its own.
-
-    In a decode step a norm over a few rows is all launch latency, so the products around it
-    share it: the Linear that finished x (adding into the residual stream) has left
-    bf16(x * weights) and partial sums of x^2 (`prepared`), and the Linear that takes this object
-    as its input multiplies its sums by 1 / sqrt(mean(x^2) + eps).  A part says with
-    `takes_normed_rows = True` that it hands its input to a Linear unchanged; any other part is
-    given `tensor()`, which runs the norm's own kernel on x."""
-
-    def __init__(self, ctx: StepContext, norm: Norm, x: torch.Tensor, prepared=None):
-        self.ctx, self.norm, self.x = ctx, norm, x
-        self.prepared = prepared            # (h bf16 [T, D], ssq f32 [parts, 16]) or None
-        self._tensor = None
-
-    @property
-    def shape(self):
-        return self.x.shape
-
-    def tensor(self) -> torch.Tensor:
-        if self._tensor is None:
-            self._tensor = self.norm.forward(self.ctx, self.x)
-        return self._tensor
+        def run(view):
+            with on_stream(view):
+                ctx = self._context(view)
+                xt = rows_view(view.inp, view.n_tokens, view.in_row_bytes, torch.float32, ctx.runtime.device)
+                out = rows_view(view.out, view.rows, view.out_row_bytes, dtype, ctx.runtime.device)
+                if rows == ROWS_WANTED and not view.every_row_wanted:
+                    y = self.forward(ctx, xt, rows=ctx.batch.want_rows, n_rows=view.n_wanted)
+                else:
+                    y = self.forward(ctx, xt)
+                out[:, :y.shape[1]].copy_(y)
+        b.call(run, out=h, inp=x, rows=rows, recordable=forward_is_graph_safe(self))
+        return Rows(h)
 
 
 class PositionEncoding(Part):
@@ -245,14 +308,52 @@ class Mixer(Part):
     def forward(self, ctx: StepContext, h: torch.Tensor, residual: torch.Tensor) -> None:
         raise NotImplementedError
 
+    def emit(self, b, src, x: int, out_norm=None, out_norm_when: int = 0) -> None:
+        """x += mixer(src) as operations of a launch program.  This one hands the step to `forward`."""
+        _emit_forward(self, b, src, x, *self.cache_requests())
+
 
 class FeedForward(Part):
     def forward(self, ctx: StepContext, h: torch.Tensor, residual: torch.Tensor) -> None:
         raise NotImplementedError
 
+    def emit(self, b, src, x: int, out_norm=None, out_norm_when: int = 0) -> None:
+        """x += ffn(src) as operations of a launch program.  This one hands the step to `forward`."""
+        _emit_forward(self, b, src, x, None, None)
+
+
+def _emit_forward(part, b, src, x: int, kv_request, state_request) -> None:
+    h = b.materialize(src)
+    h_dtype = b.buffer_dtype(h)
+
+    def run(view):
+        with on_stream(view):
+            ctx = part._context(view, state_request)
+            dev = ctx.runtime.device
+            part.forward(ctx, rows_view(view.inp, view.n_tokens, view.in_row_bytes, h_dtype, dev),
+                         rows_view(view.out, view.n_tokens, view.out_row_bytes, torch.float32, dev))
+    b.call(run, out=x, inp=h, uses_kv=kv_request is not None, uses_state=state_request is not None,
+           recordable=forward_is_graph_safe(part))
+
 
 class Block(Part):
     mixer: Mixer
 
+    def first_norm(self):
+        """The norm this block applies to the residual stream on entry, if the block before may
+        prepare it."""
+        return None
+
     def forward(self, ctx: StepContext, x: torch.Tensor) -> None:
         raise NotImplementedError
+
+    def emit(self, b, x: int, after=None, after_when: int = 0) -> None:
+        """The block over the residual rows in buffer `x`.  This one hands the step to `forward`."""
+        kv_request, state_request = self.mixer.cache_requests()
+
+        def run(view):
+            with on_stream(view):
+                ctx = self._context(view, state_request)
+                self.forward(ctx, rows_view(view.out, view.n_tokens, view.out_row_bytes, torch.float32, ctx.runtime.device))
+        b.call(run, out=x, uses_kv=kv_request is not None, uses_state=state_request is not None,
+               recordable=forward_is_graph_safe(self))

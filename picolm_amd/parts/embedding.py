@@ -8,7 +8,7 @@ import torch
 
 from .. import kernels
 from ..weights import TensorSpec
-from .base import NormedRows, Part, Runtime, StepContext
+from .base import Part, Runtime
 
 
 class TokenEmbedding(Part):
@@ -27,17 +27,15 @@ class TokenEmbedding(Part):
 
     def emit(self, b) -> int:
         """The lookup as an operation of a launch program; returns the buffer of the residual rows."""
-        from ..engine.program import CannotEmit
-        if type(self) is not TokenEmbedding or self.table is None:
-            raise CannotEmit(f"{type(self).__name__} is no plain embedding with a loaded table")
+        if self.table is None:
+            raise ValueError(f"embedding {self.name} has no table loaded")
         x = b.buffer("residual", self.D, torch.float32)
         b.embed(self.table, x)
         return x
 
-    def forward(self, ctx: StepContext, tokens: torch.Tensor, n_tokens: int) -> torch.Tensor:
-        x = ctx.ws.get("residual", (n_tokens, self.D), torch.float32)
+    def forward(self, tokens: torch.Tensor, x: torch.Tensor) -> None:
+        """The same on tensors, now: rows of the table for `tokens`, widened to float, into x."""
         kernels.embed(self.table, tokens, x)
-        return x
 
 
 class LMHead(Part):
@@ -59,27 +57,15 @@ class LMHead(Part):
             t = fetch.get(self.name)
             self.weight = (t.to(torch.float32) if runtime.is_f32 else t).contiguous()
 
-    takes_normed_rows = True   # the input goes to the product unchanged
-
-    def emit(self, b, norm, x: int) -> None:
-        """logits = W norm(x) on the wanted rows, as an operation of a launch program."""
-        from ..engine.program import ROWS_WANTED, CannotEmit
-        if type(self) is not LMHead or self.weight is None:
-            raise CannotEmit(f"{type(self).__name__} is no plain head with loaded weights")
-        h = b.buffer("norm.final", self.D, b.dtype, ROWS_WANTED)
+    def emit(self, b, src) -> None:
+        """logits = W h for the wanted rows h of `src`, as an operation of a launch program."""
+        from ..engine.program import ROWS_WANTED
+        if self.weight is None:
+            raise ValueError(f"head {self.name} has no weights loaded")
         logits = b.buffer("logits", self.V, torch.float32, ROWS_WANTED)
-        b.linear(self.weight, h, logits, kernels.EPI_STORE, rows=ROWS_WANTED, in_norm=norm, in_norm_x=x)
+        b.linear(self.weight, src, logits, kernels.EPI_STORE, rows=ROWS_WANTED)
         b.logits_buffer = logits
 
-    def forward(self, ctx: StepContext, h) -> torch.Tensor:
-        """h: the final hidden rows, or NormedRows of them."""
-        logits = ctx.ws.get("logits", (h.shape[0], self.V), torch.float32)
-        if isinstance(h, NormedRows):
-            rms = h.norm.rms_parameters()
-            hp = h.prepared[0] if h.prepared is not None else None
-            if hp is not None and rms is not None and kernels.gemm_links_norms(hp, self.weight, logits, kernels.EPI_STORE, prepares=False):
-                kernels.gemm_linked(hp, self.weight, logits, kernels.EPI_STORE, None, (h.prepared[1], h.x.shape[1], rms[1]))
-                return logits
-            h = h.tensor()
+    def forward(self, h: torch.Tensor, logits: torch.Tensor) -> None:
+        """The same on tensors, now."""
         kernels.gemm(h, self.weight, logits, kernels.EPI_STORE)
-        return logits

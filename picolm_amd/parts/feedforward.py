@@ -4,13 +4,12 @@ whose epilogue applies silu(g) * u; the down product adds into the residual."""
 from __future__ import annotations
 
 from .. import kernels
-from .base import FeedForward, StepContext
+from .base import FeedForward, StepContext, keeps_forward
 from .linear import Linear
 
 
 class SwiGLU(FeedForward):
     graph_safe = True      # launches depend on device memory only
-    takes_normed_rows = True   # the input goes to a Linear unchanged
 
     def __init__(self, prefix: str, hidden_size: int, intermediate_size: int,
                  names=("gate_proj.weight", "up_proj.weight", "down_proj.weight")):
@@ -22,18 +21,17 @@ class SwiGLU(FeedForward):
     def children(self):
         return [self.gate_up, self.down]
 
-    def emit(self, b, norm, x: int, out_norm=None, out_norm_when: int = 0) -> None:
-        """x += down(silu(gate h) * (up h)) with h = norm(x), as operations of a launch program."""
-        import torch
-        from ..engine.program import CannotEmit
-        if type(self) is not SwiGLU:
-            raise CannotEmit(f"{type(self).__name__} changes what SwiGLU does")
-        h = b.buffer("norm.out", self.D, b.dtype)
+    def emit(self, b, src, x: int, out_norm=None, out_norm_when: int = 0) -> None:
+        """x += down(silu(gate h) * (up h)) for the rows h of `src`, as operations of a launch program."""
+        if not keeps_forward(self, SwiGLU):
+            return FeedForward.emit(self, b, src, x, out_norm, out_norm_when)
         act = b.buffer("ffn.act", self.F, b.dtype)
-        self.gate_up.emit(b, h, act, kernels.EPI_SWIGLU, in_norm=norm, in_norm_x=x)
+        self.gate_up.emit(b, src, act, kernels.EPI_SWIGLU)
         self.down.emit(b, act, x, kernels.EPI_ACCUMULATE, out_norm=out_norm, out_norm_when=out_norm_when)
 
     def forward(self, ctx: StepContext, h, residual) -> None:
+        """The same on tensors, now: for parts that run from Python (a routed feed-forward calls
+        its experts on the rows it sends them)."""
         act = ctx.ws.get("ffn.act", (h.shape[0], self.F), ctx.dtype)
         self.gate_up.forward(h, act, kernels.EPI_SWIGLU)
-        self.down.forward(act, residual, kernels.EPI_ACCUMULATE, ctx)
+        self.down.forward(act, residual, kernels.EPI_ACCUMULATE)

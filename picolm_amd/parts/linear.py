@@ -11,7 +11,7 @@ import torch
 
 from .. import kernels
 from ..weights import TensorSpec
-from .base import NormedRows, Part, Runtime
+from .base import Part, Runtime
 
 
 class Linear(Part):
@@ -21,7 +21,6 @@ class Linear(Part):
     2j+1 of the second): the layout the gated epilogue reads.
     """
     graph_safe = True      # launches depend on device memory only
-
 
     def __init__(self, names, out_sizes, in_size: int, interleave: bool = False):
         self.names = list(names)
@@ -52,39 +51,14 @@ class Linear(Part):
             w = ws[0] if len(ws) == 1 else torch.cat(ws, dim=0)
         self.weight = w.contiguous()
 
-    def emit(self, b, inp: int, out: int, epilogue: int = kernels.EPI_STORE, **norms) -> None:
-        """The same product as an operation of a launch program; `norms` as ProgramBuilder.linear
-        takes them (the norm of the input, the norm that meets the output next)."""
-        from ..engine.program import CannotEmit
-        if type(self) is not Linear or self.weight is None:
-            raise CannotEmit(f"{type(self).__name__} is no plain Linear with loaded weights")
-        b.linear(self.weight, inp, out, epilogue, **norms)
+    def emit(self, b, src, out: int, epilogue: int = kernels.EPI_STORE, **kw) -> None:
+        """The product as an operation of a launch program; `src` is a buffer or `Rows` (rows with
+        the norm they are the result of), `kw` as ProgramBuilder.linear takes them (the rows
+        covered, the norm that meets the output next)."""
+        if self.weight is None:
+            raise ValueError(f"product {self.names} has no weights loaded")
+        b.linear(self.weight, src, out, epilogue, **kw)
 
-    def forward(self, a, out: torch.Tensor, epilogue: int = kernels.EPI_STORE, ctx=None) -> None:
-        """out (=, +=, = silu-gated) a W^T.  `a` is a tensor, or NormedRows: rows whose norm the
-        products compute between them.  With `ctx` and the accumulating epilogue, the norm that
-        the context says comes after (`ctx.norm_after`) is prepared for the product that follows,
-        where the kernels can do that; the result is left in `ctx.prepared_norm`."""
-        prepared = None
-        if isinstance(a, NormedRows):
-            rms = a.norm.rms_parameters()
-            h = a.prepared[0] if a.prepared is not None else None
-            if h is not None and rms is not None and kernels.gemm_links_norms(h, self.weight, out, epilogue, prepares=False):
-                prepared = (a.prepared[1], a.x.shape[1], rms[1])
-                a = h
-            else:
-                a = a.tensor()
-        prepare = None
-        nxt = ctx.norm_after if ctx is not None and epilogue == kernels.EPI_ACCUMULATE else None
-        if nxt is not None and nxt.rms_parameters() is not None and kernels.gemm_links_norms(a, self.weight, out, epilogue, prepares=True):
-            T, N = out.shape
-            which = ctx.ws.flip("norm.prepared")
-            prepare = (nxt.rms_parameters()[0], ctx.ws.get(f"norm.prepared.h{which}", (T, N), torch.bfloat16),
-                       ctx.ws.get(f"norm.prepared.ssq{which}", (kernels.linked_norm_parts(T, N, a.shape[1]), kernels.linked_norm_rows(T)),
-                                  torch.float32))
-        if prepare is None and prepared is None:
-            kernels.gemm(a, self.weight, out, epilogue)
-            return
-        kernels.gemm_linked(a, self.weight, out, epilogue, prepare, prepared)
-        if prepare is not None:
-            ctx.prepared_norm = NormedRows(ctx, nxt, out, prepared=(prepare[1], prepare[2]))
+    def forward(self, a: torch.Tensor, out: torch.Tensor, epilogue: int = kernels.EPI_STORE) -> None:
+        """out (=, +=, = silu-gated) a W^T on tensors, now: for parts that run from Python."""
+        kernels.gemm(a, self.weight, out, epilogue)

@@ -5,7 +5,7 @@ import torch
 
 from .. import kernels
 from ..weights import TensorSpec
-from .base import Norm, Runtime, StepContext
+from .base import Norm, Runtime, StepContext, keeps_forward
 
 
 class RMSNorm(Norm):
@@ -30,15 +30,20 @@ class RMSNorm(Norm):
             w = w + self.weight_offset
         self.weight = w.contiguous()
 
-    def rms_parameters(self):
-        return self.weight, self.eps
-
     def norm_ref(self):
-        """This norm as a launch program's operations carry it."""
-        from ..engine.program import CannotEmit, NormRef
-        if type(self) is not RMSNorm or self.weight is None:
-            raise CannotEmit(f"{type(self).__name__} is no plain RMSNorm with loaded weights")
-        return NormRef(self.weight, self.eps)
+        """This norm as the products around it can carry it (they compute it on their way in and,
+        in decode steps, share it between them), or None if a subclass has changed what it does."""
+        from ..engine.program import NormRef
+        if self.weight is None:
+            raise ValueError(f"norm {self.name} has no weights loaded")
+        return NormRef(self.weight, self.eps) if keeps_forward(self, RMSNorm) else None
+
+    def emit(self, b, x: int, rows: int = 0):
+        from ..engine.program import ROWS_WANTED, Rows
+        ref = self.norm_ref()
+        if ref is None:
+            return Norm.emit(self, b, x, rows)
+        return Rows(b.buffer("norm.final" if rows == ROWS_WANTED else "norm.out", self.size, b.dtype, rows), ref, x)
 
     def forward(self, ctx: StepContext, x, rows=None, n_rows=None, out_name="norm.out"):
         n = x.shape[0] if rows is None else (n_rows if n_rows is not None else rows.numel())

@@ -1,6 +1,7 @@
-"""One step's description: which sequences run, where each stands, which tokens it brings
-and which rows' logits are wanted.  Built and checked on the host, sent to the GPU as one
-int32 block.
+"""A plain planner of a step's index arrays, in NumPy: which sequences run, where each stands,
+which tokens it brings, which rows' logits are wanted, the prefill's tiles, the decode attention's
+work list, every token's cache page.  The engine in the library plans every step itself
+(csrc/engine.hip); the tests hold its arrays to these, and call single kernels with them.
 
 The sequences of a step either all bring their first tokens (a prefill step; lengths may
 differ) or each bring one more token (a decode step).  picolm has the two as separate
@@ -12,11 +13,8 @@ from __future__ import annotations
 import numpy as np
 import torch
 
-from ..cache.slots import PAGE_TOKENS, pages_for
-
-
-class StepError(ValueError):
-    """A step that cannot run: a dead slot, a token outside the vocabulary, no room."""
+from picolm_amd.cache import PAGE_TOKENS, pages_for
+from picolm_amd.engine.errors import StepError
 
 
 def _to_device(host: torch.Tensor, device) -> torch.Tensor:
@@ -234,163 +232,3 @@ class _Chunk:
         })
 
     prefill_tiles = StepBatch.prefill_tiles
-
-
-class DecodeBatch:
-    """A decode step (one new token per sequence) over buffers that stay in place, so that the
-    step's kernel launches can be recorded once as a HIP graph and replayed: only the contents
-    of the int32 block change from step to step."""
-
-    is_decode = True
-    max_new = 1
-    wants_every_row = True
-
-    def __init__(self, n_seq: int, pages_per_chunk: int, device, reserve_ints: int = 0):
-        """`reserve_ints`: room behind the step's arrays for the work lists and page arrays that
-        parts ask for, so that everything goes to the device in one copy; what does not fit gets
-        a block and a copy of its own."""
-        self.n_seq = self.T = self.n_want = n_seq
-        self.pages_per_chunk = pages_per_chunk
-        self.n_new = [1] * n_seq
-        self.want_counts = [1] * n_seq
-        n = n_seq
-        self._spans = {}
-        off = 0
-        for name, size in (("seq_slot", n), ("seq_pos0", n), ("seq_nnew", n), ("cu_seqlens", n + 1), ("tok_pos", n),
-                           ("tok_seq", n), ("tokens", n), ("want_rows", n)):
-            self._spans[name] = (off, size)
-            off += size
-        off = (off + 3) // 4 * 4                    # what follows is read 16 bytes at a time
-        self._used, self._size = off, off + (reserve_ints + 3) // 4 * 4
-        self._device = torch.device(device)
-        self._host = torch.zeros(self._size, dtype=torch.int32)
-        self._dev = torch.zeros(self._size, dtype=torch.int32, device=device)
-        # The block goes to the device through one of two pinned copies, in turn, and the copy does
-        # not wait: a step can be handed to the GPU while the one before it still runs.  A pinned
-        # copy is written again only after the transfer that read it has ended.
-        self._pinned = [self._host_block(self._size), self._host_block(self._size)] if self._device.type == "cuda" else []
-        self._sent = [None, None]
-        self._turn = 0
-        h = self._host.numpy()
-        ar = np.arange(n + 1, dtype=np.int32)
-        self._np = {k: h[o:o + s] for k, (o, s) in self._spans.items()}
-        self._np["seq_nnew"][:] = 1
-        self._np["cu_seqlens"][:] = ar
-        self._np["tok_seq"][:] = ar[:n]
-        self._np["want_rows"][:] = ar[:n]
-        for k, (o, s) in self._spans.items():
-            setattr(self, k, self._dev[o:o + s])
-        self.slots, self.pos0 = [], []
-        self._lists = {}        # (window, group) -> (host array, device array, most chunks, page table, ring, own block or None)
-        self._pages = {}        # group -> (host array, device array, page table, ring, own block or None)
-        self._live = {}         # (window, group) -> entries in use
-        self._cache_version = None
-        self.frozen = False     # set once the launches are recorded: no further work list can join
-
-    @staticmethod
-    def _host_block(n: int):
-        t = torch.zeros(n, dtype=torch.int32)
-        return t.pin_memory() if torch.cuda.is_available() else t
-
-    def _region(self, n_ints: int):
-        """(host numpy view, device view, own host block or None) of n_ints more ints."""
-        n4 = (n_ints + 3) // 4 * 4
-        if self._used + n4 <= self._size:
-            o = self._used
-            self._used += n4
-            return self._host.numpy()[o:o + n_ints], self._dev[o:o + n_ints], None
-        own = self._host_block(n_ints)
-        return own.numpy(), torch.zeros(n_ints, dtype=torch.int32, device=self._device), own
-
-    def fill(self, slots, pos0, tokens, cache_version=None, tokens_on_device=None) -> None:
-        """`cache_version`: the cache's counter of slot and page changes; while it stands still
-        (and is given), what the last fill looked up in the page tables still holds.
-        `tokens_on_device`: an int32 tensor with the step's tokens, in place of `tokens`: the
-        host need not know them yet (they may come from a sampling kernel that has not run)."""
-        # between page boundaries only the positions move: the lists and pages stay as they are
-        same_pages = (cache_version is not None and cache_version == self._cache_version
-                      and list(slots) == self.slots and len(pos0) == len(self.pos0)
-                      and all(p == q + 1 and p % PAGE_TOKENS for p, q in zip(pos0, self.pos0)))
-        self._cache_version = cache_version
-        self.slots, self.pos0 = list(slots), list(pos0)
-        self._np["seq_slot"][:] = slots
-        self._np["seq_pos0"][:] = pos0
-        self._np["tok_pos"][:] = pos0
-        if tokens_on_device is None:
-            self._np["tokens"][:] = tokens
-        for key in self._lists:
-            if same_pages and key[0] == 0:          # (a window's first page can move on any step)
-                self._lists[key][0].reshape(-1, CHUNK_ENTRY_INTS)[1:1 + self._live[key], 2] += 1
-            else:
-                self._fill_list(key)
-        if not same_pages:
-            for group in self._pages:
-                self._fill_pages(group)
-        self._send()
-        if tokens_on_device is not None:
-            self.tokens.copy_(tokens_on_device)
-        for host, dev, *_, own in list(self._lists.values()) + list(self._pages.values()):
-            if own is not None:
-                dev.copy_(own, non_blocking=False)
-
-    def _send(self) -> None:
-        if not self._pinned:
-            self._dev.copy_(self._host)
-            return
-        t = self._turn
-        self._turn ^= 1
-        if self._sent[t] is None:
-            self._sent[t] = torch.cuda.Event()
-        else:
-            self._sent[t].synchronize()
-        self._pinned[t].copy_(self._host)
-        self._dev.copy_(self._pinned[t], non_blocking=True)
-        self._sent[t].record()
-
-    def _fill_pages(self, group: int) -> None:
-        host, dev, table_host, ring_pages, own = self._pages[group]
-        host[:] = token_pages(np.arange(self.n_seq), self.pos0, self.slots, table_host, ring_pages)
-
-    def write_pages(self, group: int, table_host, ring_pages: int):
-        if group not in self._pages:
-            if self.frozen:
-                raise StepError("a recorded decode step cannot take another cache group")
-            host, dev, own = self._region(self.n_seq)
-            self._pages[group] = (host, dev, table_host, ring_pages, own)
-            self._fill_pages(group)
-            dev.copy_(torch.from_numpy(host), non_blocking=False)
-        return self._pages[group][1]
-
-    def _fill_list(self, key) -> None:
-        host, dev, most, table_host, ring_pages, own = self._lists[key]
-        entries, n_most = decode_chunk_list(self.slots, self.pos0, key[0], self.pages_per_chunk, table_host, ring_pages)
-        if n_most > most:
-            raise StepError(f"a sequence of {max(self.pos0) + 1} tokens has more pages than the cache was sized for")
-        h = host.reshape(-1, CHUNK_ENTRY_INTS)
-        h[0, 0] = len(entries)          # workgroups past this count leave at once
-        h[1:1 + len(entries)] = entries
-        self._live[key] = len(entries)
-
-    def decode_chunks(self, blocks_per_chunk: int, max_pages_per_chunk: int, window: int, group: int, table_host,
-                      ring_pages: int):
-        """As StepBatch.decode_chunks, over a list of fixed capacity (every sequence at the
-        cache's full length) that `fill` rewrites in place; the chunk size was chosen when the
-        batch was made."""
-        key = (window, group)
-        if key not in self._lists:
-            if self.frozen:
-                raise StepError("a recorded decode step cannot take another work list")
-            most = (table_host.shape[1] + self.pages_per_chunk - 1) // self.pages_per_chunk
-            cap = self.n_seq * most
-            host, dev, own = self._region((cap + 1) * CHUNK_ENTRY_INTS)
-            self._lists[key] = (host, dev, most, table_host, ring_pages, own)
-            self._fill_list(key)
-            dev.copy_(torch.from_numpy(host), non_blocking=False)
-        host, dev, most, *_ = self._lists[key]
-        return dev, len(host) // CHUNK_ENTRY_INTS - 1, self.pages_per_chunk, most
-
-    @staticmethod
-    def ints_for(n_seq: int, pages_per_chunk: int, max_pages: int) -> int:
-        """Room that one cache group's work list and page array take (see `reserve_ints`)."""
-        most = (max_pages + pages_per_chunk - 1) // pages_per_chunk
-        return (n_seq * most + 1) * CHUNK_ENTRY_INTS + n_seq + 8

@@ -1,8 +1,8 @@
 """The engine behind the C ABI (csrc/engine.h).  Its entry points are called through ctypes as a C
 program would call them, over the three ways of cutting the work (each request whole; its last
 tokens one by one; unequal batches one after another in slots that are used again), against the
-plain implementation; its steps give the same bits as the step that Python runs part by part
-with the same kernels; its generation loop makes the tokens that the Python loop makes."""
+plain implementation; its generation loop makes the tokens that the Python loop makes, and the
+tokens that the plain sampler draws from the plain logits."""
 import ctypes
 from ctypes import byref, c_int32, c_void_p
 
@@ -34,10 +34,8 @@ class CEngine:
         from picolm_amd.engine import program as P
         self.lib = kernels.lib()
         P.declare(self.lib)
-        for b in model.blocks:
-            b.mixer.prepare(model.runtime, model.config.max_position_embeddings)
+        model.prepare(model.config.max_position_embeddings)
         self.built = model.program()
-        assert self.built is not None
         self.V = model.head.V
         self.h = c_void_p()
         rc = self.lib.picolm_engine_create(byref(self.built.struct), max_tokens, model.config.max_position_embeddings, n_slots,
@@ -128,38 +126,6 @@ def test_the_c_entry_points_over_the_three_cuttings(which, dtype, folders):
     e.close()
 
 
-@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("which", ["A", "B", "C", "D", "E", "F"])
-def test_the_library_steps_as_python_steps_part_by_part(which, dtype, folders):
-    """The same model through the engine in the library and through `DecoderModel.step`: the same
-    kernels in the same order, so the same bits, in prompts, continuation steps, decode steps that
-    are launched and decode steps that are replayed."""
-    from picolm_amd.engine import Session, load_model
-    d = folders[which]
-    V = tiny.read_config(d)["vocab_size"]
-    model = load_model(d, dtype=dtype)
-    rng = np.random.default_rng(41)
-    prompts = [tiny.random_tokens(rng, n, V) for n in (70, 5, 33)]
-    more = [tiny.random_tokens(rng, n, V) for n in (9, 1, 66)]
-    cont = [tiny.random_tokens(rng, 12, V) for _ in prompts]
-    outs = []
-    for native in (True, False):
-        s = Session(model, max_tokens=1024, native=native)
-        assert (s.engine is not None) == native
-        slots = s.begin(3)
-        rows = [s.step(slots, prompts, [list(range(len(p))) for p in prompts]).clone(),
-                s.step(slots, more, [[0, len(m) - 1] for m in more]).clone()]          # several tokens onto what is there
-        for j in range(12):
-            rows.append(s.step(slots, [[c[j]] for c in cont]).clone())
-        rows.append(s.step(slots[:2], [[1, 2, 3], [4]]).clone())                       # a longer and a single token together
-        if native:
-            assert s.recorded_steps() == 1
-        s.release(slots)
-        outs.append(rows)
-    for a, b in zip(*outs):
-        assert torch.equal(a, b)
-
-
 @pytest.mark.parametrize("params", [(0.0, 0, 1.0, 0.0, 42), (0.8, 40, 0.9, 0.05, 7), (1.1, 0, 1.0, 0.0, 0)])
 def test_the_library_loop_makes_the_tokens_of_the_python_loop(params, folders):
     from picolm_amd import SamplingParams, generate
@@ -183,6 +149,50 @@ def test_the_library_loop_makes_the_tokens_of_the_python_loop(params, folders):
     small = Session(model, max_tokens=128, max_seq_len=70)
     toks, finish = small.engine.generate([prompts[3]], 25, SamplingParams(), [], batch_size=1)
     assert finish == ["capacity"] and len(toks[0]) == 70 - 64 + 1
+
+
+@pytest.mark.parametrize("params", [(0.0, 0, 1.0, 0.0, 42), (0.8, 40, 0.9, 0.05, 7)])
+def test_the_library_loop_against_the_plain_sampler_at_matrix_core_sizes(params, folders):
+    """picolm_engine_generate on configuration E (width 1,024, heads of 128, four query heads a KV
+    head: the sizes the matrix-core kernels are made for), batches of three after one another with
+    stop tokens.  In 32-bit every token is what the plain sampler draws from the plain logits of
+    the sequence so far, with that request's generator stream.  In bfloat16 (greedy) every token's
+    plain logit lies within the engine's distance of the largest."""
+    from plain import sampler_plain as SP
+    from picolm_amd import SamplingParams
+    from picolm_amd.engine import Session, load_model
+    from picolm_amd.sampling import stream_state
+    from plain import llama_plain
+    d = folders["E"]
+    V = tiny.TINY_E["vocab_size"]
+    weights, config = tiny.read_weights_f64(d), tiny.read_config(d)
+    plain_logits = lambda seq: llama_plain.forward(weights, config, seq)
+    rng = np.random.default_rng(44)
+    prompts = [tiny.random_tokens(rng, n, V) for n in (1, 70, 9, 130, 33, 64, 65)]
+    sp = SamplingParams(*params)
+    n_new = 10
+    model = load_model(d, dtype="float32")
+    free, _ = Session(model, max_tokens=3 * 256).engine.generate(prompts, n_new, sp, [], batch_size=3)
+    stop = [free[1][4], free[5][7]]
+    toks, finish = Session(model, max_tokens=3 * 256).engine.generate(prompts, n_new, sp, stop, batch_size=3)
+    assert "stop" in finish and "length" in finish
+    for i, (p, got) in enumerate(zip(prompts, toks)):
+        state, seq = stream_state(sp.seed, i), list(p)
+        for k, t in enumerate(got):
+            lg = plain_logits(seq)[-1]
+            want, state = SP.sample(lg, sp.temperature, sp.top_k, sp.top_p, sp.min_p, state)
+            assert want == t, f"request {i} token {k}: library {t}, plain sampler {want}"
+            seq.append(t)
+        assert finish[i] == ("stop" if got[-1] in stop else "length") and (got[-1] in stop or len(got) == n_new)
+        assert not any(t in stop for t in got[:-1])
+    if sp.greedy:
+        model = load_model(d, dtype="bfloat16")
+        toks, _ = Session(model, max_tokens=3 * 256).engine.generate(prompts, n_new, sp, [], batch_size=3)
+        for i, (p, got) in enumerate(zip(prompts, toks)):
+            ref = plain_logits(list(p) + got)
+            for k, t in enumerate(got):
+                row = ref[len(p) - 1 + k]
+                assert row[t] >= row.max() - 2 * tolerance("bfloat16", ref, tiny.spread_of("E")), (i, k, t)
 
 
 def test_prompts_beyond_the_budget_of_a_step_go_in_as_several_steps(folders):

@@ -2,43 +2,19 @@
 an engine made with the host-only flag keeps slots, pages and page tables and plans every step's
 index arrays, but holds no device memory and launches nothing.  Checked here: no slot or page is
 lost, held twice or freed twice; a refused step changes nothing; the arrays of a step are those
-that the step run from Python builds for the same batch (engine/batch.py), which has tests of
-its own."""
+of the plain planner (tests/plan_reference.py), which has tests of its own."""
 import random
 
 import numpy as np
 import pytest
 import torch
 
-from picolm_amd.cache import CacheError, CacheFull, CacheSpec, KVGroupSpec
+from host_engine import D, G, H, V, d, host_engine
+from picolm_amd.cache import CacheError, CacheFull, CacheSpec
+from picolm_amd.engine import StepError
 from picolm_amd.engine import program as P
-from picolm_amd.engine.batch import StepBatch, StepError, decode_chunk_list, decode_pages_per_chunk, token_pages
 from picolm_amd.engine.native import NativeEngine
-from picolm_amd.parts.base import CacheBinding
-
-D, H, G, d, V = 64, 4, 2, 16, 100
-
-
-def host_engine(max_tokens=64 * 10, max_seq_len=64 * 4, n_slots=3, layers=2):
-    """A program of `layers` attention layers and a head, with made-up weights that nothing reads."""
-    b = P.ProgramBuilder(torch.float32, host_only=True)
-    x = b.buffer("residual", D, torch.float32)
-    b.embed(torch.zeros(V, D), x)
-    norm = P.NormRef(torch.ones(D), 1e-5)
-    for layer in range(layers):
-        b.binding = CacheBinding((0, layer), None, True)
-        h = b.buffer("norm.out", D, torch.float32)
-        qkv = b.buffer("attn.qkv", (H + 2 * G) * d, torch.float32)
-        b.linear(torch.zeros((H + 2 * G) * d, D), h, qkv, 0, in_norm=norm, in_norm_x=x)
-        q, o = b.buffer("attn.q", H * d, torch.float32), b.buffer("attn.out", H * d, torch.float32)
-        b.attention(qkv, q, o, H, G, d, 0, 0.25, None)
-        b.linear(torch.zeros(D, H * d), o, x, 1, out_norm=norm, out_norm_when=int(layer == layers - 1))
-    hf = b.buffer("norm.final", D, torch.float32, P.ROWS_WANTED)
-    lg = b.buffer("logits", V, torch.float32, P.ROWS_WANTED)
-    b.linear(torch.zeros(V, D), hf, lg, 0, rows=P.ROWS_WANTED, in_norm=norm, in_norm_x=x)
-    b.logits_buffer = lg
-    built = b.finish(V, CacheSpec([KVGroupSpec(layers, G, d, 0)], []))
-    return NativeEngine(built, max_tokens, max_seq_len, n_slots, "cpu", host_only=True)
+from plan_reference import StepBatch, decode_chunk_list, decode_pages_per_chunk, token_pages
 
 
 def test_an_ill_formed_program_is_refused_with_the_operation_named():
@@ -135,15 +111,15 @@ def test_random_walk_keeps_the_books_balanced():
         assert e.info(2) + len(live) == 6
 
 
-def table_of(e, n_slots, max_pages):
+def table_of(e, n_slots, max_pages, group=0):
     t = np.zeros((n_slots, max_pages), dtype=np.int32)
     for s in range(n_slots):
-        pages = e.slot_pages(0, s)
+        pages = e.slot_pages(group, s)
         t[s, :len(pages)] = pages
     return t
 
 
-def test_a_prefill_step_is_planned_as_the_python_step_plans_it():
+def test_a_prefill_step_is_planned_as_the_plain_planner_plans_it():
     e = host_engine(max_tokens=64 * 40, max_seq_len=64 * 8, n_slots=4)
     slots = [e.slot_alloc() for _ in range(4)]
     order = [slots[2], slots[0], slots[3]]
@@ -165,7 +141,7 @@ def test_a_prefill_step_is_planned_as_the_python_step_plans_it():
 
 
 @pytest.mark.parametrize("lengths", [[70, 5, 130], [500, 1, 64, 63], [507] * 4, [300] * 40])
-def test_a_decode_step_is_planned_as_the_python_step_plans_it(lengths):
+def test_a_decode_step_is_planned_as_the_plain_planner_plans_it(lengths):
     n = len(lengths)
     e = host_engine(max_tokens=64 * 8 * n, max_seq_len=512, n_slots=n)
     slots = [e.slot_alloc() for _ in range(n)]
@@ -209,3 +185,53 @@ def test_a_slot_that_changes_hands_is_looked_up_again_by_the_decode_step():
     rows = {int(r[0]): r for r in second[1:3]}
     assert rows[0][2] == 11 and rows[0][4] == e.slot_pages(0, c)[0] != first[1 + list(first[1:3, 0]).index(0)][4]
     assert np.array_equal(e.step_array("write_pages.0"), [e.slot_pages(0, c)[0], e.slot_pages(0, b)[0]])
+
+
+@pytest.mark.parametrize("window", [1, 64, 100, 200])
+def test_a_decode_step_over_a_window_is_planned_as_the_plain_planner_plans_it(window):
+    """A group that keeps a window of keys: the work list covers the pages of the last `window` keys
+    only, its first page moves with every step, and pages lie in the slot's ring.  Walked over 150
+    steps (page boundaries, laps of the ring), in the block that stays in place."""
+    from picolm_amd.cache import window_ring_pages
+    lengths = [500, 3, 130]
+    e = host_engine(max_tokens=64 * 64, max_seq_len=1024, n_slots=3, layers=2, windows=(0, window))
+    ring = min(window_ring_pages(window), 16)
+    slots = [e.slot_alloc() for _ in range(3)]
+    for lo in range(0, 500, 250):
+        live = [i for i in range(3) if lengths[i] > lo]
+        e.step([slots[i] for i in live], [[1] * min(250, lengths[i] - lo) for i in live])
+    for step in range(150):
+        pos0 = [L + step for L in lengths]
+        e.step(slots, [[7]] * 3)
+        ppc = decode_pages_per_chunk(pos0, G, 16)
+        for group, (w, r) in enumerate(((0, 16), (window, ring))):
+            entries, _ = decode_chunk_list(slots, pos0, w, ppc, table_of(e, 3, 16, group), r)
+            got = e.step_array(f"chunks.{group}").reshape(-1, 8)
+            assert got[0, 0] == len(entries) and np.array_equal(got[1:1 + len(entries)], entries), (step, group)
+            assert np.array_equal(e.step_array(f"write_pages.{group}"), token_pages(np.arange(3), pos0, slots, table_of(e, 3, 16, group), r))
+        assert all(len(e.slot_pages(1, s)) <= ring for s in slots)
+
+
+def test_a_long_prefill_step_over_a_window_is_cut_along_positions():
+    """Where a group keeps a ring, a step of more than 256 tokens a sequence is planned a second
+    time as slices of 256 positions, each with sequences, rows and tiles of its own."""
+    e = host_engine(max_tokens=64 * 64, max_seq_len=1024, n_slots=3, layers=2, windows=(0, 100))
+    slots = [e.slot_alloc() for _ in range(3)]
+    e.step([slots[1]], [[1] * 40])
+    news = [[1] * 700, [2] * 30, [3] * 257]
+    e.step(slots, news)
+    ref = StepBatch(slots, [0, 40, 0], news, [[], [], []], V, "cpu")
+    chunks = list(ref.chunks(256))
+    assert len(chunks) == 3
+    for c, want in enumerate(chunks):
+        for name, have in (("seq_slot", want.seq_slot), ("seq_pos0", want.seq_pos0), ("seq_nnew", want.seq_nnew),
+                           ("first_row", want.cu_seqlens), ("rows", want.rows)):
+            assert np.array_equal(e.step_array(f"window_chunk.{c}.{name}"), have.numpy()[:len(e.step_array(f"window_chunk.{c}.{name}"))]), (c, name)
+        seq, q0, n = want.prefill_tiles(16)
+        assert np.array_equal(e.step_array(f"window_chunk.{c}.tiles.16.seq"), seq.numpy())
+        assert np.array_equal(e.step_array(f"window_chunk.{c}.tiles.16.q0"), q0.numpy())
+    with pytest.raises(Exception, match="no array"):
+        e.step_array("window_chunk.3.rows")
+    e.step(slots, [[1] * 200, [2] * 256, [3] * 9])          # no sequence brings more than 256: no slices
+    with pytest.raises(Exception, match="no array"):
+        e.step_array("window_chunk.0.rows")

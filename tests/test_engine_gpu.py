@@ -132,6 +132,38 @@ def test_a_wide_batch_decodes_like_its_sequences_alone(which, n_seq, dtype, fold
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("which", ["B", "E"])
+def test_single_token_steps_that_do_not_want_every_row(which, dtype, folders):
+    """Steps of one token per sequence in which one sequence wants nothing, another its one row and
+    a third the same row twice: such a step is planned like a prefill step with a gather of the
+    wanted rows, not as the decode step that replays a recording.  They alternate with plain decode
+    steps of the same batch, before and after that batch size's recording exists; every row against
+    the plain implementation."""
+    d = folders[which]
+    V = tiny.read_config(d)["vocab_size"]
+    rng = np.random.default_rng(17)
+    lens, n_dec = [70, 5, 33], 12
+    seqs = [tiny.random_tokens(rng, n + n_dec, V) for n in lens]
+    truth = [tiny.plain_logits(d, q) for q in seqs]
+    s = session(d, dtype, max_tokens=1024, n_slots=3)
+    slots = s.begin(3)
+    s.step(slots, [q[:n] for q, n in zip(seqs, lens)], [[], [], []])
+    wants = [None, [[], [0], [0, 0]], None, None, [[0], [], []], [[], [], [0]], None, [[], [], []], [[0], [0], [0]], None,
+             [[0, 0], [], [0]], None]
+    recorded_before = s.recorded_steps()
+    for j, want in enumerate(wants):
+        got = s.step(slots, [[q[n + j]] for q, n in zip(seqs, lens)], want)
+        rows = [i for i in range(3) for _ in (want[i] if want is not None else [0])]
+        assert got.shape[0] == len(rows)
+        got = got.double().cpu().numpy()
+        for k, i in enumerate(rows):
+            err = np.abs(got[k] - truth[i][lens[i] + j]).max()
+            assert err <= tolerance(dtype, truth[i], tiny.spread_of(which)), (which, dtype, "step", j, "sequence", i, err)
+    assert recorded_before == 0 and s.recorded_steps() == 1     # the plain decode steps were recorded meanwhile
+    s.release(slots)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_long_decoding_and_first_tokens(dtype, folders):
     d = folders["C"]
     rng = np.random.default_rng(11)
@@ -146,8 +178,7 @@ def test_long_decoding_and_first_tokens(dtype, folders):
     assert s.length(a) == 400
 
 
-@pytest.mark.parametrize("native", [True, False])
-def test_decoding_at_contexts_of_thousands_of_tokens(native, tmp_path):
+def test_decoding_at_contexts_of_thousands_of_tokens(tmp_path):
     """Twelve sequences of about 5,000 tokens: enough pages for the decode attention to take chunks
     of 64 (and, when most sequences have ended, 32 and 16), each sequence several chunks whose
     partial results are merged.  All twelve are beginnings of one token sequence, so that one pass
@@ -162,14 +193,13 @@ def test_decoding_at_contexts_of_thousands_of_tokens(native, tmp_path):
     toks = tiny.random_tokens(rng, 5010, 300)
     truth = tiny.plain_logits(d, toks)
     lens = [5000 - 37 * i for i in range(12)]
-    s = Session(load_model(d, dtype="bfloat16"), max_tokens=12 * 5120, native=native)
-    assert (s.engine is not None) == native
+    s = Session(load_model(d, dtype="bfloat16"), max_tokens=12 * 5120)
     slots = s.begin(12)
     got = s.step(slots, [toks[:n] for n in lens]).double().cpu().numpy()          # the prompts, all in one step
     tol_ = tiny.tolerance("bfloat16", truth, tiny.spread(256, 0.05))
     for i, n in enumerate(lens):
         assert np.abs(got[i] - truth[n - 1]).max() <= tol_, ("prefill", i)
-    from picolm_amd.engine.batch import decode_pages_per_chunk
+    from plan_reference import decode_pages_per_chunk
     seen = set()
     live = list(range(12))
     for step in range(6):
@@ -565,13 +595,12 @@ def test_steps_that_append_several_tokens_to_what_a_slot_holds(which, dtype, fol
     s.release(slots)
 
 
-@pytest.mark.parametrize("native", [True, False])
 @pytest.mark.parametrize("which", ["D", "E"])
-def test_a_prefill_step_of_a_thousand_tokens_and_more(which, native, folders):
+def test_a_prefill_step_of_a_thousand_tokens_and_more(which, folders):
     """From 1,024 tokens a step on, the matrix-core path writes no rotated copy of q: the attention
     kernel rotates q itself and a tile-wise kernel writes keys and values.  Prompts that make
     such a step together, one of them continued from what its slot holds; then decode steps, which
-    read what that kernel wrote.  In the library's step and in the one from Python."""
+    read what that kernel wrote."""
     d = folders[which]
     cfg = tiny.read_config(d)
     rng = np.random.default_rng(77)
@@ -582,7 +611,7 @@ def test_a_prefill_step_of_a_thousand_tokens_and_more(which, native, folders):
     n = len(lens)
     seqs = [tiny.random_tokens(rng, m + 4, cfg["vocab_size"]) for m in lens]
     truth = [tiny.plain_logits(d, q) for q in seqs]
-    s = session(d, "bfloat16", max_tokens=2048, native=native)
+    s = session(d, "bfloat16", max_tokens=2048)
     slots = s.begin(n)
     s.step([slots[1]], [seqs[1][:37]])                       # the second prompt's first 37 tokens are held already
     first = [0, 37] + [0] * (n - 2)

@@ -423,7 +423,7 @@ class PagedCase:
         self.q_dev = torch.from_numpy(qnew).reshape(-1, H * d).to(dtype).to(DEV)
 
     def batch(self):
-        from picolm_amd.engine.batch import StepBatch
+        from plan_reference import StepBatch
         toks = [[0] * n for n in self.lens_new]
         return StepBatch([int(s) for s in self.slots], self.lens_old, toks, [[] for _ in toks], 10, DEV)
 
@@ -527,7 +527,7 @@ def test_attention_prefill_with_rotation_inside(H, G, d, style, window):
 def decode_work_list(case, window, pages_per_chunk, spare=0):
     """The work list the engine would build, with room for `spare` more entries behind it (a
     recorded step's list has room for full-length sequences): those hold garbage."""
-    from picolm_amd.engine.batch import decode_chunk_list, with_header
+    from plan_reference import decode_chunk_list, with_header
     b = case.batch()
     entries, most = decode_chunk_list(b.slots, b.pos0, window, pages_per_chunk, case.table_host,
                                       case.table_host.shape[1])
@@ -710,6 +710,56 @@ def test_attention_finds_a_far_key(dtype):
             assert np.abs(got[h] - case.v[0][target, h // 2]).max() < 2e-2
 
 
+@pytest.mark.parametrize("pages_per_chunk", [32, 64])
+@pytest.mark.parametrize("where", ["fifth page of a chunk", "last page of a chunk", "second chunk"])
+def test_attention_finds_a_far_key_in_a_long_chunk(pages_per_chunk, where):
+    """Chunks of 32 and 64 pages: a work list's entry carries a chunk's first four pages and the
+    matrix-core kernel looks the others up in the page table itself.  The key that dominates lies
+    in such a page: the fifth of the first chunk, the chunk's last, or a page past the fourth of
+    the second chunk, whose partial result is merged.  A wrong or dropped page gives another
+    value row.  With a second kernel merging the chunks, with the attention kernel merging them
+    itself, and in the kernel that also takes the new token unrotated and writes it to the cache."""
+    H, G, d = 8, 2, 128
+    n_old = 64 * (pages_per_chunk + 30) - 7              # two chunks of 64 pages, three of 32
+    page = {"fifth page of a chunk": 4, "last page of a chunk": pages_per_chunk - 1, "second chunk": pages_per_chunk + 6}[where]
+    target = 64 * page + 37
+
+    def boost(c):
+        c.k[0][target] = 0.0
+        c.k[0][target, :, 0] = 30.0
+        c.q[0][-1] = 0.0
+        c.q[0][-1, :, 0] = 30.0
+    case = PagedCase(H, G, d, [n_old], [1], torch.bfloat16, seed=pages_per_chunk, scale_q=boost)
+    b = case.batch()
+    chunk_list, n_chunks, most = decode_work_list(case, 0, pages_per_chunk, spare=1)
+    assert most >= 2
+    partial = torch.full((H * most * (d + 2),), float("nan"), device=DEV)
+    done = torch.zeros(K().attn_decode_counters(1, H, G), dtype=torch.int32, device=DEV)
+
+    def check(out):
+        got = out.double().cpu().numpy().reshape(H, d)
+        for h in range(H):
+            assert np.abs(got[h] - case.v[0][target, h // (H // G)]).max() < 2e-2, (where, h)
+    for counters in (None, done):
+        out = torch.zeros_like(case.q_dev)
+        K().attn_decode(case.q_dev, case.k_pages, case.v_pages, out, partial, 1, chunk_list, n_chunks, pages_per_chunk, most,
+                        b.seq_pos0, case.table, case.table.shape[1], H, G, d, 0, 1.0 / math.sqrt(d), counters)
+        check(out)
+    # the one-launch kernel: q, k, v of the new token in float, no rotation
+    qkv = torch.zeros(1, (H + 2 * G) * d, device=DEV)
+    qkv[0, :H * d] = case.q_dev[0].float()
+    qkv[0, H * d:(H + G) * d] = torch.from_numpy(case.k[0][-1].reshape(-1)).float().to(DEV)
+    qkv[0, (H + G) * d:] = torch.from_numpy(case.v[0][-1].reshape(-1)).float().to(DEV)
+    tok_page = b.write_pages(0, case.table_host, case.table_host.shape[1])
+    for counters in (None, done):
+        out = torch.zeros(1, H * d, dtype=torch.bfloat16, device=DEV)
+        K().attn_decode_rope(qkv, case.k_pages, case.v_pages, out, partial, 1, chunk_list, n_chunks, pages_per_chunk, most,
+                             b.seq_pos0, case.table, case.table.shape[1], H, G, d, 0, 1.0 / math.sqrt(d), None, None, 0,
+                             tok_page, counters)
+        check(out)
+    assert not done.any()
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_attention_over_pages_beyond_four_gigabytes(dtype):
     """A cache of a large batch of long sequences: the pages of this case lie more than 2^32 bytes
@@ -735,7 +785,7 @@ def test_attention_over_pages_beyond_four_gigabytes(dtype):
     err = np.abs(out.double().cpu().numpy() - ref).max()
     assert err <= tol(dtype, np.abs(ref).max()), err
     # the last sequence alone as a decode step, its chunks combined by the kernel and by the merge kernel
-    from picolm_amd.engine.batch import StepBatch, decode_chunk_list, with_header
+    from plan_reference import StepBatch, decode_chunk_list, with_header
     slot, pos0 = int(case.slots[2]), 650
     db = StepBatch([slot], [pos0], [[0]], [[]], 10, DEV)
     q1 = case.q_dev[-1:].contiguous()
@@ -831,7 +881,7 @@ def test_kv_page_order_is_a_permutation(d):
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("style", ["pairwise", "half"])
 def test_rope_kv_store(dtype, style):
-    from picolm_amd.engine.batch import StepBatch
+    from plan_reference import StepBatch
     H, G, d = 3, 1, 32
     rng = np.random.default_rng(0)
     slots, pos0, n_new = [2, 0], [61, 0], [5, 70]

@@ -1,6 +1,9 @@
-"""Each part of a layer alone against its plain function, and a toy architecture whose mixer
-keeps state of its own: defined, registered, built, loaded from a random model folder and
-stepped here, without a change to the library's files."""
+"""Each part of a layer alone against its plain function, and toy architectures whose parts are
+defined here: registered, built, loaded from a random model folder and stepped by the engine,
+without a change to the library's files.  A part written in Python (its `forward` runs torch
+operators on the engine's memory) and a part with HIP kernels of its own (tests/toy_parts) both run
+inside the library's step, through its cache, its planner and its generation loop."""
+import ctypes
 import json
 import math
 import os
@@ -16,26 +19,6 @@ pytestmark = pytest.mark.gpu
 DEV = torch.device("cuda:0")
 
 
-def harness(dtype, requests, slots, pos0, new_lens, n_slots=4, max_tokens=1024):
-    """A step context over a fresh cache that holds what `requests` ask for."""
-    from picolm_amd.cache import Cache, CacheSpec, KVGroupSpec, StateGroupSpec
-    from picolm_amd.engine.batch import StepBatch
-    from picolm_amd.parts import CacheBinding, Runtime, StepContext, Workspace
-    kv_req, st_req = requests
-    spec = CacheSpec([KVGroupSpec(1, kv_req.n_kv_heads, kv_req.head_dim, kv_req.window, kv_req.v_head_dim)] if kv_req else [],
-                     [StateGroupSpec(1, tuple(st_req.shape), st_req.dtype)] if st_req else [])
-    rt = Runtime(DEV, dtype)
-    cache = Cache(spec, max_tokens, 512, dtype, DEV, n_slots)
-    for _ in range(n_slots):
-        cache.alloc_slot()
-    cache.reserve_many(slots, [p + n for p, n in zip(pos0, new_lens)])
-    cache.flush()
-    batch = StepBatch(slots, pos0, [[0] * n for n in new_lens], [[] for _ in slots], 10, DEV)
-    ctx = StepContext(rt, batch, cache, Workspace(DEV))
-    ctx.binding = CacheBinding((0, 0) if kv_req else None, (0, 0) if st_req else None, True)
-    return rt, ctx
-
-
 def tol(dtype, ref):
     return (3e-5 if dtype == torch.float32 else 3e-2) * max(1.0, float(np.abs(ref).max()))
 
@@ -44,25 +27,41 @@ def rounded(x, dtype):
     return torch.from_numpy(x).to(dtype).double().numpy()
 
 
+def fetcher(tensors, dtype=torch.bfloat16):
+    from picolm_amd.weights import TensorDict, WeightFetcher
+    return WeightFetcher(TensorDict({k: torch.from_numpy(np.ascontiguousarray(v)).to(dtype) for k, v in tensors.items()}), DEV)
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_rmsnorm_part(dtype):
-    from picolm_amd.parts import RMSNorm
-    from picolm_amd.weights import TensorDict, WeightFetcher
+    from part_harness import PartEngine
+    from picolm_amd.engine import program as Pr
+    from picolm_amd.parts import RMSNorm, Runtime
     rng = np.random.default_rng(0)
     w = rng.standard_normal(96)
-    x = rng.standard_normal((7, 96)) * 4
-    rt, ctx = harness(dtype, (None, None), [0], [0], [7])
+    x = (rng.standard_normal((7, 96)) * 4).astype(np.float32)
+    rt = Runtime(DEV, dtype)
     part = RMSNorm("n.weight", 96, 1e-3)
     assert [(s.name, s.shape, s.init) for s in part.tensor_specs()] == [("n.weight", (96,), "ones")]
-    part.load_all(WeightFetcher(TensorDict({"n.weight": torch.from_numpy(w).to(torch.bfloat16)}), DEV), rt)
-    out = part.forward(ctx, torch.from_numpy(x).float().to(DEV))
-    ref = P.rmsnorm(x.astype(np.float32), rounded(w, torch.bfloat16), 1e-3)
-    assert out.dtype == dtype and np.abs(out.double().cpu().numpy() - ref).max() <= tol(dtype, ref)
+    part.load_all(fetcher({"n.weight": w}), rt)
     shifted = RMSNorm("n.weight", 96, 1e-3, weight_offset=1.0)            # the convention of other architectures
-    shifted.load_all(WeightFetcher(TensorDict({"n.weight": torch.from_numpy(w).float()}), DEV), rt)
-    out = shifted.forward(ctx, torch.from_numpy(x).float().to(DEV))
-    ref = P.rmsnorm(x.astype(np.float32), w.astype(np.float32).astype(np.float64) + 1.0, 1e-3)
-    assert np.abs(out.double().cpu().numpy() - ref).max() <= tol(dtype, ref)
+    shifted.load_all(fetcher({"n.weight": w}, torch.float32), rt)
+    for norm, weights in ((part, rounded(w, torch.bfloat16)), (shifted, w.astype(np.float32).astype(np.float64) + 1.0)):
+        # as a part's input it is a norm that a product may carry; alone it runs as an operation of its own
+        def emit(b, xb, h, norm=norm):
+            src = norm.emit(b, xb)
+            assert src.norm is not None and src.x == xb
+            return b.materialize(src), 96
+        e = PartEngine(dtype, x, emit, parts=[norm])
+        out = e.step(e.alloc(1), [range(7)])
+        ref = P.rmsnorm(x, weights, 1e-3)
+        assert np.abs(out - ref).max() <= tol(dtype, ref)
+    # on the wanted rows only, as before the head
+    e = PartEngine(dtype, x, lambda b, xb, h: (b.materialize(part.emit(b, xb, Pr.ROWS_WANTED), Pr.ROWS_WANTED), 96), parts=[part],
+                   read_rows=Pr.ROWS_WANTED)
+    out = e.step(e.alloc(1), [range(7)], [[5, 0, 5]])
+    ref = P.rmsnorm(x, rounded(w, torch.bfloat16), 1e-3)[[5, 0, 5]]
+    assert np.abs(out - ref).max() <= tol(dtype, ref)
 
 
 def test_rotary_tables():
@@ -80,12 +79,24 @@ def test_rotary_tables():
         assert np.abs(sin.double().cpu().numpy() - rs).max() < 300 * 2.0 ** -24 + 1e-7
 
 
+def attention_engine(dtype, part, rows, **kw):
+    """The attention part alone: input rows in the compute dtype, its output added to zeros."""
+    from part_harness import PartEngine
+    from picolm_amd.engine.program import Rows
+    D = rows.shape[1]
+
+    def emit(b, x, h):
+        res = h.zeros(b, part.o.out_size)
+        part.emit(b, Rows(h.cast(b, x, D)), res)
+        return res, part.o.out_size
+    return PartEngine(dtype, rows, emit, requests=part.cache_requests(), parts=[part], **kw)
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("H,G,d,style,window", [(4, 2, 16, "pairwise", 0), (6, 6, 32, "half", 0), (8, 2, 64, "pairwise", 0),
                                                 (3, 1, 32, "half", 40)])
 def test_attention_part(dtype, H, G, d, style, window):
-    from picolm_amd.parts import Attention, RotaryEmbedding
-    from picolm_amd.weights import TensorDict, WeightFetcher
+    from picolm_amd.parts import Attention, RotaryEmbedding, Runtime
     rng = np.random.default_rng(H * d)
     D = 80
     names = ["a.q_proj.weight", "a.k_proj.weight", "a.v_proj.weight", "a.o_proj.weight"]
@@ -94,23 +105,22 @@ def test_attention_part(dtype, H, G, d, style, window):
     part = Attention("a.", D, H, G, d, position=RotaryEmbedding(d, 1000.0, None, style), window=window)
     assert sorted(s.name for s in part.all_specs()) == sorted(names)
     lens = [70, 9] if window == 0 else [300, 9]         # longer than one chunk of a windowed group's ring
-    rt, ctx = harness(dtype, part.cache_requests(), [2, 0], [0, 0], lens)
-    part.load_all(WeightFetcher(TensorDict({k: torch.from_numpy(v).to(torch.bfloat16) for k, v in w.items()}), DEV), rt)
-    part.prepare(rt, 512)
+    part.load_all(fetcher(w), Runtime(DEV, dtype))
     hs = [rounded(rng.standard_normal((n, D)), dtype) for n in lens]
-    h = torch.from_numpy(np.concatenate(hs)).to(dtype).to(DEV)
-    res = torch.zeros(sum(lens), D, device=DEV)
-    part.forward(ctx, h, res)
+    e = attention_engine(dtype, part, np.concatenate(hs))
+    slots = e.alloc(3)
+    got = e.step([slots[2], slots[0]], [range(lens[0]), range(lens[0], sum(lens))])
     cfg = dict(num_attention_heads=H, num_key_value_heads=G, head_dim=d, rope_theta=1000.0, rope_style=style, window=window)
     pw = {"self_attn." + k[2:]: v for k, v in w.items()}
     ref = np.concatenate([P.attention_block(x, pw, "self_attn.", cfg, np.arange(len(x))) for x in hs])
-    assert np.abs(res.double().cpu().numpy() - ref).max() <= tol(dtype, ref)
+    assert np.abs(got - ref).max() <= tol(dtype, ref)
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_swiglu_and_block_parts(dtype):
-    from picolm_amd.parts import Attention, NoPosition, PreNormBlock, RMSNorm, SwiGLU
-    from picolm_amd.weights import TensorDict, WeightFetcher
+    from part_harness import PartEngine
+    from picolm_amd.engine.program import Rows
+    from picolm_amd.parts import Attention, NoPosition, PreNormBlock, RMSNorm, Runtime, SwiGLU
     rng = np.random.default_rng(5)
     D, F, H, G, d = 48, 104, 3, 3, 16
     shapes = {"f.gate_proj.weight": (F, D), "f.up_proj.weight": (F, D), "f.down_proj.weight": (D, F),
@@ -119,20 +129,27 @@ def test_swiglu_and_block_parts(dtype):
     w = {n: rounded(rng.standard_normal(s) * 0.3, torch.bfloat16) for n, s in shapes.items()}
     ffn = SwiGLU("f.", D, F)
     block = PreNormBlock(RMSNorm("n1", D, 1e-5), Attention("a.", D, H, G, d, position=NoPosition()), RMSNorm("n2", D, 1e-5), ffn)
-    rt, ctx = harness(dtype, block.mixer.cache_requests(), [1], [0], [21])
-    block.load_all(WeightFetcher(TensorDict({k: torch.from_numpy(v).to(torch.bfloat16) for k, v in w.items()}), DEV), rt)
-    block.mixer.prepare(rt, 512)
+    block.load_all(fetcher(w), Runtime(DEV, dtype))
     x = rng.standard_normal((21, D))
     # the feed-forward alone
     hin = rounded(x, dtype)
-    res = torch.zeros(21, D, device=DEV)
-    ffn.forward(ctx, torch.from_numpy(hin).to(dtype).to(DEV), res)
+
+    def emit_ffn(b, xb, h):
+        res = h.zeros(b, D)
+        ffn.emit(b, Rows(h.cast(b, xb, D)), res)
+        return res, D
+    e = PartEngine(dtype, hin, emit_ffn, parts=[ffn])
+    got = e.step(e.alloc(1), [range(21)])
     ref = P.swiglu(hin, w["f.gate_proj.weight"], w["f.up_proj.weight"], w["f.down_proj.weight"])
-    assert np.abs(res.double().cpu().numpy() - ref).max() <= tol(dtype, ref)
+    assert np.abs(got - ref).max() <= tol(dtype, ref)
     # the block: x += attn(norm(x)); x += ffn(norm(x)), here without any rotation
     xf = x.astype(np.float32).astype(np.float64)
-    xt = torch.from_numpy(xf).float().to(DEV)
-    block.forward(ctx, xt)
+
+    def emit_block(b, xb, h):
+        block.emit(b, xb)
+        return xb, D
+    e = PartEngine(dtype, xf, emit_block, requests=block.mixer.cache_requests(), parts=[block, block.mixer])
+    got = e.step([e.alloc(2)[1]], [range(21)])
     hh = P.rmsnorm(xf, w["n1"], 1e-5)
     T = len(xf)
     q = (hh @ w["a.q_proj.weight"].T).reshape(T, H, d)
@@ -140,34 +157,51 @@ def test_swiglu_and_block_parts(dtype):
     v = (hh @ w["a.v_proj.weight"].T).reshape(T, G, d)
     y = xf + P.causal_attention(q, k, v).reshape(T, H * d) @ w["a.o_proj.weight"].T
     y = y + P.swiglu(P.rmsnorm(y, w["n2"], 1e-5), w["f.gate_proj.weight"], w["f.up_proj.weight"], w["f.down_proj.weight"])
-    assert np.abs(xt.double().cpu().numpy() - y).max() <= tol(dtype, y)
+    assert np.abs(got - y).max() <= tol(dtype, y)
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_embedding_and_head_parts(dtype):
-    from picolm_amd.parts import LMHead, TokenEmbedding
-    from picolm_amd.weights import TensorDict, WeightFetcher
+    from part_harness import PartEngine
+    from picolm_amd.engine import program as Pr
+    from picolm_amd.engine.native import NativeEngine
+    from picolm_amd.cache import CacheSpec
+    from picolm_amd.parts import LMHead, Runtime, TokenEmbedding
     rng = np.random.default_rng(6)
     V, D = 131, 40
-    e, hd = rounded(rng.standard_normal((V, D)), torch.bfloat16), rounded(rng.standard_normal((V, D)), torch.bfloat16)
-    rt, ctx = harness(dtype, (None, None), [0], [0], [5])
+    e_, hd = rounded(rng.standard_normal((V, D)), torch.bfloat16), rounded(rng.standard_normal((V, D)), torch.bfloat16)
+    rt = Runtime(DEV, dtype)
+    hrows = rounded(rng.standard_normal((5, D)), dtype)
     for tied, have_head in ((True, False), (False, True), (False, False), (True, True)):
         emb = TokenEmbedding("e", V, D)
         head = LMHead("h", V, D, emb, tied)
-        t = {"e": torch.from_numpy(e).to(torch.bfloat16)}
+        t = {"e": e_}
         if have_head:
-            t["h"] = torch.from_numpy(hd).to(torch.bfloat16)
-        f = WeightFetcher(TensorDict(t), DEV)
+            t["h"] = hd
+        f = fetcher(t)
         emb.load_all(f, rt)
         head.load_all(f, rt)
-        toks = torch.tensor([3, 130, 0, 7, 7], dtype=torch.int32, device=DEV)
-        x = emb.forward(ctx, toks, 5)
-        assert x.dtype == torch.float32 and np.array_equal(x.double().cpu().numpy(), e[[3, 130, 0, 7, 7]])
-        hrows = rounded(rng.standard_normal((5, D)), dtype)
-        lg = head.forward(ctx, torch.from_numpy(hrows).to(dtype).to(DEV))
-        table = hd if (have_head and not tied) else e
+        # the embedding: a program of its lookup and a read-out of the residual rows as "logits"
+        b = Pr.ProgramBuilder(dtype)
+        x = emb.emit(b)
+        lg = b.buffer("logits", V, torch.float32, Pr.ROWS_WANTED)
+
+        def read(view):
+            from picolm_amd.parts.base import rows_view
+            src = rows_view(view.inp, view.n_tokens, view.in_row_bytes, torch.float32, DEV)
+            rows_view(view.out, view.n_wanted, view.out_row_bytes, torch.float32, DEV)[:, :D] = src
+        b.call(read, out=lg, inp=x, rows=Pr.ROWS_WANTED)
+        b.logits_buffer = lg
+        eng = NativeEngine(b.finish(V, CacheSpec([], [])), 64, 64, 1, DEV)
+        got = eng.step([eng.slot_alloc()], [[3, 130, 0, 7, 7]], [list(range(5))])[:, :D]
+        assert got.dtype == torch.float32 and np.array_equal(got.double().cpu().numpy(), e_[[3, 130, 0, 7, 7]])
+        # the head: wanted rows in the compute dtype in, logits out
+        pe = PartEngine(dtype, hrows, lambda b, xb, h: (head.emit(b, h.cast(b, xb, D, Pr.ROWS_WANTED, "norm.final")) or "logits", V),
+                        parts=[head])
+        got = pe.step(pe.alloc(1), [range(5)])
+        table = hd if (have_head and not tied) else e_
         ref = hrows @ table.T
-        assert np.abs(lg.double().cpu().numpy() - ref).max() <= tol(dtype, ref)
+        assert np.abs(got[:, :V] - ref).max() <= tol(dtype, ref)
 
 
 # ------------------------------------------------------------------------------------------- a toy architecture
@@ -176,6 +210,7 @@ def test_toy_architecture_with_a_stateful_mixer(tmp_path):
     output at a position is W times the mean of all inputs so far.  It needs no keys or
     values, only a state row per slot.  The layer order names its block twice and the second
     call has a state entry of its own."""
+    from picolm_amd import SamplingParams
     from picolm_amd.config import register_architecture, unregister_architecture
     from picolm_amd.engine import DecoderModel, Session, load_model
     from picolm_amd.parts import LMHead, Mixer, PreNormBlock, RMSNorm, StateRequest, SwiGLU, TokenEmbedding
@@ -249,6 +284,7 @@ def test_toy_architecture_with_a_stateful_mixer(tmp_path):
         reqs = [tiny.random_tokens(rng, n, 77) for n in (19, 3, 40)]
         truth = [plain(r) for r in reqs]
         s = Session(model, max_tokens=512, n_slots=3)
+        assert tuple(s.cache.state[0].shape) == (2, 3, 41)         # the engine holds the state: [entry][slot][D + 1]
         slots = s.begin(3)                                        # whole, as one unequal batch
         got = s.step(slots, reqs, [list(range(len(r))) for r in reqs]).double().cpu().numpy()
         assert np.abs(got - np.concatenate(truth)).max() < 5e-5
@@ -264,19 +300,27 @@ def test_toy_architecture_with_a_stateful_mixer(tmp_path):
                 assert np.abs(out[k] - truth[i][pos[i]]).max() < 5e-5
                 pos[i] += 1
             live = [i for i in live if pos[i] < len(reqs[i])]
+        assert s.recorded_steps() == 0                            # a part that runs torch operators: its steps are launched
+        s.release(slots)
+        # the library's generation loop steps it too: greedy tokens against the plain implementation
+        toks, _ = s.engine.generate([r[:5] for r in reqs], 6, SamplingParams(), [], batch_size=2)
+        for r, got in zip(reqs, toks):
+            seq = list(r[:5])
+            for t in got:
+                row = plain(np.asarray(seq))[-1]
+                assert row[t] >= row.max() - 1e-4
+                seq.append(t)
     finally:
         unregister_architecture("ToyRunningMeanLM")
 
 
-@pytest.mark.parametrize("native", [True, False])
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-def test_layer_order_names_a_block_twice_and_lets_a_call_read_anothers_cache(dtype, native, tmp_path):
+def test_layer_order_names_a_block_twice_and_lets_a_call_read_anothers_cache(dtype, tmp_path):
     """The order of layers is data.  Three blocks of the library's own parts run as four calls:
     block 0, block 1, block 0 again (the same weights, keys and values of its own) and block 2,
     whose attention writes nothing and reads the keys and values that the call of block 1 left
     (its own k and v projections are loaded and unused).  Whole prompts as an unequal batch, then
-    token by token from a cut, in the library's step and in the one from Python, against the
-    plain functions."""
+    token by token from a cut, against the plain functions."""
     from picolm_amd.config import LlamaConfig, register_architecture, unregister_architecture
     from picolm_amd.engine import DecoderModel, LayerCall, Session, load_model
     from picolm_amd.parts import Attention, LMHead, PreNormBlock, RMSNorm, RotaryEmbedding, SwiGLU, TokenEmbedding
@@ -340,8 +384,7 @@ def test_layer_order_names_a_block_twice_and_lets_a_call_read_anothers_cache(dty
         reqs = [tiny.random_tokens(rng, n, 301) for n in (150, 9, 70)]
         truth = [plain(r) for r in reqs]
         tol_ = lambda t: tiny.tolerance(dtype, t, tiny.spread(192, 0.06))
-        s = Session(model, max_tokens=1024, n_slots=3, native=native)
-        assert (s.engine is not None) == native
+        s = Session(model, max_tokens=1024, n_slots=3)
         slots = s.begin(3)
         got = s.step(slots, reqs, [list(range(len(r))) for r in reqs]).double().cpu().numpy()
         row = 0
@@ -368,7 +411,7 @@ def test_toy_mixer_whose_values_are_wider_than_its_keys(tmp_path):
     """A one-head attention defined here with keys of 16 and values of 24: the cache gives its
     group keys and values of their own sizes.  Whole prompts as an unequal batch, then the same
     requests cut into a prompt and single tokens in slots that were used before."""
-    from picolm_amd.cache.slots import PAGE_TOKENS
+    from picolm_amd.cache import PAGE_TOKENS
     from picolm_amd.config import register_architecture, unregister_architecture
     from picolm_amd.engine import DecoderModel, Session, load_model
     from picolm_amd.parts import KVRequest, LMHead, Mixer, PreNormBlock, RMSNorm, SwiGLU, TokenEmbedding
@@ -401,7 +444,7 @@ def test_toy_mixer_whose_values_are_wider_than_its_keys(tmp_path):
             return KVRequest(1, DK, 0, DV), None
 
         def forward(self, ctx, h, residual):
-            k_pages, v_pages, table, _ = ctx.kv()          # [page][1][64][DK], [page][1][DV][64]
+            k_pages, v_pages, table, _ = ctx.kv()          # [page][1][64][DK], [page][1][DV][64]: the engine's memory
             assert k_pages.shape[-1] == DK and v_pages.shape[-2] == DV
             b, row = ctx.batch, 0
             for slot, p0, n in zip(b.slots, b.pos0, b.n_new):
@@ -433,7 +476,6 @@ def test_toy_mixer_whose_values_are_wider_than_its_keys(tmp_path):
         model = load_model(d, dtype="float32")
         (group,) = model.cache_spec.kv_groups
         assert (group.n_entries, group.head_dim, group.value_dim) == (2, DK, DV)
-        assert model.program() is None            # a part without `emit`: stepped part by part
         w = tiny.read_weights_f64(d)
 
         def plain(tokens):
@@ -475,12 +517,10 @@ def test_toy_mixer_whose_values_are_wider_than_its_keys(tmp_path):
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_toy_position_encoding_that_is_no_rotation(dtype):
     """A position encoding defined here: it damps queries and keys with their position.  The
-    attention part takes it through `PositionEncoding.apply`, in a prefill step and in decode steps
-    (where the bfloat16 kernel that writes the cache itself gets rows that are already encoded)."""
-    from picolm_amd.cache.slots import PAGE_TOKENS
-    from picolm_amd.engine.batch import StepBatch
-    from picolm_amd.parts import Attention, PositionEncoding
-    from picolm_amd.weights import TensorDict, WeightFetcher
+    attention part emits it as a call of its `apply` on the float rows of q, k, v, between the
+    product and the attention operation, in a prefill step and in decode steps (where the
+    bfloat16 kernel that writes the cache itself gets rows that are already encoded)."""
+    from picolm_amd.parts import Attention, PositionEncoding, Runtime
 
     class Damping(PositionEncoding):
         """q and k of the token at position p are multiplied by 1 / (1 + p / 32)."""
@@ -496,10 +536,9 @@ def test_toy_position_encoding_that_is_no_rotation(dtype):
     w = {n: rounded(rng.standard_normal(s) * 0.2, torch.bfloat16) for n, s in zip(names, shapes)}
     part = Attention("a.", D, H, G, d, position=Damping())
     lens, tail = [70, 9], 3
-    rt, ctx = harness(dtype, part.cache_requests(), [2, 0], [0, 0], [n + tail for n in lens])
-    part.load_all(WeightFetcher(TensorDict({k: torch.from_numpy(v).to(torch.bfloat16) for k, v in w.items()}), DEV), rt)
-    part.prepare(rt, 512)
+    part.load_all(fetcher(w), Runtime(DEV, dtype))
     hs = [rounded(rng.standard_normal((n + tail, D)), dtype) for n in lens]
+    first = [0, lens[0] + tail]                         # where each sequence's rows start in the table
 
     def plain(x):
         T = len(x)
@@ -509,18 +548,18 @@ def test_toy_position_encoding_that_is_no_rotation(dtype):
         v = (x @ w["a.v_proj.weight"].T).reshape(T, G, d)
         return P.causal_attention(q, k, v).reshape(T, H * d) @ w["a.o_proj.weight"].T
     ref = [plain(x) for x in hs]
+    e = attention_engine(dtype, part, np.concatenate(hs))
+    assert sum(op.kind == 5 for op in e.builder.ops) == 4          # the cast, the zeros, the encoding and the read-out are calls
+    slots = e.alloc(3)
+    slots = [slots[2], slots[0]]
     # the prompts in one step, then one token each
-    ctx.batch = StepBatch([2, 0], [0, 0], [[0] * n for n in lens], [[], []], 10, DEV)
-    res = torch.zeros(sum(lens), D, device=DEV)
-    part.forward(ctx, torch.from_numpy(np.concatenate([x[:n] for x, n in zip(hs, lens)])).to(dtype).to(DEV), res)
+    got = e.step(slots, [range(f, f + n) for f, n in zip(first, lens)])
     want = np.concatenate([r[:n] for r, n in zip(ref, lens)])
-    assert np.abs(res.double().cpu().numpy() - want).max() <= tol(dtype, want)
+    assert np.abs(got - want).max() <= tol(dtype, want)
     for j in range(tail):
-        ctx.batch = StepBatch([2, 0], [n + j for n in lens], [[0], [0]], [[], []], 10, DEV)
-        res = torch.zeros(2, D, device=DEV)
-        part.forward(ctx, torch.from_numpy(np.stack([x[n + j] for x, n in zip(hs, lens)])).to(dtype).to(DEV), res)
+        got = e.step(slots, [[f + n + j] for f, n in zip(first, lens)])
         want = np.stack([r[n + j] for r, n in zip(ref, lens)])
-        assert np.abs(res.double().cpu().numpy() - want).max() <= tol(dtype, want)
+        assert np.abs(got - want).max() <= tol(dtype, want)
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
@@ -603,7 +642,6 @@ def test_toy_norm_that_is_no_rmsnorm(dtype, tmp_path):
         truth = [plain(r) for r in reqs]
         tol_ = lambda t: tiny.tolerance(dtype, t, tiny.spread(128, 0.08))
         s = Session(model, max_tokens=512, n_slots=3)
-        assert s.engine is None                       # a part the library has no operations for: stepped from Python
         slots = s.begin(3)
         got = s.step(slots, reqs, [list(range(len(r))) for r in reqs]).double().cpu().numpy()
         row = 0
@@ -629,9 +667,11 @@ def test_toy_norm_that_is_no_rmsnorm(dtype, tmp_path):
 def test_toy_feed_forward_with_routing():
     """A feed-forward defined here: two gated experts and a router that sends every row to the
     expert with the larger logit (router logits in float).  It is built from the library's Linear
-    and SwiGLU parts and runs in a block next to attention, without a change to the library."""
-    from picolm_amd.parts import FeedForward, Linear, SwiGLU
-    from picolm_amd.weights import TensorDict, WeightFetcher
+    and SwiGLU parts, whose `forward` it calls on the rows it picks, and runs inside the engine's
+    step as a call of its own `forward`, without a change to the library."""
+    from part_harness import PartEngine
+    from picolm_amd.engine.program import Rows
+    from picolm_amd.parts import FeedForward, Linear, Runtime, SwiGLU
 
     class TwoExperts(FeedForward):
         def __init__(self, prefix, D, F):
@@ -661,16 +701,20 @@ def test_toy_feed_forward_with_routing():
     w = {n: rounded(rng.standard_normal(s) * 0.3, torch.bfloat16) for n, s in shapes.items()}
     ffn = TwoExperts("f.", D, F)
     assert sorted(s.name for s in ffn.all_specs()) == sorted(shapes)
-    rt, ctx = harness(torch.bfloat16, (None, None), [0], [0], [T])
-    ffn.load_all(WeightFetcher(TensorDict({k: torch.from_numpy(v).to(torch.bfloat16) for k, v in w.items()}), DEV), rt)
+    ffn.load_all(fetcher(w), Runtime(DEV, torch.bfloat16))
     x = rounded(rng.standard_normal((T, D)), torch.bfloat16)
-    res = torch.zeros(T, D, device=DEV)
-    ffn.forward(ctx, torch.from_numpy(x).to(torch.bfloat16).to(DEV), res)
+
+    def emit(b, xb, h):
+        res = h.zeros(b, D)
+        ffn.emit(b, Rows(h.cast(b, xb, D)), res)
+        return res, D
+    e = PartEngine(torch.bfloat16, x, emit, parts=[ffn])
+    got = e.step(e.alloc(1), [range(T)])
     choice = (x @ w["f.router.weight"].T).argmax(axis=1)
     assert 0 < choice.sum() < T                          # both experts get rows
     ref = np.stack([P.swiglu(x[t:t + 1], w[f"f.experts.{c}.gate_proj.weight"], w[f"f.experts.{c}.up_proj.weight"],
                              w[f"f.experts.{c}.down_proj.weight"])[0] for t, c in enumerate(choice)])
-    assert np.abs(res.double().cpu().numpy() - ref).max() <= tol(torch.bfloat16, ref)
+    assert np.abs(got - ref).max() <= tol(torch.bfloat16, ref)
 
 
 # ------------------------------------------------------------------------------------------- a window's ring, lap after lap
@@ -680,7 +724,7 @@ def test_a_window_of_keys_through_several_laps_of_its_ring(dtype, window, tmp_pa
     """A decoder whose attention keeps a window of keys: its cache group is a ring of pages per
     slot.  A prompt longer than one chunk, then decoding far past the ring's first lap, launched
     step by step and replayed from the recording; every step against the plain implementation
-    with the same window.  (Such a model is stepped from Python: the engine keeps all keys.)"""
+    with the same window."""
     from picolm_amd import LlamaConfig
     from picolm_amd.engine import DecoderModel, Session
     from picolm_amd.parts import (Attention, LMHead, PreNormBlock, RMSNorm, RotaryEmbedding, Runtime, SwiGLU, TokenEmbedding)
@@ -707,7 +751,6 @@ def test_a_window_of_keys_through_several_laps_of_its_ring(dtype, window, tmp_pa
     ref = P.forward(tiny.read_weights_f64(d), dict(tiny.read_config(d), window=window), toks)
     for graphs in (False, True):
         s = Session(model, max_tokens=2048, graphs=graphs)
-        assert s.engine is None                                   # a window is stepped from Python
         ring = s.cache.kv[0].ring_pages
         assert ring < s.cache.max_pages and 64 * ring < n_all - 64      # decoding laps the ring more than once
         [a] = s.begin(1)
@@ -718,7 +761,7 @@ def test_a_window_of_keys_through_several_laps_of_its_ring(dtype, window, tmp_pa
             err = np.abs(got[0] - ref[j]).max()
             assert err <= tol(dtype, ref), (window, dtype, "graphs", graphs, "position", j, err)
         assert (s.recorded_steps() > 0) == graphs
-        assert len(s.cache.kv[0].book.pages[a]) == ring           # the slot never holds more than its ring
+        assert len(s.engine.slot_pages(0, a)) == ring             # the slot never holds more than its ring
         s.release([a])
 
 
@@ -729,18 +772,15 @@ def test_the_edge_of_a_window_in_decode_steps_past_the_first_lap(window):
     row's value while the row is inside the window and small once it has left.  The last step
     that sees it has it exactly at position - window + 1; the next one must drop it, also when its
     page of the ring has meanwhile been written again."""
-    from picolm_amd.engine.batch import StepBatch
-    from picolm_amd.parts import Attention
-    from picolm_amd.weights import TensorDict, WeightFetcher
+    from picolm_amd.cache import window_ring_pages
+    from picolm_amd.parts import Attention, Runtime
     d = 16
-    eye = torch.eye(d)
+    eye = np.eye(d)
     part = Attention("a.", d, 1, 1, d, window=window)
-    from picolm_amd.cache.kv import window_ring_pages
     ring = window_ring_pages(window)
-    n_prompt, n_all = 300, 64 * ring + 5 + window + 8          # (the harness's cache takes sequences of 512)
-    rt, ctx = harness(torch.float32, part.cache_requests(), [1], [0], [n_all], max_tokens=1024)
-    assert ctx.cache.kv[0].ring_pages == ring and n_all <= 512
-    part.load_all(WeightFetcher(TensorDict({f"a.{n}_proj.weight": eye.clone() for n in "qkvo"}), DEV), rt)
+    n_prompt, n_all = 300, 64 * ring + 5 + window + 8          # (the cache takes sequences of 512)
+    assert n_all <= 512
+    part.load_all(fetcher({f"a.{n}_proj.weight": eye for n in "qkvo"}), Runtime(DEV, torch.float32))
     rng = np.random.default_rng(window)
     u = np.zeros(d)
     u[3] = 1.0
@@ -749,19 +789,281 @@ def test_the_edge_of_a_window_in_decode_steps_past_the_first_lap(window):
     big = [305, 64 * ring + 5]                     # one in the first lap, one just after the ring has wrapped; never both in a window
     for j in big:
         h[j] = 60.0 * u                            # score 60 / 4 = 15 against about 0.25 for the others
+    h = h.astype(np.float32).astype(np.float64)
     ref = P.causal_attention(h[:, None, :], h[:, None, :], h[:, None, :], window)[:, 0, :]
-    ctx.batch = StepBatch([1], [0], [[0] * n_prompt], [[]], 10, DEV)
-    res = torch.zeros(n_prompt, d, device=DEV)
-    part.forward(ctx, torch.from_numpy(h[:n_prompt]).float().to(DEV), res)
-    assert np.abs(res.double().cpu().numpy() - ref[:n_prompt]).max() <= 1e-4
+    e = attention_engine(torch.float32, part, h, max_tokens=1024)
+    [_, a] = e.alloc(2)
+    got = e.step([a], [range(n_prompt)])
+    assert np.abs(got - ref[:n_prompt]).max() <= 1e-4
+    assert len(e.engine.slot_pages(0, a)) <= ring
     for p in range(n_prompt, n_all):
-        ctx.batch = StepBatch([1], [p], [[0]], [[]], 10, DEV)
-        res = torch.zeros(1, d, device=DEV)
-        part.forward(ctx, torch.from_numpy(h[p:p + 1]).float().to(DEV), res)
-        out = res.double().cpu().numpy()[0]
+        out = e.step([a], [[p]])[0]
         assert np.abs(out - ref[p]).max() <= 1e-4, p
         for j in big:
             if p == j + window - 1:
                 assert out[3] > 50.0, (p, "the key at position - window + 1 is visible")
             if p == j + window:
                 assert out[3] < 2.0, (p, "the key at position - window is dropped")
+    assert len(e.engine.slot_pages(0, a)) == ring
+
+
+# ------------------------------------------------------------------------------------------- parts with kernels of their own
+class ToyConfig:
+    def __init__(self, d):
+        self.d = dict(d)
+        self.hidden_size, self.vocab_size, self.intermediate_size = d["hidden_size"], d["vocab_size"], d["intermediate_size"]
+        self.max_position_embeddings = d["max_position_embeddings"]
+        self.torch_dtype = "bfloat16"
+        self.eos_token_ids = ()
+
+    def to_dict(self):
+        return dict(self.d)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_toy_parts_with_hip_kernels_of_their_own_run_in_the_engines_step(dtype, tmp_path):
+    """A mixer with state of its own and a norm that is no RMSNorm, each a HIP kernel and a C
+    function in a library beside the tests (tests/toy_parts).  Their parts, defined here, emit a
+    called operation that names the C function; the engine hands it the running step.  Nothing
+    of the library changes: the model is registered, built, loaded from a random folder and
+    stepped through Session (prompts whole, from a cut token by token in reused slots, with decode
+    steps that are recorded and replayed) and through the library's generation loop."""
+    from toy_parts import build as toy_build
+    from picolm_amd import SamplingParams
+    from picolm_amd.config import register_architecture, unregister_architecture
+    from picolm_amd.engine import DecoderModel, Session, load_model
+    from picolm_amd.engine.program import Rows
+    from picolm_amd.parts import LMHead, Mixer, Norm, PreNormBlock, RMSNorm, StateRequest, SwiGLU, TokenEmbedding
+    from picolm_amd.weights import TensorSpec, write_random_model
+    toy = toy_build.load()
+
+    class MeanArgs(ctypes.Structure):
+        _fields_ = [("w", ctypes.c_void_p), ("D", ctypes.c_int32), ("in_bf16", ctypes.c_int32)]
+
+    class NormArgs(ctypes.Structure):
+        _fields_ = [("w", ctypes.c_void_p), ("b", ctypes.c_void_p), ("D", ctypes.c_int32), ("eps", ctypes.c_float),
+                    ("out_bf16", ctypes.c_int32)]
+
+    class RunningMean(Mixer):
+        def __init__(self, name, D):
+            self.name, self.D, self.w = name, D, None
+
+        def tensor_specs(self):
+            return [TensorSpec(self.name, (self.D, self.D))]
+
+        def load(self, fetch, runtime):
+            self.w = fetch.get(self.name).float().contiguous()
+
+        def cache_requests(self):
+            return None, StateRequest((self.D + 1,), torch.float32)
+
+        def emit(self, b, src, x, out_norm=None, out_norm_when=0):
+            h = b.materialize(src)
+            args = MeanArgs(self.w.data_ptr(), self.D, int(b.buffer_dtype(h) == torch.bfloat16))
+            b.keep.append(self.w)
+            b.call(toy.toy_running_mean, out=x, inp=h, user=args, uses_state=True, recordable=True)
+
+    class CenteredNorm(Norm):
+        def __init__(self, name, size, eps):
+            self.name, self.size, self.eps = name, size, eps
+            self.weight = self.bias = None
+
+        def tensor_specs(self):
+            return [TensorSpec(self.name + ".weight", (self.size,), init="ones"), TensorSpec(self.name + ".bias", (self.size,))]
+
+        def load(self, fetch, runtime):
+            self.weight = fetch.get(self.name + ".weight").float().contiguous()
+            self.bias = fetch.get(self.name + ".bias").float().contiguous()
+
+        def emit(self, b, x, rows=0):
+            h = b.buffer("norm.final" if rows else "norm.out", self.size, b.dtype, rows)
+            args = NormArgs(self.weight.data_ptr(), self.bias.data_ptr(), self.size, self.eps, int(b.dtype == torch.bfloat16))
+            b.keep += [self.weight, self.bias]
+            b.call(toy.toy_centered_norm, out=h, inp=x, rows=rows, user=args, recordable=True)
+            return Rows(h)
+
+    def build(cfg):
+        D = cfg.hidden_size
+        emb = TokenEmbedding("emb.weight", cfg.vocab_size, D)
+        block = PreNormBlock(CenteredNorm("norm1", D, 1e-5), RunningMean("mean.weight", D),
+                             RMSNorm("norm2.weight", D, 1e-5), SwiGLU("ffn.", D, cfg.intermediate_size))
+        return DecoderModel(cfg, emb, [block], CenteredNorm("final", D, 1e-5),
+                            LMHead("head.weight", cfg.vocab_size, D, emb, tied=True), order=[0, 0])
+
+    name = "ToyKernelsLM"
+    register_architecture(name, ToyConfig, build)
+    try:
+        cfg = ToyConfig(dict(architectures=[name], hidden_size=40, vocab_size=77, intermediate_size=56, max_position_embeddings=256))
+        d = write_random_model(cfg, str(tmp_path / "toy"), seed=4, std=0.3)
+        model = load_model(d, dtype=dtype)
+        w = tiny.read_weights_f64(d)
+
+        def centered(x, n):
+            xc = x - x.mean(axis=1, keepdims=True)
+            return xc / np.sqrt((xc * xc).mean(axis=1, keepdims=True) + 1e-5) * w[n + ".weight"] + w[n + ".bias"]
+
+        def plain(tokens):
+            x = w["emb.weight"][tokens]
+            for _ in range(2):
+                hh = centered(x, "norm1")
+                mean = np.cumsum(hh, axis=0) / np.arange(1, len(tokens) + 1)[:, None]
+                x = x + mean @ w["mean.weight"].T
+                x = x + P.swiglu(P.rmsnorm(x, w["norm2.weight"], 1e-5), w["ffn.gate_proj.weight"],
+                                 w["ffn.up_proj.weight"], w["ffn.down_proj.weight"])
+            return centered(x, "final") @ w["emb.weight"].T
+        rng = np.random.default_rng(7)
+        reqs = [tiny.random_tokens(rng, n, 77) for n in (19, 3, 40)]
+        truth = [plain(r) for r in reqs]
+        bound = lambda t: tiny.tolerance(dtype, t, tiny.spread(40, 0.3)) * (1 if dtype == "float32" else 2)
+        s = Session(model, max_tokens=512, n_slots=3)
+        assert s.engine.program.recordable
+        slots = s.begin(3)                                        # whole, as one unequal batch; some rows wanted, some not
+        got = s.step(slots, reqs, [list(range(len(r))) for r in reqs]).double().cpu().numpy()
+        row = 0
+        for r, t in zip(reqs, truth):
+            assert np.abs(got[row:row + len(r)] - t).max() <= bound(t)
+            row += len(r)
+        s.release(slots)
+        slots = s.begin(3)                                        # reused slots: state starts from zero again
+        cut = [7, 1, 33]
+        got = s.step(slots, [r[:c] for r, c in zip(reqs, cut)], [[0], [], [5, 32]]).double().cpu().numpy()
+        assert np.abs(got - np.stack([truth[0][0], truth[2][5], truth[2][32]])).max() <= bound(truth[2])
+        pos = dict(zip(range(3), cut))
+        live = [0, 1, 2]
+        while live:
+            out = s.step([slots[i] for i in live], [[reqs[i][pos[i]]] for i in live]).double().cpu().numpy()
+            for k, i in enumerate(live):
+                assert np.abs(out[k] - truth[i][pos[i]]).max() <= bound(truth[i]), (i, pos[i])
+                pos[i] += 1
+            live = [i for i in live if pos[i] < len(reqs[i])]
+        assert s.recorded_steps() >= 2                            # three, two and one sequence: each shape recorded at its second use
+        s.release(slots)
+        if dtype == "float32":
+            toks, finish = s.engine.generate([r[:5] for r in reqs], 6, SamplingParams(), [], batch_size=2)
+            assert finish == ["length"] * 3
+            for r, got in zip(reqs, toks):
+                seq = list(r[:5])
+                for t in got:
+                    row = plain(np.asarray(seq))[-1]
+                    assert row[t] >= row.max() - 1e-4
+                    seq.append(t)
+    finally:
+        unregister_architecture(name)
+
+
+def test_a_called_operation_that_fails_fails_the_step():
+    """What a Python part raises inside the engine's step comes back to the step's caller as that
+    exception; the sequences stay where they were."""
+    from part_harness import PartEngine
+    from picolm_amd.parts import FeedForward
+
+    class Broken(FeedForward):
+        def forward(self, ctx, h, residual):
+            if ctx.batch.T > 3:
+                raise ZeroDivisionError("more rows than this toy takes")
+            residual += 1.0
+    from picolm_amd.engine.program import Rows
+    ffn = Broken()
+
+    def emit(b, xb, h):
+        ffn.emit(b, Rows(h.cast(b, xb, 8)), xb)
+        return xb, 8
+    e = PartEngine(torch.float32, np.zeros((6, 8), np.float32), emit, parts=[ffn])
+    [a] = e.alloc(1)
+    assert np.array_equal(e.step([a], [range(3)]), np.ones((3, 8)))
+    with pytest.raises(ZeroDivisionError, match="more rows"):
+        e.step([a], [range(4)])
+    assert e.engine.length(a) == 3
+    assert np.array_equal(e.step([a], [range(2)]), np.ones((2, 8)))
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_subclasses_of_the_librarys_parts(dtype, tmp_path):
+    """A subclass that changes a constant keeps the engine's own operations (and recorded decode
+    steps); a subclass that changes `forward` runs through its `forward`.  Here: an attention with
+    another scale, an RMSNorm whose weights are offset by a half, and a gated feed-forward whose
+    output is halved."""
+    from picolm_amd import LlamaConfig
+    from picolm_amd.config import register_architecture, unregister_architecture
+    from picolm_amd.engine import DecoderModel, Session, load_model
+    from picolm_amd.engine.program import OP_CALL
+    from picolm_amd.parts import Attention, LMHead, PreNormBlock, RMSNorm, RotaryEmbedding, SwiGLU, TokenEmbedding
+    from picolm_amd.weights import write_random_model
+
+    class SharpAttention(Attention):
+        def __init__(self, *a, **kw):
+            super().__init__(*a, **kw)
+            self.scale *= 1.5
+
+    class OffsetNorm(RMSNorm):
+        def __init__(self, name, size, eps):
+            super().__init__(name, size, eps, weight_offset=0.5)
+
+    class HalvedSwiGLU(SwiGLU):
+        def forward(self, ctx, h, residual):
+            out = torch.zeros_like(residual)
+            super().forward(ctx, h, out)
+            residual += 0.5 * out
+
+    def build(cfg, halved=True):
+        D = cfg.hidden_size
+        rotary = RotaryEmbedding(cfg.head_dim, cfg.rope_theta, None, cfg.rope_style)
+        blocks = []
+        for l in range(2):
+            q = f"model.layers.{l}."
+            ffn = (HalvedSwiGLU if halved and l == 1 else SwiGLU)(q + "mlp.", D, cfg.intermediate_size)
+            blocks.append(PreNormBlock(OffsetNorm(q + "input_layernorm.weight", D, cfg.rms_norm_eps),
+                                       SharpAttention(q + "self_attn.", D, cfg.num_attention_heads, cfg.num_key_value_heads,
+                                                      cfg.head_dim, position=rotary),
+                                       RMSNorm(q + "post_attention_layernorm.weight", D, cfg.rms_norm_eps), ffn))
+        emb = TokenEmbedding("model.embed_tokens.weight", cfg.vocab_size, D)
+        return DecoderModel(cfg, emb, blocks, RMSNorm("model.norm.weight", D, cfg.rms_norm_eps),
+                            LMHead("lm_head.weight", cfg.vocab_size, D, emb, True))
+
+    c = dict(architectures=["ToySubclassLM"], hidden_size=128, num_attention_heads=4, num_key_value_heads=2, head_dim=32,
+             intermediate_size=192, num_hidden_layers=2, vocab_size=211, rms_norm_eps=1e-5, rope_theta=10000.0,
+             max_position_embeddings=256, tie_word_embeddings=True, torch_dtype="bfloat16")
+    cfg = LlamaConfig.from_dict(c)
+    register_architecture("ToySubclassLM", LlamaConfig.from_dict, build)
+    try:
+        d = write_random_model(cfg, str(tmp_path / "sub"), seed=5, std=0.08)
+    finally:
+        unregister_architecture("ToySubclassLM")
+    w = tiny.read_weights_f64(d)
+    pc = dict(c, rope_style=cfg.rope_style)
+
+    def plain(tokens, halved):
+        pos = np.arange(len(tokens))
+        x = w["model.embed_tokens.weight"][np.asarray(tokens)]
+        for l in range(2):
+            q = f"model.layers.{l}."
+            h = P.rmsnorm(x, w[q + "input_layernorm.weight"] + 0.5, 1e-5)
+            sharp = {k: (v * 1.5 if k == q + "self_attn.q_proj.weight" else v) for k, v in w.items() if k.startswith(q)}
+            x = x + P.attention_block(h, sharp, q + "self_attn.", pc, pos)      # (a scale on the scores is a scale on q)
+            h = P.rmsnorm(x, w[q + "post_attention_layernorm.weight"], 1e-5)
+            y = P.swiglu(h, w[q + "mlp.gate_proj.weight"], w[q + "mlp.up_proj.weight"], w[q + "mlp.down_proj.weight"])
+            x = x + (0.5 * y if halved and l == 1 else y)
+        return P.rmsnorm(x, w["model.norm.weight"], 1e-5) @ w["model.embed_tokens.weight"].T
+    rng = np.random.default_rng(9)
+    reqs = [tiny.random_tokens(rng, n, 211) for n in (70, 5, 33)]
+    for halved in (False, True):
+        register_architecture("ToySubclassLM", LlamaConfig.from_dict, lambda cf: build(cf, halved))
+        try:
+            model = load_model(d, dtype=dtype)
+        finally:
+            unregister_architecture("ToySubclassLM")
+        truth = [plain(r, halved) for r in reqs]
+        tol_ = lambda t: tiny.tolerance(dtype, t, tiny.spread(128, 0.08))
+        s = Session(model, max_tokens=512, n_slots=3)
+        assert sum(op.kind == OP_CALL for op in s.engine.program.ops) == int(halved)       # only the changed forward is a call
+        slots = s.begin(3)
+        cut = [50, 2, 20]
+        s.step(slots, [r[:c_] for r, c_ in zip(reqs, cut)])
+        pos, live = dict(zip(range(3), cut)), [0, 1, 2]
+        while live:
+            out = s.step([slots[i] for i in live], [[reqs[i][pos[i]]] for i in live]).double().cpu().numpy()
+            for k, i in enumerate(live):
+                assert np.abs(out[k] - truth[i][pos[i]]).max() <= tol_(truth[i]), (halved, i, pos[i])
+                pos[i] += 1
+            live = [i for i in live if pos[i] < len(reqs[i])]
+        assert (s.recorded_steps() > 0) == (not halved)
