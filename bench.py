@@ -12,8 +12,9 @@ step over the batch from the cache, the sampler, and the hand-over of the sample
 are random bf16 made on the GPU, prompts are seeded uniform-random token ids; they go through the
 model as the generation loop sends them (one step, or the steps of its token budget).  Prints one
 JSON line: tokens a second, the step's fraction of HBM's peak, a prefill of 2,048 tokens, further
-batch sizes, and for each class of kernels (decode products, decode attention, prefill products,
-prefill attention) what it reaches against the nominal peak and against what a plain read or a
+batch sizes (each right after its prompts, and with every sequence near 2,000 tokens and near the
+full context), whole generation loops (the library's own and the Python one), and for each class
+of kernels (decode products, decode attention, prefill products, prefill attention) what it reaches against the nominal peak and against what a plain read or a
 register-only MFMA loop reaches on the same GPU (picolm prints effective weight throughput of its
 layers likewise, picolm/picolm.c:305-317; its harness discards a warm-up and takes medians,
 picolm/bench.zsh:46, :272).
@@ -104,6 +105,9 @@ def main() -> int:
     ap.add_argument("--no-points", action="store_true", help="skip the further batch sizes, the prefill and the kernel classes")
     ap.add_argument("--prefill-only", action="store_true", help="run only the prefill (for profiling)")
     ap.add_argument("--batch-only", action="store_true", help="run only the decode at --batch (for profiling)")
+    ap.add_argument("--sweep", action="store_true",
+                    help="instead of the record: prefill of 128 to 32,768 tokens and decode at contexts of 16,384 to 131,072 "
+                         "tokens, as one JSON line")
     ap.add_argument("--sampling", choices=["greedy", "picolm"], default="greedy",
                     help="greedy (the measured default) or picolm's command-line defaults: temperature 0.8, top_k 40, top_p 0.9, min_p 0.05")
     ap.add_argument("--prefill-tokens", type=int, default=PREFILL_TOKENS,
@@ -126,7 +130,7 @@ def main() -> int:
 
     from picolm_amd import LlamaConfig, kernels
     from picolm_amd.engine import Session, random_model
-    from picolm_amd.generation import SessionStepper
+    from picolm_amd.generation import SessionStepper, generate
     from picolm_amd.sampling import Sampler, SamplingParams
     from picolm_amd.sampling.params import CLI_DEFAULTS
 
@@ -151,11 +155,15 @@ def main() -> int:
     prompt_lo, prompt_hi = (int(x) for x in args.prompt_range.split(",")) if args.prompt_range else shape["prompt_range"]
     context = args.context
 
-    def decode_run(n_seq: int, n_steps: int, n_warm: int, time_ops: bool = False):
-        lens = [int(x) for x in rng.integers(prompt_lo, prompt_hi + 1, size=n_seq)]
+    def decode_run(n_seq: int, n_steps: int, n_warm: int, time_ops: bool = False, prompt_len: int = 0, seq_len: int = 0):
+        """Decode steps of `n_seq` sequences after prompts of random lengths in the shape's range, or
+        of `prompt_len` tokens each: (tokens a second, seconds a step, live context summed over the
+        sequences in the middle of the timed steps, op times)."""
+        seq_len = seq_len or context
+        lens = [prompt_len] * n_seq if prompt_len else [int(x) for x in rng.integers(prompt_lo, prompt_hi + 1, size=n_seq)]
         prompts = [[int(t) for t in rng.integers(0, cfg.vocab_size, size=n)] for n in lens]
-        pages = sum((min(n + n_steps + n_warm + 1, context) + 63) // 64 for n in lens)
-        sess = Session(model, max_tokens=pages * 64, max_seq_len=context, n_slots=n_seq, time_ops=time_ops)
+        pages = sum((min(n + n_steps + n_warm + 1, seq_len) + 63) // 64 for n in lens)
+        sess = Session(model, max_tokens=pages * 64, max_seq_len=seq_len, n_slots=n_seq, time_ops=time_ops)
         sampler = Sampler(CLI_DEFAULTS if args.sampling == "picolm" else SamplingParams(), n_seq, dev)
         slots = sess.begin(n_seq)
         logits = SessionStepper(sess).step(slots, prompts)          # the prompts, as the generation loop sends them
@@ -193,6 +201,31 @@ def main() -> int:
         del sess
         torch.cuda.empty_cache()
         return n_seq * n_steps / dt, dt / n_steps, ctx, ops
+
+    def generation_loops(n_seq: int, few: int = 8, many: int = 72):
+        """Tokens a second of whole generation loops over a batch of `n_seq` prompts: the library's
+        own (picolm_engine_generate, one wait a step) and the Python loop (one step ahead), each as
+        the time that `many - few` more tokens a sequence take."""
+        lens = [int(x) for x in rng.integers(prompt_lo, prompt_hi + 1, size=n_seq)]
+        prompts = [[int(t) for t in rng.integers(0, cfg.vocab_size, size=n)] for n in lens]
+        pages = sum((min(n + many + 1, context) + 63) // 64 for n in lens)
+        sess = Session(model, max_tokens=pages * 64, max_seq_len=context, n_slots=n_seq)
+        params = CLI_DEFAULTS if args.sampling == "picolm" else SamplingParams()
+        out = {}
+        for name, run in (("c_api", lambda n: sess.engine.generate(prompts, n, params, [], batch_size=n_seq)),
+                          ("python", lambda n: generate(sess, prompts, n, params, stop_ids=[], batch_size=n_seq))):
+            run(few)                                  # the shapes' first uses (recordings) lie outside the clock
+            times = []
+            for n in (few, many):
+                torch.cuda.synchronize()
+                t = time.perf_counter()
+                run(n)
+                torch.cuda.synchronize()
+                times.append(time.perf_counter() - t)
+            out[name] = n_seq * (many - few) / (times[1] - times[0])
+        del sess
+        torch.cuda.empty_cache()
+        return out
 
     def prefill_run(T: int, reps: int = 3, time_ops: bool = False):
         sess = Session(model, max_tokens=T + 64, max_seq_len=max(context, T + 64), n_slots=1, time_ops=time_ops)
@@ -265,6 +298,26 @@ def main() -> int:
         out["prefill_products_of_ceiling_random_operands"] = round(out["prefill_products_tflops"] / mfma_real_tflops, 4)
         return out
 
+    if args.sweep:
+        # further sizes and contexts: each prefill is one prompt from an empty cache; each decode
+        # point has every sequence at the named context
+        big = cfg.hidden_size >= 8192
+        out = {"model": shape["name"], "layers": cfg.num_hidden_layers, "prefill": {}, "decode": {}}
+        for T in ((2048, 8192) if big else (128, 512, 1024, 2048, 4096, 8192, 16384, 32768)):
+            sec = prefill_run(T, reps=2)
+            out["prefill"][str(T)] = {"ms": round(sec * 1e3, 3), "tok_s": round(T / sec, 1),
+                                      "frac": round(prefill_flops(cfg, T) / sec / (PEAK_TFLOPS["bf16"] * 1e12), 4)}
+            print(f"[bench] prefill {T}: {sec * 1e3:.2f} ms", file=sys.stderr, flush=True)
+        for b, ctx_len in (((8, 32768), (1, 32768)) if big else ((8, 16384), (4, 65536), (1, 131072))):
+            n, warm = 12, 3
+            tps, sps, ctx, _ = decode_run(b, n, warm, prompt_len=ctx_len - warm - n // 2 - 1, seq_len=ctx_len + 64)
+            gbs = (weight_bytes(cfg) + ctx * kv_bytes_per_token(cfg)) / sps / 1e9
+            out["decode"][f"b{b}_ctx{ctx_len}"] = {"tok_s": round(tps, 2), "ms_per_step": round(sps * 1e3, 4),
+                                                   "mean_context": round(ctx / b, 1), "gb_s": round(gbs, 1),
+                                                   "hbm_frac": round(gbs / HBM_PEAK_GBS, 4)}
+            print(f"[bench] decode b{b} at {ctx_len}: {sps * 1e3:.2f} ms a step", file=sys.stderr, flush=True)
+        print(json.dumps(out))
+        return 0
     if args.prefill_only:
         sec = prefill_run(args.prefill_tokens)
         print(json.dumps({"prefill_ms": round(sec * 1e3, 3), "tokens": args.prefill_tokens, "layers": cfg.num_hidden_layers}))
@@ -305,6 +358,20 @@ def main() -> int:
             points[f"decode_b{b}_ms_per_step"] = round(sps * 1e3, 4)
             points[f"decode_b{b}_mean_context"] = round(ctx / b, 1)
             points[f"decode_b{b}_hbm_frac"] = round((weight_bytes(cfg) + ctx * kv_bytes_per_token(cfg)) / sps / 1e9 / HBM_PEAK_GBS, 4)
+        # the stated workload goes up to a total of `context` tokens: the same batches where the cache
+        # weighs most, every sequence near 2,000 and near the full context
+        for b in sorted(set(shape["points"]) | {batch}):
+            for ctx_len in (2000, context - 96):
+                n, warm = (16, 2) if b > 1 else (24, 3)
+                tps, sps, ctx, _ = decode_run(b, n, warm, prompt_len=ctx_len - warm - n // 2)
+                key = f"decode_b{b}_ctx{ctx_len}"
+                points[key] = round(tps, 2)
+                points[key + "_ms_per_step"] = round(sps * 1e3, 4)
+                points[key + "_mean_context"] = round(ctx / b, 1)
+                points[key + "_hbm_frac"] = round((weight_bytes(cfg) + ctx * kv_bytes_per_token(cfg)) / sps / 1e9 / HBM_PEAK_GBS, 4)
+        loops = generation_loops(batch)
+        points[f"generate_c_api_b{batch}"] = round(loops["c_api"], 2)
+        points[f"generate_python_b{batch}"] = round(loops["python"], 2)
         record["points"] = points
         record["kernel_classes"] = kernel_classes(batch)
     print(json.dumps(record))
