@@ -28,6 +28,7 @@ int picolm_mfma_probe(void* sink, int blocks, int iters, int random_operands, hi
 
 int picolm_embed(const void* table, int table_dt, const int32_t* tokens, float* x, int T, int D,
                  int V, hipStream_t stream);
+int picolm_gather_i32(int32_t* out, const int32_t* src, const int32_t* index, int n, hipStream_t stream);   // out[i] = src[index[i]]
 int picolm_rmsnorm(const float* x, const float* w, void* out, int out_dt, const int32_t* rows,
                    int n_rows, int D, float eps, hipStream_t stream);
 int picolm_rope_kv_store(const float* qkv, void* q_out, void* k_pages, void* v_pages, int dt,

@@ -17,6 +17,21 @@ __global__ void embed_kernel(const TW* __restrict__ table, const int32_t* __rest
     for (int i = threadIdx.x; i < D; i += blockDim.x) out[i] = to_f32<TW>(row[i]);
 }
 
+// out[i] = src[index[i]]: the tokens of the sequences that go on, picked from what a sampling kernel
+// drew for a larger batch, without the host having seen them.
+__global__ void gather_i32_kernel(int32_t* __restrict__ out, const int32_t* __restrict__ src, const int32_t* __restrict__ index, int n) {
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) out[i] = src[index[i]];
+}
+
+extern "C" int picolm_gather_i32(int32_t* out, const int32_t* src, const int32_t* index, int n, hipStream_t stream) {
+    PICOLM_REQUIRE(out && src && index && n >= 0, "gather_i32: null argument");
+    if (n == 0) return 0;
+    gather_i32_kernel<<<ceil_div(n, 256), 256, 0, stream>>>(out, src, index, n);
+    PICOLM_LAUNCH_CHECK("gather_i32");
+    return 0;
+}
+
 extern "C" int picolm_embed(const void* table, int table_dt, const int32_t* tokens, float* x,
                             int T, int D, int V, hipStream_t stream) {
     PICOLM_REQUIRE(T >= 0 && D > 0 && V > 0, "embed: bad sizes T=%d D=%d V=%d", T, D, V);

@@ -211,7 +211,10 @@ typedef struct {
 // max_new tokens, or at the cache's capacity, leaves the batch and gives its slot back; batches of
 // up to batch_size requests follow each other until all are done.  prompts: packed token ids,
 // prompt_lens[i] >= 1 each.  out_tokens: [n_prompts][max_new]; out_counts[i] tokens were made;
-// out_finish[i]: 1 stop token, 2 length, 3 capacity.  It waits for the GPU once a step.  Prompts
+// out_finish[i]: 1 stop token, 2 length, 3 capacity.  Decoding runs one step ahead of the host: a
+// step is queued before the tokens of the step before it have been read, so the GPU does not stand
+// still while the host decides (a sequence that a stop token ends has then been stepped once more;
+// that step's token is dropped).  Prompts
 // of a batch that together exceed the step's token budget (16,384 unless set otherwise; it sizes
 // the workspace) go in as several steps, each appending to what the slots hold.
 int picolm_engine_set_prefill_step_tokens(picolm_engine* e, int32_t tokens);

@@ -393,8 +393,11 @@ struct picolm_engine {
     std::vector<hipEvent_t> spare_events;
     bool timing() const { return (flags & PICOLM_ENGINE_TIME_OPS) != 0; }
     // generation
-    int32_t* gen_tokens_dev = nullptr;
-    int32_t* gen_tokens_host = nullptr;    // pinned
+    // (the sampled tokens of two steps in turn, [2][rows]: one is drawn while the other is still on its
+    // way to the host; then the tokens picked for a smaller batch and their indices)
+    int32_t* gen_tokens_dev = nullptr;     // [4][rows]: two draws, the picked tokens, the indices to pick
+    int32_t* gen_tokens_host = nullptr;    // pinned, [2][rows]
+    hipEvent_t gen_arrived[2] = {nullptr, nullptr};
     uint64_t* gen_states = nullptr;
     int32_t* gen_index = nullptr;
     void* gen_scratch = nullptr;
@@ -663,6 +666,8 @@ extern "C" void picolm_engine_destroy(picolm_engine* e) {
     if (e->gen_states) (void)hipFree(e->gen_states);
     if (e->gen_index) (void)hipFree(e->gen_index);
     if (e->gen_scratch) (void)hipFree(e->gen_scratch);
+    for (int t = 0; t < 2; ++t)
+        if (e->gen_arrived[t]) (void)hipEventDestroy(e->gen_arrived[t]);
     e->stager.destroy();
     for (auto& t : e->timed) {
         (void)hipEventDestroy(t.before);
@@ -1622,11 +1627,13 @@ static int gen_buffers(picolm_engine* e, int n_prompts, int rows, const picolm_s
         if (e->gen_tokens_dev) HIP_TRY(hipFree(e->gen_tokens_dev));
         if (e->gen_tokens_host) HIP_TRY(hipHostFree(e->gen_tokens_host));
         if (e->gen_index) HIP_TRY(hipFree(e->gen_index));
-        HIP_TRY(hipMalloc((void**)&e->gen_tokens_dev, (size_t)rows * 4));
-        HIP_TRY(hipHostMalloc((void**)&e->gen_tokens_host, (size_t)rows * 4, hipHostMallocDefault));
+        HIP_TRY(hipMalloc((void**)&e->gen_tokens_dev, (size_t)rows * 4 * 4));
+        HIP_TRY(hipHostMalloc((void**)&e->gen_tokens_host, (size_t)rows * 4 * 2, hipHostMallocDefault));
         HIP_TRY(hipMalloc((void**)&e->gen_index, (size_t)rows * 4));
         e->gen_rows = rows;
     }
+    for (int t = 0; t < 2; ++t)
+        if (!e->gen_arrived[t]) HIP_TRY(hipEventCreateWithFlags(&e->gen_arrived[t], hipEventDisableTiming));
     if (e->gen_states) HIP_TRY(hipFree(e->gen_states));
     e->gen_states = nullptr;
     std::vector<uint64_t> states(n_prompts);
@@ -1643,20 +1650,28 @@ static int gen_buffers(picolm_engine* e, int n_prompts, int rows, const picolm_s
     return 0;
 }
 
-// one token for each row of logits; row i belongs to request ids[i]; the tokens arrive in
-// e->gen_tokens_host after the wait
-static int gen_sample(picolm_engine* e, const float* logits, const std::vector<int>& ids, const picolm_sampling* sp, hipStream_t stream) {
+// One token for each row of logits; row i belongs to request ids[i].  The draw and the tokens' way
+// to the host are queued, nothing is waited for: the tokens lie in gen_tokens_dev + turn * gen_rows
+// when the stream gets there and in gen_tokens_host + turn * gen_rows after gen_wait(turn).
+static int gen_draw(picolm_engine* e, const float* logits, const std::vector<int>& ids, const picolm_sampling* sp, int turn,
+                    hipStream_t stream) {
     const int n = (int)ids.size();
+    int32_t* out = e->gen_tokens_dev + (size_t)turn * e->gen_rows;
     if (sp->temperature > 0.f) {
         TRY(e->stager.upload(e->gen_index, ids.data(), (size_t)n * 4, stream));
         const int64_t scratch = picolm_sample_scratch_bytes(n, e->vocab, sp->temperature, sp->top_k);
         TRY(picolm_sample(logits, e->vocab, n, e->vocab, sp->temperature, sp->top_k, sp->top_p, sp->min_p, e->gen_states, e->gen_index,
-                          e->gen_tokens_dev, scratch ? e->gen_scratch : nullptr, scratch, stream));
+                          out, scratch ? e->gen_scratch : nullptr, scratch, stream));
     } else {
-        TRY(picolm_argmax(logits, e->gen_tokens_dev, n, e->vocab, e->vocab, (float*)e->gen_scratch, stream));
+        TRY(picolm_argmax(logits, out, n, e->vocab, e->vocab, (float*)e->gen_scratch, stream));
     }
-    HIP_TRY(hipMemcpyAsync(e->gen_tokens_host, e->gen_tokens_dev, (size_t)n * 4, hipMemcpyDeviceToHost, stream));
-    HIP_TRY(hipStreamSynchronize(stream));
+    HIP_TRY(hipMemcpyAsync(e->gen_tokens_host + (size_t)turn * e->gen_rows, out, (size_t)n * 4, hipMemcpyDeviceToHost, stream));
+    HIP_TRY(hipEventRecord(e->gen_arrived[turn], stream));
+    return 0;
+}
+static int gen_wait(picolm_engine* e, int turn, const int32_t** tokens) {
+    HIP_TRY(hipEventSynchronize(e->gen_arrived[turn]));
+    *tokens = e->gen_tokens_host + (size_t)turn * e->gen_rows;
     return 0;
 }
 
@@ -1776,12 +1791,22 @@ extern "C" int picolm_engine_generate(picolm_engine* e, int32_t n_prompts, const
             if (idx.empty()) idx.push_back(0);
             rc = picolm_engine_step(e, (int)sl.size(), sl.data(), nn.data(), toks.data(), counts.data(), idx.data(), &logits, nullptr, stream);
             if (rc || ending.empty()) continue;
-            rc = gen_sample(e, logits, ending, sampling, stream);
+            const int32_t* drawn = nullptr;
+            rc = gen_draw(e, logits, ending, sampling, 0, stream);
+            if (!rc) rc = gen_wait(e, 0, &drawn);
             for (size_t x = 0; !rc && x < ending.size(); ++x)
-                if (accept(ending[x], e->gen_tokens_host[x])) live.push_back(ending[x]);
+                if (accept(ending[x], drawn[x])) live.push_back(ending[x]);
         }
         std::sort(live.begin(), live.end());
-        while (!rc && !live.empty()) {
+        // Decoding, one step ahead of the host: the step that takes the tokens of a draw is queued
+        // before those tokens have been read here.  Whether a sequence ends by its count of tokens
+        // or at the cache's capacity is known without its token; only a stop token is found out one
+        // step late, and such a sequence has by then been stepped once more (that step's token is
+        // dropped; its slot is given back at once: what still runs for it touches its own pages
+        // only, and whatever uses them next comes after it in the stream).
+        std::vector<int> rows;               // the sequences that the pending tokens belong to, row by row
+        int turn = 0;
+        if (!rc && !live.empty()) {          // the first step takes its tokens from the host
             sl.resize(live.size());
             nn.assign(live.size(), 1);
             toks.resize(live.size());
@@ -1791,13 +1816,52 @@ extern "C" int picolm_engine_generate(picolm_engine* e, int32_t n_prompts, const
                 length[live[x]] += 1;
             }
             rc = picolm_engine_step(e, (int)live.size(), sl.data(), nn.data(), toks.data(), nullptr, nullptr, &logits, nullptr, stream);
+            if (!rc) rc = gen_draw(e, logits, live, sampling, turn, stream);
+            if (!rc) rows = live;
+        }
+        std::vector<char> ended(n_prompts, 0);
+        while (!rc && !rows.empty()) {
+            std::vector<int> ahead, pick;
+            for (size_t x = 0; x < rows.size(); ++x) {
+                const int i = rows[x];
+                if (!ended[i] && out_counts[i] + 1 < max_new && length[i] + 1 <= e->max_seq_len) {
+                    ahead.push_back(i);
+                    pick.push_back((int)x);
+                }
+            }
+            if (!ahead.empty()) {
+                const int32_t* step_tokens = e->gen_tokens_dev + (size_t)turn * e->gen_rows;
+                if (ahead.size() != rows.size()) {       // a smaller batch goes on: its tokens, picked on the device
+                    int32_t* picked = e->gen_tokens_dev + (size_t)2 * e->gen_rows;
+                    int32_t* index = e->gen_tokens_dev + (size_t)3 * e->gen_rows;
+                    rc = e->stager.upload(index, pick.data(), pick.size() * 4, stream);
+                    if (!rc) rc = picolm_gather_i32(picked, step_tokens, index, (int)pick.size(), stream);
+                    step_tokens = picked;
+                }
+                sl.resize(ahead.size());
+                for (size_t x = 0; x < ahead.size(); ++x) sl[x] = slot_of[ahead[x]];
+                if (!rc) rc = picolm_engine_step_device_tokens(e, (int)ahead.size(), sl.data(), step_tokens, &logits, stream);
+                if (!rc) rc = gen_draw(e, logits, ahead, sampling, turn ^ 1, stream);
+                if (rc) break;
+                for (int i : ahead) length[i] += 1;
+            }
+            const int32_t* drawn = nullptr;
+            rc = gen_wait(e, turn, &drawn);
             if (rc) break;
-            rc = gen_sample(e, logits, live, sampling, stream);
-            if (rc) break;
-            std::vector<int> next;
-            for (size_t x = 0; x < live.size(); ++x)
-                if (accept(live[x], e->gen_tokens_host[x])) next.push_back(live[x]);
-            live = next;
+            for (size_t x = 0; x < rows.size(); ++x) {
+                const int i = rows[x];
+                if (ended[i]) continue;                  // stepped once more before its stop token was seen
+                const int tok = drawn[x];
+                out_tokens[(int64_t)i * max_new + out_counts[i]++] = tok;
+                if (is_stop(tok)) out_finish[i] = 1;
+                else if (std::find(ahead.begin(), ahead.end(), i) != ahead.end()) continue;
+                else out_finish[i] = out_counts[i] >= max_new ? 2 : 3;
+                ended[i] = 1;
+                (void)picolm_engine_slot_free(e, slot_of[i]);
+                slot_of[i] = -1;
+            }
+            rows = ahead;
+            turn ^= 1;
         }
         release_all();
         if (rc) return rc;

@@ -40,7 +40,7 @@ def lib():
 
 
 def dir_entry_points():
-    return ["picolm_abi_version", "picolm_device_check", "picolm_embed", "picolm_rmsnorm",
+    return ["picolm_abi_version", "picolm_device_check", "picolm_embed", "picolm_gather_i32", "picolm_rmsnorm",
             "picolm_rope_kv_store", "picolm_gemm_generic",
             "picolm_attn_prefill_tile_rows", "picolm_attn_prefill_generic",
             "picolm_attn_decode_generic", "picolm_argmax", "picolm_argmax_scratch_floats", "picolm_sample", "picolm_sample_scratch_bytes", "picolm_gemm_skinny", "picolm_gemm_tiled", "picolm_gemm_tiled_splitk", "picolm_gemm_linked", "picolm_gemm_tiled_norm_parts", "picolm_kv_page_order",
