@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Decode and prefill throughput of a Llama shape on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--shape llama31-8b|llama2-7b|llama31-70b|llama32-1b]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--shape llama31-8b|llama2-7b|llama31-70b|llama32-1b|heads96]
                     [--batch B] [--layers L]
 
 The default run is the Llama-3.1-8B shape at batch 8 and a context of up to 4,096; the other
@@ -55,6 +55,13 @@ SHAPES = {
                     num_key_value_heads=8, num_hidden_layers=16, vocab_size=128256, head_dim=64, rms_norm_eps=1e-5,
                     rope_theta=500000.0, rope_scaling=dict(LLAMA3_SCALING, factor=32.0), tie_word_embeddings=True,
                     max_position_embeddings=131072, eos_token_id=128001, bos_token_id=128000)),
+    # no checkpoint's shape: a head size that is no power of two (96), for the attention kernels at such sizes
+    "heads96": dict(
+        name="width 3072, heads of 96", std=0.02, batch=8, steps=64, warmup=8, prompt_range=(128, 2048), points=(1, 64),
+        config=dict(architectures=["LlamaForCausalLM"], hidden_size=3072, intermediate_size=8192, num_attention_heads=32,
+                    num_key_value_heads=8, num_hidden_layers=32, vocab_size=32064, head_dim=96, rms_norm_eps=1e-5,
+                    rope_theta=10000.0, rope_scaling=None, tie_word_embeddings=False, max_position_embeddings=4096,
+                    eos_token_id=2, bos_token_id=1)),
     "llama31-70b": dict(
         name="Llama-3.1-70B shape", std=0.01, batch=8, steps=16, warmup=3, prompt_range=(128, 2048), points=(1,),
         config=dict(architectures=["LlamaForCausalLM"], hidden_size=8192, intermediate_size=28672, num_attention_heads=64,

@@ -95,7 +95,8 @@ int picolm_linear(const void* A, int a_dt, const void* W, int w_dt, void* C, int
                   int norm_len, float eps, float* ws, hipStream_t stream);
 
 // Within a group's part of a page, K[64][d] and V^T[d][64] lie as plain arrays, except in bfloat16
-// pages of head size 32, 64 or 128: those are in the order of the matrix-core kernels' operands.
+// pages of a head size that is a multiple of 32 up to 256: those are in the order of the matrix-core
+// kernels' operands.
 // Fills k_idx[key * d + i] and v_idx[i * 64 + key] with the offsets of K[key][i] and V^T[i][key].
 int picolm_kv_page_order(int dt, int d, int32_t* k_idx, int32_t* v_idx);
 int picolm_attn_prefill_tile_rows(void);
@@ -118,8 +119,11 @@ int picolm_attn_decode_generic(const void* q, const void* k_pages, const void* v
                                const int32_t* page_table, int max_pages, int ring_pages, int H, int G, int d,
                                int window, float scale, hipStream_t stream);
 
-// bf16 attention on the matrix cores, head sizes 32, 64, 128
+// bf16 attention on the matrix cores: head sizes in multiples of 32 up to 256 (the cache's pages of
+// such heads are in the order of the MFMA operands); picolm_attn_mfma_fits: and a group's query
+// heads, of which a decode workgroup keeps partial results in LDS, fit there
 int picolm_attn_mfma_takes(int d);
+int picolm_attn_mfma_fits(int H, int G, int d);
 int picolm_attn_prefill_mfma_heads(int H, int G);
 int picolm_attn_prefill_mfma_tile_tokens(int H, int G);
 int picolm_attn_prefill_mfma(const void* q, const void* k_pages, const void* v_pages, void* out,

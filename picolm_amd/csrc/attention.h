@@ -46,7 +46,7 @@ struct AttnArgs {
 // ---- the order of a page's elements ---------------------------------------------------------
 // A page holds, per KV group, the keys K[64][d] and the values transposed V^T[d][64].  Pages of
 // the vector-ALU kernels (32-bit, or head sizes the matrix-core kernels do not take) keep these
-// as plain arrays.  Pages of the matrix-core kernels (bfloat16, d = 32, 64, 128) keep their
+// as plain arrays.  Pages of the matrix-core kernels (bfloat16, d a multiple of 32 up to 256) keep their
 // 16-byte chunks in the order in which a wave takes them as MFMA operands, so that every
 // wave-wide load reads 1 KB of adjacent memory:
 //   K   chunk ((tile * d/16 + kstep) * 64 + lane): key 32*tile + key_of_row(lane % 32),
@@ -67,7 +67,7 @@ __host__ __device__ __forceinline__ int row_of_key(int k) {
 }
 // whether pages of this dtype and head size are in the matrix-core kernels' order
 __host__ __device__ __forceinline__ bool kv_pages_tiled(int dt, int d) {
-    return dt == PICOLM_BF16 && (d == 32 || d == 64 || d == 128);
+    return dt == PICOLM_BF16 && d >= 32 && d <= 256 && d % 32 == 0;
 }
 // offset of K[key][i] and of V^T[i][key] within one group's part of a page
 __host__ __device__ __forceinline__ int k_page_offset(int key, int i, int d, bool tiled) {

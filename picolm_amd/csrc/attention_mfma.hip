@@ -1,4 +1,5 @@
-// bf16 attention over the paged cache on the matrix cores of gfx950, head sizes 32, 64, 128.
+// bf16 attention over the paged cache on the matrix cores of gfx950, head sizes in multiples of 32
+// up to 256.
 //
 // Both kernels compute S^T = K Q^T with 32x32x16 MFMAs, so that an accumulator lane holds one
 // query (column) and 16 keys (rows): a query's maximum and sum are an in-lane reduction plus
@@ -143,8 +144,9 @@ __device__ __forceinline__ void attend_page(const bf16x8 (&Qf)[D / 16], f32x16 (
                                             float& l_run, int key0, int qpos, bool q_ok, int window,
                                             float scale2, int h, KOP kop, VOP vop) {
     constexpr int NP = D / 16;                  // products of a tile, in either role
-    static_assert(NP % 2 == 0 && 16 % (NP / 2) == 0, "the softmax's pieces go between the products");
-    constexpr int PIECE = 16 / (NP / 2);        // elements per piece: half of the products see the maximum, half the exponentials
+    static_assert(NP % 2 == 0, "half of the products see the maximum, half the exponentials");
+    constexpr int NH = NP / 2;                  // the 16 elements of a lane go between them in NH pieces each time:
+    // piece s covers elements 16 s / NH .. 16 (s + 1) / NH (as even as NH allows)
     f32x16 S0, S1;
 #pragma unroll
     for (int e = 0; e < 16; ++e) S0[e] = 0.f, S1[e] = 0.f;
@@ -170,9 +172,16 @@ __device__ __forceinline__ void attend_page(const bf16x8 (&Qf)[D / 16], f32x16 (
         ahead2 = s + 2 < NP ? kop(1, s + 2) : vop((s + 2 - NP) / 2, 0, (s + 2 - NP) % 2);
         S1 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(now, Qf[s], S1, 0, 0, 0);
         __builtin_amdgcn_sched_barrier(0);
-        if (s < NP / 2) softmax_mask_max<MASKED>(S0, PIECE * s, PIECE, key0, qpos, q_ok, window, h, t);
-        if (s == NP / 2 - 1) softmax_reference(t, m_run, scale2);
-        if (s >= NP / 2) softmax_exp<MASKED>(S0, PIECE * (s - NP / 2), PIECE, scale2, t, P0);
+        if constexpr (16 % NH == 0) {
+            constexpr int PIECE = 16 / NH;
+            if (s < NH) softmax_mask_max<MASKED>(S0, PIECE * s, PIECE, key0, qpos, q_ok, window, h, t);
+            if (s == NH - 1) softmax_reference(t, m_run, scale2);
+            if (s >= NH) softmax_exp<MASKED>(S0, PIECE * (s - NH), PIECE, scale2, t, P0);
+        } else {
+            if (s < NH) softmax_mask_max<MASKED>(S0, 16 * s / NH, 16 * (s + 1) / NH - 16 * s / NH, key0, qpos, q_ok, window, h, t);
+            if (s == NH - 1) softmax_reference(t, m_run, scale2);
+            if (s >= NH) softmax_exp<MASKED>(S0, 16 * (s - NH) / NH, 16 * (s - NH + 1) / NH - 16 * (s - NH) / NH, scale2, t, P0);
+        }
         __builtin_amdgcn_sched_barrier(0);
     }
     softmax_finish(t, m_run, l_run);
@@ -189,9 +198,16 @@ __device__ __forceinline__ void attend_page(const bf16x8 (&Qf)[D / 16], f32x16 (
         ahead2 = s + 2 < NP ? vop((s + 2) / 2, 0, (s + 2) % 2) : vop((s + 2 - NP) / 2, 1, (s + 2 - NP) % 2);
         O[s / 2] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(now, P0[s % 2], O[s / 2], 0, 0, 0);
         __builtin_amdgcn_sched_barrier(0);
-        if (s < NP / 2) softmax_mask_max<MASKED>(S1, PIECE * s, PIECE, key0 + 32, qpos, q_ok, window, h, t);
-        if (s == NP / 2 - 1) softmax_reference(t, m_run, scale2);
-        if (s >= NP / 2) softmax_exp<MASKED>(S1, PIECE * (s - NP / 2), PIECE, scale2, t, P1);
+        if constexpr (16 % NH == 0) {
+            constexpr int PIECE = 16 / NH;
+            if (s < NH) softmax_mask_max<MASKED>(S1, PIECE * s, PIECE, key0 + 32, qpos, q_ok, window, h, t);
+            if (s == NH - 1) softmax_reference(t, m_run, scale2);
+            if (s >= NH) softmax_exp<MASKED>(S1, PIECE * (s - NH), PIECE, scale2, t, P1);
+        } else {
+            if (s < NH) softmax_mask_max<MASKED>(S1, 16 * s / NH, 16 * (s + 1) / NH - 16 * s / NH, key0 + 32, qpos, q_ok, window, h, t);
+            if (s == NH - 1) softmax_reference(t, m_run, scale2);
+            if (s >= NH) softmax_exp<MASKED>(S1, 16 * (s - NH) / NH, 16 * (s - NH + 1) / NH - 16 * (s - NH) / NH, scale2, t, P1);
+        }
         __builtin_amdgcn_sched_barrier(0);
     }
     softmax_finish(t, m_run, l_run);
@@ -313,9 +329,11 @@ __device__ __forceinline__ void rotated_q(const AttnArgs& a, const float* row, i
 // each takes every other page of the keys, with LDS stages of its own; at the end the second half
 // hands its sums and softmax statistics to the first through LDS.  The longest tiles, which set
 // the kernel's time when a prompt gives each CU only a tile or two, then take half as long.
+// (up to head size 128 two waves share a SIMD's registers, 256 each; the sums and operands of a
+// larger head need more, and a wave then has the SIMD to itself)
 template <int D, int HALVES>
-__global__ __launch_bounds__(256 * HALVES) __attribute__((amdgpu_waves_per_eu(2))) void attn_prefill_mfma_kernel(AttnArgs a, int HB, int tile_tokens,
-                                                                                                                 int n_tiles, int n_cus) {
+__global__ __launch_bounds__(256 * HALVES) __attribute__((amdgpu_waves_per_eu(D <= 128 ? 2 : 1))) void attn_prefill_mfma_kernel(
+    AttnArgs a, int HB, int tile_tokens, int n_tiles, int n_cus) {
     constexpr int LOADS = D / 32;                     // KB of a page's K (and of its V^T) that a wave brings in
     constexpr int STAGE = 2 * PAGE_TOKENS * D;        // K tile + V^T tile, in bf16
     extern __shared__ __attribute__((aligned(1024))) bf16_t lds_all[];    // two stages for each half
@@ -537,7 +555,7 @@ __device__ __forceinline__ float load_agent(const float* p) {
 }
 
 template <int D, int DEC_WAVES>
-__global__ __launch_bounds__(DEC_WAVES * 64) __attribute__((amdgpu_waves_per_eu(2))) void attn_decode_mfma_kernel(AttnArgs a) {
+__global__ __launch_bounds__(DEC_WAVES * 64) __attribute__((amdgpu_waves_per_eu(D <= 128 ? 2 : 1))) void attn_decode_mfma_kernel(AttnArgs a) {
     extern __shared__ float mrg[];       // [DEC_WAVES + 1][Rc][D + 2], then the new key and value [2][D]
     const int tid = threadIdx.x, wave = tid / WAVE, lane = tid % WAVE;
     const int l32 = lane % 32, h = lane / 32;
@@ -773,15 +791,28 @@ __global__ __launch_bounds__(DEC_WAVES * 64) __attribute__((amdgpu_waves_per_eu(
 }
 
 // =============================================================================================
+extern "C" int picolm_attn_mfma_takes(int d);
 static int check_sizes(const char* who, int H, int G, int d, int max_pages, int ring_pages) {
     PICOLM_REQUIRE(H > 0 && G > 0 && H % G == 0, "%s: %d heads do not split over %d groups", who, H, G);
-    PICOLM_REQUIRE(d == 32 || d == 64 || d == 128, "%s: head size %d is not 32, 64 or 128", who, d);
+    PICOLM_REQUIRE(picolm_attn_mfma_takes(d), "%s: head size %d is no multiple of 32 up to 256", who, d);
     PICOLM_REQUIRE(max_pages > 0 && ring_pages > 0 && ring_pages <= max_pages,
                    "%s: bad page table geometry max_pages=%d ring_pages=%d", who, max_pages, ring_pages);
     return 0;
 }
 
-extern "C" int picolm_attn_mfma_takes(int d) { return d == 32 || d == 64 || d == 128; }
+extern "C" int picolm_attn_mfma_takes(int d) { return d >= 32 && d <= 256 && d % 32 == 0; }
+
+// LDS of a decode workgroup of `waves` waves: the waves' partial results and the new token's, then
+// the new key and value
+static size_t decode_lds_bytes(int R, int d, int waves) { return sizeof(float) * ((waves + 1) * (size_t)min(R, 32) * (d + 2) + 2 * d); }
+static const size_t LDS_LIMIT = 160 * 1024;
+
+// Whether the matrix-core kernels take this shape: the head size, and a decode workgroup's partial
+// results (32 query heads of a group at most, each of d + 2 floats, from four waves) within LDS.
+extern "C" int picolm_attn_mfma_fits(int H, int G, int d) {
+    if (!picolm_attn_mfma_takes(d) || G <= 0 || H % G) return 0;
+    return decode_lds_bytes(H / G, d, 4) <= LDS_LIMIT;
+}
 
 // heads of a group that share a workgroup, and the new tokens one workgroup covers
 extern "C" int picolm_attn_prefill_mfma_heads(int H, int G) {
@@ -810,7 +841,8 @@ static int launch_prefill_mfma(AttnArgs a, int n_tiles, hipStream_t stream) {
     // that share its pages halve it (measured at head size 128: 43 -> 33 us for 1,024 tokens, 85 -> 75
     // for 2,048); with more tiles the CUs even out by themselves and two independent workgroups a CU
     // overlap better than eight waves in step (219 against 243 us for 4,096 tokens).
-    const int halves = (int64_t)n_tiles * G * head_chunks <= 2 * (int64_t)n_cus ? 2 : 1;
+    // (two halves have two stages of K and V^T each: head sizes above 128 would not fit LDS)
+    const int halves = (int64_t)n_tiles * G * head_chunks <= 2 * (int64_t)n_cus && d <= 128 ? 2 : 1;
     dim3 grid(n_tiles * G * head_chunks), block(256 * halves);
     const size_t lds = halves * 2 * 2 * (size_t)PAGE_TOKENS * d * sizeof(bf16_t);       // two stages of K and V^T a half
 #define PREFILL_LAUNCH(D, HALVES)                                                                             \
@@ -825,12 +857,20 @@ static int launch_prefill_mfma(AttnArgs a, int n_tiles, hipStream_t stream) {
         }                                                                                                     \
         attn_prefill_mfma_kernel<D, HALVES><<<grid, block, lds, stream>>>(a, HB, tile_tokens, n_tiles, n_cus); \
     }
-    if (d == 32 && halves == 2) PREFILL_LAUNCH(32, 2)
-    else if (d == 64 && halves == 2) PREFILL_LAUNCH(64, 2)
-    else if (halves == 2) PREFILL_LAUNCH(128, 2)
-    else if (d == 32) PREFILL_LAUNCH(32, 1)
-    else if (d == 64) PREFILL_LAUNCH(64, 1)
-    else PREFILL_LAUNCH(128, 1)
+#define PREFILL_BOTH(D)                   \
+    if (halves == 2) PREFILL_LAUNCH(D, 2) \
+    else PREFILL_LAUNCH(D, 1)
+    switch (d) {
+        case 32: PREFILL_BOTH(32) break;
+        case 64: PREFILL_BOTH(64) break;
+        case 96: PREFILL_BOTH(96) break;
+        case 128: PREFILL_BOTH(128) break;
+        case 160: PREFILL_LAUNCH(160, 1) break;
+        case 192: PREFILL_LAUNCH(192, 1) break;
+        case 224: PREFILL_LAUNCH(224, 1) break;
+        default: PREFILL_LAUNCH(256, 1) break;
+    }
+#undef PREFILL_BOTH
 #undef PREFILL_LAUNCH
     PICOLM_LAUNCH_CHECK("attn_prefill_mfma");
     return 0;
@@ -898,9 +938,13 @@ extern "C" int picolm_attn_decode_mfma_waves(int n_seq, int H, int G) {
 static int launch_decode_mfma(const AttnArgs& a, int n_seq, int n_chunks, hipStream_t stream) {
     const int R = a.H / a.G, chunks = ceil_div(R, 32), d = a.d;
     PICOLM_REQUIRE((int64_t)n_chunks * a.G * chunks < (1ll << 31), "attn_decode_mfma: %d chunks of %d workgroups exceed the grid", n_chunks, a.G * chunks);
-    const int waves = picolm_attn_decode_mfma_waves(n_seq, a.H, a.G);
+    int waves = picolm_attn_decode_mfma_waves(n_seq, a.H, a.G);
+    // (a head above 128 needs a SIMD's registers for one wave; many wide heads a group: the partial
+    // results of eight waves do not fit LDS)
+    if (d > 128 || decode_lds_bytes(R, d, waves) > LDS_LIMIT) waves = 4;
+    PICOLM_REQUIRE(decode_lds_bytes(R, d, waves) <= LDS_LIMIT, "attn_decode_mfma: %d heads of size %d a group need more LDS than a CU has", R, d);
     dim3 grid(n_chunks * a.G * chunks), block(waves * 64);
-    const size_t lds = sizeof(float) * ((waves + 1) * (size_t)min(R, 32) * (d + 2) + 2 * d);
+    const size_t lds = decode_lds_bytes(R, d, waves);
 #define DEC_LAUNCH(D, W)                                                                                    \
     {                                                                                                       \
         static size_t raised = 48 * 1024;                                                                   \
@@ -913,12 +957,20 @@ static int launch_decode_mfma(const AttnArgs& a, int n_seq, int n_chunks, hipStr
         }                                                                                                   \
         attn_decode_mfma_kernel<D, W><<<grid, block, lds, stream>>>(a);                                     \
     }
-    if (d == 32 && waves == 4) DEC_LAUNCH(32, 4)
-    else if (d == 32) DEC_LAUNCH(32, 8)
-    else if (d == 64 && waves == 4) DEC_LAUNCH(64, 4)
-    else if (d == 64) DEC_LAUNCH(64, 8)
-    else if (waves == 4) DEC_LAUNCH(128, 4)
-    else DEC_LAUNCH(128, 8)
+#define DEC_BOTH(D)                  \
+    if (waves == 4) DEC_LAUNCH(D, 4) \
+    else DEC_LAUNCH(D, 8)
+    switch (d) {
+        case 32: DEC_BOTH(32) break;
+        case 64: DEC_BOTH(64) break;
+        case 96: DEC_BOTH(96) break;
+        case 128: DEC_BOTH(128) break;
+        case 160: DEC_LAUNCH(160, 4) break;
+        case 192: DEC_LAUNCH(192, 4) break;
+        case 224: DEC_LAUNCH(224, 4) break;
+        default: DEC_LAUNCH(256, 4) break;
+    }
+#undef DEC_BOTH
 #undef DEC_LAUNCH
     PICOLM_LAUNCH_CHECK("attn_decode_mfma");
     return a.max_splits > 1 && !a.chunks_done ? picolm_attn_merge_launch(a, PICOLM_BF16, n_seq, stream) : 0;

@@ -535,7 +535,9 @@ static void add_unique(std::vector<int>& v, int x) {
     if (std::find(v.begin(), v.end(), x) == v.end()) v.push_back(x);
 }
 
-static bool attn_on_matrix_cores(const picolm_engine* e, int d) { return e->dtype == PICOLM_BF16 && picolm_attn_mfma_takes(d); }
+static bool attn_on_matrix_cores(const picolm_engine* e, int H, int G, int d) {
+    return e->dtype == PICOLM_BF16 && picolm_attn_mfma_fits(H, G, d);
+}
 
 extern "C" int picolm_engine_create(const picolm_program* program, int64_t max_tokens, int32_t max_seq_len, int32_t n_slots,
                                     int32_t flags, picolm_engine** out) {
@@ -611,7 +613,7 @@ extern "C" int picolm_engine_create(const picolm_program* program, int64_t max_t
         if (o.kv_writes) e->group_written[o.kv_group] = 1;
         e->group_attended[o.kv_group] = 1;
         const int R = o.n_heads / o.n_kv_heads;
-        const bool mfma = !e->host_only() && attn_on_matrix_cores(e.get(), o.head_dim);
+        const bool mfma = !e->host_only() && attn_on_matrix_cores(e.get(), o.n_heads, o.n_kv_heads, o.head_dim);
         add_unique(e->tile_rows, mfma ? picolm_attn_prefill_mfma_tile_tokens(o.n_heads, o.n_kv_heads) : picolm_attn_prefill_tile_rows());
         // workgroups a chunk of the decode work list gets: the widest launch sizes the step's list
         e->decode_blocks_per_chunk = std::max(e->decode_blocks_per_chunk, o.n_kv_heads * ((R + (mfma ? 31 : 15)) / (mfma ? 32 : 16)));
@@ -1125,7 +1127,7 @@ static int run_attention(Run& r, const picolm_op& o) {
     char* v_pages = g.v + (size_t)o.kv_entry * g.v_entry_bytes;
     const bool writes = o.kv_writes != 0;
     const int32_t* tok_page = writes ? p.at(p.write_pages[o.kv_group]) : nullptr;
-    const bool mfma = attn_on_matrix_cores(e, d);
+    const bool mfma = attn_on_matrix_cores(e, H, G, d);
     if (p.is_decode) {
         const DecodeList& l = p.lists[o.kv_group];
         float* partial = l.most > 1 ? (float*)(r.w.base + r.w.partial) : nullptr;

@@ -434,7 +434,8 @@ class PagedCase:
         return np.concatenate(outs).reshape(-1, self.H * self.d)
 
 
-ATTN_SHAPES = [(4, 2, 16), (6, 6, 32), (3, 1, 32), (8, 2, 64), (32, 8, 128), (5, 5, 128), (2, 1, 256), (40, 1, 64)]
+ATTN_SHAPES = [(4, 2, 16), (6, 6, 32), (3, 1, 32), (8, 2, 64), (32, 8, 128), (5, 5, 128), (2, 1, 256), (40, 1, 64),
+               (6, 2, 96), (6, 3, 160), (8, 4, 192), (4, 1, 224), (3, 3, 48)]
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
@@ -469,7 +470,7 @@ def test_attention_prefill_with_more_tiles_than_places(H, G, d, old, new):
     assert err <= tol(torch.bfloat16, np.abs(ref).max()), err
 
 
-@pytest.mark.parametrize("H,G,d", [(6, 6, 32), (8, 2, 64), (32, 8, 128), (40, 1, 64)])
+@pytest.mark.parametrize("H,G,d", [(6, 6, 32), (8, 2, 64), (32, 8, 128), (40, 1, 64), (6, 2, 96), (4, 2, 192), (2, 1, 256)])
 @pytest.mark.parametrize("style", ["pairwise", "half", None])
 @pytest.mark.parametrize("window", [0, 70])
 def test_attention_prefill_with_rotation_inside(H, G, d, style, window):
@@ -621,7 +622,7 @@ def test_attention_decode_many_sequences(d, pages_per_chunk):
         assert torch.equal(outs[1], o)            # whichever workgroup came last, the sum is the same
 
 
-@pytest.mark.parametrize("H,G,d", [(6, 6, 32), (8, 2, 64), (32, 8, 128), (40, 1, 64)])
+@pytest.mark.parametrize("H,G,d", [(6, 6, 32), (8, 2, 64), (32, 8, 128), (40, 1, 64), (6, 2, 96), (4, 2, 160), (2, 1, 256)])
 @pytest.mark.parametrize("style", ["pairwise", "half", None])
 @pytest.mark.parametrize("pages_per_chunk,window", [(4, 0), (1, 0), (16, 0), (2, 100), (4, 1)])
 def test_attention_decode_with_rotation_and_cache_write_inside(H, G, d, style, pages_per_chunk, window):
@@ -678,7 +679,10 @@ def test_attention_decode_with_rotation_and_cache_write_inside(H, G, d, style, p
     k_plain, v_plain = K().kv_pages_unpack(case.k_pages, case.v_pages)
     for i in range(n):
         pg, row = int(tok_page[i]), pos0[i] % PAGE
-        assert torch.equal(k_plain[pg, :, row, :].cpu(), bf(k_ref[i]))
+        if style is None:
+            assert torch.equal(k_plain[pg, :, row, :].cpu(), bf(k_ref[i]))
+        else:       # (a key rotated in 32-bit and one rotated in 64-bit may round to neighbouring bfloat16 values)
+            assert np.abs(k_plain[pg, :, row, :].double().cpu().numpy() - k_ref[i]).max() <= tol(torch.bfloat16, 4.0)
         assert torch.equal(v_plain[pg, :, :, row].cpu(), bf(v_ref[i]))
 
 
@@ -860,7 +864,7 @@ def test_attention_over_pages_beyond_four_gigabytes(dtype):
 
 
 # ------------------------------------------------------------------------------------------ rope
-@pytest.mark.parametrize("d", [16, 32, 48, 64, 128, 256])
+@pytest.mark.parametrize("d", [16, 32, 48, 64, 96, 128, 160, 192, 224, 256])
 def test_kv_page_order_is_a_permutation(d):
     """Every element of a page has one place; 32-bit pages and head sizes outside the matrix-core
     kernels' are plain arrays; packing and unpacking undo each other."""
@@ -868,7 +872,7 @@ def test_kv_page_order_is_a_permutation(d):
         k_idx, v_idx = K().kv_page_order(dtype, d)
         assert sorted(k_idx.reshape(-1).tolist()) == list(range(PAGE * d))
         assert sorted(v_idx.reshape(-1).tolist()) == list(range(PAGE * d))
-        plain = dtype == torch.float32 or d not in (32, 64, 128)
+        plain = dtype == torch.float32 or d % 32 != 0
         assert (k_idx.reshape(-1).tolist() == list(range(PAGE * d))) == plain
         assert (v_idx.reshape(-1).tolist() == list(range(PAGE * d))) == plain
         k = torch.randn(3, 2, PAGE, d).to(dtype).to(DEV)

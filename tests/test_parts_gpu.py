@@ -1067,3 +1067,35 @@ def test_subclasses_of_the_librarys_parts(dtype, tmp_path):
                 pos[i] += 1
             live = [i for i in live if pos[i] < len(reqs[i])]
         assert (s.recorded_steps() > 0) == (not halved)
+
+
+def test_a_prepared_norm_is_forgotten_when_its_rows_are_written_again():
+    """A product that adds into the residual rows may prepare the norm that meets them next.  If
+    another operation writes those rows before the norm is taken (two branches that add into the
+    stream one after the other), what was prepared describes rows that are no more: the product that
+    takes the norm must see the rows as they are.  Few rows, where the products share norms."""
+    from part_harness import PartEngine
+    from picolm_amd import kernels as K
+    from picolm_amd.engine.program import NormRef, Rows
+    rng = np.random.default_rng(12)
+    D, T = 256, 5
+    x0 = rounded(rng.standard_normal((T, D)), torch.bfloat16)
+    w = {n: rounded(rng.standard_normal((D, D)) * 0.05, torch.bfloat16) for n in ("w1", "w2", "w3")}
+    nw = rng.standard_normal(D)
+    dev = {n: torch.from_numpy(v).to(torch.bfloat16).to(DEV) for n, v in w.items()}
+    norm = NormRef(torch.from_numpy(nw).float().to(DEV), 1e-5)
+
+    def emit(b, x, h):
+        hb = h.cast(b, x, D)
+        b.linear(dev["w1"], hb, x, K.EPI_ACCUMULATE, out_norm=norm)       # prepares norm(x) where its kernel can
+        b.linear(dev["w2"], hb, x, K.EPI_ACCUMULATE)                       # and x changes again
+        y = b.buffer("y", D, torch.float32)
+        b.linear(dev["w3"], Rows(b.buffer("norm.out", D, torch.bfloat16), norm, x), y, K.EPI_STORE)
+        return y, D
+    e = PartEngine(torch.bfloat16, x0, emit)
+    got = e.step(e.alloc(1), [range(T)])
+    x = x0 + x0 @ w["w1"].T + x0 @ w["w2"].T
+    ref = P.rmsnorm(x, nw.astype(np.float32), 1e-5) @ w["w3"].T
+    stale = P.rmsnorm(x0 + x0 @ w["w1"].T, nw.astype(np.float32), 1e-5) @ w["w3"].T
+    assert np.abs(ref - stale).max() > 20 * tol(torch.bfloat16, ref)          # the fault would show
+    assert np.abs(got - ref).max() <= tol(torch.bfloat16, ref)

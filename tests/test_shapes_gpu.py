@@ -1,12 +1,13 @@
 """Logits at the layer sizes that the benchmark times, with seeded random weights made on the GPU:
-the four shapes of bench.py (Llama-3.1-8B, Llama-2-7B, Llama-3.1-70B, Llama-3.2-1B) at one or two
-layers, and the Llama-3.1-8B shape at its full depth of 32 layers.
+the shapes of bench.py (Llama-3.1-8B, Llama-2-7B, Llama-3.1-70B, Llama-3.2-1B, and one with heads of
+96) at one or two layers, and the Llama-3.1-8B shape at its full depth of 32 layers.
 
 The kernels that only such sizes reach are checked here in the model: 256x256 prefill tiles, a
 head of 128,256 rows (tied to the embedding in the 1B shape), tiles of 128 weight rows for up to
 16 activation rows, skinny products staged through LDS with K of 11,008 to 28,672, 320-column
 tiles for a qkv product of 10,240 rows, one query head per KV head in the decode attention (7B),
-head size 64 at a width of 2,048 (1B).  The bfloat16 engine is held to the 32-bit engine under
+head size 64 at a width of 2,048 (1B), and a head size that is no power of two (96) on the matrix
+cores.  The bfloat16 engine is held to the 32-bit engine under
 every cutting of the work, and the 32-bit engine to the plain implementation on a short request.
 picolm checks its fast path against its plain one in the same way (picolm/picolm.c:1437-1463,
 warning above 1e-2; :1592-1604)."""
@@ -24,7 +25,7 @@ pytestmark = pytest.mark.gpu
 DEV = "cuda:0"
 SEED = 8
 # (layers, context the rotary tables are laid out for)
-LAYERS = {"llama31-8b": 2, "llama2-7b": 2, "llama31-70b": 1, "llama32-1b": 2}
+LAYERS = {"llama31-8b": 2, "llama2-7b": 2, "llama31-70b": 1, "llama32-1b": 2, "heads96": 2}
 
 
 def shape_config(name: str, layers: int) -> dict:
