@@ -1099,3 +1099,88 @@ def test_a_prepared_norm_is_forgotten_when_its_rows_are_written_again():
     stale = P.rmsnorm(x0 + x0 @ w["w1"].T, nw.astype(np.float32), 1e-5) @ w["w3"].T
     assert np.abs(ref - stale).max() > 20 * tol(torch.bfloat16, ref)          # the fault would show
     assert np.abs(got - ref).max() <= tol(torch.bfloat16, ref)
+
+
+def test_a_python_part_that_says_graph_safe_is_recorded_and_replayed(tmp_path):
+    """A feed-forward written in Python whose `forward` only launches the library's kernels on
+    buffers that exist after its first use, and says so (`graph_safe = True`): the decode steps of
+    its model are recorded on the engine's own stream and replayed, and give the bits of steps that
+    are launched one by one, and the plain implementation's logits."""
+    from picolm_amd import LlamaConfig
+    from picolm_amd import kernels as K
+    from picolm_amd.config import register_architecture, unregister_architecture
+    from picolm_amd.engine import DecoderModel, Session, load_model
+    from picolm_amd.parts import (Attention, FeedForward, Linear, LMHead, PreNormBlock, RMSNorm, RotaryEmbedding, TokenEmbedding)
+    from picolm_amd.weights import write_random_model
+
+    class TwoProducts(FeedForward):
+        """down(up(h)): no gate, no activation"""
+        graph_safe = True
+
+        def __init__(self, prefix, D, F):
+            self.F = F
+            self.up = Linear([prefix + "up_proj.weight"], [F], D)
+            self.down = Linear([prefix + "down_proj.weight"], [D], F)
+
+        def children(self):
+            return [self.up, self.down]
+
+        def forward(self, ctx, h, residual):
+            act = ctx.ws.get("toy.act", (h.shape[0], self.F), ctx.dtype)
+            self.up.forward(h, act)
+            self.down.forward(act, residual, K.EPI_ACCUMULATE)
+
+    def build(cfg):
+        D = cfg.hidden_size
+        rotary = RotaryEmbedding(cfg.head_dim, cfg.rope_theta, None, cfg.rope_style)
+        blocks = [PreNormBlock(RMSNorm(f"model.layers.{l}.input_layernorm.weight", D, cfg.rms_norm_eps),
+                               Attention(f"model.layers.{l}.self_attn.", D, cfg.num_attention_heads, cfg.num_key_value_heads,
+                                         cfg.head_dim, position=rotary),
+                               RMSNorm(f"model.layers.{l}.post_attention_layernorm.weight", D, cfg.rms_norm_eps),
+                               TwoProducts(f"model.layers.{l}.mlp.", D, cfg.intermediate_size)) for l in range(2)]
+        emb = TokenEmbedding("model.embed_tokens.weight", cfg.vocab_size, D)
+        return DecoderModel(cfg, emb, blocks, RMSNorm("model.norm.weight", D, cfg.rms_norm_eps),
+                            LMHead("lm_head.weight", cfg.vocab_size, D, emb, True))
+
+    name = "ToyTwoProductsLM"
+    c = dict(architectures=[name], hidden_size=128, num_attention_heads=4, num_key_value_heads=2, head_dim=32,
+             intermediate_size=192, num_hidden_layers=2, vocab_size=211, rms_norm_eps=1e-5, rope_theta=10000.0,
+             max_position_embeddings=256, tie_word_embeddings=True, torch_dtype="bfloat16")
+    cfg = LlamaConfig.from_dict(c)
+    register_architecture(name, LlamaConfig.from_dict, build)
+    try:
+        d = write_random_model(cfg, str(tmp_path / "two"), seed=6, std=0.08)
+        model = load_model(d, dtype="bfloat16")
+    finally:
+        unregister_architecture(name)
+    w = tiny.read_weights_f64(d)
+    pc = dict(c, rope_style=cfg.rope_style)
+
+    def plain(tokens):
+        pos = np.arange(len(tokens))
+        x = w["model.embed_tokens.weight"][np.asarray(tokens)]
+        for l in range(2):
+            q = f"model.layers.{l}."
+            x = x + P.attention_block(P.rmsnorm(x, w[q + "input_layernorm.weight"], 1e-5), w, q + "self_attn.", pc, pos)
+            h = P.rmsnorm(x, w[q + "post_attention_layernorm.weight"], 1e-5)
+            x = x + (h @ w[q + "mlp.up_proj.weight"].T) @ w[q + "mlp.down_proj.weight"].T
+        return P.rmsnorm(x, w["model.norm.weight"], 1e-5) @ w["model.embed_tokens.weight"].T
+    rng = np.random.default_rng(10)
+    reqs = [tiny.random_tokens(rng, n, 211) for n in (40, 9)]
+    truth = [plain(r) for r in reqs]
+    outs = []
+    for graphs in (True, False):
+        s = Session(model, max_tokens=512, n_slots=2, graphs=graphs)
+        assert s.engine.program.recordable
+        slots = s.begin(2)
+        rows = [s.step(slots, [r[:5] for r in reqs]).clone()]
+        for j in range(5, 9):
+            rows.append(s.step(slots, [[r[j]] for r in reqs]).clone())
+        assert (s.recorded_steps() == 1) == graphs
+        outs.append(rows)
+    for a, b in zip(*outs):
+        assert torch.equal(a, b)
+    for j, row in enumerate(outs[0]):
+        for i in range(2):
+            ref = truth[i][4 + j]
+            assert np.abs(row[i].double().cpu().numpy() - ref).max() <= tiny.tolerance("bfloat16", truth[i], tiny.spread(128, 0.08))
