@@ -13,7 +13,7 @@ import os
 from dataclasses import dataclass, field
 
 
-MAX_HEAD_DIM = 256
+MAX_HEAD_DIM = 1024
 
 
 class ConfigError(ValueError):

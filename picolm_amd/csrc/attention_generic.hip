@@ -1,6 +1,7 @@
-// Attention over the paged cache on the vector ALU, for any head size up to 256 (a size that is
-// no multiple of 16 leaves the last of a row's column groups partly empty), any number of heads
-// and groups, float or bf16 storage.  One kernel serves
+// Attention over the paged cache on the vector ALU, for any head size up to 1,024 (a size that is
+// no multiple of 16 leaves the last of a row's column groups partly empty; one above 256 goes
+// through LDS in pieces of 256 columns), any number of heads and groups, float or bf16 storage.
+// One kernel serves
 // both kinds of step: a tile is up to 16 "rows" that share one KV head.
 //   prefill: rows = consecutive new tokens of one sequence, for one query head;
 //   decode : rows = the query heads of one KV group, for a sequence's single new token,
@@ -17,15 +18,19 @@
 
 #define AT_ROWS 16
 #define AT_THREADS 256
-#define AT_MAX_D 256
+#define AT_MAX_D 1024
+#define AT_CHUNK 256        // columns of a head that lie in LDS at a time: a larger head goes through in pieces
 
 
-template <typename T>
+// MAXD: the largest head size of this instance (its accumulators are registers: MAXD / 16 a thread).
+template <typename T, int MAXD>
 __global__ __launch_bounds__(AT_THREADS) void attn_tile_kernel(AttnArgs a) {
     extern __shared__ float lds[];
-    const int d = a.d, dp = d + 1;
-    float* Qs = lds;                            // [AT_ROWS][d]
-    float* KVs = Qs + AT_ROWS * d;              // [PAGE][d+1]
+    const int d = a.d;
+    const int dl = min(d, AT_CHUNK), dp = dl + 1;
+    const bool whole = d <= AT_CHUNK;           // the queries lie in LDS once and for all
+    float* Qs = lds;                            // [AT_ROWS][dl]
+    float* KVs = Qs + AT_ROWS * dl;             // [PAGE][dl+1]
     float* Ps = KVs + PAGE_TOKENS * dp;         // [AT_ROWS][PAGE]
     float* alpha_s = Ps + AT_ROWS * PAGE_TOKENS;  // [AT_ROWS]
     float* l_s = alpha_s + AT_ROWS;             // [AT_ROWS]
@@ -74,10 +79,14 @@ __global__ __launch_bounds__(AT_THREADS) void attn_tile_kernel(AttnArgs a) {
     }
 
     const T* q = (const T*)a.q;
-    for (int idx = tid; idx < AT_ROWS * d; idx += AT_THREADS) {
-        const int r = idx / d, c = idx % d;
-        Qs[idx] = r < n_rows ? to_f32<T>(q[(size_t)row_tok[r] * a.H * d + (size_t)row_head[r] * d + c]) : 0.f;
-    }
+    // columns c0 .. c0 + dc of the tile's queries into LDS
+    auto load_q = [&](int c0, int dc) {
+        for (int idx = tid; idx < AT_ROWS * dc; idx += AT_THREADS) {
+            const int r = idx / dc, c = idx % dc;
+            Qs[r * dl + c] = r < n_rows ? to_f32<T>(q[(size_t)row_tok[r] * a.H * d + (size_t)row_head[r] * d + c0 + c]) : 0.f;
+        }
+    };
+    if (whole) load_q(0, d);
     // per-wave running statistics of its 4 rows (uniform across the wave)
     float m_run[4], l_run[4];
 #pragma unroll
@@ -88,9 +97,9 @@ __global__ __launch_bounds__(AT_THREADS) void attn_tile_kernel(AttnArgs a) {
     // PV ownership: thread -> (row pr, column group pc), columns pc + 16*j
     const int pr = tid / 16, pc = tid % 16;
     const int n_cg = pc < d ? (d - pc + 15) / 16 : 0;      // this thread's columns pc + 16*j below d
-    float acc[AT_MAX_D / 16];
+    float acc[MAXD / 16];
 #pragma unroll
-    for (int j = 0; j < AT_MAX_D / 16; ++j) acc[j] = 0.f;
+    for (int j = 0; j < MAXD / 16; ++j) acc[j] = 0.f;
 
     const int slot = a.decode ? work.slot : a.seq_slot[seq];
     const int32_t* pt = a.page_table + (size_t)slot * a.max_pages;
@@ -101,25 +110,27 @@ __global__ __launch_bounds__(AT_THREADS) void attn_tile_kernel(AttnArgs a) {
         const size_t base = (size_t)phys * page_elems + (size_t)g * PAGE_TOKENS * d;
         const int key0 = page * PAGE_TOKENS;
         const int n_keys = min(PAGE_TOKENS, hi - key0 + 1);   // rows beyond are not this sequence's
-        __syncthreads();                                       // previous PV done with KVs / Ps
-        {
+        // scores: wave handles rows 4*wave .. +3, lane = key; a head wider than the chunk adds up piece by piece
+        float s[4] = {0.f, 0.f, 0.f, 0.f};
+        for (int c0 = 0; c0 < d; c0 += AT_CHUNK) {
+            const int dc = min(AT_CHUNK, d - c0);
+            __syncthreads();                                   // whoever read KVs, Qs or Ps before is done
+            if (!whole) load_q(c0, dc);
             const T* kp = (const T*)a.k_pages + base;
-            for (int idx = tid; idx < PAGE_TOKENS * d; idx += AT_THREADS) {
-                const int r = idx / d, c = idx % d;
-                KVs[r * dp + c] = r < n_keys ? to_f32<T>(kp[idx]) : 0.f;
+            for (int idx = tid; idx < PAGE_TOKENS * dc; idx += AT_THREADS) {
+                const int r = idx / dc, c = idx % dc;
+                KVs[r * dp + c] = r < n_keys ? to_f32<T>(kp[(size_t)r * d + c0 + c]) : 0.f;
             }
-        }
-        __syncthreads();
-        // scores: wave handles rows 4*wave .. +3, lane = key
-        {
-            float s[4] = {0.f, 0.f, 0.f, 0.f};
+            __syncthreads();
             const float* kr = KVs + lane * dp;
-            const float* q0p = Qs + (4 * wave) * d;
-            for (int c = 0; c < d; ++c) {
+            const float* q0p = Qs + (4 * wave) * dl;
+            for (int c = 0; c < dc; ++c) {
                 const float kv = kr[c];
 #pragma unroll
-                for (int i = 0; i < 4; ++i) s[i] = fmaf(q0p[i * d + c], kv, s[i]);
+                for (int i = 0; i < 4; ++i) s[i] = fmaf(q0p[i * dl + c], kv, s[i]);
             }
+        }
+        {
             const int kpos = key0 + lane;
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
@@ -137,25 +148,29 @@ __global__ __launch_bounds__(AT_THREADS) void attn_tile_kernel(AttnArgs a) {
             }
         }
         __syncthreads();
-        {
-            const T* vp = (const T*)a.v_pages + base;       // transposed: [d][PAGE]
-            for (int idx = tid; idx < PAGE_TOKENS * d; idx += AT_THREADS) {
+        const float al = alpha_s[pr];
+#pragma unroll
+        for (int j = 0; j < MAXD / 16; ++j) acc[j] *= al;
+#pragma unroll
+        for (int ci = 0; ci < MAXD / AT_CHUNK; ++ci) {
+            const int c0 = ci * AT_CHUNK;
+            if (c0 >= d) break;
+            const int dc = min(AT_CHUNK, d - c0);
+            if (ci > 0) __syncthreads();                       // the piece before has been used
+            const T* vp = (const T*)a.v_pages + base + (size_t)c0 * PAGE_TOKENS;       // transposed: [d][PAGE]
+            for (int idx = tid; idx < PAGE_TOKENS * dc; idx += AT_THREADS) {
                 const int c = idx / PAGE_TOKENS, r = idx % PAGE_TOKENS;
                 KVs[r * dp + c] = r < n_keys ? to_f32<T>(vp[idx]) : 0.f;
             }
-        }
-        __syncthreads();
-        {
-            const float al = alpha_s[pr];
+            __syncthreads();
             const float* p = Ps + pr * PAGE_TOKENS;
-#pragma unroll
-            for (int j = 0; j < AT_MAX_D / 16; ++j) acc[j] *= al;
+            const int n_here = pc < dc ? (dc - pc + 15) / 16 : 0;      // this thread's columns of the piece
             for (int key = 0; key < n_keys; ++key) {
                 const float pk = p[key];
                 const float* vr = KVs + key * dp + pc;
 #pragma unroll
-                for (int j = 0; j < AT_MAX_D / 16; ++j)
-                    if (j < n_cg) acc[j] = fmaf(pk, vr[16 * j], acc[j]);
+                for (int j = 0; j < AT_CHUNK / 16; ++j)
+                    if (j < n_here) acc[ci * (AT_CHUNK / 16) + j] = fmaf(pk, vr[16 * j], acc[ci * (AT_CHUNK / 16) + j]);
             }
         }
     }
@@ -176,14 +191,14 @@ __global__ __launch_bounds__(AT_THREADS) void attn_tile_kernel(AttnArgs a) {
             po[1] = l_s[pr];
         }
 #pragma unroll
-        for (int j = 0; j < AT_MAX_D / 16; ++j)
+        for (int j = 0; j < MAXD / 16; ++j)
             if (j < n_cg) po[2 + pc + 16 * j] = acc[j];
     } else {
         const float l = l_s[pr];
         const float inv = l > 0.f ? 1.0f / l : 0.f;
         T* o = (T*)a.out + (size_t)tok * a.H * d + (size_t)head * d;
 #pragma unroll
-        for (int j = 0; j < AT_MAX_D / 16; ++j)
+        for (int j = 0; j < MAXD / 16; ++j)
             if (j < n_cg) o[pc + 16 * j] = from_f32<T>(acc[j] * inv);
     }
 }
@@ -233,26 +248,38 @@ __global__ __launch_bounds__(MERGE_WAVES * WAVE) void attn_merge_kernel(AttnArgs
         for (int i = EARLY; i < n_splits; ++i) acc += expf(p[(size_t)i * stride] - M) * p[(size_t)i * stride + 2 + c];
         o[c] = from_f32<T>(acc * inv);
     }
+    for (int c = lane + 4 * WAVE; c < d; c += WAVE) {       // a head wider than 256
+        float acc = 0.f;
+        for (int i = 0; i < n_splits; ++i) acc += expf(p[(size_t)i * stride] - M) * p[(size_t)i * stride + 2 + c];
+        o[c] = from_f32<T>(acc * inv);
+    }
 }
 
 static size_t attn_lds_bytes(int d) {
-    return sizeof(float) * ((size_t)AT_ROWS * d + (size_t)PAGE_TOKENS * (d + 1) + AT_ROWS * PAGE_TOKENS + 3 * AT_ROWS);
+    const int dl = d < AT_CHUNK ? d : AT_CHUNK;
+    return sizeof(float) * ((size_t)AT_ROWS * dl + (size_t)PAGE_TOKENS * (dl + 1) + AT_ROWS * PAGE_TOKENS + 3 * AT_ROWS);
 }
 
-template <typename T>
-static int launch_attn(const AttnArgs& a, dim3 grid, hipStream_t stream) {
+template <typename T, int MAXD>
+static int launch_attn_sized(const AttnArgs& a, dim3 grid, hipStream_t stream) {
     const size_t lds = attn_lds_bytes(a.d);
     static size_t raised = 48 * 1024;      // what a kernel may use without asking
     if (lds > raised) {
-        hipError_t e = hipFuncSetAttribute((const void*)attn_tile_kernel<T>,
+        hipError_t e = hipFuncSetAttribute((const void*)attn_tile_kernel<T, MAXD>,
                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
         PICOLM_REQUIRE(e == hipSuccess, "attention: cannot raise the LDS limit to %zu: %s", lds,
                        hipGetErrorString(e));
         raised = lds;
     }
-    attn_tile_kernel<T><<<grid, dim3(AT_THREADS), lds, stream>>>(a);
+    attn_tile_kernel<T, MAXD><<<grid, dim3(AT_THREADS), lds, stream>>>(a);
     PICOLM_LAUNCH_CHECK("attention");
     return 0;
+}
+
+// (heads of up to 256 have the kernel with 16 accumulators a thread, wider ones that with 64)
+template <typename T>
+static int launch_attn(const AttnArgs& a, dim3 grid, hipStream_t stream) {
+    return a.d <= AT_CHUNK ? launch_attn_sized<T, AT_CHUNK>(a, grid, stream) : launch_attn_sized<T, AT_MAX_D>(a, grid, stream);
 }
 
 int check_decode_chunks(const char* who, const float* partial, const int32_t* chunk_list, int n_chunks,

@@ -477,7 +477,7 @@ static int check_program(const picolm_program* p, picolm_engine* e) {
             }
             case PICOLM_OP_ATTENTION: {
                 const int H = o.n_heads, G = o.n_kv_heads, d = o.head_dim;
-                E_REQUIRE(-1, H > 0 && G > 0 && H % G == 0 && d >= 1 && d <= 256, "engine: operation %d (attention): %d heads, %d groups, size %d", i, H, G, d);
+                E_REQUIRE(-1, H > 0 && G > 0 && H % G == 0 && d >= 1 && d <= 1024, "engine: operation %d (attention): %d heads, %d groups, size %d", i, H, G, d);
                 E_REQUIRE(-1, o.window >= 0, "engine: operation %d: a window of %d keys", i, o.window);
                 E_REQUIRE(-1, buf_ok(o.in) && buf_ok(o.q_buffer) && o.rows == PICOLM_ROWS_STEP, "engine: operation %d (attention) is incomplete", i);
                 const picolm_buffer &in = p->buffers[o.in], &q = p->buffers[o.q_buffer];

@@ -18,7 +18,7 @@ from .base import KVRequest, Mixer, Runtime, forward_is_graph_safe, on_stream, r
 from .linear import Linear
 from .position import NoPosition, PositionEncoding
 
-MAX_HEAD_DIM = 256      # what a tile of the vector-ALU attention kernel holds in LDS
+MAX_HEAD_DIM = 1024      # what a tile of the vector-ALU attention kernel holds in LDS
 
 
 class Attention(Mixer):

@@ -124,6 +124,7 @@ def test_head_size_limits_are_named_when_the_configuration_is_read():
         LlamaConfig.from_dict(d)                                   # picolm would floor to 16 silently
     assert LlamaConfig.from_dict(dict(d, head_dim=20)).head_dim == 20     # given: no division takes place
     assert LlamaConfig.from_dict(dict(d, num_attention_heads=5)).head_dim == 20      # any even size, not only 16s
-    with pytest.raises(ConfigError, match="head_dim.*256"):
-        LlamaConfig.from_dict(dict(d, head_dim=320))
-    assert LlamaConfig.from_dict(dict(d, head_dim=256)).head_dim == 256
+    with pytest.raises(ConfigError, match="head_dim.*1024"):
+        LlamaConfig.from_dict(dict(d, head_dim=1026))
+    assert LlamaConfig.from_dict(dict(d, head_dim=1024)).head_dim == 1024
+    assert LlamaConfig.from_dict(dict(d, head_dim=320)).head_dim == 320              # four times picolm's own bound

@@ -21,7 +21,8 @@ pytestmark = pytest.mark.gpu
 DEV = "cuda:0"
 
 LENGTHS = {"A": [33, 47, 64, 65, 100, 128], "B": [33, 40, 64, 129, 200, 256], "C": [34, 63, 65, 128, 190, 300],
-           "D": [33, 50, 64, 127, 130, 260], "E": [33, 64, 70, 129, 200, 320], "F": [33, 45, 64, 66, 131, 250]}
+           "D": [33, 50, 64, 127, 130, 260], "E": [33, 64, 70, 129, 200, 320], "F": [33, 45, 64, 66, 131, 250],
+           "G": [33, 64, 65, 130, 300, 700]}
 
 
 tolerance = tiny.tolerance      # 2e-5 / 2e-2 of the largest logit, wider by sqrt(spread) for weights of a spread above 1
@@ -45,7 +46,7 @@ def requests_and_truth(folders):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("which", ["A", "B", "C", "D", "E", "F"])
+@pytest.mark.parametrize("which", ["A", "B", "C", "D", "E", "F", "G"])
 def test_replay_whole_tail_and_batches(which, dtype, folders, requests_and_truth, tmp_path):
     reqs, truth = requests_and_truth[which]
     one_batch = sum((len(r) + 63) // 64 for r in reqs[3:]) * 64          # room for the larger batch only

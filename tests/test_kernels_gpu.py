@@ -1,5 +1,5 @@
 """Each hand-written kernel alone against a plain float64 reference, at sizes other than the
-tiny models': head sizes 16..256, odd head counts and groups, widths and vocabularies that are
+tiny models': head sizes 16..1024, odd head counts and groups, widths and vocabularies that are
 no power of two, ragged row counts."""
 import math
 
@@ -435,7 +435,8 @@ class PagedCase:
 
 
 ATTN_SHAPES = [(4, 2, 16), (6, 6, 32), (3, 1, 32), (8, 2, 64), (32, 8, 128), (5, 5, 128), (2, 1, 256), (40, 1, 64),
-               (6, 2, 96), (6, 3, 160), (8, 4, 192), (4, 1, 224), (3, 3, 48)]
+               (6, 2, 96), (6, 3, 160), (8, 4, 192), (4, 1, 224), (3, 3, 48),
+               (4, 2, 320), (2, 1, 264), (3, 1, 512), (2, 2, 1024)]     # wider than a piece of 256 columns
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])

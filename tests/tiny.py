@@ -66,8 +66,19 @@ TINY_F = dict(
     eos_token_id=2, rope_style="half")
 TINY_F_WEIGHTS = dict(seed=5, std=0.06, norm_sigma=0.1)
 
+# a seventh with a head wider than the 256 columns that the attention kernel holds in LDS at a
+# time (picolm's own bound, picolm/model_attention.c:163): keys, values and the merge of a split
+# context go through in pieces
+TINY_G = dict(
+    architectures=["LlamaForCausalLM"], hidden_size=144, intermediate_size=208, num_attention_heads=3,
+    num_key_value_heads=1, num_hidden_layers=2, vocab_size=203, head_dim=328, rms_norm_eps=1e-6,
+    rope_theta=100000.0, rope_scaling=None, tie_word_embeddings=True, max_position_embeddings=1024,
+    eos_token_id=4, rope_style="pairwise")
+TINY_G_WEIGHTS = dict(seed=6, std=0.05, norm_sigma=0.1)
+
 CONFIGS = {"A": (TINY_A, TINY_A_WEIGHTS), "B": (TINY_B, TINY_B_WEIGHTS), "C": (TINY_C, TINY_C_WEIGHTS),
-           "D": (TINY_D, TINY_D_WEIGHTS), "E": (TINY_E, TINY_E_WEIGHTS), "F": (TINY_F, TINY_F_WEIGHTS)}
+           "D": (TINY_D, TINY_D_WEIGHTS), "E": (TINY_E, TINY_E_WEIGHTS), "F": (TINY_F, TINY_F_WEIGHTS),
+           "G": (TINY_G, TINY_G_WEIGHTS)}
 
 
 def make_model_dir(tmp_path, which: str, dtype: str = "bfloat16") -> str:
