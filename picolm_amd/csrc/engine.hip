@@ -370,6 +370,7 @@ struct picolm_engine {
     int decode_blocks_per_chunk = 1, decode_max_pages_per_chunk = 64;
     int counters_needed = 0;
     bool recordable = true;                // every called operation says that its launches may be recorded
+    bool call_on_ring = false;             // a called operation uses a cache group that keeps a ring of pages
     size_t partial_floats_per_seq_chunk = 0;   // max over attention operations of H * (d + 2)
     int prep_n = 0;                        // widest output that prepares a norm
     // the running step
@@ -471,6 +472,7 @@ static int check_program(const picolm_program* p, picolm_engine* e) {
                 }
                 if (o.out_norm_weight) {
                     E_REQUIRE(-1, o.epilogue == 1 && o.out_norm_eps > 0.f, "engine: operation %d: only an accumulating product prepares a norm", i);
+                    E_REQUIRE(-1, o.rows == PICOLM_ROWS_STEP, "engine: operation %d: only a product over every row of the step prepares a norm", i);
                     e->prep_n = std::max(e->prep_n, o.n);
                 }
                 break;
@@ -597,6 +599,7 @@ extern "C" int picolm_engine_create(const picolm_program* program, int64_t max_t
             if (!(o.call_flags & PICOLM_CALL_RECORDABLE)) e->recordable = false;
             if (!(o.call_flags & PICOLM_CALL_KV)) continue;
             const KVGroup& g = e->kv[o.kv_group];
+            if (g.is_ring()) e->call_on_ring = true;
             if (o.kv_writes) e->group_written[o.kv_group] = 1;
             if (!(o.call_flags & PICOLM_CALL_ATTENDS)) continue;
             e->group_attended[o.kv_group] = 1;
@@ -1472,6 +1475,13 @@ extern "C" int picolm_engine_step(picolm_engine* e, int32_t n_seq, const int32_t
         for (auto& w : wanted) *n_rows += (int)w.size();
     }
     if (T == n_seq && last_of_each) return decode_step(e, sl, pos0, tokens, nullptr, logits, stream);
+    // A ring holds a window and WINDOW_STEP_TOKENS new tokens.  The ATTENTION operation writes and
+    // answers a longer prompt slice by slice; a called operation sees the step as a whole.
+    if (e->call_on_ring)
+        for (int i = 0; i < n_seq; ++i)
+            E_REQUIRE(PICOLM_ERR_STEP, nn[i] <= WINDOW_STEP_TOKENS,
+                      "a called operation on a cache group with a window takes steps of up to %d tokens a sequence, sequence %d brings %d",
+                      WINDOW_STEP_TOKENS, i, nn[i]);
     TRY(reserve_many(e, sl, lengths));
     TRY(flush_tables(e, stream));
     plan_step(e, e->plan, sl, pos0, nn, tokens, wanted);
@@ -1517,6 +1527,7 @@ extern "C" int64_t picolm_engine_info(picolm_engine* e, int32_t what) {
         case 5: return e->max_pages;
         case 6: return (int64_t)e->device_bytes;
         case 7: return e->version;
+        case 8: return e->call_on_ring ? WINDOW_STEP_TOKENS : 0;
     }
     return -1;
 }
@@ -1770,7 +1781,8 @@ extern "C" int picolm_engine_generate(picolm_engine* e, int32_t n_prompts, const
                 if (done[i] < prompt_lens[ids[i]]) left.push_back(i);
             if (left.empty()) break;
             const int budget = e->prefill_step_tokens;
-            const int share = total <= budget ? (1 << 30) : std::max(64, budget / (int)left.size() / 64 * 64);
+            int share = total <= budget ? (1 << 30) : std::max(64, budget / (int)left.size() / 64 * 64);
+            if (e->call_on_ring) share = std::min(share, WINDOW_STEP_TOKENS);      // what such a step may bring a sequence
             int64_t room = total <= budget ? total : std::max<int64_t>(budget, 64 * (int64_t)left.size());
             sl.clear(), nn.clear(), toks.clear(), counts.clear(), idx.clear();
             std::vector<int> ending;

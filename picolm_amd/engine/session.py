@@ -39,6 +39,9 @@ class Session:
                                    time_ops=time_ops)
         self.cache = EngineCache(self.engine, model.cache_spec, model.runtime.dtype, model.runtime.device)
         self.graphs = graphs and self.engine.program.recordable
+        # the most tokens a sequence may bring in one step (0: any number): a called operation on a
+        # group with a window sees a step whole, and the group's ring takes in 256 tokens at once
+        self.most_new_tokens = self.engine.info(8)
 
     # -- slots -------------------------------------------------------------------------------
     def begin(self, n: int = 1) -> list[int]:

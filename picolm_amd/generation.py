@@ -186,20 +186,23 @@ class GenerationLoop:
 PREFILL_STEP_TOKENS = 16384        # most tokens of one prefill step: what sizes the step's workspace
 
 
-def prefill_steps(lengths, budget: int = PREFILL_STEP_TOKENS):
+def prefill_steps(lengths, budget: int = PREFILL_STEP_TOKENS, most: int = 0):
     """How a batch of prompts of these lengths goes through the model: a list of steps, each a list
     of (sequence, first token, count).  Prompts that fit the budget together are one step (picolm
     prefills a prompt in one call too, picolm/picolm.c:1502-1530).  Otherwise every step gives each
     unfinished sequence an equal share of the budget, in whole cache pages, and a sequence joins
-    the later steps with what it has left, appended to what its slot already holds."""
+    the later steps with what it has left, appended to what its slot already holds.  `most`: the
+    most tokens a sequence may bring in one step (0: any number)."""
     lengths = [int(n) for n in lengths]
-    if sum(lengths) <= budget:
+    if sum(lengths) <= budget and not (most and max(lengths, default=0) > most):
         return [[(i, 0, n) for i, n in enumerate(lengths)]]
     done = [0] * len(lengths)
     steps = []
     while any(d < n for d, n in zip(done, lengths)):
         left = [i for i, n in enumerate(lengths) if done[i] < n]
         share = max(64, budget // len(left) // 64 * 64)
+        if most:
+            share = min(share, most)
         step, room = [], max(budget, 64 * len(left))
         for i in left:
             take = min(lengths[i] - done[i], share, room)
@@ -258,7 +261,7 @@ class SessionStepper:
     def step(self, slots, tokens):
         """The last row's logits of every sequence.  Prompts beyond the budget of one step go in as
         several steps (`prefill_steps`); each sequence's row is kept from the step that ends it."""
-        plan = prefill_steps([len(t) for t in tokens], self.prefill_step_tokens)
+        plan = prefill_steps([len(t) for t in tokens], self.prefill_step_tokens, self.session.most_new_tokens)
         if len(plan) == 1:
             return self.session.step(slots, tokens)
         import torch

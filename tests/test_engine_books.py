@@ -30,6 +30,36 @@ def test_an_ill_formed_program_is_refused_with_the_operation_named():
         NativeEngine(b.finish(V, CacheSpec([], [])), 64, 64, 1, "cpu", host_only=True)
     with pytest.raises(CacheError, match="positive"):
         host_engine(max_tokens=0)
+    # a norm is prepared for every row of the step or not at all
+    b = P.ProgramBuilder(torch.float32, host_only=True)
+    x = b.buffer("residual", D, torch.float32)
+    b.embed(torch.zeros(V, D), x)
+    few = b.buffer("few", D, torch.float32, P.ROWS_WANTED)
+    acc = b.buffer("acc", D, torch.float32, P.ROWS_WANTED)
+    b.linear(torch.zeros(D, D), few, acc, 1, rows=P.ROWS_WANTED, out_norm=P.NormRef(torch.ones(D), 1e-5))
+    lg = b.buffer("logits", V, torch.float32, P.ROWS_WANTED)
+    b.linear(torch.zeros(V, D), acc, lg, 0, rows=P.ROWS_WANTED)
+    b.logits_buffer = lg
+    with pytest.raises(KernelError, match="operation 1: only a product over every row of the step prepares a norm"):
+        NativeEngine(b.finish(V, CacheSpec([], [])), 64, 64, 1, "cpu", host_only=True)
+
+
+def test_a_called_operation_on_a_ring_is_given_no_more_than_the_ring_takes_in():
+    """The attention operation answers a long prompt over a window slice by slice; a called
+    operation sees a step whole, so a step that its ring cannot take in at once is refused
+    before anything moves."""
+    e = host_engine(max_tokens=64 * 40, max_seq_len=1024, n_slots=2, layers=2, windows=(0, 100), v_head_dim=16)
+    a, b = e.slot_alloc(), e.slot_alloc()
+    free = [e.free_pages(0), e.free_pages(1)]
+    with pytest.raises(StepError, match="up to 256 tokens a sequence, sequence 1 brings 257"):
+        e.step([a, b], [[1] * 10, [2] * 257])
+    assert [e.free_pages(0), e.free_pages(1)] == free and (e.length(a), e.length(b)) == (0, 0)
+    e.step([a, b], [[1] * 10, [2] * 256])
+    e.step([a, b], [[1] * 256, [2] * 200])                  # and goes on in further steps
+    assert (e.length(a), e.length(b)) == (266, 456)
+    whole = host_engine(max_tokens=64 * 40, max_seq_len=1024, n_slots=2, layers=2, windows=(0,), v_head_dim=16)
+    s = whole.slot_alloc()
+    whole.step([s], [[1] * 700])                             # no ring: any length
 
 
 def test_slots_and_pages_are_handed_out_and_taken_back():

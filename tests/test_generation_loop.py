@@ -213,3 +213,7 @@ def test_prompts_are_cut_into_steps_within_the_token_budget():
             seen[i] += count
     assert seen == lens
     assert len(prefill_steps([100] * 40, 64)) == 2                       # more sequences than the budget has pages: a page each
+    # a model whose steps take no more than 256 tokens of a sequence: further steps, also within the budget
+    assert prefill_steps([10, 300, 600], 4096, most=256) == [[(0, 0, 10), (1, 0, 256), (2, 0, 256)], [(1, 256, 44), (2, 256, 256)],
+                                                             [(2, 512, 88)]]
+    assert prefill_steps([10, 200], 4096, most=256) == [[(0, 0, 10), (1, 0, 200)]]

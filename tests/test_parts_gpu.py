@@ -1184,3 +1184,127 @@ def test_a_python_part_that_says_graph_safe_is_recorded_and_replayed(tmp_path):
         for i in range(2):
             ref = truth[i][4 + j]
             assert np.abs(row[i].double().cpu().numpy() - ref).max() <= tiny.tolerance("bfloat16", truth[i], tiny.spread(128, 0.08))
+
+
+def test_a_toy_mixer_over_a_window_takes_long_prompts_in_steps_that_fit_its_ring(tmp_path):
+    """A one-head attention with a window of 40 keys, defined here and run as a called operation
+    on a group that keeps a ring of pages.  The attention operation answers a long prompt over a
+    ring slice by slice; a called operation sees its step whole, so the engine refuses a step of
+    more than 256 tokens a sequence, says how many a step may bring, and both generation loops cut
+    the prompts accordingly: their tokens are those of the plain model with the same window."""
+    from picolm_amd import SamplingParams
+    from picolm_amd.cache import PAGE_TOKENS, window_ring_pages
+    from picolm_amd.config import register_architecture, unregister_architecture
+    from picolm_amd.engine import DecoderModel, Session, StepError, load_model
+    from picolm_amd.generation import generate
+    from picolm_amd.parts import KVRequest, LMHead, Mixer, PreNormBlock, RMSNorm, SwiGLU, TokenEmbedding
+    from picolm_amd.weights import TensorSpec, write_random_model
+    DK, WINDOW = 16, 40
+
+    class ToyConfig:
+        def __init__(self, d):
+            self.d = dict(d)
+            self.hidden_size, self.vocab_size, self.intermediate_size = d["hidden_size"], d["vocab_size"], d["intermediate_size"]
+            self.max_position_embeddings = d["max_position_embeddings"]
+            self.torch_dtype = "bfloat16"
+            self.eos_token_ids = ()
+
+        def to_dict(self):
+            return dict(self.d)
+
+    class NearKeys(Mixer):
+        def __init__(self, prefix, D):
+            self.prefix, self.D, self.w = prefix, D, {}
+
+        def tensor_specs(self):
+            return [TensorSpec(self.prefix + c, (DK, self.D)) for c in "qkv"] + [TensorSpec(self.prefix + "o", (self.D, DK))]
+
+        def load(self, fetch, runtime):
+            self.w = {n: fetch.get(self.prefix + n).float() for n in "qkvo"}
+
+        def cache_requests(self):
+            return KVRequest(1, DK, WINDOW), None
+
+        def forward(self, ctx, h, residual):
+            k_pages, v_pages, table, ring = ctx.kv()
+            assert ring == window_ring_pages(WINDOW) < table.shape[1]
+            b, row = ctx.batch, 0
+            for slot, p0, n in zip(b.slots, b.pos0, b.n_new):
+                x = h[row:row + n].float()
+                q, k, v = x @ self.w["q"].T, x @ self.w["k"].T, x @ self.w["v"].T
+                lo = max(0, p0 - WINDOW + 1)                              # the oldest key that any of the new queries sees
+                pos = torch.arange(lo, p0 + n, device=x.device)
+                page, at = table[slot, (pos // PAGE_TOKENS) % ring].long(), pos % PAGE_TOKENS
+                new = slice(p0 - lo, None)
+                k_pages[page[new], 0, at[new]] = k.to(k_pages.dtype)
+                v_pages[page[new], 0, :, at[new]] = v.to(v_pages.dtype)
+                keys, values = k_pages[page, 0, at].float(), v_pages[page, 0, :, at].float()
+                s = q @ keys.T / math.sqrt(DK)
+                hidden = (pos[None, :] > pos[new, None]) | (pos[new, None] - pos[None, :] >= WINDOW)
+                residual[row:row + n] += (torch.softmax(s.masked_fill(hidden, float("-inf")), dim=-1) @ values) @ self.w["o"].T
+                row += n
+
+    def build(cfg):
+        D = cfg.hidden_size
+        emb = TokenEmbedding("emb.weight", cfg.vocab_size, D)
+        blocks = [PreNormBlock(RMSNorm(f"l{i}.norm1.weight", D, 1e-5), NearKeys(f"l{i}.mix.", D),
+                               RMSNorm(f"l{i}.norm2.weight", D, 1e-5), SwiGLU(f"l{i}.ffn.", D, cfg.intermediate_size)) for i in range(2)]
+        return DecoderModel(cfg, emb, blocks, RMSNorm("final.weight", D, 1e-5),
+                            LMHead("head.weight", cfg.vocab_size, D, emb, tied=True))
+
+    register_architecture("ToyNearKeysLM", ToyConfig, build)
+    try:
+        cfg = ToyConfig(dict(architectures=["ToyNearKeysLM"], hidden_size=40, vocab_size=77, intermediate_size=56,
+                             max_position_embeddings=1024))
+        d = write_random_model(cfg, str(tmp_path / "toy"), seed=6, std=0.3)
+        model = load_model(d, dtype="float32")
+        w = tiny.read_weights_f64(d)
+
+        def plain(tokens):
+            x = w["emb.weight"][tokens]
+            n = len(tokens)
+            far = np.arange(n)[:, None] - np.arange(n)[None, :]
+            for i in range(2):
+                hh = P.rmsnorm(x, w[f"l{i}.norm1.weight"], 1e-5)
+                q, k, v = (hh @ w[f"l{i}.mix.{c}"].T for c in "qkv")
+                s = q @ k.T / math.sqrt(DK)
+                s[(far < 0) | (far >= WINDOW)] = -np.inf
+                p = np.exp(s - s.max(axis=1, keepdims=True))
+                x = x + (p / p.sum(axis=1, keepdims=True)) @ v @ w[f"l{i}.mix.o"].T
+                x = x + P.swiglu(P.rmsnorm(x, w[f"l{i}.norm2.weight"], 1e-5), w[f"l{i}.ffn.gate_proj.weight"],
+                                 w[f"l{i}.ffn.up_proj.weight"], w[f"l{i}.ffn.down_proj.weight"])
+            return P.rmsnorm(x, w["final.weight"], 1e-5) @ w["emb.weight"].T
+
+        def plain_greedy(prompt, n_new):
+            toks = list(prompt)
+            for _ in range(n_new):
+                toks.append(int(np.argmax(plain(toks)[-1])))
+            return toks[len(prompt):]
+        rng = np.random.default_rng(12)
+        reqs = [tiny.random_tokens(rng, n, 77) for n in (300, 20, 600)]
+        s = Session(model, max_tokens=2048, n_slots=3)
+        assert s.most_new_tokens == 256
+        slots = s.begin(3)
+        with pytest.raises(StepError, match="up to 256 tokens a sequence, sequence 0 brings 300"):
+            s.step(slots, reqs)
+        assert [s.length(x) for x in slots] == [0, 0, 0]
+        # whole prompts in steps that fit, every position against the plain model
+        got = [[], [], []]
+        for lo in range(0, 600, 256):
+            live = [i for i in range(3) if len(reqs[i]) > lo]
+            out = s.step([slots[i] for i in live], [reqs[i][lo:lo + 256] for i in live],
+                         [list(range(len(reqs[i][lo:lo + 256]))) for i in live]).double().cpu().numpy()
+            for i in live:
+                n = len(reqs[i][lo:lo + 256])
+                got[i].append(out[:n])
+                out = out[n:]
+        for i in range(3):
+            assert np.abs(np.concatenate(got[i]) - plain(reqs[i])).max() < 1e-4, i
+        s.release(slots)
+        want = [plain_greedy(r, 6) for r in reqs]
+        outs = generate(s, reqs, max_new_tokens=6, params=SamplingParams(temperature=0.0), stop_ids=(), batch_size=3)
+        assert [o.tokens for o in outs] == want
+        tokens, reasons = s.engine.generate(reqs, 6, SamplingParams(temperature=0.0), (), batch_size=3)
+        assert tokens == want and reasons == ["length"] * 3
+    finally:
+        unregister_architecture("ToyNearKeysLM")
