@@ -250,6 +250,9 @@ class ProgramBuilder:
 
         def entry(_user, view):
             try:
+                if view.contents.struct_bytes != ctypes.sizeof(StepView):
+                    raise RuntimeError(f"the library's step view has {view.contents.struct_bytes} bytes, this module's "
+                                       f"{ctypes.sizeof(StepView)}: picolm_amd/engine/program.py and csrc/engine.h differ")
                 fn(view.contents)
                 return 0
             except BaseException as exc:        # nothing may cross the C frames between here and the step's caller
