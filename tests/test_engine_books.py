@@ -265,3 +265,28 @@ def test_a_long_prefill_step_over_a_window_is_cut_along_positions():
     e.step(slots, [[1] * 200, [2] * 256, [3] * 9])          # no sequence brings more than 256: no slices
     with pytest.raises(Exception, match="no array"):
         e.step_array("window_chunk.0.rows")
+
+
+def test_more_shapes_of_decode_steps_than_the_engine_keeps():
+    """The engine keeps the blocks (and recordings) of 48 shapes of decode steps and lets the least
+    recently used go: batches of 1 to 60 sequences in turn, then the first shapes again, are all
+    planned as the plain planner plans them."""
+    n_slots = 60
+    e = host_engine(max_tokens=64 * 4 * n_slots, max_seq_len=256, n_slots=n_slots)
+    slots = [e.slot_alloc() for _ in range(n_slots)]
+    e.step(slots, [[1] * (3 + i % 5) for i in range(n_slots)])
+    length = [3 + i % 5 for i in range(n_slots)]
+    for n in list(range(1, n_slots + 1)) + [1, 2, 3, 60, 30]:
+        for _ in range(2):
+            pos0 = length[:n]
+            e.step(slots[:n], [[9 + i] for i in range(n)])
+            table = table_of(e, n_slots, 4)
+            ppc = decode_pages_per_chunk(pos0, G, 16)
+            entries, _ = decode_chunk_list(slots[:n], pos0, 0, ppc, table, 4)
+            got = e.step_array("chunks.0").reshape(-1, 8)
+            assert got[0, 0] == len(entries) and np.array_equal(got[1:1 + len(entries)], entries), n
+            assert np.array_equal(e.step_array("tok_pos"), pos0) and np.array_equal(e.step_array("seq_slot"), slots[:n])
+            assert np.array_equal(e.step_array("write_pages.0"), token_pages(np.arange(n), pos0, slots[:n], table, 4))
+            for i in range(n):
+                length[i] += 1
+    assert [e.length(s) for s in slots] == length

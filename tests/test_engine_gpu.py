@@ -437,6 +437,38 @@ def test_recorded_decode_steps_equal_eager_ones(folders):
     assert torch.equal(outs[True], outs[False])
 
 
+def test_more_shapes_of_recorded_decode_steps_than_the_engine_keeps(folders):
+    """Batches of 1 to 56 sequences, three decode steps each: every batch size is a recorded step
+    of its own, the engine keeps 48 of them and lets the least recently used go.  Each step gives
+    the same bits as in a session that launches its kernels one by one, also the shapes that come
+    back after they were dropped."""
+    from picolm_amd.engine import Session, load_model
+    d = folders["A"]
+    model = load_model(d, dtype="bfloat16")
+    V = tiny.TINY_A["vocab_size"]
+    rng = np.random.default_rng(48)
+    n_all = 56
+    prompts = [tiny.random_tokens(rng, 3 + i % 7, V) for i in range(n_all)]
+    order = list(range(1, n_all + 1)) + [1, 2, 3, 56, 30]
+    feed = [[tiny.random_tokens(rng, n, V) for _ in range(3)] for n in order]
+    outs = {}
+    for graphs in (True, False):
+        s = Session(model, max_tokens=64 * 2 * n_all, max_seq_len=128, n_slots=n_all, graphs=graphs)
+        slots = s.begin(n_all)
+        s.step(slots, prompts)
+        rows, start = [], 0
+        for n, toks in zip(order, feed):
+            batch = [slots[(start + k) % n_all] for k in range(n)]      # in turn, so that no sequence outgrows the cache
+            start += n
+            for t in toks:
+                rows.append(s.step(batch, [[x] for x in t]).clone())
+        outs[graphs] = rows
+        if graphs:
+            assert s.recorded_steps() == 48
+    for a, b in zip(outs[True], outs[False]):
+        assert torch.equal(a, b)
+
+
 @pytest.mark.parametrize("which", ["C", "D"])
 def test_a_batch_that_continues_where_another_stopped(which, folders):
     """One batch ends and gives its slots back; the next gets the same slots (with other pages)
