@@ -57,9 +57,6 @@ class _SlotCount:
     def n_free(self) -> int:
         return self._e.info(2)
 
-    def is_live(self, slot: int) -> bool:
-        return self._e.length(slot) >= 0
-
 
 class _KVEntries:
     """keys [entry][page][G][64][d] and values [entry][page][G][d][64] of one cache group, as the

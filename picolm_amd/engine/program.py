@@ -116,11 +116,6 @@ class Rows:
     x: int = -1
 
 
-class CallFailed(Exception):
-    """Raised by `NativeEngine` in place of the engine's error when a called Python operation
-    raised: it carries that exception."""
-
-
 class ProgramBuilder:
     """Collects the operations and buffers that parts emit.  Buffers are named; two parts that
     ask for the same name share the memory (a layer's scratch is the next layer's), and the

@@ -283,18 +283,6 @@ def _decode_check(q, partial, n_seq, chunk_list, n_chunks, pages_per_chunk, max_
     _i32("attn.seq_pos0", seq_pos0, n_seq)
 
 
-def attn_decode_geometry(dtype: torch.dtype, n_seq: int, H: int, G: int, d: int) -> tuple[int, int]:
-    """(workgroups per chunk of the work list, the most pages a chunk should have) of the decode
-    attention kernel that will run for these sizes."""
-    R = H // G
-    if attn_decode_rope_takes(dtype, d):
-        # up to 64 pages a chunk: 16 tiles of 32 keys for each of eight waves, 32 for each of the four
-        # that run for many sequences (longer chunks are longer streams and fewer partial results:
-        # 3 % less step time at contexts of 16,000 tokens, 2 % at batch 64 with 4,000)
-        return G * ((R + 31) // 32), 64
-    return G * ((R + 15) // 16), 16
-
-
 def attn_decode_generic(q, k_pages, v_pages, out, partial, n_seq, chunk_list, n_chunks, pages_per_chunk,
                         max_splits, seq_pos0, page_table, ring_pages, H, G, d, window, scale) -> None:
     _attn_check(q, k_pages, v_pages, out, page_table, H, G, d)
@@ -474,14 +462,6 @@ def kv_store_tiles(qkv, k_pages, v_pages, cos, sin, style: int, batch, page_tabl
         _ptr(page_table), page_table.shape[1], ring_pages, H, G, d, _stream()))
 
 
-def attn_prefill_rope_takes(dtype: torch.dtype, d: int, T: int | None = None) -> bool:
-    """Whether the prefill attention that rotates q itself takes this case and, given the step's
-    number of tokens, whether the library would take that way (long prompts gain by it)."""
-    if not (dtype == torch.bfloat16 and bool(lib().picolm_attn_mfma_takes(d))):
-        return False
-    return T is None or bool(lib().picolm_attn_prefill_rotates_q(int(T)))
-
-
 def attn_prefill_rope(qkv, k_pages, v_pages, out, batch, page_table, ring_pages, H, G, d, window, scale, cos, sin, style) -> None:
     """attn_prefill_mfma with q taken from the float rows qkv [T, (H+2G)d] and rotated inside the
     kernel (cos, sin None: no rotation).  The step's keys and values must be in the cache already
@@ -527,11 +507,6 @@ def attn_decode_mfma(q, k_pages, v_pages, out, partial, n_seq, chunk_list, n_chu
         _ptr(q), _ptr(k_pages), _ptr(v_pages), _ptr(out), _ptr(partial if max_splits > 1 else None), n_seq,
         _ptr(chunk_list), n_chunks, pages_per_chunk, max_splits, _ptr(seq_pos0), _ptr(page_table),
         page_table.shape[1], ring_pages, H, G, d, window, c_float(scale), _ptr(chunks_done), _stream()))
-
-
-def attn_decode_rope_takes(dtype: torch.dtype, d: int) -> bool:
-    """Whether the decode kernel that rotates and writes the cache itself takes this case."""
-    return dtype == torch.bfloat16 and bool(lib().picolm_attn_mfma_takes(d))
 
 
 def attn_decode_rope(qkv, k_pages, v_pages, out, partial, n_seq, chunk_list, n_chunks, pages_per_chunk, max_splits,
