@@ -4,6 +4,11 @@ picolm has no such table: it sniffs the architecture from substrings of GGUF met
 (picolm/model_gguf.c:729-751) and from which tensors exist.  Here an architecture is an
 entry with two callables: one that types the config.json, one that builds the model's
 parts from the typed configuration.
+
+An architecture that lives outside the package registers itself when its module is imported.
+The command line, trace replay and every other entry point import the modules named in the
+environment variable PICOLM_ARCHITECTURES (comma-separated, found on sys.path like any module)
+before they look a name up, so that such an architecture needs no change to the package.
 """
 from __future__ import annotations
 
@@ -49,8 +54,37 @@ def _load_builtin() -> None:
         from ..engine import llama  # noqa: F401
 
 
-def known_architectures() -> list[str]:
+_OUTSIDE_LOADED = False
+
+
+def _load_all() -> None:
+    """Before a name is looked up: the library's own architectures and those of the modules that
+    PICOLM_ARCHITECTURES names (which import the package, so they wait until it is whole)."""
+    global _OUTSIDE_LOADED
     _load_builtin()
+    if not _OUTSIDE_LOADED:
+        _OUTSIDE_LOADED = True
+        import_architecture_modules(os.environ.get("PICOLM_ARCHITECTURES", ""))
+
+
+def import_architecture_modules(names: str) -> list[str]:
+    """Imports the comma-separated modules, each of which calls `register_architecture`; returns
+    their names.  A module that cannot be imported is a configuration error that names it."""
+    import importlib
+    done = []
+    for name in (n.strip() for n in names.split(",")):
+        if not name:
+            continue
+        try:
+            importlib.import_module(name)
+        except Exception as exc:
+            raise ConfigError(f"PICOLM_ARCHITECTURES: cannot import '{name}': {type(exc).__name__}: {exc}") from exc
+        done.append(name)
+    return done
+
+
+def known_architectures() -> list[str]:
+    _load_all()
     return sorted(_REGISTRY)
 
 
@@ -65,7 +99,7 @@ def architecture_name(config_dict: dict) -> str:
 
 
 def resolve(config_dict: dict) -> Architecture:
-    _load_builtin()
+    _load_all()
     name = architecture_name(config_dict)
     if name not in _REGISTRY:
         raise ConfigError(f"architectures: '{name}' is not registered "

@@ -1515,6 +1515,7 @@ extern "C" int64_t picolm_engine_info(picolm_engine* e, int32_t what) {
         case 1: return e->n_slots;
         case 2: return (int64_t)e->slots.free_.size();
         case 3: {
+            if (e->kv.empty()) return (int64_t)1 << 40;       // a model without keys and values has no pages to run out of
             int64_t free_pages = -1;
             for (const KVGroup& g : e->kv) free_pages = free_pages < 0 ? g.pool.n_free() : std::min<int64_t>(free_pages, g.pool.n_free());
             return std::max<int64_t>(free_pages, 0) * PAGE_TOKENS;

@@ -13,12 +13,12 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
 
 class TraceRun:
-    def __init__(self, model_dir, dtype, out_dir, max_tokens):
+    def __init__(self, model_dir, dtype, out_dir, max_tokens, env=None):
         self.out_dir = out_dir
         self.proc = subprocess.Popen(
             [sys.executable, os.path.join(ROOT, "bin", "trace_run"), "--model", model_dir, "--dtype", dtype,
              "--out", out_dir, "--max-tokens", str(max_tokens)],
-            stdin=subprocess.PIPE, stdout=subprocess.PIPE, text=True, bufsize=1)
+            stdin=subprocess.PIPE, stdout=subprocess.PIPE, text=True, bufsize=1, env=env)
         self.n = 0
 
     def step(self, entries, end=()):

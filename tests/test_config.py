@@ -1,5 +1,6 @@
 """Configuration and registry (no GPU)."""
 import json
+import os
 
 import pytest
 
@@ -128,3 +129,26 @@ def test_head_size_limits_are_named_when_the_configuration_is_read():
         LlamaConfig.from_dict(dict(d, head_dim=1026))
     assert LlamaConfig.from_dict(dict(d, head_dim=1024)).head_dim == 1024
     assert LlamaConfig.from_dict(dict(d, head_dim=320)).head_dim == 320              # four times picolm's own bound
+
+
+def test_modules_named_in_the_environment_register_their_architectures(tmp_path, monkeypatch):
+    """An architecture outside the package: its module is named in PICOLM_ARCHITECTURES and
+    imported before the first name is looked up; one that cannot be imported is an error that
+    names it."""
+    import subprocess
+    import sys
+    from picolm_amd.config import import_architecture_modules
+    (tmp_path / "my_arch.py").write_text(
+        "from picolm_amd.config import register_architecture, LlamaConfig\n"
+        "register_architecture('MyLM', LlamaConfig.from_dict, lambda cfg: None)\n")
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    env = dict(os.environ, PYTHONPATH=os.pathsep.join([str(tmp_path), root]), PICOLM_ARCHITECTURES=" my_arch ,")
+    out = subprocess.run([sys.executable, "-c", "from picolm_amd import known_architectures; print(known_architectures())"],
+                         env=env, capture_output=True, text=True)
+    assert out.returncode == 0 and "'LlamaForCausalLM', 'MyLM'" in out.stdout, out.stderr
+    out = subprocess.run([sys.executable, "-c", "from picolm_amd import known_architectures; print(known_architectures())"],
+                         env=dict(env, PICOLM_ARCHITECTURES="no_such_module_here"), capture_output=True, text=True)
+    assert out.returncode != 0 and "PICOLM_ARCHITECTURES: cannot import 'no_such_module_here'" in out.stderr
+    assert import_architecture_modules("") == [] and import_architecture_modules(" , ") == []
+    with pytest.raises(ConfigError, match="cannot import 'no_such_module_here'"):
+        import_architecture_modules("no_such_module_here")

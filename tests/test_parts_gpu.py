@@ -1308,3 +1308,130 @@ def test_a_toy_mixer_over_a_window_takes_long_prompts_in_steps_that_fit_its_ring
         assert tokens == want and reasons == ["length"] * 3
     finally:
         unregister_architecture("ToyNearKeysLM")
+
+
+TOY_ARCHITECTURE_MODULE = '''
+"""An architecture outside the package: a decoder whose mixer is the running mean of its inputs,
+kept as state per sequence.  Importing the module registers it."""
+import torch
+
+from picolm_amd.config import register_architecture
+from picolm_amd.engine import DecoderModel
+from picolm_amd.parts import LMHead, Mixer, PreNormBlock, RMSNorm, StateRequest, SwiGLU, TokenEmbedding
+from picolm_amd.weights import TensorSpec
+
+
+class Config:
+    def __init__(self, d):
+        self.d = dict(d)
+        self.hidden_size, self.vocab_size, self.intermediate_size = d["hidden_size"], d["vocab_size"], d["intermediate_size"]
+        self.max_position_embeddings = d["max_position_embeddings"]
+        self.torch_dtype = "bfloat16"
+        self.eos_token_ids = ()
+
+    def to_dict(self):
+        return dict(self.d)
+
+
+class RunningMean(Mixer):
+    def __init__(self, name, D):
+        self.name, self.D, self.w = name, D, None
+
+    def tensor_specs(self):
+        return [TensorSpec(self.name, (self.D, self.D))]
+
+    def load(self, fetch, runtime):
+        self.w = fetch.get(self.name).float()
+
+    def cache_requests(self):
+        return None, StateRequest((self.D + 1,), torch.float32)
+
+    def forward(self, ctx, h, residual):
+        state, b, row = ctx.state(), ctx.batch, 0
+        for slot, n in zip(b.slots, b.n_new):
+            x = h[row:row + n].float()
+            sums = state[slot, :self.D] + torch.cumsum(x, dim=0)
+            counts = state[slot, self.D] + torch.arange(1, n + 1, device=x.device, dtype=torch.float32)
+            residual[row:row + n] += (sums / counts[:, None]) @ self.w.T
+            state[slot, :self.D] = sums[-1]
+            state[slot, self.D] = counts[-1]
+            row += n
+
+
+def build(cfg):
+    D = cfg.hidden_size
+    emb = TokenEmbedding("emb.weight", cfg.vocab_size, D)
+    block = PreNormBlock(RMSNorm("norm1.weight", D, 1e-5), RunningMean("mean.weight", D),
+                         RMSNorm("norm2.weight", D, 1e-5), SwiGLU("ffn.", D, cfg.intermediate_size))
+    return DecoderModel(cfg, emb, [block], RMSNorm("final.weight", D, 1e-5), LMHead("head.weight", cfg.vocab_size, D, emb, tied=True))
+
+
+register_architecture("ToyOutsideLM", Config, build)
+'''
+
+
+def test_an_architecture_from_a_module_outside_the_package_runs_through_the_programs(tmp_path):
+    """The module above lies in a folder of its own.  With that folder on the module path and the
+    module's name in PICOLM_ARCHITECTURES, `bin/trace_run` and `bin/picolm` load a model of that
+    architecture, step it and generate with it, with no file of the package changed: the replayed
+    logits are those of a session in this process and of the plain form of the model."""
+    import subprocess
+    import sys
+    from picolm_amd.config import import_architecture_modules, unregister_architecture
+    from picolm_amd.engine import Session, load_model
+    from picolm_amd.weights import write_random_model
+    from replay_util import ROOT, TraceRun
+    folder = tmp_path / "outside"
+    folder.mkdir()
+    (folder / "toy_outside_arch.py").write_text(TOY_ARCHITECTURE_MODULE)
+    env = dict(os.environ, PICOLM_ARCHITECTURES="toy_outside_arch",
+               PYTHONPATH=os.pathsep.join([str(folder)] + [p for p in [os.environ.get("PYTHONPATH")] if p]))
+    sys.path.insert(0, str(folder))
+    try:
+        assert import_architecture_modules("toy_outside_arch") == ["toy_outside_arch"]
+        import toy_outside_arch
+        cfg = toy_outside_arch.Config(dict(architectures=["ToyOutsideLM"], hidden_size=40, vocab_size=77, intermediate_size=56,
+                                           max_position_embeddings=256))
+        d = write_random_model(cfg, str(tmp_path / "toy"), seed=14, std=0.3)
+        w = tiny.read_weights_f64(d)
+
+        def plain(tokens):
+            x = w["emb.weight"][tokens]
+            hh = P.rmsnorm(x, w["norm1.weight"], 1e-5)
+            x = x + (np.cumsum(hh, axis=0) / np.arange(1, len(tokens) + 1)[:, None]) @ w["mean.weight"].T
+            x = x + P.swiglu(P.rmsnorm(x, w["norm2.weight"], 1e-5), w["ffn.gate_proj.weight"], w["ffn.up_proj.weight"],
+                             w["ffn.down_proj.weight"])
+            return P.rmsnorm(x, w["final.weight"], 1e-5) @ w["emb.weight"].T
+        rng = np.random.default_rng(3)
+        a, b = tiny.random_tokens(rng, 30, 77), tiny.random_tokens(rng, 9, 77)
+        tr = TraceRun(d, "float32", str(tmp_path / "out"), 256, env=env)
+        got = tr.step([("a", a[:25], [0, 24]), ("b", b[:8], [7])])
+        assert np.abs(got - np.stack([plain(a)[0], plain(a)[24], plain(b)[7]])).max() < 5e-5
+        got = tr.step([("a", [a[25]], [0]), ("b", [b[8]], [0])], end=["b"])
+        assert np.abs(got - np.stack([plain(a)[25], plain(b)[8]])).max() < 5e-5
+        got = tr.step([("a", [a[26]], [0])], end=["a"])
+        assert np.abs(got[0] - plain(a)[26]).max() < 5e-5
+        tr.close()
+        # the command line generates with it: greedy tokens as a session in this process gives them
+        s = Session(load_model(d, dtype="float32"), max_tokens=256)
+        [slot] = s.begin(1)
+        seq = list(a[:12])
+        row = s.step([slot], [seq])[0]
+        want = []
+        for _ in range(5):
+            want.append(int(torch.argmax(row)))
+            row = s.step([slot], [[want[-1]]])[0]
+        out = subprocess.run([sys.executable, os.path.join(ROOT, "bin", "picolm"), d, "-p", " ".join(map(str, a[:12])), "-n", "5",
+                              "-t", "0", "--dtype", "float32"], env=env, capture_output=True, text=True, timeout=300)
+        assert out.returncode == 0, out.stderr
+        assert [int(t) for t in out.stdout.split()] == want
+        # without the variable the name is unknown, and the message says which names are known
+        bare = dict(env)
+        del bare["PICOLM_ARCHITECTURES"]
+        out = subprocess.run([sys.executable, os.path.join(ROOT, "bin", "picolm"), d, "-p", "1 2", "-n", "1"], env=bare,
+                             capture_output=True, text=True, timeout=300)
+        assert out.returncode != 0 and "ToyOutsideLM" in out.stderr and "LlamaForCausalLM" in out.stderr
+    finally:
+        sys.path.remove(str(folder))
+        sys.modules.pop("toy_outside_arch", None)
+        unregister_architecture("ToyOutsideLM")
