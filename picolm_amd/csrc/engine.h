@@ -237,7 +237,7 @@ int picolm_engine_op_times(picolm_engine* e, double* ms);
 // times 64; 2^40 for a model without cache groups), 4 recorded decode steps, 5 pages of a
 // sequence's table row, 6 bytes of device memory held, 7 the counter that moves when a slot or
 // page changes hands, 8 the most tokens a sequence may bring in one step (0: any number; 256
-// where a called operation uses a group with a window)
+// where a called operation uses a group with a window), 9 bytes of keys, values and state
 int64_t picolm_engine_info(picolm_engine* e, int32_t what);
 // keys [n_pages][G][64][d] and values [n_pages][G][d][64] of one cache entry (device memory)
 int picolm_engine_kv_entry(picolm_engine* e, int32_t group, int32_t entry, void** k, void** v, int64_t* n_pages);

@@ -1529,6 +1529,12 @@ extern "C" int64_t picolm_engine_info(picolm_engine* e, int32_t what) {
         case 6: return (int64_t)e->device_bytes;
         case 7: return e->version;
         case 8: return e->call_on_ring ? WINDOW_STEP_TOKENS : 0;
+        case 9: {
+            int64_t bytes = 0;
+            for (const KVGroup& g : e->kv) bytes += (int64_t)(g.k_entry_bytes + g.v_entry_bytes) * g.spec.n_entries;
+            for (const StateGroup& s : e->state) bytes += (int64_t)s.spec.n_entries * e->n_slots * s.spec.bytes_per_slot;
+            return bytes;
+        }
     }
     return -1;
 }

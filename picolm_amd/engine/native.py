@@ -104,7 +104,9 @@ class EngineCache:
         return self._e.info(3)
 
     def bytes(self) -> int:
-        return self._e.info(6)
+        """Bytes of the keys, values and per-sequence state (the engine's other device memory,
+        workspace and page tables, is in `engine.info(6)`)."""
+        return self._e.info(9)
 
     @property
     def version(self) -> int:

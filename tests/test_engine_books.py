@@ -65,6 +65,9 @@ def test_a_called_operation_on_a_ring_is_given_no_more_than_the_ring_takes_in():
 def test_slots_and_pages_are_handed_out_and_taken_back():
     e = host_engine()
     assert [e.info(i) for i in (0, 1, 2, 3, 5)] == [256, 3, 3, 640, 4]      # max_seq_len, slots, free slots, free tokens, pages a row
+    # keys and values: two entries of ten pages of G x 64 x d floats, twice; no state here, and one with state
+    assert e.info(9) == 2 * 2 * 10 * G * 64 * d * 4 and e.info(8) == 0
+    assert host_engine(state_shape=(4, 2)).info(9) == e.info(9) + 2 * 3 * 8 * 4
     a, b, c = e.slot_alloc(), e.slot_alloc(), e.slot_alloc()
     assert (a, b, c) == (0, 1, 2)
     with pytest.raises(CacheFull, match="all 3 slots"):
