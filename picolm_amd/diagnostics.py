@@ -84,8 +84,9 @@ def gpu_attn_diff(n_tok: int, H: int, G: int, d: int, seed: int = 42) -> int:
     (matrix cores where the head size allows) and the 32-bit kernels, against float64 on the host."""
     from . import kernels
     from .cache import PAGE_TOKENS
-    if min(n_tok, H, G, d) < 1 or H % G or d % 2 or d > 256:
-        raise SystemExit("--gpu-attn-diff n_tok n_heads n_kv_heads head_dim: heads in whole groups, an even head size up to 256")
+    from .parts.attention import MAX_HEAD_DIM
+    if min(n_tok, H, G, d) < 1 or H % G or d % 2 or d > MAX_HEAD_DIM:
+        raise SystemExit(f"--gpu-attn-diff n_tok n_heads n_kv_heads head_dim: heads in whole groups, an even head size up to {MAX_HEAD_DIM}")
     dev = _device()
     g = torch.Generator().manual_seed(seed)
     qkv = torch.randn(n_tok, (H + 2 * G) * d, generator=g)

@@ -386,7 +386,11 @@ def test_command_line_checks_and_speed_runs(folders, capsys):
     # attention: a head size of the matrix-core kernels, and one that only the plain kernels take
     assert cli.main(["--gpu-attn-diff", "200", "8", "2", "64"]) == 0
     assert cli.main(["--gpu-attn-diff", "70", "6", "3", "20", "-s", "5"]) == 0
-    assert capsys.readouterr().err.count("PASS") == 2
+    assert cli.main(["--gpu-attn-diff", "150", "4", "2", "96"]) == 0          # matrix cores at another head size
+    assert cli.main(["--gpu-attn-diff", "130", "2", "1", "320"]) == 0         # wider than the 256 columns a tile holds at a time
+    with pytest.raises(SystemExit, match="up to 1024"):
+        cli.main(["--gpu-attn-diff", "10", "2", "1", "1026"])
+    assert capsys.readouterr().err.count("PASS") == 4
     d = folders["A"]
     assert cli.main([d, "--benchmark-ctx", "-p", "5 6 7 8 9", "-n", "11", "-c", "100", "-t", "0"]) == 0
     rows = [l for l in capsys.readouterr().err.splitlines() if l and l[0].isdigit()]
