@@ -101,6 +101,59 @@ def prefill_flops(cfg, T: int) -> float:
     return product_flops(cfg, T) + attention_flops(cfg, T) + 2.0 * cfg.hidden_size * cfg.vocab_size
 
 
+def library_products(cfg, dev, prefill_rows: int) -> dict:
+    """A layer's four products (qkv, o, gate and up, down) at decode and prefill row counts: this
+    library's kernels with the epilogue each has in the model, and the vendor library's plain
+    product of the same shape (torch.matmul), in microseconds.  Every measurement replays a
+    recorded graph that walks copies of the weights in turn, more of them than the memory-side
+    cache holds, so that neither the host's launches nor that cache decide it."""
+    import torch
+
+    from picolm_amd import kernels
+    D, F = cfg.hidden_size, cfg.intermediate_size
+    shapes = [("qkv", cfg.q_size + 2 * cfg.kv_size, D, kernels.EPI_STORE, torch.float32), ("o", D, cfg.q_size, kernels.EPI_ACCUMULATE, torch.float32),
+              ("gate_up", 2 * F, D, kernels.EPI_SWIGLU, torch.bfloat16), ("down", D, F, kernels.EPI_ACCUMULATE, torch.float32)]
+
+    def replayed(calls, reps=3):
+        stream = torch.cuda.Stream()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.stream(stream):
+            for f in calls:
+                f()
+            stream.synchronize()
+            with torch.cuda.graph(graph, stream=stream):
+                for f in calls:
+                    f()
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        begin, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        begin.record()
+        for _ in range(reps):
+            graph.replay()
+        end.record()
+        torch.cuda.synchronize()
+        return begin.elapsed_time(end) / (reps * len(calls)) * 1e3
+
+    out = {}
+    for M in (1, 8, 64, prefill_rows):
+        row = {}
+        for name, N, K, epilogue, c_dtype in shapes:
+            copies = max(3, int(1.5e9 // (N * K * 2)))
+            a = torch.randn(M, K, device=dev).to(torch.bfloat16)
+            ws = [(torch.randn(N, K, device=dev) * 0.02).to(torch.bfloat16) for _ in range(copies)]
+            c = torch.zeros(M, N // 2 if epilogue == kernels.EPI_SWIGLU else N, device=dev, dtype=c_dtype)
+            plain = torch.empty(M, N, device=dev, dtype=torch.bfloat16)
+            row[name] = {"library_us": round(replayed([(lambda w=w: torch.matmul(a, w.t(), out=plain)) for w in ws]), 1),
+                         "ours_us": round(replayed([(lambda w=w: kernels.gemm(a, w, c, epilogue)) for w in ws]), 1)}
+            del ws
+        row["layer"] = {k: round(sum(v[k] for v in row.values()), 1) for k in ("library_us", "ours_us")}
+        out[f"rows_{M}"] = row
+        print(f"[bench] {M} rows: the library's four products {row['layer']['library_us']} us, ours {row['layer']['ours_us']} us",
+              file=sys.stderr, flush=True)
+    return {"library_products": out, "model": "layer sizes of " + str(cfg.hidden_size) + " x " + str(cfg.intermediate_size)}
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -125,6 +178,10 @@ def main() -> int:
     ap.add_argument("--weight-std", type=float, default=None,
                     help="standard deviation of the random weights (default: the shape's); 0 makes every operand of "
                          "every product zero, which shows what the GPU's power limit costs the same kernels on real data")
+    ap.add_argument("--library-products", action="store_true",
+                    help="time a layer's four products at 1, 8 and 64 rows and at the prefill's rows, this library's kernels "
+                         "(with their epilogues) beside torch.matmul (the vendor library's plain product), both replayed "
+                         "from a recorded graph over copies of the weights taken in turn; prints one JSON line")
     ap.add_argument("--steps-ahead", type=int, choices=[0, 1], default=1,
                     help="1 (the generation loop's way): the next step is launched before this step's tokens are "
                          "read on the host; 0: the host reads every step's tokens first")
@@ -151,6 +208,9 @@ def main() -> int:
         cfg_dict["num_hidden_layers"] = args.layers
     cfg = LlamaConfig.from_dict(cfg_dict)
     dev = torch.device("cuda:0")
+    if args.library_products:
+        print(json.dumps(library_products(cfg, dev, args.prefill_tokens)))
+        return 0
     t0 = time.time()
     if args.weight_std is not None:
         shape = dict(shape, std=args.weight_std)
