@@ -9,6 +9,12 @@
 extern "C" {
 #endif
 
+// element types of tensors and buffers: float, or bfloat16 stored as 16 bits
+#ifndef PICOLM_ELEMENT_TYPES
+#define PICOLM_ELEMENT_TYPES
+enum { PICOLM_F32 = 0, PICOLM_BF16 = 1 };
+#endif
+
 const char* picolm_last_error(void);
 // leaves a message for picolm_last_error(): for code outside the library that fails a call of the
 // library's (an operation of the caller's inside an engine's program)

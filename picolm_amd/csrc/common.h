@@ -7,7 +7,10 @@
 
 // ---- element types ------------------------------------------------------------------
 // Tensors are float (32-bit) or bf16 stored as uint16_t.  All arithmetic is float.
+#ifndef PICOLM_ELEMENT_TYPES
+#define PICOLM_ELEMENT_TYPES
 enum { PICOLM_F32 = 0, PICOLM_BF16 = 1 };
+#endif
 typedef uint16_t bf16_t;
 
 #define PAGE_TOKENS 64       // tokens of one cache page; also the key tile of attention

@@ -28,6 +28,12 @@
 extern "C" {
 #endif
 
+// element types of tensors and buffers: float, or bfloat16 stored as 16 bits
+#ifndef PICOLM_ELEMENT_TYPES
+#define PICOLM_ELEMENT_TYPES
+enum { PICOLM_F32 = 0, PICOLM_BF16 = 1 };
+#endif
+
 // return codes beside -1 (bad argument) and -2 (a launch failed)
 #define PICOLM_ERR_STEP (-10)        // a step that cannot run: a dead slot, a token outside the vocabulary
 #define PICOLM_ERR_CACHE_FULL (-11)  // no free slot or page, or a sequence longer than the cache takes

@@ -218,3 +218,22 @@ def test_prompts_beyond_the_budget_of_a_step_go_in_as_several_steps(folders):
         assert toks == [r.tokens for r in cut]
         if sp.greedy:
             assert toks == [r.tokens for r in whole]
+
+
+@pytest.mark.parametrize("dtype", ["f32", "bf16"])
+def test_a_client_written_in_c_builds_a_program_by_hand_and_steps_it(dtype):
+    """tests/c_client/tiny_llama.c sees the library through engine.h and api.h alone (compiled as
+    C11): it writes the launch program of a two-layer Llama by hand, steps unequal prompts and
+    single tokens, lets the library's loop generate, and holds the logits against a plain forward
+    pass of its own in double precision.  It exits with 0 when all of that agrees."""
+    import os
+    import subprocess
+    from c_client import build as c_client
+    from picolm_amd import kernels
+    library = kernels.lib()._name
+    exe = c_client.binary(library)
+    env = dict(os.environ, LD_LIBRARY_PATH=os.pathsep.join([os.path.dirname(library), os.environ.get("LD_LIBRARY_PATH", "")]))
+    out = subprocess.run([exe, dtype], env=env, capture_output=True, text=True, timeout=300)
+    assert out.returncode == 0, out.stdout + out.stderr
+    assert out.stdout.startswith(f"ok {dtype}: worst difference of the logits"), out.stdout
+    print(out.stdout.strip())
