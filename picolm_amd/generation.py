@@ -19,6 +19,8 @@ a stop token ends has by then been stepped once more, and that step's token is d
 """
 from __future__ import annotations
 
+import os
+
 import time
 from dataclasses import dataclass, field
 
@@ -217,10 +219,11 @@ def prefill_steps(lengths, budget: int = PREFILL_STEP_TOKENS, most: int = 0):
 
 def generate(model_or_session, prompts, max_new_tokens: int = 256, params: SamplingParams | None = None,
              stop_ids=None, batch_size: int = 64, max_tokens: int | None = None, on_token=None,
-             return_stats: bool = False, prefill_step_tokens: int = PREFILL_STEP_TOKENS):
+             return_stats: bool = False, prefill_step_tokens: int = PREFILL_STEP_TOKENS, dtype: str = "bfloat16"):
     """The Python entry point: token ids in, generated token ids out.
 
-    `model_or_session`: a loaded model (a session sized for the work is made) or a Session.
+    `model_or_session`: a model folder (loaded in `dtype`, as picolm's entry takes a file name,
+    picolm/model.h:504), a loaded model (a session sized for the work is made) or a Session.
     `prompts`: a list of token-id lists.  `stop_ids`: default, the configuration's
     eos_token_id.  Returns one `Generated` per prompt (and the timing record on request).
     """
@@ -231,6 +234,9 @@ def generate(model_or_session, prompts, max_new_tokens: int = 256, params: Sampl
     from .sampling.sampler import Sampler
     params = params or SamplingParams()
     prompts = [list(p) for p in prompts]
+    if isinstance(model_or_session, (str, os.PathLike)):
+        from .engine import load_model
+        model_or_session = load_model(os.fspath(model_or_session), dtype=dtype)
     if isinstance(model_or_session, Session):
         session = model_or_session
     else:

@@ -299,6 +299,10 @@ def test_greedy_generation_through_the_entry_point(dtype, folders):
             assert r.tokens[k] == int(np.argmax(lg)), (k, r.tokens)
             seq.append(r.tokens[k])
         assert len(r.tokens) == 8 and r.finish == "length"
+    # the entry point takes the model's folder as well, as picolm's takes a file name
+    import picolm_amd
+    again = picolm_amd.generate(d, prompts, max_new_tokens=8, stop_ids=(), dtype=dtype)
+    assert [r.tokens for r in again] == [r.tokens for r in got]
 
 
 def test_temperature_generation_follows_the_plain_sampler(folders):
