@@ -105,6 +105,15 @@ class LlamaConfig:
                 raise ConfigError(f"{key}: expected an integer, got {v!r}")
             return int(v)
 
+        # What this architecture's layers do not have.  picolm reads none of these keys (its layers
+        # have no bias tensors, picolm/safetensors.c:242-277, and one activation,
+        # picolm/tensor.c:3306-3315); a checkpoint that says otherwise would be computed wrongly.
+        for key in ("attention_bias", "mlp_bias"):
+            if d.get(key):
+                raise ConfigError(f"{key}: true is not supported (the products of this architecture have no bias)")
+        act = d.get("hidden_act", "silu")
+        if act not in ("silu", "swish"):
+            raise ConfigError(f"hidden_act: '{act}' is not supported (the feed-forward is silu(gate) * up)")
         H = integer("num_attention_heads")
         D = integer("hidden_size")
         if H <= 0:

@@ -152,3 +152,13 @@ def test_modules_named_in_the_environment_register_their_architectures(tmp_path,
     assert import_architecture_modules("") == [] and import_architecture_modules(" , ") == []
     with pytest.raises(ConfigError, match="cannot import 'no_such_module_here'"):
         import_architecture_modules("no_such_module_here")
+
+
+def test_options_that_the_layers_do_not_have_are_refused():
+    """Bias tensors and other activations than silu: picolm ignores the keys and has neither; a
+    config.json that asks for them is refused by name, not computed without them."""
+    d = dict(tiny.TINY_A)
+    assert LlamaConfig.from_dict(dict(d, attention_bias=False, mlp_bias=False, hidden_act="silu")).hidden_size == 64
+    for key, value, word in (("attention_bias", True, "attention_bias"), ("mlp_bias", True, "mlp_bias"), ("hidden_act", "gelu", "hidden_act")):
+        with pytest.raises(ConfigError, match=word):
+            LlamaConfig.from_dict(dict(d, **{key: value}))
